@@ -1,0 +1,184 @@
+/*
+ * C-ABI of the MI355X (gfx950) quantized-linear library: GGUF block-quantized
+ * weight x Q8_1-quantized activation products.  This is the whole boundary a
+ * host engine binds: plain device pointers and sizes, no C++ or framework
+ * types.
+ *
+ * Conventions (the ones the reference's own extern "C" HIP launchers follow,
+ * e.g. rocmGemv_native_vnni_fp32, src/v2/kernels/rocm/gemm/ROCmGemvKernel_native_VNNI.hip:5228-5260):
+ *   - every entry point returns bool; false = invalid argument or launch
+ *     failure, with a "[fn] reason" line on stderr and llam_ql_last_error()
+ *     holding the same text for the calling thread;
+ *   - all pointers named d_* are device pointers on `device_id`; the call makes
+ *     that device current, enqueues on `stream` (a hipStream_t, NULL = default
+ *     stream) and returns without synchronising;
+ *   - nothing is allocated, freed or synchronised inside a call;
+ *   - results are deterministic: no floating-point atomics, fixed reduction
+ *     order (the reference's LLAMINAR_DETERMINISTIC contract,
+ *     ROCmGemvKernel_native_VNNI.hip:5260-5261).
+ *
+ * Weight matrices are [N rows x K columns], row-major in super-blocks of 256
+ * columns (K % 256 == 0).  `fmt` is a llam_weight_format value.
+ *
+ * Arithmetic contract (reference CPU path, CPUNativeVNNIGemv.h:412-518):
+ *   per 32-column block  idot = sum_i a.qs[i]*w[i]           (int32, exact)
+ *                        acc += float(idot) * (f32(a.d)*f32(b_scale))
+ *                        acc += (float(a.sum_qs)*f32(a.d)) * f32(b_min)
+ * with (w, b_scale, b_min) the effective int8 sub-block the reference's weight
+ * packer derives from the GGUF block (CPUNativeVNNIWeightPacker.h:598-1136).
+ */
+#ifndef LLAMINAR_AMD_QL_API_H
+#define LLAMINAR_AMD_QL_API_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "llaminar_amd/ql_blocks.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLAM_QL_MAX_GEMV_M 8      /* rows of activations one GEMV launch accepts */
+#define LLAM_QL_MAX_FUSED 16      /* projections per fused launch (reference: <=16 FusedGemvDesc) */
+
+/* Text of the calling thread's most recent failure ("" if none). */
+const char *llam_ql_last_error(void);
+
+/* Library ABI version (bumped on any signature change). */
+int llam_ql_abi_version(void);
+
+/* ---- P1: activation quantiser --------------------------------------------------
+ * fp32 [M x K] (row stride K) -> llam_block_q8_1 [M x K/32].  K % 32 == 0.
+ * Replaces simd::quantize_single_block / quantize_two_blocks_avx512 and
+ * quantize_activations_to_q8_1 (src/v2/tensors/SIMDHelpers.h:4716-4959,
+ * src/v2/kernels/cpu/native_vnni/CPUNativeVNNIGemv.h:2000-2036); device-side
+ * counterpart of rocmQuantGemm_quantizeActivationsBlockwise
+ * (src/v2/kernels/rocm/gemm/ROCmQuantisedGemmKernel.hip:1187-1193).
+ * Output bytes equal the reference CPU quantiser's bit for bit. */
+bool llam_ql_quantize_q8_1(const float *d_x, void *d_q8, int M, int K,
+                           int device_id, void *stream);
+
+/* ---- weight preparation -----------------------------------------------------------
+ * Device layout the GEMV/GEMM kernels read.  Q4_K: the GGUF super-blocks
+ * unchanged (144 B is 16-byte aligned).  Q6_K (210 B) and IQ3_S (110 B) are
+ * split into 16-byte-aligned planes of the same total size (IQ3_S +2 B/block
+ * padding).  No value is changed; this only moves bytes.
+ * Replaces packWeightsCPUNativeVNNI (CPUNativeVNNIWeightPacker.h:598) /
+ * repack_*_to_vnni (src/v2/kernels/rocm/repack/VnniRepackKernels.hip:65-887).
+ * d_prepared must be 16-byte aligned and llam_ql_prepared_bytes() large; it may
+ * equal d_gguf for Q4_K only. */
+size_t llam_ql_prepared_bytes(uint8_t fmt, int N, int K);
+bool llam_ql_prepare_weights(uint8_t fmt, const void *d_gguf, void *d_prepared,
+                             int N, int K, int device_id, void *stream);
+
+/* ---- P2: decode GEMV (M = 1..LLAM_QL_MAX_GEMV_M) -----------------------------------
+ * d_y[m*ldy + n] = sum_k W[n,k] * A[m,k] for prepared weights and Q8_1
+ * activations A[m][K/32].  Replaces gemv_native_vnni_preq
+ * (CPUNativeVNNIGemv.h:712-954) and, for M>1, the small-M decode rows;
+ * device-side counterpart of rocmGemv_native_vnni_fp32
+ * (ROCmGemvKernel_native_VNNI.hip:5228). */
+bool llam_ql_gemv(uint8_t fmt, const void *d_w, const void *d_q8, float *d_y,
+                  int M, int N, int K, int ldy, int device_id, void *stream);
+
+/* One projection of a fused launch (reference: FusedGemvDesc,
+ * CPUNativeVNNIGemv.h:3782-3881 / TensorProjectionDesc, TensorKernels.h:601). */
+typedef struct
+{
+    const void *d_w;   /* prepared weights [N x K] */
+    float *d_y;        /* output, row stride ldy   */
+    int N;
+    int ldy;
+    uint8_t fmt;
+} llam_ql_proj;
+
+/* Several projections of ONE quantised input in one launch (QKV, gate+up,
+ * 2*top_k MoE gate/up).  Replaces gemv_native_vnni_fused_preq
+ * (CPUNativeVNNIGemv.h:3807-3881).  num <= LLAM_QL_MAX_FUSED; `projs` is a host
+ * array read during the call. */
+bool llam_ql_gemv_fused(const llam_ql_proj *projs, int num, const void *d_q8,
+                        int M, int K, int device_id, void *stream);
+
+/* Parity hook: the exact per-block int32 sums the GEMV forms, for rows
+ * [row0, row0+nrows): d_sums[(m*nrows + r)*(K/32) + kb].  Runs the same integer
+ * pipeline as llam_ql_gemv.  (The reference exposes the same quantity only
+ * inside its kernels: int_acc in CPUNativeVNNIGemv.h:417-487.) */
+bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,
+                             int32_t *d_sums, int M, int N, int K, int row0,
+                             int nrows, int device_id, void *stream);
+
+/* ---- P3: prefill GEMM (any M) -------------------------------------------------------
+ * Same contract as llam_ql_gemv for many activation rows, on int8 MFMA with
+ * int32 accumulation per 32-column block and fp32 rescale.  Replaces
+ * gemm_native_vnni_preq (CPUNativeVNNIGemv.h:2046-2287); device-side
+ * counterpart of launch_native_vnni_gemm
+ * (src/v2/kernels/rocm/gemm/ROCmQuantisedGemmKernel_native_VNNI.hip:2580-2632). */
+bool llam_ql_gemm(uint8_t fmt, const void *d_w, const void *d_q8, float *d_y,
+                  int M, int N, int K, int ldy, int device_id, void *stream);
+
+/* C = beta*C + alpha*T (+ bias per column), the operator's epilogue
+ * (CPUNativeVNNIGemmKernel.h:154-214).  beta == 0 overwrites.  T row stride N. */
+bool llam_ql_epilogue(float *d_c, const float *d_t, const float *d_bias, int M,
+                      int N, int ldc, float alpha, float beta, int device_id,
+                      void *stream);
+
+/* ---- P4: MoE ---------------------------------------------------------------------------
+ * Router: softmax over all experts, top_k by probability (ties: lower expert
+ * id first), weights renormalised over the top_k when normalize != 0.
+ * Replaces CPUMoEKernel::route's selection stage
+ * (src/v2/kernels/cpu/moe/CPUMoEKernel.cpp:87-124; IMoEKernel::route,
+ * src/v2/kernels/IMoEKernel.h:56).  d_logits [n_tokens x n_experts]. */
+bool llam_ql_moe_route(const float *d_logits, int n_tokens, int n_experts,
+                       int top_k, int normalize, int32_t *d_ids,
+                       float *d_weights, int device_id, void *stream);
+
+/* Expert weight table on the device: one entry per expert id (reference:
+ * DeviceNativeVNNIMatrixDesc tables, src/v2/tensors/TensorKernels.h:39-55,
+ * uploaded via IMoEKernel::upload...DescriptorTable, IMoEKernel.h:378-643). */
+typedef struct
+{
+    const void *d_gate; /* prepared [inter x hidden] */
+    const void *d_up;   /* prepared [inter x hidden] */
+    const void *d_down; /* prepared [hidden x inter] */
+} llam_ql_expert;
+
+/* Gate/up GEMVs of the routed experts, driven by device-resident routing ids:
+ * for token t, slot s, expert e = d_ids[t*top_k+s]:
+ *   d_gate_out[(t*top_k+s)*inter + i] = W_gate[e][i,:] . q8(hidden[t])
+ *   d_up_out  [(t*top_k+s)*inter + i] = W_up  [e][i,:] . q8(hidden[t])
+ * d_q8 holds the Q8_1 hidden state [n_tokens x hidden/32].  Replaces the
+ * 2*top_k-projection multiply_fused_tensor of MoEExpertComputeStage
+ * (src/v2/execution/compute_stages/stages/MoEExpertComputeStage.cpp:1450-1482);
+ * counterpart of groupedExpertGateUpDecodeFromRouting (IMoEKernel.h:378-643). */
+bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts,
+                         const int32_t *d_ids, const void *d_q8,
+                         float *d_gate_out, float *d_up_out, int n_tokens,
+                         int top_k, int hidden, int inter, int device_id,
+                         void *stream);
+
+/* act[i] = silu(gate[i]) * up[i] over n values, then Q8_1-quantise rows of
+ * `inter` values: d_q8_out [rows x inter/32].  d_act_out (optional) receives the
+ * fp32 activations.  Replaces compute_swiglu_serial + the per-expert quantise
+ * of multiply_fused_expert_down (MoEExpertComputeStage.cpp:1646,
+ * CPUNativeVNNIGemmKernel.h:1094-1107). */
+bool llam_ql_swiglu_quantize(const float *d_gate, const float *d_up,
+                             float *d_act_out, void *d_q8_out, int rows,
+                             int inter, int device_id, void *stream);
+
+/* Down GEMVs and weighted accumulation:
+ *   d_out[t*hidden + h] (+)= sum_s d_weights[t*top_k+s] * (W_down[e_s][h,:] . q8_act[t,s])
+ * Slots are added in ascending s; accumulate != 0 adds onto d_out, else
+ * overwrites.  Replaces multiply_fused_expert_down + vec_axpy
+ * (MoEExpertComputeStage.cpp:1664-1673); counterpart of
+ * groupedExpertDownDecode* (IMoEKernel.h:378-643). */
+bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts,
+                      const int32_t *d_ids, const float *d_weights,
+                      const void *d_q8_act, float *d_out, int n_tokens,
+                      int top_k, int hidden, int inter, int accumulate,
+                      int device_id, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,93 @@
+"""Compile the gfx950 quantized-linear library in-tree with hipcc.
+
+Every ``*.hip`` / ``*.cpp`` source under ``llaminar_amd/csrc`` is compiled into
+one shared object, ``llaminar_amd/lib/libllaminar_ql.so``.  hipcc cross-compiles
+for gfx950 without a GPU, so this runs anywhere the ROCm toolchain is present.
+
+Usage: ``python -m llaminar_amd.build [--force]``
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+ROOT = PKG.parent
+CSRC = PKG / "csrc"
+LIBDIR = PKG / "lib"
+LIB = LIBDIR / "libllaminar_ql.so"
+OBJDIR = PKG / "build"
+
+ARCH = "gfx950"
+# -packed-fp32-ops is switched OFF: scalar fp32 code must not be fused into
+# v_pk_*_f32 forms.  The host pass warns that it does not know the feature.
+HIP_FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    f"-I{ROOT / 'include'}",
+    f"-I{CSRC}",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(exe).exists():
+        raise RuntimeError("hipcc not found: the ROCm toolchain is required to build llaminar_amd")
+    return exe
+
+
+def sources() -> list[Path]:
+    return sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.cpp")))
+
+
+def _deps_mtime() -> float:
+    files = list(CSRC.glob("*")) + list((ROOT / "include" / "llaminar_amd").glob("*.h"))
+    return max(f.stat().st_mtime for f in files)
+
+
+def _compile(src: Path) -> Path:
+    obj = OBJDIR / (src.stem + ".o")
+    cmd = [hipcc(), *HIP_FLAGS, "-c", str(src), "-o", str(obj)]
+    if src.suffix == ".cpp":
+        cmd.insert(1, "-x")
+        cmd.insert(2, "hip")
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src.name}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(force: bool = True, verbose: bool = True) -> Path:
+    """Compile and link the library.  With force=False an up-to-date library is kept."""
+    if not force and LIB.exists() and LIB.stat().st_mtime >= _deps_mtime():
+        return LIB
+    OBJDIR.mkdir(exist_ok=True)
+    LIBDIR.mkdir(exist_ok=True)
+    srcs = sources()
+    if verbose:
+        print(f"[llaminar_amd.build] hipcc {ARCH}: {len(srcs)} sources", flush=True)
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        objs = list(pool.map(_compile, srcs))
+    cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stderr}")
+    if verbose:
+        print(f"[llaminar_amd.build] wrote {LIB} ({LIB.stat().st_size} bytes)", flush=True)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force=True)

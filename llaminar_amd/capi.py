@@ -1,0 +1,239 @@
+"""ctypes binding of the C-ABI in ``include/llaminar_amd/ql_api.h``.
+
+Python here is plumbing only: PyTorch supplies device memory and streams, every
+computation happens in the HIP library.  There is no fallback: if the shared
+object is missing or fails to load, importing the binding raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_bool, c_char_p, c_float, c_int, c_int32, c_size_t, c_uint8, c_void_p
+from pathlib import Path
+
+FMT_Q4_K = 5
+FMT_Q6_K = 8
+FMT_IQ3_S = 11
+FORMATS = {"q4_k": FMT_Q4_K, "q6_k": FMT_Q6_K, "iq3_s": FMT_IQ3_S}
+BLOCK_BYTES = {FMT_Q4_K: 144, FMT_Q6_K: 210, FMT_IQ3_S: 110}
+MAX_GEMV_M = 8
+MAX_FUSED = 16
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libllaminar_ql.so"
+
+
+class QLError(RuntimeError):
+    """A C-ABI call returned false; the message is llam_ql_last_error()."""
+
+
+class Proj(ctypes.Structure):
+    _fields_ = [("d_w", c_void_p), ("d_y", c_void_p), ("N", c_int), ("ldy", c_int), ("fmt", c_uint8)]
+
+
+class Expert(ctypes.Structure):
+    _fields_ = [("d_gate", c_void_p), ("d_up", c_void_p), ("d_down", c_void_p)]
+
+
+# name -> (restype, argtypes); mirrors ql_api.h declaration by declaration
+SIGNATURES = {
+    "llam_ql_last_error": (c_char_p, []),
+    "llam_ql_abi_version": (c_int, []),
+    "llam_ql_quantize_q8_1": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_prepared_bytes": (c_size_t, [c_uint8, c_int, c_int]),
+    "llam_ql_prepare_weights": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv_fused": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv_block_sums": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                         c_int, c_void_p]),
+    "llam_ql_gemm": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_epilogue": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int,
+                                  c_void_p]),
+    "llam_ql_moe_route": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "llam_ql_moe_gate_up": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                     c_int, c_int, c_void_p]),
+    "llam_ql_swiglu_quantize": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                  c_int, c_int, c_int, c_void_p]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m llaminar_amd.build` "
+            "(hipcc --offload-arch=gfx950).  There is no CPU fallback.")
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().llam_ql_last_error().decode()
+
+
+def _check(ok: bool, what: str) -> None:
+    if not ok:
+        raise QLError(f"{what}: {last_error()}")
+
+
+def _ptr(t) -> int:
+    """Device (or host) address of a torch tensor, or a raw int."""
+    if t is None:
+        return 0
+    if isinstance(t, int):
+        return t
+    return t.data_ptr()
+
+
+def _stream(stream=None) -> int:
+    if stream is None:
+        import torch
+
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream
+
+
+def _dev(t) -> int:
+    return t.device.index if t.device.index is not None else 0
+
+
+# ---------------------------------------------------------------------------
+# Thin call wrappers (tensor in, tensor out; all allocation is the caller's or
+# torch's, never the library's)
+# ---------------------------------------------------------------------------
+
+def quantize_q8_1(x, out=None, stream=None):
+    """fp32 [M,K] (or [K]) on the GPU -> uint8 tensor of M*(K/32) 36-byte Q8_1 blocks."""
+    import torch
+
+    x2 = x.reshape(1, -1) if x.dim() == 1 else x
+    M, K = x2.shape
+    assert x2.dtype == torch.float32 and x2.is_contiguous() and x2.is_cuda
+    if out is None:
+        out = torch.empty(M * (K // 32) * 36, dtype=torch.uint8, device=x.device)
+    _check(load().llam_ql_quantize_q8_1(_ptr(x2), _ptr(out), M, K, _dev(x2), _stream(stream)), "quantize_q8_1")
+    return out
+
+
+def prepared_bytes(fmt: int, N: int, K: int) -> int:
+    return int(load().llam_ql_prepared_bytes(fmt, N, K))
+
+
+def prepare_weights(fmt: int, gguf, N: int, K: int, stream=None):
+    """Raw GGUF super-block bytes (uint8 GPU tensor) -> device layout the kernels read."""
+    import torch
+
+    assert gguf.dtype == torch.uint8 and gguf.is_cuda and gguf.is_contiguous()
+    assert gguf.numel() == N * (K // 256) * BLOCK_BYTES[fmt], "weight byte count does not match N,K,fmt"
+    nbytes = prepared_bytes(fmt, N, K)
+    out = torch.empty(nbytes, dtype=torch.uint8, device=gguf.device)
+    _check(load().llam_ql_prepare_weights(fmt, _ptr(gguf), _ptr(out), N, K, _dev(gguf), _stream(stream)),
+           "prepare_weights")
+    return out
+
+
+def gemv(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None):
+    import torch
+
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32, device=w.device)
+    _check(load().llam_ql_gemv(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, out.stride(0) if out.dim() == 2 else N,
+                               _dev(w), _stream(stream)), "gemv")
+    return out
+
+
+def gemv_fused(projs, q8, M: int, K: int, stream=None):
+    """projs: list of (fmt, w, out[M,N]) sharing one quantised input."""
+    arr = (Proj * len(projs))()
+    for i, (fmt, w, out) in enumerate(projs):
+        arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], out.stride(0) if out.dim() == 2 else out.shape[-1], fmt)
+    dev = _dev(q8)
+    _check(load().llam_ql_gemv_fused(arr, len(projs), _ptr(q8), M, K, dev, _stream(stream)), "gemv_fused")
+
+
+def gemv_block_sums(fmt: int, w, q8, M: int, N: int, K: int, row0: int, nrows: int, stream=None):
+    import torch
+
+    out = torch.empty(M, nrows, K // 32, dtype=torch.int32, device=w.device)
+    _check(load().llam_ql_gemv_block_sums(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, row0, nrows, _dev(w),
+                                          _stream(stream)), "gemv_block_sums")
+    return out
+
+
+def gemm(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None):
+    import torch
+
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32, device=w.device)
+    _check(load().llam_ql_gemm(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, out.stride(0), _dev(w), _stream(stream)),
+           "gemm")
+    return out
+
+
+def epilogue(c, t, bias, alpha: float, beta: float, stream=None):
+    M, N = t.shape
+    _check(load().llam_ql_epilogue(_ptr(c), _ptr(t), _ptr(bias), M, N, c.stride(0), alpha, beta, _dev(c),
+                                   _stream(stream)), "epilogue")
+    return c
+
+
+def moe_route(logits, top_k: int, normalize: bool = True, stream=None):
+    import torch
+
+    T, E = logits.shape
+    ids = torch.empty(T, top_k, dtype=torch.int32, device=logits.device)
+    wts = torch.empty(T, top_k, dtype=torch.float32, device=logits.device)
+    _check(load().llam_ql_moe_route(_ptr(logits), T, E, top_k, int(normalize), _ptr(ids), _ptr(wts), _dev(logits),
+                                    _stream(stream)), "moe_route")
+    return ids, wts
+
+
+def expert_table(experts, device):
+    """experts: list of (gate, up, down) prepared-weight tensors -> device table (uint8 tensor)."""
+    import torch
+
+    arr = (Expert * len(experts))()
+    for i, (g, u, d) in enumerate(experts):
+        arr[i] = Expert(_ptr(g), _ptr(u), _ptr(d))
+    host = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8)
+    return host.to(device)
+
+
+def moe_gate_up(fmt: int, table, ids, q8, n_tokens: int, top_k: int, hidden: int, inter: int, stream=None):
+    import torch
+
+    gate = torch.empty(n_tokens * top_k, inter, dtype=torch.float32, device=q8.device)
+    up = torch.empty_like(gate)
+    _check(load().llam_ql_moe_gate_up(fmt, _ptr(table), _ptr(ids), _ptr(q8), _ptr(gate), _ptr(up), n_tokens, top_k,
+                                      hidden, inter, _dev(q8), _stream(stream)), "moe_gate_up")
+    return gate, up
+
+
+def swiglu_quantize(gate, up, want_act: bool = False, stream=None):
+    import torch
+
+    rows, inter = gate.shape
+    q8 = torch.empty(rows * (inter // 32) * 36, dtype=torch.uint8, device=gate.device)
+    act = torch.empty_like(gate) if want_act else None
+    _check(load().llam_ql_swiglu_quantize(_ptr(gate), _ptr(up), _ptr(act), _ptr(q8), rows, inter, _dev(gate),
+                                          _stream(stream)), "swiglu_quantize")
+    return (q8, act) if want_act else q8
+
+
+def moe_down(fmt: int, table, ids, weights, q8_act, out, n_tokens: int, top_k: int, hidden: int, inter: int,
+             accumulate: bool = False, stream=None):
+    _check(load().llam_ql_moe_down(fmt, _ptr(table), _ptr(ids), _ptr(weights), _ptr(q8_act), _ptr(out), n_tokens,
+                                   top_k, hidden, inter, int(accumulate), _dev(out), _stream(stream)), "moe_down")
+    return out

@@ -1,0 +1,109 @@
+// Device-side helpers shared by the gfx950 quantized-linear kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "llaminar_amd/ql_blocks.h"
+
+namespace llamql
+{
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    typedef int v16i __attribute__((ext_vector_type(16)));
+
+    constexpr int WAVE = 64;
+
+    // ---- binary16 helpers ---------------------------------------------------
+
+    __device__ __forceinline__ float h2f(uint16_t bits)
+    {
+        return __half2float(__ushort_as_half(bits));
+    }
+
+    // fp32 -> fp16 -> fp32 with the rounding the reference's weight packer
+    // applies to effective block scales and mins (tensors/FP16Utils.h:75-118):
+    // nearest-even when the fp16 result is normal, truncation toward zero when
+    // it is subnormal (|x| < 2^-14), signed zero below 2^-25.
+    __device__ __forceinline__ float f16_round_packer(float x)
+    {
+        float r = __half2float(__float2half_rn(x));
+        if (fabsf(x) < 6.103515625e-05f)
+            r = truncf(x * 16777216.0f) * 5.9604644775390625e-08f;
+        return r;
+    }
+
+    // ---- cross-lane -----------------------------------------------------------
+
+    template <int CTRL>
+    __device__ __forceinline__ int dpp_i32(int v)
+    {
+        return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+    }
+    template <int CTRL>
+    __device__ __forceinline__ float dpp_f32(float v)
+    {
+        return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+    }
+
+    constexpr int DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]
+    constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
+    constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+    constexpr int DPP_ROW_MIRROR = 0x140;
+
+    // Sum over the 64 lanes of a wavefront; every lane returns the total.
+    // Fixed association order, so results are run-to-run identical.
+    __device__ __forceinline__ float wave_sum(float v)
+    {
+        v += dpp_f32<DPP_QUAD_XOR1>(v);
+        v += dpp_f32<DPP_QUAD_XOR2>(v);
+        v += dpp_f32<DPP_ROW_HALF_MIRROR>(v);
+        v += dpp_f32<DPP_ROW_MIRROR>(v);
+        const int b = __float_as_int(v);
+        const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0));
+        const float r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+        const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32));
+        const float r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+        return (r0 + r1) + (r2 + r3);
+    }
+
+    // ---- integer dot ------------------------------------------------------------
+
+    // acc + sum of four signed-byte products (v_dot4_i32_i8).
+    __device__ __forceinline__ int dot4(int a, int b, int acc)
+    {
+        return __builtin_amdgcn_sdot4(a, b, acc, false);
+    }
+
+    __device__ __forceinline__ int dot16(const v4i a, const v4i b, int acc)
+    {
+        acc = dot4(a.x, b.x, acc);
+        acc = dot4(a.y, b.y, acc);
+        acc = dot4(a.z, b.z, acc);
+        acc = dot4(a.w, b.w, acc);
+        return acc;
+    }
+
+    // ---- Q4_K -------------------------------------------------------------------
+
+    // 6-bit (scale, min) pair j of a Q4_K super-block whose 12 packed bytes are
+    // given as three little-endian words (bytes 0-3, 4-7, 8-11).
+    __device__ __forceinline__ void q4k_scale_min(int j, uint32_t s0, uint32_t s1, uint32_t s2,
+                                                  uint32_t &sc, uint32_t &mn)
+    {
+        const int sh = 8 * (j & 3);
+        const uint32_t a = (s0 >> sh) & 0xFFu;
+        const uint32_t b = (s1 >> sh) & 0xFFu;
+        const uint32_t p = (s2 >> sh) & 0xFFu;
+        if (j < 4)
+        {
+            sc = a & 63u;
+            mn = b & 63u;
+        }
+        else
+        {
+            sc = (p & 15u) | ((a >> 6) << 4);
+            mn = (p >> 4) | ((b >> 6) << 4);
+        }
+    }
+} // namespace llamql

@@ -1,0 +1,47 @@
+// Host-side plumbing shared by the C-ABI launchers: error text, argument
+// checks, device selection.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+namespace llamql
+{
+    // Records "[fn] message" for llam_ql_last_error() and prints it to stderr.
+    // Always returns false so launchers can `return fail(...)`.
+    bool fail(const char *fn, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+    void clear_error();
+    const char *last_error_text();
+
+    inline bool set_device(const char *fn, int device_id)
+    {
+        int count = 0;
+        hipError_t e = hipGetDeviceCount(&count);
+        if (e != hipSuccess || count <= 0)
+            return fail(fn, "no HIP device available (%s)", hipGetErrorString(e));
+        if (device_id < 0 || device_id >= count)
+            return fail(fn, "device_id %d out of range [0,%d)", device_id, count);
+        e = hipSetDevice(device_id);
+        if (e != hipSuccess)
+            return fail(fn, "hipSetDevice(%d): %s", device_id, hipGetErrorString(e));
+        return true;
+    }
+
+    inline bool launched(const char *fn)
+    {
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return fail(fn, "kernel launch failed: %s", hipGetErrorString(e));
+        return true;
+    }
+
+    inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+    inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
+    // Number of compute units of the current device (cached per device).
+    int cu_count(int device_id);
+
+    inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+} // namespace llamql

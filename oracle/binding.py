@@ -1,0 +1,251 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes doors onto the checkers.
+
+``Oracle``  -> oracle/libql_oracle.so        (scalar C restatement, ql_oracle.c)
+``Ref``     -> oracle/_ref/libllaminar_ref.so (the reference's own CPU kernels,
+                                               present only where it was built)
+
+Only tests, the smoke check and the benchmark's cpu_baseline leg import this.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from ctypes import POINTER, c_float, c_int, c_int32, c_long, c_uint8, c_uint16, c_void_p
+from pathlib import Path
+
+import numpy as np
+
+HERE = Path(__file__).resolve().parent
+ORACLE_LIB = HERE / "libql_oracle.so"
+REF_LIB = HERE / "_ref" / "libllaminar_ref.so"
+
+FMT_Q4_K, FMT_Q6_K, FMT_IQ3_S = 5, 8, 11
+BLOCK_BYTES = {FMT_Q4_K: 144, FMT_Q6_K: 210, FMT_IQ3_S: 110}
+
+
+def build(reference: str = "/root/reference") -> None:
+    """Compile the restatement (always) and the reference shim (when the tree is there)."""
+    subprocess.run(["make", "-C", str(HERE), f"REFERENCE={reference}", "all"], check=True,
+                   stdout=subprocess.DEVNULL)
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(c_void_p)
+
+
+class Oracle:
+    def __init__(self):
+        if not ORACLE_LIB.exists():
+            build()
+        L = ctypes.CDLL(str(ORACLE_LIB))
+        L.qlo_f16_to_f32.restype = c_float
+        L.qlo_f16_to_f32.argtypes = [c_uint16]
+        L.qlo_f32_to_f16_sw.restype = c_uint16
+        L.qlo_f32_to_f16_sw.argtypes = [c_float]
+        L.qlo_f32_to_f16_rne.restype = c_uint16
+        L.qlo_f32_to_f16_rne.argtypes = [c_float]
+        L.qlo_quantize_block_q8_1.argtypes = [c_void_p, c_int, c_void_p]
+        L.qlo_quantize_q8_1.argtypes = [c_void_p, c_int, c_int, c_void_p]
+        L.qlo_get_scale_min_k4.argtypes = [c_int, c_void_p, c_void_p, c_void_p]
+        L.qlo_subblocks.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_void_p]
+        L.qlo_gemm_rows.argtypes = [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int,
+                                    c_void_p, c_int]
+        L.qlo_epilogue.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]
+        L.qlo_moe_route.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+        L.qlo_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_void_p]
+        self.L = L
+
+    # -- fp16 ---------------------------------------------------------------
+    def f16_to_f32(self, h: int) -> float:
+        return float(self.L.qlo_f16_to_f32(h))
+
+    def f32_to_f16_sw(self, f: float) -> int:
+        return int(self.L.qlo_f32_to_f16_sw(np.float32(f)))
+
+    def f32_to_f16_rne(self, f: float) -> int:
+        return int(self.L.qlo_f32_to_f16_rne(np.float32(f)))
+
+    # -- Q8_1 ---------------------------------------------------------------
+    def quantize_block(self, x: np.ndarray, valid: int = 32) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.zeros(36, dtype=np.uint8)
+        self.L.qlo_quantize_block_q8_1(_p(x), valid, _p(out))
+        return out
+
+    def quantize(self, x: np.ndarray) -> np.ndarray:
+        """fp32 [M,K] -> uint8 [M, ceil(K/32), 36]"""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None]
+        M, K = x.shape
+        out = np.zeros((M, (K + 31) // 32, 36), dtype=np.uint8)
+        self.L.qlo_quantize_q8_1(_p(x), M, K, _p(out))
+        return out
+
+    # -- weights --------------------------------------------------------------
+    def scale_min_k4(self, j: int, scales12: np.ndarray):
+        sc = np.zeros(1, np.uint8)
+        m = np.zeros(1, np.uint8)
+        s = np.ascontiguousarray(scales12, dtype=np.uint8)
+        self.L.qlo_get_scale_min_k4(j, _p(s), _p(sc), _p(m))
+        return int(sc[0]), int(m[0])
+
+    def subblocks(self, fmt: int, sb: np.ndarray):
+        """one super-block's bytes -> (int8[256], fp16-bits scales[8], fp16-bits mins[8])"""
+        sb = np.ascontiguousarray(sb, dtype=np.uint8)
+        assert sb.size == BLOCK_BYTES[fmt]
+        w = np.zeros(256, np.int8)
+        sc = np.zeros(8, np.uint16)
+        mn = np.zeros(8, np.uint16)
+        self.L.qlo_subblocks(fmt, _p(sb), _p(w), _p(sc), _p(mn))
+        return w, sc, mn
+
+    # -- GEMV / GEMM ------------------------------------------------------------
+    def gemm(self, fmt: int, W: np.ndarray, K: int, q8: np.ndarray, n0: int = 0, n1: int | None = None,
+             want_sums: bool = False, k_tiles: int = 0):
+        """W: uint8 raw GGUF rows; q8: uint8 [M, K/32, 36].  Returns C[M, n1-n0] (and sums[M, n1-n0, K/32])."""
+        W = np.ascontiguousarray(W, dtype=np.uint8).reshape(-1)
+        row_bytes = (K // 256) * BLOCK_BYTES[fmt]
+        N = W.size // row_bytes
+        if n1 is None:
+            n1 = N
+        q8 = np.ascontiguousarray(q8, dtype=np.uint8)
+        M = q8.shape[0]
+        C = np.zeros((M, N), np.float32)
+        sums = np.zeros((M, n1 - n0, K // 32), np.int32) if want_sums else None
+        self.L.qlo_gemm_rows(fmt, _p(W), K, n0, n1, _p(q8), M, _p(C), N, _p(sums) if want_sums else None, k_tiles)
+        C = C[:, n0:n1].copy()
+        return (C, sums) if want_sums else C
+
+    def epilogue(self, C: np.ndarray, T: np.ndarray, alpha: float, beta: float, bias=None) -> np.ndarray:
+        C = np.ascontiguousarray(C, dtype=np.float32).copy()
+        T = np.ascontiguousarray(T, dtype=np.float32)
+        M, N = T.shape
+        b = np.ascontiguousarray(bias, dtype=np.float32) if bias is not None else None
+        self.L.qlo_epilogue(_p(C), _p(T), M, N, N, alpha, beta, _p(b) if b is not None else None)
+        return C
+
+    # -- MoE ----------------------------------------------------------------------
+    def route(self, logits: np.ndarray, top_k: int, normalize: bool = True):
+        logits = np.ascontiguousarray(logits, dtype=np.float32)
+        T, E = logits.shape
+        ids = np.zeros((T, top_k), np.int32)
+        w = np.zeros((T, top_k), np.float32)
+        probs = np.zeros((T, E), np.float32)
+        self.L.qlo_moe_route(_p(logits), T, E, top_k, int(normalize), _p(ids), _p(w), _p(probs))
+        return ids, w, probs
+
+    def swiglu(self, gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+        gate = np.ascontiguousarray(gate, dtype=np.float32)
+        up = np.ascontiguousarray(up, dtype=np.float32)
+        out = np.zeros_like(gate)
+        self.L.qlo_swiglu(_p(gate), _p(up), gate.size, _p(out))
+        return out
+
+
+class Ref:
+    """The reference's own code.  `available()` is False where it was not built
+    (for instance on a machine that never saw the reference tree)."""
+
+    @staticmethod
+    def available() -> bool:
+        return REF_LIB.exists()
+
+    def __init__(self):
+        L = ctypes.CDLL(str(REF_LIB), mode=os.RTLD_LAZY)
+        L.ref_f16_to_f32.restype = c_float
+        L.ref_f16_to_f32.argtypes = [c_uint16]
+        L.ref_f32_to_f16.restype = c_uint16
+        L.ref_f32_to_f16.argtypes = [c_float]
+        L.ref_f32_to_f16_f16c.restype = c_uint16
+        L.ref_f32_to_f16_f16c.argtypes = [c_float]
+        L.ref_iq3s_grid.restype = POINTER(ctypes.c_uint32)
+        L.ref_get_scale_min_k4.argtypes = [c_int, c_void_p, c_void_p, c_void_p]
+        L.ref_quantize_block_q8_1.argtypes = [c_void_p, c_int, c_void_p, c_int]
+        L.ref_quantize_q8_1.argtypes = [c_void_p, c_int, c_int, c_void_p]
+        L.ref_unpack_superblock.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int]
+        L.ref_pack.restype = c_void_p
+        L.ref_pack.argtypes = [c_int, c_void_p, c_int, c_int]
+        L.ref_pack_free.argtypes = [c_void_p]
+        L.ref_pack_bytes.restype = c_long
+        L.ref_pack_bytes.argtypes = [c_void_p]
+        L.ref_gemm_packed.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int]
+        L.ref_gemm_fp32_packed.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int]
+        L.ref_gemm.restype = c_int
+        L.ref_gemm.argtypes = [c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int]
+        L.ref_omp_threads.restype = c_int
+        self.L = L
+
+    def f16_to_f32(self, h):
+        return float(self.L.ref_f16_to_f32(h))
+
+    def f32_to_f16(self, f):
+        return int(self.L.ref_f32_to_f16(np.float32(f)))
+
+    def f32_to_f16_f16c(self, f):
+        return int(self.L.ref_f32_to_f16_f16c(np.float32(f)))
+
+    def iq3s_grid(self) -> np.ndarray:
+        return np.ctypeslib.as_array(self.L.ref_iq3s_grid(), shape=(512,)).copy()
+
+    def scale_min_k4(self, j, scales12):
+        sc = np.zeros(1, np.uint8)
+        m = np.zeros(1, np.uint8)
+        s = np.ascontiguousarray(scales12, dtype=np.uint8)
+        self.L.ref_get_scale_min_k4(j, _p(s), _p(sc), _p(m))
+        return int(sc[0]), int(m[0])
+
+    def quantize_block(self, x, valid=32, variant=0):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.zeros(36, np.uint8)
+        self.L.ref_quantize_block_q8_1(_p(x), valid, _p(out), variant)
+        return out
+
+    def quantize(self, x):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None]
+        M, K = x.shape
+        out = np.zeros((M, (K + 31) // 32, 36), np.uint8)
+        self.L.ref_quantize_q8_1(_p(x), M, K, _p(out))
+        return out
+
+    def unpack_superblock(self, fmt, sb, variant=0):
+        sb = np.ascontiguousarray(sb, dtype=np.uint8)
+        w = np.zeros(256, np.int8)
+        sc = np.zeros(8, np.float32)
+        mn = np.zeros(8, np.float32)
+        self.L.ref_unpack_superblock(fmt, _p(sb), _p(w), _p(sc), _p(mn), variant)
+        return w, sc, mn
+
+    def gemm(self, fmt, W, N, K, q8, isa=0):
+        W = np.ascontiguousarray(W, dtype=np.uint8).reshape(-1)
+        q8 = np.ascontiguousarray(q8, dtype=np.uint8)
+        M = q8.shape[0]
+        C = np.zeros((M, N), np.float32)
+        ok = self.L.ref_gemm(fmt, _p(W), N, K, _p(q8), M, _p(C), N, isa)
+        assert ok
+        return C
+
+    def pack(self, fmt, W, N, K):
+        W = np.ascontiguousarray(W, dtype=np.uint8).reshape(-1)
+        h = self.L.ref_pack(fmt, _p(W), N, K)
+        assert h
+        return h
+
+    def pack_free(self, h):
+        self.L.ref_pack_free(h)
+
+    def pack_bytes(self, h) -> int:
+        return int(self.L.ref_pack_bytes(h))
+
+    def gemm_packed(self, h, q8, N, isa=0, out=None):
+        q8 = np.ascontiguousarray(q8, dtype=np.uint8)
+        M = q8.shape[0]
+        C = out if out is not None else np.zeros((M, N), np.float32)
+        self.L.ref_gemm_packed(h, _p(q8), M, _p(C), N, isa)
+        return C
+
+    def omp_threads(self) -> int:
+        return int(self.L.ref_omp_threads())
