@@ -49,6 +49,12 @@ const char *llam_ql_last_error(void);
 /* Library ABI version (bumped on any signature change). */
 int llam_ql_abi_version(void);
 
+/* Tuning overrides for sweeps (reference: rocmGemv_native_vnni_set_tuning_overrides /
+ * ..._reset_tuning_overrides, ROCmGemvKernel_native_VNNI.hip:182-196).
+ * rows_per_wave <= 0 restores the built-in choice.  Not thread-safe. */
+void llam_ql_set_gemv_tuning(int rows_per_wave);
+void llam_ql_reset_gemv_tuning(void);
+
 /* ---- P1: activation quantiser --------------------------------------------------
  * fp32 [M x K] (row stride K) -> llam_block_q8_1 [M x K/32].  K % 32 == 0.
  * Replaces simd::quantize_single_block / quantize_two_blocks_avx512 and
@@ -150,9 +156,11 @@ typedef struct
  * d_q8 holds the Q8_1 hidden state [n_tokens x hidden/32].  Replaces the
  * 2*top_k-projection multiply_fused_tensor of MoEExpertComputeStage
  * (src/v2/execution/compute_stages/stages/MoEExpertComputeStage.cpp:1450-1482);
- * counterpart of groupedExpertGateUpDecodeFromRouting (IMoEKernel.h:378-643). */
+ * counterpart of groupedExpertGateUpDecodeFromRouting (IMoEKernel.h:378-643).
+ * The table has n_experts entries; a slot whose id is outside [0,n_experts) is
+ * skipped (its outputs are left untouched). */
 bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts,
-                         const int32_t *d_ids, const void *d_q8,
+                         int n_experts, const int32_t *d_ids, const void *d_q8,
                          float *d_gate_out, float *d_up_out, int n_tokens,
                          int top_k, int hidden, int inter, int device_id,
                          void *stream);
@@ -173,10 +181,20 @@ bool llam_ql_swiglu_quantize(const float *d_gate, const float *d_up,
  * (MoEExpertComputeStage.cpp:1664-1673); counterpart of
  * groupedExpertDownDecode* (IMoEKernel.h:378-643). */
 bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts,
-                      const int32_t *d_ids, const float *d_weights,
+                      int n_experts, const int32_t *d_ids, const float *d_weights,
                       const void *d_q8_act, float *d_out, int n_tokens,
                       int top_k, int hidden, int inter, int accumulate,
                       int device_id, void *stream);
+
+/* Shared expert: d_out[t,:] += g_t * d_shared[t,:] with
+ * g_t = sigmoid(dot(d_gate_inp, d_hidden[t,:])), or g_t = 1 when d_gate_inp is
+ * NULL.  Replaces CPUMoEKernel::sharedExpertGate + the add into the token output
+ * (src/v2/kernels/cpu/moe/CPUMoEKernel.cpp:162-197; IMoEKernel::weightedAdd,
+ * src/v2/kernels/IMoEKernel.h:189). */
+bool llam_ql_shared_expert_add(float *d_out, const float *d_shared,
+                               const float *d_hidden, const float *d_gate_inp,
+                               int n_tokens, int d_model, int device_id,
+                               void *stream);
 
 #ifdef __cplusplus
 }

@@ -38,6 +38,8 @@ class Expert(ctypes.Structure):
 SIGNATURES = {
     "llam_ql_last_error": (c_char_p, []),
     "llam_ql_abi_version": (c_int, []),
+    "llam_ql_set_gemv_tuning": (None, [c_int]),
+    "llam_ql_reset_gemv_tuning": (None, []),
     "llam_ql_quantize_q8_1": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_prepared_bytes": (c_size_t, [c_uint8, c_int, c_int]),
     "llam_ql_prepare_weights": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
@@ -49,11 +51,12 @@ SIGNATURES = {
     "llam_ql_epilogue": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int,
                                   c_void_p]),
     "llam_ql_moe_route": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
-    "llam_ql_moe_gate_up": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                     c_int, c_int, c_void_p]),
+    "llam_ql_moe_gate_up": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                     c_int, c_int, c_int, c_void_p]),
     "llam_ql_swiglu_quantize": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
-    "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                  c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                  c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_shared_expert_add": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
 }
 
 _lib = None
@@ -211,13 +214,14 @@ def expert_table(experts, device):
     return host.to(device)
 
 
-def moe_gate_up(fmt: int, table, ids, q8, n_tokens: int, top_k: int, hidden: int, inter: int, stream=None):
+def moe_gate_up(fmt: int, table, n_experts: int, ids, q8, n_tokens: int, top_k: int, hidden: int, inter: int,
+                stream=None):
     import torch
 
     gate = torch.empty(n_tokens * top_k, inter, dtype=torch.float32, device=q8.device)
     up = torch.empty_like(gate)
-    _check(load().llam_ql_moe_gate_up(fmt, _ptr(table), _ptr(ids), _ptr(q8), _ptr(gate), _ptr(up), n_tokens, top_k,
-                                      hidden, inter, _dev(q8), _stream(stream)), "moe_gate_up")
+    _check(load().llam_ql_moe_gate_up(fmt, _ptr(table), n_experts, _ptr(ids), _ptr(q8), _ptr(gate), _ptr(up),
+                                      n_tokens, top_k, hidden, inter, _dev(q8), _stream(stream)), "moe_gate_up")
     return gate, up
 
 
@@ -232,8 +236,16 @@ def swiglu_quantize(gate, up, want_act: bool = False, stream=None):
     return (q8, act) if want_act else q8
 
 
-def moe_down(fmt: int, table, ids, weights, q8_act, out, n_tokens: int, top_k: int, hidden: int, inter: int,
-             accumulate: bool = False, stream=None):
-    _check(load().llam_ql_moe_down(fmt, _ptr(table), _ptr(ids), _ptr(weights), _ptr(q8_act), _ptr(out), n_tokens,
-                                   top_k, hidden, inter, int(accumulate), _dev(out), _stream(stream)), "moe_down")
+def moe_down(fmt: int, table, n_experts: int, ids, weights, q8_act, out, n_tokens: int, top_k: int, hidden: int,
+             inter: int, accumulate: bool = False, stream=None):
+    _check(load().llam_ql_moe_down(fmt, _ptr(table), n_experts, _ptr(ids), _ptr(weights), _ptr(q8_act), _ptr(out),
+                                   n_tokens, top_k, hidden, inter, int(accumulate), _dev(out), _stream(stream)),
+           "moe_down")
+    return out
+
+
+def shared_expert_add(out, shared, hidden=None, gate_inp=None, stream=None):
+    T, D = out.shape
+    _check(load().llam_ql_shared_expert_add(_ptr(out), _ptr(shared), _ptr(hidden), _ptr(gate_inp), T, D, _dev(out),
+                                            _stream(stream)), "shared_expert_add")
     return out

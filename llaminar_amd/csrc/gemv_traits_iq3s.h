@@ -1,0 +1,163 @@
+// IQ3_S x Q8_1 decode GEMV for gfx950: format traits for the shared skeleton.
+//
+// The reference's CPU path REQUANTISES every 32-element IQ3_S sub-block to int8
+// at pack time (src/v2/tensors/SIMDHelpers.h:8612-8768): codebook magnitudes
+// g in {1,3,..,15} times db = d*(1+2*nib), signed, then scale = max|v|/127 and
+// w = rne(v/scale).  Because v = +-g*db with one db per sub-block this is the pure
+// integer map  w = +-round(g*127/gmax)  (gmax = largest magnitude in the
+// sub-block; never a tie) with  b_scale = f16((gmax*db)/127).  The kernel keeps
+// the eight possible maps (gmax = 1,3,..,15) applied to the whole 512-entry
+// codebook as lookup tables in LDS, so one ds_read_b32 yields four requantised
+// magnitudes; signs are applied with a byte permute.  HBM traffic stays at the
+// format's 110 B per 256 weights (+2 B alignment padding).
+//
+// Device layout (llam_ql_prepare_weights): three planes over T = N*K/256
+// super-blocks -- qs [T][64], signs [T][32], meta [T][16] = qh[8] scales[4] d[2]
+// pad[2].  Lane c of an 8-lane group owns sub-block c.
+#pragma once
+#include "gemv_core.h"
+
+#define LLAM_IQ3S_GRID_QUALIFIER static constexpr
+#include "llaminar_amd/iq3s_grid.h"
+
+namespace llamql
+{
+    struct IQ3STables
+    {
+        uint32_t req[8 * 512]; // req[gi*512 + idx]: bytes round(g*127/(2*gi+1)) of codebook entry idx
+        uint32_t gmax[128];    // byte idx: largest magnitude in codebook entry idx
+    };
+
+    constexpr IQ3STables make_iq3s_tables()
+    {
+        IQ3STables t{};
+        for (int idx = 0; idx < 512; ++idx)
+        {
+            const uint32_t g4 = llam_iq3s_grid[idx];
+            uint32_t mx = 0;
+            for (int b = 0; b < 4; ++b)
+            {
+                const uint32_t g = (g4 >> (8 * b)) & 0xFFu;
+                if (g > mx)
+                    mx = g;
+            }
+            t.gmax[idx >> 2] |= mx << (8 * (idx & 3));
+            for (int gi = 0; gi < 8; ++gi)
+            {
+                const uint32_t gm = 2u * (uint32_t)gi + 1u;
+                uint32_t out = 0;
+                for (int b = 0; b < 4; ++b)
+                {
+                    const uint32_t g = (g4 >> (8 * b)) & 0xFFu;
+                    uint32_t q = (2u * g * 127u + gm) / (2u * gm); // round half up; never exactly half
+                    if (q > 127u)
+                        q = 127u; // entries with g > gm are never looked up
+                    out |= q << (8 * b);
+                }
+                t.req[gi * 512 + idx] = out;
+            }
+        }
+        return t;
+    }
+
+    static __device__ const IQ3STables g_iq3s_tables = make_iq3s_tables();
+
+    struct IQ3STraits
+    {
+        static constexpr bool PAIR = false;
+        static constexpr bool HAS_MIN = false;
+        static constexpr int TABLE_BYTES = (int)sizeof(IQ3STables);
+
+        __device__ static void stage_tables(void *lds_tab)
+        {
+            const uint4 *src = reinterpret_cast<const uint4 *>(&g_iq3s_tables);
+            uint4 *dst = static_cast<uint4 *>(lds_tab);
+            constexpr int n = (int)(sizeof(IQ3STables) / 16);
+            for (int i = threadIdx.x; i < n; i += blockDim.x)
+                dst[i] = src[i];
+        }
+
+        struct Raw
+        {
+            uint2 qs;
+            uint32_t signs;
+            uint4 meta;
+        };
+
+        // natural layout: block j is unit j, dword q at position q
+        __device__ __forceinline__ static void unit_of(int j, int q, int &c, int &p)
+        {
+            c = j;
+            p = q >> 2;
+        }
+
+        __device__ __forceinline__ static void where(int c, int &j0, int &e0, int &j1, int &e1)
+        {
+            j0 = j1 = c;
+            e0 = 0;
+            e1 = 16;
+        }
+
+        __device__ __forceinline__ static Raw load(const GemvArgs &a, long row, int sb, int c)
+        {
+            const size_t T = (size_t)a.N * a.SB;
+            const size_t t = (size_t)row * a.SB + sb;
+            const uint8_t *base = static_cast<const uint8_t *>(a.w);
+            Raw r;
+            r.qs = reinterpret_cast<const uint2 *>(base)[t * 8 + c];
+            r.signs = reinterpret_cast<const uint32_t *>(base + T * 64)[t * 8 + c];
+            r.meta = reinterpret_cast<const uint4 *>(base + T * 96)[t];
+            return r;
+        }
+
+        __device__ __forceinline__ static void decode(const Raw &r, int c, v4i &w0, v4i &w1, int &j,
+                                                      float &bscale, float &bmin, const void *tab)
+        {
+            const uint32_t *req = static_cast<const uint32_t *>(tab);
+            const uint8_t *gmaxb = reinterpret_cast<const uint8_t *>(req + 8 * 512);
+
+            const uint32_t qh = (((c & 4) ? r.meta.y : r.meta.x) >> (8 * (c & 3))) & 0xFFu;
+            const uint32_t nib = (r.meta.z >> (4 * c)) & 0xFu; // scales[c/2], low nibble for even c
+            const float d = h2f((uint16_t)(r.meta.w & 0xFFFFu));
+
+            uint32_t idx[8];
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+            {
+                const uint32_t qsb = ((l < 4 ? r.qs.x : r.qs.y) >> (8 * (l & 3))) & 0xFFu;
+                idx[l] = qsb | (((qh >> l) & 1u) << 8);
+            }
+            uint32_t gm = 0;
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+                gm = max(gm, (uint32_t)gmaxb[idx[l]]);
+
+            const float db = d * (1.0f + 2.0f * (float)nib);
+            const float amax = (float)gm * db;
+            float scale = __fdiv_rn(amax, 127.0f);
+            if (scale > 65504.0f)
+                scale = 65504.0f;
+            if (amax < 1e-6f)
+                scale = 0.0f;
+
+            const uint32_t *rq = req + (gm >> 1) * 512;
+            int ws[8];
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+            {
+                const uint32_t w = rq[idx[l]];
+                const uint32_t sg = (r.signs >> (4 * l)) & 0xFu;
+                // bit k of sg -> bit 0 of byte k, then selector byte k = k (keep) or k+4 (negated)
+                const uint32_t spread = (sg * 0x00204081u) & 0x01010101u;
+                const uint32_t sel = 0x03020100u | (spread << 2);
+                const uint32_t neg = 0x01010100u - w; // bytewise -w: every byte of w is in 1..127
+                ws[l] = (scale != 0.0f) ? (int)__builtin_amdgcn_perm(neg, w, sel) : 0;
+            }
+            w0 = (v4i){ws[0], ws[1], ws[2], ws[3]};
+            w1 = (v4i){ws[4], ws[5], ws[6], ws[7]};
+            j = c;
+            bscale = f16_round_packer(scale);
+            bmin = 0.0f;
+        }
+    };
+} // namespace llamql

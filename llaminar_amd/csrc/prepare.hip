@@ -1,0 +1,128 @@
+// Weight preparation: raw GGUF super-blocks -> the device layout the kernels
+// read.  Only moves bytes; no value changes.
+//
+//   Q4_K  : unchanged (144-byte blocks are 16-byte aligned)
+//   Q6_K  : planes ql [T][128] | qh [T][64] | scales [T][16] | d [T] fp16      (T*210 B)
+//   IQ3_S : planes qs [T][64] | signs [T][32] | meta [T][16]                   (T*112 B)
+//           meta = qh[8] scales[4] d[2] pad[2]
+// with T = N*K/256 super-blocks in row-major order.  Raw Q6_K / IQ3_S blocks are
+// 210 / 110 bytes, i.e. only 2-byte aligned, so the copy works in halfwords.
+#include "ql_device.h"
+#include "ql_host.h"
+
+#include "llaminar_amd/ql_api.h"
+
+namespace llamql
+{
+    __global__ void __launch_bounds__(256)
+        prepare_q6k_kernel(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, size_t T)
+    {
+        const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (i >= T * 105)
+            return;
+        const size_t t = i / 105;
+        const int u = (int)(i - t * 105);
+        const uint16_t v = src[i];
+        size_t o;
+        if (u < 64)
+            o = t * 64 + u; // ql
+        else if (u < 96)
+            o = T * 64 + t * 32 + (u - 64); // qh
+        else if (u < 104)
+            o = T * 96 + t * 8 + (u - 96); // scales
+        else
+            o = T * 104 + t; // d
+        dst[o] = v;
+    }
+
+    __global__ void __launch_bounds__(256)
+        prepare_iq3s_kernel(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, size_t T)
+    {
+        // 56 halfwords are written per block (55 copied + 1 zero pad)
+        const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (i >= T * 56)
+            return;
+        const size_t t = i / 56;
+        const int u = (int)(i - t * 56);
+        uint16_t v = 0;
+        size_t o;
+        if (u == 55)
+        {
+            o = T * 48 + t * 8 + 7; // pad
+        }
+        else
+        {
+            v = src[t * 55 + u];
+            if (u == 0)
+                o = T * 48 + t * 8 + 6; // d
+            else if (u < 33)
+                o = t * 32 + (u - 1); // qs
+            else if (u < 37)
+                o = T * 48 + t * 8 + (u - 33); // qh
+            else if (u < 53)
+                o = T * 32 + t * 16 + (u - 37); // signs
+            else
+                o = T * 48 + t * 8 + 4 + (u - 53); // scales
+        }
+        dst[o] = v;
+    }
+} // namespace llamql
+
+extern "C" size_t llam_ql_prepared_bytes(uint8_t fmt, int N, int K)
+{
+    if (N <= 0 || K <= 0 || (K % 256) != 0)
+        return 0;
+    const size_t T = (size_t)N * (size_t)(K / 256);
+    switch (fmt)
+    {
+    case LLAM_FMT_Q4_K: return T * 144;
+    case LLAM_FMT_Q6_K: return T * 210;
+    case LLAM_FMT_IQ3_S: return T * 112;
+    default: return 0;
+    }
+}
+
+extern "C" bool llam_ql_prepare_weights(uint8_t fmt, const void *d_gguf, void *d_prepared,
+                                        int N, int K, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_prepare_weights";
+    if (fmt != LLAM_FMT_Q4_K && fmt != LLAM_FMT_Q6_K && fmt != LLAM_FMT_IQ3_S)
+        return fail(fn, "unsupported weight format id %d", (int)fmt);
+    if (N < 1 || K < 1 || (K % 256) != 0)
+        return fail(fn, "need N >= 1 and K a positive multiple of 256 (N=%d K=%d)", N, K);
+    if (!d_gguf || !d_prepared)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_prepared))
+        return fail(fn, "d_prepared must be 16-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(d_gguf) & 1u) != 0)
+        return fail(fn, "d_gguf must be 2-byte aligned");
+    if (!set_device(fn, device_id))
+        return false;
+    const size_t T = (size_t)N * (size_t)(K / 256);
+    hipStream_t st = as_stream(stream);
+    if (fmt == LLAM_FMT_Q4_K)
+    {
+        if (d_gguf == d_prepared)
+            return true;
+        if (!aligned16(d_gguf))
+            return fail(fn, "Q4_K source must be 16-byte aligned");
+        hipError_t e = hipMemcpyAsync(d_prepared, d_gguf, T * 144, hipMemcpyDeviceToDevice, st);
+        if (e != hipSuccess)
+            return fail(fn, "hipMemcpyAsync: %s", hipGetErrorString(e));
+        return true;
+    }
+    if (d_gguf == d_prepared)
+        return fail(fn, "in-place preparation is only possible for Q4_K");
+    const size_t items = T * (fmt == LLAM_FMT_Q6_K ? 105 : 56);
+    const size_t grid = (items + 255) / 256;
+    if (grid > 0x7FFFFFFFull)
+        return fail(fn, "matrix too large (N=%d K=%d)", N, K);
+    if (fmt == LLAM_FMT_Q6_K)
+        hipLaunchKernelGGL(prepare_q6k_kernel, dim3((unsigned)grid), dim3(256), 0, st,
+                           static_cast<const uint16_t *>(d_gguf), static_cast<uint16_t *>(d_prepared), T);
+    else
+        hipLaunchKernelGGL(prepare_iq3s_kernel, dim3((unsigned)grid), dim3(256), 0, st,
+                           static_cast<const uint16_t *>(d_gguf), static_cast<uint16_t *>(d_prepared), T);
+    return launched(fn);
+}

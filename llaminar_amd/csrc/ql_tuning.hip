@@ -1,0 +1,16 @@
+// Tuning overrides (for sweeps; production callers never need them).
+#include "ql_host.h"
+
+#include "llaminar_amd/ql_api.h"
+
+namespace llamql
+{
+    namespace
+    {
+        int g_rows_per_wave = 0;
+    }
+    int gemv_rows_per_wave_override() { return g_rows_per_wave; }
+} // namespace llamql
+
+extern "C" void llam_ql_set_gemv_tuning(int rows_per_wave) { llamql::g_rows_per_wave = rows_per_wave; }
+extern "C" void llam_ql_reset_gemv_tuning(void) { llamql::g_rows_per_wave = 0; }

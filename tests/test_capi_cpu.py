@@ -1,0 +1,98 @@
+"""CPU-side checks of the boundary: the built library exports every symbol the
+header declares, the Python binding mirrors it, argument validation fails with
+the documented error text, and without a GPU a valid call fails loudly instead of
+falling back to anything."""
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "llaminar_amd" / "ql_api.h"
+
+
+def declared_symbols():
+    text = HEADER.read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(llam_ql_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from llaminar_amd import capi
+
+    assert capi.LIB_PATH.exists(), "build the library first: python -m llaminar_amd.build"
+    lib = ctypes.CDLL(str(capi.LIB_PATH))
+    names = declared_symbols()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in ql_api.h but not exported"
+    assert set(names) == set(capi.SIGNATURES), "capi.SIGNATURES out of step with ql_api.h"
+
+
+def test_block_layouts_match_header():
+    from llaminar_amd import capi
+
+    text = (ROOT / "include" / "llaminar_amd" / "ql_blocks.h").read_text()
+    for fmt, size in capi.BLOCK_BYTES.items():
+        assert re.search(rf"== {size},", text)
+    assert re.search(r"LLAM_FMT_Q4_K = 5", text) and capi.FMT_Q4_K == 5
+    assert re.search(r"LLAM_FMT_Q6_K = 8", text) and capi.FMT_Q6_K == 8
+    assert re.search(r"LLAM_FMT_IQ3_S = 11", text) and capi.FMT_IQ3_S == 11
+
+
+def test_argument_validation_and_error_text():
+    from llaminar_amd import capi
+
+    lib = capi.load()
+    assert lib.llam_ql_abi_version() == 1
+    buf = np.zeros(4096, np.uint8)
+    p = buf.ctypes.data
+    p16 = p + (-p % 16)
+    assert not lib.llam_ql_quantize_q8_1(p16, p16, 1, 33, 0, None)
+    assert "multiple of 32" in capi.last_error() and "llam_ql_quantize_q8_1" in capi.last_error()
+    assert not lib.llam_ql_gemv(capi.FMT_Q4_K, p16, p16, p16, 9, 4, 256, 4, 0, None)
+    assert "M=9" in capi.last_error()
+    assert not lib.llam_ql_gemv(capi.FMT_Q4_K, p16, p16, p16, 1, 4, 100, 4, 0, None)
+    assert "multiple of 256" in capi.last_error()
+    assert not lib.llam_ql_gemv(77, p16, p16, p16, 1, 4, 256, 4, 0, None)
+    assert "unsupported weight format" in capi.last_error()
+    assert not lib.llam_ql_gemv(capi.FMT_Q4_K, p16 + 4, p16, p16, 1, 4, 256, 4, 0, None)
+    assert "aligned" in capi.last_error()
+    assert not lib.llam_ql_gemv(capi.FMT_Q4_K, p16, p16, p16, 1, 4, 256, 3, 0, None)
+    assert "ldy" in capi.last_error()
+    assert not lib.llam_ql_moe_route(p16, 1, 8, 9, 1, p16, p16, 0, None)
+    assert "top_k" in capi.last_error()
+    assert lib.llam_ql_prepared_bytes(capi.FMT_Q6_K, 4, 512) == 4 * 2 * 210
+    assert lib.llam_ql_prepared_bytes(capi.FMT_IQ3_S, 4, 512) == 4 * 2 * 112
+    assert lib.llam_ql_prepared_bytes(capi.FMT_Q4_K, 4, 100) == 0
+    # empty problems are a successful no-op
+    assert lib.llam_ql_quantize_q8_1(None, None, 0, 0, 0, None)
+
+
+def test_valid_call_without_gpu_fails_loudly():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from llaminar_amd import capi
+
+    lib = capi.load()
+    buf = np.zeros(4096, np.uint8)
+    p16 = buf.ctypes.data + (-buf.ctypes.data % 16)
+    assert not lib.llam_ql_quantize_q8_1(p16, p16, 1, 32, 0, None)
+    assert "no HIP device" in capi.last_error()
+
+
+def test_synthetic_generators_are_seeded_and_in_range():
+    from llaminar_amd import capi, synth
+
+    for fmt in (capi.FMT_Q4_K, capi.FMT_Q6_K, capi.FMT_IQ3_S):
+        a = synth.weights_numpy(fmt, 8, 512, 3)
+        b = synth.weights_numpy(fmt, 8, 512, 3)
+        assert np.array_equal(a, b) and a.shape == (8, 2, capi.BLOCK_BYTES[fmt])
+        off = {capi.FMT_Q4_K: 0, capi.FMT_Q6_K: 208, capi.FMT_IQ3_S: 0}[fmt]
+        d = a[:, :, off:off + 2].copy().view(np.float16).astype(np.float32)
+        assert d.min() >= 0.000999 and d.max() <= 0.02
+    assert synth.gemv_bytes(capi.FMT_Q4_K, 25600, 5120) == 25600 * 20 * 144 + 160 * 36 + 25600 * 4

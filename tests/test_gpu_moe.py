@@ -1,0 +1,194 @@
+"""P4 on the GPU: router, routed gate/up GEMVs from device-resident ids, fused
+SwiGLU + Q8_1, weighted down GEMVs -- each stage against the oracle, then the
+whole expert FFN at the BASELINE MoE shape (hidden 2048, 256+1 experts, top-8,
+intermediate 512, IQ3_S) for 1 and 16 tokens."""
+import numpy as np
+import pytest
+
+from llaminar_amd import synth
+from oracle.binding import FMT_IQ3_S, FMT_Q4_K, FMT_Q6_K
+from tests.helpers import FMTS, TOL, rel_err, sync, upload_q8, upload_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def test_router(capi, dev, oracle):
+    import torch
+
+    rng = np.random.default_rng(12)
+    for T, E, k in ((1, 256, 8), (16, 256, 8), (3, 64, 4), (2, 1000, 6), (1, 8, 8)):
+        logits = rng.standard_normal((T, E)).astype(np.float32)
+        ids, w = capi.moe_route(torch.from_numpy(logits).to(dev), k, True)
+        ids_n, w_n = capi.moe_route(torch.from_numpy(logits).to(dev), k, False)
+        sync()
+        rids, rw, probs = oracle.route(logits, k, True)
+        assert np.array_equal(ids.cpu().numpy(), rids)
+        assert np.allclose(w.cpu().numpy(), rw, rtol=2e-6, atol=1e-8)
+        assert np.array_equal(ids_n.cpu().numpy(), rids)
+        assert np.allclose(w_n.cpu().numpy(), np.take_along_axis(probs, rids, 1), rtol=2e-6, atol=1e-9)
+    tie = torch.zeros(1, 16, device=dev)
+    ids, w = capi.moe_route(tie, 4, True)
+    sync()
+    assert ids.cpu().numpy().tolist() == [[0, 1, 2, 3]]
+    assert np.allclose(w.cpu().numpy(), 0.25)
+
+
+def test_swiglu_quantize(capi, dev, oracle):
+    import torch
+
+    rng = np.random.default_rng(3)
+    g = (rng.standard_normal((9, 512)) * 3).astype(np.float32)
+    u = rng.standard_normal((9, 512)).astype(np.float32)
+    q8, act = capi.swiglu_quantize(torch.from_numpy(g).to(dev), torch.from_numpy(u).to(dev), want_act=True)
+    sync()
+    act_h = act.cpu().numpy()
+    want = oracle.swiglu(g, u)
+    assert np.abs(act_h - want).max() <= 4e-6 * max(1.0, np.abs(want).max())
+    # the quantiser stage is bit-exact on the activations the GPU actually produced
+    assert np.array_equal(q8.cpu().numpy().reshape(9, 16, 36), oracle.quantize(act_h))
+
+
+def _experts(capi, dev, fmt, n_exp, hidden, inter, seed):
+    host, devs = [], []
+    for e in range(n_exp):
+        g = synth.weights_numpy(fmt, inter, hidden, seed + 3 * e)
+        u = synth.weights_numpy(fmt, inter, hidden, seed + 3 * e + 1)
+        d = synth.weights_numpy(fmt, hidden, inter, seed + 3 * e + 2)
+        host.append((g, u, d))
+        devs.append(tuple(upload_weights(capi, dev, fmt, w) for w in (g, u, d)))
+    return host, devs, capi.expert_table(devs, dev)
+
+
+@pytest.mark.parametrize("fmt", list(FMTS.values()), ids=list(FMTS))
+def test_stages_small(capi, dev, oracle, fmt):
+    """Every stage against the oracle on a 6-expert toy (hidden 512, inter 256, top-3, 4 tokens)."""
+    import torch
+
+    n_exp, hidden, inter, k, T = 6, 512, 256, 3, 4
+    host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 40)
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, n_exp)).astype(np.float32)
+    ids, w = capi.moe_route(torch.from_numpy(logits).to(dev), k, True)
+    qd = capi.quantize_q8_1(torch.from_numpy(x).to(dev))
+    gate, up = capi.moe_gate_up(fmt, table, n_exp, ids, qd, T, k, hidden, inter)
+    q8a, act = capi.swiglu_quantize(gate, up, want_act=True)
+    out = torch.full((T, hidden), float("nan"), device=dev)
+    capi.moe_down(fmt, table, n_exp, ids, w, q8a, out, T, k, hidden, inter, accumulate=False)
+    sync()
+    rids, rw, _ = oracle.route(logits, k, True)
+    assert np.array_equal(ids.cpu().numpy(), rids)
+    q8 = oracle.quantize(x)
+    gate_h, up_h, act_h = gate.cpu().numpy(), up.cpu().numpy(), act.cpu().numpy()
+    q8a_h = q8a.cpu().numpy().reshape(T * k, inter // 32, 36)
+    want_out = np.zeros((T, hidden), np.float64)
+    for t in range(T):
+        for s in range(k):
+            e = int(rids[t, s])
+            g_ref = oracle.gemm(fmt, host[e][0], hidden, q8[t:t + 1])[0]
+            u_ref = oracle.gemm(fmt, host[e][1], hidden, q8[t:t + 1])[0]
+            assert rel_err(gate_h[t * k + s], g_ref) <= TOL[fmt] * 1e-2
+            assert rel_err(up_h[t * k + s], u_ref) <= TOL[fmt] * 1e-2
+            # down: same Q8_1 input on both sides (the GPU's), so the stage is checked tightly
+            d_ref = oracle.gemm(fmt, host[e][2], inter, q8a_h[t * k + s][None])[0]
+            want_out[t] += float(rw[t, s]) * d_ref
+    assert rel_err(out.cpu().numpy(), want_out.astype(np.float32)) <= TOL[fmt] * 1e-2
+    # accumulate mode adds onto the existing output
+    base = torch.ones((T, hidden), device=dev)
+    capi.moe_down(fmt, table, n_exp, ids, w, q8a, base, T, k, hidden, inter, accumulate=True)
+    sync()
+    assert rel_err(base.cpu().numpy() - 1.0, want_out.astype(np.float32)) <= 1e-5
+
+
+def test_out_of_range_expert_ids_are_skipped(capi, dev, oracle):
+    import torch
+
+    fmt, n_exp, hidden, inter, k, T = FMT_Q4_K, 2, 256, 256, 2, 1
+    host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 90)
+    x = synth.activations_numpy(T, hidden, 1)
+    qd = capi.quantize_q8_1(torch.from_numpy(x).to(dev))
+    ids = torch.tensor([[1, 7]], dtype=torch.int32, device=dev)   # 7 is not a valid expert
+    gate, up = capi.moe_gate_up(fmt, table, n_exp, ids, qd, T, k, hidden, inter)
+    gate2 = torch.full_like(gate, 5.0)
+    up2 = torch.full_like(up, 5.0)
+    lib = capi.load()
+    assert lib.llam_ql_moe_gate_up(fmt, table.data_ptr(), n_exp, ids.data_ptr(), qd.data_ptr(), gate2.data_ptr(),
+                                   up2.data_ptr(), T, k, hidden, inter, 0, None)
+    sync()
+    assert (gate2[1] == 5.0).all() and (up2[1] == 5.0).all()      # untouched
+    q8 = oracle.quantize(x)
+    assert rel_err(gate2[0].cpu().numpy(), oracle.gemm(fmt, host[1][0], hidden, q8)[0]) <= 1e-5
+
+
+@pytest.mark.parametrize("T", [1, 16])
+def test_expert_ffn_baseline_shape(capi, dev, oracle, T):
+    """Config 4: hidden 2048, 256 routed + 1 shared expert, top-8, intermediate 512, IQ3_S."""
+    import torch
+
+    fmt, n_exp, hidden, inter, k = FMT_IQ3_S, 256, 2048, 512, 8
+    rng = np.random.default_rng(100 + T)
+    # one big seeded slab per matrix kind, generated on the device; expert e is a slice
+    def slab(rows, cols, seed):
+        raw = synth.weights_torch(fmt, (n_exp + 1) * rows, cols, seed, dev)
+        per = rows * (cols // 256) * 110
+        return raw, per
+    graw, gper = slab(inter, hidden, 1)
+    uraw, uper = slab(inter, hidden, 2)
+    draw, dper = slab(hidden, inter, 3)
+    devs = []
+    for e in range(n_exp + 1):
+        devs.append((capi.prepare_weights(fmt, graw[e * gper:(e + 1) * gper].clone(), inter, hidden),
+                     capi.prepare_weights(fmt, uraw[e * uper:(e + 1) * uper].clone(), inter, hidden),
+                     capi.prepare_weights(fmt, draw[e * dper:(e + 1) * dper].clone(), hidden, inter)))
+    table = capi.expert_table(devs, dev)
+    x = rng.standard_normal((T, hidden)).astype(np.float32)
+    logits = rng.standard_normal((T, n_exp)).astype(np.float32)
+    xd = torch.from_numpy(x).to(dev)
+
+    ids, w = capi.moe_route(torch.from_numpy(logits).to(dev), k, True)
+    qd = capi.quantize_q8_1(xd)
+    gate, up = capi.moe_gate_up(fmt, table, n_exp + 1, ids, qd, T, k, hidden, inter)
+    q8a = capi.swiglu_quantize(gate, up)
+    out = torch.empty((T, hidden), device=dev)
+    capi.moe_down(fmt, table, n_exp + 1, ids, w, q8a, out, T, k, hidden, inter, accumulate=False)
+    # shared expert (id n_exp) for every token with weight 1, added ungated
+    sid = torch.full((T, 1), n_exp, dtype=torch.int32, device=dev)
+    sw = torch.ones((T, 1), device=dev)
+    sg, su = capi.moe_gate_up(fmt, table, n_exp + 1, sid, qd, T, 1, hidden, inter)
+    sq = capi.swiglu_quantize(sg, su)
+    capi.moe_down(fmt, table, n_exp + 1, sid, sw, sq, out, T, 1, hidden, inter, accumulate=True)
+    sync()
+
+    # oracle: the same chain on the CPU (own SwiGLU, own quantisation of it)
+    rids, rw, _ = oracle.route(logits, k, True)
+    assert np.array_equal(ids.cpu().numpy(), rids)
+    q8 = oracle.quantize(x)
+    gh, uh, dh = graw.cpu().numpy(), uraw.cpu().numpy(), draw.cpu().numpy()
+    want = np.zeros((T, hidden), np.float32)
+    for t in range(T):
+        for e, wt in list(zip(rids[t].tolist(), rw[t].tolist())) + [(n_exp, 1.0)]:
+            g = oracle.gemm(fmt, gh[e * gper:(e + 1) * gper], hidden, q8[t:t + 1])[0]
+            u = oracle.gemm(fmt, uh[e * uper:(e + 1) * uper], hidden, q8[t:t + 1])[0]
+            a = oracle.swiglu(g, u)
+            d = oracle.gemm(fmt, dh[e * dper:(e + 1) * dper], inter, oracle.quantize(a[None]))[0]
+            want[t] += np.float32(wt) * d
+    # chained end to end: the SwiGLU differs by ulps between CPU and GPU, which can flip a
+    # Q8_1 rounding in the down input; the IQ3_S output contract (1e-2) holds with margin
+    assert rel_err(out.cpu().numpy(), want) <= 1e-3
+
+
+def test_shared_expert_gate(capi, dev):
+    import torch
+
+    rng = np.random.default_rng(5)
+    T, D = 3, 2048
+    out = rng.standard_normal((T, D)).astype(np.float32)
+    sh = rng.standard_normal((T, D)).astype(np.float32)
+    h = rng.standard_normal((T, D)).astype(np.float32)
+    gi = (rng.standard_normal(D) * 0.05).astype(np.float32)
+    od = torch.from_numpy(out.copy()).to(dev)
+    capi.shared_expert_add(od, torch.from_numpy(sh).to(dev), torch.from_numpy(h).to(dev), torch.from_numpy(gi).to(dev))
+    sync()
+    gate = 1.0 / (1.0 + np.exp(-(h.astype(np.float64) @ gi.astype(np.float64))))
+    want = out + gate[:, None] * sh
+    assert np.allclose(od.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
