@@ -71,6 +71,11 @@ def load() -> ctypes.CDLL:
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `python -m llaminar_amd.build` "
             "(hipcc --offload-arch=gfx950).  There is no CPU fallback.")
+    # PyTorch ships its own copy of the HIP runtime under the same soname as the
+    # system one.  A process must use exactly one of them: import torch first so the
+    # dynamic loader binds this library to the runtime torch's allocator uses.
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(str(LIB_PATH))
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the library does not export it
