@@ -51,8 +51,10 @@ int llam_ql_abi_version(void);
 
 /* Tuning overrides for sweeps (reference: rocmGemv_native_vnni_set_tuning_overrides /
  * ..._reset_tuning_overrides, ROCmGemvKernel_native_VNNI.hip:182-196).
- * rows_per_wave <= 0 restores the built-in choice.  Not thread-safe. */
-void llam_ql_set_gemv_tuning(int rows_per_wave);
+ * rows_per_wave: row batches one wavefront walks; unroll: 1..4 forces the chunked
+ * kernel with that many load batches in flight instead of the row-streaming
+ * kernel.  Values <= 0 restore the built-in choice.  Not thread-safe. */
+void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll);
 void llam_ql_reset_gemv_tuning(void);
 
 /* ---- P1: activation quantiser --------------------------------------------------

@@ -126,7 +126,12 @@ namespace llamql
 
     // The workgroup-level GEMV: workgroup `wg` of the launch described by `a`.
     // Requires blockDim.x == GEMV_WAVES*WAVE and the dynamic LDS of gemv_lds_bytes().
-    template <class F, int M, bool DUMP>
+    //
+    // U = iterations (8 super-blocks each, or G when rows are short) whose loads are
+    // issued together; the next chunk -- of this row or of the wavefront's next row --
+    // is already in flight while the current one is decoded, so a wavefront keeps
+    // 2*U global loads per lane outstanding.
+    template <class F, int M, int U, bool DUMP>
     __device__ __forceinline__ void gemv_body(const GemvArgs &a, long wg, uint32_t *lds)
     {
         const int nkb = a.nsb * 8;
@@ -134,11 +139,6 @@ namespace llamql
         float *ad = reinterpret_cast<float *>(aq + M * nkb * 8); // M * nkb
         float *asd = ad + M * nkb;                               // M * nkb
         void *tab = asd + M * nkb;                               // F::TABLE_BYTES
-
-        if (F::TABLE_BYTES > 0)
-            F::stage_tables(tab);
-        stage_q8<F, M>(a.q8, a.SB * 8, a.sb0 * 8, nkb, aq, ad, asd);
-        __syncthreads();
 
         const int lane = threadIdx.x & (WAVE - 1);
         const int wave = threadIdx.x >> 6;
@@ -151,6 +151,28 @@ namespace llamql
         const int s_first = grp & (G - 1);    // first super-block of this lane
         const int rows_per_wg = GEMV_WAVES * R * a.rows_per_wave;
         const long wg_row0 = wg * rows_per_wg;
+        const int chunk_sb = G * U;                                // super-blocks per chunk and row
+        const int nchunks = (a.nsb + chunk_sb - 1) / chunk_sb;
+
+        // Issue the first chunk's weight loads before touching the activations, so HBM
+        // latency overlaps the LDS staging.
+        typename F::Raw buf[U];
+        {
+            const long row = wg_row0 + (long)wave * R + rsub;
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+            {
+                const int s = s_first + u * G;
+                buf[u] = typename F::Raw{};
+                if (row < a.N && s < a.nsb)
+                    buf[u] = F::load(a, row, a.sb0 + s, c);
+            }
+        }
+
+        if (F::TABLE_BYTES > 0)
+            F::stage_tables(tab);
+        stage_q8<F, M>(a.q8, a.SB * 8, a.sb0 * 8, nkb, aq, ad, asd);
+        __syncthreads();
 
         for (int r = 0; r < a.rows_per_wave; ++r)
         {
@@ -165,52 +187,71 @@ namespace llamql
             for (int m = 0; m < M; ++m)
                 acc[m] = 0.0f;
 
-            int s = row_ok ? s_first : a.nsb;
-            typename F::Raw next = {};
-            if (s < a.nsb)
-                next = F::load(a, row, a.sb0 + s, c);
-            for (; s < a.nsb; s += G)
+            for (int ch = 0; ch < nchunks; ++ch)
             {
-                const typename F::Raw cur = next;
-                if (s + G < a.nsb)
-                    next = F::load(a, row, a.sb0 + s + G, c);
-
-                v4i w0, w1;
-                int j;
-                float bscale, bmin;
-                F::decode(cur, c, w0, w1, j, bscale, bmin, tab);
-
-                const int unit = s * 8 + c; // LDS unit of this lane
-                const int kb = s * 8 + j;   // block this lane finishes (slice-relative)
+                typename F::Raw cur[U];
 #pragma unroll
-                for (int m = 0; m < M; ++m)
+                for (int u = 0; u < U; ++u)
+                    cur[u] = buf[u];
+
+                // prefetch the next chunk: same row, or the first chunk of the next row
                 {
-                    const v4i *ap = reinterpret_cast<const v4i *>(aq + (size_t)m * nkb * 8 + (size_t)unit * 8);
-                    const v4i a0 = ap[0];
-                    const v4i a1 = ap[1];
-                    int idot;
-                    if (F::PAIR)
+                    const bool same_row = (ch + 1 < nchunks);
+                    const long nrow = same_row ? row : row + (long)GEMV_WAVES * R;
+                    const int nch = same_row ? ch + 1 : 0;
+                    const bool more = same_row || (r + 1 < a.rows_per_wave);
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
                     {
-                        const int p0 = dot16(a0, w0, 0);
-                        const int p1 = dot16(a1, w1, 0);
-                        // even lane finishes the w0 sub-block, odd lane the w1 sub-block
-                        const int got = dpp_i32<DPP_QUAD_XOR1>(odd ? p0 : p1);
-                        idot = (odd ? p1 : p0) + got;
+                        const int s = s_first + (nch * U + u) * G;
+                        if (more && nrow < a.N && s < a.nsb)
+                            buf[u] = F::load(a, nrow, a.sb0 + s, c);
                     }
-                    else
+                }
+
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                {
+                    const int s = s_first + (ch * U + u) * G;
+                    if (!row_ok || s >= a.nsb)
+                        continue;
+                    v4i w0, w1;
+                    int j;
+                    float bscale, bmin;
+                    F::decode(cur[u], c, w0, w1, j, bscale, bmin, tab);
+
+                    const int unit = s * 8 + c; // LDS unit of this lane
+                    const int kb = s * 8 + j;   // block this lane finishes (slice-relative)
+#pragma unroll
+                    for (int m = 0; m < M; ++m)
                     {
-                        idot = dot16(a1, w1, dot16(a0, w0, 0));
+                        const v4i *ap = reinterpret_cast<const v4i *>(aq + (size_t)m * nkb * 8 + (size_t)unit * 8);
+                        const v4i a0 = ap[0];
+                        const v4i a1 = ap[1];
+                        int idot;
+                        if (F::PAIR)
+                        {
+                            const int p0 = dot16(a0, w0, 0);
+                            const int p1 = dot16(a1, w1, 0);
+                            // even lane finishes the w0 sub-block, odd lane the w1 sub-block
+                            const int got = dpp_i32<DPP_QUAD_XOR1>(odd ? p0 : p1);
+                            idot = (odd ? p1 : p0) + got;
+                        }
+                        else
+                        {
+                            idot = dot16(a1, w1, dot16(a0, w0, 0));
+                        }
+                        if (DUMP)
+                        {
+                            const long rr = row - a.row0;
+                            if (rr >= 0 && rr < a.nrows)
+                                a.sums[((size_t)m * a.nrows + rr) * ((size_t)a.SB * 8) + (size_t)(a.sb0 + s) * 8 + j] = idot;
+                        }
+                        const float cs = ad[m * nkb + kb] * bscale;
+                        acc[m] = fmaf((float)idot, cs, acc[m]);
+                        if (F::HAS_MIN)
+                            acc[m] = fmaf(asd[m * nkb + kb], bmin, acc[m]);
                     }
-                    if (DUMP)
-                    {
-                        const long rr = row - a.row0;
-                        if (rr >= 0 && rr < a.nrows)
-                            a.sums[((size_t)m * a.nrows + rr) * ((size_t)a.SB * 8) + (size_t)(a.sb0 + s) * 8 + j] = idot;
-                    }
-                    const float cs = ad[m * nkb + kb] * bscale;
-                    acc[m] = fmaf((float)idot, cs, acc[m]);
-                    if (F::HAS_MIN)
-                        acc[m] = fmaf(asd[m * nkb + kb], bmin, acc[m]);
                 }
             }
 
@@ -231,27 +272,36 @@ namespace llamql
         }
     }
 
-    template <class F, int M, bool DUMP>
+    template <class F, int M, int U, bool DUMP>
     __global__ void __launch_bounds__(GEMV_WAVES *WAVE) gemv_kernel(const GemvArgs a)
     {
         extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
-        gemv_body<F, M, DUMP>(a, (long)blockIdx.x, lds);
+        gemv_body<F, M, U, DUMP>(a, (long)blockIdx.x, lds);
     }
 
-    template <class F, bool DUMP>
-    inline void gemv_launch_m(int M, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
+    // The generic kernel is only instantiated with U = 1: it serves short rows, the
+    // block-sum dump and the MoE kernels; long rows go through gemv_fast.h.
+    template <class F, int M>
+    inline void gemv_launch_u(bool dump, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
     {
         dim3 block(GEMV_WAVES * WAVE);
+        if (dump)
+            hipLaunchKernelGGL((gemv_kernel<F, M, 1, true>), grid, block, lds, st, a);
+        else
+            hipLaunchKernelGGL((gemv_kernel<F, M, 1, false>), grid, block, lds, st, a);
+    }
+
+    // M is one of 1,2,3,4,8 (other batch sizes are split by the caller).
+    template <class F>
+    inline void gemv_launch_m(int M, bool dump, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
+    {
         switch (M)
         {
-        case 1: hipLaunchKernelGGL((gemv_kernel<F, 1, DUMP>), grid, block, lds, st, a); break;
-        case 2: hipLaunchKernelGGL((gemv_kernel<F, 2, DUMP>), grid, block, lds, st, a); break;
-        case 3: hipLaunchKernelGGL((gemv_kernel<F, 3, DUMP>), grid, block, lds, st, a); break;
-        case 4: hipLaunchKernelGGL((gemv_kernel<F, 4, DUMP>), grid, block, lds, st, a); break;
-        case 5: hipLaunchKernelGGL((gemv_kernel<F, 5, DUMP>), grid, block, lds, st, a); break;
-        case 6: hipLaunchKernelGGL((gemv_kernel<F, 6, DUMP>), grid, block, lds, st, a); break;
-        case 7: hipLaunchKernelGGL((gemv_kernel<F, 7, DUMP>), grid, block, lds, st, a); break;
-        default: hipLaunchKernelGGL((gemv_kernel<F, 8, DUMP>), grid, block, lds, st, a); break;
+        case 1: gemv_launch_u<F, 1>(dump, grid, lds, st, a); break;
+        case 2: gemv_launch_u<F, 2>(dump, grid, lds, st, a); break;
+        case 3: gemv_launch_u<F, 3>(dump, grid, lds, st, a); break;
+        case 4: gemv_launch_u<F, 4>(dump, grid, lds, st, a); break;
+        default: gemv_launch_u<F, 8>(dump, grid, lds, st, a); break;
         }
     }
 
@@ -263,67 +313,4 @@ namespace llamql
         return (size_t)M * nsb * GEMV_LDS_PER_SB + F::TABLE_BYTES;
     }
 
-    // Shared host launcher.  Arguments are validated by the callers; the device
-    // is current.
-    template <class F>
-    bool gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                     int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
-    {
-        const int SB = K / 256;
-        const bool dump = d_sums != nullptr;
-        // K slices keep the staged activations (+ tables) within 64 KiB of LDS.
-        int slice = (64 * 1024 - F::TABLE_BYTES) / (M * GEMV_LDS_PER_SB);
-        if (slice > SB)
-            slice = SB;
-        if (slice < 1)
-            return fail(fn, "activation rows do not fit LDS (M=%d)", M);
-
-        // short rows: several rows share a wavefront (G groups of 8 lanes per row)
-        int gshift = 3;
-        while (gshift > 0 && (1 << (gshift - 1)) >= slice)
-            --gshift;
-        const int R = 8 >> gshift;
-
-        int rpw = gemv_rows_per_wave_override();
-        if (rpw <= 0)
-        {
-            // enough workgroups for every CU several times over, while amortising the LDS staging
-            const long target_wgs = (long)cu_count(device_id) * 8;
-            rpw = (int)((long)N / (target_wgs * GEMV_WAVES * R));
-            if (rpw < 1)
-                rpw = 1;
-            if (rpw > 8)
-                rpw = 8;
-        }
-        const int rows_per_wg = GEMV_WAVES * R * rpw;
-        const long grid = ((long)N + rows_per_wg - 1) / rows_per_wg;
-
-        for (int sb0 = 0; sb0 < SB; sb0 += slice)
-        {
-            GemvArgs a;
-            a.w = d_w;
-            a.q8 = static_cast<const uint32_t *>(d_q8);
-            a.y = d_y;
-            a.sums = d_sums;
-            a.ldy = ldy;
-            a.N = N;
-            a.SB = SB;
-            a.sb0 = sb0;
-            a.nsb = (SB - sb0 < slice) ? (SB - sb0) : slice;
-            a.rows_per_wave = rpw;
-            a.gshift = gshift;
-            a.accumulate = sb0 > 0;
-            a.out_scale = 1.0f;
-            a.row0 = row0;
-            a.nrows = nrows;
-            const size_t lds = gemv_lds_bytes<F>(M, a.nsb);
-            if (dump)
-                gemv_launch_m<F, true>(M, dim3((unsigned)grid), lds, st, a);
-            else
-                gemv_launch_m<F, false>(M, dim3((unsigned)grid), lds, st, a);
-            if (!launched(fn))
-                return false;
-        }
-        return true;
-    }
 } // namespace llamql

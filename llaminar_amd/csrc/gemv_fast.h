@@ -1,0 +1,435 @@
+// Full-row decode GEMV (gfx950): the streaming kernel used whenever a weight row
+// spans at least five super-blocks, i.e. for every dense-layer projection.
+//
+// Same arithmetic and lane roles as the generic skeleton in gemv_core.h; what
+// differs is how the work is fed:
+//   - one wavefront per row at a time (8 lanes per super-block, 8 super-blocks per
+//     load batch), U load batches issued together, and the next U -- of this row
+//     or of the wavefront's next row -- already in flight while the current ones
+//     are decoded, so a wavefront keeps 2*U x (16..52) bytes per lane outstanding;
+//   - per-lane weight pointers advanced by constants (immediate offsets inside a
+//     chunk), per-lane bit-field constants for the header decode, no per-element
+//     predicates on full chunks;
+//   - the first chunk's loads are issued BEFORE the activations are staged in LDS,
+//     so HBM latency overlaps the staging.
+//
+// LDS: aq [M][K/32 units of 32 B]  int8 quants laid out per lane (see gemv_core.h)
+//      ads[M][K/32] float2 = { f32(d), float(sum_qs)*f32(d) }
+#pragma once
+
+#include "gemv_core.h"
+
+namespace llamql
+{
+    // Stage nkb Q8_1 blocks of each of M activation rows: one thread per block.
+    template <class F, int M>
+    __device__ __forceinline__ void stage_q8_blocks(const uint32_t *__restrict__ q8, int KB_total, int kb0, int nkb,
+                                                    uint32_t *aq, float2 *ads)
+    {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+        {
+            for (int kb = threadIdx.x; kb < nkb; kb += blockDim.x)
+            {
+                const uint32_t *src = q8 + ((size_t)m * KB_total + kb0 + kb) * 9;
+                uint32_t v[9];
+#pragma unroll
+                for (int i = 0; i < 9; ++i)
+                    v[i] = src[i];
+                const float d = h2f((uint16_t)(v[0] & 0xFFFFu));
+                ads[m * nkb + kb] = make_float2(d, (float)(int16_t)(v[0] >> 16) * d);
+                int c0, p0, c1, p1;
+                F::unit_of(kb & 7, 0, c0, p0);
+                F::unit_of(kb & 7, 4, c1, p1);
+                uint32_t *base = aq + (size_t)m * nkb * 8 + (size_t)(kb >> 3) * 64;
+                *reinterpret_cast<uint4 *>(base + c0 * 8 + p0 * 4) = make_uint4(v[1], v[2], v[3], v[4]);
+                *reinterpret_cast<uint4 *>(base + c1 * 8 + p1 * 4) = make_uint4(v[5], v[6], v[7], v[8]);
+            }
+        }
+    }
+
+    template <class F, int M, int U, bool PARTIAL>
+    __device__ __forceinline__ void gemv_fast_chunk(const typename F::Raw (&cur)[U], const typename F::Lane &lc,
+                                                    bool odd, int s_base, int nsb, const uint8_t *aq_lane,
+                                                    const uint8_t *ads_lane, int m_stride_aq, int m_stride_ads,
+                                                    const void *tab, float (&acc)[M])
+    {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+        {
+            if (PARTIAL && s_base + 8 * u >= nsb)
+                continue;
+            v4i w0, w1;
+            float bscale, bmin;
+            F::decode2(cur[u], lc, w0, w1, bscale, bmin, tab);
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+            {
+                const v4i *ap = reinterpret_cast<const v4i *>(aq_lane + m * m_stride_aq + u * 2048);
+                const v4i a0 = ap[0];
+                const v4i a1 = ap[1];
+                const float2 sd = *reinterpret_cast<const float2 *>(ads_lane + m * m_stride_ads + u * 512);
+                int idot;
+                if (F::PAIR)
+                {
+                    const int p0 = dot16(a0, w0, 0);
+                    const int p1 = dot16(a1, w1, 0);
+                    const int got = dpp_i32<DPP_QUAD_XOR1>(odd ? p0 : p1);
+                    idot = (odd ? p1 : p0) + got;
+                }
+                else
+                {
+                    idot = dot16(a1, w1, dot16(a0, w0, 0));
+                }
+                const float cs = sd.x * bscale;
+                acc[m] = fmaf((float)idot, cs, acc[m]);
+                if (F::HAS_MIN)
+                    acc[m] = fmaf(sd.y, bmin, acc[m]);
+            }
+        }
+    }
+
+    template <class F, int M, int U>
+    __global__ void __launch_bounds__(GEMV_WAVES *WAVE) gemv_fast_kernel(const GemvArgs a)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+        const int nkb = a.nsb * 8;
+        uint32_t *aq = lds;                                          // M * nkb * 8 dwords
+        float2 *ads = reinterpret_cast<float2 *>(aq + M * nkb * 8);  // M * nkb
+        void *tab = ads + M * nkb;                                   // F::TABLE_BYTES
+
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = threadIdx.x >> 6;
+        const int c = lane & 7;
+        const int grp = lane >> 3;
+        const bool odd = (c & 1) != 0;
+        const typename F::Lane lc = F::lane_consts(c);
+
+        const long wg_row0 = (long)blockIdx.x * (GEMV_WAVES * a.rows_per_wave);
+        const int chunk_sb = 8 * U;
+        const int nfull = a.nsb / chunk_sb;
+        const int nchunks = (a.nsb + chunk_sb - 1) / chunk_sb;
+
+        // weight loads of the first chunk go out before anything else
+        long row = wg_row0 + wave;
+        const bool any_row = row < a.N;
+        typename F::Ptr p = F::ptr(a, any_row ? row : (long)a.N - 1, a.sb0 + grp, c);
+        typename F::Raw buf[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+        {
+            buf[u] = typename F::Raw{};
+            if (any_row && grp + 8 * u < a.nsb)
+                buf[u] = F::load_at(p, 8 * u);
+        }
+
+        if (F::TABLE_BYTES > 0)
+            F::stage_tables(tab);
+        stage_q8_blocks<F, M>(a.q8, a.SB * 8, a.sb0 * 8, nkb, aq, ads);
+        __syncthreads();
+
+        const uint8_t *aq_lane0 = reinterpret_cast<const uint8_t *>(aq) + (grp * 8 + c) * 32;
+        const uint8_t *ads_lane0 = reinterpret_cast<const uint8_t *>(ads) + (grp * 8 + lc.j) * 8;
+        const int m_stride_aq = nkb * 32;
+        const int m_stride_ads = nkb * 8;
+
+        for (int r = 0; r < a.rows_per_wave; ++r, row += GEMV_WAVES)
+        {
+            if (row >= a.N)
+                break;
+            float acc[M];
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+                acc[m] = 0.0f;
+
+            for (int ch = 0; ch < nchunks; ++ch)
+            {
+                typename F::Raw cur[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    cur[u] = buf[u];
+
+                // ---- prefetch: next chunk of this row, else first chunk of the next row
+                const bool last = (ch + 1 == nchunks);
+                int next_base; // first super-block (of this lane) in the chunk being fetched
+                bool more;
+                if (!last)
+                {
+                    F::advance(p, chunk_sb);
+                    next_base = grp + (ch + 1) * chunk_sb;
+                    more = true;
+                }
+                else
+                {
+                    F::advance(p, GEMV_WAVES * a.SB - ch * chunk_sb);
+                    next_base = grp;
+                    more = (r + 1 < a.rows_per_wave) && (row + GEMV_WAVES < a.N);
+                }
+                if (more)
+                {
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        if (next_base + 8 * u < a.nsb)
+                            buf[u] = F::load_at(p, 8 * u);
+                }
+
+                // ---- decode + dot
+                const uint8_t *aql = aq_lane0 + ch * (U * 2048);
+                const uint8_t *adl = ads_lane0 + ch * (U * 512);
+                if (ch < nfull)
+                    gemv_fast_chunk<F, M, U, false>(cur, lc, odd, grp + ch * chunk_sb, a.nsb, aql, adl, m_stride_aq,
+                                                    m_stride_ads, tab, acc);
+                else
+                    gemv_fast_chunk<F, M, U, true>(cur, lc, odd, grp + ch * chunk_sb, a.nsb, aql, adl, m_stride_aq,
+                                                   m_stride_ads, tab, acc);
+            }
+
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+            {
+                const float total = wave_sum(acc[m]);
+                if (lane == 0)
+                {
+                    float *dst = a.y + (size_t)m * a.ldy + row;
+                    const float v = a.out_scale * total;
+                    *dst = a.accumulate ? (*dst + v) : v;
+                }
+            }
+        }
+    }
+
+    template <class F, int M>
+    inline void gemv_fast_launch_u(int U, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
+    {
+        dim3 block(GEMV_WAVES * WAVE);
+        switch (U)
+        {
+        case 1: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1>), grid, block, lds, st, a); break;
+        case 2: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 2>), grid, block, lds, st, a); break;
+        case 3: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 3>), grid, block, lds, st, a); break;
+        default: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 4>), grid, block, lds, st, a); break;
+        }
+    }
+
+    // M is one of 1,2,3,4,8.
+    template <class F>
+    inline void gemv_fast_launch(int M, int U, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
+    {
+        switch (M)
+        {
+        case 1: gemv_fast_launch_u<F, 1>(U, grid, lds, st, a); break;
+        case 2: gemv_fast_launch_u<F, 2>(U, grid, lds, st, a); break;
+        case 3: gemv_fast_launch_u<F, 3>(U, grid, lds, st, a); break;
+        case 4: gemv_fast_launch_u<F, 4>(U, grid, lds, st, a); break;
+        default: gemv_fast_launch_u<F, 8>(U, grid, lds, st, a); break;
+        }
+    }
+
+    int gemv_unroll_override();
+    bool gemv_stream_enabled();
+
+    // defined in gemv_stream.h
+    template <class F>
+    inline void gemv_stream_launch(int M, int RP, int waves, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a);
+    int gemv_stream_max_waves();
+
+    // Workgroup shape for `npass` passes: one workgroup per compute unit when there is
+    // enough work, `waves` wavefronts of `ppw` passes each, chosen to pad the per-CU
+    // share as little as possible (every CU then finishes at the same time).
+    struct StreamShape
+    {
+        int waves, ppw;
+        long grid;
+    };
+    inline StreamShape gemv_stream_shape(long npass, int cus, int max_waves)
+    {
+        StreamShape sh;
+        const long per_cu = (npass + cus - 1) / cus;
+        int ppw_override = gemv_rows_per_wave_override();
+        long best_pad = 1L << 60;
+        sh.waves = 4;
+        sh.ppw = 1;
+        for (int w = max_waves; w >= 2; --w)
+        {
+            long ppw = (per_cu + w - 1) / w;
+            if (ppw_override > 0)
+                ppw = ppw_override;
+            if (ppw > 64)
+                continue;
+            const long cap = (long)w * ppw;
+            if (cap < per_cu && ppw_override <= 0)
+                continue;
+            // padding, with a mild preference for at least 8 wavefronts
+            long pad = (cap >= per_cu ? cap - per_cu : 0) * 16 + (w < 8 ? (8 - w) : 0);
+            if (pad < best_pad)
+            {
+                best_pad = pad;
+                sh.waves = w;
+                sh.ppw = (int)ppw;
+            }
+        }
+        const long per_wg = (long)sh.waves * sh.ppw;
+        sh.grid = (npass + per_wg - 1) / per_wg;
+        return sh;
+    }
+
+
+    // Launch shape for N rows of nsb super-blocks (one LDS slice) on a device with
+    // `cus` compute units.  Rows are dealt to workgroups so that every compute unit
+    // receives (nearly) the same number of rows in a single round of workgroups.
+    struct GemvShape
+    {
+        int gshift, rpw, U;
+        long grid;
+    };
+
+    inline GemvShape gemv_shape(long N, int nsb, int cus)
+    {
+        GemvShape sh;
+        sh.gshift = 3;
+        while (sh.gshift > 0 && (1 << (sh.gshift - 1)) >= nsb)
+            --sh.gshift;
+        const int G = 1 << sh.gshift;
+        const int R = 8 >> sh.gshift;
+        const int iters = (nsb + G - 1) / G; // wavefront iterations per row
+        // unroll: whole row when short, else the depth that wastes the fewest slots
+        sh.U = iters;
+        if (iters > 4)
+        {
+            int best = 4, waste = (4 - iters % 4) % 4;
+            for (int u = 3; u >= 2; --u)
+            {
+                const int w = (u - iters % u) % u;
+                if (w < waste)
+                {
+                    best = u;
+                    waste = w;
+                }
+            }
+            sh.U = best;
+        }
+        if (gemv_unroll_override() > 0)
+            sh.U = gemv_unroll_override() > 4 ? 4 : gemv_unroll_override();
+
+        // rows (in units of R) each compute unit must cover
+        const long units = (N + R - 1) / R;
+        const long per_cu = (units + cus - 1) / cus;
+        int rpw = gemv_rows_per_wave_override();
+        if (rpw <= 0)
+        {
+            // candidates: 1..8 row batches per wavefront; cost = padded work per CU, with
+            // at least 16 wavefronts per CU when there is enough work, at most 32
+            double best_cost = 1e30;
+            rpw = 1;
+            for (int cand = 1; cand <= 8; ++cand)
+            {
+                const long wg_units = (long)GEMV_WAVES * cand;
+                const long wgs_per_cu = (per_cu + wg_units - 1) / wg_units;
+                double cost = (double)(wgs_per_cu * wg_units) / (double)per_cu;
+                const long waves = wgs_per_cu * GEMV_WAVES;
+                if (waves > 32)
+                    cost *= 1.0 + 0.05 * (double)((waves + 31) / 32 - 1); // extra rounds: restaging + tail
+                if (waves < 16 && per_cu >= 16)
+                    cost *= 1.25; // too little memory-level parallelism
+                if (cost < best_cost - 1e-9)
+                {
+                    best_cost = cost;
+                    rpw = cand;
+                }
+            }
+        }
+        sh.rpw = rpw;
+        const long rows_per_wg = (long)GEMV_WAVES * R * rpw;
+        sh.grid = (N + rows_per_wg - 1) / rows_per_wg;
+        return sh;
+    }
+
+    // Shared host launcher.  Arguments are validated by the callers; the device
+    // is current.  M is 1..8.
+    template <class F>
+    bool gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
+                     int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
+    {
+        const int SB = K / 256;
+        const bool dump = d_sums != nullptr;
+        // batch sizes without a dedicated kernel are run as 4 + (M-4)
+        if (M > 4 && M < 8)
+        {
+            if (!gemv_launch<F>(fn, d_w, d_q8, d_y, d_sums, 4, N, K, ldy, row0, nrows, device_id, st))
+                return false;
+            const uint8_t *q8b = static_cast<const uint8_t *>(d_q8) + (size_t)4 * (K / 32) * 36;
+            return gemv_launch<F>(fn, d_w, q8b, d_y ? d_y + (size_t)4 * ldy : nullptr,
+                                  d_sums ? d_sums + (size_t)4 * nrows * (K / 32) : nullptr, M - 4, N, K, ldy, row0,
+                                  nrows, device_id, st);
+        }
+        // K slices keep the staged activations (+ tables) within 64 KiB of LDS.
+        int slice = (64 * 1024 - F::TABLE_BYTES) / (M * GEMV_LDS_PER_SB);
+        if (slice > SB)
+            slice = SB;
+        if (slice < 1)
+            return fail(fn, "activation rows do not fit LDS (M=%d)", M);
+        // Whole rows of 8k or 8k+4 super-blocks in one LDS slice: the row-streaming kernel.
+        if (F::USE_STREAM && M <= 2 && !dump && slice == SB && gemv_stream_enabled())
+        {
+            // RP = 1: rows of 8k super-blocks; RP = 2: row pairs of 8k+4 super-blocks
+            const int RP = (SB % 8 == 0) ? 1 : ((SB % 8 == 4 && SB > 4 && (N % 2) == 0) ? 2 : 0);
+            if (RP != 0)
+            {
+                const StreamShape ps = gemv_stream_shape(N / RP, cu_count(device_id),
+                                                           gemv_stream_max_waves() < F::STREAM_MAX_THREADS / WAVE
+                                                               ? gemv_stream_max_waves()
+                                                               : F::STREAM_MAX_THREADS / WAVE);
+                GemvArgs a;
+                a.w = d_w;
+                a.q8 = static_cast<const uint32_t *>(d_q8);
+                a.y = d_y;
+                a.sums = nullptr;
+                a.ldy = ldy;
+                a.N = N;
+                a.SB = SB;
+                a.sb0 = 0;
+                a.nsb = SB;
+                a.rows_per_wave = ps.ppw; // passes per wavefront
+                a.gshift = 3;
+                a.accumulate = 0;
+                a.out_scale = 1.0f;
+                a.row0 = 0;
+                a.nrows = 0;
+                gemv_stream_launch<F>(M, RP, ps.waves, dim3((unsigned)ps.grid), gemv_lds_bytes<F>(M, SB), st, a);
+                return launched(fn);
+            }
+        }
+
+        GemvShape sh = gemv_shape(N, slice, cu_count(device_id));
+        if (gemv_unroll_override() <= 0 && sh.U > F::FAST_MAX_U)
+            sh.U = F::FAST_MAX_U;
+
+        for (int sb0 = 0; sb0 < SB; sb0 += slice)
+        {
+            GemvArgs a;
+            a.w = d_w;
+            a.q8 = static_cast<const uint32_t *>(d_q8);
+            a.y = d_y;
+            a.sums = d_sums;
+            a.ldy = ldy;
+            a.N = N;
+            a.SB = SB;
+            a.sb0 = sb0;
+            a.nsb = (SB - sb0 < slice) ? (SB - sb0) : slice;
+            a.rows_per_wave = sh.rpw;
+            a.gshift = sh.gshift;
+            a.accumulate = sb0 > 0;
+            a.out_scale = 1.0f;
+            a.row0 = row0;
+            a.nrows = nrows;
+            const size_t lds = gemv_lds_bytes<F>(M, a.nsb);
+            if (!dump && sh.gshift == 3)
+                gemv_fast_launch<F>(M, sh.U, dim3((unsigned)sh.grid), lds, st, a);
+            else
+                gemv_launch_m<F>(M, dump, dim3((unsigned)sh.grid), lds, st, a);
+            if (!launched(fn))
+                return false;
+        }
+        return true;
+    }
+} // namespace llamql

@@ -66,6 +66,11 @@ namespace llamql
     {
         static constexpr bool PAIR = false;
         static constexpr bool HAS_MIN = false;
+        static constexpr bool USE_STREAM = false;      // row-streaming kernel pays off for this format
+        static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
+        static constexpr int STREAM_MAX_THREADS = 1024; // workgroup size bound of the row-streaming kernel
+        static constexpr int STREAM_U_PAIR = 5;   // loads per lane and chunk, row-pair passes
+        static constexpr int STREAM_U_SINGLE = 4; // ... single-row passes
         static constexpr int TABLE_BYTES = (int)sizeof(IQ3STables);
 
         __device__ static void stage_tables(void *lds_tab)
@@ -159,5 +164,73 @@ namespace llamql
             bscale = f16_round_packer(scale);
             bmin = 0.0f;
         }
+
+        // ---- streaming interface of the full-row kernel ------------------------------
+        struct Lane
+        {
+            int c, j;
+        };
+        __device__ __forceinline__ static Lane lane_consts(int c)
+        {
+            Lane l;
+            l.c = c;
+            l.j = c;
+            return l;
+        }
+
+        struct Ptr
+        {
+            const uint2 *qs;
+            const uint32_t *signs;
+            const uint4 *meta;
+        };
+        __device__ __forceinline__ static Ptr ptr(const GemvArgs &a, long row, int sb, int c)
+        {
+            const size_t T = (size_t)a.N * a.SB;
+            const size_t t = (size_t)row * a.SB + sb;
+            const uint8_t *base = static_cast<const uint8_t *>(a.w);
+            Ptr p;
+            p.qs = reinterpret_cast<const uint2 *>(base) + t * 8 + c;
+            p.signs = reinterpret_cast<const uint32_t *>(base + T * 64) + t * 8 + c;
+            p.meta = reinterpret_cast<const uint4 *>(base + T * 96) + t;
+            return p;
+        }
+        __device__ __forceinline__ static void advance(Ptr &p, int nsb)
+        {
+            p.qs += (size_t)nsb * 8;
+            p.signs += (size_t)nsb * 8;
+            p.meta += nsb;
+        }
+        __device__ __forceinline__ static Raw load_at(const Ptr &p, int off_sb)
+        {
+            Raw r;
+            r.qs = p.qs[off_sb * 8];
+            r.signs = p.signs[off_sb * 8];
+            r.meta = p.meta[off_sb];
+            return r;
+        }
+        __device__ __forceinline__ static void decode2(const Raw &r, const Lane &l, v4i &w0, v4i &w1,
+                                                       float &bscale, float &bmin, const void *tab)
+        {
+            int j;
+            decode(r, l.c, w0, w1, j, bscale, bmin, tab);
+        }
+
+        // ---- row-streaming kernel interface (generic form) -------------------------------
+        struct Scale
+        {
+            float bs;
+        };
+        typedef Lane Lane3;
+        __device__ __forceinline__ static Lane3 lane3_consts(int c) { return lane_consts(c); }
+        __device__ __forceinline__ static void decode3(const Raw &r, const Lane3 &l, v4i &w0, v4i &w1, Scale &S,
+                                                       const void *tab)
+        {
+            int j;
+            float bmin;
+            decode(r, l.c, w0, w1, j, S.bs, bmin, tab);
+        }
+        __device__ __forceinline__ static float cs(const Scale &S, float ad) { return ad * S.bs; }
+        __device__ __forceinline__ static float add_min(const Scale &, float, float acc) { return acc; }
     };
 } // namespace llamql

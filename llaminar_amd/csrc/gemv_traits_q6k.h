@@ -48,6 +48,11 @@ namespace llamql
     {
         static constexpr bool PAIR = true;
         static constexpr bool HAS_MIN = false; // the reference's mins plane is all zero for Q6_K
+        static constexpr bool USE_STREAM = false;      // row-streaming kernel pays off for this format
+        static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
+        static constexpr int STREAM_MAX_THREADS = 1024; // workgroup size bound of the row-streaming kernel
+        static constexpr int STREAM_U_PAIR = 2;   // loads per lane and chunk, row-pair passes
+        static constexpr int STREAM_U_SINGLE = 2; // ... single-row passes
         static constexpr int TABLE_BYTES = 0;
         __device__ static void stage_tables(void *) {}
 
@@ -147,5 +152,77 @@ namespace llamql
             bscale = (msc != 0.0f) ? f16_round_packer(__fdiv_rn(d * msc * 32.0f, 127.0f)) : 0.0f;
             bmin = 0.0f;
         }
+
+        // ---- streaming interface of the full-row kernel ------------------------------
+        struct Lane
+        {
+            int c, j;
+        };
+        __device__ __forceinline__ static Lane lane_consts(int c)
+        {
+            Lane l;
+            l.c = c;
+            l.j = (c & 4) + ((c >> 1) & 1) + 2 * (c & 1);
+            return l;
+        }
+
+        struct Ptr
+        {
+            const uint4 *ql;
+            const uint4 *qh;
+            const uint4 *sc;
+            const uint16_t *d;
+        };
+        __device__ __forceinline__ static Ptr ptr(const GemvArgs &a, long row, int sb, int c)
+        {
+            const size_t T = (size_t)a.N * a.SB;
+            const size_t t = (size_t)row * a.SB + sb;
+            const uint8_t *base = static_cast<const uint8_t *>(a.w);
+            Ptr p;
+            p.ql = reinterpret_cast<const uint4 *>(base) + t * 8 + c;
+            p.qh = reinterpret_cast<const uint4 *>(base + T * 128) + t * 4 + 2 * (c >> 2) + (c & 1);
+            p.sc = reinterpret_cast<const uint4 *>(base + T * 192) + t;
+            p.d = reinterpret_cast<const uint16_t *>(base + T * 208) + t;
+            return p;
+        }
+        __device__ __forceinline__ static void advance(Ptr &p, int nsb)
+        {
+            p.ql += (size_t)nsb * 8;
+            p.qh += (size_t)nsb * 4;
+            p.sc += nsb;
+            p.d += nsb;
+        }
+        __device__ __forceinline__ static Raw load_at(const Ptr &p, int off_sb)
+        {
+            Raw r;
+            r.ql = p.ql[off_sb * 8];
+            r.qh = p.qh[off_sb * 4];
+            r.sc = p.sc[off_sb];
+            r.d = p.d[off_sb];
+            return r;
+        }
+        __device__ __forceinline__ static void decode2(const Raw &r, const Lane &l, v4i &w0, v4i &w1,
+                                                       float &bscale, float &bmin, const void *tab)
+        {
+            int j;
+            decode(r, l.c, w0, w1, j, bscale, bmin, tab);
+        }
+
+        // ---- row-streaming kernel interface (generic form) -------------------------------
+        struct Scale
+        {
+            float bs;
+        };
+        typedef Lane Lane3;
+        __device__ __forceinline__ static Lane3 lane3_consts(int c) { return lane_consts(c); }
+        __device__ __forceinline__ static void decode3(const Raw &r, const Lane3 &l, v4i &w0, v4i &w1, Scale &S,
+                                                       const void *tab)
+        {
+            int j;
+            float bmin;
+            decode(r, l.c, w0, w1, j, S.bs, bmin, tab);
+        }
+        __device__ __forceinline__ static float cs(const Scale &S, float ad) { return ad * S.bs; }
+        __device__ __forceinline__ static float add_min(const Scale &, float, float acc) { return acc; }
     };
 } // namespace llamql

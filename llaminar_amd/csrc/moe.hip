@@ -180,7 +180,7 @@ namespace llamql
         a.out_scale = 1.0f;
         a.row0 = 0;
         a.nrows = 0;
-        gemv_body<F, 1, false>(a, (long)blockIdx.x, lds);
+        gemv_body<F, 1, 1, false>(a, (long)blockIdx.x, lds);
     }
 
     // grid: (workgroups per matrix, n_tokens).  Slots are walked in ascending
@@ -214,7 +214,7 @@ namespace llamql
             a.out_scale = m.weights[slot];
             a.row0 = 0;
             a.nrows = 0;
-            gemv_body<F, 1, false>(a, (long)blockIdx.x, lds);
+            gemv_body<F, 1, 1, false>(a, (long)blockIdx.x, lds);
             first = false;
             __syncthreads(); // LDS is restaged by the next slot
         }

@@ -33,6 +33,27 @@ namespace llamql
         return r;
     }
 
+    // Same rounding for two values at once.  The truncating branch is only needed when a
+    // value lies below the fp16 normal range, which real weights almost never produce:
+    // one rarely-taken branch (fp16 exponent field 0 or 1 in either result) guards the
+    // exact test for both.
+    __device__ __forceinline__ void f16_round_packer2(float x0, float x1, float &r0, float &r1)
+    {
+        const __half h0 = __float2half_rn(x0);
+        const __half h1 = __float2half_rn(x1);
+        r0 = __half2float(h0);
+        r1 = __half2float(h1);
+        const uint32_t e = ((uint32_t)__half_as_ushort(h0) | ((uint32_t)__half_as_ushort(h1) << 16)) & 0x7C007C00u;
+        // a 16-bit half below 0x0800 makes the subtraction borrow into bit 15 / bit 31
+        if (__builtin_expect(((e - 0x08000800u) & 0x80008000u) != 0u, 0))
+        {
+            if (fabsf(x0) < 6.103515625e-05f)
+                r0 = truncf(x0 * 16777216.0f) * 5.9604644775390625e-08f;
+            if (fabsf(x1) < 6.103515625e-05f)
+                r1 = truncf(x1 * 16777216.0f) * 5.9604644775390625e-08f;
+        }
+    }
+
     // ---- cross-lane -----------------------------------------------------------
 
     template <int CTRL>
@@ -78,6 +99,24 @@ namespace llamql
     __device__ __forceinline__ int dot16(const v4i a, const v4i b, int acc)
     {
         acc = dot4(a.x, b.x, acc);
+        acc = dot4(a.y, b.y, acc);
+        acc = dot4(a.z, b.z, acc);
+        acc = dot4(a.w, b.w, acc);
+        return acc;
+    }
+
+    // Same with a zero start value.  Spelled as the three-operand VOP3P form so no
+    // register has to be cleared first.
+    __device__ __forceinline__ int dot4z(int a, int b)
+    {
+        int r;
+        asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+        return r;
+    }
+
+    __device__ __forceinline__ int dot16z(const v4i a, const v4i b)
+    {
+        int acc = dot4z(a.x, b.x);
         acc = dot4(a.y, b.y, acc);
         acc = dot4(a.z, b.z, acc);
         acc = dot4(a.w, b.w, acc);

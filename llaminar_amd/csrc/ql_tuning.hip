@@ -8,9 +8,21 @@ namespace llamql
     namespace
     {
         int g_rows_per_wave = 0;
+        int g_unroll = 0;
     }
     int gemv_rows_per_wave_override() { return g_rows_per_wave; }
+    int gemv_unroll_override() { return g_unroll; }
+    bool gemv_stream_enabled() { return g_unroll <= 0; }
+    int gemv_stream_max_waves() { return g_unroll < 0 ? -g_unroll : 16; }
 } // namespace llamql
 
-extern "C" void llam_ql_set_gemv_tuning(int rows_per_wave) { llamql::g_rows_per_wave = rows_per_wave; }
-extern "C" void llam_ql_reset_gemv_tuning(void) { llamql::g_rows_per_wave = 0; }
+extern "C" void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll)
+{
+    llamql::g_rows_per_wave = rows_per_wave;
+    llamql::g_unroll = unroll;
+}
+extern "C" void llam_ql_reset_gemv_tuning(void)
+{
+    llamql::g_rows_per_wave = 0;
+    llamql::g_unroll = 0;
+}

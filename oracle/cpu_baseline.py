@@ -1,0 +1,97 @@
+"""TEST/BENCH INFRASTRUCTURE: time the CPU path on a bounded sample and print one
+JSON object.  Run as a subprocess by bench.py's cpu_baseline leg.
+
+kind "reference": the reference's own AVX512-VNNI GEMV (oracle/_ref), when that
+library was built and this host has the instruction sets it was compiled for;
+kind "port": the scalar C restatement (oracle/ql_oracle.c, OpenMP over rows).
+
+Sample: the headline kernel's shape -- Q4_K GEMV, N=25600 x K=5120, batch 1 --
+on seeded synthetic blocks; GB/s counts the same algorithmic bytes as the GPU
+figure (GGUF weight bytes + Q8_1 activations + fp32 outputs).
+"""
+from __future__ import annotations
+
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent.parent
+sys.path.insert(0, str(ROOT))
+
+from oracle.binding import BLOCK_BYTES, FMT_Q4_K, Oracle, Ref  # noqa: E402
+
+NEEDED = {"avx512f", "avx512bw", "avx512vl", "avx512dq", "avx512_vnni", "avx2", "fma", "f16c"}
+
+
+def cpu_flags() -> set:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("flags"):
+                return set(line.split(":", 1)[1].split())
+    except OSError:
+        pass
+    return set()
+
+
+def main():
+    N, K, fmt = 25600, 5120, FMT_Q4_K
+    budget_s = float(os.environ.get("QL_CPU_BASELINE_SECONDS", "12"))
+    rng = np.random.default_rng(1)
+    W = rng.integers(0, 256, size=(N, K // 256, BLOCK_BYTES[fmt]), dtype=np.uint8)
+    for off in (0, 2):
+        d = rng.uniform(0.001, 0.02, size=(N, K // 256)).astype(np.float16)
+        W[:, :, off:off + 2] = d.view(np.uint8).reshape(N, K // 256, 2)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    o = Oracle()
+    q8 = o.quantize(x)
+    nbytes = N * (K // 256) * BLOCK_BYTES[fmt] + (K // 32) * 36 + N * 4
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+
+    use_ref = Ref.available() and NEEDED <= cpu_flags() and os.environ.get("QL_CPU_BASELINE_KIND", "") != "port"
+    times = []
+    if use_ref:
+        r = Ref()
+        threads = r.omp_threads()
+        h = r.pack(fmt, W, N, K)
+        packed = r.pack_bytes(h)
+        C = np.zeros((1, N), np.float32)
+        for _ in range(3):
+            r.gemm_packed(h, q8, N, isa=0, out=C)
+        t_end = time.perf_counter() + budget_s
+        while time.perf_counter() < t_end and len(times) < 5000:
+            t0 = time.perf_counter()
+            r.gemm_packed(h, q8, N, isa=0, out=C)
+            times.append(time.perf_counter() - t0)
+        r.pack_free(h)
+        kind = "reference"
+        detail = f"reference AVX512-VNNI gemv_native_vnni_preq, packed {packed / 1e6:.1f} MB"
+    else:
+        # scalar port: decode + dot per call (the restatement keeps no packed form)
+        rows = 2048  # bounded sample of the rows; GB/s scales linearly in rows
+        nbytes = rows * (K // 256) * BLOCK_BYTES[fmt] + (K // 32) * 36 + rows * 4
+        Wp = np.ascontiguousarray(W[:rows])
+        o.gemm(fmt, Wp, K, q8)
+        t_end = time.perf_counter() + budget_s
+        while time.perf_counter() < t_end and len(times) < 200:
+            t0 = time.perf_counter()
+            o.gemm(fmt, Wp, K, q8)
+            times.append(time.perf_counter() - t0)
+        kind = "port"
+        detail = f"scalar C restatement on {rows} of {N} rows, OpenMP over rows"
+    med = float(np.median(times))
+    print(json.dumps({
+        "value": nbytes / med / 1e9,
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": kind,
+        "sample": f"Q4_K GEMV N={N} K={K} batch 1, {len(times)} timed calls (median {med * 1e3:.3f} ms, "
+                  f"min {min(times) * 1e3:.3f} ms), {detail}",
+    }))
+
+
+if __name__ == "__main__":
+    main()

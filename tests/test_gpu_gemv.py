@@ -111,8 +111,13 @@ def test_tuning_override_does_not_change_results(capi, dev, oracle, fmt):
     base = capi.gemv(fmt, wd, qd, 2, N, K)
     lib = capi.load()
     try:
+        # rows per wavefront only changes which wavefront owns a row: bitwise identical
         for rpw in (1, 3, 8):
-            lib.llam_ql_set_gemv_tuning(rpw)
+            lib.llam_ql_set_gemv_tuning(rpw, 0)
+            assert torch.equal(capi.gemv(fmt, wd, qd, 2, N, K), base)
+        # the unroll depth does not change the per-lane accumulation order either
+        for unroll in (1, 2, 3, 4):
+            lib.llam_ql_set_gemv_tuning(0, unroll)
             assert torch.equal(capi.gemv(fmt, wd, qd, 2, N, K), base)
     finally:
         lib.llam_ql_reset_gemv_tuning()
