@@ -47,6 +47,9 @@ def parse():
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times, so a rocprofv3 --pmc run of this "
+                         "command records FETCH_SIZE / WRITE_SIZE for a kernel of known traffic")
     return ap.parse_args()
 
 
@@ -165,6 +168,13 @@ def main():
         k_us = e0.elapsed_time(e1) * 1e3 / reps
         k_bytes = synth.gemv_bytes(FMT_Q4_K, FFN, HIDDEN, 1)
         achieved = k_bytes / (k_us * 1e-6) / 1e9
+
+    if args.pmc_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -202,12 +202,21 @@ namespace llamql
     inline void gemv_fast_launch_u(int U, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
     {
         dim3 block(GEMV_WAVES * WAVE);
-        switch (U)
+        // formats whose decode is register-hungry only build (and run) the shallow variant
+        if constexpr (F::FAST_MAX_U >= 4)
         {
-        case 1: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1>), grid, block, lds, st, a); break;
-        case 2: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 2>), grid, block, lds, st, a); break;
-        case 3: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 3>), grid, block, lds, st, a); break;
-        default: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 4>), grid, block, lds, st, a); break;
+            switch (U)
+            {
+            case 1: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1>), grid, block, lds, st, a); break;
+            case 2: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 2>), grid, block, lds, st, a); break;
+            case 3: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 3>), grid, block, lds, st, a); break;
+            default: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 4>), grid, block, lds, st, a); break;
+            }
+        }
+        else
+        {
+            (void)U;
+            hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1>), grid, block, lds, st, a);
         }
     }
 
@@ -369,7 +378,8 @@ namespace llamql
         if (slice < 1)
             return fail(fn, "activation rows do not fit LDS (M=%d)", M);
         // Whole rows of 8k or 8k+4 super-blocks in one LDS slice: the row-streaming kernel.
-        if (F::USE_STREAM && M <= 2 && !dump && slice == SB && gemv_stream_enabled())
+        if constexpr (F::USE_STREAM)
+        if (M <= 2 && !dump && slice == SB && gemv_stream_enabled())
         {
             // RP = 1: rows of 8k super-blocks; RP = 2: row pairs of 8k+4 super-blocks
             const int RP = (SB % 8 == 0) ? 1 : ((SB % 8 == 4 && SB > 4 && (N % 2) == 0) ? 2 : 0);

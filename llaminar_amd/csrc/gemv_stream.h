@@ -229,17 +229,13 @@ namespace llamql
             hipLaunchKernelGGL((gemv_stream_kernel<F, M, F::STREAM_U_SINGLE, 1>), grid, block, lds, st, a);
     }
 
-    // M is one of 1,2,3,4,8.
+    // M is 1 or 2 (larger batches use the chunked kernel).
     template <class F>
     inline void gemv_stream_launch(int M, int RP, int waves, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
     {
-        switch (M)
-        {
-        case 1: gemv_stream_launch_rp<F, 1>(RP, waves, grid, lds, st, a); break;
-        case 2: gemv_stream_launch_rp<F, 2>(RP, waves, grid, lds, st, a); break;
-        case 3: gemv_stream_launch_rp<F, 3>(RP, waves, grid, lds, st, a); break;
-        case 4: gemv_stream_launch_rp<F, 4>(RP, waves, grid, lds, st, a); break;
-        default: gemv_stream_launch_rp<F, 8>(RP, waves, grid, lds, st, a); break;
-        }
+        if (M == 1)
+            gemv_stream_launch_rp<F, 1>(RP, waves, grid, lds, st, a);
+        else
+            gemv_stream_launch_rp<F, 2>(RP, waves, grid, lds, st, a);
     }
 } // namespace llamql

@@ -96,10 +96,17 @@ namespace llamql
             return r;
         }
 
+        // Byte i (0..15) of the 16 int8 sub-scales, sign-extended.  Dwords are picked with
+        // bit masks rather than a conditional on the vector's members, which would turn
+        // into an indexed access through memory.
         __device__ __forceinline__ static int sc_byte(const uint4 &s, int i)
         {
-            const uint32_t w = (i & 8) ? ((i & 4) ? s.w : s.z) : ((i & 4) ? s.y : s.x);
-            return (int)(int8_t)((w >> (8 * (i & 3))) & 0xFFu);
+            const uint32_t m8 = (uint32_t)0 - (uint32_t)((i >> 3) & 1);
+            const uint32_t m4 = (uint32_t)0 - (uint32_t)((i >> 2) & 1);
+            const uint32_t lo = (s.y & m4) | (s.x & ~m4);
+            const uint32_t hi = (s.w & m4) | (s.z & ~m4);
+            const uint32_t w = (hi & m8) | (lo & ~m8);
+            return __builtin_amdgcn_sbfe((int)w, 8u * (uint32_t)(i & 3), 8u);
         }
 
         __device__ __forceinline__ static void factor(int sc, float msc, v2s &ff, v2s &cc)
