@@ -31,9 +31,10 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs (see profiles/gemv_q4k_25600x5120_pmc.txt); None until measured.
-DOMINANT_TRAFFIC_BYTES = None
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# runs of this script (profiles/gemv_q4k_25600x5120_batch1_pmc.txt): (36104.2 KiB x 2.000 +
+# 104.4 KiB x 1.000), the factors being what the same counters read for a plain 256 MiB kernel.
+DOMINANT_TRAFFIC_BYTES = 74048307
 
 HIDDEN, QDIM, KVDIM, FFN = 5120, 8192, 1024, 25600
 
@@ -48,7 +49,7 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
-                    help="also run a plain 256 MiB device copy a few times, so a rocprofv3 --pmc run of this "
+                    help="also run a plain 256 MiB read + 256 MiB write elementwise kernel a few times, so a rocprofv3 --pmc run of this "
                          "command records FETCH_SIZE / WRITE_SIZE for a kernel of known traffic")
     return ap.parse_args()
 
@@ -170,10 +171,11 @@ def main():
         achieved = k_bytes / (k_us * 1e-6) / 1e9
 
     if args.pmc_calibration:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        # a plain streaming kernel: reads 256 MiB, writes 256 MiB
+        src = torch.arange(64 << 20, dtype=torch.int32, device=dev)
         dst = torch.empty_like(src)
         for _ in range(5):
-            dst.copy_(src)
+            torch.add(src, 1, out=dst)
         torch.cuda.synchronize()
 
     cpu = None
@@ -215,7 +217,7 @@ def main():
             "launch": "eager" if graphs is None else "hip-graph replay",
         },
         "roofline": {
-            "kernel": "gemv_kernel<Q4KTraits,1> N=25600 K=5120",
+            "kernel": "gemv_stream_kernel<Q4KTraits,1,5,2> N=25600 K=5120",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
