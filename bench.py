@@ -39,12 +39,155 @@ DOMINANT_TRAFFIC_BYTES = 74048307
 HIDDEN, QDIM, KVDIM, FFN = 5120, 8192, 1024, 25600
 
 
+INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X published dense int8 rate
+
+
+def _time_launches(torch, stream, fn, reps, warm=5):
+    """Average duration in microseconds of fn(i), timed with events on the launch stream."""
+    for i in range(warm):
+        fn(i)
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    stream.synchronize()
+    e0.record(stream)
+    for i in range(reps):
+        fn(i)
+    e1.record(stream)
+    stream.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def _common(args, metric, value, unit, ms, dtype, config, roofline):
+    return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
+            "data": "synthetic", "config": config, "roofline": roofline, "cpu_baseline": None}
+
+
+def bench_gemm(args, torch, capi, synth, dev):
+    """Prefill: M x 5120 Q8_1 activations times Q4_K [25600 x 5120], int8 MFMA."""
+    from llaminar_amd.capi import FMT_Q4_K
+
+    M = args.batch if args.batch > 8 else 512
+    N, K = FFN, HIDDEN
+    mats = [capi.prepare_weights(FMT_Q4_K, synth.weights_torch(FMT_Q4_K, N, K, 50 + i, dev), N, K) for i in range(2)]
+    g = torch.Generator(device=dev)
+    g.manual_seed(9)
+    x = torch.randn(M, K, device=dev, generator=g)
+    q8 = capi.quantize_q8_1(x)
+    y = torch.empty(M, N, device=dev)
+    stream = torch.cuda.Stream()
+    steps = min(args.steps, 50)
+    with torch.cuda.stream(stream):
+        us = _time_launches(torch, stream, lambda i: capi.gemm(FMT_Q4_K, mats[i % 2], q8, M, N, K, out=y), steps,
+                            max(2, min(args.warmup, 5)))
+        us_q = _time_launches(torch, stream, lambda i: capi.quantize_q8_1(x, out=q8), steps)
+    ops = 2.0 * M * N * K
+    tops = ops / (us * 1e-6) / 1e12
+    return _common(args, "prefill int8 GEMM TOPS", round(tops, 2), "TOP/s", round(us * 1e-3, 5), "int8",
+                   {"workload": "prefill GEMM of the gate/up projection: M=%d tokens x K=5120 x N=25600, Q4_K weights, "
+                                "Q8_1 activations" % M, "M": M, "N": N, "K": K, "ops_per_step": ops,
+                    "quantize_us": round(us_q, 2)},
+                   {"kernel": "gemm_kernel<Q4KTraits> M=%d N=25600 K=5120" % M, "bound": "mfma",
+                    "achieved": round(tops, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
+                    "frac": round(tops / INT8_MFMA_PEAK_TOPS, 4), "traffic": None, "ops_per_launch": ops,
+                    "us_per_launch": round(us, 2), "launches_timed": steps})
+
+
+def bench_moe(args, torch, capi, synth, dev):
+    """MoE expert FFN decode: route, gate/up, SwiGLU+quantise, down, shared expert."""
+    from llaminar_amd.capi import FMT_IQ3_S
+
+    T = args.batch
+    H, I, E, TOPK = 2048, 512, 256, 8
+    fmt = FMT_IQ3_S
+    experts = []
+    for e in range(E + 1):  # the last one is the shared expert
+        experts.append(tuple(capi.prepare_weights(fmt, synth.weights_torch(fmt, n, k, 10 * e + j, dev), n, k)
+                             for j, (n, k) in enumerate(((I, H), (I, H), (H, I)))))
+    table = capi.expert_table(experts[:E], dev)
+    shared = capi.expert_table(experts[E:], dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    x = torch.randn(T, H, device=dev, generator=g)
+    logits = torch.randn(T, E, device=dev, generator=g)
+    q8 = torch.empty(T * (H // 32) * 36, dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, device=dev)
+    sid = torch.zeros(T, 1, dtype=torch.int32, device=dev)
+    sw = torch.ones(T, 1, device=dev)
+    def step(_i=0):
+        ids, w = capi.moe_route(logits, TOPK)
+        capi.quantize_q8_1(x, out=q8)
+        gate, up = capi.moe_gate_up(fmt, table, E, ids, q8, T, TOPK, H, I)
+        qa = capi.swiglu_quantize(gate, up)
+        capi.moe_down(fmt, table, E, ids, w, qa, out, T, TOPK, H, I, accumulate=False)
+        sgate, sup = capi.moe_gate_up(fmt, shared, 1, sid, q8, T, 1, H, I)
+        qs = capi.swiglu_quantize(sgate, sup)
+        capi.moe_down(fmt, shared, 1, sid, sw, qs, out, T, 1, H, I, accumulate=True)
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(max(args.warmup, 2)):
+            step()
+        stream.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=stream):
+            step()
+        us = _time_launches(torch, stream, lambda i: gr.replay(), args.steps, 3)
+    blk = 112  # device bytes per IQ3_S super-block
+    w_bytes = (TOPK + 1) * T * 3 * I * (H // 256) * blk  # every token slot streams its expert's three matrices
+    value = w_bytes / (us * 1e-6) / 1e9
+    return _common(args, "MoE expert FFN decode effective GB/s", round(value, 1), "GB/s", round(us * 1e-3, 5), "int8",
+                   {"workload": "MoE expert FFN decode: hidden 2048, 256 routed experts + 1 shared, top-8, expert "
+                                "intermediate 512, IQ3_S, %d token(s); route + gate/up + SwiGLU + down + shared" % T,
+                    "tokens": T, "weight_bytes_per_step": w_bytes, "tokens_per_s": round(T / (us * 1e-6), 1),
+                    "launch": "hip-graph replay"},
+                   {"kernel": "moe step (8 launches)", "bound": "hbm", "achieved": round(value, 1),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None,
+                    "bytes_per_launch": w_bytes, "us_per_launch": round(us, 2), "launches_timed": args.steps})
+
+
+def bench_gemv(args, torch, capi, synth, dev):
+    """Single GEMVs: every format on the layer shapes, rotating over matrices beyond the cache."""
+    from llaminar_amd.capi import FMT_IQ3_S, FMT_Q4_K, FMT_Q6_K
+
+    M = args.batch
+    rows = []
+    stream = torch.cuda.Stream()
+    names = {FMT_Q4_K: "Q4_K", FMT_Q6_K: "Q6_K", FMT_IQ3_S: "IQ3_S"}
+    for fmt in (FMT_Q4_K, FMT_Q6_K, FMT_IQ3_S):
+        for N, K in ((FFN, HIDDEN), (HIDDEN, FFN), (QDIM, HIDDEN), (HIDDEN, QDIM), (KVDIM, HIDDEN)):
+            nmat = max(2, min(8, int(600e6 // synth.gemv_bytes(fmt, N, K, 1)) + 1))
+            mats = [capi.prepare_weights(fmt, synth.weights_torch(fmt, N, K, 70 + i, dev), N, K) for i in range(nmat)]
+            x = torch.randn(M, K, device=dev)
+            q8 = capi.quantize_q8_1(x)
+            y = torch.empty(M, N, device=dev)
+            with torch.cuda.stream(stream):
+                us = _time_launches(torch, stream,
+                                    lambda i: capi.gemv(fmt, mats[i % nmat], q8, M, N, K, out=y), args.steps, 10)
+            b = synth.gemv_bytes(fmt, N, K, M)
+            rows.append({"fmt": names[fmt], "N": N, "K": K, "M": M, "us": round(us, 2),
+                         "GBps": round(b / (us * 1e-6) / 1e9, 1), "frac": round(b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+            del mats
+    head = rows[0]
+    return _common(args, "GEMV effective GB/s per shape", head["GBps"], "GB/s", round(head["us"] * 1e-3, 5), "int8",
+                   {"workload": "single decode GEMVs, batch %d, all formats x layer shapes" % M, "shapes": rows},
+                   {"kernel": "Q4_K GEMV N=25600 K=5120", "bound": "hbm", "achieved": head["GBps"],
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["frac"], "traffic": None,
+                    "us_per_launch": head["us"], "launches_timed": args.steps})
+
+
+OTHER_WORKLOADS = {"gemm": bench_gemm, "moe": bench_moe, "gemv": bench_gemv}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--batch", type=int, default=1, help="activation rows per step (1 or 8)")
+    ap.add_argument("--workload", choices=["layer", "gemm", "moe", "gemv"], default="layer",
+                    help="layer: the headline decode-layer step (default); gemm: prefill int8 GEMM 512x25600x5120 Q4_K; "
+                         "moe: 256-expert top-8 IQ3_S expert FFN decode; gemv: single GEMVs of every format and layer shape")
+    ap.add_argument("--batch", type=int, default=1, help="activation rows / tokens per step")
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -72,6 +215,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     M = args.batch
+    if args.workload != "layer":
+        print(json.dumps(OTHER_WORKLOADS[args.workload](args, torch, capi, synth, dev)))
+        return
     assert 1 <= M <= capi.MAX_GEMV_M
 
     projs = [("q", QDIM, HIDDEN, FMT_Q4_K), ("k", KVDIM, HIDDEN, FMT_Q4_K), ("v", KVDIM, HIDDEN, FMT_Q6_K),

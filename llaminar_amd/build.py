@@ -4,7 +4,10 @@ Every ``*.hip`` / ``*.cpp`` source under ``llaminar_amd/csrc`` is compiled into
 one shared object, ``llaminar_amd/lib/libllaminar_ql.so``.  hipcc cross-compiles
 for gfx950 without a GPU, so this runs anywhere the ROCm toolchain is present.
 
-Usage: ``python -m llaminar_amd.build [--force]``
+The host-side operator (``csrc/host``) is linked into a second library,
+``libllaminar_ql_host.so``, on top of the first.
+
+Usage: ``python -m llaminar_amd.build``
 """
 from __future__ import annotations
 
@@ -20,6 +23,7 @@ ROOT = PKG.parent
 CSRC = PKG / "csrc"
 LIBDIR = PKG / "lib"
 LIB = LIBDIR / "libllaminar_ql.so"
+HOST_LIB = LIBDIR / "libllaminar_ql_host.so"
 OBJDIR = PKG / "build"
 
 ARCH = "gfx950"
@@ -49,8 +53,21 @@ def sources() -> list[Path]:
 
 
 def _deps_mtime() -> float:
-    files = list(CSRC.glob("*")) + list((ROOT / "include" / "llaminar_amd").glob("*.h"))
+    files = [f for f in CSRC.rglob("*") if f.is_file()] + list((ROOT / "include" / "llaminar_amd").glob("*.h*"))
     return max(f.stat().st_mtime for f in files)
+
+
+def build_host(verbose: bool = True) -> Path:
+    """Link the C++ operator layer against the kernel library (no device code)."""
+    srcs = sorted((CSRC / "host").glob("*.cpp"))
+    cmd = [hipcc(), "-std=c++17", "-O2", "-fPIC", "-shared", f"-I{ROOT / 'include'}", *map(str, srcs),
+           f"-L{LIBDIR}", "-lllaminar_ql", "-Wl,-rpath,$ORIGIN", "-o", str(HOST_LIB)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"host library build failed:\n{proc.stderr}")
+    if verbose:
+        print(f"[llaminar_amd.build] wrote {HOST_LIB} ({HOST_LIB.stat().st_size} bytes)", flush=True)
+    return HOST_LIB
 
 
 def _compile(src: Path) -> Path:
@@ -71,7 +88,7 @@ def _compile(src: Path) -> Path:
 
 def build(force: bool = True, verbose: bool = True) -> Path:
     """Compile and link the library.  With force=False an up-to-date library is kept."""
-    if not force and LIB.exists() and LIB.stat().st_mtime >= _deps_mtime():
+    if not force and LIB.exists() and HOST_LIB.exists() and LIB.stat().st_mtime >= _deps_mtime():
         return LIB
     OBJDIR.mkdir(exist_ok=True)
     LIBDIR.mkdir(exist_ok=True)
@@ -86,6 +103,7 @@ def build(force: bool = True, verbose: bool = True) -> Path:
         raise RuntimeError(f"link failed:\n{proc.stderr}")
     if verbose:
         print(f"[llaminar_amd.build] wrote {LIB} ({LIB.stat().st_size} bytes)", flush=True)
+    build_host(verbose)
     return LIB
 
 
