@@ -18,6 +18,7 @@
 #pragma once
 
 #include "gemv_core.h"
+#include "gemv_quad.h"
 
 namespace llamql
 {
@@ -361,6 +362,43 @@ namespace llamql
     {
         const int SB = K / 256;
         const bool dump = d_sums != nullptr;
+        // Rows of at least 16 super-blocks in a format with a quad-lane decoder: the
+        // quad kernel, which stages whole activation rows (up to 160 KiB of LDS).
+        if constexpr (F::USE_QUAD)
+        if (!dump && SB >= QUAD_STEP_SB && gemv_unroll_override() == 0)
+        {
+            if (quad_lds_bytes(M, SB) > QUAD_MAX_LDS)
+            {
+                if (M == 1)
+                    return fail(fn, "K=%d is too long for one activation row in LDS", K);
+                const int M0 = M / 2;
+                if (!gemv_launch<F>(fn, d_w, d_q8, d_y, d_sums, M0, N, K, ldy, row0, nrows, device_id, st))
+                    return false;
+                const uint8_t *q8b = static_cast<const uint8_t *>(d_q8) + (size_t)M0 * (K / 32) * 36;
+                return gemv_launch<F>(fn, d_w, q8b, d_y + (size_t)M0 * ldy, nullptr, M - M0, N, K, ldy, row0, nrows,
+                                      device_id, st);
+            }
+            const QuadShape qs = gemv_quad_shape(N, SB, cu_count(device_id), quad_max_threads(M) / WAVE);
+            GemvArgs a;
+            a.w = d_w;
+            a.q8 = static_cast<const uint32_t *>(d_q8);
+            a.y = d_y;
+            a.sums = nullptr;
+            a.ldy = ldy;
+            a.N = N;
+            a.SB = SB;
+            a.sb0 = 0;
+            a.nsb = SB;
+            a.rows_per_wave = qs.rows_per_wave;
+            a.gshift = 3;
+            a.accumulate = 0;
+            a.out_scale = 1.0f;
+            a.row0 = 0;
+            a.nrows = 0;
+            gemv_quad_launch<typename F::Quad>(M, dim3((unsigned)qs.grid), dim3((unsigned)qs.waves * WAVE),
+                                               quad_lds_bytes(M, SB), st, a);
+            return launched(fn);
+        }
         // batch sizes without a dedicated kernel are run as 4 + (M-4)
         if (M > 4 && M < 8)
         {

@@ -1,0 +1,475 @@
+// Quad-lane decode GEMV (gfx950): four lanes own one 256-element super-block.
+//
+// Lane l of a quad decodes 64 weights -- the two complete 32-element blocks 2l and
+// 2l+1 of its super-block -- so it forms both exact int32 block sums by itself (no
+// exchange between lanes) and decodes the super-block header once for two blocks.
+// A wavefront step covers 16 consecutive super-blocks.
+//
+// A wavefront owns a contiguous range of weight rows and walks it as ONE run of
+// super-blocks, 16 per step, whatever the row length: a step may contain the end of
+// one row and the start of the next.  Two running sums per lane (`cur`: the row being
+// finished, `nxt`: the row after it) take the step's contribution according to the
+// lane's position; when a row ends inside a step its 64 partial sums are reduced in a
+// fixed order and stored, and `nxt` becomes `cur`.  Rows must have at least 16
+// super-blocks (K >= 4096) so that a step touches at most two rows.
+//
+// Loads run U steps ahead in two alternating register buffers.  Activations (Q8_1)
+// are staged once per workgroup in LDS, laid out so that each of a lane's reads is a
+// conflict-free ds_read_b128:
+//   quants  [m][sb/16][part 0..3][sb%16][l][16 B]   part = 2*(block&1) + half
+//   scales  [m][sb][l]{f32 d, f32 sum*d of block 2l ; same of block 2l+1}
+//
+// Per block: idot exact; acc = fma(float(idot), f32(a.d)*b_scale, acc);
+// acc = fma(float(a.sum)*f32(a.d), b_min, acc) -- the reference's arithmetic
+// (CPUNativeVNNIGemv.h:417-487); only the order in which blocks are added differs.
+#pragma once
+
+#include "gemv_core.h"
+
+namespace llamql
+{
+    constexpr int QUAD_STEP_SB = 16; // super-blocks per wavefront step
+    // workgroup size bound: one activation row leaves room for 16 wavefronts of 128 registers
+    constexpr int quad_max_threads(int M) { return M == 1 ? 1024 : 512; }
+    constexpr size_t QUAD_MAX_LDS = 160 * 1024; // LDS of one gfx950 compute unit
+
+    // LDS bytes for M activation rows of nsb super-blocks.
+    inline size_t quad_lds_bytes(int M, int nsb)
+    {
+        const size_t chunks = (size_t)(nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+        return (size_t)M * (chunks * 4096 + (size_t)nsb * 64);
+    }
+
+    // One thread per Q8_1 block.
+    template <int M>
+    __device__ __forceinline__ void quad_stage_q8(const uint32_t *__restrict__ q8, int nsb, uint8_t *aq, uint8_t *ads,
+                                                  int aq_stride, int ads_stride)
+    {
+        const int nkb = nsb * 8;
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+        {
+            for (int kb = threadIdx.x; kb < nkb; kb += blockDim.x)
+            {
+                const uint32_t *src = q8 + ((size_t)m * nkb + kb) * 9;
+                uint32_t v[9];
+#pragma unroll
+                for (int i = 0; i < 9; ++i)
+                    v[i] = src[i];
+                const float d = h2f((uint16_t)(v[0] & 0xFFFFu));
+                const int sb = kb >> 3, j = kb & 7, l = j >> 1, odd = j & 1;
+                *reinterpret_cast<float2 *>(ads + m * ads_stride + sb * 64 + l * 16 + odd * 8) =
+                    make_float2(d, (float)(int16_t)(v[0] >> 16) * d);
+                uint8_t *base = aq + m * aq_stride + (sb >> 4) * 4096 + (odd * 2) * 1024 + (sb & 15) * 64 + l * 16;
+                *reinterpret_cast<uint4 *>(base) = make_uint4(v[1], v[2], v[3], v[4]);
+                *reinterpret_cast<uint4 *>(base + 1024) = make_uint4(v[5], v[6], v[7], v[8]);
+            }
+        }
+    }
+
+    // ---- Q4_K ------------------------------------------------------------------------
+    // Super-block = 144 bytes: header piece {d, dmin, scales[12]} and four 32-byte groups;
+    // group l holds blocks 2l (low nibbles) and 2l+1 (high nibbles), element e in byte e
+    // (Q4_KTensor.cpp:768-792).  Effective scale f16(d*sc), min f16(-dmin*m) with the
+    // packer's fp16 rounding (Q4_KTensor.cpp:794-799, FP16Utils.h:75-118).
+    struct Q4KQuad
+    {
+        static constexpr int SB_BYTES = 144;
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+        struct Raw
+        {
+            v4i head, qa, qb;
+        };
+        static constexpr int LOADS = 3; // vector memory loads per Raw
+        struct Lane
+        {
+            uint32_t sel, m1, m2, m3;
+            int byte_off; // of this lane's group inside the super-block
+        };
+        struct Scale
+        {
+            h2 s; // {b_scale of block 2l, of block 2l+1}
+            h2 m; // {|b_min| ...}
+        };
+
+        __device__ __forceinline__ static Lane lane_consts(int l)
+        {
+            Lane c;
+            const uint32_t h = (uint32_t)(l & 1);
+            // bytes {2h, zero, 2h+1, zero} of a dword
+            c.sel = (2u * h) | (0x0Cu << 8) | ((2u * h + 1u) << 16) | (0x0Cu << 24);
+            c.m1 = (l < 2) ? 0x003F003Fu : 0u;
+            c.m2 = (l < 2) ? 0u : 0x00300030u;
+            c.m3 = (l < 2) ? 0u : 0x000F000Fu;
+            c.byte_off = 16 + 32 * l;
+            return c;
+        }
+
+        // sb: this lane's super-block, grp: the same plus the lane's group offset.  The
+        // loads are issued as assembly so that the kernel, not the compiler, decides where
+        // they are waited for (wait() below); the compiler would wait right after issue.
+        __device__ __forceinline__ static void load(Raw &r, const uint8_t *sb, const uint8_t *grp)
+        {
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.head) : "v"(sb));
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.qa) : "v"(grp));
+            asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=&v"(r.qb) : "v"(grp));
+        }
+        // Marks r's registers as in use up to this point (emits nothing).
+        __device__ __forceinline__ static void keep(Raw &r)
+        {
+            asm volatile("" : "+v"(r.head), "+v"(r.qa), "+v"(r.qb));
+        }
+        // Until at most `newer` vector memory operations issued after r's loads are pending.
+        template <int NEWER>
+        __device__ __forceinline__ static void wait(Raw &r)
+        {
+            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r.head), "+v"(r.qa), "+v"(r.qb) : "n"(NEWER));
+        }
+
+        __device__ __forceinline__ static uint16_t f16_trunc_bits(float x)
+        {
+            const uint32_t mag = (uint32_t)truncf(fabsf(x) * 16777216.0f);
+            return (uint16_t)(mag | ((__float_as_uint(x) >> 16) & 0x8000u));
+        }
+
+        // w[0], w[1]: elements 0-15, 16-31 of block 2l; w[2], w[3]: of block 2l+1.
+        __device__ __forceinline__ static void decode(const Raw &r, const Lane &c, v4i (&w)[4], Scale &S)
+        {
+            const uint32_t k = 0x0F0F0F0Fu;
+            w[0] = (v4i){(int)((uint32_t)r.qa.x & k), (int)((uint32_t)r.qa.y & k), (int)((uint32_t)r.qa.z & k), (int)((uint32_t)r.qa.w & k)};
+            w[1] = (v4i){(int)((uint32_t)r.qb.x & k), (int)((uint32_t)r.qb.y & k), (int)((uint32_t)r.qb.z & k), (int)((uint32_t)r.qb.w & k)};
+            w[2] = (v4i){(int)(((uint32_t)r.qa.x >> 4) & k), (int)(((uint32_t)r.qa.y >> 4) & k),
+                         (int)(((uint32_t)r.qa.z >> 4) & k), (int)(((uint32_t)r.qa.w >> 4) & k)};
+            w[3] = (v4i){(int)(((uint32_t)r.qb.x >> 4) & k), (int)(((uint32_t)r.qb.y >> 4) & k),
+                         (int)(((uint32_t)r.qb.z >> 4) & k), (int)(((uint32_t)r.qb.w >> 4) & k)};
+            // 6-bit scales / mins of blocks j0 = 2l, j1 = 2l+1 as two 16-bit integers each
+            // (get_scale_min_k4: j<4: q[j]&63, q[j+4]&63; else (q[j+4]&15)|((q[j-4]>>6)<<4),
+            // (q[j+4]>>4)|((q[j]>>6)<<4) -- SIMDHelpers.h:10791-10803)
+            const uint32_t A = __builtin_amdgcn_perm(0u, (uint32_t)r.head.y, c.sel);
+            const uint32_t B = __builtin_amdgcn_perm(0u, (uint32_t)r.head.z, c.sel);
+            const uint32_t P = __builtin_amdgcn_perm(0u, (uint32_t)r.head.w, c.sel);
+            const uint32_t bias = 0x64006400u; // fp16 1024.0: 0x6400|n is 1024+n
+            const uint32_t sc = (P & c.m3) | (((A >> 2) & c.m2) | ((A & c.m1) | bias));
+            const uint32_t mn = ((P >> 4) & c.m3) | (((B >> 2) & c.m2) | ((B & c.m1) | bias));
+            const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+            const h2 scf = __builtin_bit_cast(h2, sc) - k1024;
+            const h2 mnf = __builtin_bit_cast(h2, mn) - k1024;
+            const uint32_t hx = (uint32_t)r.head.x;
+            const h2 dd = __builtin_bit_cast(h2, hx); // {d, dmin}
+            // d (11-bit significand) times a 6-bit integer is exact before rounding, so the
+            // fp16 multiply equals f16(fp32 product) wherever the result is normal
+            S.s = (h2){dd.x, dd.x} * scf;
+            S.m = (h2){dd.y, dd.y} * mnf;
+            const uint32_t e = hx & 0x7C007C00u;
+            if (__builtin_expect(((e - 0x08000800u) & 0x80008000u) != 0u, 0))
+            {
+                // d or dmin below 2^-13: results may be fp16-subnormal, which the packer truncates
+                const float d = (float)dd.x, dmin = (float)dd.y;
+                uint32_t sb = __builtin_bit_cast(uint32_t, S.s), mb = __builtin_bit_cast(uint32_t, S.m);
+                const float s0 = d * (float)(sc & 0x3Fu), s1 = d * (float)((sc >> 16) & 0x3Fu);
+                const float m0 = dmin * (float)(mn & 0x3Fu), m1 = dmin * (float)((mn >> 16) & 0x3Fu);
+                if (fabsf(s0) < 6.103515625e-05f)
+                    sb = (sb & 0xFFFF0000u) | f16_trunc_bits(s0);
+                if (fabsf(s1) < 6.103515625e-05f)
+                    sb = (sb & 0x0000FFFFu) | ((uint32_t)f16_trunc_bits(s1) << 16);
+                if (fabsf(m0) < 6.103515625e-05f)
+                    mb = (mb & 0xFFFF0000u) | f16_trunc_bits(m0);
+                if (fabsf(m1) < 6.103515625e-05f)
+                    mb = (mb & 0x0000FFFFu) | ((uint32_t)f16_trunc_bits(m1) << 16);
+                S.s = __builtin_bit_cast(h2, sb);
+                S.m = __builtin_bit_cast(h2, mb);
+            }
+        }
+
+        // contribution of the lane's two blocks, added onto acc
+        __device__ __forceinline__ static float apply(const Scale &S, int idot0, int idot1, const float4 sd, float acc)
+        {
+            // sd = {d0, sum0*d0, d1, sum1*d1}
+            const float cs0 = fmaf(sd.x, (float)S.s.x, 0.0f);
+            const float cs1 = fmaf(sd.z, (float)S.s.y, 0.0f);
+            acc = fmaf((float)idot0, cs0, acc);
+            acc = fmaf(sd.y, -(float)S.m.x, acc);
+            acc = fmaf((float)idot1, cs1, acc);
+            acc = fmaf(sd.w, -(float)S.m.y, acc);
+            return acc;
+        }
+    };
+
+    // ---- kernel ----------------------------------------------------------------------
+
+    template <class Q, int M, int U>
+    __device__ __forceinline__ void quad_compute_step(const typename Q::Raw &r, const typename Q::Lane &lc,
+                                                      const uint8_t *aq_lane, const uint8_t *ads_lane, int aq_stride,
+                                                      int ads_stride, float (&t)[M])
+    {
+        v4i w[4];
+        typename Q::Scale S;
+        Q::decode(r, lc, w, S);
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+        {
+            const uint8_t *ap = aq_lane + m * aq_stride;
+            const v4i a0 = *reinterpret_cast<const v4i *>(ap);
+            const v4i a1 = *reinterpret_cast<const v4i *>(ap + 1024);
+            const v4i a2 = *reinterpret_cast<const v4i *>(ap + 2048);
+            const v4i a3 = *reinterpret_cast<const v4i *>(ap + 3072);
+            const float4 sd = *reinterpret_cast<const float4 *>(ads_lane + m * ads_stride);
+            const int idot0 = dot16(a1, w[1], dot16(a0, w[0], 0));
+            const int idot1 = dot16(a3, w[3], dot16(a2, w[2], 0));
+            t[m] = Q::apply(S, idot0, idot1, sd, 0.0f);
+        }
+    }
+
+    // Wait for step u of a chunk whose successor chunk has been issued after it.
+    template <class Q, int U>
+    __device__ __forceinline__ void wait_for(typename Q::Raw &r, int u)
+    {
+        // u is a compile-time constant after unrolling
+        switch (u)
+        {
+        case 0: Q::template wait<Q::LOADS *(2 * U - 1)>(r); break;
+        case 1: Q::template wait<Q::LOADS *(2 * U - 2)>(r); break;
+        case 2: Q::template wait<Q::LOADS *(2 * U - 3 > 0 ? 2 * U - 3 : 0)>(r); break;
+        case 3: Q::template wait<Q::LOADS *(2 * U - 4 > 0 ? 2 * U - 4 : 0)>(r); break;
+        default: Q::template wait<0>(r); break;
+        }
+    }
+
+    template <class Q, int M, int U>
+    __global__ void __launch_bounds__(quad_max_threads(M)) gemv_quad_kernel(const GemvArgs a)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
+        const int nsb = a.SB;
+        const int aq_stride = ((nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB) * 4096;
+        const int ads_stride = nsb * 64;
+        uint8_t *aq = quad_lds;
+        uint8_t *ads = quad_lds + M * aq_stride;
+
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int NW = (int)(blockDim.x >> 6);
+        const int l = lane & 3;
+        const int grp = lane >> 2;
+        const typename Q::Lane lc = Q::lane_consts(l);
+
+        // rows [r0, r1) of this wavefront: one run of `total` super-blocks
+        const long wid = (long)blockIdx.x * NW + wave;
+        const long r0 = wid * a.rows_per_wave;
+        long r1 = r0 + a.rows_per_wave;
+        if (r1 > a.N)
+            r1 = a.N;
+        const int total = r1 > r0 ? (int)(r1 - r0) * nsb : 0;
+        const int nsteps = (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+
+        // (an idle wavefront -- no rows left -- points at row 0 and uses nothing it loads)
+        const uint8_t *wp = static_cast<const uint8_t *>(a.w) + ((size_t)(total > 0 ? r0 : 0) * nsb + grp) * Q::SB_BYTES;
+        const uint8_t *const wp_safe = wp; // lanes past the end of the run re-read their first super-block
+        int ld_step = 0;
+        auto load_chunk = [&](typename Q::Raw(&buf)[U]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+            {
+                // no predicated loads: a load under a lane mask would be waited for at once
+                const uint8_t *p = wp + (size_t)u * (QUAD_STEP_SB * Q::SB_BYTES);
+                if ((ld_step + u) * QUAD_STEP_SB + grp >= total)
+                    p = wp_safe;
+                Q::load(buf[u], p, p + lc.byte_off);
+            }
+            wp += (size_t)U * (QUAD_STEP_SB * Q::SB_BYTES);
+            ld_step += U;
+        };
+
+        typename Q::Raw bufA[U], bufB[U];
+        load_chunk(bufA); // in flight while the activations are staged
+
+        quad_stage_q8<M>(a.q8, nsb, aq, ads, aq_stride, ads_stride);
+        __syncthreads();
+        // the staging code above must not reuse the registers of the loads in flight
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            Q::keep(bufA[u]);
+
+        float cur[M], nxt[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+            cur[m] = nxt[m] = 0.0f;
+
+        int first = 0;  // super-block (inside its row) that lane group 0 handles in this step
+        long row = r0;  // row `cur` belongs to
+        int step = 0;
+
+        auto compute_step = [&](const typename Q::Raw &r) {
+            int sbr = first + grp;
+            if (sbr >= nsb)
+                sbr -= nsb;
+            const uint8_t *aq_lane = aq + ((sbr >> 4) << 12) + ((sbr & 15) << 6) + (l << 4);
+            const uint8_t *ads_lane = ads + (sbr << 6) + (l << 4);
+            float t[M];
+            quad_compute_step<Q, M, U>(r, lc, aq_lane, ads_lane, aq_stride, ads_stride, t);
+
+            const int gb = nsb - first;                       // lane groups still in the current row
+            const int ge = total - step * QUAD_STEP_SB;       // lane groups with data at all
+            {
+                // one code shape for every step keeps cur/nxt in registers
+                const bool in_cur = grp < gb && grp < ge;
+                const bool in_nxt = grp >= gb && grp < ge;
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                {
+                    cur[m] += in_cur ? t[m] : 0.0f;
+                    nxt[m] += in_nxt ? t[m] : 0.0f;
+                }
+            }
+            if (gb <= QUAD_STEP_SB)
+            {
+                // the current row ends in this step
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                {
+                    const float tot = wave_sum(cur[m]);
+                    if (lane == 0)
+                    {
+                        float *dst = a.y + (size_t)m * a.ldy + row;
+                        *dst = a.accumulate ? (*dst + a.out_scale * tot) : a.out_scale * tot;
+                    }
+                    cur[m] = nxt[m];
+                    nxt[m] = 0.0f;
+                }
+                ++row;
+                first = QUAD_STEP_SB - gb;
+            }
+            else
+                first += QUAD_STEP_SB;
+            ++step;
+        };
+
+        // buf was loaded one chunk ago; the loads of the chunk after it (U steps) are in flight.
+        // Every buffer is waited for, also when its step lies past the end of the run: a
+        // register whose load is still in flight must not look free to the compiler.
+        auto compute_chunk = [&](typename Q::Raw(&buf)[U]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+            {
+                wait_for<Q, U>(buf[u], u);
+                if (step < nsteps) // uniform
+                    compute_step(buf[u]);
+            }
+        };
+
+        // The next chunk is loaded unconditionally (past the end of the run the lanes re-read
+        // their first super-block): a load under a condition would need register copies that
+        // wait for it straight away.
+        for (int c0 = 0; c0 < nsteps; c0 += 2 * U)
+        {
+            load_chunk(bufB);
+            compute_chunk(bufA);
+            __builtin_amdgcn_sched_barrier(0); // keep the loads below the last use of their registers
+            load_chunk(bufA);
+            compute_chunk(bufB);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the run
+    }
+
+    template <class Q, int M, int U>
+    inline void gemv_quad_launch_mu(dim3 grid, dim3 block, size_t lds, hipStream_t st, const GemvArgs &a)
+    {
+        static bool attr_set = false;
+        if (!attr_set)
+        {
+            // dynamic LDS beyond 64 KiB has to be allowed per kernel once
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U>), grid, block, lds, st, a);
+    }
+
+    template <class Q>
+    inline void gemv_quad_launch(int M, dim3 grid, dim3 block, size_t lds, hipStream_t st, const GemvArgs &a)
+    {
+        switch (M)
+        {
+        case 1: gemv_quad_launch_mu<Q, 1, 3>(grid, block, lds, st, a); break;
+        case 2: gemv_quad_launch_mu<Q, 2, 3>(grid, block, lds, st, a); break;
+        case 3: gemv_quad_launch_mu<Q, 3, 2>(grid, block, lds, st, a); break;
+        case 4: gemv_quad_launch_mu<Q, 4, 2>(grid, block, lds, st, a); break;
+        case 5: gemv_quad_launch_mu<Q, 5, 2>(grid, block, lds, st, a); break;
+        case 6: gemv_quad_launch_mu<Q, 6, 2>(grid, block, lds, st, a); break;
+        case 7: gemv_quad_launch_mu<Q, 7, 2>(grid, block, lds, st, a); break;
+        default: gemv_quad_launch_mu<Q, 8, 2>(grid, block, lds, st, a); break;
+        }
+    }
+
+    // Launch shape.  R, the rows one wavefront walks, fixes which lane handles which
+    // super-block of a row and with it the bits of the result, so it is chosen from N and
+    // nsb alone: every batch size then shares the row partition and a batch row is
+    // bit-identical to its single-row result.  The cost of a candidate is the number of
+    // steps the busiest SIMD unit runs one after another (a compute unit has four; its
+    // wavefronts are dealt round robin), which covers ragged last steps and uneven
+    // wavefront counts; measured, that tracks the kernel time as long as a compute unit
+    // has at least four wavefronts to keep loads in flight, two per SIMD unit being best.
+    struct QuadShape
+    {
+        int waves, rows_per_wave;
+        long grid;
+    };
+    inline QuadShape gemv_quad_shape(long N, int nsb, int cus, int max_waves)
+    {
+        const int rpw_override = gemv_rows_per_wave_override();
+        // the search below costs a microsecond or two: remember the last answers
+        struct Memo
+        {
+            long N;
+            int nsb, cus, max_waves, rpw;
+            QuadShape sh;
+        };
+        thread_local Memo memo[8] = {};
+        thread_local int memo_next = 0;
+        for (const Memo &e : memo)
+            if (e.N == N && e.nsb == nsb && e.cus == cus && e.max_waves == max_waves && e.rpw == rpw_override)
+                return e.sh;
+        int best_R = 1;
+        long best_wpc = 1;
+        double best_cost = 1e30;
+        for (int R = 1; R <= 512; ++R)
+        {
+            if (rpw_override > 0 && R != rpw_override)
+                continue;
+            const long steps = ((long)R * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+            const long waves = (N + R - 1) / R;
+            const long wpc = (waves + cus - 1) / cus; // wavefronts on the busiest compute unit
+            // at most 8 wavefronts of the widest variant fit a compute unit at once
+            const long rounds = (wpc + 7) / 8;
+            const long per_simd = rounds > 1 ? 2 * rounds : (wpc + 3) / 4;
+            double cost = (double)(per_simd * steps) / ((double)N * nsb / cus / (4.0 * QUAD_STEP_SB));
+            if (wpc < 4)
+                cost *= 1.0 + 0.25 * (double)(4 - wpc); // too few loads in flight
+            else if (wpc < 8)
+                cost *= 1.10;                           // one wavefront cannot keep a SIMD unit busy
+            if (steps < 4)
+                cost *= 1.0 + 0.10 * (double)(4 - steps); // short runs do not amortise their start
+            if (cost < best_cost - 1e-9)
+            {
+                best_cost = cost;
+                best_R = R;
+                best_wpc = wpc;
+            }
+            if (waves <= 1)
+                break;
+        }
+        QuadShape sh;
+        sh.rows_per_wave = best_R;
+        const long waves = (N + best_R - 1) / best_R;
+        const long wgs_per_cu = (best_wpc + max_waves - 1) / max_waves;
+        long nw = (best_wpc + wgs_per_cu - 1) / wgs_per_cu;
+        if (nw > waves)
+            nw = waves;
+        sh.waves = (int)(nw < 1 ? 1 : nw);
+        sh.grid = (waves + sh.waves - 1) / sh.waves;
+        memo[memo_next] = Memo{N, nsb, cus, max_waves, rpw_override, sh};
+        memo_next = (memo_next + 1) % 8;
+        return sh;
+    }
+} // namespace llamql

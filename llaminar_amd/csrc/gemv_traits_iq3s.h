@@ -66,6 +66,7 @@ namespace llamql
     {
         static constexpr bool PAIR = false;
         static constexpr bool HAS_MIN = false;
+        static constexpr bool USE_QUAD = false;
         static constexpr bool USE_STREAM = false;      // row-streaming kernel pays off for this format
         static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
         static constexpr int STREAM_MAX_THREADS = 1024; // workgroup size bound of the row-streaming kernel

@@ -11,6 +11,7 @@
 // (Q4_KTensor.cpp:794-799).  HBM-bound: 144 B per 256 weights.
 #pragma once
 #include "gemv_core.h"
+#include "gemv_quad.h"
 
 
 namespace llamql
@@ -19,6 +20,8 @@ namespace llamql
     {
         static constexpr bool PAIR = true;
         static constexpr bool HAS_MIN = true;
+        static constexpr bool USE_QUAD = true;        // quad-lane kernel for rows of >= 16 super-blocks
+        typedef Q4KQuad Quad;
         static constexpr bool USE_STREAM = true;      // row-streaming kernel pays off for this format
         static constexpr int FAST_MAX_U = 4;          // load batches in flight in the chunked kernel
         static constexpr int STREAM_MAX_THREADS = 1024; // workgroup size bound of the row-streaming kernel
