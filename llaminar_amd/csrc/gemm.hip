@@ -7,19 +7,22 @@
 // idot is formed by ONE v_mfma_i32_32x32x32_i8 per 32x32 output tile and K-block
 // (K depth 32 = exactly one Q8_1 block, zero accumulator input), so it is the
 // same exact integer the reference forms with vpdpbusd
-// (CPUNativeVNNIGemv.h:1046-1231); the per-block rescale is fp32 VALU work and
-// the rank-1 min term goes through v_mfma_f32_32x32x2f32 into its own
-// accumulator.
+// (CPUNativeVNNIGemv.h:1046-1231); the per-block rescale is fp32 VALU work (three
+// operations per output element and block: convert, scale product, multiply-add --
+// this, not the matrix unit, bounds the kernel) and the rank-1 min term goes
+// through v_mfma_f32_32x32x2f32 straight into the accumulator.
 //
-// Workgroup: 512 threads = 8 wavefronts, tile 128 tokens x 128 weight rows,
-// K advanced one 256-column super-block at a time.  Per step the weights of the
-// tile are decoded (nibble unpack / requantise, shared with the GEMV traits)
-// into LDS as int8 [row][k], the activations copied beside them, both with a
-// 272-byte row stride (conflict-free ds_read_b128 for MFMA operands).  Wavefront
-// w owns weight rows 32*(w%4).. and tokens 64*(w/4)..: two 32x32 MFMA tiles that
-// share the weight operand.  The MFMA's A operand is the activation tile, B the
-// weight tile, so a lane holds one weight row n and 16 tokens: stores of C are
-// 128-byte coalesced and b_scale is one register per block.
+// Workgroup: 512 threads = 8 wavefronts, tile 128 tokens x 64 weight rows, 64 KiB
+// of LDS, so two workgroups share a compute unit and one's staging overlaps the
+// other's multiply.  K advances one 256-column super-block at a time.  The global
+// data of a step (raw weight blocks, 72 bytes of Q8_1 per thread) is fetched into
+// registers while the previous step is multiplied; then the weights are decoded
+// (nibble unpack / requantise, shared with the GEMV decoders) into LDS as int8
+// [row][k], the activations copied beside them, both with a 272-byte row stride
+// (conflict-free ds_read_b128 for MFMA operands).  Wavefront w owns weight rows
+// 32*(w%2).. and tokens 32*(w/2)..: one 32x32 MFMA tile.  The MFMA's A operand is
+// the activation tile, B the weight tile, so a lane holds one weight row n and 16
+// tokens: stores of C are 128-byte coalesced and b_scale is one register per block.
 #include "gemv_traits_all.h"
 
 #include "llaminar_amd/ql_api.h"
@@ -29,7 +32,7 @@ namespace llamql
     typedef float v16f __attribute__((ext_vector_type(16)));
 
     constexpr int GEMM_BM = 128;        // tokens per workgroup
-    constexpr int GEMM_BN = 128;        // weight rows per workgroup
+    constexpr int GEMM_BN = 64;         // weight rows per workgroup
     constexpr int GEMM_THREADS = 512;
     constexpr int GEMM_STRIDE = 256 + 16; // bytes per LDS row (one super-block + pad)
 
@@ -44,11 +47,129 @@ namespace llamql
     template <class F>
     constexpr size_t gemm_lds_bytes()
     {
-        return (size_t)(GEMM_BM + GEMM_BN) * GEMM_STRIDE + (size_t)4 * 8 * 128 * sizeof(float) + F::TABLE_BYTES;
+        return (size_t)(GEMM_BM + GEMM_BN) * GEMM_STRIDE + (size_t)2 * 8 * (GEMM_BM + GEMM_BN) * sizeof(float) +
+               F::TABLE_BYTES;
     }
 
+    // Two adjacent Q8_1 blocks (72 bytes, 4-byte aligned) of one token, fetched with loads
+    // the kernel waits for itself: written as ordinary loads the compiler moves them down
+    // to their first use, behind the multiply they are meant to overlap.
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    struct GemmActRaw
+    {
+        v4i q0, q1, q2, q3;
+        v2i q4;
+        __device__ __forceinline__ void load(const uint32_t *p)
+        {
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(q0) : "v"(p));
+            asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=&v"(q1) : "v"(p));
+            asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=&v"(q2) : "v"(p));
+            asm volatile("global_load_dwordx4 %0, %1, off offset:48" : "=&v"(q3) : "v"(p));
+            asm volatile("global_load_dwordx2 %0, %1, off offset:64" : "=&v"(q4) : "v"(p));
+        }
+        // every load issued so far has arrived
+        __device__ __forceinline__ void wait()
+        {
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(q0), "+v"(q1), "+v"(q2), "+v"(q3), "+v"(q4));
+        }
+        __device__ __forceinline__ uint32_t dword(int i) const
+        {
+            // i is a compile-time constant after unrolling
+            return (uint32_t)(i < 4 ? q0[i] : i < 8 ? q1[i - 4] : i < 12 ? q2[i - 8] : i < 16 ? q3[i - 12] : q4[i - 16]);
+        }
+    };
+
+    // Weight data of one K step held in registers while the previous step is multiplied.
+    template <class F, bool QUAD = F::USE_QUAD>
+    struct GemmPrefetch;
+
+    // Formats with a quad-lane decoder: thread = (weight row, quad lane), 64 weights.
     template <class F>
-    __global__ void __launch_bounds__(GEMM_THREADS) gemm_kernel(const GemmArgs g)
+    struct GemmPrefetch<F, true>
+    {
+        typedef typename F::Quad Q;
+        typename Q::Raw raw;
+        typename Q::Lane lc;
+        const uint8_t *wp;
+        int row, l;
+        bool active; // wavefront-uniform: BN rows x 4 quad lanes = the first 4*BN threads
+
+        __device__ __forceinline__ void init(const GemmArgs &g, long n0, int tid)
+        {
+            active = __builtin_amdgcn_readfirstlane(tid) < GEMM_BN * 4;
+            row = (tid >> 2) & (GEMM_BN - 1);
+            l = tid & 3;
+            lc = Q::lane_consts(l);
+            long n = n0 + row;
+            if (n >= g.w.N)
+                n = g.w.N - 1; // tail rows: decode a valid row, never stored
+            wp = static_cast<const uint8_t *>(g.w.w) + (size_t)n * g.w.SB * Q::SB_BYTES;
+        }
+        __device__ __forceinline__ void issue(const GemmArgs &, int sb)
+        {
+            // the other wavefronts load the same bytes again (cache hits) and drop them: a
+            // load under a condition would need a register copy that waits for it at once
+            const uint8_t *p = wp + (size_t)sb * Q::SB_BYTES;
+            Q::load(raw, p, p + lc.byte_off);
+        }
+        __device__ __forceinline__ void store(uint8_t *Wl, float *bs, float *bm, const void *)
+        {
+            Q::template wait<0>(raw);
+            if (!active)
+                return;
+            v4i w[4];
+            typename Q::Scale S;
+            Q::decode(raw, lc, w, S);
+            v4i *dst = reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 64 * l);
+            dst[0] = w[0];
+            dst[1] = w[1];
+            dst[2] = w[2];
+            dst[3] = w[3];
+            bs[(2 * l) * GEMM_BN + row] = Q::scale_f32(S, 0);
+            bs[(2 * l + 1) * GEMM_BN + row] = Q::scale_f32(S, 1);
+            bm[(2 * l) * GEMM_BN + row] = Q::min_f32(S, 0);
+            bm[(2 * l + 1) * GEMM_BN + row] = Q::min_f32(S, 1);
+        }
+        __device__ __forceinline__ void finish() { Q::template wait<0>(raw); }
+    };
+
+    // Other formats: the 8-lane decode of the GEMV skeleton, one task per thread.
+    template <class F>
+    struct GemmPrefetch<F, false>
+    {
+        static_assert(GEMM_BN * 8 == GEMM_THREADS, "one (row, lane) task per thread");
+        typename F::Raw raw;
+        long n;
+        int row, c;
+
+        __device__ __forceinline__ void init(const GemmArgs &g, long n0, int tid)
+        {
+            row = tid >> 3;
+            c = tid & 7;
+            n = n0 + row;
+            if (n >= g.w.N)
+                n = g.w.N - 1;
+        }
+        __device__ __forceinline__ void issue(const GemmArgs &g, int sb) { raw = F::load(g.w, n, sb, c); }
+        __device__ __forceinline__ void store(uint8_t *Wl, float *bs, float *bm, const void *tab)
+        {
+            v4i w0, w1;
+            int j;
+            float bscale, bmin;
+            F::decode(raw, c, w0, w1, j, bscale, bmin, tab);
+            int j0, e0, j1, e1;
+            F::where(c, j0, e0, j1, e1);
+            *reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 32 * j0 + e0) = w0;
+            *reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 32 * j1 + e1) = w1;
+            bs[j * GEMM_BN + row] = bscale;
+            bm[j * GEMM_BN + row] = bmin;
+        }
+        __device__ __forceinline__ void finish() {}
+    };
+
+    template <class F>
+    __global__ void __launch_bounds__(GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
+        gemm_kernel(const GemmArgs g)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         uint8_t *Al = smem;                             // [BM][STRIDE] activations int8
@@ -65,8 +186,8 @@ namespace llamql
         const int tid = threadIdx.x;
         const int lane = tid & 63;
         const int wave = tid >> 6;
-        const int ntile = wave & 3;
-        const int mhalf = wave >> 2;
+        const int ntile = wave & 1;
+        const int mtile = wave >> 1;
         const int l32 = lane & 31;
         const int lh = lane >> 5;
 
@@ -74,124 +195,115 @@ namespace llamql
         const long m0 = (long)blockIdx.y * GEMM_BM;
         const int KB = g.w.SB * 8;
 
-        v16f acc[2], accmin[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-            {
-                acc[t][r] = 0.0f;
-                accmin[t][r] = 0.0f;
-            }
+        // activations: thread = (token, pair of adjacent Q8_1 blocks) -> 72 contiguous bytes
+        const int am = tid >> 2;
+        const int ap = tid & 3;
+        long am_src = m0 + am;
+        if (am_src >= g.M)
+            am_src = g.M - 1; // tail tokens: a valid row, never stored
+        const uint32_t *asrc = g.q8 + ((size_t)am_src * KB + 2 * ap) * 9;
+        GemmActRaw areg;
 
+        GemmPrefetch<F> pf;
+        pf.init(g, n0, tid);
+
+        auto issue = [&](int sb) {
+            pf.issue(g, sb);
+            areg.load(asrc + (size_t)sb * 72);
+        };
+
+        v16f acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            acc[r] = 0.0f;
+
+        issue(0);
         for (int sb = 0; sb < g.w.SB; ++sb)
         {
             __syncthreads(); // previous step's LDS reads (and the table staging) are done
 
-            // ---- weights: 128 rows x 8 lanes each -> int8 + scales -------------------
+            // ---- registers -> LDS: weights as int8 [row][k] + scales, activations beside them
+            pf.store(Wl, bs, bm, tab);
+            areg.wait();
 #pragma unroll
-            for (int it = 0; it < (GEMM_BN * 8) / GEMM_THREADS; ++it)
+            for (int i = 0; i < 2; ++i)
             {
-                const int task = tid + it * GEMM_THREADS;
-                const int row = task >> 3;
-                const int c = task & 7;
-                long n = n0 + row;
-                if (n >= g.w.N)
-                    n = g.w.N - 1; // tail rows: decode a valid row, never stored
-                const typename F::Raw raw = F::load(g.w, n, sb, c);
-                v4i w0, w1;
-                int j;
-                float bscale, bmin;
-                F::decode(raw, c, w0, w1, j, bscale, bmin, tab);
-                int j0, e0, j1, e1;
-                F::where(c, j0, e0, j1, e1);
-                *reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 32 * j0 + e0) = w0;
-                *reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 32 * j1 + e1) = w1;
-                bs[j * GEMM_BN + row] = bscale;
-                bm[j * GEMM_BN + row] = bmin;
-            }
-
-            // ---- activations: 128 tokens x 8 blocks x 9 dwords ------------------------
-#pragma unroll
-            for (int it = 0; it < (GEMM_BM * 72) / GEMM_THREADS; ++it)
-            {
-                const int i = tid + it * GEMM_THREADS;
-                const int m = i / 72;
-                const int rem = i - m * 72;
-                const int kb = rem / 9;
-                const int r = rem - kb * 9;
-                uint32_t v = 0;
-                if (m0 + m < g.M)
-                    v = g.q8[((size_t)(m0 + m) * KB + (size_t)sb * 8 + kb) * 9 + r];
-                if (r == 0)
-                {
-                    const float d = h2f((uint16_t)(v & 0xFFFFu));
-                    ad[kb * GEMM_BM + m] = d;
-                    asd[kb * GEMM_BM + m] = (float)(int16_t)(v >> 16) * d;
-                }
-                else
-                {
-                    *reinterpret_cast<uint32_t *>(Al + m * GEMM_STRIDE + kb * 32 + (r - 1) * 4) = v;
-                }
+                const uint32_t h = areg.dword(9 * i);
+                const float d = h2f((uint16_t)(h & 0xFFFFu));
+                const int kb = 2 * ap + i;
+                ad[kb * GEMM_BM + am] = d;
+                asd[kb * GEMM_BM + am] = (float)(int16_t)(h >> 16) * d;
+                v4i *dst = reinterpret_cast<v4i *>(Al + am * GEMM_STRIDE + kb * 32);
+                dst[0] = (v4i){(int)areg.dword(9 * i + 1), (int)areg.dword(9 * i + 2), (int)areg.dword(9 * i + 3),
+                               (int)areg.dword(9 * i + 4)};
+                dst[1] = (v4i){(int)areg.dword(9 * i + 5), (int)areg.dword(9 * i + 6), (int)areg.dword(9 * i + 7),
+                               (int)areg.dword(9 * i + 8)};
             }
             __syncthreads();
 
+            // ---- next step's global data travels while this one is multiplied (the last
+            //      step re-reads itself: every issued load is consumed, none is conditional)
+            issue(sb + 1 < g.w.SB ? sb + 1 : sb);
+
             // ---- multiply ------------------------------------------------------------------
+            // 8 block products per step.  The MFMA of product kb+1 is issued before product kb
+            // is rescaled, so the matrix unit and the VALU work side by side: the results
+            // alternate between two register sets.
             const uint8_t *wrow = Wl + (ntile * 32 + l32) * GEMM_STRIDE + lh * 16;
-            const uint8_t *arow = Al + (mhalf * 64 + l32) * GEMM_STRIDE + lh * 16;
+            const uint8_t *arow = Al + (mtile * 32 + l32) * GEMM_STRIDE + lh * 16;
+            v16i zero;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                zero[r] = 0;
+            auto product = [&](int kb) {
+                const v4i bw = *reinterpret_cast<const v4i *>(wrow + kb * 32);
+                const v4i aa = *reinterpret_cast<const v4i *>(arow + kb * 32);
+                return __builtin_amdgcn_mfma_i32_32x32x32_i8(aa, bw, zero, 0, 0, 0);
+            };
+            v16i idot[2];
+            idot[0] = product(0);
 #pragma unroll
             for (int kb = 0; kb < 8; ++kb)
             {
-                const v4i bw = *reinterpret_cast<const v4i *>(wrow + kb * 32);
+                if (kb + 1 < 8)
+                    idot[(kb + 1) & 1] = product(kb + 1);
                 const float bscale = bs[kb * GEMM_BN + ntile * 32 + l32];
+                const float *adp = ad + kb * GEMM_BM + mtile * 32 + 4 * lh;
+                const v16i d = idot[kb & 1];
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
+                for (int q = 0; q < 4; ++q)
                 {
-                    const v4i aa = *reinterpret_cast<const v4i *>(arow + t * 32 * GEMM_STRIDE + kb * 32);
-                    v16i zero;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        zero[r] = 0;
-                    const v16i idot = __builtin_amdgcn_mfma_i32_32x32x32_i8(aa, bw, zero, 0, 0, 0);
-                    const float *adp = ad + kb * GEMM_BM + mhalf * 64 + t * 32 + 4 * lh;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                    {
-                        const float4 a4 = *reinterpret_cast<const float4 *>(adp + 8 * q);
-                        acc[t][4 * q + 0] = fmaf((float)idot[4 * q + 0], a4.x * bscale, acc[t][4 * q + 0]);
-                        acc[t][4 * q + 1] = fmaf((float)idot[4 * q + 1], a4.y * bscale, acc[t][4 * q + 1]);
-                        acc[t][4 * q + 2] = fmaf((float)idot[4 * q + 2], a4.z * bscale, acc[t][4 * q + 2]);
-                        acc[t][4 * q + 3] = fmaf((float)idot[4 * q + 3], a4.w * bscale, acc[t][4 * q + 3]);
-                    }
+                    const float4 a4 = *reinterpret_cast<const float4 *>(adp + 8 * q);
+                    acc[4 * q + 0] = fmaf((float)d[4 * q + 0], a4.x * bscale, acc[4 * q + 0]);
+                    acc[4 * q + 1] = fmaf((float)d[4 * q + 1], a4.y * bscale, acc[4 * q + 1]);
+                    acc[4 * q + 2] = fmaf((float)d[4 * q + 2], a4.z * bscale, acc[4 * q + 2]);
+                    acc[4 * q + 3] = fmaf((float)d[4 * q + 3], a4.w * bscale, acc[4 * q + 3]);
                 }
                 if (F::HAS_MIN && (kb & 1))
                 {
-                    // rank-2 update over blocks kb-1, kb: lane half lh supplies block kb-1+lh
+                    // rank-2 update over blocks kb-1, kb, straight into the accumulator: lane
+                    // half lh supplies block kb-1+lh
                     const int kk = kb - 1 + lh;
                     const float bmin = bm[kk * GEMM_BN + ntile * 32 + l32];
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-                    {
-                        const float av = asd[kk * GEMM_BM + mhalf * 64 + t * 32 + l32];
-                        accmin[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bmin, accmin[t], 0, 0, 0);
-                    }
+                    const float av = asd[kk * GEMM_BM + mtile * 32 + l32];
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bmin, acc, 0, 0, 0);
                 }
             }
         }
+        pf.finish();
+        areg.wait();
 
-        // ---- store: lane holds weight row n, 16 tokens per tile --------------------------
+        // ---- store: lane holds weight row n, 16 tokens -------------------------------------
         const long n = n0 + ntile * 32 + l32;
         if (n < g.w.N)
         {
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                {
-                    const long m = m0 + mhalf * 64 + t * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                    if (m < g.M)
-                        g.y[(size_t)m * g.ldy + n] = F::HAS_MIN ? (acc[t][r] + accmin[t][r]) : acc[t][r];
-                }
+            for (int r = 0; r < 16; ++r)
+            {
+                const long m = m0 + mtile * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                if (m < g.M)
+                    g.y[(size_t)m * g.ldy + n] = acc[r];
+            }
         }
     }
 

@@ -182,6 +182,10 @@ namespace llamql
             }
         }
 
+        // effective scale / min (fp32 value of the fp16 the packer stores) of block 2l+i
+        __device__ __forceinline__ static float scale_f32(const Scale &S, int i) { return i ? (float)S.s.y : (float)S.s.x; }
+        __device__ __forceinline__ static float min_f32(const Scale &S, int i) { return i ? -(float)S.m.y : -(float)S.m.x; }
+
         // contribution of the lane's two blocks, added onto acc
         __device__ __forceinline__ static float apply(const Scale &S, int idot0, int idot1, const float4 sd, float acc)
         {
