@@ -35,6 +35,10 @@ namespace llamql
     constexpr int GEMM_BN = 64;         // weight rows per workgroup
     constexpr int GEMM_THREADS = 512;
     constexpr int GEMM_STRIDE = 256 + 16; // bytes per LDS row (one super-block + pad)
+    // per-block scale tables [8][rows + 8]: the pad spreads the four threads that write one
+    // row's scales of different blocks over different banks
+    constexpr int GEMM_SM = GEMM_BM + 8;
+    constexpr int GEMM_SN = GEMM_BN + 8;
 
     struct GemmArgs
     {
@@ -47,7 +51,7 @@ namespace llamql
     template <class F>
     constexpr size_t gemm_lds_bytes()
     {
-        return (size_t)(GEMM_BM + GEMM_BN) * GEMM_STRIDE + (size_t)2 * 8 * (GEMM_BM + GEMM_BN) * sizeof(float) +
+        return (size_t)(GEMM_BM + GEMM_BN) * GEMM_STRIDE + (size_t)2 * 8 * (GEMM_SM + GEMM_SN) * sizeof(float) +
                F::TABLE_BYTES;
     }
 
@@ -125,10 +129,10 @@ namespace llamql
             dst[1] = w[1];
             dst[2] = w[2];
             dst[3] = w[3];
-            bs[(2 * l) * GEMM_BN + row] = Q::scale_f32(S, 0);
-            bs[(2 * l + 1) * GEMM_BN + row] = Q::scale_f32(S, 1);
-            bm[(2 * l) * GEMM_BN + row] = Q::min_f32(S, 0);
-            bm[(2 * l + 1) * GEMM_BN + row] = Q::min_f32(S, 1);
+            bs[(2 * l) * GEMM_SN + row] = Q::scale_f32(S, 0);
+            bs[(2 * l + 1) * GEMM_SN + row] = Q::scale_f32(S, 1);
+            bm[(2 * l) * GEMM_SN + row] = Q::min_f32(S, 0);
+            bm[(2 * l + 1) * GEMM_SN + row] = Q::min_f32(S, 1);
         }
         __device__ __forceinline__ void finish() { Q::template wait<0>(raw); }
     };
@@ -161,8 +165,8 @@ namespace llamql
             F::where(c, j0, e0, j1, e1);
             *reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 32 * j0 + e0) = w0;
             *reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 32 * j1 + e1) = w1;
-            bs[j * GEMM_BN + row] = bscale;
-            bm[j * GEMM_BN + row] = bmin;
+            bs[j * GEMM_SN + row] = bscale;
+            bm[j * GEMM_SN + row] = bmin;
         }
         __device__ __forceinline__ void finish() {}
     };
@@ -174,11 +178,11 @@ namespace llamql
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         uint8_t *Al = smem;                             // [BM][STRIDE] activations int8
         uint8_t *Wl = Al + GEMM_BM * GEMM_STRIDE;       // [BN][STRIDE] weights int8
-        float *ad = reinterpret_cast<float *>(Wl + GEMM_BN * GEMM_STRIDE); // [8][BM]
-        float *asd = ad + 8 * GEMM_BM;                  // [8][BM]
-        float *bs = asd + 8 * GEMM_BM;                  // [8][BN]
-        float *bm = bs + 8 * GEMM_BN;                   // [8][BN]
-        void *tab = bm + 8 * GEMM_BN;
+        float *ad = reinterpret_cast<float *>(Wl + GEMM_BN * GEMM_STRIDE); // [8][SM]
+        float *asd = ad + 8 * GEMM_SM;                  // [8][SM]
+        float *bs = asd + 8 * GEMM_SM;                  // [8][SN]
+        float *bm = bs + 8 * GEMM_SN;                   // [8][SN]
+        void *tab = bm + 8 * GEMM_SN;
 
         if (F::TABLE_BYTES > 0)
             F::stage_tables(tab);
@@ -231,8 +235,8 @@ namespace llamql
                 const uint32_t h = areg.dword(9 * i);
                 const float d = h2f((uint16_t)(h & 0xFFFFu));
                 const int kb = 2 * ap + i;
-                ad[kb * GEMM_BM + am] = d;
-                asd[kb * GEMM_BM + am] = (float)(int16_t)(h >> 16) * d;
+                ad[kb * GEMM_SM + am] = d;
+                asd[kb * GEMM_SM + am] = (float)(int16_t)(h >> 16) * d;
                 v4i *dst = reinterpret_cast<v4i *>(Al + am * GEMM_STRIDE + kb * 32);
                 dst[0] = (v4i){(int)areg.dword(9 * i + 1), (int)areg.dword(9 * i + 2), (int)areg.dword(9 * i + 3),
                                (int)areg.dword(9 * i + 4)};
@@ -267,8 +271,8 @@ namespace llamql
             {
                 if (kb + 1 < 8)
                     idot[(kb + 1) & 1] = product(kb + 1);
-                const float bscale = bs[kb * GEMM_BN + ntile * 32 + l32];
-                const float *adp = ad + kb * GEMM_BM + mtile * 32 + 4 * lh;
+                const float bscale = bs[kb * GEMM_SN + ntile * 32 + l32];
+                const float *adp = ad + kb * GEMM_SM + mtile * 32 + 4 * lh;
                 const v16i d = idot[kb & 1];
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
@@ -284,8 +288,8 @@ namespace llamql
                     // rank-2 update over blocks kb-1, kb, straight into the accumulator: lane
                     // half lh supplies block kb-1+lh
                     const int kk = kb - 1 + lh;
-                    const float bmin = bm[kk * GEMM_BN + ntile * 32 + l32];
-                    const float av = asd[kk * GEMM_BM + mtile * 32 + l32];
+                    const float bmin = bm[kk * GEMM_SN + ntile * 32 + l32];
+                    const float av = asd[kk * GEMM_SM + mtile * 32 + l32];
                     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bmin, acc, 0, 0, 0);
                 }
             }
