@@ -188,3 +188,35 @@ def test_error_paths(capi, dev):
     assert not lib.llam_ql_gemv(FMT_Q4_K, w.data_ptr(), w.data_ptr(), None, 1, 4, 256, 4, 0, None)
     assert not lib.llam_ql_gemv_block_sums(FMT_Q4_K, w.data_ptr(), w.data_ptr(), y.data_ptr(), 1, 4, 256, 2, 3, 0, None)
     assert "row window" in capi.last_error()
+
+
+@pytest.mark.parametrize("N,K", [(1, 4096), (37, 4096), (250, 4352), (129, 5120), (64, 8192), (19, 25600)])
+def test_q4k_long_rows_all_batches(capi, dev, oracle, N, K):
+    """Rows of 16 and more super-blocks take the kernel that walks a wavefront's rows as one
+    run: row ends inside a step (K/256 not a multiple of 16), ragged last steps, wavefronts
+    without rows, every batch size; a batch row equals the single-row result bit for bit."""
+    import torch
+
+    fmt = FMT_Q4_K
+    W = synth.weights_numpy(fmt, N, K, 31 + N)
+    q8 = oracle.quantize(synth.activations_numpy(8, K, 7 + N))
+    wd = upload_weights(capi, dev, fmt, W)
+    qd = upload_q8(dev, q8)
+    C = oracle.gemm(fmt, W, K, q8)
+    y1 = [capi.gemv(fmt, wd, upload_q8(dev, q8[m:m + 1]), 1, N, K) for m in range(8)]
+    for M in range(1, 9):
+        y = capi.gemv(fmt, wd, qd, M, N, K)
+        sync()
+        assert rel_err(y.cpu().numpy(), C[:M]) <= TOL[fmt] * 1e-2, M
+        for m in range(M):
+            assert torch.equal(y[m], y1[m][0]), (M, m)
+    lib = capi.load()
+    try:
+        # another row partition moves rows to other lanes: same values up to summation order
+        for rpw in (1, 2, 5, 64):
+            lib.llam_ql_set_gemv_tuning(rpw, 0)
+            y = capi.gemv(fmt, wd, qd, 3, N, K)
+            sync()
+            assert rel_err(y.cpu().numpy(), C[:3]) <= TOL[fmt] * 1e-2, rpw
+    finally:
+        lib.llam_ql_reset_gemv_tuning()
