@@ -51,9 +51,9 @@ int llam_ql_abi_version(void);
 
 /* Tuning overrides for sweeps (reference: rocmGemv_native_vnni_set_tuning_overrides /
  * ..._reset_tuning_overrides, ROCmGemvKernel_native_VNNI.hip:182-196).
- * rows_per_wave: row batches one wavefront walks; unroll: 1..4 forces the chunked
- * kernel with that many load batches in flight instead of the row-streaming
- * kernel.  Values <= 0 restore the built-in choice.  Not thread-safe. */
+ * rows_per_wave: rows (row batches) one wavefront walks; unroll: 1..4 forces the
+ * chunked kernel with that many load batches in flight, also where the quad-lane
+ * kernel would be used.  Values <= 0 restore the built-in choice.  Not thread-safe. */
 void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll);
 void llam_ql_reset_gemv_tuning(void);
 
@@ -140,6 +140,16 @@ bool llam_ql_epilogue(float *d_c, const float *d_t, const float *d_bias, int M,
 bool llam_ql_moe_route(const float *d_logits, int n_tokens, int n_experts,
                        int top_k, int normalize, int32_t *d_ids,
                        float *d_weights, int device_id, void *stream);
+
+/* Same with the slots of a token slot_stride (>= top_k) entries apart in d_ids and
+ * d_weights: columns top_k.. are left alone, so a caller can keep always-on experts
+ * (the shared expert of MoEExpertComputeStage.cpp:1450-1708, weight 1 or its sigmoid
+ * gate) in them and run routed and shared experts through one gate/up and one down
+ * launch with top_k = slot_stride. */
+bool llam_ql_moe_route_ex(const float *d_logits, int n_tokens, int n_experts,
+                          int top_k, int normalize, int32_t *d_ids,
+                          float *d_weights, int slot_stride, int device_id,
+                          void *stream);
 
 /* Expert weight table on the device: one entry per expert id (reference:
  * DeviceNativeVNNIMatrixDesc tables, src/v2/tensors/TensorKernels.h:39-55,

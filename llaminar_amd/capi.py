@@ -50,6 +50,7 @@ SIGNATURES = {
     "llam_ql_gemm": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_epilogue": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int,
                                   c_void_p]),
+    "llam_ql_moe_route_ex": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "llam_ql_moe_route": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "llam_ql_moe_gate_up": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                      c_int, c_int, c_int, c_void_p]),
@@ -197,15 +198,19 @@ def epilogue(c, t, bias, alpha: float, beta: float, stream=None):
     return c
 
 
-def moe_route(logits, top_k: int, normalize: bool = True, stream=None):
+def moe_route(logits, top_k: int, normalize: bool = True, stream=None, ids=None, weights=None):
+    """Top-k routing.  With preallocated ids / weights [T, S >= top_k] only the first top_k
+    columns are written (the rest can hold always-on experts such as a shared expert)."""
     import torch
 
     T, E = logits.shape
-    ids = torch.empty(T, top_k, dtype=torch.int32, device=logits.device)
-    wts = torch.empty(T, top_k, dtype=torch.float32, device=logits.device)
-    _check(load().llam_ql_moe_route(_ptr(logits), T, E, top_k, int(normalize), _ptr(ids), _ptr(wts), _dev(logits),
-                                    _stream(stream)), "moe_route")
-    return ids, wts
+    if ids is None:
+        ids = torch.empty(T, top_k, dtype=torch.int32, device=logits.device)
+        weights = torch.empty(T, top_k, dtype=torch.float32, device=logits.device)
+    assert ids.shape == weights.shape and ids.shape[0] == T and ids.is_contiguous() and weights.is_contiguous()
+    _check(load().llam_ql_moe_route_ex(_ptr(logits), T, E, top_k, int(normalize), _ptr(ids), _ptr(weights),
+                                       ids.shape[1], _dev(logits), _stream(stream)), "moe_route")
+    return ids, weights
 
 
 def expert_table(experts, device):

@@ -1,7 +1,6 @@
 // Decode GEMV launchers: one instantiation of the shared skeleton per weight format.
 #include "gemv_traits_all.h"
 #include "gemv_fast.h"
-#include "gemv_stream.h"
 
 #include "llaminar_amd/ql_api.h"
 

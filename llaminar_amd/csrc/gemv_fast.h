@@ -1,5 +1,6 @@
-// Full-row decode GEMV (gfx950): the streaming kernel used whenever a weight row
-// spans at least five super-blocks, i.e. for every dense-layer projection.
+// Chunked full-row decode GEMV (gfx950): rows of at least five super-blocks in
+// formats without a quad-lane decoder (Q6_K, IQ3_S), Q4_K rows shorter than 16
+// super-blocks, and the host-side launcher that picks a kernel for every shape.
 //
 // Same arithmetic and lane roles as the generic skeleton in gemv_core.h; what
 // differs is how the work is fed:
@@ -236,54 +237,6 @@ namespace llamql
     }
 
     int gemv_unroll_override();
-    bool gemv_stream_enabled();
-
-    // defined in gemv_stream.h
-    template <class F>
-    inline void gemv_stream_launch(int M, int RP, int waves, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a);
-    int gemv_stream_max_waves();
-
-    // Workgroup shape for `npass` passes: one workgroup per compute unit when there is
-    // enough work, `waves` wavefronts of `ppw` passes each, chosen to pad the per-CU
-    // share as little as possible (every CU then finishes at the same time).
-    struct StreamShape
-    {
-        int waves, ppw;
-        long grid;
-    };
-    inline StreamShape gemv_stream_shape(long npass, int cus, int max_waves)
-    {
-        StreamShape sh;
-        const long per_cu = (npass + cus - 1) / cus;
-        int ppw_override = gemv_rows_per_wave_override();
-        long best_pad = 1L << 60;
-        sh.waves = 4;
-        sh.ppw = 1;
-        for (int w = max_waves; w >= 2; --w)
-        {
-            long ppw = (per_cu + w - 1) / w;
-            if (ppw_override > 0)
-                ppw = ppw_override;
-            if (ppw > 64)
-                continue;
-            const long cap = (long)w * ppw;
-            if (cap < per_cu && ppw_override <= 0)
-                continue;
-            // padding, with a mild preference for at least 8 wavefronts
-            long pad = (cap >= per_cu ? cap - per_cu : 0) * 16 + (w < 8 ? (8 - w) : 0);
-            if (pad < best_pad)
-            {
-                best_pad = pad;
-                sh.waves = w;
-                sh.ppw = (int)ppw;
-            }
-        }
-        const long per_wg = (long)sh.waves * sh.ppw;
-        sh.grid = (npass + per_wg - 1) / per_wg;
-        return sh;
-    }
-
-
     // Launch shape for N rows of nsb super-blocks (one LDS slice) on a device with
     // `cus` compute units.  Rows are dealt to workgroups so that every compute unit
     // receives (nearly) the same number of rows in a single round of workgroups.
@@ -415,39 +368,6 @@ namespace llamql
             slice = SB;
         if (slice < 1)
             return fail(fn, "activation rows do not fit LDS (M=%d)", M);
-        // Whole rows of 8k or 8k+4 super-blocks in one LDS slice: the row-streaming kernel.
-        if constexpr (F::USE_STREAM)
-        if (M <= 2 && !dump && slice == SB && gemv_stream_enabled())
-        {
-            // RP = 1: rows of 8k super-blocks; RP = 2: row pairs of 8k+4 super-blocks
-            const int RP = (SB % 8 == 0) ? 1 : ((SB % 8 == 4 && SB > 4 && (N % 2) == 0) ? 2 : 0);
-            if (RP != 0)
-            {
-                const StreamShape ps = gemv_stream_shape(N / RP, cu_count(device_id),
-                                                           gemv_stream_max_waves() < F::STREAM_MAX_THREADS / WAVE
-                                                               ? gemv_stream_max_waves()
-                                                               : F::STREAM_MAX_THREADS / WAVE);
-                GemvArgs a;
-                a.w = d_w;
-                a.q8 = static_cast<const uint32_t *>(d_q8);
-                a.y = d_y;
-                a.sums = nullptr;
-                a.ldy = ldy;
-                a.N = N;
-                a.SB = SB;
-                a.sb0 = 0;
-                a.nsb = SB;
-                a.rows_per_wave = ps.ppw; // passes per wavefront
-                a.gshift = 3;
-                a.accumulate = 0;
-                a.out_scale = 1.0f;
-                a.row0 = 0;
-                a.nrows = 0;
-                gemv_stream_launch<F>(M, RP, ps.waves, dim3((unsigned)ps.grid), gemv_lds_bytes<F>(M, SB), st, a);
-                return launched(fn);
-            }
-        }
-
         GemvShape sh = gemv_shape(N, slice, cu_count(device_id));
         if (gemv_unroll_override() <= 0 && sh.U > F::FAST_MAX_U)
             sh.U = F::FAST_MAX_U;

@@ -67,11 +67,7 @@ namespace llamql
         static constexpr bool PAIR = false;
         static constexpr bool HAS_MIN = false;
         static constexpr bool USE_QUAD = false;
-        static constexpr bool USE_STREAM = false;      // row-streaming kernel pays off for this format
         static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
-        static constexpr int STREAM_MAX_THREADS = 1024; // workgroup size bound of the row-streaming kernel
-        static constexpr int STREAM_U_PAIR = 5;   // loads per lane and chunk, row-pair passes
-        static constexpr int STREAM_U_SINGLE = 4; // ... single-row passes
         static constexpr int TABLE_BYTES = (int)sizeof(IQ3STables);
 
         __device__ static void stage_tables(void *lds_tab)
@@ -83,11 +79,12 @@ namespace llamql
                 dst[i] = src[i];
         }
 
-        struct Raw
+        struct Raw // no padding between members: arrays of it stay in registers
         {
+            uint4 meta;
             uint2 qs;
             uint32_t signs;
-            uint4 meta;
+            uint32_t spare;
         };
 
         // natural layout: block j is unit j, dword q at position q
@@ -110,6 +107,7 @@ namespace llamql
             const size_t t = (size_t)row * a.SB + sb;
             const uint8_t *base = static_cast<const uint8_t *>(a.w);
             Raw r;
+            r.spare = 0;
             r.qs = reinterpret_cast<const uint2 *>(base)[t * 8 + c];
             r.signs = reinterpret_cast<const uint32_t *>(base + T * 64)[t * 8 + c];
             r.meta = reinterpret_cast<const uint4 *>(base + T * 96)[t];
@@ -122,7 +120,10 @@ namespace llamql
             const uint32_t *req = static_cast<const uint32_t *>(tab);
             const uint8_t *gmaxb = reinterpret_cast<const uint8_t *>(req + 8 * 512);
 
-            const uint32_t qh = (((c & 4) ? r.meta.y : r.meta.x) >> (8 * (c & 3))) & 0xFFu;
+            // picked with a bit mask: a conditional on two members of r would become a load
+            // through a computed address and force arrays of Raw into memory
+            const uint32_t m4 = (uint32_t)0 - (uint32_t)((c >> 2) & 1);
+            const uint32_t qh = ((((r.meta.y & m4) | (r.meta.x & ~m4))) >> (8 * (c & 3))) & 0xFFu;
             const uint32_t nib = (r.meta.z >> (4 * c)) & 0xFu; // scales[c/2], low nibble for even c
             const float d = h2f((uint16_t)(r.meta.w & 0xFFFFu));
 
@@ -216,22 +217,5 @@ namespace llamql
             int j;
             decode(r, l.c, w0, w1, j, bscale, bmin, tab);
         }
-
-        // ---- row-streaming kernel interface (generic form) -------------------------------
-        struct Scale
-        {
-            float bs;
-        };
-        typedef Lane Lane3;
-        __device__ __forceinline__ static Lane3 lane3_consts(int c) { return lane_consts(c); }
-        __device__ __forceinline__ static void decode3(const Raw &r, const Lane3 &l, v4i &w0, v4i &w1, Scale &S,
-                                                       const void *tab)
-        {
-            int j;
-            float bmin;
-            decode(r, l.c, w0, w1, j, S.bs, bmin, tab);
-        }
-        __device__ __forceinline__ static float cs(const Scale &S, float ad) { return ad * S.bs; }
-        __device__ __forceinline__ static float add_min(const Scale &, float, float acc) { return acc; }
     };
 } // namespace llamql

@@ -49,11 +49,7 @@ namespace llamql
         static constexpr bool PAIR = true;
         static constexpr bool HAS_MIN = false; // the reference's mins plane is all zero for Q6_K
         static constexpr bool USE_QUAD = false;
-        static constexpr bool USE_STREAM = false;      // row-streaming kernel pays off for this format
         static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
-        static constexpr int STREAM_MAX_THREADS = 1024; // workgroup size bound of the row-streaming kernel
-        static constexpr int STREAM_U_PAIR = 2;   // loads per lane and chunk, row-pair passes
-        static constexpr int STREAM_U_SINGLE = 2; // ... single-row passes
         static constexpr int TABLE_BYTES = 0;
         __device__ static void stage_tables(void *) {}
 
@@ -215,22 +211,5 @@ namespace llamql
             int j;
             decode(r, l.c, w0, w1, j, bscale, bmin, tab);
         }
-
-        // ---- row-streaming kernel interface (generic form) -------------------------------
-        struct Scale
-        {
-            float bs;
-        };
-        typedef Lane Lane3;
-        __device__ __forceinline__ static Lane3 lane3_consts(int c) { return lane_consts(c); }
-        __device__ __forceinline__ static void decode3(const Raw &r, const Lane3 &l, v4i &w0, v4i &w1, Scale &S,
-                                                       const void *tab)
-        {
-            int j;
-            float bmin;
-            decode(r, l.c, w0, w1, j, S.bs, bmin, tab);
-        }
-        __device__ __forceinline__ static float cs(const Scale &S, float ad) { return ad * S.bs; }
-        __device__ __forceinline__ static float add_min(const Scale &, float, float acc) { return acc; }
     };
 } // namespace llamql

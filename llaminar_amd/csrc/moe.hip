@@ -10,53 +10,42 @@
 namespace llamql
 {
     // ---- router ------------------------------------------------------------------
-    // One workgroup (256 threads) per token.  Softmax as the reference computes it
-    // (kernels/cpu/primitives/SoftmaxPrimitivesImpl.h:584-693): max, sum of
-    // exp(l-max) in double, p = exp(l-max) * float(1/sum); then top_k rounds of
-    // arg-max (ties -> lower expert id) and optional renormalisation over the top_k.
-    constexpr int ROUTE_THREADS = 256;
-    constexpr int ROUTE_MAX_PER_THREAD = 8; // up to 2048 experts
+    // One wavefront per token; lane l owns experts l, l+64, ...  Softmax as the
+    // reference computes it (kernels/cpu/primitives/SoftmaxPrimitivesImpl.h:584-693):
+    // max, sum of exp(l-max) in double, p = exp(l-max) * float(1/sum); then top_k
+    // rounds of arg-max (ties -> lower expert id) and optional renormalisation over
+    // the top_k.  All reductions are wavefront shuffles: no LDS, no barriers.
+    constexpr int ROUTE_MAX_PER_LANE = 32; // up to 2048 experts
 
-    __global__ void __launch_bounds__(ROUTE_THREADS)
+    template <int PER>
+    __global__ void __launch_bounds__(WAVE)
         moe_route_kernel(const float *__restrict__ logits, int n_experts, int top_k, int normalize,
-                         int32_t *__restrict__ ids, float *__restrict__ weights)
+                         int32_t *__restrict__ ids, float *__restrict__ weights, int slot_stride)
     {
-        __shared__ float s_f[ROUTE_THREADS];
-        __shared__ double s_d[ROUTE_THREADS];
-        __shared__ int s_i[ROUTE_THREADS];
-        __shared__ float s_top[64];
-
         const int t = blockIdx.x;
-        const int tid = threadIdx.x;
+        const int lane = threadIdx.x;
         const float *l = logits + (size_t)t * n_experts;
 
-        float p[ROUTE_MAX_PER_THREAD];
+        float p[PER];
         float mx = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < ROUTE_MAX_PER_THREAD; ++i)
+        for (int i = 0; i < PER; ++i)
         {
-            const int e = tid + i * ROUTE_THREADS;
+            const int e = lane + i * WAVE;
             p[i] = (e < n_experts) ? l[e] : -INFINITY;
             mx = fmaxf(mx, p[i]);
         }
-        s_f[tid] = mx;
-        __syncthreads();
-        for (int off = ROUTE_THREADS / 2; off > 0; off >>= 1)
-        {
-            if (tid < off)
-                s_f[tid] = fmaxf(s_f[tid], s_f[tid + off]);
-            __syncthreads();
-        }
-        mx = s_f[0];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+            mx = fmaxf(mx, __shfl_xor(mx, off));
         if (!isfinite(mx))
             mx = 0.0f;
-        __syncthreads();
 
         double sum = 0.0;
 #pragma unroll
-        for (int i = 0; i < ROUTE_MAX_PER_THREAD; ++i)
+        for (int i = 0; i < PER; ++i)
         {
-            const int e = tid + i * ROUTE_THREADS;
+            const int e = lane + i * WAVE;
             if (e < n_experts)
             {
                 p[i] = expf(p[i] - mx);
@@ -67,78 +56,56 @@ namespace llamql
                 p[i] = -1.0f; // never selected: probabilities are >= 0
             }
         }
-        s_d[tid] = sum;
-        __syncthreads();
-        for (int off = ROUTE_THREADS / 2; off > 0; off >>= 1)
-        {
-            if (tid < off)
-                s_d[tid] += s_d[tid + off];
-            __syncthreads();
-        }
-        sum = s_d[0];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+            sum += __shfl_xor(sum, off);
         if (sum <= 0.0)
             sum = 1.0;
         const float inv = (float)(1.0 / sum);
 #pragma unroll
-        for (int i = 0; i < ROUTE_MAX_PER_THREAD; ++i)
+        for (int i = 0; i < PER; ++i)
             if (p[i] >= 0.0f)
                 p[i] = p[i] * inv;
-        __syncthreads();
 
+        float my_top = 0.0f; // lane k keeps the k-th winner's probability
+        float topk_sum = 0.0f;
         for (int k = 0; k < top_k; ++k)
         {
             float best = -1.0f;
             int best_e = 0x7FFFFFFF;
 #pragma unroll
-            for (int i = 0; i < ROUTE_MAX_PER_THREAD; ++i)
+            for (int i = 0; i < PER; ++i)
             {
-                const int e = tid + i * ROUTE_THREADS;
-                if (p[i] > best) // ascending e within a thread: first maximum wins
+                if (p[i] > best) // ascending e within a lane: first maximum wins
                 {
                     best = p[i];
-                    best_e = e;
+                    best_e = lane + i * WAVE;
                 }
             }
-            s_f[tid] = best;
-            s_i[tid] = best_e;
-            __syncthreads();
-            for (int off = ROUTE_THREADS / 2; off > 0; off >>= 1)
-            {
-                if (tid < off)
-                {
-                    const float ov = s_f[tid + off];
-                    const int oe = s_i[tid + off];
-                    if (ov > s_f[tid] || (ov == s_f[tid] && oe < s_i[tid]))
-                    {
-                        s_f[tid] = ov;
-                        s_i[tid] = oe;
-                    }
-                }
-                __syncthreads();
-            }
-            const int win = s_i[0];
-            const float winp = s_f[0];
-            __syncthreads();
-            if (tid == 0)
-            {
-                ids[(size_t)t * top_k + k] = win;
-                s_top[k] = winp;
-            }
-            // retire the winner
 #pragma unroll
-            for (int i = 0; i < ROUTE_MAX_PER_THREAD; ++i)
-                if (tid + i * ROUTE_THREADS == win)
-                    p[i] = -1.0f;
+            for (int off = 32; off > 0; off >>= 1)
+            {
+                const float ov = __shfl_xor(best, off);
+                const int oe = __shfl_xor(best_e, off);
+                if (ov > best || (ov == best && oe < best_e))
+                {
+                    best = ov;
+                    best_e = oe;
+                }
+            }
+            // every lane now holds the winner
+            if (lane == k)
+                my_top = best;
+            if (lane == 0)
+                ids[(size_t)t * slot_stride + k] = best_e;
+            topk_sum += best; // same order on every lane: k = 0, 1, ...
+#pragma unroll
+            for (int i = 0; i < PER; ++i)
+                if (lane + i * WAVE == best_e)
+                    p[i] = -1.0f; // retire the winner
         }
-        __syncthreads();
-        if (tid == 0)
-        {
-            float topk_sum = 0.0f;
-            for (int k = 0; k < top_k; ++k)
-                topk_sum += s_top[k];
-            for (int k = 0; k < top_k; ++k)
-                weights[(size_t)t * top_k + k] = normalize ? __fdiv_rn(s_top[k], topk_sum) : s_top[k];
-        }
+        if (lane < top_k)
+            weights[(size_t)t * slot_stride + lane] = normalize ? __fdiv_rn(my_top, topk_sum) : my_top;
     }
 
     // ---- routed gate/up ---------------------------------------------------------
@@ -217,6 +184,139 @@ namespace llamql
             gemv_body<F, 1, 1, false>(a, (long)blockIdx.x, lds);
             first = false;
             __syncthreads(); // LDS is restaged by the next slot
+        }
+    }
+
+    // Down projection for short expert rows (at most 8 super-blocks, i.e. one load per
+    // lane and row) and up to S slots per token.  The activations of all slots of the
+    // token (contiguous Q8_1 rows) are staged in ONE pass, and for each row batch the
+    // weight loads of ALL slots are issued before the first is decoded, so a workgroup
+    // waits for memory once per row batch instead of once per slot.  Same arithmetic and
+    // slot order as moe_down_kernel.  grid: (workgroups per matrix, n_tokens).
+    template <class F, int S>
+    __global__ void __launch_bounds__(GEMV_WAVES *WAVE) moe_down_multi_kernel(const MoEArgs m)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+        const int t = blockIdx.y;
+        const int nsb = m.inter / 256;
+        const int nkb = nsb * 8;
+        const int nkb_all = nkb * m.top_k; // the token's slots form one long activation row
+        uint32_t *aq = lds;
+        float *ad = reinterpret_cast<float *>(aq + nkb_all * 8);
+        float *asd = ad + nkb_all;
+        void *tab = asd + nkb_all;
+
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = threadIdx.x >> 6;
+        const int c = lane & 7;
+        const int grp = lane >> 3;
+        const bool odd = (c & 1) != 0;
+        const int G = 1 << m.gshift;
+        const int R = 8 >> m.gshift;
+        const int rsub = grp >> m.gshift;
+        const int sb = grp & (G - 1); // the one super-block of this lane
+
+        GemvArgs a; // weight addressing only
+        a.N = m.hidden;
+        a.SB = nsb;
+        int e[S];
+        float wt[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+        {
+            e[s] = (s < m.top_k) ? m.ids[t * m.top_k + s] : -1;
+            if (e[s] >= m.n_experts)
+                e[s] = -1;
+            wt[s] = (s < m.top_k) ? m.weights[t * m.top_k + s] : 0.0f;
+        }
+        const void *wdown[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+            wdown[s] = e[s] >= 0 ? m.experts[e[s]].d_down : nullptr;
+
+        const long wg_row0 = (long)blockIdx.x * (GEMV_WAVES * R * m.rows_per_wave);
+        auto load_rows = [&](typename F::Raw(&raw)[S], long row) {
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+            {
+                raw[s] = typename F::Raw{};
+                if (e[s] >= 0 && row < m.hidden && sb < nsb)
+                {
+                    a.w = wdown[s];
+                    raw[s] = F::load(a, row, sb, c);
+                }
+            }
+        };
+        typename F::Raw raw[S];
+        load_rows(raw, wg_row0 + (long)wave * R + rsub); // in flight during the staging
+
+        if (F::TABLE_BYTES > 0)
+            F::stage_tables(tab);
+        stage_q8<F, 1>(m.q8 + (size_t)t * nkb_all * 9, nkb_all, 0, nkb_all, aq, ad, asd);
+        __syncthreads();
+
+        for (int r = 0; r < m.rows_per_wave; ++r)
+        {
+            const long row = wg_row0 + ((long)r * GEMV_WAVES + wave) * R + rsub;
+            if (wg_row0 + ((long)r * GEMV_WAVES + wave) * R >= m.hidden) // uniform
+                break;
+            const bool row_ok = row < m.hidden && sb < nsb;
+            typename F::Raw cur[S];
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+                cur[s] = raw[s];
+            if (r + 1 < m.rows_per_wave)
+                load_rows(raw, row + (long)GEMV_WAVES * R);
+
+            float y = 0.0f;
+            bool first = (m.accumulate == 0);
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+            {
+                if (e[s] < 0) // uniform
+                    continue;
+                float acc = 0.0f;
+                if (row_ok)
+                {
+                    v4i w0, w1;
+                    int j;
+                    float bscale, bmin;
+                    F::decode(cur[s], c, w0, w1, j, bscale, bmin, tab);
+                    const v4i *ap = reinterpret_cast<const v4i *>(aq + (size_t)((s * nsb + sb) * 8 + c) * 8);
+                    const v4i a0 = ap[0];
+                    const v4i a1 = ap[1];
+                    int idot;
+                    if (F::PAIR)
+                    {
+                        const int p0 = dot16(a0, w0, 0);
+                        const int p1 = dot16(a1, w1, 0);
+                        const int got = dpp_i32<DPP_QUAD_XOR1>(odd ? p0 : p1);
+                        idot = (odd ? p1 : p0) + got;
+                    }
+                    else
+                    {
+                        idot = dot16(a1, w1, dot16(a0, w0, 0));
+                    }
+                    const int kb = (s * nsb + sb) * 8 + j;
+                    acc = fmaf((float)idot, ad[kb] * bscale, 0.0f);
+                    if (F::HAS_MIN)
+                        acc = fmaf(asd[kb], bmin, acc);
+                }
+                const float total = segment_sum(acc, m.gshift);
+                const float v = wt[s] * total;
+                if (first)
+                {
+                    y = v; // accumulate == 0: the first live slot overwrites
+                    first = false;
+                }
+                else
+                    y = y + v;
+            }
+            if (row < m.hidden && (lane & (8 * G - 1)) == 0 && !(first && m.accumulate == 0))
+            {
+                float *dst = m.out0 + (size_t)t * m.hidden + row;
+                *dst = m.accumulate ? (*dst + y) : y;
+            }
         }
     }
 
@@ -301,16 +401,22 @@ namespace llamql
 
     namespace
     {
-        void moe_shape(int N, int SB, int device_id, int &gshift, int &rpw, long &grid_x)
+        // matrices: how many [N x SB] matrices the launch walks (slots x tokens x gate|up).
+        // Every workgroup stages its activations (and the format's tables) once, so it
+        // should own as many rows as still leaves a few workgroups per compute unit.
+        void moe_shape(int N, int SB, long matrices, int device_id, int &gshift, int &rpw, long &grid_x)
         {
             gshift = 3;
             while (gshift > 0 && (1 << (gshift - 1)) >= SB)
                 --gshift;
             const int R = 8 >> gshift;
+            const long rows_total = (long)N * matrices;
+            const long per_cu = rows_total / cu_count(device_id);
             rpw = 1;
+            while (rpw < 8 && (long)GEMV_WAVES * R * rpw * 2 * 4 <= per_cu && (long)GEMV_WAVES * R * rpw * 2 <= N)
+                rpw *= 2;
             const int rows_per_wg = GEMV_WAVES * R * rpw;
             grid_x = ((long)N + rows_per_wg - 1) / rows_per_wg;
-            (void)device_id;
         }
 
         bool check_moe(const char *fn, uint8_t fmt, int n_tokens, int n_experts, int top_k, int hidden, int inter)
@@ -325,12 +431,40 @@ namespace llamql
                 return fail(fn, "too many token slots for one launch (%d x %d)", n_tokens, top_k);
             return true;
         }
+
+        // Short expert rows with few slots: one launch whose loads for all slots are in
+        // flight together; otherwise the slot-by-slot kernel.
+        template <class F>
+        bool moe_down_launch(const char *fn, const MoEArgs &m, dim3 grid, dim3 block, hipStream_t st)
+        {
+            const int nsb = m.inter / 256;
+            if (nsb <= 8 && m.top_k <= 12)
+            {
+                const int S = m.top_k <= 4 ? 4 : (m.top_k <= 8 ? 8 : 12);
+                const size_t lds = (size_t)m.top_k * nsb * GEMV_LDS_PER_SB + F::TABLE_BYTES;
+                if (lds <= 64 * 1024)
+                {
+                    if (S == 4)
+                        hipLaunchKernelGGL((moe_down_multi_kernel<F, 4>), grid, block, lds, st, m);
+                    else if (S == 8)
+                        hipLaunchKernelGGL((moe_down_multi_kernel<F, 8>), grid, block, lds, st, m);
+                    else
+                        hipLaunchKernelGGL((moe_down_multi_kernel<F, 12>), grid, block, lds, st, m);
+                    return launched(fn);
+                }
+            }
+            const size_t lds = gemv_lds_bytes<F>(1, nsb);
+            if (lds > 64 * 1024)
+                return fail(fn, "inter=%d too large for one LDS stage", m.inter);
+            hipLaunchKernelGGL((moe_down_kernel<F>), grid, block, lds, st, m);
+            return launched(fn);
+        }
     } // namespace
 } // namespace llamql
 
-extern "C" bool llam_ql_moe_route(const float *d_logits, int n_tokens, int n_experts,
-                                  int top_k, int normalize, int32_t *d_ids,
-                                  float *d_weights, int device_id, void *stream)
+extern "C" bool llam_ql_moe_route_ex(const float *d_logits, int n_tokens, int n_experts,
+                                     int top_k, int normalize, int32_t *d_ids,
+                                     float *d_weights, int slot_stride, int device_id, void *stream)
 {
     using namespace llamql;
     static const char *fn = "llam_ql_moe_route";
@@ -338,17 +472,40 @@ extern "C" bool llam_ql_moe_route(const float *d_logits, int n_tokens, int n_exp
         return fail(fn, "negative n_tokens");
     if (n_tokens == 0)
         return true;
-    if (n_experts < 1 || n_experts > ROUTE_THREADS * ROUTE_MAX_PER_THREAD)
-        return fail(fn, "n_experts=%d outside 1..%d", n_experts, ROUTE_THREADS * ROUTE_MAX_PER_THREAD);
+    if (n_experts < 1 || n_experts > WAVE * ROUTE_MAX_PER_LANE)
+        return fail(fn, "n_experts=%d outside 1..%d", n_experts, WAVE * ROUTE_MAX_PER_LANE);
     if (top_k < 1 || top_k > n_experts || top_k > 64)
         return fail(fn, "top_k=%d outside 1..min(n_experts,64)", top_k);
+    if (slot_stride < top_k)
+        return fail(fn, "slot_stride=%d smaller than top_k=%d", slot_stride, top_k);
     if (!d_logits || !d_ids || !d_weights)
         return fail(fn, "null pointer");
     if (!set_device(fn, device_id))
         return false;
-    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)n_tokens), dim3(ROUTE_THREADS), 0, as_stream(stream),
-                       d_logits, n_experts, top_k, normalize, d_ids, d_weights);
+    const dim3 grid((unsigned)n_tokens), block(WAVE);
+    hipStream_t st = as_stream(stream);
+    const int per = (n_experts + WAVE - 1) / WAVE;
+    if (per <= 4)
+        hipLaunchKernelGGL((moe_route_kernel<4>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
+                           d_weights, slot_stride);
+    else if (per <= 8)
+        hipLaunchKernelGGL((moe_route_kernel<8>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
+                           d_weights, slot_stride);
+    else if (per <= 16)
+        hipLaunchKernelGGL((moe_route_kernel<16>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
+                           d_weights, slot_stride);
+    else
+        hipLaunchKernelGGL((moe_route_kernel<32>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
+                           d_weights, slot_stride);
     return launched(fn);
+}
+
+extern "C" bool llam_ql_moe_route(const float *d_logits, int n_tokens, int n_experts,
+                                  int top_k, int normalize, int32_t *d_ids,
+                                  float *d_weights, int device_id, void *stream)
+{
+    return llam_ql_moe_route_ex(d_logits, n_tokens, n_experts, top_k, normalize, d_ids, d_weights, top_k, device_id,
+                                stream);
 }
 
 extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
@@ -378,7 +535,7 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     m.inter = inter;
     m.accumulate = 0;
     long gx;
-    moe_shape(inter, hidden / 256, device_id, m.gshift, m.rows_per_wave, gx);
+    moe_shape(inter, hidden / 256, (long)n_tokens * top_k * 2, device_id, m.gshift, m.rows_per_wave, gx);
     const dim3 grid((unsigned)gx, (unsigned)(n_tokens * top_k), 2);
     const dim3 block(GEMV_WAVES * WAVE);
     hipStream_t st = as_stream(stream);
@@ -465,38 +622,16 @@ extern "C" bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts, i
     m.inter = inter;
     m.accumulate = accumulate;
     long gx;
-    moe_shape(hidden, inter / 256, device_id, m.gshift, m.rows_per_wave, gx);
+    moe_shape(hidden, inter / 256, (long)n_tokens, device_id, m.gshift, m.rows_per_wave, gx);
     const dim3 grid((unsigned)gx, (unsigned)n_tokens);
     const dim3 block(GEMV_WAVES * WAVE);
     hipStream_t st = as_stream(stream);
     switch (fmt)
     {
-    case LLAM_FMT_Q4_K:
-    {
-        const size_t lds = gemv_lds_bytes<Q4KTraits>(1, inter / 256);
-        if (lds > 64 * 1024)
-            return fail(fn, "inter=%d too large for one LDS stage", inter);
-        hipLaunchKernelGGL((moe_down_kernel<Q4KTraits>), grid, block, lds, st, m);
-        break;
+    case LLAM_FMT_Q4_K: return moe_down_launch<Q4KTraits>(fn, m, grid, block, st);
+    case LLAM_FMT_Q6_K: return moe_down_launch<Q6KTraits>(fn, m, grid, block, st);
+    default: return moe_down_launch<IQ3STraits>(fn, m, grid, block, st);
     }
-    case LLAM_FMT_Q6_K:
-    {
-        const size_t lds = gemv_lds_bytes<Q6KTraits>(1, inter / 256);
-        if (lds > 64 * 1024)
-            return fail(fn, "inter=%d too large for one LDS stage", inter);
-        hipLaunchKernelGGL((moe_down_kernel<Q6KTraits>), grid, block, lds, st, m);
-        break;
-    }
-    default:
-    {
-        const size_t lds = gemv_lds_bytes<IQ3STraits>(1, inter / 256);
-        if (lds > 64 * 1024)
-            return fail(fn, "inter=%d too large for one LDS stage", inter);
-        hipLaunchKernelGGL((moe_down_kernel<IQ3STraits>), grid, block, lds, st, m);
-        break;
-    }
-    }
-    return launched(fn);
 }
 
 extern "C" bool llam_ql_shared_expert_add(float *d_out, const float *d_shared,

@@ -12,8 +12,6 @@ namespace llamql
     }
     int gemv_rows_per_wave_override() { return g_rows_per_wave; }
     int gemv_unroll_override() { return g_unroll; }
-    bool gemv_stream_enabled() { return g_unroll <= 0; }
-    int gemv_stream_max_waves() { return g_unroll < 0 ? -g_unroll : 16; }
 } // namespace llamql
 
 extern "C" void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll)

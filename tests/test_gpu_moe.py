@@ -157,7 +157,19 @@ def test_expert_ffn_baseline_shape(capi, dev, oracle, T):
     sg, su = capi.moe_gate_up(fmt, table, n_exp + 1, sid, qd, T, 1, hidden, inter)
     sq = capi.swiglu_quantize(sg, su)
     capi.moe_down(fmt, table, n_exp + 1, sid, sw, sq, out, T, 1, hidden, inter, accumulate=True)
+    # the same in one gate/up and one down launch: the shared expert sits in a ninth slot
+    # that the router leaves alone
+    ids9 = torch.full((T, k + 1), n_exp, dtype=torch.int32, device=dev)
+    w9 = torch.ones((T, k + 1), device=dev)
+    capi.moe_route(torch.from_numpy(logits).to(dev), k, True, ids=ids9, weights=w9)
+    gate9, up9 = capi.moe_gate_up(fmt, table, n_exp + 1, ids9, qd, T, k + 1, hidden, inter)
+    out9 = torch.full((T, hidden), float("nan"), device=dev)
+    capi.moe_down(fmt, table, n_exp + 1, ids9, w9, capi.swiglu_quantize(gate9, up9), out9, T, k + 1, hidden, inter,
+                  accumulate=False)
     sync()
+    assert torch.equal(ids9[:, :k], ids) and torch.equal(w9[:, :k], w)
+    assert (ids9[:, k] == n_exp).all() and (w9[:, k] == 1.0).all()
+    assert rel_err(out9.cpu().numpy(), out.cpu().numpy()) <= 2e-6
 
     # oracle: the same chain on the CPU (own SwiGLU, own quantisation of it)
     rids, rw, _ = oracle.route(logits, k, True)
