@@ -17,6 +17,27 @@ namespace llamql
     // the top_k.  All reductions are wavefront shuffles: no LDS, no barriers.
     constexpr int ROUTE_MAX_PER_LANE = 32; // up to 2048 experts
 
+    // Maximum of a 64-bit key over the wavefront (data-parallel primitives inside a row of
+    // 16 lanes, four lane reads across rows); every lane returns it.
+    __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
+    {
+        auto step = [&](unsigned long long o) { v = o > v ? o : v; };
+        auto join = [](int hi, int lo) { return ((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo; };
+        step(join(dpp_i32<DPP_QUAD_XOR1>((int)(v >> 32)), dpp_i32<DPP_QUAD_XOR1>((int)v)));
+        step(join(dpp_i32<DPP_QUAD_XOR2>((int)(v >> 32)), dpp_i32<DPP_QUAD_XOR2>((int)v)));
+        step(join(dpp_i32<DPP_ROW_HALF_MIRROR>((int)(v >> 32)), dpp_i32<DPP_ROW_HALF_MIRROR>((int)v)));
+        step(join(dpp_i32<DPP_ROW_MIRROR>((int)(v >> 32)), dpp_i32<DPP_ROW_MIRROR>((int)v)));
+        unsigned long long r = 0ull;
+#pragma unroll
+        for (int row = 0; row < 4; ++row)
+        {
+            const unsigned long long o = join(__builtin_amdgcn_readlane((int)(v >> 32), 16 * row),
+                                              __builtin_amdgcn_readlane((int)v, 16 * row));
+            r = o > r ? o : r;
+        }
+        return r;
+    }
+
     template <int PER>
     __global__ void __launch_bounds__(WAVE)
         moe_route_kernel(const float *__restrict__ logits, int n_experts, int top_k, int normalize,
@@ -67,38 +88,32 @@ namespace llamql
             if (p[i] >= 0.0f)
                 p[i] = p[i] * inv;
 
+        // arg-max as a maximum over 64-bit keys: probability bits above, inverted expert id
+        // below (probabilities are >= 0, so their bit patterns order like the values; the
+        // lower id wins a tie); retired and padding entries get key 0
+        auto key_of = [&](int i) -> unsigned long long {
+            return p[i] >= 0.0f ? ((unsigned long long)__float_as_uint(p[i]) << 32) | (0xFFFFFFFFu - (uint32_t)(lane + i * WAVE))
+                                : 0ull;
+        };
         float my_top = 0.0f; // lane k keeps the k-th winner's probability
         float topk_sum = 0.0f;
         for (int k = 0; k < top_k; ++k)
         {
-            float best = -1.0f;
-            int best_e = 0x7FFFFFFF;
+            unsigned long long best = 0ull;
 #pragma unroll
             for (int i = 0; i < PER; ++i)
             {
-                if (p[i] > best) // ascending e within a lane: first maximum wins
-                {
-                    best = p[i];
-                    best_e = lane + i * WAVE;
-                }
+                const unsigned long long ki = key_of(i);
+                best = ki > best ? ki : best;
             }
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1)
-            {
-                const float ov = __shfl_xor(best, off);
-                const int oe = __shfl_xor(best_e, off);
-                if (ov > best || (ov == best && oe < best_e))
-                {
-                    best = ov;
-                    best_e = oe;
-                }
-            }
-            // every lane now holds the winner
+            best = wave_max_u64(best); // every lane now holds the winner
+            const float bp = __uint_as_float((uint32_t)(best >> 32));
+            const int best_e = (int)(0xFFFFFFFFu - (uint32_t)best);
             if (lane == k)
-                my_top = best;
+                my_top = bp;
             if (lane == 0)
                 ids[(size_t)t * slot_stride + k] = best_e;
-            topk_sum += best; // same order on every lane: k = 0, 1, ...
+            topk_sum += bp; // same order on every lane: k = 0, 1, ...
 #pragma unroll
             for (int i = 0; i < PER; ++i)
                 if (lane + i * WAVE == best_e)
