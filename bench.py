@@ -162,7 +162,7 @@ def bench_gemv(args, torch, capi, synth, dev):
             y = torch.empty(M, N, device=dev)
             with torch.cuda.stream(stream):
                 us = _time_launches(torch, stream,
-                                    lambda i: capi.gemv(fmt, mats[i % nmat], q8, M, N, K, out=y), args.steps, 10)
+                                    lambda i: capi.gemv(fmt, mats[i % nmat], q8, M, N, K, out=y), args.steps, 60)
             b = synth.gemv_bytes(fmt, N, K, M)
             rows.append({"fmt": names[fmt], "N": N, "K": K, "M": M, "us": round(us, 2),
                          "GBps": round(b / (us * 1e-6) / 1e9, 1), "frac": round(b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})

@@ -94,7 +94,7 @@ namespace llamql
         typedef typename F::Quad Q;
         typename Q::Raw raw;
         typename Q::Lane lc;
-        const uint8_t *wp;
+        typename Q::Cursor wc;
         int row, l;
         bool active; // wavefront-uniform: BN rows x 4 quad lanes = the first 4*BN threads
 
@@ -107,14 +107,13 @@ namespace llamql
             long n = n0 + row;
             if (n >= g.w.N)
                 n = g.w.N - 1; // tail rows: decode a valid row, never stored
-            wp = static_cast<const uint8_t *>(g.w.w) + (size_t)n * g.w.SB * Q::SB_BYTES;
+            wc = Q::cursor(g.w, (size_t)n * g.w.SB, lc);
         }
         __device__ __forceinline__ void issue(const GemmArgs &, int sb)
         {
             // the other wavefronts load the same bytes again (cache hits) and drop them: a
             // load under a condition would need a register copy that waits for it at once
-            const uint8_t *p = wp + (size_t)sb * Q::SB_BYTES;
-            Q::load(raw, p, p + lc.byte_off);
+            Q::load_at(raw, wc, lc, sb);
         }
         __device__ __forceinline__ void store(uint8_t *Wl, float *bs, float *bm, const void *)
         {
@@ -124,15 +123,16 @@ namespace llamql
             v4i w[4];
             typename Q::Scale S;
             Q::decode(raw, lc, w, S);
-            v4i *dst = reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 64 * l);
-            dst[0] = w[0];
-            dst[1] = w[1];
-            dst[2] = w[2];
-            dst[3] = w[3];
-            bs[(2 * l) * GEMM_SN + row] = Q::scale_f32(S, 0);
-            bs[(2 * l + 1) * GEMM_SN + row] = Q::scale_f32(S, 1);
-            bm[(2 * l) * GEMM_SN + row] = Q::min_f32(S, 0);
-            bm[(2 * l + 1) * GEMM_SN + row] = Q::min_f32(S, 1);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+            {
+                const int j = Q::block_of(l, i);
+                v4i *dst = reinterpret_cast<v4i *>(Wl + row * GEMM_STRIDE + 32 * j);
+                dst[0] = w[2 * i];
+                dst[1] = w[2 * i + 1];
+                bs[j * GEMM_SN + row] = Q::scale_f32(S, i);
+                bm[j * GEMM_SN + row] = Q::min_f32(S, i);
+            }
         }
         __device__ __forceinline__ void finish() { Q::template wait<0>(raw); }
     };

@@ -318,7 +318,7 @@ namespace llamql
         // Rows of at least 16 super-blocks in a format with a quad-lane decoder: the
         // quad kernel, which stages whole activation rows (up to 160 KiB of LDS).
         if constexpr (F::USE_QUAD)
-        if (!dump && SB >= QUAD_STEP_SB && gemv_unroll_override() == 0)
+        if (!dump && SB >= QUAD_STEP_SB && gemv_unroll_override() == 0 && F::Quad::addressable(N, SB))
         {
             if (quad_lds_bytes(M, SB) > QUAD_MAX_LDS)
             {
@@ -331,7 +331,7 @@ namespace llamql
                 return gemv_launch<F>(fn, d_w, q8b, d_y + (size_t)M0 * ldy, nullptr, M - M0, N, K, ldy, row0, nrows,
                                       device_id, st);
             }
-            const QuadShape qs = gemv_quad_shape(N, SB, cu_count(device_id), quad_max_threads(M) / WAVE);
+            const QuadShape qs = gemv_quad_shape(N, SB, cu_count(device_id), F::Quad::max_threads(M) / WAVE);
             GemvArgs a;
             a.w = d_w;
             a.q8 = static_cast<const uint32_t *>(d_q8);

@@ -29,8 +29,6 @@
 namespace llamql
 {
     constexpr int QUAD_STEP_SB = 16; // super-blocks per wavefront step
-    // workgroup size bound: one activation row leaves room for 16 wavefronts of 128 registers
-    constexpr int quad_max_threads(int M) { return M == 1 ? 1024 : 512; }
     constexpr size_t QUAD_MAX_LDS = 160 * 1024; // LDS of one gfx950 compute unit
 
     // LDS bytes for M activation rows of nsb super-blocks.
@@ -40,8 +38,9 @@ namespace llamql
         return (size_t)M * (chunks * 4096 + (size_t)nsb * 64);
     }
 
-    // One thread per Q8_1 block.
-    template <int M>
+    // One thread per Q8_1 block.  Block j of a super-block goes to the quad lane that
+    // decodes it (Q::owner) as that lane's first or second block.
+    template <class Q, int M>
     __device__ __forceinline__ void quad_stage_q8(const uint32_t *__restrict__ q8, int nsb, uint8_t *aq, uint8_t *ads,
                                                   int aq_stride, int ads_stride)
     {
@@ -57,7 +56,9 @@ namespace llamql
                 for (int i = 0; i < 9; ++i)
                     v[i] = src[i];
                 const float d = h2f((uint16_t)(v[0] & 0xFFFFu));
-                const int sb = kb >> 3, j = kb & 7, l = j >> 1, odd = j & 1;
+                const int sb = kb >> 3, j = kb & 7;
+                int l, odd;
+                Q::owner(j, l, odd);
                 *reinterpret_cast<float2 *>(ads + m * ads_stride + sb * 64 + l * 16 + odd * 8) =
                     make_float2(d, (float)(int16_t)(v[0] >> 16) * d);
                 uint8_t *base = aq + m * aq_stride + (sb >> 4) * 4096 + (odd * 2) * 1024 + (sb & 15) * 64 + l * 16;
@@ -76,6 +77,17 @@ namespace llamql
     {
         static constexpr int SB_BYTES = 144;
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        // workgroup size bound: one activation row leaves room for 16 wavefronts of 128 registers
+        static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
+        // whether this matrix can be addressed by the kernel at all
+        static bool addressable(long, int) { return true; }
+        // lane l decodes blocks 2l (first) and 2l+1 (second)
+        __device__ __forceinline__ static void owner(int j, int &l, int &which)
+        {
+            l = j >> 1;
+            which = j & 1;
+        }
+        __device__ __forceinline__ static int block_of(int l, int which) { return 2 * l + which; }
 
         struct Raw
         {
@@ -106,6 +118,36 @@ namespace llamql
             return c;
         }
 
+        // Where a lane reads: its current super-block and the first one of its run (what
+        // lanes past the end of the run read instead: loads are never predicated, a load
+        // under a lane mask would be waited for at once).
+        struct Cursor
+        {
+            const uint8_t *p, *first;
+        };
+        __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, const Lane &)
+        {
+            Cursor c;
+            c.p = c.first = static_cast<const uint8_t *>(a.w) + t * SB_BYTES;
+            return c;
+        }
+        __device__ __forceinline__ static void advance(Cursor &c, int steps)
+        {
+            c.p += (size_t)steps * (QUAD_STEP_SB * SB_BYTES);
+        }
+        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, int step, bool valid)
+        {
+            const uint8_t *p = c.p + (size_t)step * (QUAD_STEP_SB * SB_BYTES);
+            if (!valid)
+                p = c.first;
+            load(r, p, p + lc.byte_off);
+        }
+        // super-block sb_off after the cursor's
+        __device__ __forceinline__ static void load_at(Raw &r, const Cursor &c, const Lane &lc, int sb_off)
+        {
+            const uint8_t *p = c.p + (size_t)sb_off * SB_BYTES;
+            load(r, p, p + lc.byte_off);
+        }
         // sb: this lane's super-block, grp: the same plus the lane's group offset.  The
         // loads are issued as assembly so that the kernel, not the compiler, decides where
         // they are waited for (wait() below); the compiler would wait right after issue.
@@ -200,6 +242,195 @@ namespace llamql
         }
     };
 
+    // ---- Q6_K ------------------------------------------------------------------------
+    // Device layout: planes ql [T][128], qh [T][64], scales [T][16], d [T] over T = N*K/256
+    // super-blocks.  Quad lane l = 2n + h works on half n of the super-block: its 32 ql
+    // bytes 64n+32h.. hold block 4n+h in the low and block 4n+2+h in the high nibbles, the
+    // 32 qh bytes 32n.. their upper two bits at bit offsets 2h and 2h+4.  Each block is
+    // requantised to int8 as the reference's packer does (SIMDHelpers.h:12023-12204):
+    //   msc = max(|sc0|,|sc1|) ; f_i = rne(sc_i*127*256 / (msc*32)) ; w = ((q-32)*f_i + 128) >> 8
+    //   b_scale = f16(d*msc*32/127)
+    // The half whose |sc| equals msc has f = +-1016 exactly, so one division per block
+    // suffices.  Weight addresses are 32-bit offsets from the plane bases.
+    struct Q6KQuad
+    {
+        typedef unsigned short v2s __attribute__((ext_vector_type(2)));
+        typedef int v2i_ __attribute__((ext_vector_type(2)));
+        static constexpr int LOADS = 6;
+        static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
+        static bool addressable(long N, int SB) { return (double)N * SB * 128.0 < 4.0e9; }
+
+        struct Raw
+        {
+            v4i qla, qlb, qha, qhb;
+            v2i_ sc;
+            int d;
+        };
+        struct Lane
+        {
+            uint32_t ql_off, qh_off, sc_off; // byte offsets of this lane inside a super-block's planes
+            uint32_t hshift;                 // 2h: bit offset of the low-nibble block's upper bits
+            uint32_t sshift;                 // 16h: bit offset of the lane's two scales in a dword
+        };
+        struct Scale
+        {
+            float bs0, bs1;
+        };
+        struct Cursor
+        {
+            const uint8_t *ql, *qh, *sc, *d; // plane bases (uniform)
+            uint32_t t, first;               // this lane's super-block index: current, start of run
+        };
+
+        __device__ __forceinline__ static Lane lane_consts(int l)
+        {
+            Lane c;
+            const uint32_t n = (uint32_t)l >> 1, h = (uint32_t)l & 1u;
+            c.ql_off = 64u * n + 32u * h;
+            c.qh_off = 32u * n;
+            c.sc_off = 8u * n;
+            c.hshift = 2u * h;
+            c.sshift = 16u * h;
+            return c;
+        }
+        // block j = 4n + sub: lane 2n + (sub & 1), its first (sub < 2) or second block
+        __device__ __forceinline__ static void owner(int j, int &l, int &which)
+        {
+            l = 2 * (j >> 2) + (j & 1);
+            which = (j >> 1) & 1;
+        }
+        __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, const Lane &)
+        {
+            const size_t T = (size_t)a.N * a.SB;
+            Cursor c;
+            c.ql = static_cast<const uint8_t *>(a.w);
+            c.qh = c.ql + T * 128;
+            c.sc = c.ql + T * 192;
+            c.d = c.ql + T * 208;
+            c.t = c.first = (uint32_t)t;
+            return c;
+        }
+        __device__ __forceinline__ static void advance(Cursor &c, int steps) { c.t += (uint32_t)(steps * QUAD_STEP_SB); }
+        __device__ __forceinline__ static int block_of(int l, int which) { return 4 * (l >> 1) + (l & 1) + 2 * which; }
+
+        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, int step, bool valid)
+        {
+            load_index(r, c, lc, valid ? c.t + (uint32_t)(step * QUAD_STEP_SB) : c.first);
+        }
+        __device__ __forceinline__ static void load_at(Raw &r, const Cursor &c, const Lane &lc, int sb_off)
+        {
+            load_index(r, c, lc, c.t + (uint32_t)sb_off);
+        }
+        // Loads issued as assembly so that the kernel decides where they are waited for.
+        __device__ __forceinline__ static void load_index(Raw &r, const Cursor &c, const Lane &lc, uint32_t t)
+        {
+            const uint32_t oql = t * 128u + lc.ql_off, oqh = t * 64u + lc.qh_off, osc = t * 16u + lc.sc_off, od = t * 2u;
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qla) : "v"(oql), "s"(c.ql));
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(r.qlb) : "v"(oql), "s"(c.ql));
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qha) : "v"(oqh), "s"(c.qh));
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(r.qhb) : "v"(oqh), "s"(c.qh));
+            asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(r.sc) : "v"(osc), "s"(c.sc));
+            asm volatile("global_load_ushort %0, %1, %2" : "=&v"(r.d) : "v"(od), "s"(c.d));
+        }
+        __device__ __forceinline__ static void keep(Raw &r)
+        {
+            asm volatile("" : "+v"(r.qla), "+v"(r.qlb), "+v"(r.qha), "+v"(r.qhb), "+v"(r.sc), "+v"(r.d));
+        }
+        template <int NEWER>
+        __device__ __forceinline__ static void wait(Raw &r)
+        {
+            asm volatile("s_waitcnt vmcnt(%6)"
+                         : "+v"(r.qla), "+v"(r.qlb), "+v"(r.qha), "+v"(r.qhb), "+v"(r.sc), "+v"(r.d)
+                         : "n"(NEWER));
+        }
+
+        // ((q-32)*f + 128) >> 8 on four 6-bit values packed in the bytes of q: in wrapping
+        // 16-bit arithmetic q*f + (128 - 32 f) is exact (|value| < 2^15 for |f| <= 1016) and
+        // ">> 8, keep the low byte" is "take the high byte".
+        __device__ __forceinline__ static int requant4(uint32_t q, v2s ff, v2s cc)
+        {
+            const uint32_t e = q & 0x00FF00FFu;
+            const uint32_t o = (q >> 8) & 0x00FF00FFu;
+            const v2s re = __builtin_bit_cast(v2s, e) * ff + cc;
+            const v2s ro = __builtin_bit_cast(v2s, o) * ff + cc;
+            return (int)__builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, ro), __builtin_bit_cast(uint32_t, re),
+                                              0x07030501u);
+        }
+
+        // The two 8.8 factors and the effective scale of one block from its two sub-scales.
+        __device__ __forceinline__ static void block_factors(int s0, int s1, float d, v2s &f0, v2s &c0, v2s &f1,
+                                                             v2s &c1, float &bscale)
+        {
+            const int a0 = s0 < 0 ? -s0 : s0, a1 = s1 < 0 ? -s1 : s1;
+            const bool big0 = a0 >= a1;
+            const int msc = big0 ? a0 : a1;
+            const int s_small = big0 ? s1 : s0, s_big = big0 ? s0 : s1;
+            const float fm = (float)msc;
+            int f_small = 0, f_big = 0;
+            bscale = 0.0f;
+            if (msc != 0)
+            {
+                f_big = s_big < 0 ? -1016 : 1016; // rne(+-msc*32512 / (msc*32))
+                f_small = (int)rintf(__fdiv_rn((float)s_small * 32512.0f, fm * 32.0f));
+                bscale = f16_round_packer(__fdiv_rn(d * fm * 32.0f, 127.0f));
+            }
+            const int fi0 = big0 ? f_big : f_small, fi1 = big0 ? f_small : f_big;
+            const unsigned short u0 = (unsigned short)fi0, u1 = (unsigned short)fi1;
+            const unsigned short k0 = (unsigned short)(128 - 32 * fi0), k1 = (unsigned short)(128 - 32 * fi1);
+            f0 = (v2s){u0, u0};
+            c0 = (v2s){k0, k0};
+            f1 = (v2s){u1, u1};
+            c1 = (v2s){k1, k1};
+        }
+
+        // w[0], w[1]: elements 0-15, 16-31 of block 4n+h; w[2], w[3]: of block 4n+2+h.
+        __device__ __forceinline__ static void decode(const Raw &r, const Lane &lc, v4i (&w)[4], Scale &S)
+        {
+            const float d = h2f((uint16_t)r.d);
+            const int sA0 = __builtin_amdgcn_sbfe(r.sc.x, lc.sshift, 8u);
+            const int sA1 = __builtin_amdgcn_sbfe(r.sc.x, lc.sshift + 8u, 8u);
+            const int sB0 = __builtin_amdgcn_sbfe(r.sc.y, lc.sshift, 8u);
+            const int sB1 = __builtin_amdgcn_sbfe(r.sc.y, lc.sshift + 8u, 8u);
+            v2s fA0, cA0, fA1, cA1, fB0, cB0, fB1, cB1;
+            block_factors(sA0, sA1, d, fA0, cA0, fA1, cA1, S.bs0);
+            block_factors(sB0, sB1, d, fB0, cB0, fB1, cB1, S.bs1);
+
+            const uint32_t k4 = 0x0F0F0F0Fu, k2 = 0x03030303u;
+            auto pair = [&](uint32_t ql, uint32_t qh, v2s fa, v2s ca, v2s fb, v2s cb, int &wa, int &wb) {
+                const uint32_t hs = qh >> lc.hshift;
+                const uint32_t qa = (ql & k4) | ((hs & k2) << 4);
+                const uint32_t qb = ((ql >> 4) & k4) | (((hs >> 4) & k2) << 4);
+                wa = requant4(qa, fa, ca); // f == 0 (msc == 0) yields 0 bytes
+                wb = requant4(qb, fb, cb);
+            };
+            // dwords 0-3 are elements 0-15 (first sub-scale), dwords 4-7 elements 16-31
+            int a0[4], b0[4], a1[4], b1[4];
+            pair((uint32_t)r.qla.x, (uint32_t)r.qha.x, fA0, cA0, fB0, cB0, a0[0], b0[0]);
+            pair((uint32_t)r.qla.y, (uint32_t)r.qha.y, fA0, cA0, fB0, cB0, a0[1], b0[1]);
+            pair((uint32_t)r.qla.z, (uint32_t)r.qha.z, fA0, cA0, fB0, cB0, a0[2], b0[2]);
+            pair((uint32_t)r.qla.w, (uint32_t)r.qha.w, fA0, cA0, fB0, cB0, a0[3], b0[3]);
+            pair((uint32_t)r.qlb.x, (uint32_t)r.qhb.x, fA1, cA1, fB1, cB1, a1[0], b1[0]);
+            pair((uint32_t)r.qlb.y, (uint32_t)r.qhb.y, fA1, cA1, fB1, cB1, a1[1], b1[1]);
+            pair((uint32_t)r.qlb.z, (uint32_t)r.qhb.z, fA1, cA1, fB1, cB1, a1[2], b1[2]);
+            pair((uint32_t)r.qlb.w, (uint32_t)r.qhb.w, fA1, cA1, fB1, cB1, a1[3], b1[3]);
+            w[0] = (v4i){a0[0], a0[1], a0[2], a0[3]};
+            w[1] = (v4i){a1[0], a1[1], a1[2], a1[3]};
+            w[2] = (v4i){b0[0], b0[1], b0[2], b0[3]};
+            w[3] = (v4i){b1[0], b1[1], b1[2], b1[3]};
+        }
+
+        __device__ __forceinline__ static float scale_f32(const Scale &S, int i) { return i ? S.bs1 : S.bs0; }
+        __device__ __forceinline__ static float min_f32(const Scale &, int) { return 0.0f; }
+
+        // the reference's mins plane is all zero for Q6_K
+        __device__ __forceinline__ static float apply(const Scale &S, int idot0, int idot1, const float4 sd, float acc)
+        {
+            acc = fmaf((float)idot0, sd.x * S.bs0, acc);
+            acc = fmaf((float)idot1, sd.z * S.bs1, acc);
+            return acc;
+        }
+    };
+
     // ---- kernel ----------------------------------------------------------------------
 
     template <class Q, int M, int U>
@@ -241,7 +472,7 @@ namespace llamql
     }
 
     template <class Q, int M, int U>
-    __global__ void __launch_bounds__(quad_max_threads(M)) gemv_quad_kernel(const GemvArgs a)
+    __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const GemvArgs a)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
         const int nsb = a.SB;
@@ -267,32 +498,29 @@ namespace llamql
         const int nsteps = (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
 
         // (an idle wavefront -- no rows left -- points at row 0 and uses nothing it loads)
-        const uint8_t *wp = static_cast<const uint8_t *>(a.w) + ((size_t)(total > 0 ? r0 : 0) * nsb + grp) * Q::SB_BYTES;
-        const uint8_t *const wp_safe = wp; // lanes past the end of the run re-read their first super-block
+        typename Q::Cursor wc = Q::cursor(a, (size_t)(total > 0 ? r0 : 0) * nsb + grp, lc);
         int ld_step = 0;
         auto load_chunk = [&](typename Q::Raw(&buf)[U]) {
 #pragma unroll
             for (int u = 0; u < U; ++u)
-            {
-                // no predicated loads: a load under a lane mask would be waited for at once
-                const uint8_t *p = wp + (size_t)u * (QUAD_STEP_SB * Q::SB_BYTES);
-                if ((ld_step + u) * QUAD_STEP_SB + grp >= total)
-                    p = wp_safe;
-                Q::load(buf[u], p, p + lc.byte_off);
-            }
-            wp += (size_t)U * (QUAD_STEP_SB * Q::SB_BYTES);
+                Q::load(buf[u], wc, lc, u, (ld_step + u) * QUAD_STEP_SB + grp < total);
+            Q::advance(wc, U);
             ld_step += U;
         };
 
         typename Q::Raw bufA[U], bufB[U];
-        load_chunk(bufA); // in flight while the activations are staged
+        load_chunk(bufA); // two chunks in flight while the activations are staged
+        load_chunk(bufB);
 
-        quad_stage_q8<M>(a.q8, nsb, aq, ads, aq_stride, ads_stride);
+        quad_stage_q8<Q, M>(a.q8, nsb, aq, ads, aq_stride, ads_stride);
         __syncthreads();
         // the staging code above must not reuse the registers of the loads in flight
 #pragma unroll
         for (int u = 0; u < U; ++u)
+        {
             Q::keep(bufA[u]);
+            Q::keep(bufB[u]);
+        }
 
         float cur[M], nxt[M];
 #pragma unroll
@@ -361,17 +589,18 @@ namespace llamql
             }
         };
 
-        // The next chunk is loaded unconditionally (past the end of the run the lanes re-read
-        // their first super-block): a load under a condition would need register copies that
-        // wait for it straight away.
+        // Each buffer is reloaded (with the chunk two ahead) as soon as it has been consumed.
+        // Loads are unconditional -- past the end of the run the lanes re-read their first
+        // super-block: a load under a condition would need register copies that wait for
+        // it straight away.
         for (int c0 = 0; c0 < nsteps; c0 += 2 * U)
         {
-            load_chunk(bufB);
             compute_chunk(bufA);
             __builtin_amdgcn_sched_barrier(0); // keep the loads below the last use of their registers
             load_chunk(bufA);
             compute_chunk(bufB);
             __builtin_amdgcn_sched_barrier(0);
+            load_chunk(bufB);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the run
     }
@@ -395,14 +624,15 @@ namespace llamql
     {
         switch (M)
         {
-        case 1: gemv_quad_launch_mu<Q, 1, 3>(grid, block, lds, st, a); break;
-        case 2: gemv_quad_launch_mu<Q, 2, 3>(grid, block, lds, st, a); break;
+        case 1: gemv_quad_launch_mu<Q, 1, Q::LOADS <= 3 ? 3 : 2>(grid, block, lds, st, a); break;
+        case 2: gemv_quad_launch_mu<Q, 2, Q::LOADS <= 3 ? 3 : 2>(grid, block, lds, st, a); break;
         case 3: gemv_quad_launch_mu<Q, 3, 2>(grid, block, lds, st, a); break;
         case 4: gemv_quad_launch_mu<Q, 4, 2>(grid, block, lds, st, a); break;
-        case 5: gemv_quad_launch_mu<Q, 5, 2>(grid, block, lds, st, a); break;
-        case 6: gemv_quad_launch_mu<Q, 6, 2>(grid, block, lds, st, a); break;
-        case 7: gemv_quad_launch_mu<Q, 7, 2>(grid, block, lds, st, a); break;
-        default: gemv_quad_launch_mu<Q, 8, 2>(grid, block, lds, st, a); break;
+        // (formats with many loads per step run out of registers at two steps per chunk)
+        case 5: gemv_quad_launch_mu<Q, 5, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
+        case 6: gemv_quad_launch_mu<Q, 6, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
+        case 7: gemv_quad_launch_mu<Q, 7, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
+        default: gemv_quad_launch_mu<Q, 8, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
         }
     }
 

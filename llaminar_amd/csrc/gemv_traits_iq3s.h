@@ -67,7 +67,7 @@ namespace llamql
         static constexpr bool PAIR = false;
         static constexpr bool HAS_MIN = false;
         static constexpr bool USE_QUAD = false;
-        static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
+        static constexpr int FAST_MAX_U = 3;          // load batches in flight in the chunked kernel
         static constexpr int TABLE_BYTES = (int)sizeof(IQ3STables);
 
         __device__ static void stage_tables(void *lds_tab)

@@ -23,6 +23,7 @@
 // factor f.
 #pragma once
 #include "gemv_core.h"
+#include "gemv_quad.h"
 
 
 namespace llamql
@@ -48,7 +49,8 @@ namespace llamql
     {
         static constexpr bool PAIR = true;
         static constexpr bool HAS_MIN = false; // the reference's mins plane is all zero for Q6_K
-        static constexpr bool USE_QUAD = false;
+        static constexpr bool USE_QUAD = true;        // quad-lane kernel for rows of >= 16 super-blocks
+        typedef Q6KQuad Quad;
         static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
         static constexpr int TABLE_BYTES = 0;
         __device__ static void stage_tables(void *) {}
