@@ -32,9 +32,9 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# runs of this script (profiles/gemv_q4k_25600x5120_batch1_pmc.txt): (36104.2 KiB x 2.000 +
-# 104.4 KiB x 1.000), the factors being what the same counters read for a plain 256 MiB kernel.
-DOMINANT_TRAFFIC_BYTES = 74048307
+# runs of this script (profiles/gemv_q4k_25600x5120_batch1_pmc.txt): (36156.2 KiB x 2.000 +
+# 109.9 KiB x 1.000), the factors being what the same counters read for a plain 256 MiB kernel.
+DOMINANT_TRAFFIC_BYTES = 74160435
 
 HIDDEN, QDIM, KVDIM, FFN = 5120, 8192, 1024, 25600
 
@@ -362,7 +362,7 @@ def main():
             "launch": "eager" if graphs is None else "hip-graph replay",
         },
         "roofline": {
-            "kernel": "gemv_stream_kernel<Q4KTraits,1,5,2> N=25600 K=5120",
+            "kernel": "gemv_quad_kernel<Q4KQuad,1,3> N=25600 K=5120",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,

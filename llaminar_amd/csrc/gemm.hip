@@ -107,7 +107,7 @@ namespace llamql
             long n = n0 + row;
             if (n >= g.w.N)
                 n = g.w.N - 1; // tail rows: decode a valid row, never stored
-            wc = Q::cursor(g.w, (size_t)n * g.w.SB, lc);
+            wc = Q::cursor(g.w, (size_t)n * g.w.SB, (size_t)n * g.w.SB, lc);
         }
         __device__ __forceinline__ void issue(const GemmArgs &, int sb)
         {

@@ -118,17 +118,18 @@ namespace llamql
             return c;
         }
 
-        // Where a lane reads: its current super-block and the first one of its run (what
-        // lanes past the end of the run read instead: loads are never predicated, a load
-        // under a lane mask would be waited for at once).
+        // Where a lane reads: its current super-block, and the one it reads instead once it
+        // is past the end of its run (its last valid one, still in the caches): loads are
+        // never predicated, a load under a lane mask would be waited for at once.
         struct Cursor
         {
             const uint8_t *p, *first;
         };
-        __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, const Lane &)
+        __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, size_t t_safe, const Lane &)
         {
             Cursor c;
-            c.p = c.first = static_cast<const uint8_t *>(a.w) + t * SB_BYTES;
+            c.p = static_cast<const uint8_t *>(a.w) + t * SB_BYTES;
+            c.first = static_cast<const uint8_t *>(a.w) + t_safe * SB_BYTES;
             return c;
         }
         __device__ __forceinline__ static void advance(Cursor &c, int steps)
@@ -279,7 +280,8 @@ namespace llamql
         struct Cursor
         {
             const uint8_t *ql, *qh, *sc, *d; // plane bases (uniform)
-            uint32_t t, first;               // this lane's super-block index: current, start of run
+            uint32_t t, first;               // this lane's super-block index: current, and the one
+                                             // read instead past the end of the run
         };
 
         __device__ __forceinline__ static Lane lane_consts(int l)
@@ -299,7 +301,7 @@ namespace llamql
             l = 2 * (j >> 2) + (j & 1);
             which = (j >> 1) & 1;
         }
-        __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, const Lane &)
+        __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, size_t t_safe, const Lane &)
         {
             const size_t T = (size_t)a.N * a.SB;
             Cursor c;
@@ -307,7 +309,8 @@ namespace llamql
             c.qh = c.ql + T * 128;
             c.sc = c.ql + T * 192;
             c.d = c.ql + T * 208;
-            c.t = c.first = (uint32_t)t;
+            c.t = (uint32_t)t;
+            c.first = (uint32_t)t_safe;
             return c;
         }
         __device__ __forceinline__ static void advance(Cursor &c, int steps) { c.t += (uint32_t)(steps * QUAD_STEP_SB); }
@@ -498,7 +501,10 @@ namespace llamql
         const int nsteps = (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
 
         // (an idle wavefront -- no rows left -- points at row 0 and uses nothing it loads)
-        typename Q::Cursor wc = Q::cursor(a, (size_t)(total > 0 ? r0 : 0) * nsb + grp, lc);
+        const size_t t0 = (size_t)(total > 0 ? r0 : 0) * nsb + grp;
+        // this lane's last valid super-block of the run (for an idle wavefront: of row 0)
+        const int last_step = total > grp ? (total - 1 - grp) / QUAD_STEP_SB : 0;
+        typename Q::Cursor wc = Q::cursor(a, t0, t0 + (size_t)last_step * QUAD_STEP_SB, lc);
         int ld_step = 0;
         auto load_chunk = [&](typename Q::Raw(&buf)[U]) {
 #pragma unroll
