@@ -23,4 +23,40 @@ namespace llamql
     {
         return gemv_launch<IQ3STraits>(fn, d_w, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
     }
+
+    namespace
+    {
+        template <class F>
+        int group_launch(const char *fn, const llam_ql_proj *projs, int num, const void *d_q8, int M, int K,
+                         int device_id, hipStream_t st)
+        {
+            QuadProj pr[QUAD_MAX_PROJ];
+            int n = 0;
+            while (n < num && n < QUAD_MAX_PROJ && projs[n].fmt == projs[0].fmt &&
+                   quad_eligible<F>(M, projs[n].N, K))
+            {
+                pr[n] = QuadProj{projs[n].d_w, projs[n].d_y, projs[n].N, projs[n].ldy};
+                ++n;
+            }
+            if (n < 2)
+                return 0;
+            return gemv_quad_multi<F>(fn, pr, n, d_q8, M, K, device_id, st) ? n : -1;
+        }
+    } // namespace
+
+    // Launches the longest run of projections at the head of `projs` (same format, all fit
+    // for the quad-lane kernel) as ONE kernel.  Returns how many it covered, 0 when the
+    // first projection has to go through its own launch, -1 on error.
+    int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const void *d_q8, int M, int K,
+                          int device_id, hipStream_t st)
+    {
+        if (num < 2)
+            return 0;
+        switch (projs[0].fmt)
+        {
+        case LLAM_FMT_Q4_K: return group_launch<Q4KTraits>(fn, projs, num, d_q8, M, K, device_id, st);
+        case LLAM_FMT_Q6_K: return group_launch<Q6KTraits>(fn, projs, num, d_q8, M, K, device_id, st);
+        default: return 0;
+        }
+    }
 } // namespace llamql

@@ -307,6 +307,72 @@ namespace llamql
         return sh;
     }
 
+    // Quad-lane kernel over up to QUAD_MAX_PROJ matrices of one format and row length that
+    // share their activations.  Every matrix keeps the rows-per-wavefront it has when it is
+    // launched alone, so results do not depend on what it is launched together with.
+    struct QuadProj
+    {
+        const void *w;
+        float *y;
+        int N, ldy;
+    };
+    template <class F>
+    bool quad_eligible(int M, int N, int K)
+    {
+        if constexpr (F::USE_QUAD)
+            return K / 256 >= QUAD_STEP_SB && gemv_unroll_override() == 0 && F::Quad::addressable(N, K / 256) &&
+                   quad_lds_bytes(M, K / 256) <= QUAD_MAX_LDS;
+        else
+            return false;
+    }
+    template <class F>
+    bool gemv_quad_multi(const char *fn, const QuadProj *pr, int n, const void *d_q8, int M, int K, int device_id,
+                         hipStream_t st)
+    {
+        if constexpr (F::USE_QUAD)
+        {
+            const int SB = K / 256;
+            const int cus = cu_count(device_id);
+            const int max_waves = F::Quad::max_threads(M) / WAVE;
+            QuadArgs a;
+            a.q8 = static_cast<const uint32_t *>(d_q8);
+            a.SB = SB;
+            a.nproj = n;
+            long waves = 0;
+            for (int i = 0; i < QUAD_MAX_PROJ; ++i)
+            {
+                const int j = i < n ? i : n - 1; // unused entries repeat the last matrix
+                a.w[i] = pr[j].w;
+                a.y[i] = pr[j].y;
+                a.N[i] = pr[j].N;
+                a.ldy[i] = pr[j].ldy;
+                a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves).rows_per_wave;
+                if (i < n)
+                    waves += ((long)pr[j].N + a.R[i] - 1) / a.R[i];
+                a.wave_end[i] = (int)waves;
+            }
+            if (waves > 0x7FFFFFFFL / WAVE)
+                return fail(fn, "too many rows for one launch");
+            // wavefronts per workgroup: an even share of what one compute unit gets
+            const long wpc = (waves + cus - 1) / cus;
+            const long wgs_per_cu = (wpc + max_waves - 1) / max_waves;
+            long nw = (wpc + wgs_per_cu - 1) / wgs_per_cu;
+            if (nw > waves)
+                nw = waves;
+            if (nw < 1)
+                nw = 1;
+            const long grid = (waves + nw - 1) / nw;
+            gemv_quad_launch<typename F::Quad>(M, dim3((unsigned)grid), dim3((unsigned)nw * WAVE),
+                                               quad_lds_bytes(M, SB), st, a);
+            return launched(fn);
+        }
+        else
+        {
+            (void)pr; (void)n; (void)d_q8; (void)M; (void)K; (void)device_id; (void)st;
+            return fail(fn, "format has no quad-lane kernel");
+        }
+    }
+
     // Shared host launcher.  Arguments are validated by the callers; the device
     // is current.  M is 1..8.
     template <class F>
@@ -331,26 +397,8 @@ namespace llamql
                 return gemv_launch<F>(fn, d_w, q8b, d_y + (size_t)M0 * ldy, nullptr, M - M0, N, K, ldy, row0, nrows,
                                       device_id, st);
             }
-            const QuadShape qs = gemv_quad_shape(N, SB, cu_count(device_id), F::Quad::max_threads(M) / WAVE);
-            GemvArgs a;
-            a.w = d_w;
-            a.q8 = static_cast<const uint32_t *>(d_q8);
-            a.y = d_y;
-            a.sums = nullptr;
-            a.ldy = ldy;
-            a.N = N;
-            a.SB = SB;
-            a.sb0 = 0;
-            a.nsb = SB;
-            a.rows_per_wave = qs.rows_per_wave;
-            a.gshift = 3;
-            a.accumulate = 0;
-            a.out_scale = 1.0f;
-            a.row0 = 0;
-            a.nrows = 0;
-            gemv_quad_launch<typename F::Quad>(M, dim3((unsigned)qs.grid), dim3((unsigned)qs.waves * WAVE),
-                                               quad_lds_bytes(M, SB), st, a);
-            return launched(fn);
+            QuadProj one{d_w, d_y, N, ldy};
+            return gemv_quad_multi<F>(fn, &one, 1, d_q8, M, K, device_id, st);
         }
         // batch sizes without a dedicated kernel are run as 4 + (M-4)
         if (M > 4 && M < 8)

@@ -30,6 +30,24 @@ namespace llamql
 {
     constexpr int QUAD_STEP_SB = 16; // super-blocks per wavefront step
     constexpr size_t QUAD_MAX_LDS = 160 * 1024; // LDS of one gfx950 compute unit
+    constexpr int QUAD_MAX_PROJ = 4;            // weight matrices one launch can walk
+
+    // One launch: up to QUAD_MAX_PROJ weight matrices of one format and row length against
+    // the same activations (projections that share an input: Q and K, gate and up).  The
+    // wavefronts of the launch are dealt to the matrices in order; wave_end[p] is the
+    // number of wavefronts up to and including matrix p.
+    struct QuadArgs
+    {
+        const uint32_t *q8; // Q8_1 activations as dwords (9 per block), M rows
+        int SB;             // super-blocks per weight row
+        int nproj;
+        const void *w[QUAD_MAX_PROJ];
+        float *y[QUAD_MAX_PROJ];
+        int N[QUAD_MAX_PROJ];
+        int ldy[QUAD_MAX_PROJ];
+        int R[QUAD_MAX_PROJ]; // rows per wavefront
+        int wave_end[QUAD_MAX_PROJ];
+    };
 
     // LDS bytes for M activation rows of nsb super-blocks.
     inline size_t quad_lds_bytes(int M, int nsb)
@@ -475,10 +493,10 @@ namespace llamql
     }
 
     template <class Q, int M, int U>
-    __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const GemvArgs a)
+    __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const QuadArgs qa)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
-        const int nsb = a.SB;
+        const int nsb = qa.SB;
         const int aq_stride = ((nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB) * 4096;
         const int ads_stride = nsb * 64;
         uint8_t *aq = quad_lds;
@@ -491,16 +509,32 @@ namespace llamql
         const int grp = lane >> 2;
         const typename Q::Lane lc = Q::lane_consts(l);
 
+        // which matrix this wavefront works on, and which of its wavefronts it is
+        const int wid_all = (int)blockIdx.x * NW + wave;
+        int p = 0, w_first = 0;
+#pragma unroll
+        for (int i = 0; i + 1 < QUAD_MAX_PROJ; ++i)
+            if (i + 1 < qa.nproj && wid_all >= qa.wave_end[i])
+            {
+                p = i + 1;
+                w_first = qa.wave_end[i];
+            }
+        GemvArgs a; // the matrix, for the format's addressing
+        a.w = qa.w[p];
+        a.N = qa.N[p];
+        a.SB = nsb;
+        float *const y = qa.y[p];
+        const int ldy = qa.ldy[p];
+        const int R = qa.R[p];
+
         // rows [r0, r1) of this wavefront: one run of `total` super-blocks
-        const long wid = (long)blockIdx.x * NW + wave;
-        const long r0 = wid * a.rows_per_wave;
-        long r1 = r0 + a.rows_per_wave;
+        const long r0 = (long)(wid_all - w_first) * R;
+        long r1 = r0 + R;
         if (r1 > a.N)
             r1 = a.N;
-        const int total = r1 > r0 ? (int)(r1 - r0) * nsb : 0;
+        const int total = (r1 > r0 && wid_all < qa.wave_end[p]) ? (int)(r1 - r0) * nsb : 0;
         const int nsteps = (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
 
-        // (an idle wavefront -- no rows left -- points at row 0 and uses nothing it loads)
         const size_t t0 = (size_t)(total > 0 ? r0 : 0) * nsb + grp;
         // this lane's last valid super-block of the run (for an idle wavefront: of row 0)
         const int last_step = total > grp ? (total - 1 - grp) / QUAD_STEP_SB : 0;
@@ -518,7 +552,7 @@ namespace llamql
         load_chunk(bufA); // two chunks in flight while the activations are staged
         load_chunk(bufB);
 
-        quad_stage_q8<Q, M>(a.q8, nsb, aq, ads, aq_stride, ads_stride);
+        quad_stage_q8<Q, M>(qa.q8, nsb, aq, ads, aq_stride, ads_stride);
         __syncthreads();
         // the staging code above must not reuse the registers of the loads in flight
 #pragma unroll
@@ -567,10 +601,7 @@ namespace llamql
                 {
                     const float tot = wave_sum(cur[m]);
                     if (lane == 0)
-                    {
-                        float *dst = a.y + (size_t)m * a.ldy + row;
-                        *dst = a.accumulate ? (*dst + a.out_scale * tot) : a.out_scale * tot;
-                    }
+                        y[(size_t)m * ldy + row] = tot;
                     cur[m] = nxt[m];
                     nxt[m] = 0.0f;
                 }
@@ -612,7 +643,7 @@ namespace llamql
     }
 
     template <class Q, int M, int U>
-    inline void gemv_quad_launch_mu(dim3 grid, dim3 block, size_t lds, hipStream_t st, const GemvArgs &a)
+    inline void gemv_quad_launch_mu(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         static bool attr_set = false;
         if (!attr_set)
@@ -626,7 +657,7 @@ namespace llamql
     }
 
     template <class Q>
-    inline void gemv_quad_launch(int M, dim3 grid, dim3 block, size_t lds, hipStream_t st, const GemvArgs &a)
+    inline void gemv_quad_launch(int M, dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         switch (M)
         {
@@ -665,7 +696,7 @@ namespace llamql
             int nsb, cus, max_waves, rpw;
             QuadShape sh;
         };
-        thread_local Memo memo[8] = {};
+        thread_local Memo memo[16] = {};
         thread_local int memo_next = 0;
         for (const Memo &e : memo)
             if (e.N == N && e.nsb == nsb && e.cus == cus && e.max_waves == max_waves && e.rpw == rpw_override)
@@ -709,7 +740,7 @@ namespace llamql
         sh.waves = (int)(nw < 1 ? 1 : nw);
         sh.grid = (waves + sh.waves - 1) / sh.waves;
         memo[memo_next] = Memo{N, nsb, cus, max_waves, rpw_override, sh};
-        memo_next = (memo_next + 1) % 8;
+        memo_next = (memo_next + 1) % 16;
         return sh;
     }
 } // namespace llamql

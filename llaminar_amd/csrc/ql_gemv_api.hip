@@ -11,6 +11,8 @@ namespace llamql
                          int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
     bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
                           int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
+    int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const void *d_q8, int M, int K,
+                          int device_id, hipStream_t st);
 
     namespace
     {
@@ -83,11 +85,24 @@ extern "C" bool llam_ql_gemv_fused(const llam_ql_proj *projs, int num, const voi
         return true;
     if (!set_device(fn, device_id))
         return false;
-    // One quantised input, projections enqueued back to back on the same stream.
-    for (int i = 0; i < num; ++i)
+    // One quantised input.  Neighbouring projections of one format share a launch where
+    // the kernel allows it (each keeps the row partition of its own launch, so the results
+    // are those of separate calls); the rest are enqueued back to back on the same stream.
+    for (int i = 0; i < num;)
+    {
+        const int took = gemv_group_launch(fn, projs + i, num - i, d_q8, M, K, device_id, as_stream(stream));
+        if (took < 0)
+            return false;
+        if (took > 0)
+        {
+            i += took;
+            continue;
+        }
         if (!dispatch(fn, projs[i].fmt, projs[i].d_w, d_q8, projs[i].d_y, nullptr, M, projs[i].N, K,
                       projs[i].ldy, 0, 0, device_id, as_stream(stream)))
             return false;
+        ++i;
+    }
     return true;
 }
 
