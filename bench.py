@@ -189,6 +189,8 @@ def parse():
     ap.add_argument("--batch", type=int, default=1, help="activation rows / tokens per step")
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    ap.add_argument("--separate-quantise", action="store_true",
+                    help="layer workload: quantiser kernels of their own instead of the fp32-input GEMV calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 256 MiB read + 256 MiB write elementwise kernel a few times, so a rocprofv3 --pmc run of this "
@@ -248,7 +250,8 @@ def main():
     down = torch.empty(M, HIDDEN, device=dev)
     lib = capi.load()
 
-    def step(w):
+    def step_separate(w):
+        # quantiser kernels of their own, Q8_1 blocks through memory
         capi.quantize_q8_1(x, out=q8_x)
         capi.gemv_fused([(FMT_Q4_K, w["q"], qkv[:, :QDIM]), (FMT_Q4_K, w["k"], qkv[:, QDIM:QDIM + KVDIM]),
                          (FMT_Q6_K, w["v"], qkv[:, QDIM + KVDIM:])], q8_x, M, HIDDEN)
@@ -261,6 +264,19 @@ def main():
         assert ok, capi.last_error()
         capi.gemv(FMT_Q6_K, w["down"], q8_act, M, HIDDEN, FFN, out=down)
 
+    def step_fp32(w):
+        # the operator's fp32-input calls: every GEMV quantises its input itself (same bits)
+        capi.gemv_fused_f32([(FMT_Q4_K, w["q"], qkv[:, :QDIM]), (FMT_Q4_K, w["k"], qkv[:, QDIM:QDIM + KVDIM]),
+                             (FMT_Q6_K, w["v"], qkv[:, QDIM + KVDIM:])], x, M, HIDDEN, q8_scratch=q8_x)
+        capi.gemv_f32(FMT_Q4_K, w["o"], attn, M, HIDDEN, QDIM, out=o_out, q8_scratch=q8_attn)
+        capi.gemv_fused_f32([(FMT_Q4_K, w["gate"], gate), (FMT_Q4_K, w["up"], up)], x2, M, HIDDEN,
+                            q8_scratch=q8_x2)
+        capi.gemv_swiglu_f32(FMT_Q6_K, w["down"], gate, up, M, HIDDEN, FFN, out=down, q8_scratch=q8_act)
+        # (with the scratch buffers given, the library quantises inside the GEMV only where that is
+        # cheaper than a quantiser launch: single short rows)
+
+    step = step_separate if args.separate_quantise else step_fp32
+
     bytes_per_step = sum(synth.gemv_bytes(fmt, N, K, M) for _, N, K, fmt in projs)
     bytes_per_step += M * (2 * HIDDEN + QDIM) * 4 + M * 2 * FFN * 4  # fp32 read by the quantisers
 
@@ -270,22 +286,32 @@ def main():
         for i in range(max(args.warmup, 1)):
             step(layers[i % args.layers])
         stream.synchronize()
+        group = None
         if not args.no_graph:
+            # one graph per weight set, and one graph of `layers` consecutive steps (a decode
+            # pass captures all of its layers in one graph: one graph launch per pass)
             graphs = []
             for w in layers:
                 gr = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(gr, stream=stream):
                     step(w)
                 graphs.append(gr)
-            for gr in graphs:
+            group = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(group, stream=stream):
+                for w in layers:
+                    step(w)
+            for gr in graphs + [group]:
                 gr.replay()
             stream.synchronize()
 
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         if graphs is not None:
-            for i in range(args.steps):
-                graphs[i % args.layers].replay()
+            whole, rest = divmod(args.steps, args.layers)
+            for i in range(whole):
+                group.replay()
+            for i in range(rest):
+                graphs[i].replay()
         else:
             for i in range(args.steps):
                 step(layers[i % args.layers])

@@ -108,6 +108,30 @@ typedef struct
 bool llam_ql_gemv_fused(const llam_ql_proj *projs, int num, const void *d_q8,
                         int M, int K, int device_id, void *stream);
 
+/* The same from fp32 activations (rows of ldx floats, 16-byte aligned, ldx % 4 == 0):
+ * the Q8_1 quantisation of llam_ql_quantize_q8_1 happens inside the GEMV kernels, so
+ * the results are the bits of "quantise, then llam_ql_gemv / llam_ql_gemv_fused" without
+ * the quantiser's launch and its round trip through memory.  These are the operator's
+ * fp32-input decode calls: multiply_tensor with small m and multiply_fused_tensor
+ * (CPUNativeVNNIGemmKernel.h:154-214, 572-700: quantize_activations_to_q8_1 followed by
+ * gemv_native_vnni_preq / gemv_native_vnni_fused_preq).
+ * d_q8_scratch: M * K/32 * 36 bytes, or NULL.  It is written only when a projection's
+ * kernel cannot quantise for itself (IQ3_S, K < 4096, M*K too large for LDS); with NULL
+ * such a call fails. */
+bool llam_ql_gemv_f32(uint8_t fmt, const void *d_w, const float *d_x, int ldx, float *d_y,
+                      int M, int N, int K, int ldy, void *d_q8_scratch, int device_id,
+                      void *stream);
+bool llam_ql_gemv_fused_f32(const llam_ql_proj *projs, int num, const float *d_x, int ldx,
+                            int M, int K, void *d_q8_scratch, int device_id, void *stream);
+
+/* d_y = (silu(gate) * up) @ W^T for fp32 gate/up rows of ld_gu floats: the bits of
+ * llam_ql_swiglu_quantize followed by llam_ql_gemv, in one launch.  Replaces
+ * multiply_tensor_with_fused_swiglu (CPUNativeVNNIGemmKernel.h:325-431: compute_swiglu,
+ * then the quantising GEMV).  d_q8_scratch as above. */
+bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const float *d_gate,
+                             const float *d_up, int ld_gu, float *d_y, int M, int N, int K,
+                             int ldy, void *d_q8_scratch, int device_id, void *stream);
+
 /* Parity hook: the exact per-block int32 sums the GEMV forms, for rows
  * [row0, row0+nrows): d_sums[(m*nrows + r)*(K/32) + kb].  Runs the same integer
  * pipeline as llam_ql_gemv.  (The reference exposes the same quantity only

@@ -45,6 +45,12 @@ SIGNATURES = {
     "llam_ql_prepare_weights": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_gemv": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_gemv_fused": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                                  c_int, c_void_p]),
+    "llam_ql_gemv_fused_f32": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int,
+                                        c_void_p]),
+    "llam_ql_gemv_swiglu_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                         c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_gemv_block_sums": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                          c_int, c_void_p]),
     "llam_ql_gemm": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
@@ -170,6 +176,42 @@ def gemv_fused(projs, q8, M: int, K: int, stream=None):
         arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], out.stride(0) if out.dim() == 2 else out.shape[-1], fmt)
     dev = _dev(q8)
     _check(load().llam_ql_gemv_fused(arr, len(projs), _ptr(q8), M, K, dev, _stream(stream)), "gemv_fused")
+
+
+def _ld(t) -> int:
+    return t.stride(0) if t.dim() == 2 else t.shape[-1]
+
+
+def gemv_f32(fmt: int, w, x, M: int, N: int, K: int, out=None, q8_scratch=None, stream=None):
+    """out[M,N] from fp32 activations x[M,K] (quantised inside the kernel)."""
+    import torch
+
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32, device=w.device)
+    _check(load().llam_ql_gemv_f32(fmt, _ptr(w), _ptr(x), _ld(x), _ptr(out), M, N, K, _ld(out), _ptr(q8_scratch),
+                                   _dev(w), _stream(stream)), "gemv_f32")
+    return out
+
+
+def gemv_fused_f32(projs, x, M: int, K: int, q8_scratch=None, stream=None):
+    """projs: list of (fmt, w, out[M,N]) sharing the fp32 input x[M,K]."""
+    arr = (Proj * len(projs))()
+    for i, (fmt, w, out) in enumerate(projs):
+        arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], _ld(out), fmt)
+    _check(load().llam_ql_gemv_fused_f32(arr, len(projs), _ptr(x), _ld(x), M, K, _ptr(q8_scratch), _dev(x),
+                                         _stream(stream)), "gemv_fused_f32")
+
+
+def gemv_swiglu_f32(fmt: int, w, gate, up, M: int, N: int, K: int, out=None, q8_scratch=None, stream=None):
+    """out[M,N] = (silu(gate) * up)[M,K] @ W^T."""
+    import torch
+
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32, device=w.device)
+    assert _ld(gate) == _ld(up)
+    _check(load().llam_ql_gemv_swiglu_f32(fmt, _ptr(w), _ptr(gate), _ptr(up), _ld(gate), _ptr(out), M, N, K, _ld(out),
+                                          _ptr(q8_scratch), _dev(w), _stream(stream)), "gemv_swiglu_f32")
+    return out
 
 
 def gemv_block_sums(fmt: int, w, q8, M: int, N: int, K: int, row0: int, nrows: int, stream=None):

@@ -27,7 +27,7 @@ namespace llamql
     namespace
     {
         template <class F>
-        int group_launch(const char *fn, const llam_ql_proj *projs, int num, const void *d_q8, int M, int K,
+        int group_launch(const char *fn, const llam_ql_proj *projs, int num, const ActSource &src, int M, int K,
                          int device_id, hipStream_t st)
         {
             QuadProj pr[QUAD_MAX_PROJ];
@@ -38,24 +38,25 @@ namespace llamql
                 pr[n] = QuadProj{projs[n].d_w, projs[n].d_y, projs[n].N, projs[n].ldy};
                 ++n;
             }
-            if (n < 2)
+            // a single matrix on Q8_1 input goes through the general launcher
+            if (n < (src.kind == ACT_SRC_Q8 ? 2 : 1))
                 return 0;
-            return gemv_quad_multi<F>(fn, pr, n, d_q8, M, K, device_id, st) ? n : -1;
+            return gemv_quad_multi<F>(fn, pr, n, src, M, K, device_id, st) ? n : -1;
         }
     } // namespace
 
     // Launches the longest run of projections at the head of `projs` (same format, all fit
     // for the quad-lane kernel) as ONE kernel.  Returns how many it covered, 0 when the
-    // first projection has to go through its own launch, -1 on error.
-    int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const void *d_q8, int M, int K,
+    // first projection has to go through its own launch on Q8_1 input, -1 on error.
+    int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const ActSource &src, int M, int K,
                           int device_id, hipStream_t st)
     {
-        if (num < 2)
+        if (num < 1)
             return 0;
         switch (projs[0].fmt)
         {
-        case LLAM_FMT_Q4_K: return group_launch<Q4KTraits>(fn, projs, num, d_q8, M, K, device_id, st);
-        case LLAM_FMT_Q6_K: return group_launch<Q6KTraits>(fn, projs, num, d_q8, M, K, device_id, st);
+        case LLAM_FMT_Q4_K: return group_launch<Q4KTraits>(fn, projs, num, src, M, K, device_id, st);
+        case LLAM_FMT_Q6_K: return group_launch<Q6KTraits>(fn, projs, num, src, M, K, device_id, st);
         default: return 0;
         }
     }

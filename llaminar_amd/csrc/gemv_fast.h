@@ -325,9 +325,12 @@ namespace llamql
         else
             return false;
     }
+    static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU,
+                  "activation source kinds");
+
     template <class F>
-    bool gemv_quad_multi(const char *fn, const QuadProj *pr, int n, const void *d_q8, int M, int K, int device_id,
-                         hipStream_t st)
+    bool gemv_quad_multi(const char *fn, const QuadProj *pr, int n, const ActSource &src, int M, int K,
+                         int device_id, hipStream_t st)
     {
         if constexpr (F::USE_QUAD)
         {
@@ -335,7 +338,10 @@ namespace llamql
             const int cus = cu_count(device_id);
             const int max_waves = F::Quad::max_threads(M) / WAVE;
             QuadArgs a;
-            a.q8 = static_cast<const uint32_t *>(d_q8);
+            a.q8 = static_cast<const uint32_t *>(src.q8);
+            a.x = src.x;
+            a.x2 = src.x2;
+            a.ldx = src.ldx;
             a.SB = SB;
             a.nproj = n;
             long waves = 0;
@@ -362,13 +368,13 @@ namespace llamql
             if (nw < 1)
                 nw = 1;
             const long grid = (waves + nw - 1) / nw;
-            gemv_quad_launch<typename F::Quad>(M, dim3((unsigned)grid), dim3((unsigned)nw * WAVE),
+            gemv_quad_launch<typename F::Quad>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE),
                                                quad_lds_bytes(M, SB), st, a);
             return launched(fn);
         }
         else
         {
-            (void)pr; (void)n; (void)d_q8; (void)M; (void)K; (void)device_id; (void)st;
+            (void)pr; (void)n; (void)src; (void)M; (void)K; (void)device_id; (void)st;
             return fail(fn, "format has no quad-lane kernel");
         }
     }
@@ -398,7 +404,7 @@ namespace llamql
                                       device_id, st);
             }
             QuadProj one{d_w, d_y, N, ldy};
-            return gemv_quad_multi<F>(fn, &one, 1, d_q8, M, K, device_id, st);
+            return gemv_quad_multi<F>(fn, &one, 1, act_source_q8(d_q8), M, K, device_id, st);
         }
         // batch sizes without a dedicated kernel are run as 4 + (M-4)
         if (M > 4 && M < 8)

@@ -32,13 +32,24 @@ namespace llamql
     constexpr size_t QUAD_MAX_LDS = 160 * 1024; // LDS of one gfx950 compute unit
     constexpr int QUAD_MAX_PROJ = 4;            // weight matrices one launch can walk
 
+    // Where the activations come from.  The fp32 kinds quantise to Q8_1 inside the kernel,
+    // every workgroup for itself while its first weight loads are in flight, with the
+    // arithmetic of the stand-alone quantisers: the launch of a quantiser kernel and the
+    // round trip of its output through memory are saved, the results are the same bits.
+    constexpr int QUAD_SRC_Q8 = 0;     // Q8_1 blocks
+    constexpr int QUAD_SRC_F32 = 1;    // fp32 rows
+    constexpr int QUAD_SRC_SWIGLU = 2; // silu(gate) * up of two fp32 inputs
+
     // One launch: up to QUAD_MAX_PROJ weight matrices of one format and row length against
     // the same activations (projections that share an input: Q and K, gate and up).  The
     // wavefronts of the launch are dealt to the matrices in order; wave_end[p] is the
     // number of wavefronts up to and including matrix p.
     struct QuadArgs
     {
-        const uint32_t *q8; // Q8_1 activations as dwords (9 per block), M rows
+        const uint32_t *q8; // Q8_1 activations as dwords (9 per block), M rows (QUAD_SRC_Q8)
+        const float *x;     // fp32 activations, M rows of ldx floats (QUAD_SRC_F32); the gate
+        const float *x2;    // rows for QUAD_SRC_SWIGLU, whose up rows are x2
+        int ldx;
         int SB;             // super-blocks per weight row
         int nproj;
         const void *w[QUAD_MAX_PROJ];
@@ -82,6 +93,58 @@ namespace llamql
                 uint8_t *base = aq + m * aq_stride + (sb >> 4) * 4096 + (odd * 2) * 1024 + (sb & 15) * 64 + l * 16;
                 *reinterpret_cast<uint4 *>(base) = make_uint4(v[1], v[2], v[3], v[4]);
                 *reinterpret_cast<uint4 *>(base + 1024) = make_uint4(v[5], v[6], v[7], v[8]);
+            }
+        }
+    }
+
+    // The same from fp32 rows (SRC = QUAD_SRC_F32) or from silu(x) * x2 (QUAD_SRC_SWIGLU):
+    // eight neighbouring threads quantise one 32-element block.
+    template <class Q, int M, int SRC>
+    __device__ __forceinline__ void quad_stage_f32(const float *__restrict__ x, const float *__restrict__ x2, int ldx,
+                                                   int nsb, uint8_t *aq, uint8_t *ads, int aq_stride, int ads_stride)
+    {
+        const int nvec = nsb * 64; // float4 per row; workgroup sizes are multiples of 64
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+        {
+            const float4 *row = reinterpret_cast<const float4 *>(x + (size_t)m * ldx);
+            const float4 *row2 = reinterpret_cast<const float4 *>(x2 + (size_t)m * ldx);
+            // four loads in flight per thread: the latency of a round trip is paid per batch
+            constexpr int UN = SRC == QUAD_SRC_SWIGLU ? 2 : 4;
+            for (int i0 = threadIdx.x; i0 < nvec; i0 += UN * (int)blockDim.x)
+            {
+                float4 v[UN], v2[UN];
+#pragma unroll
+                for (int u = 0; u < UN; ++u)
+                {
+                    const int i = min(i0 + u * (int)blockDim.x, nvec - 1);
+                    v[u] = row[i];
+                    if constexpr (SRC == QUAD_SRC_SWIGLU)
+                        v2[u] = row2[i];
+                }
+#pragma unroll
+                for (int u = 0; u < UN; ++u)
+                {
+                    const int i = i0 + u * (int)blockDim.x;
+                    if (i >= nvec) // whole 8-thread groups leave together
+                        break;
+                    if constexpr (SRC == QUAD_SRC_SWIGLU)
+                        v[u] = swiglu4(v[u], v2[u]);
+                    const Q8Lane q = q8_1_quantize_lane(v[u]);
+                    const int kb = i >> 3, sub = i & 7;
+                    const int sb = kb >> 3, j = kb & 7;
+                    int l, odd;
+                    Q::owner(j, l, odd);
+                    if (sub == 0)
+                    {
+                        const float d = h2f((uint16_t)(q.head & 0xFFFFu));
+                        *reinterpret_cast<float2 *>(ads + m * ads_stride + sb * 64 + l * 16 + odd * 8) =
+                            make_float2(d, (float)(int16_t)(q.head >> 16) * d);
+                    }
+                    uint8_t *base = aq + m * aq_stride + (sb >> 4) * 4096 + (odd * 2 + (sub >> 2)) * 1024 +
+                                    (sb & 15) * 64 + l * 16 + (sub & 3) * 4;
+                    *reinterpret_cast<uint32_t *>(base) = q.packed;
+                }
             }
         }
     }
@@ -492,7 +555,7 @@ namespace llamql
         }
     }
 
-    template <class Q, int M, int U>
+    template <class Q, int M, int U, int SRC>
     __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const QuadArgs qa)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
@@ -552,7 +615,10 @@ namespace llamql
         load_chunk(bufA); // two chunks in flight while the activations are staged
         load_chunk(bufB);
 
-        quad_stage_q8<Q, M>(qa.q8, nsb, aq, ads, aq_stride, ads_stride);
+        if constexpr (SRC == QUAD_SRC_Q8)
+            quad_stage_q8<Q, M>(qa.q8, nsb, aq, ads, aq_stride, ads_stride);
+        else
+            quad_stage_f32<Q, M, SRC>(qa.x, qa.x2, qa.ldx, nsb, aq, ads, aq_stride, ads_stride);
         __syncthreads();
         // the staging code above must not reuse the registers of the loads in flight
 #pragma unroll
@@ -642,34 +708,46 @@ namespace llamql
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the run
     }
 
-    template <class Q, int M, int U>
-    inline void gemv_quad_launch_mu(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
+    template <class Q, int M, int U, int SRC>
+    inline void gemv_quad_launch_mus(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         static bool attr_set = false;
         if (!attr_set)
         {
             // dynamic LDS beyond 64 KiB has to be allowed per kernel once
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U>),
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             attr_set = true;
         }
-        hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U>), grid, block, lds, st, a);
+        hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U, SRC>), grid, block, lds, st, a);
+    }
+
+    template <class Q, int M, int U>
+    inline void gemv_quad_launch_mu(int src, dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
+    {
+        switch (src)
+        {
+        case QUAD_SRC_F32: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_F32>(grid, block, lds, st, a); break;
+        case QUAD_SRC_SWIGLU: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_SWIGLU>(grid, block, lds, st, a); break;
+        default: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_Q8>(grid, block, lds, st, a); break;
+        }
     }
 
     template <class Q>
-    inline void gemv_quad_launch(int M, dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
+    inline void gemv_quad_launch(int M, int src, dim3 grid, dim3 block, size_t lds, hipStream_t st,
+                                 const QuadArgs &a)
     {
         switch (M)
         {
-        case 1: gemv_quad_launch_mu<Q, 1, Q::LOADS <= 3 ? 3 : 2>(grid, block, lds, st, a); break;
-        case 2: gemv_quad_launch_mu<Q, 2, Q::LOADS <= 3 ? 3 : 2>(grid, block, lds, st, a); break;
-        case 3: gemv_quad_launch_mu<Q, 3, 2>(grid, block, lds, st, a); break;
-        case 4: gemv_quad_launch_mu<Q, 4, 2>(grid, block, lds, st, a); break;
+        case 1: gemv_quad_launch_mu<Q, 1, Q::LOADS <= 3 ? 3 : 2>(src, grid, block, lds, st, a); break;
+        case 2: gemv_quad_launch_mu<Q, 2, Q::LOADS <= 3 ? 3 : 2>(src, grid, block, lds, st, a); break;
+        case 3: gemv_quad_launch_mu<Q, 3, 2>(src, grid, block, lds, st, a); break;
+        case 4: gemv_quad_launch_mu<Q, 4, 2>(src, grid, block, lds, st, a); break;
         // (formats with many loads per step run out of registers at two steps per chunk)
-        case 5: gemv_quad_launch_mu<Q, 5, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
-        case 6: gemv_quad_launch_mu<Q, 6, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
-        case 7: gemv_quad_launch_mu<Q, 7, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
-        default: gemv_quad_launch_mu<Q, 8, Q::LOADS <= 3 ? 2 : 1>(grid, block, lds, st, a); break;
+        case 5: gemv_quad_launch_mu<Q, 5, Q::LOADS <= 3 ? 2 : 1>(src, grid, block, lds, st, a); break;
+        case 6: gemv_quad_launch_mu<Q, 6, Q::LOADS <= 3 ? 2 : 1>(src, grid, block, lds, st, a); break;
+        case 7: gemv_quad_launch_mu<Q, 7, Q::LOADS <= 3 ? 2 : 1>(src, grid, block, lds, st, a); break;
+        default: gemv_quad_launch_mu<Q, 8, Q::LOADS <= 3 ? 2 : 1>(src, grid, block, lds, st, a); break;
         }
     }
 

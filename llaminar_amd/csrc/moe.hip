@@ -348,39 +348,15 @@ namespace llamql
             return;
         const float4 g = gate[lane_global];
         const float4 u = up[lane_global];
-        float4 v;
-        v.x = __fdiv_rn(g.x, 1.0f + expf(-g.x)) * u.x;
-        v.y = __fdiv_rn(g.y, 1.0f + expf(-g.y)) * u.y;
-        v.z = __fdiv_rn(g.z, 1.0f + expf(-g.z)) * u.z;
-        v.w = __fdiv_rn(g.w, 1.0f + expf(-g.w)) * u.w;
+        const float4 v = swiglu4(g, u);
         if (act_out)
             act_out[lane_global] = v;
 
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR1>(amax));
-        amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR2>(amax));
-        amax = fmaxf(amax, dpp_f32<DPP_ROW_HALF_MIRROR>(amax));
-        uint32_t packed = 0, head = 0;
-        if (amax >= 1e-10f)
-        {
-            const float d = __fdiv_rn(amax, 127.0f);
-            const float id = __fdiv_rn(1.0f, d);
-            int q0 = max(-128, min(127, (int)rintf(v.x * id)));
-            int q1 = max(-128, min(127, (int)rintf(v.y * id)));
-            int q2 = max(-128, min(127, (int)rintf(v.z * id)));
-            int q3 = max(-128, min(127, (int)rintf(v.w * id)));
-            int sum = q0 + q1 + q2 + q3;
-            sum += dpp_i32<DPP_QUAD_XOR1>(sum);
-            sum += dpp_i32<DPP_QUAD_XOR2>(sum);
-            sum += dpp_i32<DPP_ROW_HALF_MIRROR>(sum);
-            packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
-                     ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
-            head = (uint32_t)__half_as_ushort(__float2half_rn(d)) | ((uint32_t)(sum & 0xFFFF) << 16);
-        }
+        const Q8Lane q = q8_1_quantize_lane(v);
         uint32_t *dst = out + blk * 9;
-        dst[1 + sub] = packed;
+        dst[1 + sub] = q.packed;
         if (sub == 0)
-            dst[0] = head;
+            dst[0] = q.head;
     }
 
     // ---- shared expert gate -----------------------------------------------------------

@@ -88,6 +88,56 @@ namespace llamql
         return (r0 + r1) + (r2 + r3);
     }
 
+    // ---- Q8_1 quantiser, one lane's share ---------------------------------------------
+    // Eight neighbouring lanes (lane & 7 = 0..7) own one 32-element block, four values
+    // each; all eight must be active.  Arithmetic of the reference's quantiser
+    // (src/v2/tensors/SIMDHelpers.h:4716-4785): amax = max|x|, below 1e-10 an all-zero
+    // block; d = amax/127 and id = 1/d as IEEE divides; q = saturate(rne(x*id));
+    // d stored as nearest-even fp16 next to the int16 sum of the 32 quants.
+    struct Q8Lane
+    {
+        uint32_t packed; // this lane's four quants
+        uint32_t head;   // fp16 d | int16 sum << 16 (the same in all eight lanes)
+    };
+    __device__ __forceinline__ Q8Lane q8_1_quantize_lane(const float4 v)
+    {
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR1>(amax));
+        amax = fmaxf(amax, dpp_f32<DPP_QUAD_XOR2>(amax));
+        amax = fmaxf(amax, dpp_f32<DPP_ROW_HALF_MIRROR>(amax));
+        Q8Lane r;
+        r.packed = 0;
+        r.head = 0;
+        if (amax >= 1e-10f)
+        {
+            const float d = __fdiv_rn(amax, 127.0f);
+            const float id = __fdiv_rn(1.0f, d);
+            const int q0 = max(-128, min(127, (int)rintf(v.x * id)));
+            const int q1 = max(-128, min(127, (int)rintf(v.y * id)));
+            const int q2 = max(-128, min(127, (int)rintf(v.z * id)));
+            const int q3 = max(-128, min(127, (int)rintf(v.w * id)));
+            int sum = q0 + q1 + q2 + q3;
+            sum += dpp_i32<DPP_QUAD_XOR1>(sum);
+            sum += dpp_i32<DPP_QUAD_XOR2>(sum);
+            sum += dpp_i32<DPP_ROW_HALF_MIRROR>(sum);
+            r.packed = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
+                       ((uint32_t)(q3 & 0xFF) << 24);
+            r.head = (uint32_t)__half_as_ushort(__float2half_rn(d)) | ((uint32_t)(sum & 0xFFFF) << 16);
+        }
+        return r;
+    }
+
+    // silu(gate) * up, element by element (gate / (1 + exp(-gate)) with an IEEE divide).
+    __device__ __forceinline__ float4 swiglu4(const float4 g, const float4 u)
+    {
+        float4 v;
+        v.x = __fdiv_rn(g.x, 1.0f + expf(-g.x)) * u.x;
+        v.y = __fdiv_rn(g.y, 1.0f + expf(-g.y)) * u.y;
+        v.z = __fdiv_rn(g.z, 1.0f + expf(-g.z)) * u.z;
+        v.w = __fdiv_rn(g.w, 1.0f + expf(-g.w)) * u.w;
+        return v;
+    }
+
     // ---- integer dot ------------------------------------------------------------
 
     // acc + sum of four signed-byte products (v_dot4_i32_i8).

@@ -11,11 +11,28 @@ namespace llamql
                          int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
     bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
                           int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
-    int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const void *d_q8, int M, int K,
+    int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const ActSource &src, int M, int K,
                           int device_id, hipStream_t st);
 
     namespace
     {
+        bool check_matrix(const char *fn, uint8_t fmt, const void *d_w, int M, int N, int K)
+        {
+            if (fmt != LLAM_FMT_Q4_K && fmt != LLAM_FMT_Q6_K && fmt != LLAM_FMT_IQ3_S)
+                return fail(fn, "unsupported weight format id %d", (int)fmt);
+            if (M < 1 || M > LLAM_QL_MAX_GEMV_M)
+                return fail(fn, "M=%d outside 1..%d", M, LLAM_QL_MAX_GEMV_M);
+            if (N < 1 || K < 1)
+                return fail(fn, "empty matrix (N=%d K=%d)", N, K);
+            if ((K % 256) != 0)
+                return fail(fn, "K must be a multiple of 256 (N=%d K=%d)", N, K);
+            if (!d_w)
+                return fail(fn, "null pointer");
+            if (!aligned16(d_w))
+                return fail(fn, "d_w must be 16-byte aligned");
+            return true;
+        }
+
         bool check_common(const char *fn, uint8_t fmt, const void *d_w, const void *d_q8, int M, int N, int K)
         {
             if (fmt != LLAM_FMT_Q4_K && fmt != LLAM_FMT_Q6_K && fmt != LLAM_FMT_IQ3_S)
@@ -65,45 +82,166 @@ extern "C" bool llam_ql_gemv(uint8_t fmt, const void *d_w, const void *d_q8, flo
     return dispatch(fn, fmt, d_w, d_q8, d_y, nullptr, M, N, K, ldy, 0, 0, device_id, as_stream(stream));
 }
 
+namespace llamql
+{
+    namespace
+    {
+        // Projections of one input, in order.  Neighbouring projections of one format share a
+        // launch where the kernel allows it (each keeps the row partition of its own launch,
+        // so the results are those of separate calls); the rest are enqueued back to back on
+        // the same stream.  fp32 input is quantised inside the kernels; for the first
+        // projection whose kernel cannot do that it is quantised into d_q8_scratch, which
+        // then serves the remaining projections.
+        bool run_projections(const char *fn, const llam_ql_proj *projs, int num, ActSource src, int M, int K,
+                             void *d_q8_scratch, int device_id, void *stream)
+        {
+            // Every workgroup of a self-quantising launch quantises all M*K activations again.
+            // Measured against a quantiser launch of its own (about 4.5 us) that pays off for a
+            // single short row; beyond it the scratch buffer, when there is one, is used.
+            const bool self_quantise =
+                src.kind == ACT_SRC_Q8 || !d_q8_scratch || (src.kind == ACT_SRC_F32 && (long)M * K <= 6144);
+            for (int i = 0; i < num;)
+            {
+                const int took = (self_quantise || src.kind == ACT_SRC_Q8)
+                                     ? gemv_group_launch(fn, projs + i, num - i, src, M, K, device_id,
+                                                         as_stream(stream))
+                                     : 0;
+                if (took < 0)
+                    return false;
+                if (took > 0)
+                {
+                    i += took;
+                    continue;
+                }
+                if (src.kind != ACT_SRC_Q8)
+                {
+                    if (!d_q8_scratch)
+                        return fail(fn, "projection %d (format %d, N=%d, K=%d) needs d_q8_scratch", i,
+                                    (int)projs[i].fmt, projs[i].N, K);
+                    const size_t row_bytes = (size_t)(K / 32) * sizeof(llam_block_q8_1);
+                    const int rows_per_call = src.ldx == K ? M : 1;
+                    for (int m = 0; m < M; m += rows_per_call)
+                    {
+                        void *dst = static_cast<uint8_t *>(d_q8_scratch) + (size_t)m * row_bytes;
+                        const float *x = src.x + (size_t)m * src.ldx;
+                        const bool ok = src.kind == ACT_SRC_F32
+                                            ? llam_ql_quantize_q8_1(x, dst, rows_per_call, K, device_id, stream)
+                                            : llam_ql_swiglu_quantize(x, src.x2 + (size_t)m * src.ldx, nullptr, dst,
+                                                                      rows_per_call, K, device_id, stream);
+                        if (!ok)
+                            return false;
+                    }
+                    src = act_source_q8(d_q8_scratch);
+                    continue; // groups may form again on the Q8_1 input
+                }
+                if (!dispatch(fn, projs[i].fmt, projs[i].d_w, src.q8, projs[i].d_y, nullptr, M, projs[i].N, K,
+                              projs[i].ldy, 0, 0, device_id, as_stream(stream)))
+                    return false;
+                ++i;
+            }
+            return true;
+        }
+
+        bool check_projections(const char *fn, const llam_ql_proj *projs, int num, int M, int K)
+        {
+            if (num < 0 || num > LLAM_QL_MAX_FUSED)
+                return fail(fn, "num=%d outside 0..%d", num, LLAM_QL_MAX_FUSED);
+            if (num > 0 && !projs)
+                return fail(fn, "null projection table");
+            for (int i = 0; i < num; ++i)
+            {
+                if (!check_matrix(fn, projs[i].fmt, projs[i].d_w, M, projs[i].N, K))
+                    return false;
+                if (!projs[i].d_y || projs[i].ldy < projs[i].N)
+                    return fail(fn, "projection %d: bad output (ldy=%d N=%d)", i, projs[i].ldy, projs[i].N);
+            }
+            return true;
+        }
+
+        bool check_f32(const char *fn, const float *x, int ldx, int K, const void *d_q8_scratch)
+        {
+            if (!x)
+                return fail(fn, "null activations");
+            if (ldx < K || (ldx % 4) != 0 || !aligned16(x))
+                return fail(fn, "fp32 activations need 16-byte aligned rows (ldx=%d K=%d)", ldx, K);
+            if (d_q8_scratch && !aligned4(d_q8_scratch))
+                return fail(fn, "d_q8_scratch must be 4-byte aligned");
+            return true;
+        }
+    } // namespace
+} // namespace llamql
+
 extern "C" bool llam_ql_gemv_fused(const llam_ql_proj *projs, int num, const void *d_q8,
                                    int M, int K, int device_id, void *stream)
 {
     using namespace llamql;
     static const char *fn = "llam_ql_gemv_fused";
-    if (num < 0 || num > LLAM_QL_MAX_FUSED)
-        return fail(fn, "num=%d outside 0..%d", num, LLAM_QL_MAX_FUSED);
-    if (num > 0 && !projs)
-        return fail(fn, "null projection table");
-    for (int i = 0; i < num; ++i)
-    {
-        if (!check_common(fn, projs[i].fmt, projs[i].d_w, d_q8, M, projs[i].N, K))
-            return false;
-        if (!projs[i].d_y || projs[i].ldy < projs[i].N)
-            return fail(fn, "projection %d: bad output (ldy=%d N=%d)", i, projs[i].ldy, projs[i].N);
-    }
+    if (!check_projections(fn, projs, num, M, K))
+        return false;
     if (num == 0)
         return true;
+    if (!d_q8 || !aligned4(d_q8))
+        return fail(fn, "d_q8 must be a 4-byte aligned device pointer");
     if (!set_device(fn, device_id))
         return false;
-    // One quantised input.  Neighbouring projections of one format share a launch where
-    // the kernel allows it (each keeps the row partition of its own launch, so the results
-    // are those of separate calls); the rest are enqueued back to back on the same stream.
-    for (int i = 0; i < num;)
-    {
-        const int took = gemv_group_launch(fn, projs + i, num - i, d_q8, M, K, device_id, as_stream(stream));
-        if (took < 0)
-            return false;
-        if (took > 0)
-        {
-            i += took;
-            continue;
-        }
-        if (!dispatch(fn, projs[i].fmt, projs[i].d_w, d_q8, projs[i].d_y, nullptr, M, projs[i].N, K,
-                      projs[i].ldy, 0, 0, device_id, as_stream(stream)))
-            return false;
-        ++i;
-    }
-    return true;
+    return run_projections(fn, projs, num, act_source_q8(d_q8), M, K, nullptr, device_id, stream);
+}
+
+extern "C" bool llam_ql_gemv_f32(uint8_t fmt, const void *d_w, const float *d_x, int ldx, float *d_y,
+                                 int M, int N, int K, int ldy, void *d_q8_scratch, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_f32";
+    llam_ql_proj p;
+    p.d_w = d_w;
+    p.d_y = d_y;
+    p.N = N;
+    p.ldy = ldy;
+    p.fmt = fmt;
+    if (!check_projections(fn, &p, 1, M, K) || !check_f32(fn, d_x, ldx, K, d_q8_scratch))
+        return false;
+    if (!set_device(fn, device_id))
+        return false;
+    return run_projections(fn, &p, 1, ActSource{ACT_SRC_F32, nullptr, d_x, nullptr, ldx}, M, K, d_q8_scratch,
+                           device_id, stream);
+}
+
+extern "C" bool llam_ql_gemv_fused_f32(const llam_ql_proj *projs, int num, const float *d_x, int ldx,
+                                       int M, int K, void *d_q8_scratch, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_fused_f32";
+    if (!check_projections(fn, projs, num, M, K))
+        return false;
+    if (num == 0)
+        return true;
+    if (!check_f32(fn, d_x, ldx, K, d_q8_scratch))
+        return false;
+    if (!set_device(fn, device_id))
+        return false;
+    return run_projections(fn, projs, num, ActSource{ACT_SRC_F32, nullptr, d_x, nullptr, ldx}, M, K, d_q8_scratch,
+                           device_id, stream);
+}
+
+extern "C" bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const float *d_gate, const float *d_up,
+                                        int ld_gu, float *d_y, int M, int N, int K, int ldy, void *d_q8_scratch,
+                                        int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_swiglu_f32";
+    llam_ql_proj p;
+    p.d_w = d_w;
+    p.d_y = d_y;
+    p.N = N;
+    p.ldy = ldy;
+    p.fmt = fmt;
+    if (!check_projections(fn, &p, 1, M, K) || !check_f32(fn, d_gate, ld_gu, K, d_q8_scratch) ||
+        !check_f32(fn, d_up, ld_gu, K, nullptr))
+        return false;
+    if (!set_device(fn, device_id))
+        return false;
+    return run_projections(fn, &p, 1, ActSource{ACT_SRC_SWIGLU, nullptr, d_gate, d_up, ld_gu}, M, K, d_q8_scratch,
+                           device_id, stream);
 }
 
 extern "C" bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,

@@ -44,4 +44,17 @@ namespace llamql
     int cu_count(int device_id);
 
     inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+
+    // The activations of a decode GEMV: Q8_1 blocks, or fp32 rows that the kernel quantises
+    // itself (plain, or silu(x) * x2 first).
+    constexpr int ACT_SRC_Q8 = 0, ACT_SRC_F32 = 1, ACT_SRC_SWIGLU = 2;
+    struct ActSource
+    {
+        int kind;        // ACT_SRC_*
+        const void *q8;  // ACT_SRC_Q8: [M][K/32] blocks
+        const float *x;  // ACT_SRC_F32: rows of ldx floats; the gate rows for ACT_SRC_SWIGLU
+        const float *x2; // ACT_SRC_SWIGLU: the up rows
+        int ldx;
+    };
+    inline ActSource act_source_q8(const void *d_q8) { return ActSource{ACT_SRC_Q8, d_q8, nullptr, nullptr, 0}; }
 } // namespace llamql

@@ -172,6 +172,68 @@ def test_fused_groups_equal_separate_calls(capi, dev, M):
     assert torch.isnan(out[:, total:]).all()
 
 
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_fp32_input_equals_quantise_then_gemv(capi, dev, M):
+    """llam_ql_gemv_f32 / _fused_f32 / _swiglu_f32 quantise inside the kernel: bits of the
+    two-step path, for kernels that quantise themselves (Q4_K, Q6_K, K >= 4096), for the ones
+    that need the scratch buffer (IQ3_S, short K), with padded input rows, and with tiny
+    and zero blocks in the input."""
+    import torch
+
+    for K in (5120, 1024):
+        ldx = K + 64
+        xbuf = torch.from_numpy(synth.activations_numpy(8, ldx, 31 + K)).to(dev)
+        xbuf[:, 32:64] = 0.0          # an all-zero block
+        xbuf[:, 64:96] *= 1e-12       # below the quantiser's zero threshold
+        xbuf[:, 96:128] *= 1e4
+        x = xbuf[:M, :K]
+        gbuf = torch.from_numpy(synth.activations_numpy(8, ldx, 77 + K)).to(dev) * 3.0
+        g = gbuf[:M, :K]
+        qd = capi.quantize_q8_1(x.contiguous())
+        qa = capi.swiglu_quantize(g.contiguous(), x.contiguous())
+        scratch = torch.empty(M * (K // 32) * 36, dtype=torch.uint8, device=dev)
+        specs = [(FMT_Q4_K, 300), (FMT_Q4_K, 65), (FMT_Q6_K, 130), (FMT_IQ3_S, 70), (FMT_Q4_K, 40)]
+        total = sum(n for _, n in specs)
+        out = torch.full((M, total), float("nan"), device=dev)
+        projs, col = [], 0
+        for i, (fmt, N) in enumerate(specs):
+            wd = capi.prepare_weights(fmt, synth.weights_torch(fmt, N, K, 300 + i, dev), N, K)
+            projs.append((fmt, wd, out[:, col:col + N]))
+            ref = capi.gemv(fmt, wd, qd, M, N, K)
+            ref_s = capi.gemv(fmt, wd, qa, M, N, K)
+            # with a scratch buffer the library picks the cheaper way; without one the kernel
+            # has to quantise for itself, which IQ3_S and short rows cannot
+            for sc in (scratch, None) if (fmt != FMT_IQ3_S and K >= 4096) else (scratch,):
+                assert torch.equal(capi.gemv_f32(fmt, wd, x, M, N, K, q8_scratch=sc), ref), (K, fmt, "f32")
+                assert torch.equal(capi.gemv_swiglu_f32(fmt, wd, g, x, M, N, K, q8_scratch=sc), ref_s), (K, fmt)
+            col += N
+        if K >= 4096:
+            capi.gemv_fused_f32(projs[:3], x, M, K)  # no scratch: one launch per format group
+            col = 0
+            for (fmt, N), (_, wd, _) in zip(specs[:3], projs[:3]):
+                assert torch.equal(out[:, col:col + N], capi.gemv(fmt, wd, qd, M, N, K)), (K, fmt, "fused/self")
+                col += N
+            out.fill_(float("nan"))
+        capi.gemv_fused_f32(projs, x, M, K, q8_scratch=scratch)
+        col = 0
+        for (fmt, N), (_, wd, _) in zip(specs, projs):
+            assert torch.equal(out[:, col:col + N], capi.gemv(fmt, wd, qd, M, N, K)), (K, fmt, "fused")
+            col += N
+    sync()
+
+
+def test_fp32_input_without_scratch_fails_cleanly(capi, dev):
+    import torch
+
+    K, N = 1024, 64   # too short for the self-quantising kernel
+    wd = capi.prepare_weights(FMT_Q4_K, synth.weights_torch(FMT_Q4_K, N, K, 1, dev), N, K)
+    x = torch.zeros(1, K, device=dev)
+    with pytest.raises(capi.QLError, match="d_q8_scratch"):
+        capi.gemv_f32(FMT_Q4_K, wd, x, 1, N, K)
+    with pytest.raises(capi.QLError, match="aligned"):
+        capi.gemv_f32(FMT_Q4_K, wd, torch.zeros(1, K + 1, device=dev)[:, 1:], 1, N, K)
+
+
 def test_q4k_prepare_is_identity(capi, dev):
     import torch
 
