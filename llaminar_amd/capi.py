@@ -64,6 +64,18 @@ SIGNATURES = {
     "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                   c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_shared_expert_add": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    # decode_api.h
+    "llam_dec_embed_q4k": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_dec_rmsnorm_q8_1": (c_bool, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
+                                       c_void_p]),
+    "llam_dec_rope_inv_freq": (None, [c_int, c_float, c_void_p]),
+    "llam_dec_rope_kv_append": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                         c_int, c_int, c_int, c_void_p]),
+    "llam_dec_attention_scratch_floats": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "llam_dec_attention": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                    c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_dec_argmax_scratch_bytes": (c_size_t, [c_int, c_int]),
+    "llam_dec_argmax": (c_bool, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
 
 _lib = None
@@ -301,3 +313,85 @@ def shared_expert_add(out, shared, hidden=None, gate_inp=None, stream=None):
     _check(load().llam_ql_shared_expert_add(_ptr(out), _ptr(shared), _ptr(hidden), _ptr(gate_inp), T, D, _dev(out),
                                             _stream(stream)), "shared_expert_add")
     return out
+
+
+# ---- decode-step operators (decode_api.h) -----------------------------------------------------
+def embed_q4k(table, vocab: int, ids, H: int, out=None, stream=None):
+    import torch
+
+    B = ids.numel()
+    if out is None:
+        out = torch.empty(B, H, dtype=torch.float32, device=ids.device)
+    _check(load().llam_dec_embed_q4k(_ptr(table), vocab, _ptr(ids), _ptr(out), B, H, _ld(out), _dev(ids),
+                                     _stream(stream)), "embed_q4k")
+    return out
+
+
+def rmsnorm_q8_1(x, gamma, eps: float, delta=None, want_y: bool = True, want_q8: bool = True, y=None, q8=None,
+                 stream=None):
+    """x [M,H] contiguous; with delta, x += delta in place first.  Returns (y, q8)."""
+    import torch
+
+    M, H = x.shape
+    assert x.is_contiguous()
+    if want_y and y is None:
+        y = torch.empty_like(x)
+    if want_q8 and q8 is None:
+        q8 = torch.empty(M * (H // 32) * 36, dtype=torch.uint8, device=x.device)
+    _check(load().llam_dec_rmsnorm_q8_1(_ptr(x), _ptr(delta), _ptr(gamma), eps, _ptr(y), _ptr(q8), M, H, _dev(x),
+                                        _stream(stream)), "rmsnorm_q8_1")
+    return y, q8
+
+
+def rope_inv_freq(head_dim: int, theta: float, device=None):
+    import numpy as np
+    import torch
+
+    f = np.zeros(head_dim // 2, np.float32)
+    load().llam_dec_rope_inv_freq(head_dim, theta, f.ctypes.data)
+    t = torch.from_numpy(f)
+    return t.to(device) if device is not None else t
+
+
+def rope_kv_append(qkv, inv_freq, pos, kcache, vcache, n_heads: int, n_kv: int, head_dim: int, stream=None):
+    """qkv [B, >= (n_heads+2 n_kv)*head_dim] fp32, rotated in place; caches [B, n_kv, cap, head_dim] fp16."""
+    B = qkv.shape[0]
+    cap = kcache.shape[2]
+    _check(load().llam_dec_rope_kv_append(_ptr(qkv), _ld(qkv), _ptr(inv_freq), _ptr(pos), _ptr(kcache), _ptr(vcache),
+                                          B, n_heads, n_kv, head_dim, cap, _dev(qkv), _stream(stream)),
+           "rope_kv_append")
+
+
+def attention_scratch(B: int, n_heads: int, head_dim: int, cap: int, device):
+    import torch
+
+    n = load().llam_dec_attention_scratch_floats(B, n_heads, head_dim, cap)
+    return torch.empty(n, dtype=torch.float32, device=device)
+
+
+def attention(q, kcache, vcache, pos, n_heads: int, n_kv: int, head_dim: int, out=None, scratch=None, stream=None):
+    import torch
+
+    B = q.shape[0]
+    cap = kcache.shape[2]
+    if out is None:
+        out = torch.empty(B, n_heads * head_dim, dtype=torch.float32, device=q.device)
+    if scratch is None:
+        scratch = attention_scratch(B, n_heads, head_dim, cap, q.device)
+    _check(load().llam_dec_attention(_ptr(q), _ld(q), _ptr(kcache), _ptr(vcache), _ptr(pos), _ptr(out), _ld(out),
+                                     _ptr(scratch), B, n_heads, n_kv, head_dim, cap, _dev(q), _stream(stream)),
+           "attention")
+    return out
+
+
+def argmax(logits, n: int, ids=None, pos=None, scratch=None, stream=None):
+    import torch
+
+    B = logits.shape[0]
+    if ids is None:
+        ids = torch.empty(B, dtype=torch.int32, device=logits.device)
+    if scratch is None:
+        scratch = torch.empty(load().llam_dec_argmax_scratch_bytes(B, n), dtype=torch.uint8, device=logits.device)
+    _check(load().llam_dec_argmax(_ptr(logits), _ld(logits), n, B, _ptr(ids), _ptr(pos), _ptr(scratch), _dev(logits),
+                                  _stream(stream)), "argmax")
+    return ids

@@ -1,0 +1,638 @@
+// Operators between the quantized-linear launches of a decode step, for gfx950:
+// embedding rows, RMSNorm (+ residual add, + Q8_1), rotary embedding with the fp16
+// KV-cache append, single-token GQA attention, greedy sampling.
+//
+// All of them move a few KB to a few MB per launch and are bound by launch latency or,
+// for attention, by streaming the KV cache once; none is GEMM-shaped.
+#include "ql_device.h"
+#include "ql_host.h"
+
+#include <cfloat>
+#include <climits>
+#include <cmath>
+
+#include "llaminar_amd/decode_api.h"
+#include "llaminar_amd/ql_api.h"
+
+namespace llamql
+{
+    // ---- embedding ---------------------------------------------------------------------
+    // One workgroup of 256 threads per (token, super-block); thread e owns element e.
+    // Element e of a super-block: group g = e/64 of 32 bytes, low nibbles for e%64 < 32
+    // (sub-block 2g), high nibbles otherwise (sub-block 2g+1).
+    __global__ void __launch_bounds__(256)
+        embed_q4k_kernel(const llam_block_q4_K *__restrict__ table, int vocab, const int32_t *__restrict__ ids,
+                         float *__restrict__ x, int nsb, int ldx)
+    {
+        const int b = blockIdx.y, sb = blockIdx.x, e = threadIdx.x;
+        const int id = ids[b];
+        float y = 0.0f;
+        if (id >= 0 && id < vocab)
+        {
+            const llam_block_q4_K *blk = table + (size_t)id * nsb + sb;
+            const int g = e >> 6, l = e & 31, hi = (e >> 5) & 1;
+            const uint32_t *sc32 = reinterpret_cast<const uint32_t *>(blk->scales);
+            uint32_t sc, mn;
+            q4k_scale_min(2 * g + hi, sc32[0], sc32[1], sc32[2], sc, mn);
+            const float d = h2f(blk->d), dmin = h2f(blk->dmin);
+            const uint32_t byte = blk->qs[g * 32 + l];
+            const float q = (float)(hi ? (byte >> 4) : (byte & 0xFu));
+            const float d1 = d * (float)sc;
+            const float m1 = dmin * (float)mn;
+            y = d1 * q - m1;
+        }
+        x[(size_t)b * ldx + sb * 256 + e] = y;
+    }
+
+    // ---- RMSNorm -------------------------------------------------------------------------
+    // One workgroup per row.  Pass 1 adds the delta (when given), stores the new residual
+    // and accumulates the sum of squares in double; pass 2 re-reads the row (the same
+    // thread reads what it wrote), scales it and, eight threads per 32-element block,
+    // quantises it.
+    constexpr int NORM_THREADS = 512;
+
+    __global__ void __launch_bounds__(NORM_THREADS)
+        rmsnorm_q8_1_kernel(float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ gamma,
+                            float eps, float *__restrict__ y, uint32_t *__restrict__ q8, int H)
+    {
+        __shared__ double s_part[NORM_THREADS / WAVE];
+        const int m = blockIdx.x;
+        const int nvec = H >> 2;
+        float4 *row = reinterpret_cast<float4 *>(x + (size_t)m * H);
+        const float4 *drow = delta ? reinterpret_cast<const float4 *>(delta + (size_t)m * H) : nullptr;
+        const float4 *g4 = reinterpret_cast<const float4 *>(gamma);
+
+        double acc = 0.0;
+        for (int i = threadIdx.x; i < nvec; i += NORM_THREADS)
+        {
+            float4 v = row[i];
+            if (drow)
+            {
+                const float4 d = drow[i];
+                v.x += d.x;
+                v.y += d.y;
+                v.z += d.z;
+                v.w += d.w;
+                row[i] = v;
+            }
+            acc += (double)v.x * (double)v.x;
+            acc += (double)v.y * (double)v.y;
+            acc += (double)v.z * (double)v.z;
+            acc += (double)v.w * (double)v.w;
+        }
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1)
+            acc += __shfl_xor(acc, off, WAVE);
+        if ((threadIdx.x & (WAVE - 1)) == 0)
+            s_part[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        double sum_sq = 0.0;
+#pragma unroll
+        for (int w = 0; w < NORM_THREADS / WAVE; ++w)
+            sum_sq += s_part[w];
+
+        const float rms = __fsqrt_rn(__fadd_rn((float)(sum_sq / (double)H), eps));
+        const float inv = __fdiv_rn(1.0f, rms);
+
+        float4 *yrow = y ? reinterpret_cast<float4 *>(y + (size_t)m * H) : nullptr;
+        uint32_t *qrow = q8 ? q8 + (size_t)m * (H >> 5) * 9 : nullptr;
+        for (int i = threadIdx.x; i < nvec; i += NORM_THREADS) // whole 8-thread groups stay together
+        {
+            const float4 v = row[i];
+            const float4 g = g4[i];
+            float4 o;
+            o.x = __fmul_rn(__fmul_rn(v.x, inv), g.x);
+            o.y = __fmul_rn(__fmul_rn(v.y, inv), g.y);
+            o.z = __fmul_rn(__fmul_rn(v.z, inv), g.z);
+            o.w = __fmul_rn(__fmul_rn(v.w, inv), g.w);
+            if (yrow)
+                yrow[i] = o;
+            if (qrow)
+            {
+                const Q8Lane q = q8_1_quantize_lane(o);
+                uint32_t *dst = qrow + (size_t)(i >> 3) * 9;
+                dst[1 + (i & 7)] = q.packed;
+                if ((i & 7) == 0)
+                    dst[0] = q.head;
+            }
+        }
+    }
+
+    // ---- rotary embedding + KV append -----------------------------------------------------
+    // One workgroup of head_dim/2 threads per (sequence, head); heads n_heads.. are the K
+    // heads, whose workgroups also copy the matching V head.
+    __global__ void rope_kv_append_kernel(float *__restrict__ qkv, int ld_qkv, const float *__restrict__ inv_freq,
+                                          const int32_t *__restrict__ pos, __half *__restrict__ kcache,
+                                          __half *__restrict__ vcache, int n_heads, int n_kv, int head_dim,
+                                          int ctx_cap)
+    {
+        const int b = blockIdx.y, h = blockIdx.x, i = threadIdx.x;
+        const int half_dim = head_dim >> 1;
+        const int p = pos[b];
+        float *row = qkv + (size_t)b * ld_qkv;
+        const float angle = (float)p * inv_freq[i];
+        const float c = cosf(angle), s = sinf(angle);
+        float *head = row + (size_t)h * head_dim;
+        const float x0 = head[i], x1 = head[i + half_dim];
+        const float r0 = x0 * c - x1 * s;
+        const float r1 = x0 * s + x1 * c;
+        if (h < n_heads)
+        {
+            head[i] = r0;
+            head[i + half_dim] = r1;
+            return;
+        }
+        if (p < 0 || p >= ctx_cap)
+            return;
+        const int kh = h - n_heads;
+        const size_t at = (((size_t)b * n_kv + kh) * ctx_cap + p) * head_dim;
+        kcache[at + i] = __float2half_rn(r0);
+        kcache[at + i + half_dim] = __float2half_rn(r1);
+        const float *vhead = row + (size_t)(n_heads + n_kv + kh) * head_dim;
+        vcache[at + i] = __float2half_rn(vhead[i]);
+        vcache[at + i + half_dim] = __float2half_rn(vhead[i + half_dim]);
+    }
+
+    // ---- attention --------------------------------------------------------------------------
+    // Workgroup = (chunk of ATT_CHUNK cache positions, KV head, sequence); its G = n_heads/n_kv
+    // query heads share every K and V row it reads.  Sixteen lanes cover the 128 columns of
+    // a row (8 fp16 = 16 bytes each), so a wavefront takes four positions per pass.
+    //   pass 1: scores s[p][g] = q_g . K[p] / sqrt(d)          -> LDS
+    //   softmax statistics of the chunk per head: m = max, e = exp(s - m), l = sum e
+    //   pass 2: o_g = sum_p e[p][g] V[p]                       -> partial result per chunk
+    // A second kernel merges the chunks: o = sum_c o_c exp(m_c - M) / sum_c l_c exp(m_c - M).
+    constexpr int ATT_CHUNK = 128;
+    constexpr int ATT_THREADS = 256;
+    constexpr int ATT_HD = 128;
+
+    __device__ __forceinline__ void load_row8(const __half *p, float (&v)[8])
+    {
+        const uint4 raw = *reinterpret_cast<const uint4 *>(p);
+        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const float2 f = __half22float2(h[j]);
+            v[2 * j] = f.x;
+            v[2 * j + 1] = f.y;
+        }
+    }
+
+    template <int G>
+    __global__ void __launch_bounds__(ATT_THREADS)
+        attention_partial_kernel(const float *__restrict__ q, int ld_q, const __half *__restrict__ kcache,
+                                 const __half *__restrict__ vcache, const int32_t *__restrict__ pos,
+                                 float *__restrict__ part_o, float *__restrict__ part_ml, int n_heads, int n_kv,
+                                 int ctx_cap, int n_chunks)
+    {
+        __shared__ float s_sc[ATT_CHUNK][G];
+        __shared__ float s_o[ATT_THREADS / WAVE][G][ATT_HD];
+        const int chunk = blockIdx.x, kh = blockIdx.y, b = blockIdx.z;
+        const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
+        const int col = (lane & 15) * 8, prow = lane >> 4;
+        const int last = pos[b] < ctx_cap - 1 ? pos[b] : ctx_cap - 1; // newest position, inclusive
+        const int p0 = chunk * ATT_CHUNK;
+        const size_t out_base = ((size_t)b * n_heads + (size_t)kh * G) * n_chunks + chunk;
+        if (p0 > last)
+        {
+            // nothing to attend to in this chunk: weight zero in the merge
+            if (threadIdx.x < G)
+            {
+                part_ml[(out_base + (size_t)threadIdx.x * n_chunks) * 2 + 0] = -INFINITY;
+                part_ml[(out_base + (size_t)threadIdx.x * n_chunks) * 2 + 1] = 0.0f;
+            }
+            return;
+        }
+        const __half *kbase = kcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
+        const __half *vbase = vcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
+
+        float qv[G][8];
+        const float scale = 0.08838834764831845f; // 1/sqrt(128)
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+        {
+            const float *qh = q + (size_t)b * ld_q + (size_t)(kh * G + g) * ATT_HD + col;
+            const float4 a = *reinterpret_cast<const float4 *>(qh);
+            const float4 c = *reinterpret_cast<const float4 *>(qh + 4);
+            qv[g][0] = a.x * scale, qv[g][1] = a.y * scale, qv[g][2] = a.z * scale, qv[g][3] = a.w * scale;
+            qv[g][4] = c.x * scale, qv[g][5] = c.y * scale, qv[g][6] = c.z * scale, qv[g][7] = c.w * scale;
+        }
+
+        // pass 1
+        constexpr int PER_WAVE = ATT_CHUNK / (ATT_THREADS / WAVE); // positions per wavefront
+#pragma unroll 2
+        for (int it = 0; it < PER_WAVE / 4; ++it)
+        {
+            const int pl = wave * PER_WAVE + it * 4 + prow;
+            const int p = p0 + pl;
+            const bool valid = p <= last;
+            float kv[8];
+            load_row8(kbase + (size_t)(valid ? p : last) * ATT_HD + col, kv);
+            float s[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+            {
+                float a = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    a = fmaf(qv[g][j], kv[j], a);
+                a += dpp_f32<DPP_QUAD_XOR1>(a);
+                a += dpp_f32<DPP_QUAD_XOR2>(a);
+                a += dpp_f32<DPP_ROW_HALF_MIRROR>(a);
+                a += dpp_f32<DPP_ROW_MIRROR>(a);
+                s[g] = valid ? a : -INFINITY;
+            }
+            if ((lane & 15) == 0)
+            {
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+                    s_sc[pl][g] = s[g];
+            }
+        }
+        __syncthreads();
+
+        // statistics: wavefront w takes heads w, w + 4, ...
+        for (int g = wave; g < G; g += ATT_THREADS / WAVE)
+        {
+            const float a0 = s_sc[lane][g], a1 = s_sc[lane + 64][g];
+            float mx = fmaxf(a0, a1);
+#pragma unroll
+            for (int off = WAVE / 2; off > 0; off >>= 1)
+                mx = fmaxf(mx, __shfl_xor(mx, off, WAVE));
+            const float e0 = expf(a0 - mx), e1 = expf(a1 - mx); // position p0 is valid: mx is finite
+            s_sc[lane][g] = e0;
+            s_sc[lane + 64][g] = e1;
+            float l = e0 + e1;
+#pragma unroll
+            for (int off = WAVE / 2; off > 0; off >>= 1)
+                l += __shfl_xor(l, off, WAVE);
+            if (lane == 0)
+            {
+                part_ml[(out_base + (size_t)g * n_chunks) * 2 + 0] = mx;
+                part_ml[(out_base + (size_t)g * n_chunks) * 2 + 1] = l;
+            }
+        }
+        __syncthreads();
+
+        // pass 2
+        float o[G][8];
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                o[g][j] = 0.0f;
+#pragma unroll 2
+        for (int it = 0; it < PER_WAVE / 4; ++it)
+        {
+            const int pl = wave * PER_WAVE + it * 4 + prow;
+            const int p = p0 + pl;
+            float vv[8];
+            load_row8(vbase + (size_t)(p <= last ? p : last) * ATT_HD + col, vv); // weight 0 past the end
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+            {
+                const float w = s_sc[pl][g];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    o[g][j] = fmaf(w, vv[j], o[g][j]);
+            }
+        }
+        // the four position rows of a wavefront, then the wavefronts
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+            {
+                float a = o[g][j];
+                a += __shfl_xor(a, 16, WAVE);
+                a += __shfl_xor(a, 32, WAVE);
+                o[g][j] = a;
+            }
+        if (prow == 0)
+        {
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    s_o[wave][g][col + j] = o[g][j];
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < G * ATT_HD; i += ATT_THREADS)
+        {
+            const int g = i / ATT_HD, c = i % ATT_HD;
+            float a = 0.0f;
+#pragma unroll
+            for (int w = 0; w < ATT_THREADS / WAVE; ++w)
+                a += s_o[w][g][c];
+            part_o[(out_base + (size_t)g * n_chunks) * ATT_HD + c] = a;
+        }
+    }
+
+    // One workgroup of 128 threads per (sequence, head).
+    __global__ void __launch_bounds__(ATT_HD)
+        attention_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                               float *__restrict__ out, int ld_out, int n_heads, int n_chunks)
+    {
+        const int h = blockIdx.x, b = blockIdx.y, c = threadIdx.x;
+        const size_t base = ((size_t)b * n_heads + h) * n_chunks;
+        float M = -INFINITY;
+        for (int k = 0; k < n_chunks; ++k)
+            M = fmaxf(M, part_ml[(base + k) * 2]);
+        float L = 0.0f, acc = 0.0f;
+        for (int k = 0; k < n_chunks; ++k)
+        {
+            const float mk = part_ml[(base + k) * 2];
+            if (mk == -INFINITY)
+                continue; // chunk past the newest position: its partial row was not written
+            const float w = expf(mk - M);
+            L = fmaf(part_ml[(base + k) * 2 + 1], w, L);
+            acc = fmaf(part_o[(base + k) * ATT_HD + c], w, acc);
+        }
+        out[(size_t)b * ld_out + (size_t)h * ATT_HD + c] = L > 0.0f ? __fdiv_rn(acc, L) : 0.0f; // pos < 0: nothing attended
+    }
+
+    // ---- greedy sampling -----------------------------------------------------------------------
+    constexpr int ARGMAX_THREADS = 256;
+    constexpr int ARGMAX_PER_THREAD = 8;
+
+    __device__ __forceinline__ bool argmax_better(float cv, int ci, float v, int i)
+    {
+        return cv > v || (cv == v && ci < i);
+    }
+
+    __device__ __forceinline__ void argmax_block_reduce(float &v, int &idx, float *s_v, int *s_i)
+    {
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1)
+        {
+            const float ov = __shfl_xor(v, off, WAVE);
+            const int oi = __shfl_xor(idx, off, WAVE);
+            if (argmax_better(ov, oi, v, idx))
+            {
+                v = ov;
+                idx = oi;
+            }
+        }
+        if ((threadIdx.x & (WAVE - 1)) == 0)
+        {
+            s_v[threadIdx.x >> 6] = v;
+            s_i[threadIdx.x >> 6] = idx;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0)
+        {
+            for (int w = 1; w < ARGMAX_THREADS / WAVE; ++w)
+                if (argmax_better(s_v[w], s_i[w], v, idx))
+                {
+                    v = s_v[w];
+                    idx = s_i[w];
+                }
+        }
+    }
+
+    __global__ void __launch_bounds__(ARGMAX_THREADS)
+        argmax_partial_kernel(const float *__restrict__ logits, int ld, int n, float *__restrict__ pv,
+                              int *__restrict__ pi)
+    {
+        __shared__ float s_v[ARGMAX_THREADS / WAVE];
+        __shared__ int s_i[ARGMAX_THREADS / WAVE];
+        const int b = blockIdx.y;
+        const float *row = logits + (size_t)b * ld;
+        float v = -FLT_MAX;
+        int idx = INT_MAX;
+        const int stride = ARGMAX_THREADS * gridDim.x;
+        for (int i = blockIdx.x * ARGMAX_THREADS + threadIdx.x; i < n; i += stride)
+        {
+            const float x = row[i];
+            if (argmax_better(x, i, v, idx))
+            {
+                v = x;
+                idx = i;
+            }
+        }
+        argmax_block_reduce(v, idx, s_v, s_i);
+        if (threadIdx.x == 0)
+        {
+            pv[(size_t)b * gridDim.x + blockIdx.x] = v;
+            pi[(size_t)b * gridDim.x + blockIdx.x] = idx;
+        }
+    }
+
+    __global__ void __launch_bounds__(ARGMAX_THREADS)
+        argmax_final_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int n_part,
+                            int32_t *__restrict__ ids, int32_t *__restrict__ pos)
+    {
+        __shared__ float s_v[ARGMAX_THREADS / WAVE];
+        __shared__ int s_i[ARGMAX_THREADS / WAVE];
+        const int b = blockIdx.x;
+        float v = -FLT_MAX;
+        int idx = INT_MAX;
+        for (int i = threadIdx.x; i < n_part; i += ARGMAX_THREADS)
+        {
+            const float x = pv[(size_t)b * n_part + i];
+            const int xi = pi[(size_t)b * n_part + i];
+            if (argmax_better(x, xi, v, idx))
+            {
+                v = x;
+                idx = xi;
+            }
+        }
+        argmax_block_reduce(v, idx, s_v, s_i);
+        if (threadIdx.x == 0)
+        {
+            ids[b] = idx;
+            if (pos)
+                pos[b] += 1;
+        }
+    }
+
+    inline int argmax_blocks(int n)
+    {
+        const int per_block = ARGMAX_THREADS * ARGMAX_PER_THREAD;
+        return (n + per_block - 1) / per_block;
+    }
+} // namespace llamql
+
+using namespace llamql;
+
+extern "C" bool llam_dec_embed_q4k(const void *d_table, int vocab, const int32_t *d_ids, float *d_x,
+                                   int B, int H, int ldx, int device_id, void *stream)
+{
+    static const char *fn = "llam_dec_embed_q4k";
+    if (B < 0 || vocab < 1 || H < 1)
+        return fail(fn, "bad size (B=%d vocab=%d H=%d)", B, vocab, H);
+    if (B == 0)
+        return true;
+    if ((H % 256) != 0 || ldx < H)
+        return fail(fn, "H=%d must be a multiple of 256 and ldx=%d at least H", H, ldx);
+    if (!d_table || !d_ids || !d_x)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_table) || !aligned4(d_ids) || !aligned4(d_x))
+        return fail(fn, "misaligned pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(embed_q4k_kernel, dim3(H / 256, B), dim3(256), 0, as_stream(stream),
+                       static_cast<const llam_block_q4_K *>(d_table), vocab, d_ids, d_x, H / 256, ldx);
+    return launched(fn);
+}
+
+extern "C" bool llam_dec_rmsnorm_q8_1(float *d_x, const float *d_delta, const float *d_gamma, float eps,
+                                      float *d_y, void *d_q8, int M, int H, int device_id, void *stream)
+{
+    static const char *fn = "llam_dec_rmsnorm_q8_1";
+    if (M < 0 || H < 1)
+        return fail(fn, "bad size (M=%d H=%d)", M, H);
+    if (M == 0)
+        return true;
+    if ((H % 32) != 0)
+        return fail(fn, "H=%d must be a multiple of 32", H);
+    if (!d_x || !d_gamma)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_x) || !aligned16(d_gamma) || (d_delta && !aligned16(d_delta)) || (d_y && !aligned16(d_y)) ||
+        (d_q8 && !aligned4(d_q8)))
+        return fail(fn, "fp32 rows must be 16-byte aligned, d_q8 4-byte aligned");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(rmsnorm_q8_1_kernel, dim3(M), dim3(NORM_THREADS), 0, as_stream(stream), d_x, d_delta,
+                       d_gamma, eps, d_y, static_cast<uint32_t *>(d_q8), H);
+    return launched(fn);
+}
+
+extern "C" void llam_dec_rope_inv_freq(int head_dim, float theta, float *h_inv_freq)
+{
+    const int half_dim = head_dim / 2;
+    const float log_base = std::log(theta);
+    for (int i = 0; i < half_dim; ++i)
+    {
+        const float exponent = (2.0f * (float)i) / (float)head_dim;
+        h_inv_freq[i] = std::exp(-log_base * exponent);
+    }
+}
+
+extern "C" bool llam_dec_rope_kv_append(float *d_qkv, int ld_qkv, const float *d_inv_freq,
+                                        const int32_t *d_pos, void *d_kcache, void *d_vcache, int B,
+                                        int n_heads, int n_kv, int head_dim, int ctx_cap, int device_id,
+                                        void *stream)
+{
+    static const char *fn = "llam_dec_rope_kv_append";
+    if (B < 0 || n_heads < 1 || n_kv < 1 || head_dim < 2 || ctx_cap < 1)
+        return fail(fn, "bad size");
+    if (B == 0)
+        return true;
+    if ((head_dim % 2) != 0 || head_dim / 2 > 1024)
+        return fail(fn, "head_dim=%d must be even and at most 2048", head_dim);
+    if (ld_qkv < (n_heads + 2 * n_kv) * head_dim)
+        return fail(fn, "ld_qkv=%d smaller than (n_heads + 2 n_kv) * head_dim", ld_qkv);
+    if (!d_qkv || !d_inv_freq || !d_pos || !d_kcache || !d_vcache)
+        return fail(fn, "null pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(rope_kv_append_kernel, dim3(n_heads + n_kv, B), dim3(head_dim / 2), 0, as_stream(stream),
+                       d_qkv, ld_qkv, d_inv_freq, d_pos, static_cast<__half *>(d_kcache),
+                       static_cast<__half *>(d_vcache), n_heads, n_kv, head_dim, ctx_cap);
+    return launched(fn);
+}
+
+extern "C" size_t llam_dec_attention_scratch_floats(int B, int n_heads, int head_dim, int ctx_cap)
+{
+    if (B < 1 || n_heads < 1 || head_dim < 1 || ctx_cap < 1)
+        return 0;
+    const size_t chunks = ((size_t)ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
+    return (size_t)B * n_heads * chunks * ((size_t)head_dim + 2);
+}
+
+extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kcache, const void *d_vcache,
+                                   const int32_t *d_pos, float *d_out, int ld_out, float *d_scratch, int B,
+                                   int n_heads, int n_kv, int head_dim, int ctx_cap, int device_id,
+                                   void *stream)
+{
+    static const char *fn = "llam_dec_attention";
+    if (B < 0 || n_heads < 1 || n_kv < 1 || ctx_cap < 1)
+        return fail(fn, "bad size");
+    if (B == 0)
+        return true;
+    if (head_dim != ATT_HD)
+        return fail(fn, "head_dim=%d: only 128 is built", head_dim);
+    if ((n_heads % n_kv) != 0)
+        return fail(fn, "n_heads=%d not a multiple of n_kv=%d", n_heads, n_kv);
+    const int G = n_heads / n_kv;
+    if (G != 1 && G != 2 && G != 4 && G != 8)
+        return fail(fn, "n_heads/n_kv=%d: only 1, 2, 4 and 8 are built", G);
+    if (ld_q < n_heads * head_dim || ld_out < n_heads * head_dim)
+        return fail(fn, "row strides smaller than n_heads * head_dim");
+    if (!d_q || !d_kcache || !d_vcache || !d_pos || !d_out || !d_scratch)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_q) || (ld_q % 4) != 0 || !aligned16(d_kcache) || !aligned16(d_vcache) || !aligned4(d_out) ||
+        !aligned4(d_scratch))
+        return fail(fn, "misaligned pointer");
+    const int n_chunks = (ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
+    if ((long)n_chunks > 65535 || B > 65535)
+        return fail(fn, "too many chunks or sequences");
+    if (!set_device(fn, device_id))
+        return false;
+    float *part_o = d_scratch;
+    float *part_ml = d_scratch + (size_t)B * n_heads * n_chunks * ATT_HD;
+    const __half *kc = static_cast<const __half *>(d_kcache);
+    const __half *vc = static_cast<const __half *>(d_vcache);
+    const dim3 grid(n_chunks, n_kv, B);
+    hipStream_t st = as_stream(stream);
+    switch (G)
+    {
+    case 1:
+        hipLaunchKernelGGL(attention_partial_kernel<1>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
+                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
+        break;
+    case 2:
+        hipLaunchKernelGGL(attention_partial_kernel<2>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
+                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
+        break;
+    case 4:
+        hipLaunchKernelGGL(attention_partial_kernel<4>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
+                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
+        break;
+    default:
+        hipLaunchKernelGGL(attention_partial_kernel<8>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
+                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
+        break;
+    }
+    if (!launched(fn))
+        return false;
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(n_heads, B), dim3(ATT_HD), 0, st, part_o, part_ml, d_out,
+                       ld_out, n_heads, n_chunks);
+    return launched(fn);
+}
+
+extern "C" size_t llam_dec_argmax_scratch_bytes(int B, int n)
+{
+    if (B < 1 || n < 1)
+        return 0;
+    return (size_t)B * argmax_blocks(n) * (sizeof(float) + sizeof(int));
+}
+
+extern "C" bool llam_dec_argmax(const float *d_logits, int ld, int n, int B, int32_t *d_ids, int32_t *d_pos,
+                                void *d_scratch, int device_id, void *stream)
+{
+    static const char *fn = "llam_dec_argmax";
+    if (B < 0 || n < 1 || ld < n)
+        return fail(fn, "bad size (B=%d n=%d ld=%d)", B, n, ld);
+    if (B == 0)
+        return true;
+    if (!d_logits || !d_ids || !d_scratch)
+        return fail(fn, "null pointer");
+    if (!aligned4(d_logits) || !aligned4(d_ids) || !aligned4(d_scratch) || (d_pos && !aligned4(d_pos)))
+        return fail(fn, "misaligned pointer");
+    if (B > 65535)
+        return fail(fn, "too many rows");
+    if (!set_device(fn, device_id))
+        return false;
+    const int blocks = argmax_blocks(n);
+    float *pv = static_cast<float *>(d_scratch);
+    int *pi = reinterpret_cast<int *>(pv + (size_t)B * blocks);
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(blocks, B), dim3(ARGMAX_THREADS), 0, as_stream(stream), d_logits,
+                       ld, n, pv, pi);
+    if (!launched(fn))
+        return false;
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(B), dim3(ARGMAX_THREADS), 0, as_stream(stream), pv, pi, blocks,
+                       d_ids, d_pos);
+    return launched(fn);
+}

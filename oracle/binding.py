@@ -54,6 +54,14 @@ class Oracle:
         L.qlo_epilogue.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]
         L.qlo_moe_route.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
         L.qlo_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_void_p]
+        L.qlo_dequant_row_q4k.argtypes = [c_void_p, c_int, c_void_p]
+        L.qlo_rmsnorm.argtypes = [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int]
+        L.qlo_rope_inv_freq.argtypes = [c_int, c_float, c_void_p]
+        L.qlo_rope_head.argtypes = [c_void_p, c_int, c_void_p, c_int]
+        L.qlo_rope_kv_append.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int]
+        L.qlo_attention_decode.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int]
+        L.qlo_argmax.restype = c_int
+        L.qlo_argmax.argtypes = [c_void_p, c_int]
         self.L = L
 
     # -- fp16 ---------------------------------------------------------------
@@ -143,6 +151,56 @@ class Oracle:
         self.L.qlo_swiglu(_p(gate), _p(up), gate.size, _p(out))
         return out
 
+    # -- decode-step operators ------------------------------------------------------
+    def dequant_rows_q4k(self, blocks: np.ndarray) -> np.ndarray:
+        """blocks: uint8 [..., nsb, 144] -> float32 [..., nsb*256]."""
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        n = blocks.size // 144
+        out = np.zeros(n * 256, np.float32)
+        self.L.qlo_dequant_row_q4k(_p(blocks), n, _p(out))
+        return out.reshape(blocks.shape[:-2] + (blocks.shape[-2] * 256,))
+
+    def rmsnorm(self, x: np.ndarray, gamma: np.ndarray, eps: float, delta=None):
+        """Returns (y, x_after): x_after = x + delta when delta is given."""
+        x = np.ascontiguousarray(x, dtype=np.float32).copy()
+        rows, cols = x.shape
+        g = np.ascontiguousarray(gamma, dtype=np.float32)
+        d = np.ascontiguousarray(delta, dtype=np.float32) if delta is not None else None
+        y = np.zeros_like(x)
+        self.L.qlo_rmsnorm(_p(x), _p(d) if d is not None else None, _p(g), eps, _p(y), rows, cols)
+        return y, x
+
+    def rope_inv_freq(self, head_dim: int, theta: float) -> np.ndarray:
+        out = np.zeros(head_dim // 2, np.float32)
+        self.L.qlo_rope_inv_freq(head_dim, theta, _p(out))
+        return out
+
+    def rope_head(self, head: np.ndarray, position: int, inv_freq: np.ndarray) -> np.ndarray:
+        h = np.ascontiguousarray(head, dtype=np.float32).copy()
+        self.L.qlo_rope_head(_p(h), position, _p(inv_freq), h.size)
+        return h
+
+    def rope_kv_append(self, qkv: np.ndarray, inv_freq, position: int, kcache: np.ndarray, vcache: np.ndarray,
+                       n_heads: int, n_kv: int, head_dim: int) -> np.ndarray:
+        """qkv: [(n_heads+2 n_kv)*head_dim]; caches uint16 [n_kv, ctx_cap, head_dim], updated in place."""
+        q = np.ascontiguousarray(qkv, dtype=np.float32).copy()
+        assert kcache.dtype == np.uint16 and kcache.flags.c_contiguous and vcache.flags.c_contiguous
+        self.L.qlo_rope_kv_append(_p(q), _p(inv_freq), position, _p(kcache), _p(vcache), n_heads, n_kv, head_dim,
+                                  kcache.shape[1])
+        return q
+
+    def attention_decode(self, q: np.ndarray, kcache: np.ndarray, vcache: np.ndarray, last: int, n_heads: int,
+                         n_kv: int, head_dim: int) -> np.ndarray:
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        out = np.zeros(n_heads * head_dim, np.float32)
+        self.L.qlo_attention_decode(_p(q), _p(kcache), _p(vcache), last, _p(out), n_heads, n_kv, head_dim,
+                                    kcache.shape[1])
+        return out
+
+    def argmax(self, x: np.ndarray) -> int:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        return int(self.L.qlo_argmax(_p(x), x.size))
+
 
 class Ref:
     """The reference's own code.  `available()` is False where it was not built
@@ -175,6 +233,13 @@ class Ref:
         L.ref_gemm.restype = c_int
         L.ref_gemm.argtypes = [c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int]
         L.ref_omp_threads.restype = c_int
+        self.has_decode = hasattr(L, "ref_rmsnorm_row")
+        if self.has_decode:
+            L.ref_rmsnorm_row.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_long, c_float]
+            L.ref_residual_rmsnorm_row.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_float]
+            L.ref_rope_inv_freq.argtypes = [c_int, c_float, c_void_p]
+            L.ref_rope_token.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float]
+            L.ref_rope_head_scalar.argtypes = [c_void_p, c_int, c_int, c_float]
         self.L = L
 
     def f16_to_f32(self, h):
@@ -249,3 +314,35 @@ class Ref:
 
     def omp_threads(self) -> int:
         return int(self.L.ref_omp_threads())
+
+    # -- decode-step primitives --------------------------------------------------------
+    def rmsnorm_row(self, x, gamma, eps, variant=3):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        g = np.ascontiguousarray(gamma, dtype=np.float32)
+        y = np.zeros_like(x)
+        self.L.ref_rmsnorm_row(variant, _p(x), _p(g), _p(y), x.size, eps)
+        return y
+
+    def residual_rmsnorm_row(self, delta, residual, gamma, eps):
+        d = np.ascontiguousarray(delta, dtype=np.float32)
+        r = np.ascontiguousarray(residual, dtype=np.float32).copy()
+        g = np.ascontiguousarray(gamma, dtype=np.float32)
+        y = np.zeros_like(r)
+        self.L.ref_residual_rmsnorm_row(_p(d), _p(r), _p(g), _p(y), r.size, eps)
+        return y, r
+
+    def rope_inv_freq(self, head_dim, theta):
+        out = np.zeros(head_dim // 2, np.float32)
+        self.L.ref_rope_inv_freq(head_dim, theta, _p(out))
+        return out
+
+    def rope_token(self, q, k, head_dim, n_past, theta):
+        q = np.ascontiguousarray(q, dtype=np.float32).copy()
+        k = np.ascontiguousarray(k, dtype=np.float32).copy()
+        self.L.ref_rope_token(_p(q), _p(k), head_dim, q.size // head_dim, k.size // head_dim, n_past, theta)
+        return q, k
+
+    def rope_head_scalar(self, head, position, theta):
+        h = np.ascontiguousarray(head, dtype=np.float32).copy()
+        self.L.ref_rope_head_scalar(_p(h), position, h.size, theta)
+        return h

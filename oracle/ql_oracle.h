@@ -92,6 +92,17 @@ void qlo_moe_route(const float *logits, int n_tokens, int n_experts, int top_k,
  * and is not bit-reproducible; this is the mathematical function it approximates. */
 void qlo_swiglu(const float *gate, const float *up, int n, float *out);
 
+/* ---- decode-step operators (decode_oracle.c) ------------------------------------- */
+void qlo_dequant_row_q4k(const llam_block_q4_K *blocks, int nblocks, float *out);
+void qlo_rmsnorm(float *x, const float *delta, const float *gamma, float eps, float *y, int rows, int cols);
+void qlo_rope_inv_freq(int head_dim, float theta, float *inv_freq);
+void qlo_rope_head(float *head, int position, const float *inv_freq, int head_dim);
+void qlo_rope_kv_append(float *qkv, const float *inv_freq, int position, uint16_t *kcache, uint16_t *vcache,
+                        int n_heads, int n_kv, int head_dim, int ctx_cap);
+void qlo_attention_decode(const float *q, const uint16_t *kcache, const uint16_t *vcache, int last, float *out,
+                          int n_heads, int n_kv, int head_dim, int ctx_cap);
+int qlo_argmax(const float *x, int n);
+
 #ifdef __cplusplus
 }
 #endif

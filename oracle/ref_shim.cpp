@@ -18,6 +18,8 @@
 #include <vector>
 
 #include "kernels/cpu/native_vnni/CPUNativeVNNIGemv.h"
+#include "kernels/cpu/primitives/RMSNormPrimitives.h"
+#include "kernels/cpu/primitives/RoPEPrimitives.h"
 #include "tensors/BlockStructures.h"
 #include "tensors/FP16Utils.h"
 #include "tensors/IQQuantTables.h"
@@ -252,4 +254,38 @@ extern "C"
     }
 
     int ref_omp_threads() { return omp_get_max_threads(); }
+
+    // ---- decode-step operators: the reference's primitives, compiled by the Makefile from
+    // kernels/cpu/primitives/{RMSNormPrimitives,RoPEPrimitives}.cpp where they lie ----------
+    // variant: 1 scalar, 2 AVX2, 3 AVX512
+    void ref_rmsnorm_row(int variant, const float *src, const float *gamma, float *dst, long cols, float eps)
+    {
+        if (variant == 1)
+            primitives::rmsnorm_fused_row_scalar(src, gamma, dst, (std::size_t)cols, eps);
+        else if (variant == 2)
+            primitives::rmsnorm_fused_row_avx2(src, gamma, dst, (std::size_t)cols, eps);
+        else
+            primitives::rmsnorm_fused_row_avx512(src, gamma, dst, (std::size_t)cols, eps);
+    }
+    // residual += input, then RMSNorm of the new residual
+    void ref_residual_rmsnorm_row(const float *input, float *residual, const float *gamma, float *output, long cols,
+                                  float eps)
+    {
+        primitives::fused_residual_rmsnorm_row_avx512(input, residual, gamma, output, (std::size_t)cols, eps);
+    }
+    void ref_rope_inv_freq(int head_dim, float theta, float *out)
+    {
+        const std::vector<float> &f = primitives::get_inv_freq_cached(head_dim, theta);
+        std::memcpy(out, f.data(), f.size() * sizeof(float));
+    }
+    // one token at position n_past: q [q_heads*head_dim], k [k_heads*head_dim], in place
+    void ref_rope_token(float *q, float *k, int head_dim, int q_heads, int k_heads, int n_past, float theta)
+    {
+        primitives::apply_rope_vectorized(q, k, 1, head_dim, q_heads, k_heads, n_past, theta, nullptr);
+    }
+    void ref_rope_head_scalar(float *head, int position, int head_dim, float theta)
+    {
+        primitives::apply_rope_to_head_scalar(head, position, primitives::get_inv_freq_cached(head_dim, theta),
+                                              head_dim, 0);
+    }
 }

@@ -11,12 +11,13 @@ import pytest
 
 ROOT = Path(__file__).resolve().parent.parent
 HEADER = ROOT / "include" / "llaminar_amd" / "ql_api.h"
+DECODE_HEADER = ROOT / "include" / "llaminar_amd" / "decode_api.h"
 
 
 def declared_symbols():
-    text = HEADER.read_text()
+    text = HEADER.read_text() + DECODE_HEADER.read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(llam_ql_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(llam_(?:ql|dec)_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -27,8 +28,8 @@ def test_library_exports_every_declared_symbol():
     names = declared_symbols()
     assert len(names) >= 14
     for n in names:
-        assert hasattr(lib, n), f"{n} declared in ql_api.h but not exported"
-    assert set(names) == set(capi.SIGNATURES), "capi.SIGNATURES out of step with ql_api.h"
+        assert hasattr(lib, n), f"{n} declared in include/ but not exported"
+    assert set(names) == set(capi.SIGNATURES), "capi.SIGNATURES out of step with the headers"
 
 
 def test_block_layouts_match_header():
