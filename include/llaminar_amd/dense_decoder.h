@@ -1,0 +1,100 @@
+/* Host-side driver of one greedy decode step of a dense decoder-only model: the order
+ * in which a layer's operators are enqueued, and the buffers between them.  C ABI over
+ * an opaque handle, exported by the host library next to the C++ operator classes.
+ *
+ * The step follows the node order the reference builds for a decoder layer
+ * (src/v2/models/qwen/QwenGraphBase.cpp: addPreAttentionNorm :2586, fused QKV projection,
+ * addRoPE :2691, addKVCacheAppend :2736, addKVCacheAndAttention :2785,
+ * addWoProjectionAndAllreduce :2937, buildFFNGraph :1974, addFinalNormToGraph :2447,
+ * buildLMHeadGraph :1789) followed by greedy sampling:
+ *
+ *   x = embed[ids]
+ *   per layer:  h  = Q8_1(rmsnorm(x += down_prev) * attn_norm)       (no add in layer 0)
+ *               q,k,v = W{q,k,v} h ; rope(q, k, pos) ; cache[pos] = fp16(k, v)
+ *               a  = attention(q, cache[0..pos])
+ *               o  = Wo Q8_1(a)
+ *               h2 = Q8_1(rmsnorm(x += o) * ffn_norm)
+ *               down = Wdown Q8_1(silu(Wgate h2) * (Wup h2))
+ *   logits = Wlm Q8_1(rmsnorm(x += down) * final_norm) ; ids = argmax(logits) ; pos += 1
+ *
+ * llam_decoder_step() only enqueues kernels on the given stream (about 12 per layer):
+ * no allocation, no synchronisation, no host read of device data.  Token ids and
+ * positions live in device memory and are advanced by the step itself, so a step can
+ * be captured in a HIP graph once and replayed for every following token.
+ *
+ * Weights are borrowed: device pointers in the layouts of ql_api.h, owned by the caller
+ * for the life of the handle.  All functions return false (NULL) on error and keep the
+ * reason for llam_decoder_last_error(). */
+#ifndef LLAMINAR_AMD_DENSE_DECODER_H
+#define LLAMINAR_AMD_DENSE_DECODER_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct
+{
+    int hidden;    /* model width, multiple of 256 */
+    int n_heads;   /* query heads */
+    int n_kv;      /* key/value heads (n_heads / n_kv in {1,2,4,8}) */
+    int head_dim;  /* 128 */
+    int ffn;       /* feed-forward width, multiple of 256 */
+    int vocab;
+    int n_layers;
+    int ctx_cap;   /* KV-cache positions per sequence */
+    int batch;     /* sequences decoded together, 1..8 */
+    float rope_theta;
+    float rms_eps;
+    int device_id;
+} llam_decoder_config;
+
+typedef struct
+{
+    const void *wq, *wk, *wv, *wo, *wgate, *wup, *wdown; /* prepared weights (llam_ql_prepare_weights) */
+    uint8_t fmt_q, fmt_k, fmt_v, fmt_o, fmt_gate, fmt_up, fmt_down;
+    const float *attn_norm; /* [hidden] */
+    const float *ffn_norm;  /* [hidden] */
+} llam_decoder_layer;
+
+typedef struct
+{
+    const void *embed_q4k;   /* GGUF Q4_K [vocab][hidden/256] */
+    const float *final_norm; /* [hidden] */
+    const void *lm_head;     /* prepared weights [vocab x hidden] */
+    uint8_t fmt_lm_head;
+} llam_decoder_globals;
+
+/* Allocates the activation buffers, the KV caches (2 * n_layers * batch * n_kv * ctx_cap *
+ * head_dim fp16) and the scratch of the operators on cfg->device_id. */
+void *llam_decoder_create(const llam_decoder_config *cfg);
+void llam_decoder_destroy(void *dec);
+
+bool llam_decoder_set_layer(void *dec, int layer, const llam_decoder_layer *w);
+bool llam_decoder_set_globals(void *dec, const llam_decoder_globals *g);
+
+/* Current token and its position per sequence (host arrays of `batch` entries); copies
+ * synchronously.  The cache must hold positions 0..pos-1 already (llam_decoder_buffer). */
+bool llam_decoder_set_state(void *dec, const int32_t *h_ids, const int32_t *h_pos);
+
+/* One token for every sequence; see the file comment. */
+bool llam_decoder_step(void *dec, void *stream);
+
+/* Device buffers, for filling caches, reading results and parity checks:
+ *   "ids" int32[batch], "pos" int32[batch], "logits" fp32[batch][vocab], "x" fp32[batch][hidden]
+ *   (the residual stream as the last step left it, before the final add of "delta"),
+ *   "delta" fp32[batch][hidden], "kcache"/"vcache" fp16[batch][n_kv][ctx_cap][head_dim] of `layer`. */
+void *llam_decoder_buffer(void *dec, const char *name, int layer);
+
+/* Bytes of device memory the handle owns. */
+size_t llam_decoder_device_bytes(void *dec);
+
+const char *llam_decoder_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

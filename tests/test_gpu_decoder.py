@@ -1,0 +1,161 @@
+"""The host library's decode step (dense_decoder.h) against a numpy walk through the same
+operators built from the CPU restatements: same weights, same cache, three tokens.
+
+The step chains about a dozen operators per layer whose fp32 results differ from the
+restatement's in the last bits (summation order, device sin/cos/exp); each Q8_1 quantiser on
+the way turns such a difference into at most one int8 step on a few elements.  The logits
+are therefore compared at 5e-3 of the largest logit, and the greedy token wherever the
+restatement's top-2 gap exceeds that."""
+import numpy as np
+import pytest
+
+from llaminar_amd.capi import FMT_Q4_K, FMT_Q6_K
+from tests.helpers import sync
+
+pytestmark = pytest.mark.gpu
+
+
+class NumpyDecoder:
+    """One sequence at a time through oracle/*.c, in the order of llam_decoder_step."""
+
+    def __init__(self, oracle, shape, raw, ctx_cap):
+        self.o, self.s, self.cap = oracle, shape, ctx_cap
+        self.w = {k: v.cpu().numpy() for k, v in raw.items()}
+        self.inv_freq = oracle.rope_inv_freq(shape.head_dim, shape.rope_theta)
+
+    def gemv(self, name, fmt, K, x):
+        return self.o.gemm(fmt, self.w[name], K, self.o.quantize(x[None]))[0]
+
+    def step(self, token, pos, kcache, vcache):
+        """kcache/vcache: uint16 [n_layers, n_kv, cap, hd] of this sequence, updated in place."""
+        o, s = self.o, self.s
+        H, hd = s.hidden, s.head_dim
+        qd, kvd = s.n_heads * hd, s.n_kv * hd
+        x = o.dequant_rows_q4k(self.w["embed"].reshape(s.vocab, H // 256, 144)[token][None])[0]
+        delta = None
+        for l in range(s.n_layers):
+            h, x2 = o.rmsnorm(x[None], self.w[f"{l}.attn_norm"], s.rms_eps, delta=None if delta is None else delta[None])
+            x = x2[0]
+            qkv = np.concatenate([self.gemv(f"{l}.wq", FMT_Q4_K, H, h[0]), self.gemv(f"{l}.wk", FMT_Q4_K, H, h[0]),
+                                  self.gemv(f"{l}.wv", FMT_Q6_K, H, h[0])])
+            qkv = o.rope_kv_append(qkv, self.inv_freq, pos, kcache[l], vcache[l], s.n_heads, s.n_kv, hd)
+            a = o.attention_decode(qkv[:qd], kcache[l], vcache[l], pos, s.n_heads, s.n_kv, hd)
+            delta = self.gemv(f"{l}.wo", FMT_Q4_K, qd, a)
+            h2, x2 = o.rmsnorm(x[None], self.w[f"{l}.ffn_norm"], s.rms_eps, delta=delta[None])
+            x = x2[0]
+            g = self.gemv(f"{l}.wgate", FMT_Q4_K, H, h2[0])
+            u = self.gemv(f"{l}.wup", FMT_Q4_K, H, h2[0])
+            delta = self.gemv(f"{l}.wdown", FMT_Q6_K, s.ffn, o.swiglu(g, u))
+        hf, _ = o.rmsnorm(x[None], self.w["final_norm"], s.rms_eps, delta=delta[None])
+        logits = self.gemv("lm_head", FMT_Q6_K, H, hf[0])
+        return logits
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
+    import torch
+
+    from llaminar_amd.decoder import DenseDecoder, Shape
+
+    shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
+    cap, start = 192, 130   # the newest position lies in the second 128-position chunk
+    # block scales large enough that activations stay O(1) through the layers
+    dec = DenseDecoder(shape, batch, cap, dev, seed=5, keep_raw=True, d_lo=0.002, d_hi=0.004)
+    ref = NumpyDecoder(oracle, shape, dec.raw, cap)
+    rng = np.random.default_rng(1)
+    ids = rng.integers(0, shape.vocab, batch).astype(np.int32)
+    pos = (start + np.arange(batch)).astype(np.int32)   # sequences at different positions
+    kc_h = np.zeros((batch, shape.n_layers, shape.n_kv, cap, 128), np.float16)
+    vc_h = np.zeros_like(kc_h)
+    for b in range(batch):
+        kc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
+        vc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
+    for l in range(shape.n_layers):
+        dec.buffer("kcache", l).copy_(torch.from_numpy(kc_h[:, l]).to(dev))
+        dec.buffer("vcache", l).copy_(torch.from_numpy(vc_h[:, l]).to(dev))
+    dec.set_state(ids, pos)
+    kc_u, vc_u = kc_h.view(np.uint16).copy(), vc_h.view(np.uint16).copy()
+
+    for step in range(3):
+        dec.step()
+        sync()
+        logits = dec.buffer("logits").cpu().numpy()
+        new_ids = dec.buffer("ids").cpu().numpy()
+        assert dec.buffer("pos").cpu().tolist() == [int(p) + step + 1 for p in pos]
+        assert np.isfinite(logits).all()
+        for b in range(batch):
+            exp = ref.step(int(ids[b]), int(pos[b]) + step, kc_u[b], vc_u[b])
+            scale = np.abs(exp).max()
+            err = np.abs(logits[b] - exp).max()
+            assert err <= 5e-3 * scale, (step, b, err, scale)
+            assert new_ids[b] == int(np.argmax(logits[b]))           # the sampler on the device's own logits
+            top2 = np.sort(exp)[-2:]
+            if top2[1] - top2[0] > 2 * 5e-3 * scale:
+                assert new_ids[b] == int(np.argmax(exp)), (step, b)
+            # the appended K/V rows: fp16 of nearly equal fp32 values
+            for l in range(shape.n_layers):
+                kg = dec.buffer("kcache", l)[b, :, int(pos[b]) + step].cpu().numpy().astype(np.float32)
+                ke = kc_u[b, l, :, int(pos[b]) + step].view(np.float16).astype(np.float32)
+                assert np.abs(kg - ke).max() <= 2e-2 * max(np.abs(ke).max(), 1.0), (step, b, l)
+        ids = new_ids.copy()   # both sides continue from the device's tokens
+    dec.close()
+
+
+def test_step_replays_as_a_graph(capi, dev):
+    """A captured step replayed three times gives the tokens of three eager steps."""
+    import torch
+
+    from llaminar_amd.decoder import DenseDecoder, Shape
+
+    shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
+    dec = DenseDecoder(shape, 2, 160, dev, seed=6, d_lo=0.002, d_hi=0.004)
+    ids0, pos0 = np.array([7, 1999], np.int32), np.array([0, 0], np.int32)
+
+    def run(n, graph):
+        for l in range(shape.n_layers):
+            dec.buffer("kcache", l).zero_()
+            dec.buffer("vcache", l).zero_()
+        dec.set_state(ids0, pos0)
+        toks, lg = [], []
+        for _ in range(n):
+            if graph is None:
+                dec.step()
+            else:
+                graph.replay()
+            torch.cuda.synchronize()
+            toks.append(dec.buffer("ids").cpu().tolist())
+            lg.append(dec.buffer("logits").clone())
+            # unrelated eager work between replays
+            torch.ones(1000, device=dev).sum().item()
+        return toks, lg
+
+    eager_t, eager_l = run(4, None)
+    stream = torch.cuda.Stream()
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        dec.step(stream)          # warm-up on the capture stream
+        stream.synchronize()
+        with torch.cuda.graph(gr, stream=stream):
+            dec.step(stream)
+    graph_t, graph_l = run(4, gr)
+    assert graph_t == eager_t
+    for a, b in zip(eager_l, graph_l):
+        assert torch.equal(a, b)
+    dec.close()
+
+
+def test_bad_configurations_are_refused(capi, dev):
+    from llaminar_amd import decoder
+
+    L = decoder.load()
+    bad = decoder.Config(5000, 64, 8, 128, 25600, 1000, 1, 16, 1, 1e6, 1e-6, 0)  # hidden not a multiple of 256
+    assert not L.llam_decoder_create(bad)
+    assert b"multiples of 256" in L.llam_decoder_last_error()
+    bad = decoder.Config(512, 6, 4, 128, 512, 1000, 1, 16, 1, 1e6, 1e-6, 0)       # 6 heads on 4 KV heads
+    assert not L.llam_decoder_create(bad)
+    ok = decoder.Config(512, 4, 4, 128, 512, 1000, 1, 16, 9, 1e6, 1e-6, 0)        # batch 9
+    assert not L.llam_decoder_create(ok)
+    h = L.llam_decoder_create(decoder.Config(512, 4, 4, 128, 512, 1000, 1, 16, 1, 1e6, 1e-6, 0))
+    assert h
+    assert not L.llam_decoder_step(h, None) and b"globals not set" in L.llam_decoder_last_error()
+    L.llam_decoder_destroy(h)
