@@ -175,7 +175,118 @@ def bench_gemv(args, torch, capi, synth, dev):
                     "us_per_launch": head["us"], "launches_timed": args.steps})
 
 
-OTHER_WORKLOADS = {"gemm": bench_gemm, "moe": bench_moe, "gemv": bench_gemv}
+def bench_decode(args, torch, capi, synth, dev):
+    """End-to-end greedy decode step of the random-init 64-layer dense model (the layer
+    workload's shapes, RMSNorm, RoPE, GQA attention over an fp16 KV cache at context 4096,
+    Q6_K lm_head 5120 -> 152064): tokens per second, with the share of the step that the
+    quantized-linear launches take when they run alone."""
+    from llaminar_amd.capi import FMT_Q4_K, FMT_Q6_K
+    from llaminar_amd.decoder import DenseDecoder, Shape
+
+    B = args.batch
+    shape = Shape(n_layers=args.decode_layers)
+    ctx = args.context
+    cap = ctx + args.steps + args.warmup + 8
+    t_build = time.perf_counter()
+    dec = DenseDecoder(shape, B, cap, dev, seed=11, keep_prepared=True)
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    for l in range(shape.n_layers):   # a cache as `ctx - 1` earlier tokens would have left it
+        for name in ("kcache", "vcache"):
+            buf = dec.buffer(name, l)
+            buf[:, :, : ctx - 1].copy_(torch.randn(B, shape.n_kv, ctx - 1, shape.head_dim, device=dev, generator=g))
+    ids0 = torch.randint(0, shape.vocab, (B,), generator=torch.Generator().manual_seed(5)).numpy()
+    dec.set_state(ids0, [ctx - 1] * B)
+    torch.cuda.synchronize()
+    t_build = time.perf_counter() - t_build
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        dec.step(stream)
+        stream.synchronize()
+        graph = None
+        if not args.no_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                dec.step(stream)
+        run = (lambda: graph.replay()) if graph is not None else (lambda: dec.step(stream))
+        for _ in range(max(args.warmup - 1, 1)):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ms = (t1 - t0) * 1e3 / args.steps
+        tokens = dec.buffer("ids").cpu().tolist()
+        last_pos = dec.buffer("pos").cpu().tolist()
+
+        # the quantized-linear launches of the same step alone (quantisers, GEMVs, lm_head)
+        H, QD, KV, F = shape.hidden, shape.n_heads * shape.head_dim, shape.n_kv * shape.head_dim, shape.ffn
+        x = torch.randn(B, H, device=dev)
+        attn = torch.randn(B, QD, device=dev)
+        q8 = torch.empty(B * (max(H, QD) // 32) * 36, dtype=torch.uint8, device=dev)
+        q8a = torch.empty(B * (F // 32) * 36, dtype=torch.uint8, device=dev)
+        qkv = torch.empty(B, QD + 2 * KV, device=dev)
+        o = torch.empty(B, H, device=dev)
+        gate = torch.randn(B, F, device=dev)
+        up = torch.randn(B, F, device=dev)
+        logits = torch.empty(B, shape.vocab, device=dev)
+        W = dec.prepared
+
+        def linear_only():
+            for l in range(shape.n_layers):
+                capi.quantize_q8_1(x, out=q8)
+                capi.gemv_fused([(FMT_Q4_K, W[f"{l}.wq"], qkv[:, :QD]), (FMT_Q4_K, W[f"{l}.wk"], qkv[:, QD:QD + KV]),
+                                 (FMT_Q6_K, W[f"{l}.wv"], qkv[:, QD + KV:])], q8, B, H)
+                capi.gemv_f32(FMT_Q4_K, W[f"{l}.wo"], attn, B, H, QD, out=o, q8_scratch=q8)
+                capi.quantize_q8_1(x, out=q8)
+                capi.gemv_fused([(FMT_Q4_K, W[f"{l}.wgate"], gate), (FMT_Q4_K, W[f"{l}.wup"], up)], q8, B, H)
+                capi.gemv_swiglu_f32(FMT_Q6_K, W[f"{l}.wdown"], gate, up, B, H, F, out=o, q8_scratch=q8a)
+            capi.quantize_q8_1(x, out=q8)
+            capi.gemv(FMT_Q6_K, W["lm_head"], q8, B, shape.vocab, H, out=logits)
+
+        linear_only()
+        stream.synchronize()
+        lin = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(lin, stream=stream):
+            linear_only()
+        for _ in range(3):
+            lin.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        reps = max(5, args.steps // 4)
+        for _ in range(reps):
+            lin.replay()
+        torch.cuda.synchronize()
+        ms_lin = (time.perf_counter() - t0) * 1e3 / reps
+
+    wbytes = shape.weight_bytes_per_token()
+    kv_bytes = shape.n_layers * B * 2 * shape.n_kv * ctx * shape.head_dim * 2
+    achieved = (wbytes + kv_bytes) / (ms * 1e-3) / 1e9
+    value = B * 1e3 / ms
+    cfg = {"workload": "end-to-end greedy decode step, random-init %d-layer dense model (hidden 5120, 64x128 heads, "
+                       "8 KV heads, ffn 25600; Q4_K projections, Q6_K V/down/lm_head 5120->152064, Q4_K embedding), "
+                       "RMSNorm, RoPE theta 1e6, fp16 KV cache at context %d, batch %d" % (shape.n_layers, ctx, B),
+           "batch": B, "context": ctx, "layers": shape.n_layers,
+           "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kv_bytes,
+           "linear_only_ms": round(ms_lin, 4), "gemv_share_of_step": round(ms_lin / ms, 4),
+           "hbm_bound_tokens_per_s": round(B * HBM_PEAK_GBS * 1e9 / (wbytes + kv_bytes), 1),
+           "launch": "eager" if graph is None else "hip-graph replay of the whole step",
+           "build_seconds": round(t_build, 1), "device_bytes_buffers": dec.device_bytes(),
+           "last_tokens": tokens, "last_positions": last_pos}
+    roof = {"kernel": "whole decode step (weights of every projection and the KV cache read once)", "bound": "hbm",
+            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "bytes_per_launch": wbytes + kv_bytes, "us_per_launch": round(ms * 1e3, 1), "launches_timed": args.steps}
+    out = _common(args, "decode tokens/s (greedy, batch %d)" % B, round(value, 2), "tokens/s", round(ms, 4), "int8",
+                  cfg, roof)
+    dec.close()
+    return out
+
+
+OTHER_WORKLOADS = {"gemm": bench_gemm, "moe": bench_moe, "gemv": bench_gemv, "decode": bench_decode}
 
 
 def parse():
@@ -183,12 +294,14 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["layer", "gemm", "moe", "gemv"], default="layer",
+    ap.add_argument("--workload", choices=["layer", "gemm", "moe", "gemv", "decode"], default="layer",
                     help="layer: the headline decode-layer step (default); gemm: prefill int8 GEMM 512x25600x5120 Q4_K; "
                          "moe: 256-expert top-8 IQ3_S expert FFN decode; gemv: single GEMVs of every format and layer shape")
     ap.add_argument("--batch", type=int, default=1, help="activation rows / tokens per step")
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    ap.add_argument("--context", type=int, default=4096, help="decode workload: tokens in the KV cache")
+    ap.add_argument("--decode-layers", type=int, default=64, help="decode workload: layers of the model")
     ap.add_argument("--separate-quantise", action="store_true",
                     help="layer workload: quantiser kernels of their own instead of the fp32-input GEMV calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")

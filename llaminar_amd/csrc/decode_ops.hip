@@ -164,10 +164,10 @@ namespace llamql
     constexpr int ATT_CHUNK = 128;
     constexpr int ATT_THREADS = 256;
     constexpr int ATT_HD = 128;
+    constexpr int ATT_ROWS = (ATT_THREADS / WAVE) * 4; // position rows in flight per workgroup
 
-    __device__ __forceinline__ void load_row8(const __half *p, float (&v)[8])
+    __device__ __forceinline__ void unpack_row8(const uint4 &raw, float (&v)[8])
     {
-        const uint4 raw = *reinterpret_cast<const uint4 *>(p);
         const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -185,8 +185,10 @@ namespace llamql
                                  float *__restrict__ part_o, float *__restrict__ part_ml, int n_heads, int n_kv,
                                  int ctx_cap, int n_chunks)
     {
-        __shared__ float s_sc[ATT_CHUNK][G];
-        __shared__ float s_o[ATT_THREADS / WAVE][G][ATT_HD];
+        // scores [ATT_CHUNK][G], then the partial output rows [ATT_ROWS][G][ATT_HD]
+        extern __shared__ __attribute__((aligned(16))) float att_lds[];
+        float(*s_sc)[G] = reinterpret_cast<float(*)[G]>(att_lds);
+        float(*s_o)[G][ATT_HD] = reinterpret_cast<float(*)[G][ATT_HD]>(att_lds + ATT_CHUNK * G);
         const int chunk = blockIdx.x, kh = blockIdx.y, b = blockIdx.z;
         const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
         const int col = (lane & 15) * 8, prow = lane >> 4;
@@ -194,15 +196,7 @@ namespace llamql
         const int p0 = chunk * ATT_CHUNK;
         const size_t out_base = ((size_t)b * n_heads + (size_t)kh * G) * n_chunks + chunk;
         if (p0 > last)
-        {
-            // nothing to attend to in this chunk: weight zero in the merge
-            if (threadIdx.x < G)
-            {
-                part_ml[(out_base + (size_t)threadIdx.x * n_chunks) * 2 + 0] = -INFINITY;
-                part_ml[(out_base + (size_t)threadIdx.x * n_chunks) * 2 + 1] = 0.0f;
-            }
-            return;
-        }
+            return; // no position in this chunk yet: the merge does not read it
         const __half *kbase = kcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
         const __half *vbase = vcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
 
@@ -218,16 +212,34 @@ namespace llamql
             qv[g][4] = c.x * scale, qv[g][5] = c.y * scale, qv[g][6] = c.z * scale, qv[g][7] = c.w * scale;
         }
 
-        // pass 1
+        // Every row this wavefront will need, K and V, is requested before the first use:
+        // one round trip to memory instead of one per pass over four positions.
         constexpr int PER_WAVE = ATT_CHUNK / (ATT_THREADS / WAVE); // positions per wavefront
-#pragma unroll 2
-        for (int it = 0; it < PER_WAVE / 4; ++it)
+        constexpr int ITERS = PER_WAVE / 4;
+        uint4 kraw[ITERS], vraw[ITERS];
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+        {
+            const int p = p0 + wave * PER_WAVE + it * 4 + prow;
+            const size_t at = (size_t)(p <= last ? p : last) * ATT_HD + col; // rows past the end: weight 0
+            kraw[it] = *reinterpret_cast<const uint4 *>(kbase + at);
+        }
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+        {
+            const int p = p0 + wave * PER_WAVE + it * 4 + prow;
+            const size_t at = (size_t)(p <= last ? p : last) * ATT_HD + col;
+            vraw[it] = *reinterpret_cast<const uint4 *>(vbase + at);
+        }
+
+        // pass 1
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
         {
             const int pl = wave * PER_WAVE + it * 4 + prow;
-            const int p = p0 + pl;
-            const bool valid = p <= last;
+            const bool valid = p0 + pl <= last;
             float kv[8];
-            load_row8(kbase + (size_t)(valid ? p : last) * ATT_HD + col, kv);
+            unpack_row8(kraw[it], kv);
             float s[G];
 #pragma unroll
             for (int g = 0; g < G; ++g)
@@ -281,13 +293,12 @@ namespace llamql
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 o[g][j] = 0.0f;
-#pragma unroll 2
-        for (int it = 0; it < PER_WAVE / 4; ++it)
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
         {
             const int pl = wave * PER_WAVE + it * 4 + prow;
-            const int p = p0 + pl;
             float vv[8];
-            load_row8(vbase + (size_t)(p <= last ? p : last) * ATT_HD + col, vv); // weight 0 past the end
+            unpack_row8(vraw[it], vv);
 #pragma unroll
             for (int g = 0; g < G; ++g)
             {
@@ -297,57 +308,94 @@ namespace llamql
                     o[g][j] = fmaf(w, vv[j], o[g][j]);
             }
         }
-        // the four position rows of a wavefront, then the wavefronts
+        // the sixteen partial rows of the workgroup (four position rows in each of four
+        // wavefronts) meet in LDS; thread t then sums four columns of one head
 #pragma unroll
         for (int g = 0; g < G; ++g)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-            {
-                float a = o[g][j];
-                a += __shfl_xor(a, 16, WAVE);
-                a += __shfl_xor(a, 32, WAVE);
-                o[g][j] = a;
-            }
-        if (prow == 0)
         {
-#pragma unroll
-            for (int g = 0; g < G; ++g)
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    s_o[wave][g][col + j] = o[g][j];
+            float4 *dst = reinterpret_cast<float4 *>(&s_o[wave * 4 + prow][g][col]);
+            dst[0] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
+            dst[1] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
         }
         __syncthreads();
-        for (int i = threadIdx.x; i < G * ATT_HD; i += ATT_THREADS)
+        for (int i = threadIdx.x; i < G * (ATT_HD / 4); i += ATT_THREADS)
         {
-            const int g = i / ATT_HD, c = i % ATT_HD;
-            float a = 0.0f;
+            const int g = i / (ATT_HD / 4), c4 = (i % (ATT_HD / 4)) * 4;
+            float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
-            for (int w = 0; w < ATT_THREADS / WAVE; ++w)
-                a += s_o[w][g][c];
-            part_o[(out_base + (size_t)g * n_chunks) * ATT_HD + c] = a;
+            for (int r = 0; r < ATT_ROWS; ++r)
+            {
+                const float4 v = *reinterpret_cast<const float4 *>(&s_o[r][g][c4]);
+                a.x += v.x, a.y += v.y, a.z += v.z, a.w += v.w;
+            }
+            *reinterpret_cast<float4 *>(part_o + (out_base + (size_t)g * n_chunks) * ATT_HD + c4) = a;
         }
     }
 
-    // One workgroup of 128 threads per (sequence, head).
+    template <int G>
+    void attention_partial_launch(dim3 grid, hipStream_t st, const float *q, int ld_q, const __half *kc,
+                                  const __half *vc, const int32_t *pos, float *part_o, float *part_ml, int n_heads,
+                                  int n_kv, int ctx_cap, int n_chunks)
+    {
+        constexpr size_t lds = (size_t)(ATT_CHUNK * G + ATT_ROWS * G * ATT_HD) * sizeof(float);
+        static bool attr_set = false;
+        if (!attr_set && lds > 64 * 1024)
+        {
+            // dynamic LDS beyond 64 KiB has to be allowed per kernel once
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attention_partial_kernel<G>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(attention_partial_kernel<G>, grid, dim3(ATT_THREADS), lds, st, q, ld_q, kc, vc, pos, part_o,
+                           part_ml, n_heads, n_kv, ctx_cap, n_chunks);
+    }
+
+    // One workgroup of 128 threads per (sequence, head): thread k weighs chunk k, then thread c
+    // sums column c over the chunks that hold positions.
+    constexpr int ATT_MAX_CHUNKS = 1024; // 131072 cache positions
+
     __global__ void __launch_bounds__(ATT_HD)
         attention_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml,
-                               float *__restrict__ out, int ld_out, int n_heads, int n_chunks)
+                               const int32_t *__restrict__ pos, float *__restrict__ out, int ld_out, int n_heads,
+                               int n_chunks, int ctx_cap)
     {
+        __shared__ float s_w[ATT_MAX_CHUNKS];
+        __shared__ float s_red[ATT_HD / WAVE];
         const int h = blockIdx.x, b = blockIdx.y, c = threadIdx.x;
+        const int last = pos[b] < ctx_cap - 1 ? pos[b] : ctx_cap - 1;
+        const int used = last < 0 ? 0 : last / ATT_CHUNK + 1; // chunks that were written
         const size_t base = ((size_t)b * n_heads + h) * n_chunks;
-        float M = -INFINITY;
-        for (int k = 0; k < n_chunks; ++k)
-            M = fmaxf(M, part_ml[(base + k) * 2]);
-        float L = 0.0f, acc = 0.0f;
-        for (int k = 0; k < n_chunks; ++k)
+
+        float mx = -INFINITY;
+        for (int k = c; k < used; k += ATT_HD)
+            mx = fmaxf(mx, part_ml[(base + k) * 2]);
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1)
+            mx = fmaxf(mx, __shfl_xor(mx, off, WAVE));
+        if ((c & (WAVE - 1)) == 0)
+            s_red[c >> 6] = mx;
+        __syncthreads();
+        const float M = fmaxf(s_red[0], s_red[1]);
+        __syncthreads();
+        float l = 0.0f;
+        for (int k = c; k < used; k += ATT_HD)
         {
-            const float mk = part_ml[(base + k) * 2];
-            if (mk == -INFINITY)
-                continue; // chunk past the newest position: its partial row was not written
-            const float w = expf(mk - M);
-            L = fmaf(part_ml[(base + k) * 2 + 1], w, L);
-            acc = fmaf(part_o[(base + k) * ATT_HD + c], w, acc);
+            const float w = expf(part_ml[(base + k) * 2] - M);
+            s_w[k] = w;
+            l = fmaf(part_ml[(base + k) * 2 + 1], w, l);
         }
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1)
+            l += __shfl_xor(l, off, WAVE);
+        if ((c & (WAVE - 1)) == 0)
+            s_red[c >> 6] = l;
+        __syncthreads();
+        const float L = s_red[0] + s_red[1];
+
+        float acc = 0.0f;
+#pragma unroll 4
+        for (int k = 0; k < used; ++k)
+            acc = fmaf(part_o[(base + k) * ATT_HD + c], s_w[k], acc);
         out[(size_t)b * ld_out + (size_t)h * ATT_HD + c] = L > 0.0f ? __fdiv_rn(acc, L) : 0.0f; // pos < 0: nothing attended
     }
 
@@ -563,11 +611,11 @@ extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kca
     if (!d_q || !d_kcache || !d_vcache || !d_pos || !d_out || !d_scratch)
         return fail(fn, "null pointer");
     if (!aligned16(d_q) || (ld_q % 4) != 0 || !aligned16(d_kcache) || !aligned16(d_vcache) || !aligned4(d_out) ||
-        !aligned4(d_scratch))
-        return fail(fn, "misaligned pointer");
+        !aligned16(d_scratch))
+        return fail(fn, "misaligned pointer (q, caches and scratch 16-byte, out 4-byte)");
     const int n_chunks = (ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
-    if ((long)n_chunks > 65535 || B > 65535)
-        return fail(fn, "too many chunks or sequences");
+    if (n_chunks > ATT_MAX_CHUNKS || B > 65535)
+        return fail(fn, "ctx_cap=%d beyond %d positions, or too many sequences", ctx_cap, ATT_MAX_CHUNKS * ATT_CHUNK);
     if (!set_device(fn, device_id))
         return false;
     float *part_o = d_scratch;
@@ -578,27 +626,15 @@ extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kca
     hipStream_t st = as_stream(stream);
     switch (G)
     {
-    case 1:
-        hipLaunchKernelGGL(attention_partial_kernel<1>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
-                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
-        break;
-    case 2:
-        hipLaunchKernelGGL(attention_partial_kernel<2>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
-                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
-        break;
-    case 4:
-        hipLaunchKernelGGL(attention_partial_kernel<4>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
-                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
-        break;
-    default:
-        hipLaunchKernelGGL(attention_partial_kernel<8>, grid, dim3(ATT_THREADS), 0, st, d_q, ld_q, kc, vc, d_pos,
-                           part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
-        break;
+    case 1: attention_partial_launch<1>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
+    case 2: attention_partial_launch<2>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
+    case 4: attention_partial_launch<4>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
+    default: attention_partial_launch<8>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
     }
     if (!launched(fn))
         return false;
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(n_heads, B), dim3(ATT_HD), 0, st, part_o, part_ml, d_out,
-                       ld_out, n_heads, n_chunks);
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(n_heads, B), dim3(ATT_HD), 0, st, part_o, part_ml, d_pos, d_out,
+                       ld_out, n_heads, n_chunks, ctx_cap);
     return launched(fn);
 }
 

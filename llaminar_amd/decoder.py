@@ -87,11 +87,11 @@ class Shape:
 
 class DenseDecoder:
     """Random-init model of the given shape: Q4_K/Q6_K projections, Q4_K embedding, Q6_K lm_head,
-    norm weights ~U(0.5,1.5).  Weights are generated on the device, seeded; `raw` keeps the GGUF
+    norm weights ~U(0.5,1.5) * norm_scale.  Weights are generated on the device, seeded; `raw` keeps the GGUF
     bytes (device tensors) when keep_raw is set, for the CPU check."""
 
     def __init__(self, shape: Shape, batch: int, ctx_cap: int, device, seed: int = 0, keep_raw: bool = False,
-                 d_lo: float = 0.001, d_hi: float = 0.02):
+                 d_lo: float = 0.001, d_hi: float = 0.02, keep_prepared: bool = False, norm_scale: float | None = None):
         import torch
 
         self.shape, self.batch, self.ctx_cap, self.device = shape, batch, ctx_cap, device
@@ -103,11 +103,19 @@ class DenseDecoder:
             raise capi.QLError(self.L.llam_decoder_last_error().decode())
         self.keep = []   # device tensors the handle borrows
         self.raw = {} if keep_raw else None
+        self.prepared = {} if keep_prepared else None   # name -> prepared weight tensor
         g = torch.Generator(device=device)
         g.manual_seed(seed)
 
+        # Random block fields give weights of mean ~2 and spread ~2.8 (at d ~ U(0.001, 0.02)), so a
+        # projection multiplies the norm of its input by about 2.8 sqrt(K).  Norm weights of
+        # that inverse size keep q, k, v and the feed-forward activations O(1): inside fp16
+        # range for the KV cache and away from SwiGLU's flat tail.
+        if norm_scale is None:
+            norm_scale = 1.0 / (2.8 * shape.hidden ** 0.5)
+
         def norm_weight(name):
-            t = torch.rand(shape.hidden, device=device, generator=g) + 0.5
+            t = (torch.rand(shape.hidden, device=device, generator=g) + 0.5) * norm_scale
             self.keep.append(t)
             if keep_raw:
                 self.raw[name] = t
@@ -119,6 +127,8 @@ class DenseDecoder:
             self.keep.append(w)
             if keep_raw:
                 self.raw[name] = raw
+            if keep_prepared:
+                self.prepared[name] = w
             return w.data_ptr()
 
         for l in range(shape.n_layers):

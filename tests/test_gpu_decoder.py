@@ -60,7 +60,7 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
     shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
     cap, start = 192, 130   # the newest position lies in the second 128-position chunk
     # block scales large enough that activations stay O(1) through the layers
-    dec = DenseDecoder(shape, batch, cap, dev, seed=5, keep_raw=True, d_lo=0.002, d_hi=0.004)
+    dec = DenseDecoder(shape, batch, cap, dev, seed=5, keep_raw=True, d_lo=0.002, d_hi=0.004, norm_scale=1.0)
     ref = NumpyDecoder(oracle, shape, dec.raw, cap)
     rng = np.random.default_rng(1)
     ids = rng.integers(0, shape.vocab, batch).astype(np.int32)
@@ -108,7 +108,7 @@ def test_step_replays_as_a_graph(capi, dev):
     from llaminar_amd.decoder import DenseDecoder, Shape
 
     shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
-    dec = DenseDecoder(shape, 2, 160, dev, seed=6, d_lo=0.002, d_hi=0.004)
+    dec = DenseDecoder(shape, 2, 160, dev, seed=6)
     ids0, pos0 = np.array([7, 1999], np.int32), np.array([0, 0], np.int32)
 
     def run(n, graph):
