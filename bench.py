@@ -32,9 +32,9 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# runs of this script (profiles/gemv_q4k_25600x5120_batch1_pmc.txt): (36156.2 KiB x 2.000 +
-# 109.9 KiB x 1.000), the factors being what the same counters read for a plain 256 MiB kernel.
-DOMINANT_TRAFFIC_BYTES = 74160435
+# runs of this script (profiles/gemv_q4k_25600x5120_batch1_pmc.txt): (36157.8 KiB x 2.000 +
+# 114.9 KiB x 1.000), the factors being what the same counters read for a plain 256 MiB kernel.
+DOMINANT_TRAFFIC_BYTES = 74168832
 
 HIDDEN, QDIM, KVDIM, FFN = 5120, 8192, 1024, 25600
 
@@ -305,6 +305,8 @@ def parse():
     ap.add_argument("--separate-quantise", action="store_true",
                     help="layer workload: quantiser kernels of their own instead of the fp32-input GEMV calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true",
+                    help="layer workload at batch 1: skip the short run of the 64-layer decode step")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 256 MiB read + 256 MiB write elementwise kernel a few times, so a rocprofv3 --pmc run of this "
                          "command records FETCH_SIZE / WRITE_SIZE for a kernel of known traffic")
@@ -501,7 +503,7 @@ def main():
             "launch": "eager" if graphs is None else "hip-graph replay",
         },
         "roofline": {
-            "kernel": "gemv_quad_kernel<Q4KQuad,1,3> N=25600 K=5120",
+            "kernel": "gemv_quad_kernel<Q4KQuad,1,3,0> N=25600 K=5120",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
@@ -514,6 +516,22 @@ def main():
         },
         "cpu_baseline": cpu,
     }
+    if M == 1 and not args.no_decode:
+        # the metric's second figure: tokens per second of the whole 64-layer decode step at
+        # batch 1 (the `decode` workload, a shorter run of it), reported beside the headline
+        del layers, graphs, group
+        torch.cuda.empty_cache()
+        try:
+            sub = argparse.Namespace(**vars(args))
+            sub.steps, sub.warmup = 24, 4
+            d = bench_decode(sub, torch, capi, synth, dev)
+            out["config"]["decode_step"] = {
+                "tokens_per_s": d["value"], "ms_per_token": d["ms_per_step"], "layers": d["config"]["layers"],
+                "context": d["config"]["context"], "gemv_share_of_step": d["config"]["gemv_share_of_step"],
+                "frac_of_hbm_bound": round(d["value"] / d["config"]["hbm_bound_tokens_per_s"], 4),
+                "steps": sub.steps, "workload": "bench.py --workload decode"}
+        except Exception as e:  # noqa: BLE001 - the headline figure must still be reported
+            out["config"]["decode_step"] = {"error": str(e)[:200]}
     print(json.dumps(out))
 
 
