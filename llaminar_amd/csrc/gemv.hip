@@ -30,10 +30,17 @@ namespace llamql
         int group_launch(const char *fn, const llam_ql_proj *projs, int num, const ActSource &src, int M, int K,
                          int device_id, hipStream_t st)
         {
+            // batches that go to the matrix-unit kernel launch one matrix at a time
+            if constexpr (F::USE_MFMA_BATCH)
+                if (mfma_eligible<F>(M, projs[0].N, K))
+                    return gemv_mfma_q4k_launch(fn, projs[0].d_w, src, projs[0].d_y, M, projs[0].N, K, projs[0].ldy,
+                                                device_id, st)
+                               ? 1
+                               : -1;
             QuadProj pr[QUAD_MAX_PROJ];
             int n = 0;
             while (n < num && n < QUAD_MAX_PROJ && projs[n].fmt == projs[0].fmt &&
-                   quad_eligible<F>(M, projs[n].N, K))
+                   quad_eligible<F>(M, projs[n].N, K) && !mfma_eligible<F>(M, projs[n].N, K))
             {
                 pr[n] = QuadProj{projs[n].d_w, projs[n].d_y, projs[n].N, projs[n].ldy};
                 ++n;

@@ -20,6 +20,7 @@
 
 #include "gemv_core.h"
 #include "gemv_quad.h"
+#include "gemv_mfma.h"
 
 namespace llamql
 {
@@ -325,6 +326,61 @@ namespace llamql
         else
             return false;
     }
+    // Batches of 5..8 rows on rows of 8..64 super-blocks (the activations of the whole batch
+    // must fit the 160 KiB of LDS) go to the matrix-unit kernel, in formats that have one.
+    template <class F>
+    bool mfma_eligible(int M, int N, int K)
+    {
+        if constexpr (F::USE_MFMA_BATCH)
+            return M >= 5 && N >= 1 && K / 256 >= 8 && mfma_lds_bytes(K / 256) <= QUAD_MAX_LDS &&
+                   gemv_unroll_override() == 0 && gemv_rows_per_wave_override() == 0;
+        else
+            return false;
+    }
+
+    template <int SRC>
+    void gemv_mfma_q4k_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const MfmaArgs &a)
+    {
+        static bool attr_set = false;
+        if (!attr_set)
+        {
+            // dynamic LDS beyond 64 KiB has to be allowed per kernel once
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<SRC>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(gemv_mfma_q4k_kernel<SRC>, grid, block, lds, st, a);
+    }
+
+    inline bool gemv_mfma_q4k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
+                                     int K, int ldy, int device_id, hipStream_t st)
+    {
+        const int SB = K / 256;
+        const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id));
+        MfmaArgs a;
+        a.w = static_cast<const uint8_t *>(d_w);
+        a.q8 = static_cast<const uint32_t *>(src.q8);
+        a.x = src.x;
+        a.x2 = src.x2;
+        a.ldx = src.ldx;
+        a.y = d_y;
+        a.ldy = ldy;
+        a.N = N;
+        a.SB = SB;
+        a.M = M;
+        a.sb_per_slice = sh.sb_per_slice;
+        a.slices = sh.slices;
+        const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles_per_wg) * WAVE);
+        const size_t lds = mfma_lds_bytes(SB);
+        switch (src.kind)
+        {
+        case ACT_SRC_F32: gemv_mfma_q4k_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;
+        case ACT_SRC_SWIGLU: gemv_mfma_q4k_launch_src<QUAD_SRC_SWIGLU>(grid, block, lds, st, a); break;
+        default: gemv_mfma_q4k_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a); break;
+        }
+        return launched(fn);
+    }
+
     static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU,
                   "activation source kinds");
 
@@ -387,6 +443,9 @@ namespace llamql
     {
         const int SB = K / 256;
         const bool dump = d_sums != nullptr;
+        if constexpr (F::USE_MFMA_BATCH)
+            if (!dump && mfma_eligible<F>(M, N, K))
+                return gemv_mfma_q4k_launch(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st);
         // Rows of at least 16 super-blocks in a format with a quad-lane decoder: the
         // quad kernel, which stages whole activation rows (up to 160 KiB of LDS).
         if constexpr (F::USE_QUAD)

@@ -1,0 +1,317 @@
+// Q4_K x Q8_1 decode GEMV for batches of 5..8 activation rows on the matrix unit.
+//
+// With several activation rows the quad-lane kernel pays 16 dot instructions and five
+// 128-bit LDS reads per 64 weights for EVERY row.  Here one v_mfma_i32_32x32x32_i8 per
+// 32-column block multiplies 32 weight rows with all activation rows at once:
+//   A operand = activations (rows m of the batch, padded to 32), lane (m = l%32, h = l/32)
+//               supplies bytes 16h..16h+15 of the block, read from LDS;
+//   B operand = weights, lane (r = l%32, h) supplies elements 16h..16h+15 of row r's block,
+//               straight from the registers the lane decoded them into: a 16-byte piece of
+//               a Q4_K group holds exactly those elements of block 2g (low nibbles) and of
+//               block 2g+1 (high nibbles);
+//   result    = the exact int32 block sums: lane (r, h) holds rows m = 4h..4h+3 of column r,
+//               i.e. the lane that decoded row r's scales also rescales row r's sums.
+// The accumulator is zero for every block, so the MFMA result is the reference's per-block
+// int32 sum, rescaled in fp32 block after block in ascending order.
+//
+// A workgroup owns 32 weight rows; its wavefronts split the row length into slices of whole
+// super-blocks (K = 5120: 4 slices of 5) so that the chip sees enough wavefronts, and their
+// partial sums are added in slice order at the end.
+#pragma once
+#include "gemv_core.h"
+#include "gemv_quad.h"
+
+namespace llamql
+{
+    constexpr int MFMA_TILE_ROWS = 32;
+    constexpr int MFMA_MAX_SLICES = 8;
+    constexpr int MFMA_LOADS = 5; // vector memory loads per super-block and lane
+
+    struct MfmaArgs
+    {
+        const uint8_t *w;   // Q4_K super-blocks, row-major
+        const uint32_t *q8; // Q8_1 activations as dwords (9 per block), M rows (QUAD_SRC_Q8)
+        const float *x;     // fp32 rows of ldx floats (QUAD_SRC_F32); the gate rows for QUAD_SRC_SWIGLU
+        const float *x2;    // the up rows for QUAD_SRC_SWIGLU
+        int ldx;
+        float *y;
+        int ldy;
+        int N;
+        int SB;           // super-blocks per weight row
+        int M;            // activation rows, 1..8
+        int sb_per_slice; // super-blocks one wavefront walks
+        int slices;       // wavefronts per 32-row tile; a workgroup holds blockDim/64/slices tiles
+    };
+
+    // LDS: per 32-column block 8 activation rows x 32 int8 (16 bytes of padding: neighbouring
+    // blocks start four banks apart, so the staging writes do not collide) and
+    // 2 x {d[4], sum*d[4]}
+    constexpr int MFMA_AQ_STRIDE = 256 + 16;
+    inline size_t mfma_lds_bytes(int nsb) { return (size_t)nsb * 8 * (MFMA_AQ_STRIDE + 64); }
+
+    struct MfmaRaw
+    {
+        v4i head, q0, q1, q2, q3;
+    };
+
+    __device__ __forceinline__ void mfma_load(MfmaRaw &r, const uint8_t *sb, const uint8_t *grp)
+    {
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.head) : "v"(sb));
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.q0) : "v"(grp));
+        asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=&v"(r.q1) : "v"(grp));
+        asm volatile("global_load_dwordx4 %0, %1, off offset:64" : "=&v"(r.q2) : "v"(grp));
+        asm volatile("global_load_dwordx4 %0, %1, off offset:96" : "=&v"(r.q3) : "v"(grp));
+    }
+    __device__ __forceinline__ void mfma_keep(MfmaRaw &r)
+    {
+        asm volatile("" : "+v"(r.head), "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3));
+    }
+    template <int NEWER>
+    __device__ __forceinline__ void mfma_wait(MfmaRaw &r)
+    {
+        asm volatile("s_waitcnt vmcnt(%5)"
+                     : "+v"(r.head), "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3)
+                     : "n"(NEWER));
+    }
+
+    // SRC: where the activations come from (QUAD_SRC_*): Q8_1 blocks, or fp32 rows quantised here.
+    template <int SRC>
+    __global__ void __launch_bounds__(MFMA_MAX_SLICES *WAVE) gemv_mfma_q4k_kernel(const MfmaArgs a)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];
+        const int nsb = a.SB;
+        const int nkb = nsb * 8;
+        uint8_t *aq = mfma_lds;                                                 // [kb][8 rows][32 B] (+16)
+        float *asc = reinterpret_cast<float *>(mfma_lds + nkb * MFMA_AQ_STRIDE); // [kb][2 halves][d x4, sum*d x4]
+
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int l32 = lane & 31, lh = lane >> 5;
+
+        // this wavefront's tile and slice of the row, and this lane's weight row
+        const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
+        const int tiles_per_wg = (int)(blockDim.x >> 6) / a.slices;
+        const int s0 = slice * a.sb_per_slice;
+        int s1 = s0 + a.sb_per_slice;
+        if (s1 > nsb)
+            s1 = nsb;
+        const int nsteps = s1 > s0 ? s1 - s0 : 0;
+        const long row = ((long)blockIdx.x * tiles_per_wg + tile_local) * MFMA_TILE_ROWS + l32;
+        const long row_ld = row < a.N ? row : a.N - 1; // rows past the end re-read the last one
+        const uint8_t *rowp = a.w + (size_t)row_ld * nsb * 144;
+        const int first_sb = nsteps > 0 ? s0 : 0;
+        const int last_sb = nsteps > 0 ? s1 - 1 : 0;
+
+        // loads are never predicated: past the end of the slice a lane re-reads its last block
+        auto issue = [&](MfmaRaw &r, int step) {
+            int sb = first_sb + step;
+            if (sb > last_sb)
+                sb = last_sb;
+            const uint8_t *p = rowp + (size_t)sb * 144;
+            mfma_load(r, p, p + 16 + 16 * lh);
+        };
+        MfmaRaw bufA, bufB;
+        issue(bufA, 0);
+        issue(bufB, 1);
+
+        // ---- activations into LDS ------------------------------------------------------------
+        if constexpr (SRC == QUAD_SRC_Q8)
+        {
+            // one thread per Q8_1 block, three blocks in flight per thread: the latency of a
+            // round trip is paid per batch of loads, not per block
+            constexpr int UN = 3;
+            const int total = a.M * nkb;
+            for (int i0 = threadIdx.x; i0 < total; i0 += UN * (int)blockDim.x)
+            {
+                uint32_t v[UN][9];
+#pragma unroll
+                for (int u = 0; u < UN; ++u)
+                {
+                    const int idx = min(i0 + u * (int)blockDim.x, total - 1);
+                    const uint32_t *src = a.q8 + (size_t)idx * 9;
+#pragma unroll
+                    for (int i = 0; i < 9; ++i)
+                        v[u][i] = src[i];
+                }
+#pragma unroll
+                for (int u = 0; u < UN; ++u)
+                {
+                    const int idx = i0 + u * (int)blockDim.x;
+                    if (idx < total)
+                    {
+                        const int m = idx / nkb, kb = idx - m * nkb;
+                        const float d = h2f((uint16_t)(v[u][0] & 0xFFFFu));
+                        uint4 *dst = reinterpret_cast<uint4 *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32);
+                        dst[0] = make_uint4(v[u][1], v[u][2], v[u][3], v[u][4]);
+                        dst[1] = make_uint4(v[u][5], v[u][6], v[u][7], v[u][8]);
+                        float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
+                        sc[0] = d;
+                        sc[4] = (float)(int16_t)(v[u][0] >> 16) * d;
+                    }
+                }
+            }
+        }
+        else
+        {
+            // eight neighbouring threads quantise one 32-element block (the stand-alone
+            // quantiser's arithmetic)
+            const int nvec = nkb * 8;
+            for (int m = 0; m < a.M; ++m)
+            {
+                const float4 *xr = reinterpret_cast<const float4 *>(a.x + (size_t)m * a.ldx);
+                const float4 *xr2 = reinterpret_cast<const float4 *>(a.x2 + (size_t)m * a.ldx);
+                for (int i = threadIdx.x; i < nvec; i += blockDim.x) // whole 8-thread groups stay together
+                {
+                    float4 v = xr[i];
+                    if constexpr (SRC == QUAD_SRC_SWIGLU)
+                        v = swiglu4(v, xr2[i]);
+                    const Q8Lane q = q8_1_quantize_lane(v);
+                    const int kb = i >> 3, sub = i & 7;
+                    *reinterpret_cast<uint32_t *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32 + sub * 4) = q.packed;
+                    if (sub == 0)
+                    {
+                        const float d = h2f((uint16_t)(q.head & 0xFFFFu));
+                        float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
+                        sc[0] = d;
+                        sc[4] = (float)(int16_t)(q.head >> 16) * d;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        mfma_keep(bufA); // the staging code must not reuse the registers of the loads in flight
+        mfma_keep(bufB);
+
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        v16i zero;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            zero[i] = 0;
+        const uint8_t *aq_lane = aq + (l32 & 7) * 32 + lh * 16; // rows beyond the batch: any row, result unused
+        const float *asc_lane = asc + lh * 8;
+        int step = 0;
+
+        auto compute = [&](const MfmaRaw &r) {
+            const int sb = first_sb + step;
+            Q4KQuad::Scale S[4];
+            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(0), S[0]);
+            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(1), S[1]);
+            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(2), S[2]);
+            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(3), S[3]);
+            const v4i q[4] = {r.q0, r.q1, r.q2, r.q3};
+            const uint8_t *ab = aq_lane + (size_t)sb * (8 * MFMA_AQ_STRIDE);
+            const float *sb_sc = asc_lane + (size_t)sb * (8 * 16);
+            const uint32_t k = 0x0F0F0F0Fu;
+            // block 2g+h of the super-block: h = 0 low nibbles, 1 high nibbles
+            auto product = [&](int j) {
+                const v4i x = q[j >> 1];
+                v4i w;
+                if (j & 1)
+                    w = (v4i){(int)(((uint32_t)x.x >> 4) & k), (int)(((uint32_t)x.y >> 4) & k),
+                              (int)(((uint32_t)x.z >> 4) & k), (int)(((uint32_t)x.w >> 4) & k)};
+                else
+                    w = (v4i){(int)((uint32_t)x.x & k), (int)((uint32_t)x.y & k), (int)((uint32_t)x.z & k),
+                              (int)((uint32_t)x.w & k)};
+                const v4i av = *reinterpret_cast<const v4i *>(ab + j * MFMA_AQ_STRIDE);
+                return __builtin_amdgcn_mfma_i32_32x32x32_i8(av, w, zero, 0, 0, 0);
+            };
+            // the product of block j+1 is issued before block j is rescaled: matrix unit and
+            // vector unit work side by side
+            v16i idot[2];
+            idot[0] = product(0);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+            {
+                if (j + 1 < 8)
+                    idot[(j + 1) & 1] = product(j + 1);
+                const float4 ad = *reinterpret_cast<const float4 *>(sb_sc + j * 16);
+                const float4 asd = *reinterpret_cast<const float4 *>(sb_sc + j * 16 + 4);
+                const float bs = Q4KQuad::scale_f32(S[j >> 1], j & 1);
+                const float bm = Q4KQuad::min_f32(S[j >> 1], j & 1);
+                const v16i d = idot[j & 1];
+                acc[0] = fmaf((float)d[0], ad.x * bs, acc[0]);
+                acc[0] = fmaf(asd.x, bm, acc[0]);
+                acc[1] = fmaf((float)d[1], ad.y * bs, acc[1]);
+                acc[1] = fmaf(asd.y, bm, acc[1]);
+                acc[2] = fmaf((float)d[2], ad.z * bs, acc[2]);
+                acc[2] = fmaf(asd.z, bm, acc[2]);
+                acc[3] = fmaf((float)d[3], ad.w * bs, acc[3]);
+                acc[3] = fmaf(asd.w, bm, acc[3]);
+            }
+            ++step;
+        };
+
+        // Two buffers alternate; each is reloaded (two steps ahead) once it has been consumed.
+        // Every buffer is waited for, also past the end of the slice: a register whose load is
+        // still in flight must not look free to the compiler.
+        for (int c0 = 0; c0 < nsteps; c0 += 2)
+        {
+            mfma_wait<MFMA_LOADS>(bufA);
+            if (step < nsteps) // uniform
+                compute(bufA);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufA, c0 + 2);
+            mfma_wait<MFMA_LOADS>(bufB);
+            if (step < nsteps)
+                compute(bufB);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufB, c0 + 3);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the slice
+        mfma_keep(bufA);
+        mfma_keep(bufB);
+
+        // ---- partial sums of the slices, added in slice order ---------------------------------
+        __syncthreads(); // every wavefront is done with the activations
+        float *red = reinterpret_cast<float *>(mfma_lds); // [wavefront][4][64]
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            red[(wave * 4 + i) * WAVE + lane] = acc[i];
+        __syncthreads();
+        if (slice == 0)
+        {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                float v = acc[i];
+                for (int s = 1; s < a.slices; ++s)
+                    v += red[((wave + s) * 4 + i) * WAVE + lane];
+                const int m = 4 * lh + i;
+                if (m < a.M && row < a.N)
+                    a.y[(size_t)m * a.ldy + row] = v;
+            }
+        }
+    }
+
+    struct MfmaShape
+    {
+        int slices, sb_per_slice, tiles_per_wg;
+        long grid;
+    };
+    // Slices so that a compute unit sees about a dozen wavefronts, each at least two
+    // super-blocks long; tiles per workgroup so that every workgroup of the launch is resident
+    // at once (a second round of workgroups would run nearly alone on the chip and cost a
+    // workgroup's whole latency again) and the activations are staged less often.
+    inline MfmaShape gemv_mfma_shape(long N, int nsb, int cus)
+    {
+        const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
+        long want = ((long)cus * 12 + tiles - 1) / tiles;
+        if (want > MFMA_MAX_SLICES)
+            want = MFMA_MAX_SLICES;
+        if (want > nsb / 2)
+            want = nsb / 2;
+        if (want < 1)
+            want = 1;
+        MfmaShape sh;
+        sh.sb_per_slice = (int)((nsb + want - 1) / want);
+        sh.slices = (nsb + sh.sb_per_slice - 1) / sh.sb_per_slice;
+        const long lds_wgs = (long)(QUAD_MAX_LDS / mfma_lds_bytes(nsb)); // workgroups the LDS of a CU holds
+        int t = 1;
+        while (t * 2 * sh.slices <= MFMA_MAX_SLICES && // wavefronts per workgroup
+               (tiles + t - 1) / t > (long)cus * (lds_wgs < 1 ? 1 : lds_wgs))
+            t *= 2;
+        sh.tiles_per_wg = t;
+        sh.grid = (tiles + t - 1) / t;
+        return sh;
+    }
+} // namespace llamql

@@ -267,19 +267,25 @@ namespace llamql
                          (int)(((uint32_t)r.qa.z >> 4) & k), (int)(((uint32_t)r.qa.w >> 4) & k)};
             w[3] = (v4i){(int)(((uint32_t)r.qb.x >> 4) & k), (int)(((uint32_t)r.qb.y >> 4) & k),
                          (int)(((uint32_t)r.qb.z >> 4) & k), (int)(((uint32_t)r.qb.w >> 4) & k)};
-            // 6-bit scales / mins of blocks j0 = 2l, j1 = 2l+1 as two 16-bit integers each
-            // (get_scale_min_k4: j<4: q[j]&63, q[j+4]&63; else (q[j+4]&15)|((q[j-4]>>6)<<4),
-            // (q[j+4]>>4)|((q[j]>>6)<<4) -- SIMDHelpers.h:10791-10803)
-            const uint32_t A = __builtin_amdgcn_perm(0u, (uint32_t)r.head.y, c.sel);
-            const uint32_t B = __builtin_amdgcn_perm(0u, (uint32_t)r.head.z, c.sel);
-            const uint32_t P = __builtin_amdgcn_perm(0u, (uint32_t)r.head.w, c.sel);
+            decode_scales(r.head, c, S);
+        }
+
+        // Effective scales and mins of blocks 2l, 2l+1 from the header piece: the 6-bit
+        // scales / mins as two 16-bit integers each
+        // (get_scale_min_k4: j<4: q[j]&63, q[j+4]&63; else (q[j+4]&15)|((q[j-4]>>6)<<4),
+        // (q[j+4]>>4)|((q[j]>>6)<<4) -- SIMDHelpers.h:10791-10803)
+        __device__ __forceinline__ static void decode_scales(const v4i &head, const Lane &c, Scale &S)
+        {
+            const uint32_t A = __builtin_amdgcn_perm(0u, (uint32_t)head.y, c.sel);
+            const uint32_t B = __builtin_amdgcn_perm(0u, (uint32_t)head.z, c.sel);
+            const uint32_t P = __builtin_amdgcn_perm(0u, (uint32_t)head.w, c.sel);
             const uint32_t bias = 0x64006400u; // fp16 1024.0: 0x6400|n is 1024+n
             const uint32_t sc = (P & c.m3) | (((A >> 2) & c.m2) | ((A & c.m1) | bias));
             const uint32_t mn = ((P >> 4) & c.m3) | (((B >> 2) & c.m2) | ((B & c.m1) | bias));
             const h2 k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
             const h2 scf = __builtin_bit_cast(h2, sc) - k1024;
             const h2 mnf = __builtin_bit_cast(h2, mn) - k1024;
-            const uint32_t hx = (uint32_t)r.head.x;
+            const uint32_t hx = (uint32_t)head.x;
             const h2 dd = __builtin_bit_cast(h2, hx); // {d, dmin}
             // d (11-bit significand) times a 6-bit integer is exact before rounding, so the
             // fp16 multiply equals f16(fp32 product) wherever the result is normal

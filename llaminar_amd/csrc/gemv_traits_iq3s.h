@@ -67,6 +67,7 @@ namespace llamql
         static constexpr bool PAIR = false;
         static constexpr bool HAS_MIN = false;
         static constexpr bool USE_QUAD = false;
+        static constexpr bool USE_MFMA_BATCH = false;  // matrix-unit kernel for 5..8 activation rows
         static constexpr int FAST_MAX_U = 3;          // load batches in flight in the chunked kernel
         static constexpr int TABLE_BYTES = (int)sizeof(IQ3STables);
 

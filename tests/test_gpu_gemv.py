@@ -282,7 +282,10 @@ def test_error_paths(capi, dev):
 def test_q4k_long_rows_all_batches(capi, dev, oracle, N, K):
     """Rows of 16 and more super-blocks take the kernel that walks a wavefront's rows as one
     run: row ends inside a step (K/256 not a multiple of 16), ragged last steps, wavefronts
-    without rows, every batch size; a batch row equals the single-row result bit for bit."""
+    without rows, every batch size; up to four rows (the decode-equivalent verifier rows of
+    the reference) a batch row equals the single-row result bit for bit.  Batches of 5..8 run
+    on the matrix unit, which adds a row's blocks in ascending order: same values up to the
+    association of the fp32 sum, and independent of what else is in the batch."""
     import torch
 
     fmt = FMT_Q4_K
@@ -297,7 +300,14 @@ def test_q4k_long_rows_all_batches(capi, dev, oracle, N, K):
         sync()
         assert rel_err(y.cpu().numpy(), C[:M]) <= TOL[fmt] * 1e-2, M
         for m in range(M):
-            assert torch.equal(y[m], y1[m][0]), (M, m)
+            if M <= 4:
+                assert torch.equal(y[m], y1[m][0]), (M, m)
+            else:
+                assert rel_err(y[m].cpu().numpy(), y1[m][0].cpu().numpy()) <= TOL[fmt] * 1e-2, (M, m)
+        if M == 5:
+            y5 = y.clone()
+        if M > 5:
+            assert torch.equal(y[:5], y5), M   # a row does not depend on the batch it rides in
     lib = capi.load()
     try:
         # another row partition moves rows to other lanes: same values up to summation order
