@@ -26,6 +26,22 @@ namespace llamql
 
     namespace
     {
+        // the other format with a quad-lane kernel
+        template <class F>
+        struct Other;
+        template <>
+        struct Other<Q4KTraits>
+        {
+            typedef Q6KTraits type;
+            static constexpr uint8_t fmt = LLAM_FMT_Q6_K;
+        };
+        template <>
+        struct Other<Q6KTraits>
+        {
+            typedef Q4KTraits type;
+            static constexpr uint8_t fmt = LLAM_FMT_Q4_K;
+        };
+
         template <class F>
         int group_launch(const char *fn, const llam_ql_proj *projs, int num, const ActSource &src, int M, int K,
                          int device_id, hipStream_t st)
@@ -45,6 +61,21 @@ namespace llamql
                 pr[n] = QuadProj{projs[n].d_w, projs[n].d_y, projs[n].N, projs[n].ldy};
                 ++n;
             }
+            // a following run in the other quad-lane format joins the launch (Q and K with V)
+            if constexpr (F::USE_QUAD)
+                if (n >= 1 && n < QUAD_MAX_PROJ && M <= 4 && src.kind != ACT_SRC_SWIGLU)
+                {
+                    typedef typename Other<F>::type G;
+                    int nb = 0;
+                    while (n + nb < num && n + nb < QUAD_MAX_PROJ && projs[n + nb].fmt == Other<F>::fmt &&
+                           quad_eligible<G>(M, projs[n + nb].N, K) && !mfma_eligible<G>(M, projs[n + nb].N, K))
+                    {
+                        pr[n + nb] = QuadProj{projs[n + nb].d_w, projs[n + nb].d_y, projs[n + nb].N, projs[n + nb].ldy};
+                        ++nb;
+                    }
+                    if (nb > 0)
+                        return gemv_quad_dual<F, G>(fn, pr, n, nb, src, M, K, device_id, st) ? n + nb : -1;
+                }
             // a single matrix on Q8_1 input goes through the general launcher
             if (n < (src.kind == ACT_SRC_Q8 ? 2 : 1))
                 return 0;

@@ -400,6 +400,7 @@ namespace llamql
             a.ldx = src.ldx;
             a.SB = SB;
             a.nproj = n;
+            a.first_b = n;
             long waves = 0;
             for (int i = 0; i < QUAD_MAX_PROJ; ++i)
             {
@@ -409,9 +410,9 @@ namespace llamql
                 a.N[i] = pr[j].N;
                 a.ldy[i] = pr[j].ldy;
                 a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves).rows_per_wave;
+                a.wave_begin[i] = (int)waves;
                 if (i < n)
                     waves += ((long)pr[j].N + a.R[i] - 1) / a.R[i];
-                a.wave_end[i] = (int)waves;
             }
             if (waves > 0x7FFFFFFFL / WAVE)
                 return fail(fn, "too many rows for one launch");
@@ -432,6 +433,71 @@ namespace llamql
         {
             (void)pr; (void)n; (void)src; (void)M; (void)K; (void)device_id; (void)st;
             return fail(fn, "format has no quad-lane kernel");
+        }
+    }
+
+    // The same over two runs of matrices in two formats (na of FA, then nb of FB; na + nb <=
+    // QUAD_MAX_PROJ), M <= 4, Q8_1 or plain fp32 activations.  The second format starts at a
+    // workgroup boundary.
+    template <class FA, class FB>
+    bool gemv_quad_dual(const char *fn, const QuadProj *pr, int na, int nb, const ActSource &src, int M, int K,
+                        int device_id, hipStream_t st)
+    {
+        if constexpr (FA::USE_QUAD && FB::USE_QUAD)
+        {
+            typedef typename FA::Quad QA;
+            typedef typename FB::Quad QB;
+            const int SB = K / 256;
+            const int cus = cu_count(device_id);
+            const int mta = QA::max_threads(M), mtb = QB::max_threads(M);
+            const int max_waves = (mta < mtb ? mta : mtb) / WAVE;
+            const int n = na + nb;
+            QuadArgs a;
+            a.q8 = static_cast<const uint32_t *>(src.q8);
+            a.x = src.x;
+            a.x2 = src.x2;
+            a.ldx = src.ldx;
+            a.SB = SB;
+            a.nproj = n;
+            a.first_b = na;
+            long cnt[QUAD_MAX_PROJ], waves = 0;
+            for (int i = 0; i < QUAD_MAX_PROJ; ++i)
+            {
+                const int j = i < n ? i : n - 1;
+                a.w[i] = pr[j].w;
+                a.y[i] = pr[j].y;
+                a.N[i] = pr[j].N;
+                a.ldy[i] = pr[j].ldy;
+                a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves).rows_per_wave;
+                cnt[i] = i < n ? ((long)pr[j].N + a.R[i] - 1) / a.R[i] : 0;
+                waves += cnt[i];
+            }
+            const long wpc = (waves + cus - 1) / cus;
+            const long wgs_per_cu = (wpc + max_waves - 1) / max_waves;
+            long nw = (wpc + wgs_per_cu - 1) / wgs_per_cu;
+            if (nw > waves)
+                nw = waves;
+            if (nw < 1)
+                nw = 1;
+            long at = 0;
+            for (int i = 0; i < QUAD_MAX_PROJ; ++i)
+            {
+                if (i == na)
+                    at = (at + nw - 1) / nw * nw; // the second format starts a workgroup
+                a.wave_begin[i] = (int)at;
+                at += cnt[i];
+            }
+            if (at > 0x7FFFFFFFL / WAVE)
+                return fail(fn, "too many rows for one launch");
+            const long grid = (at + nw - 1) / nw;
+            gemv_quad_dual_launch<QA, QB>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE),
+                                          quad_lds_bytes(M, SB), st, a);
+            return launched(fn);
+        }
+        else
+        {
+            (void)pr; (void)na; (void)nb; (void)src; (void)M; (void)K; (void)device_id; (void)st;
+            return fail(fn, "formats have no quad-lane kernel");
         }
     }
 

@@ -40,10 +40,12 @@ namespace llamql
     constexpr int QUAD_SRC_F32 = 1;    // fp32 rows
     constexpr int QUAD_SRC_SWIGLU = 2; // silu(gate) * up of two fp32 inputs
 
-    // One launch: up to QUAD_MAX_PROJ weight matrices of one format and row length against
-    // the same activations (projections that share an input: Q and K, gate and up).  The
-    // wavefronts of the launch are dealt to the matrices in order; wave_end[p] is the
-    // number of wavefronts up to and including matrix p.
+    // One launch: up to QUAD_MAX_PROJ weight matrices of one row length against the same
+    // activations (projections that share an input: Q, K and V; gate and up).  The
+    // wavefronts of the launch are dealt to the matrices in order: matrix p owns the
+    // wavefronts from wave_begin[p] on (those beyond its last row idle).  Matrices from
+    // first_b on are in the second format of a two-format launch and start at a workgroup
+    // boundary, because a workgroup stages the activations in its format's order.
     struct QuadArgs
     {
         const uint32_t *q8; // Q8_1 activations as dwords (9 per block), M rows (QUAD_SRC_Q8)
@@ -57,7 +59,8 @@ namespace llamql
         int N[QUAD_MAX_PROJ];
         int ldy[QUAD_MAX_PROJ];
         int R[QUAD_MAX_PROJ]; // rows per wavefront
-        int wave_end[QUAD_MAX_PROJ];
+        int wave_begin[QUAD_MAX_PROJ];
+        int first_b; // nproj in a launch of one format
     };
 
     // LDS bytes for M activation rows of nsb super-blocks.
@@ -561,10 +564,23 @@ namespace llamql
         }
     }
 
-    template <class Q, int M, int U, int SRC>
-    __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const QuadArgs qa)
+    // which matrix the wavefront works on, and the first wavefront of that matrix
+    __device__ __forceinline__ void quad_which(const QuadArgs &qa, int wid_all, int &p, int &w_first)
     {
-        extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
+        p = 0;
+        w_first = 0;
+#pragma unroll
+        for (int i = 1; i < QUAD_MAX_PROJ; ++i)
+            if (i < qa.nproj && wid_all >= qa.wave_begin[i])
+            {
+                p = i;
+                w_first = qa.wave_begin[i];
+            }
+    }
+
+    template <class Q, int M, int U, int SRC>
+    __device__ __forceinline__ void quad_body(const QuadArgs &qa, uint8_t *quad_lds, int p, int w_first, int wid_all)
+    {
         const int nsb = qa.SB;
         const int aq_stride = ((nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB) * 4096;
         const int ads_stride = nsb * 64;
@@ -572,22 +588,10 @@ namespace llamql
         uint8_t *ads = quad_lds + M * aq_stride;
 
         const int lane = threadIdx.x & (WAVE - 1);
-        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-        const int NW = (int)(blockDim.x >> 6);
         const int l = lane & 3;
         const int grp = lane >> 2;
         const typename Q::Lane lc = Q::lane_consts(l);
 
-        // which matrix this wavefront works on, and which of its wavefronts it is
-        const int wid_all = (int)blockIdx.x * NW + wave;
-        int p = 0, w_first = 0;
-#pragma unroll
-        for (int i = 0; i + 1 < QUAD_MAX_PROJ; ++i)
-            if (i + 1 < qa.nproj && wid_all >= qa.wave_end[i])
-            {
-                p = i + 1;
-                w_first = qa.wave_end[i];
-            }
         GemvArgs a; // the matrix, for the format's addressing
         a.w = qa.w[p];
         a.N = qa.N[p];
@@ -601,7 +605,7 @@ namespace llamql
         long r1 = r0 + R;
         if (r1 > a.N)
             r1 = a.N;
-        const int total = (r1 > r0 && wid_all < qa.wave_end[p]) ? (int)(r1 - r0) * nsb : 0;
+        const int total = r1 > r0 ? (int)(r1 - r0) * nsb : 0; // wavefronts past the last row idle
         const int nsteps = (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
 
         const size_t t0 = (size_t)(total > 0 ? r0 : 0) * nsb + grp;
@@ -715,6 +719,34 @@ namespace llamql
     }
 
     template <class Q, int M, int U, int SRC>
+    __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const QuadArgs qa)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int wid_all = (int)blockIdx.x * (int)(blockDim.x >> 6) + wave;
+        int p, w_first;
+        quad_which(qa, wid_all, p, w_first);
+        quad_body<Q, M, U, SRC>(qa, quad_lds, p, w_first, wid_all);
+    }
+
+    // Two formats in one launch (Q and K in Q4_K, V in Q6_K): whole workgroups belong to one
+    // format, so the branch is uniform per workgroup.
+    template <class QA, int UA, class QB, int UB, int M, int SRC>
+    __global__ void __launch_bounds__(QA::max_threads(M) < QB::max_threads(M) ? QA::max_threads(M) : QB::max_threads(M))
+        gemv_quad_dual_kernel(const QuadArgs qa)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int wid_all = (int)blockIdx.x * (int)(blockDim.x >> 6) + wave;
+        int p, w_first;
+        quad_which(qa, wid_all, p, w_first);
+        if (p < qa.first_b)
+            quad_body<QA, M, UA, SRC>(qa, quad_lds, p, w_first, wid_all);
+        else
+            quad_body<QB, M, UB, SRC>(qa, quad_lds, p, w_first, wid_all);
+    }
+
+    template <class Q, int M, int U, int SRC>
     inline void gemv_quad_launch_mus(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         static bool attr_set = false;
@@ -754,6 +786,50 @@ namespace llamql
         case 6: gemv_quad_launch_mu<Q, 6, Q::LOADS <= 3 ? 2 : 1>(src, grid, block, lds, st, a); break;
         case 7: gemv_quad_launch_mu<Q, 7, Q::LOADS <= 3 ? 2 : 1>(src, grid, block, lds, st, a); break;
         default: gemv_quad_launch_mu<Q, 8, Q::LOADS <= 3 ? 2 : 1>(src, grid, block, lds, st, a); break;
+        }
+    }
+
+    // steps per chunk the single-format launches use for a batch size
+    template <class Q>
+    constexpr int quad_unroll(int M)
+    {
+        return M <= 2 ? (Q::LOADS <= 3 ? 3 : 2) : M <= 4 ? 2 : (Q::LOADS <= 3 ? 2 : 1);
+    }
+
+    template <class QA, class QB, int M, int SRC>
+    inline void gemv_quad_dual_launch_ms(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
+    {
+        auto kernel = &gemv_quad_dual_kernel<QA, quad_unroll<QA>(M), QB, quad_unroll<QB>(M), M, SRC>;
+        static bool attr_set = false;
+        if (!attr_set)
+        {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      160 * 1024);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+    }
+
+    template <class QA, class QB, int M>
+    inline void gemv_quad_dual_launch_m(int src, dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
+    {
+        if (src == QUAD_SRC_F32)
+            gemv_quad_dual_launch_ms<QA, QB, M, QUAD_SRC_F32>(grid, block, lds, st, a);
+        else
+            gemv_quad_dual_launch_ms<QA, QB, M, QUAD_SRC_Q8>(grid, block, lds, st, a);
+    }
+
+    // M = 1..4, src Q8_1 or fp32
+    template <class QA, class QB>
+    inline void gemv_quad_dual_launch(int M, int src, dim3 grid, dim3 block, size_t lds, hipStream_t st,
+                                      const QuadArgs &a)
+    {
+        switch (M)
+        {
+        case 1: gemv_quad_dual_launch_m<QA, QB, 1>(src, grid, block, lds, st, a); break;
+        case 2: gemv_quad_dual_launch_m<QA, QB, 2>(src, grid, block, lds, st, a); break;
+        case 3: gemv_quad_dual_launch_m<QA, QB, 3>(src, grid, block, lds, st, a); break;
+        default: gemv_quad_dual_launch_m<QA, QB, 4>(src, grid, block, lds, st, a); break;
         }
     }
 
