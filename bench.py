@@ -107,31 +107,41 @@ def bench_moe(args, torch, capi, synth, dev):
     # the shared expert is entry E of the table and sits in a ninth slot of every token
     # (weight 1) that the router leaves alone: one gate/up and one down launch serve all
     table = capi.expert_table(experts, dev)
+    # Several independent token sets (own hidden states, router logits and buffers), so that
+    # consecutive steps route to different experts and their weights are not served from the
+    # caches: 1 token x 9 experts x 1.35 MB per step against 256 MB of Infinity Cache.  All sets
+    # are captured in ONE graph, the way a decode pass captures all of its MoE layers.
+    nsets = 32 if T == 1 else 4
     g = torch.Generator(device=dev)
     g.manual_seed(11)
-    x = torch.randn(T, H, device=dev, generator=g)
-    logits = torch.randn(T, E, device=dev, generator=g)
-    q8 = torch.empty(T * (H // 32) * 36, dtype=torch.uint8, device=dev)
-    out = torch.empty(T, H, device=dev)
-    ids = torch.full((T, TOPK + 1), E, dtype=torch.int32, device=dev)
-    w = torch.ones(T, TOPK + 1, device=dev)
+    sets = []
+    for _ in range(nsets):
+        sets.append({"x": torch.randn(T, H, device=dev, generator=g),
+                     "logits": torch.randn(T, E, device=dev, generator=g),
+                     "q8": torch.empty(T * (H // 32) * 36, dtype=torch.uint8, device=dev),
+                     "out": torch.empty(T, H, device=dev),
+                     "ids": torch.full((T, TOPK + 1), E, dtype=torch.int32, device=dev),
+                     "w": torch.ones(T, TOPK + 1, device=dev)})
 
-    def step(_i=0):
-        capi.moe_route(logits, TOPK, ids=ids, weights=w)
-        capi.quantize_q8_1(x, out=q8)
-        gate, up = capi.moe_gate_up(fmt, table, E + 1, ids, q8, T, TOPK + 1, H, I)
+    def step(s):
+        capi.moe_route(s["logits"], TOPK, ids=s["ids"], weights=s["w"])
+        capi.quantize_q8_1(s["x"], out=s["q8"])
+        gate, up = capi.moe_gate_up(fmt, table, E + 1, s["ids"], s["q8"], T, TOPK + 1, H, I)
         qa = capi.swiglu_quantize(gate, up)
-        capi.moe_down(fmt, table, E + 1, ids, w, qa, out, T, TOPK + 1, H, I, accumulate=False)
+        capi.moe_down(fmt, table, E + 1, s["ids"], s["w"], qa, s["out"], T, TOPK + 1, H, I, accumulate=False)
 
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
-        for _ in range(max(args.warmup, 2)):
-            step()
+        for i in range(max(args.warmup, 2)):
+            step(sets[i % nsets])
         stream.synchronize()
         gr = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gr, stream=stream):
-            step()
-        us = _time_launches(torch, stream, lambda i: gr.replay(), args.steps, 3)
+            for s_ in sets:
+                step(s_)
+        reps = max(1, (args.steps + nsets - 1) // nsets)
+        us = _time_launches(torch, stream, lambda i: gr.replay(), reps, 2) / nsets
+        distinct = len(set(int(v) for s_ in sets for v in s_["ids"][:, :TOPK].flatten().tolist()))
     blk = 112  # device bytes per IQ3_S super-block
     w_bytes = (TOPK + 1) * T * 3 * I * (H // 256) * blk  # every token slot streams its expert's three matrices
     value = w_bytes / (us * 1e-6) / 1e9
@@ -139,7 +149,8 @@ def bench_moe(args, torch, capi, synth, dev):
                    {"workload": "MoE expert FFN decode: hidden 2048, 256 routed experts + 1 shared, top-8, expert "
                                 "intermediate 512, IQ3_S, %d token(s); route, quantise, gate/up, SwiGLU + quantise, down; shared expert in a ninth slot" % T,
                     "tokens": T, "weight_bytes_per_step": w_bytes, "tokens_per_s": round(T / (us * 1e-6), 1),
-                    "launch": "hip-graph replay"},
+                    "token_sets_rotated": nsets, "distinct_routed_experts_over_sets": distinct,
+                    "launch": "hip-graph replay of all token sets' steps"},
                    {"kernel": "moe step (5 launches)", "bound": "hbm", "achieved": round(value, 1),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None,
                     "bytes_per_launch": w_bytes, "us_per_launch": round(us, 2), "launches_timed": args.steps})

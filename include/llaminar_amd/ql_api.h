@@ -156,7 +156,16 @@ bool llam_ql_epilogue(float *d_c, const float *d_t, const float *d_bias, int M,
                       void *stream);
 
 /* ---- P4: MoE ---------------------------------------------------------------------------
- * Router: softmax over all experts, top_k by probability (ties: lower expert
+ * Router logits: d_logits[t*n_experts + e] = dot(d_hidden[t,:], d_gate_w[e,:]) in fp32
+ * (the router matrix is not quantised).  Replaces the vec_dot loop at the top of
+ * CPUMoEKernel::route (src/v2/kernels/cpu/moe/CPUMoEKernel.cpp:45-49); floating point,
+ * summation order differs from the reference's SIMD dot (tests: 1e-5 of the largest
+ * logit).  d_model % 4 == 0. */
+bool llam_ql_moe_router_logits(const float *d_hidden, const float *d_gate_w, float *d_logits,
+                               int n_tokens, int d_model, int n_experts, int device_id,
+                               void *stream);
+
+/* Router: softmax over all experts, top_k by probability (ties: lower expert
  * id first), weights renormalised over the top_k when normalize != 0.
  * Replaces CPUMoEKernel::route's selection stage
  * (src/v2/kernels/cpu/moe/CPUMoEKernel.cpp:87-124; IMoEKernel::route,
@@ -193,7 +202,8 @@ typedef struct
  * 2*top_k-projection multiply_fused_tensor of MoEExpertComputeStage
  * (src/v2/execution/compute_stages/stages/MoEExpertComputeStage.cpp:1450-1482);
  * counterpart of groupedExpertGateUpDecodeFromRouting (IMoEKernel.h:378-643).
- * The table has n_experts entries; a slot whose id is outside [0,n_experts) is
+ * The table has n_experts entries; a slot whose id is outside [0,n_experts), or whose
+ * expert has a NULL matrix in the table (an expert that lives on another device), is
  * skipped (its outputs are left untouched). */
 bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts,
                          int n_experts, const int32_t *d_ids, const void *d_q8,

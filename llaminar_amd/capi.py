@@ -56,6 +56,7 @@ SIGNATURES = {
     "llam_ql_gemm": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_epilogue": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int,
                                   c_void_p]),
+    "llam_ql_moe_router_logits": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_route_ex": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "llam_ql_moe_route": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "llam_ql_moe_gate_up": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
@@ -250,6 +251,18 @@ def epilogue(c, t, bias, alpha: float, beta: float, stream=None):
     _check(load().llam_ql_epilogue(_ptr(c), _ptr(t), _ptr(bias), M, N, c.stride(0), alpha, beta, _dev(c),
                                    _stream(stream)), "epilogue")
     return c
+
+
+def moe_router_logits(hidden, gate_w, stream=None):
+    """logits[T, E] = hidden[T, D] @ gate_w[E, D]^T in fp32."""
+    import torch
+
+    T, D = hidden.shape
+    E = gate_w.shape[0]
+    out = torch.empty(T, E, dtype=torch.float32, device=hidden.device)
+    _check(load().llam_ql_moe_router_logits(_ptr(hidden), _ptr(gate_w), _ptr(out), T, D, E, _dev(hidden),
+                                            _stream(stream)), "moe_router_logits")
+    return out
 
 
 def moe_route(logits, top_k: int, normalize: bool = True, stream=None, ids=None, weights=None):

@@ -154,7 +154,7 @@ namespace llamql
     }
 
     // ---- attention --------------------------------------------------------------------------
-    // Workgroup = (chunk of ATT_CHUNK cache positions, KV head, sequence); its G = n_heads/n_kv
+    // Workgroup = (chunk of ATT_CHUNK = 128 cache positions, KV head, sequence); its G = n_heads/n_kv
     // query heads share every K and V row it reads.  Sixteen lanes cover the 128 columns of
     // a row (8 fp16 = 16 bytes each), so a wavefront takes four positions per pass.
     //   pass 1: scores s[p][g] = q_g . K[p] / sqrt(d)          -> LDS
@@ -266,15 +266,26 @@ namespace llamql
         // statistics: wavefront w takes heads w, w + 4, ...
         for (int g = wave; g < G; g += ATT_THREADS / WAVE)
         {
-            const float a0 = s_sc[lane][g], a1 = s_sc[lane + 64][g];
-            float mx = fmaxf(a0, a1);
+            constexpr int PER_LANE = ATT_CHUNK / WAVE;
+            float sc[PER_LANE];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int k = 0; k < PER_LANE; ++k)
+            {
+                sc[k] = s_sc[lane + WAVE * k][g];
+                mx = fmaxf(mx, sc[k]);
+            }
 #pragma unroll
             for (int off = WAVE / 2; off > 0; off >>= 1)
                 mx = fmaxf(mx, __shfl_xor(mx, off, WAVE));
-            const float e0 = expf(a0 - mx), e1 = expf(a1 - mx); // position p0 is valid: mx is finite
-            s_sc[lane][g] = e0;
-            s_sc[lane + 64][g] = e1;
-            float l = e0 + e1;
+            float l = 0.0f;
+#pragma unroll
+            for (int k = 0; k < PER_LANE; ++k)
+            {
+                const float e = expf(sc[k] - mx); // position p0 is valid: mx is finite
+                s_sc[lane + WAVE * k][g] = e;
+                l += e;
+            }
 #pragma unroll
             for (int off = WAVE / 2; off > 0; off >>= 1)
                 l += __shfl_xor(l, off, WAVE);

@@ -123,6 +123,34 @@ namespace llamql
             weights[(size_t)t * slot_stride + lane] = normalize ? __fdiv_rn(my_top, topk_sum) : my_top;
     }
 
+    // ---- router logits -------------------------------------------------------------------
+    // logits[t][e] = dot(hidden[t], gate_w[e]) in fp32: one wavefront per (token, expert),
+    // float4 loads, fused multiply-adds per lane, then the fixed-order wavefront sum.
+    __global__ void __launch_bounds__(256)
+        moe_router_logits_kernel(const float *__restrict__ hidden, const float *__restrict__ gate_w,
+                                 float *__restrict__ logits, int d_model, int n_experts)
+    {
+        const int t = blockIdx.y;
+        const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+        const int lane = threadIdx.x & (WAVE - 1);
+        if (e >= n_experts)
+            return; // whole wavefronts leave together
+        const float4 *h = reinterpret_cast<const float4 *>(hidden + (size_t)t * d_model);
+        const float4 *w = reinterpret_cast<const float4 *>(gate_w + (size_t)e * d_model);
+        float acc = 0.0f;
+        for (int i = lane; i < (d_model >> 2); i += WAVE)
+        {
+            const float4 a = h[i], b = w[i];
+            acc = fmaf(a.x, b.x, acc);
+            acc = fmaf(a.y, b.y, acc);
+            acc = fmaf(a.z, b.z, acc);
+            acc = fmaf(a.w, b.w, acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0)
+            logits[(size_t)t * n_experts + e] = acc;
+    }
+
     // ---- routed gate/up ---------------------------------------------------------
     struct MoEArgs
     {
@@ -148,6 +176,8 @@ namespace llamql
             return; // uniform for the workgroup; outputs of a bad id stay untouched
         GemvArgs a;
         a.w = blockIdx.z == 0 ? m.experts[e].d_gate : m.experts[e].d_up;
+        if (!a.w)
+            return; // an expert whose matrices live elsewhere: skipped like a bad id (uniform)
         a.q8 = m.q8 + (size_t)t * (m.hidden / 32) * 9;
         a.y = (blockIdx.z == 0 ? m.out0 : m.out1) + (size_t)slot * m.inter;
         a.sums = nullptr;
@@ -178,8 +208,8 @@ namespace llamql
         {
             const int slot = t * m.top_k + s;
             const int e = m.ids[slot];
-            if (e < 0 || e >= m.n_experts)
-                continue;
+            if (e < 0 || e >= m.n_experts || !m.experts[e].d_down)
+                continue; // bad id, or an expert whose matrices live elsewhere
             GemvArgs a;
             a.w = m.experts[e].d_down;
             a.q8 = m.q8 + (size_t)slot * (m.inter / 32) * 9;
@@ -247,7 +277,11 @@ namespace llamql
         const void *wdown[S];
 #pragma unroll
         for (int s = 0; s < S; ++s)
+        {
             wdown[s] = e[s] >= 0 ? m.experts[e[s]].d_down : nullptr;
+            if (!wdown[s])
+                e[s] = -1; // an expert whose matrices live elsewhere: skipped like a bad id
+        }
 
         const long wg_row0 = (long)blockIdx.x * (GEMV_WAVES * R * m.rows_per_wave);
         auto load_rows = [&](typename F::Raw(&raw)[S], long row) {
@@ -452,6 +486,30 @@ namespace llamql
         }
     } // namespace
 } // namespace llamql
+
+extern "C" bool llam_ql_moe_router_logits(const float *d_hidden, const float *d_gate_w, float *d_logits,
+                                          int n_tokens, int d_model, int n_experts, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_router_logits";
+    if (n_tokens < 0 || d_model < 1 || n_experts < 1)
+        return fail(fn, "bad size (n_tokens=%d d_model=%d n_experts=%d)", n_tokens, d_model, n_experts);
+    if (n_tokens == 0)
+        return true;
+    if ((d_model % 4) != 0)
+        return fail(fn, "d_model=%d must be a multiple of 4", d_model);
+    if (!d_hidden || !d_gate_w || !d_logits)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_hidden) || !aligned16(d_gate_w) || !aligned4(d_logits))
+        return fail(fn, "d_hidden and d_gate_w must be 16-byte aligned");
+    if (n_tokens > 65535)
+        return fail(fn, "too many tokens for one launch");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(moe_router_logits_kernel, dim3((unsigned)((n_experts + 3) / 4), (unsigned)n_tokens), dim3(256),
+                       0, as_stream(stream), d_hidden, d_gate_w, d_logits, d_model, n_experts);
+    return launched(fn);
+}
 
 extern "C" bool llam_ql_moe_route_ex(const float *d_logits, int n_tokens, int n_experts,
                                      int top_k, int normalize, int32_t *d_ids,

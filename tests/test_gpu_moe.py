@@ -33,6 +33,20 @@ def test_router(capi, dev, oracle):
     assert np.allclose(w.cpu().numpy(), 0.25)
 
 
+def test_router_logits(capi, dev):
+    """fp32 router matrix times hidden states against float64 numpy (floating point: 1e-5 of
+    the largest logit; the reference's SIMD dot sums in another order as well)."""
+    import torch
+
+    rng = np.random.default_rng(4)
+    for T, D, E in ((1, 2048, 256), (16, 2048, 257), (3, 5120, 7)):
+        h = rng.standard_normal((T, D)).astype(np.float32)
+        w = (rng.standard_normal((E, D)) * 0.05).astype(np.float32)
+        got = capi.moe_router_logits(torch.from_numpy(h).to(dev), torch.from_numpy(w).to(dev)).cpu().numpy()
+        exp = h.astype(np.float64) @ w.astype(np.float64).T
+        assert np.abs(got - exp).max() <= 1e-5 * np.abs(exp).max(), (T, D, E)
+
+
 def test_swiglu_quantize(capi, dev, oracle):
     import torch
 
