@@ -291,6 +291,11 @@ namespace llaminar_amd
             return false;
         void *q8 = s.take(q8_bytes(m, k));
         const float *a = A->data + (size_t)activation_row_offset * k;
+        // plain decode product: the fp32-input GEMV quantises inside its kernel where that
+        // saves the quantiser launch (same bits), else through q8
+        if (m <= LLAM_QL_MAX_GEMV_M && alpha == 1.0f && beta == 0.0f && !bias)
+            return forward(fn, llam_ql_gemv_f32(fmt_, d_weights_, a, k, C->data, m, n, k, C->stride(), q8, device_id_,
+                                                stream_));
         return forward(fn, llam_ql_quantize_q8_1(a, q8, m, k, device_id_, stream_)) &&
                run(fn, q8, C->data, C->stride(), m, n, bias, alpha, beta, s, stream_);
     }
@@ -370,8 +375,6 @@ namespace llaminar_amd
         if (!open_scratch(fn, round_up(q8_bytes(m, k)) + tmp_bytes, workspace, s))
             return false;
         void *q8 = s.take(q8_bytes(m, k));
-        if (!forward(fn, llam_ql_quantize_q8_1(input->data, q8, m, k, device_id_, stream_)))
-            return false;
 
         bool any_bias = false;
         for (const auto &p : projections)
@@ -388,8 +391,11 @@ namespace llaminar_amd
                 projs[i].ldy = p.output->stride();
                 projs[i].fmt = p.kernel->fmt_;
             }
-            return forward(fn, llam_ql_gemv_fused(projs, (int)projections.size(), q8, m, k, device_id_, stream_));
+            return forward(fn, llam_ql_gemv_fused_f32(projs, (int)projections.size(), input->data, k, m, k, q8,
+                                                      device_id_, stream_));
         }
+        if (!forward(fn, llam_ql_quantize_q8_1(input->data, q8, m, k, device_id_, stream_)))
+            return false;
         for (const auto &p : projections)
         {
             Scratch each = s; // the intermediate, if any, is reused by every projection
@@ -431,6 +437,9 @@ namespace llaminar_amd
         if (!open_scratch(fn, getWorkspaceRequirements(m, n, k), workspace, s))
             return false;
         void *q8 = s.take(q8_bytes(m, k));
+        if (m <= LLAM_QL_MAX_GEMV_M && alpha == 1.0f && beta == 0.0f)
+            return forward(fn, llam_ql_gemv_swiglu_f32(fmt_, d_weights_, gate->data, up->data, k, output->data, m, n,
+                                                       k, output->stride(), q8, device_id_, stream_));
         return forward(fn, llam_ql_swiglu_quantize(gate->data, up->data, nullptr, q8, m, k, device_id_, stream_)) &&
                run(fn, q8, output->data, output->stride(), m, n, nullptr, alpha, beta, s, stream_);
     }
