@@ -73,14 +73,16 @@ size_t llam_dec_attention_scratch_floats(int B, int n_heads, int head_dim, int c
 /* Single-token grouped-query attention over the fp16 caches:
  * d_out[b][h][:] = softmax_p(q[b][h] . K[b][h / (n_heads/n_kv)][p] / sqrt(head_dim)) . V[...][p]
  * over p = 0 .. d_pos[b] inclusive (the token appended last).  Q heads are read from
- * d_q (row stride ld_q), outputs go to d_out (row stride ld_out), fp32.
+ * d_q (row stride ld_q); outputs go to d_out (fp32, row stride ld_out) and / or to d_q8_out
+ * as the Q8_1 blocks [B][n_heads*head_dim/32] of the same rows (the quantiser of the output
+ * projection, with the arithmetic of llam_ql_quantize_q8_1); either may be NULL.
  * Replaces CPUFlashAttentionKernelT::compute_decode with fp16 KV
  * (src/v2/kernels/cpu/attention/CPUFlashAttentionKernelT.h:507-545, 633-662).
  * head_dim == 128, n_heads / n_kv in {1, 2, 4, 8}. */
 bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kcache, const void *d_vcache,
-                        const int32_t *d_pos, float *d_out, int ld_out, float *d_scratch, int B,
-                        int n_heads, int n_kv, int head_dim, int ctx_cap, int device_id,
-                        void *stream);
+                        const int32_t *d_pos, float *d_out, int ld_out, void *d_q8_out,
+                        float *d_scratch, int B, int n_heads, int n_kv, int head_dim, int ctx_cap,
+                        int device_id, void *stream);
 
 /* Scratch bytes llam_dec_argmax needs for its per-workgroup partial results. */
 size_t llam_dec_argmax_scratch_bytes(int B, int n);

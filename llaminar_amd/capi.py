@@ -73,8 +73,8 @@ SIGNATURES = {
     "llam_dec_rope_kv_append": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                          c_int, c_int, c_int, c_void_p]),
     "llam_dec_attention_scratch_floats": (c_size_t, [c_int, c_int, c_int, c_int]),
-    "llam_dec_attention": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
-                                    c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_dec_attention": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                    c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_dec_argmax_scratch_bytes": (c_size_t, [c_int, c_int]),
     "llam_dec_argmax": (c_bool, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
@@ -382,7 +382,9 @@ def attention_scratch(B: int, n_heads: int, head_dim: int, cap: int, device):
     return torch.empty(n, dtype=torch.float32, device=device)
 
 
-def attention(q, kcache, vcache, pos, n_heads: int, n_kv: int, head_dim: int, out=None, scratch=None, stream=None):
+def attention(q, kcache, vcache, pos, n_heads: int, n_kv: int, head_dim: int, out=None, scratch=None, stream=None,
+              q8_out=None):
+    """out [B, n_heads*head_dim] fp32; q8_out (optional) receives the Q8_1 blocks of the same rows."""
     import torch
 
     B = q.shape[0]
@@ -392,8 +394,8 @@ def attention(q, kcache, vcache, pos, n_heads: int, n_kv: int, head_dim: int, ou
     if scratch is None:
         scratch = attention_scratch(B, n_heads, head_dim, cap, q.device)
     _check(load().llam_dec_attention(_ptr(q), _ld(q), _ptr(kcache), _ptr(vcache), _ptr(pos), _ptr(out), _ld(out),
-                                     _ptr(scratch), B, n_heads, n_kv, head_dim, cap, _dev(q), _stream(stream)),
-           "attention")
+                                     _ptr(q8_out), _ptr(scratch), B, n_heads, n_kv, head_dim, cap, _dev(q),
+                                     _stream(stream)), "attention")
     return out
 
 

@@ -367,9 +367,10 @@ namespace llamql
 
     __global__ void __launch_bounds__(ATT_HD)
         attention_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml,
-                               const int32_t *__restrict__ pos, float *__restrict__ out, int ld_out, int n_heads,
-                               int n_chunks, int ctx_cap)
+                               const int32_t *__restrict__ pos, float *__restrict__ out, int ld_out,
+                               uint32_t *__restrict__ q8, int n_heads, int n_chunks, int ctx_cap)
     {
+        __shared__ __attribute__((aligned(16))) float s_val[ATT_HD];
         __shared__ float s_w[ATT_MAX_CHUNKS];
         __shared__ float s_red[ATT_HD / WAVE];
         const int h = blockIdx.x, b = blockIdx.y, c = threadIdx.x;
@@ -407,7 +408,23 @@ namespace llamql
 #pragma unroll 4
         for (int k = 0; k < used; ++k)
             acc = fmaf(part_o[(base + k) * ATT_HD + c], s_w[k], acc);
-        out[(size_t)b * ld_out + (size_t)h * ATT_HD + c] = L > 0.0f ? __fdiv_rn(acc, L) : 0.0f; // pos < 0: nothing attended
+        const float val = L > 0.0f ? __fdiv_rn(acc, L) : 0.0f; // pos < 0: nothing attended
+        if (out)
+            out[(size_t)b * ld_out + (size_t)h * ATT_HD + c] = val;
+        if (q8)
+        {
+            // the head's 128 outputs are four Q8_1 blocks of the row the next projection reads
+            s_val[c] = val;
+            __syncthreads();
+            if (c < ATT_HD / 4) // 32 threads, eight per block
+            {
+                const Q8Lane q = q8_1_quantize_lane(*reinterpret_cast<const float4 *>(&s_val[4 * c]));
+                uint32_t *dst = q8 + (((size_t)b * n_heads + h) * (ATT_HD / 32) + (c >> 3)) * 9;
+                dst[1 + (c & 7)] = q.packed;
+                if ((c & 7) == 0)
+                    dst[0] = q.head;
+            }
+        }
     }
 
     // ---- greedy sampling -----------------------------------------------------------------------
@@ -601,9 +618,9 @@ extern "C" size_t llam_dec_attention_scratch_floats(int B, int n_heads, int head
 }
 
 extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kcache, const void *d_vcache,
-                                   const int32_t *d_pos, float *d_out, int ld_out, float *d_scratch, int B,
-                                   int n_heads, int n_kv, int head_dim, int ctx_cap, int device_id,
-                                   void *stream)
+                                   const int32_t *d_pos, float *d_out, int ld_out, void *d_q8_out,
+                                   float *d_scratch, int B, int n_heads, int n_kv, int head_dim, int ctx_cap,
+                                   int device_id, void *stream)
 {
     static const char *fn = "llam_dec_attention";
     if (B < 0 || n_heads < 1 || n_kv < 1 || ctx_cap < 1)
@@ -617,11 +634,12 @@ extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kca
     const int G = n_heads / n_kv;
     if (G != 1 && G != 2 && G != 4 && G != 8)
         return fail(fn, "n_heads/n_kv=%d: only 1, 2, 4 and 8 are built", G);
-    if (ld_q < n_heads * head_dim || ld_out < n_heads * head_dim)
+    if (ld_q < n_heads * head_dim || (d_out && ld_out < n_heads * head_dim))
         return fail(fn, "row strides smaller than n_heads * head_dim");
-    if (!d_q || !d_kcache || !d_vcache || !d_pos || !d_out || !d_scratch)
+    if (!d_q || !d_kcache || !d_vcache || !d_pos || (!d_out && !d_q8_out) || !d_scratch)
         return fail(fn, "null pointer");
-    if (!aligned16(d_q) || (ld_q % 4) != 0 || !aligned16(d_kcache) || !aligned16(d_vcache) || !aligned4(d_out) ||
+    if (!aligned16(d_q) || (ld_q % 4) != 0 || !aligned16(d_kcache) || !aligned16(d_vcache) ||
+        (d_out && !aligned4(d_out)) || (d_q8_out && !aligned4(d_q8_out)) ||
         !aligned16(d_scratch))
         return fail(fn, "misaligned pointer (q, caches and scratch 16-byte, out 4-byte)");
     const int n_chunks = (ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
@@ -645,7 +663,7 @@ extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kca
     if (!launched(fn))
         return false;
     hipLaunchKernelGGL(attention_merge_kernel, dim3(n_heads, B), dim3(ATT_HD), 0, st, part_o, part_ml, d_pos, d_out,
-                       ld_out, n_heads, n_chunks, ctx_cap);
+                       ld_out, static_cast<uint32_t *>(d_q8_out), n_heads, n_chunks, ctx_cap);
     return launched(fn);
 }
 

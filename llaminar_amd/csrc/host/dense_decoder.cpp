@@ -268,10 +268,12 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
         if (!forward(fn, llam_dec_rope_kv_append(d->qkv, ldqkv, d->inv_freq, d->pos, d->kcache[l], d->vcache[l], B,
                                                  c.n_heads, c.n_kv, c.head_dim, c.ctx_cap, dev, stream)))
             return false;
-        if (!forward(fn, llam_dec_attention(d->qkv, ldqkv, d->kcache[l], d->vcache[l], d->pos, d->attn, QD,
+        // the attention output leaves the merge kernel as Q8_1 blocks: the output projection's
+        // quantiser costs no launch of its own
+        if (!forward(fn, llam_dec_attention(d->qkv, ldqkv, d->kcache[l], d->vcache[l], d->pos, nullptr, 0, d->q8_attn,
                                             d->att_scratch, B, c.n_heads, c.n_kv, c.head_dim, c.ctx_cap, dev, stream)))
             return false;
-        if (!forward(fn, llam_ql_gemv_f32(w.fmt_o, w.wo, d->attn, QD, d->delta, B, H, QD, H, d->q8_attn, dev, stream)))
+        if (!forward(fn, llam_ql_gemv(w.fmt_o, w.wo, d->q8_attn, d->delta, B, H, QD, H, dev, stream)))
             return false;
         // feed-forward half
         if (!forward(fn, llam_dec_rmsnorm_q8_1(d->x, d->delta, w.ffn_norm, c.rms_eps, nullptr, d->q8_h, B, H, dev,

@@ -118,9 +118,13 @@ def test_attention_decode(capi, dev, oracle, B, n_heads, n_kv, cap, positions):
     q = torch.randn(B, n_heads * hd + 32, device=dev, generator=g) * 1.5
     pos = torch.tensor(positions, dtype=torch.int32, device=dev)
     out = torch.full((B, n_heads * hd + 4), float("nan"), device=dev)
-    capi.attention(q[:, :n_heads * hd], kc, vc, pos, n_heads, n_kv, hd, out=out[:, :n_heads * hd])
+    q8 = torch.zeros(B * (n_heads * hd // 32) * 36, dtype=torch.uint8, device=dev)
+    capi.attention(q[:, :n_heads * hd], kc, vc, pos, n_heads, n_kv, hd, out=out[:, :n_heads * hd], q8_out=q8)
     sync()
     got = out.cpu().numpy()
+    # the Q8_1 side output: the bit-exact quantiser applied to the fp32 rows it wrote
+    assert np.array_equal(q8.cpu().numpy().reshape(B, n_heads * hd // 32, 36),
+                          oracle.quantize(np.ascontiguousarray(got[:, :n_heads * hd])))
     assert np.isnan(got[:, n_heads * hd:]).all()
     kh, vh = kc.cpu().numpy().view(np.uint16), vc.cpu().numpy().view(np.uint16)
     qh = q.cpu().numpy()
