@@ -26,7 +26,14 @@ def test_host_library_exports_moe_methods():
                    "groupedExpertDownDecodeFromRuntime", "groupedExpertDecodeFromRuntime", "sharedExpertGateAdd",
                    "getWorkspaceRequirements"):
         assert f"llaminar_amd::MI355MoEKernel::{method}(" in out, method
-    for fn in ("llam_decoder_create", "llam_decoder_step", "llam_decoder_set_layer", "llam_decoder_buffer"):
+    # every function include/llaminar_amd/dense_decoder.h declares
+    import re
+
+    text = (ROOT / "include" / "llaminar_amd" / "dense_decoder.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(llam_decoder_[a-z_]+)\s*\(", text)))
+    assert len(names) >= 9, names
+    for fn in names:
         assert f" T {fn}" in out, fn
 
 
