@@ -240,6 +240,9 @@ class Ref:
             L.ref_rope_inv_freq.argtypes = [c_int, c_float, c_void_p]
             L.ref_rope_token.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float]
             L.ref_rope_head_scalar.argtypes = [c_void_p, c_int, c_int, c_float]
+        self.has_swiglu = hasattr(L, "ref_swiglu")
+        if self.has_swiglu:
+            L.ref_swiglu.argtypes = [c_void_p, c_void_p, c_void_p, c_int]
         self.L = L
 
     def f16_to_f32(self, h):
@@ -330,6 +333,13 @@ class Ref:
         y = np.zeros_like(r)
         self.L.ref_residual_rmsnorm_row(_p(d), _p(r), _p(g), _p(y), r.size, eps)
         return y, r
+
+    def swiglu(self, gate, up):
+        g = np.ascontiguousarray(gate, dtype=np.float32)
+        u = np.ascontiguousarray(up, dtype=np.float32)
+        out = np.zeros_like(g)
+        self.L.ref_swiglu(_p(g), _p(u), _p(out), g.size)
+        return out
 
     def rope_inv_freq(self, head_dim, theta):
         out = np.zeros(head_dim // 2, np.float32)

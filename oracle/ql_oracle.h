@@ -87,9 +87,12 @@ void qlo_epilogue(float *C, const float *tmp, int M, int N, int ldc,
 void qlo_moe_route(const float *logits, int n_tokens, int n_experts, int top_k,
                    int normalize, int32_t *ids, float *weights, float *probs);
 
-/* silu(g)*u with an accurate expf.  The reference's CPU SwiGLU uses a
- * hardware-approximate reciprocal (kernels/cpu/primitives/SwiGLUPrimitives.cpp:137-208)
- * and is not bit-reproducible; this is the mathematical function it approximates. */
+/* silu(g)*u = (g / (1 + expf(-g))) * u, the reference's scalar routine
+ * (kernels/cpu/primitives/SwiGLUPrimitives.cpp:40-51, bit-identical on the same libm).
+ * Its vector paths (:137-208: a degree-5 exp polynomial, rcp14 and one Newton step)
+ * approximate the same function; measured against the reference's compiled code they
+ * stay within 8e-6 relative per element, which the tests check where oracle/_ref is
+ * built and on the committed vectors. */
 void qlo_swiglu(const float *gate, const float *up, int n, float *out);
 
 /* ---- decode-step operators (decode_oracle.c) ------------------------------------- */

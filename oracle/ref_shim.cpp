@@ -20,6 +20,7 @@
 #include "kernels/cpu/native_vnni/CPUNativeVNNIGemv.h"
 #include "kernels/cpu/primitives/RMSNormPrimitives.h"
 #include "kernels/cpu/primitives/RoPEPrimitives.h"
+#include "kernels/cpu/primitives/SwiGLUPrimitives.h"
 #include "tensors/BlockStructures.h"
 #include "tensors/FP16Utils.h"
 #include "tensors/IQQuantTables.h"
@@ -287,5 +288,11 @@ extern "C"
     {
         primitives::apply_rope_to_head_scalar(head, position, primitives::get_inv_freq_cached(head_dim, theta),
                                               head_dim, 0);
+    }
+    // silu(gate) * up as the CPU FFN computes it (ISA dispatch, no OpenMP region):
+    // compute_swiglu_serial, SwiGLUPrimitives.cpp:254
+    void ref_swiglu(const float *gate, const float *up, float *out, int n)
+    {
+        primitives::compute_swiglu_serial(gate, up, out, n);
     }
 }

@@ -1,5 +1,5 @@
 """Writes tests/golden/decode_goldens.npz: inputs and the outputs of the reference's own
-RMSNorm and RoPE primitives (compiled into oracle/_ref from the reference tree by
+RMSNorm, RoPE and SwiGLU primitives (compiled into oracle/_ref from the reference tree by
 oracle/Makefile).  Run in a container that holds the reference; the fixture is data only."""
 from pathlib import Path
 import sys
@@ -35,6 +35,11 @@ def main():
     out["rope_positions"] = pos
     out["rope_scalar"] = np.stack([ref.rope_head_scalar(head, int(p), theta) for p in pos])
     out["rope_token_q"] = np.stack([ref.rope_token(np.tile(head, 2), k, hd, int(p), theta)[0] for p in pos])
+    assert ref.has_swiglu
+    g = (rng.standard_normal(1037) * 4).astype(np.float32)  # 64 vectors and a scalar tail of 13
+    g[:8] = [-100, -88, -20, -1e-3, 0, 1e-3, 20, 88]
+    u = rng.standard_normal(1037).astype(np.float32)
+    out["swiglu_gate"], out["swiglu_up"], out["swiglu_out"] = g, u, ref.swiglu(g, u)
     np.savez_compressed(Path(__file__).with_name("decode_goldens.npz"), **out)
     print("wrote decode_goldens.npz", {k: np.asarray(v).shape for k, v in out.items()})
 

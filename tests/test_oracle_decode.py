@@ -205,6 +205,31 @@ def test_rope_against_reference(oracle, ref):
         assert np.abs(mine_q - rq).max() <= 5e-6 and np.abs(mine_k - rk).max() <= 5e-6
 
 
+def test_swiglu_against_reference(oracle, ref):
+    """silu(gate) * up: the reference's vector path (a degree-5 exp polynomial, rcp14 plus one
+    Newton step; SwiGLUPrimitives.cpp:137-208) stays within a few 1e-6 of the mathematical
+    function the restatement computes; its scalar tail is that function itself."""
+    if not getattr(ref, "has_swiglu", False):
+        pytest.skip("reference SwiGLU not in this build of oracle/_ref")
+    rng = np.random.default_rng(13)
+    for n, spread in ((25600, 3.0), (512, 1.0), (2048, 8.0)):
+        g = (rng.standard_normal(n) * spread).astype(np.float32)
+        u = rng.standard_normal(n).astype(np.float32)
+        mine, theirs = oracle.swiglu(g, u), ref.swiglu(g, u)
+        assert np.abs(mine - theirs).max() <= 1e-5 * np.maximum(np.abs(mine), 1e-3).max()
+        assert (np.abs(mine - theirs) <= 8e-6 * np.abs(mine) + 1e-30).all()
+    # fewer than one vector: the scalar routine, the same expression on the same libm
+    g = (rng.standard_normal(13) * 4).astype(np.float32)
+    u = rng.standard_normal(13).astype(np.float32)
+    assert np.array_equal(oracle.swiglu(g, u), ref.swiglu(g, u))
+    # closed form in float64, and the special values
+    g = np.array([-30, -8, -1, -1e-3, 0, 1e-3, 1, 8, 30], np.float32)
+    u = np.full(g.size, 1.5, np.float32)
+    want = (g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64)))) * 1.5
+    assert np.abs(oracle.swiglu(g, u) - want).max() <= 3e-7 * np.abs(want).max()
+    assert oracle.swiglu(np.zeros(4, np.float32), np.ones(4, np.float32)).tolist() == [0, 0, 0, 0]
+
+
 def test_committed_reference_vectors(oracle):
     """Outputs of the reference's primitives written by tests/golden/make_decode_goldens.py."""
     if not GOLD.exists():
@@ -222,3 +247,7 @@ def test_committed_reference_vectors(oracle):
         got = oracle.rope_head(z["rope_head"], int(pos), f)
         assert np.abs(got - z["rope_scalar"][i]).max() <= 4.8e-7 * np.abs(z["rope_head"]).max()
         assert np.abs(got - z["rope_token_q"][i][:128]).max() <= 5e-6
+    if "swiglu_out" in z:
+        mine = oracle.swiglu(z["swiglu_gate"], z["swiglu_up"])
+        assert (np.abs(mine - z["swiglu_out"]) <= 8e-6 * np.abs(mine) + 1e-30).all()
+        assert np.array_equal(mine[1024:], z["swiglu_out"][1024:])  # the scalar tail
