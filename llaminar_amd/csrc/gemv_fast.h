@@ -326,13 +326,14 @@ namespace llamql
         else
             return false;
     }
-    // Batches of 5..8 rows on rows of 8..64 super-blocks (the activations of the whole batch
-    // must fit the 160 KiB of LDS) go to the matrix-unit kernel, in formats that have one.
+    // Batches of 5..8 rows on rows of 8 super-blocks or more (the activations of the whole batch
+    // and the wavefronts' bounce buffers must fit the 160 KiB of LDS) go to the matrix-unit
+    // kernel, in formats that have one.
     template <class F>
     bool mfma_eligible(int M, int N, int K)
     {
         if constexpr (F::USE_MFMA_BATCH)
-            return M >= 5 && N >= 1 && K / 256 >= 8 && mfma_lds_bytes(K / 256) <= QUAD_MAX_LDS &&
+            return M >= 5 && N >= 1 && K / 256 >= 8 && mfma_max_slices(K / 256) >= 1 &&
                    gemv_unroll_override() == 0 && gemv_rows_per_wave_override() == 0;
         else
             return false;
@@ -368,10 +369,9 @@ namespace llamql
         a.N = N;
         a.SB = SB;
         a.M = M;
-        a.sb_per_slice = sh.sb_per_slice;
         a.slices = sh.slices;
         const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles_per_wg) * WAVE);
-        const size_t lds = mfma_lds_bytes(SB);
+        const size_t lds = mfma_lds_bytes(SB, sh.slices * sh.tiles_per_wg);
         switch (src.kind)
         {
         case ACT_SRC_F32: gemv_mfma_q4k_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;

@@ -14,9 +14,14 @@
 // The accumulator is zero for every block, so the MFMA result is the reference's per-block
 // int32 sum, rescaled in fp32 block after block in ascending order.
 //
-// A workgroup owns 32 weight rows; its wavefronts split the row length into slices of whole
-// super-blocks (K = 5120: 4 slices of 5) so that the chip sees enough wavefronts, and their
-// partial sums are added in slice order at the end.
+// The wavefronts of a 32-row tile share its super-blocks round robin (K = 5120: 4 wavefronts,
+// wavefront j takes super-blocks j, j+4, ..: at any moment they read neighbouring super-blocks
+// of every row); their partial sums are added in wavefront order at the end.
+//
+// Weight loads are coalesced: the 32 x 144 bytes of a step are 288 16-byte pieces; lane l loads
+// pieces l, l+64, .. (nine neighbouring lanes cover one super-block, so an instruction touches
+// 8 rows instead of 64) and the wavefront passes them through a private LDS buffer to the lane
+// that needs them as an operand.  No barrier: LDS instructions of one wavefront run in order.
 #pragma once
 #include "gemv_core.h"
 #include "gemv_quad.h"
@@ -25,7 +30,9 @@ namespace llamql
 {
     constexpr int MFMA_TILE_ROWS = 32;
     constexpr int MFMA_MAX_SLICES = 8;
-    constexpr int MFMA_LOADS = 5; // vector memory loads per super-block and lane
+    constexpr int MFMA_MAX_WAVES = 16;     // wavefronts per workgroup
+    constexpr int MFMA_LOADS = 5;          // vector memory loads per step and lane
+    constexpr int MFMA_BOUNCE = 5 * 1024;  // LDS bytes of a wavefront's bounce buffer (320 pieces, 288 used)
 
     struct MfmaArgs
     {
@@ -39,44 +46,56 @@ namespace llamql
         int N;
         int SB;           // super-blocks per weight row
         int M;            // activation rows, 1..8
-        int sb_per_slice; // super-blocks one wavefront walks
-        int slices;       // wavefronts per 32-row tile; a workgroup holds blockDim/64/slices tiles
+        int slices;       // wavefronts per 32-row tile (wavefront j walks super-blocks j, j + slices, ..);
+                          // a workgroup holds blockDim/64/slices tiles
     };
 
     // LDS: per 32-column block 8 activation rows x 32 int8 (16 bytes of padding: neighbouring
     // blocks start four banks apart, so the staging writes do not collide) and
     // 2 x {d[4], sum*d[4]}
     constexpr int MFMA_AQ_STRIDE = 256 + 16;
-    inline size_t mfma_lds_bytes(int nsb) { return (size_t)nsb * 8 * (MFMA_AQ_STRIDE + 64); }
+    inline size_t mfma_act_bytes(int nsb) { return (size_t)nsb * 8 * (MFMA_AQ_STRIDE + 64); }
+    inline size_t mfma_lds_bytes(int nsb, int waves) { return mfma_act_bytes(nsb) + (size_t)waves * MFMA_BOUNCE; }
 
+    // pieces l, l+64, .., l+256 of a step, as loaded
     struct MfmaRaw
     {
-        v4i head, q0, q1, q2, q3;
+        v4i c0, c1, c2, c3, c4;
     };
 
-    __device__ __forceinline__ void mfma_load(MfmaRaw &r, const uint8_t *sb, const uint8_t *grp)
+    // base: the step's super-block of the tile's first row (wavefront-uniform, scalar registers);
+    // off: this lane's five byte offsets from it
+    __device__ __forceinline__ void mfma_load(MfmaRaw &r, const uint8_t *base, const uint32_t (&off)[5])
     {
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.head) : "v"(sb));
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.q0) : "v"(grp));
-        asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=&v"(r.q1) : "v"(grp));
-        asm volatile("global_load_dwordx4 %0, %1, off offset:64" : "=&v"(r.q2) : "v"(grp));
-        asm volatile("global_load_dwordx4 %0, %1, off offset:96" : "=&v"(r.q3) : "v"(grp));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.c0) : "v"(off[0]), "s"(base));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.c1) : "v"(off[1]), "s"(base));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.c2) : "v"(off[2]), "s"(base));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.c3) : "v"(off[3]), "s"(base));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.c4) : "v"(off[4]), "s"(base));
     }
     __device__ __forceinline__ void mfma_keep(MfmaRaw &r)
     {
-        asm volatile("" : "+v"(r.head), "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3));
+        asm volatile("" : "+v"(r.c0), "+v"(r.c1), "+v"(r.c2), "+v"(r.c3), "+v"(r.c4));
     }
     template <int NEWER>
     __device__ __forceinline__ void mfma_wait(MfmaRaw &r)
     {
         asm volatile("s_waitcnt vmcnt(%5)"
-                     : "+v"(r.head), "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3)
+                     : "+v"(r.c0), "+v"(r.c1), "+v"(r.c2), "+v"(r.c3), "+v"(r.c4)
                      : "n"(NEWER));
+    }
+    // orders the LDS traffic of one wavefront as seen by the compiler; the hardware runs a
+    // wavefront's LDS instructions in order, so no instruction is needed
+    __device__ __forceinline__ void mfma_wave_sync()
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 
     // SRC: where the activations come from (QUAD_SRC_*): Q8_1 blocks, or fp32 rows quantised here.
     template <int SRC>
-    __global__ void __launch_bounds__(MFMA_MAX_SLICES *WAVE) gemv_mfma_q4k_kernel(const MfmaArgs a)
+    __global__ void __launch_bounds__(MFMA_MAX_WAVES *WAVE) gemv_mfma_q4k_kernel(const MfmaArgs a)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];
         const int nsb = a.SB;
@@ -91,24 +110,44 @@ namespace llamql
         // this wavefront's tile and slice of the row, and this lane's weight row
         const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
         const int tiles_per_wg = (int)(blockDim.x >> 6) / a.slices;
-        const int s0 = slice * a.sb_per_slice;
-        int s1 = s0 + a.sb_per_slice;
-        if (s1 > nsb)
-            s1 = nsb;
-        const int nsteps = s1 > s0 ? s1 - s0 : 0;
-        const long row = ((long)blockIdx.x * tiles_per_wg + tile_local) * MFMA_TILE_ROWS + l32;
-        const long row_ld = row < a.N ? row : a.N - 1; // rows past the end re-read the last one
-        const uint8_t *rowp = a.w + (size_t)row_ld * nsb * 144;
-        const int first_sb = nsteps > 0 ? s0 : 0;
-        const int last_sb = nsteps > 0 ? s1 - 1 : 0;
+        // slice j walks super-blocks j, j + slices, ..: at any moment the wavefronts of a tile
+        // read NEIGHBOURING super-blocks of every row, so a 128-byte line that straddles two
+        // super-blocks (144 bytes each) is asked for by two wavefronts of the workgroup at the
+        // same time and crosses the fabric once
+        const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
+        const long tile_row0 = ((long)blockIdx.x * tiles_per_wg + tile_local) * MFMA_TILE_ROWS;
+        const long row = tile_row0 + l32;
+        const int last_step = nsteps > 0 ? nsteps - 1 : 0;
+
+        // piece p = lane + 64 i of the step: 16 bytes at offset 16 (p % 9) of row p / 9.  Rows
+        // past the end of the matrix (and the 32 pieces past the tile) re-read the last row.
+        const long base_row = tile_row0 < a.N ? tile_row0 : a.N - 1;
+        const int max_local = (int)(a.N - 1 - base_row) < MFMA_TILE_ROWS - 1 ? (int)(a.N - 1 - base_row)
+                                                                             : MFMA_TILE_ROWS - 1;
+        uint32_t off[5];
+#pragma unroll
+        for (int i = 0; i < 5; ++i)
+        {
+            const int p = lane + WAVE * i;
+            int r = p / 9;
+            const int piece = p - r * 9;
+            if (r > max_local)
+                r = max_local;
+            off[i] = (uint32_t)r * (uint32_t)(nsb * 144) + (uint32_t)(piece * 16);
+        }
+        const uint8_t *tile_base = a.w + (size_t)base_row * nsb * 144;
+        uint8_t *bounce = mfma_lds + nkb * (MFMA_AQ_STRIDE + 64) + wave * MFMA_BOUNCE;
+        uint8_t *bounce_wr = bounce + lane * 16;                     // piece lane + 64 i at + 1024 i
+        const uint8_t *bounce_rd = bounce + l32 * 144;               // this lane's weight row
+        const uint8_t *bounce_rdq = bounce_rd + 16 + 16 * lh;        // its half of every group
 
         // loads are never predicated: past the end of the slice a lane re-reads its last block
         auto issue = [&](MfmaRaw &r, int step) {
-            int sb = first_sb + step;
-            if (sb > last_sb)
-                sb = last_sb;
-            const uint8_t *p = rowp + (size_t)sb * 144;
-            mfma_load(r, p, p + 16 + 16 * lh);
+            const int sb = nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0;
+            const uint64_t b = (uint64_t)(tile_base + (size_t)sb * 144);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+            const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+            mfma_load(r, reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo), off);
         };
         MfmaRaw bufA, bufB;
         issue(bufA, 0);
@@ -191,14 +230,29 @@ namespace llamql
         const float *asc_lane = asc + lh * 8;
         int step = 0;
 
-        auto compute = [&](const MfmaRaw &r) {
-            const int sb = first_sb + step;
+        // the loaded pieces go to the wavefront's bounce buffer in piece order
+        auto stage = [&](const MfmaRaw &r) {
+            mfma_wave_sync(); // the previous step's reads are done
+            *reinterpret_cast<v4i *>(bounce_wr) = r.c0;
+            *reinterpret_cast<v4i *>(bounce_wr + 1024) = r.c1;
+            *reinterpret_cast<v4i *>(bounce_wr + 2048) = r.c2;
+            *reinterpret_cast<v4i *>(bounce_wr + 3072) = r.c3;
+            *reinterpret_cast<v4i *>(bounce_wr + 4096) = r.c4;
+            mfma_wave_sync();
+        };
+
+        auto compute = [&]() {
+            const int sb = slice + step * a.slices;
+            // this lane's operands: the head of its row's super-block and its half of the four groups
+            const v4i head = *reinterpret_cast<const v4i *>(bounce_rd);
+            const v4i q[4] = {*reinterpret_cast<const v4i *>(bounce_rdq), *reinterpret_cast<const v4i *>(bounce_rdq + 32),
+                              *reinterpret_cast<const v4i *>(bounce_rdq + 64),
+                              *reinterpret_cast<const v4i *>(bounce_rdq + 96)};
             Q4KQuad::Scale S[4];
-            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(0), S[0]);
-            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(1), S[1]);
-            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(2), S[2]);
-            Q4KQuad::decode_scales(r.head, Q4KQuad::lane_consts(3), S[3]);
-            const v4i q[4] = {r.q0, r.q1, r.q2, r.q3};
+            Q4KQuad::decode_scales(head, Q4KQuad::lane_consts(0), S[0]);
+            Q4KQuad::decode_scales(head, Q4KQuad::lane_consts(1), S[1]);
+            Q4KQuad::decode_scales(head, Q4KQuad::lane_consts(2), S[2]);
+            Q4KQuad::decode_scales(head, Q4KQuad::lane_consts(3), S[3]);
             const uint8_t *ab = aq_lane + (size_t)sb * (8 * MFMA_AQ_STRIDE);
             const float *sb_sc = asc_lane + (size_t)sb * (8 * 16);
             const uint32_t k = 0x0F0F0F0Fu;
@@ -241,21 +295,28 @@ namespace llamql
             ++step;
         };
 
-        // Two buffers alternate; each is reloaded (two steps ahead) once it has been consumed.
-        // Every buffer is waited for, also past the end of the slice: a register whose load is
-        // still in flight must not look free to the compiler.
+        // Two register buffers alternate; each is reloaded (two steps ahead) as soon as its
+        // pieces are in LDS, before the step is computed.  Every buffer is waited for, also past
+        // the end of the slice: a register whose load is still in flight must not look free to
+        // the compiler.
         for (int c0 = 0; c0 < nsteps; c0 += 2)
         {
             mfma_wait<MFMA_LOADS>(bufA);
             if (step < nsteps) // uniform
-                compute(bufA);
+                stage(bufA);
             __builtin_amdgcn_sched_barrier(0);
             issue(bufA, c0 + 2);
+            if (step < nsteps)
+                compute();
+            __builtin_amdgcn_sched_barrier(0);
             mfma_wait<MFMA_LOADS>(bufB);
             if (step < nsteps)
-                compute(bufB);
+                stage(bufB);
             __builtin_amdgcn_sched_barrier(0);
             issue(bufB, c0 + 3);
+            if (step < nsteps)
+                compute();
+            __builtin_amdgcn_sched_barrier(0);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the slice
         mfma_keep(bufA);
@@ -285,9 +346,18 @@ namespace llamql
 
     struct MfmaShape
     {
-        int slices, sb_per_slice, tiles_per_wg;
+        int slices, tiles_per_wg;
         long grid;
     };
+    // Most slices the LDS of a compute unit leaves room for (0: the row is too long for this kernel).
+    inline int mfma_max_slices(int nsb)
+    {
+        const size_t act = mfma_act_bytes(nsb);
+        if (act + MFMA_BOUNCE > QUAD_MAX_LDS)
+            return 0;
+        const size_t fit = (QUAD_MAX_LDS - act) / MFMA_BOUNCE;
+        return fit < (size_t)MFMA_MAX_SLICES ? (int)fit : MFMA_MAX_SLICES;
+    }
     // Slices so that a compute unit sees about a dozen wavefronts, each at least two
     // super-blocks long; tiles per workgroup so that every workgroup of the launch is resident
     // at once (a second round of workgroups would run nearly alone on the chip and cost a
@@ -296,19 +366,25 @@ namespace llamql
     {
         const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
         long want = ((long)cus * 12 + tiles - 1) / tiles;
-        if (want > MFMA_MAX_SLICES)
-            want = MFMA_MAX_SLICES;
+        if (want > mfma_max_slices(nsb))
+            want = mfma_max_slices(nsb);
         if (want > nsb / 2)
             want = nsb / 2;
         if (want < 1)
             want = 1;
         MfmaShape sh;
-        sh.sb_per_slice = (int)((nsb + want - 1) / want);
-        sh.slices = (nsb + sh.sb_per_slice - 1) / sh.sb_per_slice;
-        const long lds_wgs = (long)(QUAD_MAX_LDS / mfma_lds_bytes(nsb)); // workgroups the LDS of a CU holds
+        const int per_slice = (int)((nsb + want - 1) / want);
+        sh.slices = (nsb + per_slice - 1) / per_slice;
+        // workgroups a compute unit holds at once: by LDS, and 16 wavefronts at this kernel's registers
+        auto resident = [&](int t) {
+            const long by_lds = (long)(QUAD_MAX_LDS / mfma_lds_bytes(nsb, t * sh.slices));
+            const long by_waves = MFMA_MAX_WAVES / (t * sh.slices);
+            const long r = by_lds < by_waves ? by_lds : by_waves;
+            return r < 1 ? 1 : r;
+        };
         int t = 1;
-        while (t * 2 * sh.slices <= MFMA_MAX_SLICES && // wavefronts per workgroup
-               (tiles + t - 1) / t > (long)cus * (lds_wgs < 1 ? 1 : lds_wgs))
+        while (t * 2 * sh.slices <= MFMA_MAX_WAVES && mfma_lds_bytes(nsb, t * 2 * sh.slices) <= QUAD_MAX_LDS &&
+               (tiles + t - 1) / t > (long)cus * resident(t))
             t *= 2;
         sh.tiles_per_wg = t;
         sh.grid = (tiles + t - 1) / t;
