@@ -49,7 +49,7 @@ namespace llamql
             // batches that go to the matrix-unit kernel launch one matrix at a time
             if constexpr (F::USE_MFMA_BATCH)
                 if (mfma_eligible<F>(M, projs[0].N, K))
-                    return gemv_mfma_q4k_launch(fn, projs[0].d_w, src, projs[0].d_y, M, projs[0].N, K, projs[0].ldy,
+                    return gemv_mfma_launch<F>(fn, projs[0].d_w, src, projs[0].d_y, M, projs[0].N, K, projs[0].ldy,
                                                 device_id, st)
                                ? 1
                                : -1;

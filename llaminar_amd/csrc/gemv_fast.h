@@ -21,6 +21,8 @@
 #include "gemv_core.h"
 #include "gemv_quad.h"
 #include "gemv_mfma.h"
+#include "gemv_mfma_q6k.h"
+#include <type_traits>
 
 namespace llamql
 {
@@ -332,11 +334,16 @@ namespace llamql
     template <class F>
     bool mfma_eligible(int M, int N, int K)
     {
-        if constexpr (F::USE_MFMA_BATCH)
-            return M >= 5 && N >= 1 && K / 256 >= 8 && mfma_max_slices(K / 256) >= 1 &&
-                   gemv_unroll_override() == 0 && gemv_rows_per_wave_override() == 0;
-        else
+        if constexpr (!F::USE_MFMA_BATCH)
             return false;
+        else if (M < 5 || N < 1 || K / 256 < 8 || gemv_unroll_override() != 0 || gemv_rows_per_wave_override() != 0)
+            return false;
+        else if constexpr (std::is_same<typename F::Quad, Q6KQuad>::value)
+            // where the quad-lane kernel cannot keep the batch in LDS and would run it as two
+            // (any row length works here: long rows are walked in chunks)
+            return quad_lds_bytes(M, K / 256) > QUAD_MAX_LDS && Q6KQuad::addressable(N, K / 256);
+        else
+            return mfma_max_slices(K / 256) >= 1;
     }
 
     template <int SRC>
@@ -379,6 +386,60 @@ namespace llamql
         default: gemv_mfma_q4k_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a); break;
         }
         return launched(fn);
+    }
+
+    template <int SRC>
+    void gemv_mfma_q6k_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const Mfma6Args &a)
+    {
+        static bool attr_set = false;
+        if (!attr_set)
+        {
+            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_q6k_kernel<SRC>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            attr_set = true;
+        }
+        hipLaunchKernelGGL(gemv_mfma_q6k_kernel<SRC>, grid, block, lds, st, a);
+    }
+
+    inline bool gemv_mfma_q6k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
+                                     int K, int ldy, int device_id, hipStream_t st)
+    {
+        const int SB = K / 256;
+        const Mfma6Shape sh = gemv_mfma6_shape(N, SB, cu_count(device_id));
+        Mfma6Args a;
+        a.w = static_cast<const uint8_t *>(d_w);
+        a.q8 = static_cast<const uint32_t *>(src.q8);
+        a.x = src.x;
+        a.x2 = src.x2;
+        a.ldx = src.ldx;
+        a.y = d_y;
+        a.ldy = ldy;
+        a.N = N;
+        a.SB = SB;
+        a.M = M;
+        a.slices = sh.slices;
+        a.tiles = sh.tiles;
+        a.chunk = sh.chunk;
+        const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles + MFMA6_PRODUCERS) * WAVE);
+        const size_t lds = mfma6_lds_bytes(SB, sh.chunk);
+        switch (src.kind)
+        {
+        case ACT_SRC_F32: gemv_mfma_q6k_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;
+        case ACT_SRC_SWIGLU: gemv_mfma_q6k_launch_src<QUAD_SRC_SWIGLU>(grid, block, lds, st, a); break;
+        default: gemv_mfma_q6k_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a); break;
+        }
+        return launched(fn);
+    }
+
+    // The matrix-unit kernel of format F (mfma_eligible<F> has said yes).
+    template <class F>
+    bool gemv_mfma_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N, int K,
+                          int ldy, int device_id, hipStream_t st)
+    {
+        if constexpr (std::is_same<typename F::Quad, Q6KQuad>::value)
+            return gemv_mfma_q6k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st);
+        else
+            return gemv_mfma_q4k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st);
     }
 
     static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU,
@@ -511,7 +572,7 @@ namespace llamql
         const bool dump = d_sums != nullptr;
         if constexpr (F::USE_MFMA_BATCH)
             if (!dump && mfma_eligible<F>(M, N, K))
-                return gemv_mfma_q4k_launch(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st);
+                return gemv_mfma_launch<F>(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st);
         // Rows of at least 16 super-blocks in a format with a quad-lane decoder: the
         // quad kernel, which stages whole activation rows (up to 160 KiB of LDS).
         if constexpr (F::USE_QUAD)

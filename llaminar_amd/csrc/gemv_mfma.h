@@ -54,7 +54,7 @@ namespace llamql
     // blocks start four banks apart, so the staging writes do not collide) and
     // 2 x {d[4], sum*d[4]}
     constexpr int MFMA_AQ_STRIDE = 256 + 16;
-    inline size_t mfma_act_bytes(int nsb) { return (size_t)nsb * 8 * (MFMA_AQ_STRIDE + 64); }
+    __host__ __device__ inline size_t mfma_act_bytes(int nsb) { return (size_t)nsb * 8 * (MFMA_AQ_STRIDE + 64); }
     inline size_t mfma_lds_bytes(int nsb, int waves) { return mfma_act_bytes(nsb) + (size_t)waves * MFMA_BOUNCE; }
 
     // pieces l, l+64, .., l+256 of a step, as loaded
@@ -91,6 +91,80 @@ namespace llamql
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
+    // Activation blocks kb0 .. kb0+nkb of all M rows into LDS, by `nthreads` threads (tid among
+    // them): aq[kb][8 rows][32 int8] (stride MFMA_AQ_STRIDE) and asc[kb][2 halves][d x4, sum*d x4].
+    // nkb_row: blocks in a whole activation row.
+    template <int SRC>
+    __device__ __forceinline__ void mfma_stage_acts(const uint32_t *q8, const float *x, const float *x2, int ldx, int M,
+                                                    int nkb_row, int kb0, int nkb, uint8_t *aq, float *asc, int tid,
+                                                    int nthreads)
+    {
+        if constexpr (SRC == QUAD_SRC_Q8)
+        {
+            // one thread per Q8_1 block, three blocks in flight per thread: the latency of a
+            // round trip is paid per batch of loads, not per block
+            constexpr int UN = 3;
+            const int total = M * nkb;
+            for (int i0 = tid; i0 < total; i0 += UN * nthreads)
+            {
+                uint32_t v[UN][9];
+#pragma unroll
+                for (int u = 0; u < UN; ++u)
+                {
+                    const int idx = min(i0 + u * nthreads, total - 1);
+                    const int m = idx / nkb, kb = idx - m * nkb;
+                    const uint32_t *src = q8 + ((size_t)m * nkb_row + kb0 + kb) * 9;
+#pragma unroll
+                    for (int i = 0; i < 9; ++i)
+                        v[u][i] = src[i];
+                }
+#pragma unroll
+                for (int u = 0; u < UN; ++u)
+                {
+                    const int idx = i0 + u * nthreads;
+                    if (idx < total)
+                    {
+                        const int m = idx / nkb, kb = idx - m * nkb;
+                        const float d = h2f((uint16_t)(v[u][0] & 0xFFFFu));
+                        uint4 *dst = reinterpret_cast<uint4 *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32);
+                        dst[0] = make_uint4(v[u][1], v[u][2], v[u][3], v[u][4]);
+                        dst[1] = make_uint4(v[u][5], v[u][6], v[u][7], v[u][8]);
+                        float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
+                        sc[0] = d;
+                        sc[4] = (float)(int16_t)(v[u][0] >> 16) * d;
+                    }
+                }
+            }
+        }
+        else
+        {
+            // eight neighbouring threads quantise one 32-element block (the stand-alone
+            // quantiser's arithmetic)
+            const int nvec = nkb * 8;
+            for (int m = 0; m < M; ++m)
+            {
+                const float4 *xr = reinterpret_cast<const float4 *>(x + (size_t)m * ldx) + (size_t)kb0 * 8;
+                const float4 *xr2 = reinterpret_cast<const float4 *>(x2 + (size_t)m * ldx) + (size_t)kb0 * 8;
+                for (int i = tid; i < nvec; i += nthreads) // whole 8-thread groups stay together
+                {
+                    float4 v = xr[i];
+                    if constexpr (SRC == QUAD_SRC_SWIGLU)
+                        v = swiglu4(v, xr2[i]);
+                    const Q8Lane q = q8_1_quantize_lane(v);
+                    const int kb = i >> 3, sub = i & 7;
+                    *reinterpret_cast<uint32_t *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32 + sub * 4) = q.packed;
+                    if (sub == 0)
+                    {
+                        const float d = h2f((uint16_t)(q.head & 0xFFFFu));
+                        float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
+                        sc[0] = d;
+                        sc[4] = (float)(int16_t)(q.head >> 16) * d;
+                    }
+                }
+            }
+        }
     }
 
     // SRC: where the activations come from (QUAD_SRC_*): Q8_1 blocks, or fp32 rows quantised here.
@@ -154,69 +228,7 @@ namespace llamql
         issue(bufB, 1);
 
         // ---- activations into LDS ------------------------------------------------------------
-        if constexpr (SRC == QUAD_SRC_Q8)
-        {
-            // one thread per Q8_1 block, three blocks in flight per thread: the latency of a
-            // round trip is paid per batch of loads, not per block
-            constexpr int UN = 3;
-            const int total = a.M * nkb;
-            for (int i0 = threadIdx.x; i0 < total; i0 += UN * (int)blockDim.x)
-            {
-                uint32_t v[UN][9];
-#pragma unroll
-                for (int u = 0; u < UN; ++u)
-                {
-                    const int idx = min(i0 + u * (int)blockDim.x, total - 1);
-                    const uint32_t *src = a.q8 + (size_t)idx * 9;
-#pragma unroll
-                    for (int i = 0; i < 9; ++i)
-                        v[u][i] = src[i];
-                }
-#pragma unroll
-                for (int u = 0; u < UN; ++u)
-                {
-                    const int idx = i0 + u * (int)blockDim.x;
-                    if (idx < total)
-                    {
-                        const int m = idx / nkb, kb = idx - m * nkb;
-                        const float d = h2f((uint16_t)(v[u][0] & 0xFFFFu));
-                        uint4 *dst = reinterpret_cast<uint4 *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32);
-                        dst[0] = make_uint4(v[u][1], v[u][2], v[u][3], v[u][4]);
-                        dst[1] = make_uint4(v[u][5], v[u][6], v[u][7], v[u][8]);
-                        float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
-                        sc[0] = d;
-                        sc[4] = (float)(int16_t)(v[u][0] >> 16) * d;
-                    }
-                }
-            }
-        }
-        else
-        {
-            // eight neighbouring threads quantise one 32-element block (the stand-alone
-            // quantiser's arithmetic)
-            const int nvec = nkb * 8;
-            for (int m = 0; m < a.M; ++m)
-            {
-                const float4 *xr = reinterpret_cast<const float4 *>(a.x + (size_t)m * a.ldx);
-                const float4 *xr2 = reinterpret_cast<const float4 *>(a.x2 + (size_t)m * a.ldx);
-                for (int i = threadIdx.x; i < nvec; i += blockDim.x) // whole 8-thread groups stay together
-                {
-                    float4 v = xr[i];
-                    if constexpr (SRC == QUAD_SRC_SWIGLU)
-                        v = swiglu4(v, xr2[i]);
-                    const Q8Lane q = q8_1_quantize_lane(v);
-                    const int kb = i >> 3, sub = i & 7;
-                    *reinterpret_cast<uint32_t *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32 + sub * 4) = q.packed;
-                    if (sub == 0)
-                    {
-                        const float d = h2f((uint16_t)(q.head & 0xFFFFu));
-                        float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
-                        sc[0] = d;
-                        sc[4] = (float)(int16_t)(q.head >> 16) * d;
-                    }
-                }
-            }
-        }
+        mfma_stage_acts<SRC>(a.q8, a.x, a.x2, a.ldx, a.M, nkb, 0, nkb, aq, asc, (int)threadIdx.x, (int)blockDim.x);
         __syncthreads();
         mfma_keep(bufA); // the staging code must not reuse the registers of the loads in flight
         mfma_keep(bufB);

@@ -1,0 +1,346 @@
+// Q6_K x Q8_1 decode GEMV for batches of 5..8 activation rows on the matrix unit.
+//
+// The exact 8.8 fixed-point requantisation of the 6-bit weights is what a Q6_K product costs
+// (several vector instructions per weight).  The quad-lane kernel keeps four activation rows
+// in LDS at most when the row is long, so a batch of eight pays that requantisation twice.
+// Here every weight is requantised once: lane (r = l%32, h = l/32) turns elements
+// 16h..16h+15 of each 32-column block of weight row r into int8 (one Q6_K sub-scale covers
+// exactly those 16 elements) and hands them to v_mfma_i32_32x32x32_i8 as the B operand; the A
+// operand is the batch's activations from LDS, the result the reference's per-block int32
+// sums of rows 4h..4h+3, rescaled in fp32 in ascending block order (gemv_mfma.h has the
+// operand layout).
+//
+// Long rows do not fit the LDS (K = 25600, eight rows: 269 KB): the row is walked in chunks
+// of at most 30 super-blocks, staged alternately into two LDS buffers by two producer
+// wavefronts of the workgroup while the compute wavefronts work on the other buffer -- one
+// barrier per chunk.  The compute wavefronts of a 32-row tile share the super-blocks round
+// robin (wavefront j takes j, j + slices, ..); with the chunk a multiple of `slices` that
+// sequence does not depend on the chunking.  Their partial sums are added in wavefront order.
+//
+// The planes of the prepared Q6_K layout suit this access: the 128 bytes of ql of a
+// super-block are one cache line, read by the two lanes of a row with four loads each.
+#pragma once
+#include "gemv_mfma.h"
+
+namespace llamql
+{
+    constexpr int MFMA6_PRODUCERS = 2;     // wavefronts that only stage activations
+    constexpr int MFMA6_MAX_COMPUTE = 10;  // compute wavefronts per workgroup
+    constexpr int MFMA6_LOADS = 8;         // vector memory loads per super-block and lane
+    constexpr int MFMA6_MAX_CHUNK = 30;    // super-blocks per LDS buffer when two are needed
+
+    struct Mfma6Args
+    {
+        const uint8_t *w;   // prepared Q6_K planes: ql | qh | scales | d over all N*SB super-blocks
+        const uint32_t *q8; // Q8_1 activations as dwords (QUAD_SRC_Q8)
+        const float *x;     // fp32 rows (QUAD_SRC_F32); the gate rows for QUAD_SRC_SWIGLU
+        const float *x2;    // the up rows for QUAD_SRC_SWIGLU
+        int ldx;
+        float *y;
+        int ldy;
+        int N;
+        int SB;     // super-blocks per weight row
+        int M;      // activation rows, 1..8
+        int slices; // compute wavefronts per 32-row tile
+        int tiles;  // tiles per workgroup
+        int chunk;  // super-blocks per activation buffer; a multiple of slices when SB > chunk
+    };
+
+    struct Mfma6Raw
+    {
+        v4i ql0, ql1, ql2, ql3, qh0, qh1, sc;
+        int d;
+    };
+    struct Mfma6Ptr
+    {
+        const uint8_t *ql, *qh, *sc, *d; // plane bases (uniform)
+    };
+    // t: the lane's super-block index (row * SB + sb); h: its half of every block
+    __device__ __forceinline__ void mfma6_load(Mfma6Raw &r, const Mfma6Ptr &p, uint32_t t, uint32_t h)
+    {
+        const uint32_t oql = t * 128u + 16u * h, oqh = t * 64u + 16u * h, osc = t * 16u, od = t * 2u;
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.ql0) : "v"(oql), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:32" : "=&v"(r.ql1) : "v"(oql), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:64" : "=&v"(r.ql2) : "v"(oql), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:96" : "=&v"(r.ql3) : "v"(oql), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qh0) : "v"(oqh), "s"(p.qh));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:32" : "=&v"(r.qh1) : "v"(oqh), "s"(p.qh));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.sc) : "v"(osc), "s"(p.sc));
+        asm volatile("global_load_ushort %0, %1, %2" : "=&v"(r.d) : "v"(od), "s"(p.d));
+    }
+    __device__ __forceinline__ void mfma6_keep(Mfma6Raw &r)
+    {
+        asm volatile(""
+                     : "+v"(r.ql0), "+v"(r.ql1), "+v"(r.ql2), "+v"(r.ql3), "+v"(r.qh0), "+v"(r.qh1), "+v"(r.sc),
+                       "+v"(r.d));
+    }
+    template <int NEWER>
+    __device__ __forceinline__ void mfma6_wait(Mfma6Raw &r)
+    {
+        asm volatile("s_waitcnt vmcnt(%8)"
+                     : "+v"(r.ql0), "+v"(r.ql1), "+v"(r.ql2), "+v"(r.ql3), "+v"(r.qh0), "+v"(r.qh1), "+v"(r.sc),
+                       "+v"(r.d)
+                     : "n"(NEWER));
+    }
+
+    // Workgroup barrier of a compute wavefront: its own LDS reads are done (their results have
+    // been consumed), and it must NOT wait for its weight loads in flight, which a
+    // __syncthreads() would.  The producers publish their LDS writes with __syncthreads().
+    __device__ __forceinline__ void mfma6_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+    inline size_t mfma6_lds_bytes(int nsb, int chunk) { return mfma_act_bytes(chunk) * (nsb > chunk ? 2 : 1); }
+
+    template <int SRC>
+    __global__ void __launch_bounds__((MFMA6_MAX_COMPUTE + MFMA6_PRODUCERS) * WAVE)
+        gemv_mfma_q6k_kernel(const Mfma6Args a)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t mfma6_lds[];
+        const int nsb = a.SB;
+        const int nph = (nsb + a.chunk - 1) / a.chunk; // activation chunks
+        const size_t buf_bytes = mfma_act_bytes(a.chunk);
+        const int ncomp = a.slices * a.tiles; // compute wavefronts
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+        auto buf_aq = [&](int ph) { return mfma6_lds + (size_t)(ph & 1) * buf_bytes; };
+        auto buf_asc = [&](int ph) {
+            return reinterpret_cast<float *>(mfma6_lds + (size_t)(ph & 1) * buf_bytes + (size_t)a.chunk * 8 * MFMA_AQ_STRIDE);
+        };
+
+        // chunk ph into its buffer, by `nthreads` threads
+        auto stage = [&](int ph, int tid, int nthreads) {
+            const int c0 = ph * a.chunk;
+            const int c1 = c0 + a.chunk < nsb ? c0 + a.chunk : nsb;
+            mfma_stage_acts<SRC>(a.q8, a.x, a.x2, a.ldx, a.M, nsb * 8, c0 * 8, (c1 - c0) * 8, buf_aq(ph), buf_asc(ph), tid,
+                                 nthreads);
+        };
+
+        if (wave >= ncomp)
+        {
+            // ---- producers: the first chunk together with everybody, then chunk ph+1 into the
+            // buffer nobody reads during chunk ph ------------------------------------------------
+            stage(0, (int)threadIdx.x, (int)blockDim.x);
+            __syncthreads();
+            for (int ph = 0; ph + 1 < nph; ++ph)
+            {
+                stage(ph + 1, (int)threadIdx.x - ncomp * WAVE, MFMA6_PRODUCERS * WAVE);
+                __syncthreads();
+            }
+        }
+        else
+        {
+            // ---- compute wavefronts --------------------------------------------------------------
+            const int l32 = lane & 31, lh = lane >> 5;
+            const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
+            const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
+            const int last_step = nsteps > 0 ? nsteps - 1 : 0;
+            const long row = ((long)blockIdx.x * a.tiles + tile_local) * MFMA_TILE_ROWS + l32;
+            const long row_ld = row < a.N ? row : a.N - 1; // rows past the end re-read the last one
+            const uint32_t t_row = (uint32_t)(row_ld * nsb);
+            const size_t T = (size_t)a.N * nsb;
+            Mfma6Ptr pl;
+            pl.ql = a.w;
+            pl.qh = a.w + T * 128;
+            pl.sc = a.w + T * 192;
+            pl.d = a.w + T * 208;
+
+            // loads are never predicated: past its last step a lane re-reads that step
+            auto issue = [&](Mfma6Raw &r, int step) {
+                const int sb = nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0;
+                mfma6_load(r, pl, t_row + (uint32_t)sb, (uint32_t)lh);
+            };
+            Mfma6Raw bufA, bufB;
+            issue(bufA, 0);
+            issue(bufB, 1);
+            stage(0, (int)threadIdx.x, (int)blockDim.x); // while the first weights are in flight
+            __syncthreads();
+            mfma6_keep(bufA); // the staging code must not reuse the registers of the loads in flight
+            mfma6_keep(bufB);
+
+            v16i zero;
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                zero[i] = 0;
+            const int a_lane = (l32 & 7) * 32 + lh * 16; // rows beyond the batch: any row, result unused
+            int step = 0, cur_ph = 0;
+
+            auto compute = [&](const Mfma6Raw &r) {
+                const int sb = slice + step * a.slices;
+                const int ph = sb / a.chunk;
+                while (cur_ph < ph) // uniform: wait until the chunk this step needs has been staged
+                {
+                    mfma6_barrier();
+                    ++cur_ph;
+                }
+                const int kb0 = (sb - ph * a.chunk) * 8;
+                const uint8_t *ab = buf_aq(ph) + (size_t)kb0 * MFMA_AQ_STRIDE + a_lane;
+                const float *sb_sc = buf_asc(ph) + (size_t)kb0 * 16 + lh * 8;
+                const float d = h2f((uint16_t)r.d);
+                const v4i ql[4] = {r.ql0, r.ql1, r.ql2, r.ql3};
+                const v4i qh[2] = {r.qh0, r.qh1};
+                const uint32_t k4 = 0x0F0F0F0Fu, k2 = 0x03030303u;
+                // The factors of a block need both its sub-scales and two divisions: the lane of
+                // half h works them out for blocks 4h..4h+3 and passes the other half's factor
+                // and the block scale to the lane of that half (lane ^ 32).
+                uint32_t fc[8]; // this lane's factor (low half-word) and constant 128 - 32 f
+                float bsc[8];
+                {
+                    const int sc_lo = lh ? r.sc.z : r.sc.x, sc_hi = lh ? r.sc.w : r.sc.y;
+                    uint32_t mine[4], theirs[4];
+                    float bmine[4];
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                    {
+                        const int sdw = (s >> 1) ? sc_hi : sc_lo;
+                        const int s0 = __builtin_amdgcn_sbfe(sdw, 16u * (s & 1), 8u);
+                        const int s1 = __builtin_amdgcn_sbfe(sdw, 16u * (s & 1) + 8u, 8u);
+                        Q6KQuad::v2s f0, c0, f1, c1;
+                        Q6KQuad::block_factors(s0, s1, d, f0, c0, f1, c1, bmine[s]);
+                        const uint32_t p0 = (uint32_t)f0.x | ((uint32_t)c0.x << 16);
+                        const uint32_t p1 = (uint32_t)f1.x | ((uint32_t)c1.x << 16);
+                        mine[s] = lh ? p1 : p0;
+                        theirs[s] = lh ? p0 : p1;
+                    }
+                    const int partner = (lane ^ 32) * 4;
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                    {
+                        const uint32_t got = (uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)theirs[s]);
+                        const float bgot = __builtin_bit_cast(
+                            float, __builtin_amdgcn_ds_bpermute(partner, __builtin_bit_cast(int, bmine[s])));
+                        // blocks 0..3 were worked out by half 0, blocks 4..7 by half 1
+                        fc[s] = lh ? got : mine[s];
+                        fc[4 + s] = lh ? mine[s] : got;
+                        bsc[s] = lh ? bgot : bmine[s];
+                        bsc[4 + s] = lh ? bmine[s] : bgot;
+                    }
+                }
+                // block j = 4n + s: nibbles of ql piece (n, s & 1), low for s < 2, high otherwise;
+                // bits 2s, 2s+1 of qh piece n; sub-scales 8n + 2s and 8n + 2s + 1
+                auto product = [&](int j, float &bscale) {
+                    const int n = j >> 2, s = j & 3;
+                    bscale = bsc[j];
+                    const Q6KQuad::v2s ff = __builtin_bit_cast(Q6KQuad::v2s, __builtin_amdgcn_perm(fc[j], fc[j], 0x01000100u));
+                    const Q6KQuad::v2s cc = __builtin_bit_cast(Q6KQuad::v2s, __builtin_amdgcn_perm(fc[j], fc[j], 0x03020302u));
+                    const v4i lo = ql[2 * n + (s & 1)], hi = qh[n];
+                    auto q4 = [&](int l, int h) {
+                        const uint32_t nib = (s >= 2 ? (uint32_t)l >> 4 : (uint32_t)l) & k4;
+                        const uint32_t q = nib | ((((uint32_t)h >> (2 * s)) & k2) << 4);
+                        return Q6KQuad::requant4(q, ff, cc); // f == 0 (both sub-scales 0) yields 0 bytes
+                    };
+                    const v4i w = {q4(lo.x, hi.x), q4(lo.y, hi.y), q4(lo.z, hi.z), q4(lo.w, hi.w)};
+                    const v4i av = *reinterpret_cast<const v4i *>(ab + j * MFMA_AQ_STRIDE);
+                    return __builtin_amdgcn_mfma_i32_32x32x32_i8(av, w, zero, 0, 0, 0);
+                };
+                // the product of block j+1 is issued before block j is rescaled
+                v16i idot[2];
+                float bs[2];
+                idot[0] = product(0, bs[0]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                {
+                    if (j + 1 < 8)
+                        idot[(j + 1) & 1] = product(j + 1, bs[(j + 1) & 1]);
+                    const float4 ad = *reinterpret_cast<const float4 *>(sb_sc + j * 16);
+                    const v16i dd = idot[j & 1];
+                    const float b = bs[j & 1];
+                    acc[0] = fmaf((float)dd[0], ad.x * b, acc[0]);
+                    acc[1] = fmaf((float)dd[1], ad.y * b, acc[1]);
+                    acc[2] = fmaf((float)dd[2], ad.z * b, acc[2]);
+                    acc[3] = fmaf((float)dd[3], ad.w * b, acc[3]);
+                }
+                ++step;
+            };
+
+            // Two buffers alternate; each is reloaded (two steps ahead) once it has been consumed.
+            // Every buffer is waited for, also past the end: a register whose load is still in
+            // flight must not look free to the compiler.
+            for (int c0 = 0; c0 < nsteps; c0 += 2)
+            {
+                mfma6_wait<MFMA6_LOADS>(bufA);
+                if (step < nsteps) // uniform
+                    compute(bufA);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufA, c0 + 2);
+                mfma6_wait<MFMA6_LOADS>(bufB);
+                if (step < nsteps)
+                    compute(bufB);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufB, c0 + 3);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end
+            mfma6_keep(bufA);
+            mfma6_keep(bufB);
+            while (cur_ph < nph - 1) // the barriers of chunks this wavefront had no part in
+            {
+                mfma6_barrier();
+                ++cur_ph;
+            }
+        }
+
+        // ---- partial sums of the slices, added in slice order -------------------------------------
+        __syncthreads(); // every wavefront is done with the activations
+        float *red = reinterpret_cast<float *>(mfma6_lds); // [compute wavefront][4][64]
+        if (wave < ncomp)
+        {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                red[(wave * 4 + i) * WAVE + lane] = acc[i];
+        }
+        __syncthreads();
+        if (wave < ncomp)
+        {
+            const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
+            const long row = ((long)blockIdx.x * a.tiles + tile_local) * MFMA_TILE_ROWS + (lane & 31);
+            if (slice == 0)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    float v = acc[i];
+                    for (int s = 1; s < a.slices; ++s)
+                        v += red[((wave + s) * 4 + i) * WAVE + lane];
+                    const int m = 4 * (lane >> 5) + i;
+                    if (m < a.M && row < a.N)
+                        a.y[(size_t)m * a.ldy + row] = v;
+                }
+            }
+        }
+    }
+
+    struct Mfma6Shape
+    {
+        int slices, tiles, chunk;
+        long grid;
+    };
+    // Slices so that a compute unit sees about ten compute wavefronts, five at least (the
+    // scales of eight neighbouring super-blocks share a cache line) and each two steps long;
+    // tiles per workgroup to fill its ten compute wavefronts when there are tiles to spare.
+    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus)
+    {
+        const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
+        long want = ((long)cus * MFMA6_MAX_COMPUTE + tiles - 1) / tiles;
+        if (want < 5)
+            want = 5;
+        if (want > MFMA6_MAX_COMPUTE)
+            want = MFMA6_MAX_COMPUTE;
+        if (want > nsb / 2)
+            want = nsb / 2;
+        if (want < 1)
+            want = 1;
+        Mfma6Shape sh;
+        sh.slices = (int)want;
+        int t = 1;
+        while ((t * 2) * sh.slices <= MFMA6_MAX_COMPUTE && tiles / (t * 2) >= 2L * cus)
+            t *= 2;
+        sh.tiles = t;
+        sh.grid = (tiles + t - 1) / t;
+        // one buffer if the whole row fits half the LDS, else two of a whole number of rounds
+        if (mfma_act_bytes(nsb) * 2 <= QUAD_MAX_LDS)
+            sh.chunk = nsb;
+        else
+            sh.chunk = (MFMA6_MAX_CHUNK / sh.slices) * sh.slices;
+        return sh;
+    }
+} // namespace llamql

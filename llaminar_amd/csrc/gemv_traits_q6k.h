@@ -50,7 +50,7 @@ namespace llamql
         static constexpr bool PAIR = true;
         static constexpr bool HAS_MIN = false; // the reference's mins plane is all zero for Q6_K
         static constexpr bool USE_QUAD = true;        // quad-lane kernel for rows of >= 16 super-blocks
-        static constexpr bool USE_MFMA_BATCH = false;  // matrix-unit kernel for 5..8 activation rows
+        static constexpr bool USE_MFMA_BATCH = true;   // matrix-unit kernel for 5..8 activation rows
         typedef Q6KQuad Quad;
         static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
         static constexpr int TABLE_BYTES = 0;

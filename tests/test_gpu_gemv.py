@@ -318,3 +318,37 @@ def test_q4k_long_rows_all_batches(capi, dev, oracle, N, K):
             assert rel_err(y.cpu().numpy(), C[:3]) <= TOL[fmt] * 1e-2, rpw
     finally:
         lib.llam_ql_reset_gemv_tuning()
+
+
+@pytest.mark.parametrize("N,K", [(19, 25600), (70, 17408), (33, 30720)])
+def test_q6k_long_rows_large_batches(capi, dev, oracle, N, K):
+    """Q6_K rows too long for eight activation rows in LDS: batches the quad-lane kernel would
+    split run on the matrix unit in one pass, the row walked in chunks staged by producer
+    wavefronts (K = 17408 and 30720: the last chunk is short; N = 19: one partial tile).  Same
+    block sums, blocks added in ascending order per wavefront: values agree with the oracle and
+    with the single-row result up to the association of the fp32 sum, a row does not depend on
+    the batch it rides in, and fp32 input quantised inside the kernel gives the same bits."""
+    import torch
+
+    fmt = FMT_Q6_K
+    W = synth.weights_numpy(fmt, N, K, 91 + N)
+    x = synth.activations_numpy(8, K, 17 + N)
+    q8 = oracle.quantize(x)
+    wd = upload_weights(capi, dev, fmt, W)
+    qd = upload_q8(dev, q8)
+    xd = torch.from_numpy(x).to(dev)
+    C = oracle.gemm(fmt, W, K, q8)
+    y1 = [capi.gemv(fmt, wd, upload_q8(dev, q8[m:m + 1]), 1, N, K) for m in range(8)]
+    ys = {}
+    for M in (4, 5, 7, 8):
+        y = capi.gemv(fmt, wd, qd, M, N, K)
+        sync()
+        ys[M] = y
+        assert rel_err(y.cpu().numpy(), C[:M]) <= TOL[fmt] * 1e-2, M
+        for m in range(M):
+            assert rel_err(y[m].cpu().numpy(), y1[m][0].cpu().numpy()) <= TOL[fmt] * 1e-2, (M, m)
+        assert torch.equal(capi.gemv(fmt, wd, qd, M, N, K), y), M  # bitwise repeatable
+        assert torch.equal(capi.gemv_f32(fmt, wd, xd[:M], M, N, K), y), (M, "fp32 input, no scratch")
+    if K >= 25600:  # seven rows of a shorter row still fit the quad-lane kernel's LDS
+        assert torch.equal(ys[8][:7], ys[7])
+    sync()
