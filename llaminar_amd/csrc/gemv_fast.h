@@ -421,7 +421,7 @@ namespace llamql
         a.tiles = sh.tiles;
         a.chunk = sh.chunk;
         const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles + MFMA6_PRODUCERS) * WAVE);
-        const size_t lds = mfma6_lds_bytes(SB, sh.chunk);
+        const size_t lds = mfma6_lds_bytes(SB, sh.chunk, sh.slices * sh.tiles);
         switch (src.kind)
         {
         case ACT_SRC_F32: gemv_mfma_q6k_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;

@@ -95,17 +95,17 @@ namespace llamql
 
     // Activation blocks kb0 .. kb0+nkb of all M rows into LDS, by `nthreads` threads (tid among
     // them): aq[kb][8 rows][32 int8] (stride MFMA_AQ_STRIDE) and asc[kb][2 halves][d x4, sum*d x4].
-    // nkb_row: blocks in a whole activation row.
-    template <int SRC>
+    // nkb_row: blocks in a whole activation row.  UN: loads a thread keeps in flight (Q8_1
+    // blocks, or 16-byte pieces of fp32 rows): the latency of a round trip is paid per batch of
+    // loads, so few threads staging much want a large UN.
+    template <int SRC, int UN = 3>
     __device__ __forceinline__ void mfma_stage_acts(const uint32_t *q8, const float *x, const float *x2, int ldx, int M,
                                                     int nkb_row, int kb0, int nkb, uint8_t *aq, float *asc, int tid,
                                                     int nthreads)
     {
         if constexpr (SRC == QUAD_SRC_Q8)
         {
-            // one thread per Q8_1 block, three blocks in flight per thread: the latency of a
-            // round trip is paid per batch of loads, not per block
-            constexpr int UN = 3;
+            // one thread per Q8_1 block
             const int total = M * nkb;
             for (int i0 = tid; i0 < total; i0 += UN * nthreads)
             {
@@ -141,26 +141,42 @@ namespace llamql
         else
         {
             // eight neighbouring threads quantise one 32-element block (the stand-alone
-            // quantiser's arithmetic)
-            const int nvec = nkb * 8;
-            for (int m = 0; m < M; ++m)
+            // quantiser's arithmetic); pieces of all rows are dealt round robin, whole 8-thread
+            // groups stay together (nthreads and the pieces of a row are multiples of 8)
+            constexpr int UF = UN < 4 ? UN : 4;
+            const int nvec = nkb * 8, total = M * nvec;
+            for (int i0 = tid; i0 < total; i0 += UF * nthreads)
             {
-                const float4 *xr = reinterpret_cast<const float4 *>(x + (size_t)m * ldx) + (size_t)kb0 * 8;
-                const float4 *xr2 = reinterpret_cast<const float4 *>(x2 + (size_t)m * ldx) + (size_t)kb0 * 8;
-                for (int i = tid; i < nvec; i += nthreads) // whole 8-thread groups stay together
+                float4 v[UF], v2[UF];
+#pragma unroll
+                for (int u = 0; u < UF; ++u)
                 {
-                    float4 v = xr[i];
+                    const int idx = min(i0 + u * nthreads, total - 8 + (tid & 7)); // past the end: the last block again
+                    const int m = idx / nvec, i = idx - m * nvec;
+                    v[u] = (reinterpret_cast<const float4 *>(x + (size_t)m * ldx) + (size_t)kb0 * 8)[i];
                     if constexpr (SRC == QUAD_SRC_SWIGLU)
-                        v = swiglu4(v, xr2[i]);
-                    const Q8Lane q = q8_1_quantize_lane(v);
-                    const int kb = i >> 3, sub = i & 7;
-                    *reinterpret_cast<uint32_t *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32 + sub * 4) = q.packed;
-                    if (sub == 0)
+                        v2[u] = (reinterpret_cast<const float4 *>(x2 + (size_t)m * ldx) + (size_t)kb0 * 8)[i];
+                }
+#pragma unroll
+                for (int u = 0; u < UF; ++u)
+                {
+                    const int idx = i0 + u * nthreads;
+                    float4 w = v[u];
+                    if constexpr (SRC == QUAD_SRC_SWIGLU)
+                        w = swiglu4(w, v2[u]);
+                    const Q8Lane q = q8_1_quantize_lane(w); // exchanges with the 7 neighbours: no divergence before it
+                    if (idx < total)
                     {
-                        const float d = h2f((uint16_t)(q.head & 0xFFFFu));
-                        float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
-                        sc[0] = d;
-                        sc[4] = (float)(int16_t)(q.head >> 16) * d;
+                        const int m = idx / nvec, i = idx - m * nvec;
+                        const int kb = i >> 3, sub = i & 7;
+                        *reinterpret_cast<uint32_t *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32 + sub * 4) = q.packed;
+                        if (sub == 0)
+                        {
+                            const float d = h2f((uint16_t)(q.head & 0xFFFFu));
+                            float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
+                            sc[0] = d;
+                            sc[4] = (float)(int16_t)(q.head >> 16) * d;
+                        }
                     }
                 }
             }

@@ -17,17 +17,24 @@
 // robin (wavefront j takes j, j + slices, ..); with the chunk a multiple of `slices` that
 // sequence does not depend on the chunking.  Their partial sums are added in wavefront order.
 //
-// The planes of the prepared Q6_K layout suit this access: the 128 bytes of ql of a
-// super-block are one cache line, read by the two lanes of a row with four loads each.
+// Weight loads are coalesced: of the 32 x 128 bytes of ql and 32 x 64 bytes of qh of a step,
+// lane l loads the 16-byte pieces l, l+64, .. (eight neighbouring lanes cover a row's cache
+// line of ql) and the wavefront passes them through a private LDS buffer to the two lanes of
+// the row (rows 144 and 80 bytes apart there, so that the 128-bit reads of neighbouring rows
+// fall into different banks).  The 16 scale bytes and the fp16 d of a row go straight to its
+// two lanes.  No barrier for the buffer: LDS instructions of one wavefront run in order.
 #pragma once
 #include "gemv_mfma.h"
+#include <type_traits>
 
 namespace llamql
 {
     constexpr int MFMA6_PRODUCERS = 2;     // wavefronts that only stage activations
-    constexpr int MFMA6_MAX_COMPUTE = 10;  // compute wavefronts per workgroup
+    constexpr int MFMA6_MAX_COMPUTE = 8;   // compute wavefronts per workgroup
     constexpr int MFMA6_LOADS = 8;         // vector memory loads per super-block and lane
-    constexpr int MFMA6_MAX_CHUNK = 30;    // super-blocks per LDS buffer when two are needed
+    constexpr int MFMA6_QL_STRIDE = 144;   // bounce buffer: bytes between the ql lines of two rows
+    constexpr int MFMA6_QH_STRIDE = 80;    // and between their 64 bytes of qh
+    constexpr int MFMA6_BOUNCE = 32 * (MFMA6_QL_STRIDE + MFMA6_QH_STRIDE); // per compute wavefront
 
     struct Mfma6Args
     {
@@ -51,22 +58,26 @@ namespace llamql
         v4i ql0, ql1, ql2, ql3, qh0, qh1, sc;
         int d;
     };
+    // Plane bases advanced to the step's super-block (wavefront-uniform, scalar registers) and
+    // this lane's byte offsets from them: four pieces of ql, two of qh, its row's scales and d.
     struct Mfma6Ptr
     {
-        const uint8_t *ql, *qh, *sc, *d; // plane bases (uniform)
+        const uint8_t *ql, *qh, *sc, *d;
     };
-    // t: the lane's super-block index (row * SB + sb); h: its half of every block
-    __device__ __forceinline__ void mfma6_load(Mfma6Raw &r, const Mfma6Ptr &p, uint32_t t, uint32_t h)
+    struct Mfma6Off
     {
-        const uint32_t oql = t * 128u + 16u * h, oqh = t * 64u + 16u * h, osc = t * 16u, od = t * 2u;
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.ql0) : "v"(oql), "s"(p.ql));
-        asm volatile("global_load_dwordx4 %0, %1, %2 offset:32" : "=&v"(r.ql1) : "v"(oql), "s"(p.ql));
-        asm volatile("global_load_dwordx4 %0, %1, %2 offset:64" : "=&v"(r.ql2) : "v"(oql), "s"(p.ql));
-        asm volatile("global_load_dwordx4 %0, %1, %2 offset:96" : "=&v"(r.ql3) : "v"(oql), "s"(p.ql));
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qh0) : "v"(oqh), "s"(p.qh));
-        asm volatile("global_load_dwordx4 %0, %1, %2 offset:32" : "=&v"(r.qh1) : "v"(oqh), "s"(p.qh));
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.sc) : "v"(osc), "s"(p.sc));
-        asm volatile("global_load_ushort %0, %1, %2" : "=&v"(r.d) : "v"(od), "s"(p.d));
+        uint32_t ql[4], qh[2], sc, d;
+    };
+    __device__ __forceinline__ void mfma6_load(Mfma6Raw &r, const Mfma6Ptr &p, const Mfma6Off &o)
+    {
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.ql0) : "v"(o.ql[0]), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.ql1) : "v"(o.ql[1]), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.ql2) : "v"(o.ql[2]), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.ql3) : "v"(o.ql[3]), "s"(p.ql));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qh0) : "v"(o.qh[0]), "s"(p.qh));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qh1) : "v"(o.qh[1]), "s"(p.qh));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.sc) : "v"(o.sc), "s"(p.sc));
+        asm volatile("global_load_ushort %0, %1, %2" : "=&v"(r.d) : "v"(o.d), "s"(p.d));
     }
     __device__ __forceinline__ void mfma6_keep(Mfma6Raw &r)
     {
@@ -88,7 +99,14 @@ namespace llamql
     // __syncthreads() would.  The producers publish their LDS writes with __syncthreads().
     __device__ __forceinline__ void mfma6_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-    inline size_t mfma6_lds_bytes(int nsb, int chunk) { return mfma_act_bytes(chunk) * (nsb > chunk ? 2 : 1); }
+    __host__ __device__ inline size_t mfma6_act_bytes(int nsb, int chunk)
+    {
+        return mfma_act_bytes(chunk) * (nsb > chunk ? 2 : 1);
+    }
+    inline size_t mfma6_lds_bytes(int nsb, int chunk, int ncomp)
+    {
+        return mfma6_act_bytes(nsb, chunk) + (size_t)ncomp * MFMA6_BOUNCE;
+    }
 
     template <int SRC>
     __global__ void __launch_bounds__((MFMA6_MAX_COMPUTE + MFMA6_PRODUCERS) * WAVE)
@@ -108,23 +126,26 @@ namespace llamql
             return reinterpret_cast<float *>(mfma6_lds + (size_t)(ph & 1) * buf_bytes + (size_t)a.chunk * 8 * MFMA_AQ_STRIDE);
         };
 
-        // chunk ph into its buffer, by `nthreads` threads
-        auto stage = [&](int ph, int tid, int nthreads) {
+        // chunk ph into its buffer, by `nthreads` threads that keep UN loads in flight each
+        auto stage = [&](int ph, int tid, int nthreads, auto un) {
             const int c0 = ph * a.chunk;
             const int c1 = c0 + a.chunk < nsb ? c0 + a.chunk : nsb;
-            mfma_stage_acts<SRC>(a.q8, a.x, a.x2, a.ldx, a.M, nsb * 8, c0 * 8, (c1 - c0) * 8, buf_aq(ph), buf_asc(ph), tid,
-                                 nthreads);
+            mfma_stage_acts<SRC, decltype(un)::value>(a.q8, a.x, a.x2, a.ldx, a.M, nsb * 8, c0 * 8, (c1 - c0) * 8,
+                                                      buf_aq(ph), buf_asc(ph), tid, nthreads);
         };
+        typedef std::integral_constant<int, 3> Together; // everybody stages the first chunk
+        typedef std::integral_constant<int, 8> Alone;    // two wavefronts stage the others: a chunk of 16
+                                                         // super-blocks is 8 blocks a thread, all in flight
 
         if (wave >= ncomp)
         {
             // ---- producers: the first chunk together with everybody, then chunk ph+1 into the
             // buffer nobody reads during chunk ph ------------------------------------------------
-            stage(0, (int)threadIdx.x, (int)blockDim.x);
+            stage(0, (int)threadIdx.x, (int)blockDim.x, Together());
             __syncthreads();
             for (int ph = 0; ph + 1 < nph; ++ph)
             {
-                stage(ph + 1, (int)threadIdx.x - ncomp * WAVE, MFMA6_PRODUCERS * WAVE);
+                stage(ph + 1, (int)threadIdx.x - ncomp * WAVE, MFMA6_PRODUCERS * WAVE, Alone());
                 __syncthreads();
             }
         }
@@ -135,25 +156,48 @@ namespace llamql
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
             const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
             const int last_step = nsteps > 0 ? nsteps - 1 : 0;
-            const long row = ((long)blockIdx.x * a.tiles + tile_local) * MFMA_TILE_ROWS + l32;
-            const long row_ld = row < a.N ? row : a.N - 1; // rows past the end re-read the last one
-            const uint32_t t_row = (uint32_t)(row_ld * nsb);
+            const long tile_row0 = ((long)blockIdx.x * a.tiles + tile_local) * MFMA_TILE_ROWS;
             const size_t T = (size_t)a.N * nsb;
-            Mfma6Ptr pl;
-            pl.ql = a.w;
-            pl.qh = a.w + T * 128;
-            pl.sc = a.w + T * 192;
-            pl.d = a.w + T * 208;
+            // rows past the end of the matrix re-read the last one
+            auto sb_index = [&](int local_row) {
+                const long r = tile_row0 + local_row;
+                return (uint32_t)((r < a.N ? r : a.N - 1) * nsb);
+            };
+            Mfma6Off off;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) // ql piece lane + 64 i: row (lane >> 3) + 8 i, 16 bytes at 16 (lane & 7)
+                off.ql[i] = sb_index((lane >> 3) + 8 * i) * 128u + 16u * (uint32_t)(lane & 7);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) // qh piece lane + 64 i: row (lane >> 2) + 16 i, 16 bytes at 16 (lane & 3)
+                off.qh[i] = sb_index((lane >> 2) + 16 * i) * 64u + 16u * (uint32_t)(lane & 3);
+            off.sc = sb_index(l32) * 16u;
+            off.d = sb_index(l32) * 2u;
+            uint8_t *bounce = mfma6_lds + mfma6_act_bytes(nsb, a.chunk) + (size_t)wave * MFMA6_BOUNCE;
+            uint8_t *wr_ql = bounce + (lane >> 3) * MFMA6_QL_STRIDE + (lane & 7) * 16;  // piece i at + 8 i rows
+            uint8_t *wr_qh = bounce + 32 * MFMA6_QL_STRIDE + (lane >> 2) * MFMA6_QH_STRIDE + (lane & 3) * 16;
+            const uint8_t *rd_ql = bounce + l32 * MFMA6_QL_STRIDE + 16 * lh;            // piece c at + 32 c
+            const uint8_t *rd_qh = bounce + 32 * MFMA6_QL_STRIDE + l32 * MFMA6_QH_STRIDE + 16 * lh;
 
             // loads are never predicated: past its last step a lane re-reads that step
             auto issue = [&](Mfma6Raw &r, int step) {
-                const int sb = nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0;
-                mfma6_load(r, pl, t_row + (uint32_t)sb, (uint32_t)lh);
+                const uint32_t sb = nsteps > 0 ? (uint32_t)(slice + (step < last_step ? step : last_step) * a.slices) : 0u;
+                auto uniform = [](const uint8_t *p) {
+                    const uint64_t b = (uint64_t)p;
+                    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+                    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+                    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
+                };
+                Mfma6Ptr pl;
+                pl.ql = uniform(a.w + (size_t)sb * 128);
+                pl.qh = uniform(a.w + T * 128 + (size_t)sb * 64);
+                pl.sc = uniform(a.w + T * 192 + (size_t)sb * 16);
+                pl.d = uniform(a.w + T * 208 + (size_t)sb * 2);
+                mfma6_load(r, pl, off);
             };
             Mfma6Raw bufA, bufB;
             issue(bufA, 0);
             issue(bufB, 1);
-            stage(0, (int)threadIdx.x, (int)blockDim.x); // while the first weights are in flight
+            stage(0, (int)threadIdx.x, (int)blockDim.x, Together()); // while the first weights are in flight
             __syncthreads();
             mfma6_keep(bufA); // the staging code must not reuse the registers of the loads in flight
             mfma6_keep(bufB);
@@ -165,7 +209,23 @@ namespace llamql
             const int a_lane = (l32 & 7) * 32 + lh * 16; // rows beyond the batch: any row, result unused
             int step = 0, cur_ph = 0;
 
-            auto compute = [&](const Mfma6Raw &r) {
+            // the coalesced pieces of a step into the bounce buffer; its scales and d stay behind
+            v4i sc_cur;
+            int d_cur;
+            auto stage_w = [&](const Mfma6Raw &r) {
+                mfma_wave_sync(); // the previous step's reads are done
+                *reinterpret_cast<v4i *>(wr_ql) = r.ql0;
+                *reinterpret_cast<v4i *>(wr_ql + 8 * MFMA6_QL_STRIDE) = r.ql1;
+                *reinterpret_cast<v4i *>(wr_ql + 16 * MFMA6_QL_STRIDE) = r.ql2;
+                *reinterpret_cast<v4i *>(wr_ql + 24 * MFMA6_QL_STRIDE) = r.ql3;
+                *reinterpret_cast<v4i *>(wr_qh) = r.qh0;
+                *reinterpret_cast<v4i *>(wr_qh + 16 * MFMA6_QH_STRIDE) = r.qh1;
+                sc_cur = r.sc;
+                d_cur = r.d;
+                mfma_wave_sync();
+            };
+
+            auto compute = [&]() {
                 const int sb = slice + step * a.slices;
                 const int ph = sb / a.chunk;
                 while (cur_ph < ph) // uniform: wait until the chunk this step needs has been staged
@@ -176,9 +236,10 @@ namespace llamql
                 const int kb0 = (sb - ph * a.chunk) * 8;
                 const uint8_t *ab = buf_aq(ph) + (size_t)kb0 * MFMA_AQ_STRIDE + a_lane;
                 const float *sb_sc = buf_asc(ph) + (size_t)kb0 * 16 + lh * 8;
-                const float d = h2f((uint16_t)r.d);
-                const v4i ql[4] = {r.ql0, r.ql1, r.ql2, r.ql3};
-                const v4i qh[2] = {r.qh0, r.qh1};
+                const float d = h2f((uint16_t)d_cur);
+                const v4i ql[4] = {*reinterpret_cast<const v4i *>(rd_ql), *reinterpret_cast<const v4i *>(rd_ql + 32),
+                                   *reinterpret_cast<const v4i *>(rd_ql + 64), *reinterpret_cast<const v4i *>(rd_ql + 96)};
+                const v4i qh[2] = {*reinterpret_cast<const v4i *>(rd_qh), *reinterpret_cast<const v4i *>(rd_qh + 32)};
                 const uint32_t k4 = 0x0F0F0F0Fu, k2 = 0x03030303u;
                 // The factors of a block need both its sub-scales and two divisions: the lane of
                 // half h works them out for blocks 4h..4h+3 and passes the other half's factor
@@ -186,7 +247,7 @@ namespace llamql
                 uint32_t fc[8]; // this lane's factor (low half-word) and constant 128 - 32 f
                 float bsc[8];
                 {
-                    const int sc_lo = lh ? r.sc.z : r.sc.x, sc_hi = lh ? r.sc.w : r.sc.y;
+                    const int sc_lo = lh ? sc_cur.z : sc_cur.x, sc_hi = lh ? sc_cur.w : sc_cur.y;
                     uint32_t mine[4], theirs[4];
                     float bmine[4];
 #pragma unroll
@@ -253,21 +314,28 @@ namespace llamql
                 ++step;
             };
 
-            // Two buffers alternate; each is reloaded (two steps ahead) once it has been consumed.
-            // Every buffer is waited for, also past the end: a register whose load is still in
-            // flight must not look free to the compiler.
+            // Two register buffers alternate; each is reloaded (two steps ahead) as soon as its
+            // pieces are in LDS, before the step is computed.  Every buffer is waited for, also
+            // past the end: a register whose load is still in flight must not look free to the
+            // compiler.
             for (int c0 = 0; c0 < nsteps; c0 += 2)
             {
                 mfma6_wait<MFMA6_LOADS>(bufA);
                 if (step < nsteps) // uniform
-                    compute(bufA);
+                    stage_w(bufA);
                 __builtin_amdgcn_sched_barrier(0);
                 issue(bufA, c0 + 2);
+                if (step < nsteps)
+                    compute();
+                __builtin_amdgcn_sched_barrier(0);
                 mfma6_wait<MFMA6_LOADS>(bufB);
                 if (step < nsteps)
-                    compute(bufB);
+                    stage_w(bufB);
                 __builtin_amdgcn_sched_barrier(0);
                 issue(bufB, c0 + 3);
+                if (step < nsteps)
+                    compute();
+                __builtin_amdgcn_sched_barrier(0);
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end
             mfma6_keep(bufA);
@@ -336,11 +404,16 @@ namespace llamql
             t *= 2;
         sh.tiles = t;
         sh.grid = (tiles + t - 1) / t;
-        // one buffer if the whole row fits half the LDS, else two of a whole number of rounds
-        if (mfma_act_bytes(nsb) * 2 <= QUAD_MAX_LDS)
+        // one buffer if the whole row fits beside the bounce buffers and leaves half the LDS
+        // free, else two buffers of a whole number of rounds of the slices
+        const size_t bounce = (size_t)sh.slices * t * MFMA6_BOUNCE;
+        if (mfma_act_bytes(nsb) * 2 + bounce <= QUAD_MAX_LDS)
             sh.chunk = nsb;
         else
-            sh.chunk = (MFMA6_MAX_CHUNK / sh.slices) * sh.slices;
+        {
+            const int fit = (int)((QUAD_MAX_LDS - bounce) / (2 * mfma_act_bytes(1)));
+            sh.chunk = (fit / sh.slices) * sh.slices;
+        }
         return sh;
     }
 } // namespace llamql
