@@ -7,10 +7,12 @@
 // idot is formed by ONE v_mfma_i32_32x32x32_i8 per 32x32 output tile and K-block
 // (K depth 32 = exactly one Q8_1 block, zero accumulator input), so it is the
 // same exact integer the reference forms with vpdpbusd
-// (CPUNativeVNNIGemv.h:1046-1231); the per-block rescale is fp32 VALU work (three
-// operations per output element and block: convert, scale product, multiply-add --
-// this, not the matrix unit, bounds the kernel) and the rank-1 min term goes
-// through v_mfma_f32_32x32x2f32 straight into the accumulator.
+// (CPUNativeVNNIGemv.h:1046-1231); the per-block rescale is fp32 work: the scale
+// products a_d[m] * b_scale[n] of a block, a rank-1 matrix, come from one
+// v_mfma_f32_32x32x2f32 (exact), convert and multiply-add per output element stay on
+// the vector unit (two operations against 64 int8 MFMA operations: this, not the int8
+// rate of the matrix unit, bounds the kernel), and the rank-1 min term goes through
+// another v_mfma_f32_32x32x2f32 straight into the accumulator.
 //
 // Workgroup: 512 threads = 8 wavefronts, tile 128 tokens x 64 weight rows, 64 KiB
 // of LDS, so two workgroups share a compute unit and one's staging overlaps the
@@ -178,7 +180,7 @@ namespace llamql
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         uint8_t *Al = smem;                             // [BM][STRIDE] activations int8
         uint8_t *Wl = Al + GEMM_BM * GEMM_STRIDE;       // [BN][STRIDE] weights int8
-        float *ad = reinterpret_cast<float *>(Wl + GEMM_BN * GEMM_STRIDE); // [8][SM]
+        float *ad = reinterpret_cast<float *>(Wl + GEMM_BN * GEMM_STRIDE); // [8][SM] a_d / 2
         float *asd = ad + 8 * GEMM_SM;                  // [8][SM]
         float *bs = asd + 8 * GEMM_SM;                  // [8][SN]
         float *bm = bs + 8 * GEMM_SN;                   // [8][SN]
@@ -235,7 +237,7 @@ namespace llamql
                 const uint32_t h = areg.dword(9 * i);
                 const float d = h2f((uint16_t)(h & 0xFFFFu));
                 const int kb = 2 * ap + i;
-                ad[kb * GEMM_SM + am] = d;
+                ad[kb * GEMM_SM + am] = 0.5f * d; // halved for the depth-2 scale product below
                 asd[kb * GEMM_SM + am] = (float)(int16_t)(h >> 16) * d;
                 v4i *dst = reinterpret_cast<v4i *>(Al + am * GEMM_STRIDE + kb * 32);
                 dst[0] = (v4i){(int)areg.dword(9 * i + 1), (int)areg.dword(9 * i + 2), (int)areg.dword(9 * i + 3),
@@ -259,30 +261,39 @@ namespace llamql
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 zero[r] = 0;
+            v16f zerof;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                zerof[r] = 0.0f;
             auto product = [&](int kb) {
                 const v4i bw = *reinterpret_cast<const v4i *>(wrow + kb * 32);
                 const v4i aa = *reinterpret_cast<const v4i *>(arow + kb * 32);
                 return __builtin_amdgcn_mfma_i32_32x32x32_i8(aa, bw, zero, 0, 0, 0);
             };
+            // The scale products a_d[m] * b_scale[n] of a block are a rank-1 matrix: the matrix
+            // unit forms them in the layout of the block sums instead of 16 multiplies per lane.
+            // Its depth of 2 adds (a_d/2) * b_scale twice: exact, both factors are fp16 values.
+            auto scales = [&](int kb) {
+                const float av = ad[kb * GEMM_SM + mtile * 32 + l32]; // a_d / 2
+                const float bv = bs[kb * GEMM_SN + ntile * 32 + l32];
+                return __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, zerof, 0, 0, 0);
+            };
             v16i idot[2];
             idot[0] = product(0);
+            v16f cs = scales(0);
 #pragma unroll
             for (int kb = 0; kb < 8; ++kb)
             {
                 if (kb + 1 < 8)
                     idot[(kb + 1) & 1] = product(kb + 1);
-                const float bscale = bs[kb * GEMM_SN + ntile * 32 + l32];
-                const float *adp = ad + kb * GEMM_SM + mtile * 32 + 4 * lh;
                 const v16i d = idot[kb & 1];
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                {
-                    const float4 a4 = *reinterpret_cast<const float4 *>(adp + 8 * q);
-                    acc[4 * q + 0] = fmaf((float)d[4 * q + 0], a4.x * bscale, acc[4 * q + 0]);
-                    acc[4 * q + 1] = fmaf((float)d[4 * q + 1], a4.y * bscale, acc[4 * q + 1]);
-                    acc[4 * q + 2] = fmaf((float)d[4 * q + 2], a4.z * bscale, acc[4 * q + 2]);
-                    acc[4 * q + 3] = fmaf((float)d[4 * q + 3], a4.w * bscale, acc[4 * q + 3]);
-                }
+                for (int r = 0; r < 16; ++r)
+                    acc[r] = fmaf((float)d[r], cs[r], acc[r]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (kb + 1 < 8)
+                    cs = scales(kb + 1); // the other wavefronts of the unit cover its latency
+                __builtin_amdgcn_sched_barrier(0);
                 if (F::HAS_MIN && (kb & 1))
                 {
                     // rank-2 update over blocks kb-1, kb, straight into the accumulator: lane
