@@ -464,8 +464,15 @@ namespace llamql
             if (msc != 0)
             {
                 f_big = s_big < 0 ? -1016 : 1016; // rne(+-msc*32512 / (msc*32))
-                f_small = (int)rintf(__fdiv_rn((float)s_small * 32512.0f, fm * 32.0f));
-                bscale = f16_round_packer(__fdiv_rn(d * fm * 32.0f, 127.0f));
+                // rne(s_small*32512 / (msc*32)) = rne(s_small*1016 / msc) without a division: the
+                // quotient has a denominator of at most 128, so unless it is a half-integer it lies
+                // 1/256 or more from one and any value within 1e-3 rounds alike; a half-integer is a
+                // float, and one Newton step on the reciprocal reproduces representable quotients.
+                const float num = (float)(s_small * 1016);
+                const float r = __builtin_amdgcn_rcpf(fm);
+                const float q0 = num * r;
+                f_small = (int)rintf(fmaf(fmaf(-fm, q0, num), r, q0));
+                bscale = f16_round_packer(div_by_127(d * fm * 32.0f));
             }
             const int fi0 = big0 ? f_big : f_small, fi1 = big0 ? f_small : f_big;
             const unsigned short u0 = (unsigned short)fi0, u1 = (unsigned short)fi1;

@@ -33,6 +33,18 @@ namespace llamql
         return r;
     }
 
+    // x / 127 as an IEEE division gives it, for the values a Q6_K block scale takes before its
+    // fp16 rounding (x = f32(d) * msc * 32, d any fp16, msc = 1..128: checked exhaustively on the
+    // host): q0 = x * RN(1/127), one correction step through the exact remainder.  Zeros,
+    // infinities and NaN take q0, which has their sign and kind.
+    __device__ __forceinline__ float div_by_127(float x)
+    {
+        const float c = 0x1.020408p-7f;
+        const float q0 = x * c;
+        const float q1 = fmaf(fmaf(-q0, 127.0f, x), c, q0);
+        return __builtin_amdgcn_classf(x, 0x198) ? q1 : q0; // finite and not zero
+    }
+
     // Same rounding for two values at once.  The truncating branch is only needed when a
     // value lies below the fp16 normal range, which real weights almost never produce:
     // one rarely-taken branch (fp16 exponent field 0 or 1 in either result) guards the

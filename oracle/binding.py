@@ -54,6 +54,9 @@ class Oracle:
         L.qlo_epilogue.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]
         L.qlo_moe_route.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
         L.qlo_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_void_p]
+        L.qlo_check_div127.restype = ctypes.c_long
+        L.qlo_check_q6k_factor.restype = ctypes.c_long
+        L.qlo_check_q6k_factor.argtypes = [c_int]
         L.qlo_dequant_row_q4k.argtypes = [c_void_p, c_int, c_void_p]
         L.qlo_rmsnorm.argtypes = [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int]
         L.qlo_rope_inv_freq.argtypes = [c_int, c_float, c_void_p]
@@ -143,6 +146,12 @@ class Oracle:
         probs = np.zeros((T, E), np.float32)
         self.L.qlo_moe_route(_p(logits), T, E, top_k, int(normalize), _p(ids), _p(w), _p(probs))
         return ids, w, probs
+
+    def check_div127(self) -> int:
+        return int(self.L.qlo_check_div127())
+
+    def check_q6k_factor(self, ulps: int) -> int:
+        return int(self.L.qlo_check_q6k_factor(ulps))
 
     def swiglu(self, gate: np.ndarray, up: np.ndarray) -> np.ndarray:
         gate = np.ascontiguousarray(gate, dtype=np.float32)

@@ -435,3 +435,67 @@ void qlo_swiglu(const float *gate, const float *up, int n, float *out)
         out[i] = (g / (1.0f + expf(-g))) * up[i];
     }
 }
+
+/* ---- exhaustive checks of two division-free forms the GPU kernels use ---------------
+ * Both return the number of inputs on which the cheap form differs from the division the
+ * reference performs (SIMDHelpers.h:12023-12204); the tests expect 0.
+ *
+ * x / 127 for x = (f32(d) * msc) * 32, every fp16 d and msc = 1..128 (the Q6_K block scale
+ * before its fp16 rounding): q0 = x * c, r = fma(-q0, 127, x), q1 = fma(r, c, q0) with
+ * c = RN(1/127) -- Markstein's correction step; zero and non-finite x take q0 (sign of zero). */
+long qlo_check_div127(void)
+{
+    const float c = 0x1.020408p-7f;
+    long bad = 0;
+    for (unsigned h = 0; h < 65536u; ++h)
+    {
+        const float d = qlo_f16_to_f32((uint16_t)h);
+        for (int msc = 1; msc <= 128; ++msc)
+        {
+            const float x = d * (float)msc * 32.0f;
+            const float want = x / 127.0f;
+            const float q0 = x * c;
+            const float r = fmaf(-q0, 127.0f, x);
+            const float q1 = fmaf(r, c, q0);
+            const float got = (isfinite(x) && x != 0.0f) ? q1 : q0;
+            uint32_t a, b;
+            memcpy(&a, &want, 4);
+            memcpy(&b, &got, 4);
+            if (a != b && !(want != want && got != got))
+                ++bad;
+        }
+    }
+    return bad;
+}
+
+/* nearbyint(s * 32512 / (msc * 32)) for |s| <= msc <= 128 (the 8.8 factor of the smaller
+ * sub-scale) against rint of one Newton step on s * 1016 * r, for EVERY r within `ulps`
+ * units in the last place of the correctly rounded 1/msc (the GPU's reciprocal instruction
+ * is accurate to one).                                                                    */
+long qlo_check_q6k_factor(int ulps)
+{
+    long bad = 0;
+    for (int msc = 1; msc <= 128; ++msc)
+    {
+        const float fm = (float)msc;
+        const float r0 = 1.0f / fm;
+        for (int u = -ulps; u <= ulps; ++u)
+        {
+            float r = r0;
+            for (int i = 0; i < (u < 0 ? -u : u); ++i)
+                r = nextafterf(r, u < 0 ? 0.0f : 2.0f);
+            for (int sv = -msc; sv <= msc; ++sv)
+            {
+                if (sv < -128 || sv > 127)
+                    continue;
+                const float want = nearbyintf((float)sv * 127 * 256 / (fm * 32));
+                const float num = (float)(sv * 1016);
+                const float q0 = num * r;
+                const float q1 = fmaf(fmaf(-fm, q0, num), r, q0);
+                if (nearbyintf(q1) != want)
+                    ++bad;
+            }
+        }
+    }
+    return bad;
+}

@@ -95,6 +95,11 @@ void qlo_moe_route(const float *logits, int n_tokens, int n_experts, int top_k,
  * built and on the committed vectors. */
 void qlo_swiglu(const float *gate, const float *up, int n, float *out);
 
+/* Exhaustive checks of division-free forms used by the GPU kernels: number of inputs on
+ * which they differ from the reference's divisions (0 expected).                          */
+long qlo_check_div127(void);
+long qlo_check_q6k_factor(int ulps);
+
 /* ---- decode-step operators (decode_oracle.c) ------------------------------------- */
 void qlo_dequant_row_q4k(const llam_block_q4_K *blocks, int nblocks, float *out);
 void qlo_rmsnorm(float *x, const float *delta, const float *gamma, float eps, float *y, int rows, int cols);

@@ -352,3 +352,63 @@ def test_q6k_long_rows_large_batches(capi, dev, oracle, N, K):
     if K >= 25600:  # seven rows of a shorter row still fit the quad-lane kernel's LDS
         assert torch.equal(ys[8][:7], ys[7])
     sync()
+
+
+def _q6k_one_live_block_per_row(pairs, K, seed):
+    """Q6_K rows whose sub-scales are zero except for ONE block per row, which carries the
+    given pair: every other block contributes an exact zero, so a row's output is one
+    multiply-add and its bits do not depend on how a kernel orders the blocks."""
+    rng = np.random.default_rng(seed)
+    N, SB = len(pairs), K // 256
+    W = rng.integers(0, 256, size=(N, SB, 210), dtype=np.uint8)
+    W[:, :, 192:208] = 0
+    d = rng.uniform(0.0005, 0.05, size=(N, SB)).astype(np.float16)
+    d[::97] = np.float16(3e-6)   # block scales below the fp16 normal range (truncating conversion)
+    W[:, :, 208:210] = d.view(np.uint8).reshape(N, SB, 2)
+    sb = rng.integers(0, SB, N)
+    j = rng.integers(0, 8, N)
+    sc = W[:, :, 192:208].view(np.int8)
+    sc[np.arange(N), sb, 2 * j] = pairs[:, 0]
+    sc[np.arange(N), sb, 2 * j + 1] = pairs[:, 1]
+    return W
+
+
+def test_q6k_every_pair_of_subscales_bit_exact(capi, dev, oracle):
+    """All 65536 (sub-scale, sub-scale) pairs of a Q6_K block, one live block per row, through
+    the quad-lane kernel (K = 4096): the 8.8 factors (ties and signs included), the block scale
+    and its fp16 rounding must be the reference's exactly, so every output bit matches."""
+    import torch
+
+    v = np.arange(-128, 128, dtype=np.int8)
+    pairs = np.stack(np.meshgrid(v, v, indexing="ij"), -1).reshape(-1, 2)
+    K = 4096
+    W = _q6k_one_live_block_per_row(pairs, K, 5)
+    q8 = oracle.quantize(synth.activations_numpy(2, K, 6))
+    wd = upload_weights(capi, dev, FMT_Q6_K, W)
+    y = capi.gemv(FMT_Q6_K, wd, upload_q8(dev, q8), 2, len(pairs), K)
+    sync()
+    C = oracle.gemm(FMT_Q6_K, W, K, q8)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), C.view(np.uint32))
+    assert np.count_nonzero(C) > 0.9 * C.size
+
+
+def test_q6k_subscale_pairs_on_the_matrix_unit_bit_exact(capi, dev, oracle):
+    """The same construction on rows long enough for the matrix-unit kernel at batch 8
+    (K = 16640: 65 super-blocks), 4096 pairs that include every tie of the factor rounding."""
+    rng = np.random.default_rng(8)
+    v = np.arange(-128, 128)
+    a, b = np.meshgrid(v, v, indexing="ij")
+    m = np.maximum(np.abs(a), np.abs(b))
+    s = np.where(np.abs(a) >= np.abs(b), b, a)
+    tie = (m > 0) & ((2 * s * 1016) % np.maximum(m, 1) == 0) & (((2 * s * 1016) // np.maximum(m, 1)) % 2 != 0)
+    ties = np.stack([a[tie], b[tie]], -1)
+    rest = rng.integers(-128, 128, size=(4096 - min(len(ties), 2048), 2))
+    pairs = np.concatenate([ties[:2048], rest]).astype(np.int8)
+    K = 16640
+    W = _q6k_one_live_block_per_row(pairs, K, 9)
+    q8 = oracle.quantize(synth.activations_numpy(8, K, 10))
+    wd = upload_weights(capi, dev, FMT_Q6_K, W)
+    y = capi.gemv(FMT_Q6_K, wd, upload_q8(dev, q8), 8, len(pairs), K)
+    sync()
+    C = oracle.gemm(FMT_Q6_K, W, K, q8)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), C.view(np.uint32))

@@ -136,6 +136,16 @@ def test_q6k_requantisation_closed_form(oracle):
             assert np.abs(w[32 * j:32 * j + 32] * scale - native).max() <= 0.6 * scale + 1e-3 * np.abs(native).max()
 
 
+def test_division_free_forms_of_the_q6k_factors(oracle):
+    """The GPU kernels compute the Q6_K block scale and the 8.8 factor of the smaller sub-scale
+    without divisions; the same IEEE operations on the host, over every input they can see:
+    x/127 for every fp16 d and max sub-scale, and rne(s*1016/msc) for every (s, msc) with any
+    reciprocal within 4 units in the last place of the true one."""
+    assert oracle.check_div127() == 0
+    for ulps in (0, 1, 4):
+        assert oracle.check_q6k_factor(ulps) == 0
+
+
 def test_iq3s_requantisation_is_an_integer_map(oracle):
     """w = +-round(g*127/gmax) and scale = f16(gmax*db/127): a pure function of the codebook."""
     import re
