@@ -71,8 +71,11 @@ bool llam_ql_quantize_q8_1(const float *d_x, void *d_q8, int M, int K,
 /* ---- weight preparation -----------------------------------------------------------
  * Device layout the GEMV/GEMM kernels read.  Q4_K: the GGUF super-blocks
  * unchanged (144 B is 16-byte aligned).  Q6_K (210 B) and IQ3_S (110 B) are
- * split into 16-byte-aligned planes of the same total size (IQ3_S +2 B/block
- * padding).  No value is changed; this only moves bytes.
+ * split into 16-byte-aligned planes (IQ3_S +2 B/block padding); no weight byte is
+ * changed.  Q6_K additionally gets a plane of one 4-byte record per 32-element block
+ * (+32 B per super-block): the two 8.8 requantisation factors of the block and its
+ * fp16 scale, i.e. what unpack_q6_k_superblock_to_int8 (SIMDHelpers.h:12023-12204)
+ * derives from the sub-scales, worked out once instead of in every product.
  * Replaces packWeightsCPUNativeVNNI (CPUNativeVNNIWeightPacker.h:598) /
  * repack_*_to_vnni (src/v2/kernels/rocm/repack/VnniRepackKernels.hip:65-887).
  * d_prepared must be 16-byte aligned and llam_ql_prepared_bytes() large; it may

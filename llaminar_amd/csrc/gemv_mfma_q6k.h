@@ -1,7 +1,8 @@
 // Q6_K x Q8_1 decode GEMV for batches of 5..8 activation rows on the matrix unit.
 //
 // The exact 8.8 fixed-point requantisation of the 6-bit weights is what a Q6_K product costs
-// (several vector instructions per weight).  The quad-lane kernel keeps four activation rows
+// (several vector instructions per weight; its per-block factors and scales come ready-made
+// from the factor plane of the prepared layout).  The quad-lane kernel keeps four activation rows
 // in LDS at most when the row is long, so a batch of eight pays that requantisation twice.
 // Here every weight is requantised once: lane (r = l%32, h = l/32) turns elements
 // 16h..16h+15 of each 32-column block of weight row r into int8 (one Q6_K sub-scale covers
@@ -21,8 +22,9 @@
 // lane l loads the 16-byte pieces l, l+64, .. (eight neighbouring lanes cover a row's cache
 // line of ql) and the wavefront passes them through a private LDS buffer to the two lanes of
 // the row (rows 144 and 80 bytes apart there, so that the 128-bit reads of neighbouring rows
-// fall into different banks).  The 16 scale bytes and the fp16 d of a row go straight to its
-// two lanes.  No barrier for the buffer: LDS instructions of one wavefront run in order.
+// fall into different banks).  The 32 bytes of factor records of a row's super-block go
+// straight to its two lanes.  No barrier for the buffer: LDS instructions of one wavefront run
+// in order.
 #pragma once
 #include "gemv_mfma.h"
 #include <type_traits>
@@ -55,18 +57,17 @@ namespace llamql
 
     struct Mfma6Raw
     {
-        v4i ql0, ql1, ql2, ql3, qh0, qh1, sc;
-        int d;
+        v4i ql0, ql1, ql2, ql3, qh0, qh1, fc0, fc1;
     };
     // Plane bases advanced to the step's super-block (wavefront-uniform, scalar registers) and
-    // this lane's byte offsets from them: four pieces of ql, two of qh, its row's scales and d.
+    // this lane's byte offsets from them: four pieces of ql, two of qh, its row's factor records.
     struct Mfma6Ptr
     {
-        const uint8_t *ql, *qh, *sc, *d;
+        const uint8_t *ql, *qh, *fc;
     };
     struct Mfma6Off
     {
-        uint32_t ql[4], qh[2], sc, d;
+        uint32_t ql[4], qh[2], fc;
     };
     __device__ __forceinline__ void mfma6_load(Mfma6Raw &r, const Mfma6Ptr &p, const Mfma6Off &o)
     {
@@ -76,21 +77,21 @@ namespace llamql
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.ql3) : "v"(o.ql[3]), "s"(p.ql));
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qh0) : "v"(o.qh[0]), "s"(p.qh));
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qh1) : "v"(o.qh[1]), "s"(p.qh));
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.sc) : "v"(o.sc), "s"(p.sc));
-        asm volatile("global_load_ushort %0, %1, %2" : "=&v"(r.d) : "v"(o.d), "s"(p.d));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.fc0) : "v"(o.fc), "s"(p.fc));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(r.fc1) : "v"(o.fc), "s"(p.fc));
     }
     __device__ __forceinline__ void mfma6_keep(Mfma6Raw &r)
     {
         asm volatile(""
-                     : "+v"(r.ql0), "+v"(r.ql1), "+v"(r.ql2), "+v"(r.ql3), "+v"(r.qh0), "+v"(r.qh1), "+v"(r.sc),
-                       "+v"(r.d));
+                     : "+v"(r.ql0), "+v"(r.ql1), "+v"(r.ql2), "+v"(r.ql3), "+v"(r.qh0), "+v"(r.qh1), "+v"(r.fc0),
+                       "+v"(r.fc1));
     }
     template <int NEWER>
     __device__ __forceinline__ void mfma6_wait(Mfma6Raw &r)
     {
         asm volatile("s_waitcnt vmcnt(%8)"
-                     : "+v"(r.ql0), "+v"(r.ql1), "+v"(r.ql2), "+v"(r.ql3), "+v"(r.qh0), "+v"(r.qh1), "+v"(r.sc),
-                       "+v"(r.d)
+                     : "+v"(r.ql0), "+v"(r.ql1), "+v"(r.ql2), "+v"(r.ql3), "+v"(r.qh0), "+v"(r.qh1), "+v"(r.fc0),
+                       "+v"(r.fc1)
                      : "n"(NEWER));
     }
 
@@ -170,8 +171,7 @@ namespace llamql
 #pragma unroll
             for (int i = 0; i < 2; ++i) // qh piece lane + 64 i: row (lane >> 2) + 16 i, 16 bytes at 16 (lane & 3)
                 off.qh[i] = sb_index((lane >> 2) + 16 * i) * 64u + 16u * (uint32_t)(lane & 3);
-            off.sc = sb_index(l32) * 16u;
-            off.d = sb_index(l32) * 2u;
+            off.fc = sb_index(l32) * 32u;
             uint8_t *bounce = mfma6_lds + mfma6_act_bytes(nsb, a.chunk) + (size_t)wave * MFMA6_BOUNCE;
             uint8_t *wr_ql = bounce + (lane >> 3) * MFMA6_QL_STRIDE + (lane & 7) * 16;  // piece i at + 8 i rows
             uint8_t *wr_qh = bounce + 32 * MFMA6_QL_STRIDE + (lane >> 2) * MFMA6_QH_STRIDE + (lane & 3) * 16;
@@ -190,8 +190,7 @@ namespace llamql
                 Mfma6Ptr pl;
                 pl.ql = uniform(a.w + (size_t)sb * 128);
                 pl.qh = uniform(a.w + T * 128 + (size_t)sb * 64);
-                pl.sc = uniform(a.w + T * 192 + (size_t)sb * 16);
-                pl.d = uniform(a.w + T * 208 + (size_t)sb * 2);
+                pl.fc = uniform(a.w + q6k_factors_offset(T) + (size_t)sb * 32);
                 mfma6_load(r, pl, off);
             };
             Mfma6Raw bufA, bufB;
@@ -209,9 +208,8 @@ namespace llamql
             const int a_lane = (l32 & 7) * 32 + lh * 16; // rows beyond the batch: any row, result unused
             int step = 0, cur_ph = 0;
 
-            // the coalesced pieces of a step into the bounce buffer; its scales and d stay behind
-            v4i sc_cur;
-            int d_cur;
+            // the coalesced pieces of a step into the bounce buffer; its factor records stay behind
+            v4i fc_cur0, fc_cur1;
             auto stage_w = [&](const Mfma6Raw &r) {
                 mfma_wave_sync(); // the previous step's reads are done
                 *reinterpret_cast<v4i *>(wr_ql) = r.ql0;
@@ -220,8 +218,8 @@ namespace llamql
                 *reinterpret_cast<v4i *>(wr_ql + 24 * MFMA6_QL_STRIDE) = r.ql3;
                 *reinterpret_cast<v4i *>(wr_qh) = r.qh0;
                 *reinterpret_cast<v4i *>(wr_qh + 16 * MFMA6_QH_STRIDE) = r.qh1;
-                sc_cur = r.sc;
-                d_cur = r.d;
+                fc_cur0 = r.fc0;
+                fc_cur1 = r.fc1;
                 mfma_wave_sync();
             };
 
@@ -236,54 +234,22 @@ namespace llamql
                 const int kb0 = (sb - ph * a.chunk) * 8;
                 const uint8_t *ab = buf_aq(ph) + (size_t)kb0 * MFMA_AQ_STRIDE + a_lane;
                 const float *sb_sc = buf_asc(ph) + (size_t)kb0 * 16 + lh * 8;
-                const float d = h2f((uint16_t)d_cur);
                 const v4i ql[4] = {*reinterpret_cast<const v4i *>(rd_ql), *reinterpret_cast<const v4i *>(rd_ql + 32),
                                    *reinterpret_cast<const v4i *>(rd_ql + 64), *reinterpret_cast<const v4i *>(rd_ql + 96)};
                 const v4i qh[2] = {*reinterpret_cast<const v4i *>(rd_qh), *reinterpret_cast<const v4i *>(rd_qh + 32)};
                 const uint32_t k4 = 0x0F0F0F0Fu, k2 = 0x03030303u;
-                // The factors of a block need both its sub-scales and two divisions: the lane of
-                // half h works them out for blocks 4h..4h+3 and passes the other half's factor
-                // and the block scale to the lane of that half (lane ^ 32).
-                uint32_t fc[8]; // this lane's factor (low half-word) and constant 128 - 32 f
-                float bsc[8];
-                {
-                    const int sc_lo = lh ? sc_cur.z : sc_cur.x, sc_hi = lh ? sc_cur.w : sc_cur.y;
-                    uint32_t mine[4], theirs[4];
-                    float bmine[4];
-#pragma unroll
-                    for (int s = 0; s < 4; ++s)
-                    {
-                        const int sdw = (s >> 1) ? sc_hi : sc_lo;
-                        const int s0 = __builtin_amdgcn_sbfe(sdw, 16u * (s & 1), 8u);
-                        const int s1 = __builtin_amdgcn_sbfe(sdw, 16u * (s & 1) + 8u, 8u);
-                        Q6KQuad::v2s f0, c0, f1, c1;
-                        Q6KQuad::block_factors(s0, s1, d, f0, c0, f1, c1, bmine[s]);
-                        const uint32_t p0 = (uint32_t)f0.x | ((uint32_t)c0.x << 16);
-                        const uint32_t p1 = (uint32_t)f1.x | ((uint32_t)c1.x << 16);
-                        mine[s] = lh ? p1 : p0;
-                        theirs[s] = lh ? p0 : p1;
-                    }
-                    const int partner = (lane ^ 32) * 4;
-#pragma unroll
-                    for (int s = 0; s < 4; ++s)
-                    {
-                        const uint32_t got = (uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)theirs[s]);
-                        const float bgot = __builtin_bit_cast(
-                            float, __builtin_amdgcn_ds_bpermute(partner, __builtin_bit_cast(int, bmine[s])));
-                        // blocks 0..3 were worked out by half 0, blocks 4..7 by half 1
-                        fc[s] = lh ? got : mine[s];
-                        fc[4 + s] = lh ? mine[s] : got;
-                        bsc[s] = lh ? bgot : bmine[s];
-                        bsc[4 + s] = lh ? bmine[s] : bgot;
-                    }
-                }
+                // the records of the super-block's eight blocks, in the order the plane keeps them
+                const uint32_t rec[8] = {(uint32_t)fc_cur0.x, (uint32_t)fc_cur0.y, (uint32_t)fc_cur0.z, (uint32_t)fc_cur0.w,
+                                         (uint32_t)fc_cur1.x, (uint32_t)fc_cur1.y, (uint32_t)fc_cur1.z, (uint32_t)fc_cur1.w};
                 // block j = 4n + s: nibbles of ql piece (n, s & 1), low for s < 2, high otherwise;
                 // bits 2s, 2s+1 of qh piece n; sub-scales 8n + 2s and 8n + 2s + 1
                 auto product = [&](int j, float &bscale) {
                     const int n = j >> 2, s = j & 3;
-                    bscale = bsc[j];
-                    const Q6KQuad::v2s ff = __builtin_bit_cast(Q6KQuad::v2s, __builtin_amdgcn_perm(fc[j], fc[j], 0x01000100u));
-                    const Q6KQuad::v2s cc = __builtin_bit_cast(Q6KQuad::v2s, __builtin_amdgcn_perm(fc[j], fc[j], 0x03020302u));
+                    int f0, f1;
+                    q6k_block_decode(rec[q6k_code_pos(j)], f0, f1, bscale);
+                    const int f = lh ? f1 : f0; // this lane's 16 elements share one sub-scale
+                    const unsigned short fu = (unsigned short)f, ku = (unsigned short)(128 - 32 * f);
+                    const Q6KQuad::v2s ff = {fu, fu}, cc = {ku, ku};
                     const v4i lo = ql[2 * n + (s & 1)], hi = qh[n];
                     auto q4 = [&](int l, int h) {
                         const uint32_t nib = (s >= 2 ? (uint32_t)l >> 4 : (uint32_t)l) & k4;

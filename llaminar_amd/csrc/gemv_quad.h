@@ -347,21 +347,19 @@ namespace llamql
     {
         typedef unsigned short v2s __attribute__((ext_vector_type(2)));
         typedef int v2i_ __attribute__((ext_vector_type(2)));
-        static constexpr int LOADS = 6;
+        static constexpr int LOADS = 5;
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
         static bool addressable(long N, int SB) { return (double)N * SB * 128.0 < 4.0e9; }
 
         struct Raw
         {
             v4i qla, qlb, qha, qhb;
-            v2i_ sc;
-            int d;
+            v2i_ fc; // the factor records of the lane's two blocks (q6k_block_code)
         };
         struct Lane
         {
-            uint32_t ql_off, qh_off, sc_off; // byte offsets of this lane inside a super-block's planes
+            uint32_t ql_off, qh_off, fc_off; // byte offsets of this lane inside a super-block's planes
             uint32_t hshift;                 // 2h: bit offset of the low-nibble block's upper bits
-            uint32_t sshift;                 // 16h: bit offset of the lane's two scales in a dword
         };
         struct Scale
         {
@@ -369,7 +367,7 @@ namespace llamql
         };
         struct Cursor
         {
-            const uint8_t *ql, *qh, *sc, *d; // plane bases (uniform)
+            const uint8_t *ql, *qh, *fc; // plane bases (uniform)
             uint32_t t, first;               // this lane's super-block index: current, and the one
                                              // read instead past the end of the run
         };
@@ -380,9 +378,8 @@ namespace llamql
             const uint32_t n = (uint32_t)l >> 1, h = (uint32_t)l & 1u;
             c.ql_off = 64u * n + 32u * h;
             c.qh_off = 32u * n;
-            c.sc_off = 8u * n;
+            c.fc_off = 8u * (uint32_t)l; // records of blocks 4n+h and 4n+2+h are neighbours
             c.hshift = 2u * h;
-            c.sshift = 16u * h;
             return c;
         }
         // block j = 4n + sub: lane 2n + (sub & 1), its first (sub < 2) or second block
@@ -397,8 +394,7 @@ namespace llamql
             Cursor c;
             c.ql = static_cast<const uint8_t *>(a.w);
             c.qh = c.ql + T * 128;
-            c.sc = c.ql + T * 192;
-            c.d = c.ql + T * 208;
+            c.fc = c.ql + q6k_factors_offset(T);
             c.t = (uint32_t)t;
             c.first = (uint32_t)t_safe;
             return c;
@@ -417,23 +413,22 @@ namespace llamql
         // Loads issued as assembly so that the kernel decides where they are waited for.
         __device__ __forceinline__ static void load_index(Raw &r, const Cursor &c, const Lane &lc, uint32_t t)
         {
-            const uint32_t oql = t * 128u + lc.ql_off, oqh = t * 64u + lc.qh_off, osc = t * 16u + lc.sc_off, od = t * 2u;
+            const uint32_t oql = t * 128u + lc.ql_off, oqh = t * 64u + lc.qh_off, ofc = t * 32u + lc.fc_off;
             asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qla) : "v"(oql), "s"(c.ql));
             asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(r.qlb) : "v"(oql), "s"(c.ql));
             asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qha) : "v"(oqh), "s"(c.qh));
             asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(r.qhb) : "v"(oqh), "s"(c.qh));
-            asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(r.sc) : "v"(osc), "s"(c.sc));
-            asm volatile("global_load_ushort %0, %1, %2" : "=&v"(r.d) : "v"(od), "s"(c.d));
+            asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(r.fc) : "v"(ofc), "s"(c.fc));
         }
         __device__ __forceinline__ static void keep(Raw &r)
         {
-            asm volatile("" : "+v"(r.qla), "+v"(r.qlb), "+v"(r.qha), "+v"(r.qhb), "+v"(r.sc), "+v"(r.d));
+            asm volatile("" : "+v"(r.qla), "+v"(r.qlb), "+v"(r.qha), "+v"(r.qhb), "+v"(r.fc));
         }
         template <int NEWER>
         __device__ __forceinline__ static void wait(Raw &r)
         {
-            asm volatile("s_waitcnt vmcnt(%6)"
-                         : "+v"(r.qla), "+v"(r.qlb), "+v"(r.qha), "+v"(r.qhb), "+v"(r.sc), "+v"(r.d)
+            asm volatile("s_waitcnt vmcnt(%5)"
+                         : "+v"(r.qla), "+v"(r.qlb), "+v"(r.qha), "+v"(r.qhb), "+v"(r.fc)
                          : "n"(NEWER));
         }
 
@@ -450,31 +445,13 @@ namespace llamql
                                               0x07030501u);
         }
 
-        // The two 8.8 factors and the effective scale of one block from its two sub-scales.
-        __device__ __forceinline__ static void block_factors(int s0, int s1, float d, v2s &f0, v2s &c0, v2s &f1,
-                                                             v2s &c1, float &bscale)
+        // The two 8.8 factors (with their constants 128 - 32 f, each doubled into a packed pair)
+        // and the scale of one block from its record.
+        __device__ __forceinline__ static void block_factors(uint32_t code, v2s &f0, v2s &c0, v2s &f1, v2s &c1,
+                                                             float &bscale)
         {
-            const int a0 = s0 < 0 ? -s0 : s0, a1 = s1 < 0 ? -s1 : s1;
-            const bool big0 = a0 >= a1;
-            const int msc = big0 ? a0 : a1;
-            const int s_small = big0 ? s1 : s0, s_big = big0 ? s0 : s1;
-            const float fm = (float)msc;
-            int f_small = 0, f_big = 0;
-            bscale = 0.0f;
-            if (msc != 0)
-            {
-                f_big = s_big < 0 ? -1016 : 1016; // rne(+-msc*32512 / (msc*32))
-                // rne(s_small*32512 / (msc*32)) = rne(s_small*1016 / msc) without a division: the
-                // quotient has a denominator of at most 128, so unless it is a half-integer it lies
-                // 1/256 or more from one and any value within 1e-3 rounds alike; a half-integer is a
-                // float, and one Newton step on the reciprocal reproduces representable quotients.
-                const float num = (float)(s_small * 1016);
-                const float r = __builtin_amdgcn_rcpf(fm);
-                const float q0 = num * r;
-                f_small = (int)rintf(fmaf(fmaf(-fm, q0, num), r, q0));
-                bscale = f16_round_packer(div_by_127(d * fm * 32.0f));
-            }
-            const int fi0 = big0 ? f_big : f_small, fi1 = big0 ? f_small : f_big;
+            int fi0, fi1;
+            q6k_block_decode(code, fi0, fi1, bscale);
             const unsigned short u0 = (unsigned short)fi0, u1 = (unsigned short)fi1;
             const unsigned short k0 = (unsigned short)(128 - 32 * fi0), k1 = (unsigned short)(128 - 32 * fi1);
             f0 = (v2s){u0, u0};
@@ -486,14 +463,9 @@ namespace llamql
         // w[0], w[1]: elements 0-15, 16-31 of block 4n+h; w[2], w[3]: of block 4n+2+h.
         __device__ __forceinline__ static void decode(const Raw &r, const Lane &lc, v4i (&w)[4], Scale &S)
         {
-            const float d = h2f((uint16_t)r.d);
-            const int sA0 = __builtin_amdgcn_sbfe(r.sc.x, lc.sshift, 8u);
-            const int sA1 = __builtin_amdgcn_sbfe(r.sc.x, lc.sshift + 8u, 8u);
-            const int sB0 = __builtin_amdgcn_sbfe(r.sc.y, lc.sshift, 8u);
-            const int sB1 = __builtin_amdgcn_sbfe(r.sc.y, lc.sshift + 8u, 8u);
             v2s fA0, cA0, fA1, cA1, fB0, cB0, fB1, cB1;
-            block_factors(sA0, sA1, d, fA0, cA0, fA1, cA1, S.bs0);
-            block_factors(sB0, sB1, d, fB0, cB0, fB1, cB1, S.bs1);
+            block_factors((uint32_t)r.fc.x, fA0, cA0, fA1, cA1, S.bs0);
+            block_factors((uint32_t)r.fc.y, fB0, cB0, fB1, cB1, S.bs1);
 
             const uint32_t k4 = 0x0F0F0F0Fu, k2 = 0x03030303u;
             auto pair = [&](uint32_t ql, uint32_t qh, v2s fa, v2s ca, v2s fb, v2s cb, int &wa, int &wb) {

@@ -1,8 +1,10 @@
 // Weight preparation: raw GGUF super-blocks -> the device layout the kernels
-// read.  Only moves bytes; no value changes.
+// read.  Moves bytes; for Q6_K it also works out, once, the per-block requantisation
+// factors and scales that every product would otherwise recompute.
 //
 //   Q4_K  : unchanged (144-byte blocks are 16-byte aligned)
 //   Q6_K  : planes ql [T][128] | qh [T][64] | scales [T][16] | d [T] fp16      (T*210 B)
+//           | pad to 16 | factors [T][8] x 4 B (q6k_block_code, ql_device.h)    (T*32 B)
 //   IQ3_S : planes qs [T][64] | signs [T][32] | meta [T][16]                   (T*112 B)
 //           meta = qh[8] scales[4] d[2] pad[2]
 // with T = N*K/256 super-blocks in row-major order.  Raw Q6_K / IQ3_S blocks are
@@ -33,6 +35,21 @@ namespace llamql
         else
             o = T * 104 + t; // d
         dst[o] = v;
+    }
+
+    // one thread per 32-element block: its two sub-scales and the super-block's d -> record
+    __global__ void __launch_bounds__(256)
+        prepare_q6k_factors_kernel(const uint16_t *__restrict__ src, uint32_t *__restrict__ fac, size_t T)
+    {
+        const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (i >= T * 8)
+            return;
+        const size_t t = i >> 3;
+        const int j = (int)(i & 7);
+        const uint16_t pair = src[t * 105 + 96 + j]; // scales[2j], scales[2j+1] (block j = 4n+s: 8n+2s = 2j)
+        const int s0 = (int)(int8_t)(pair & 0xFF), s1 = (int)(int8_t)(pair >> 8);
+        const float d = h2f(src[t * 105 + 104]);
+        fac[t * 8 + q6k_code_pos(j)] = q6k_block_code(s0, s1, d);
     }
 
     __global__ void __launch_bounds__(256)
@@ -76,7 +93,7 @@ extern "C" size_t llam_ql_prepared_bytes(uint8_t fmt, int N, int K)
     switch (fmt)
     {
     case LLAM_FMT_Q4_K: return T * 144;
-    case LLAM_FMT_Q6_K: return T * 210;
+    case LLAM_FMT_Q6_K: return llamql::q6k_factors_offset(T) + T * 32;
     case LLAM_FMT_IQ3_S: return T * 112;
     default: return 0;
     }
@@ -119,8 +136,13 @@ extern "C" bool llam_ql_prepare_weights(uint8_t fmt, const void *d_gguf, void *d
     if (grid > 0x7FFFFFFFull)
         return fail(fn, "matrix too large (N=%d K=%d)", N, K);
     if (fmt == LLAM_FMT_Q6_K)
+    {
         hipLaunchKernelGGL(prepare_q6k_kernel, dim3((unsigned)grid), dim3(256), 0, st,
                            static_cast<const uint16_t *>(d_gguf), static_cast<uint16_t *>(d_prepared), T);
+        uint32_t *fac = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(d_prepared) + q6k_factors_offset(T));
+        hipLaunchKernelGGL(prepare_q6k_factors_kernel, dim3((unsigned)((T * 8 + 255) / 256)), dim3(256), 0, st,
+                           static_cast<const uint16_t *>(d_gguf), fac, T);
+    }
     else
         hipLaunchKernelGGL(prepare_iq3s_kernel, dim3((unsigned)grid), dim3(256), 0, st,
                            static_cast<const uint16_t *>(d_gguf), static_cast<uint16_t *>(d_prepared), T);

@@ -45,6 +45,53 @@ namespace llamql
         return __builtin_amdgcn_classf(x, 0x198) ? q1 : q0; // finite and not zero
     }
 
+    // ---- Q6_K block factors, worked out once when the weights are prepared ---------------
+    // A 32-element block has two int8 sub-scales s0, s1.  With msc = max(|s0|, |s1|) the
+    // reference requantises w = ((q - 32) * f_h + 128) >> 8, f_h = rne(s_h * 32512 / (msc * 32)),
+    // and scales the block by f16(d * msc * 32 / 127) (SIMDHelpers.h:12023-12204).  The larger
+    // sub-scale's factor is +-1016; the record keeps the other one:
+    //   bits  0..11  f of the smaller sub-scale (two's complement)
+    //   bit   12     the larger sub-scale is the second one (ties: the first)
+    //   bit   13     the larger sub-scale is negative
+    //   bit   14     both sub-scales are zero (weights and scale are zero)
+    //   bits 16..31  the block scale as fp16 bits
+    constexpr uint32_t Q6K_CODE_BIG1 = 1u << 12, Q6K_CODE_NEG = 1u << 13, Q6K_CODE_ZERO = 1u << 14;
+
+    __device__ __forceinline__ uint32_t q6k_block_code(int s0, int s1, float d)
+    {
+        const int a0 = s0 < 0 ? -s0 : s0, a1 = s1 < 0 ? -s1 : s1;
+        const bool big0 = a0 >= a1;
+        const int msc = big0 ? a0 : a1;
+        if (msc == 0)
+            return Q6K_CODE_ZERO;
+        const int s_small = big0 ? s1 : s0, s_big = big0 ? s0 : s1;
+        const float fm = (float)msc;
+        // rne(s_small * 1016 / msc) without a division: the quotient has a denominator of at most
+        // 128, so unless it is a half-integer it lies 1/256 or more from one and any value within
+        // 1e-3 rounds alike; a half-integer is a float, and one Newton step on the reciprocal
+        // reproduces representable quotients.
+        const float num = (float)(s_small * 1016);
+        const float r = __builtin_amdgcn_rcpf(fm);
+        const float q0 = num * r;
+        const int f_small = (int)rintf(fmaf(fmaf(-fm, q0, num), r, q0));
+        const float bscale = f16_round_packer(div_by_127(d * fm * 32.0f));
+        return ((uint32_t)f_small & 0xFFFu) | (big0 ? 0u : Q6K_CODE_BIG1) | (s_big < 0 ? Q6K_CODE_NEG : 0u) |
+               ((uint32_t)__half_as_ushort(__float2half_rn(bscale)) << 16); // bscale is an fp16 value: exact
+    }
+    // the two 8.8 factors and the block scale of a record
+    __device__ __forceinline__ void q6k_block_decode(uint32_t c, int &f0, int &f1, float &bscale)
+    {
+        const int fs = __builtin_amdgcn_sbfe((int)c, 0u, 12u);
+        const int fb = (c & Q6K_CODE_ZERO) ? 0 : ((c & Q6K_CODE_NEG) ? -1016 : 1016);
+        const bool big1 = (c & Q6K_CODE_BIG1) != 0;
+        f0 = big1 ? fs : fb;
+        f1 = big1 ? fb : fs;
+        bscale = h2f((uint16_t)(c >> 16));
+    }
+    // where the record of block j sits among the eight of its super-block: the two blocks a
+    // quad lane decodes (4n + h and 4n + 2 + h for lane 2n + h) are neighbours
+    __host__ __device__ constexpr int q6k_code_pos(int j) { return (j & 4) | ((j & 1) << 1) | ((j >> 1) & 1); }
+
     // Same rounding for two values at once.  The truncating branch is only needed when a
     // value lies below the fp16 normal range, which real weights almost never produce:
     // one rarely-taken branch (fp16 exponent field 0 or 1 in either result) guards the

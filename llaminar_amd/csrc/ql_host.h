@@ -37,6 +37,8 @@ namespace llamql
         return true;
     }
 
+    // byte offset of the Q6_K factor plane in a prepared matrix of T super-blocks
+    __host__ __device__ inline size_t q6k_factors_offset(size_t T) { return (T * 210 + 15) & ~(size_t)15; }
     inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
     inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 

@@ -65,7 +65,9 @@ def test_argument_validation_and_error_text():
     assert "ldy" in capi.last_error()
     assert not lib.llam_ql_moe_route(p16, 1, 8, 9, 1, p16, p16, 0, None)
     assert "top_k" in capi.last_error()
-    assert lib.llam_ql_prepared_bytes(capi.FMT_Q6_K, 4, 512) == 4 * 2 * 210
+    # Q6_K: the 210 bytes of a block in planes, padded to 16, then 8 four-byte factor records per block
+    assert lib.llam_ql_prepared_bytes(capi.FMT_Q6_K, 4, 512) == 4 * 2 * 210 + 4 * 2 * 32
+    assert lib.llam_ql_prepared_bytes(capi.FMT_Q6_K, 3, 256) == 640 + 3 * 32
     assert lib.llam_ql_prepared_bytes(capi.FMT_IQ3_S, 4, 512) == 4 * 2 * 112
     assert lib.llam_ql_prepared_bytes(capi.FMT_Q4_K, 4, 100) == 0
     # empty problems are a successful no-op

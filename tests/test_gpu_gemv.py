@@ -242,8 +242,10 @@ def test_q4k_prepare_is_identity(capi, dev):
 
 
 @pytest.mark.parametrize("fmt", [FMT_Q6_K, FMT_IQ3_S], ids=["q6_k", "iq3_s"])
-def test_prepare_moves_every_byte(capi, dev, fmt):
-    """Plane layout: a permutation of the input bytes (plus zero padding for IQ3_S)."""
+def test_prepare_moves_every_byte(capi, dev, oracle, fmt):
+    """Plane layout: a permutation of the input bytes (plus zero padding for IQ3_S).  Q6_K also
+    gets a plane of per-block records, the 8.8 factors of the two sub-scales of a block and its
+    scale, which must be the closed form of the requantisation the reference performs."""
     N, K = 5, 768
     W = synth.weights_numpy(fmt, N, K, 2)
     wd = upload_weights(capi, dev, fmt, W)
@@ -255,7 +257,32 @@ def test_prepare_moves_every_byte(capi, dev, fmt):
         assert np.array_equal(P[:T * 128].reshape(T, 128), B[:, :128])
         assert np.array_equal(P[T * 128:T * 192].reshape(T, 64), B[:, 128:192])
         assert np.array_equal(P[T * 192:T * 208].reshape(T, 16), B[:, 192:208])
-        assert np.array_equal(P[T * 208:].reshape(T, 2), B[:, 208:210])
+        assert np.array_equal(P[T * 208:T * 210].reshape(T, 2), B[:, 208:210])
+        off = (T * 210 + 15) & ~15
+        assert P.size == off + T * 32
+        rec = P[off:].view(np.uint32).reshape(T, 8)
+        sc = B[:, 192:208].view(np.int8).astype(int)
+
+        def rne_div(a, b):  # round-half-even of a/b for integers, b > 0
+            qq, rr = divmod(a, b)
+            return qq + (1 if (2 * rr > b or (2 * rr == b and (qq & 1))) else 0)
+
+        for t in range(T):
+            _, sc_h, _ = oracle.subblocks(fmt, B[t])
+            for j in range(8):
+                c = int(rec[t, (j & 4) | ((j & 1) << 1) | ((j >> 1) & 1)])
+                s0, s1 = sc[t, 2 * j], sc[t, 2 * j + 1]
+                msc = max(abs(s0), abs(s1))
+                assert (c >> 16) == int(sc_h[j]), (t, j)
+                if msc == 0:
+                    assert (c & 0xFFFF) == 1 << 14
+                    continue
+                big1 = abs(s1) > abs(s0)
+                small, big = (s0, s1) if big1 else (s1, s0)
+                fs = c & 0xFFF
+                fs -= 4096 if fs & 0x800 else 0
+                assert fs == rne_div(small * 1016, msc) and bool(c & (1 << 12)) == big1
+                assert bool(c & (1 << 13)) == (big < 0) and not c & (1 << 14)
     else:
         assert np.array_equal(P[:T * 64].reshape(T, 64), B[:, 2:66])
         assert np.array_equal(P[T * 64:T * 96].reshape(T, 32), B[:, 74:106])
