@@ -348,9 +348,9 @@ namespace llamql
         int slices, tiles, chunk;
         long grid;
     };
-    // Slices so that a compute unit sees about ten compute wavefronts, five at least (the
+    // Slices so that a compute unit sees about eight compute wavefronts, five at least (the
     // scales of eight neighbouring super-blocks share a cache line) and each two steps long;
-    // tiles per workgroup to fill its ten compute wavefronts when there are tiles to spare.
+    // tiles per workgroup to fill its compute wavefronts when there are tiles to spare.
     inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus)
     {
         const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
