@@ -349,14 +349,9 @@ namespace llamql
                                   int n_kv, int ctx_cap, int n_chunks)
     {
         constexpr size_t lds = (size_t)(ATT_CHUNK * G + ATT_ROWS * G * ATT_HD) * sizeof(float);
-        static bool attr_set = false;
-        if (!attr_set && lds > 64 * 1024)
-        {
-            // dynamic LDS beyond 64 KiB has to be allowed per kernel once
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&attention_partial_kernel<G>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            attr_set = true;
-        }
+        static LdsGrant grant;
+        if (lds > 64 * 1024)
+            (void)allow_lds(grant, reinterpret_cast<const void *>(&attention_partial_kernel<G>), lds);
         hipLaunchKernelGGL(attention_partial_kernel<G>, grid, dim3(ATT_THREADS), lds, st, q, ld_q, kc, vc, pos, part_o,
                            part_ml, n_heads, n_kv, ctx_cap, n_chunks);
     }

@@ -353,15 +353,10 @@ namespace llamql
         g.M = M;
         g.ldy = ldy;
         constexpr size_t lds = gemm_lds_bytes<F>();
-        static bool attr_set = false;
-        if (!attr_set)
-        {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<F>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess)
-                return fail(fn, "cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-            attr_set = true;
-        }
+        static LdsGrant grant;
+        const hipError_t e = allow_lds(grant, reinterpret_cast<const void *>(&gemm_kernel<F>), lds);
+        if (e != hipSuccess)
+            return fail(fn, "cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
         const dim3 grid((unsigned)((N + GEMM_BN - 1) / GEMM_BN), (unsigned)((M + GEMM_BM - 1) / GEMM_BM));
         hipLaunchKernelGGL((gemm_kernel<F>), grid, dim3(GEMM_THREADS), lds, st, g);
         return launched(fn);

@@ -349,14 +349,8 @@ namespace llamql
     template <int SRC>
     void gemv_mfma_q4k_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const MfmaArgs &a)
     {
-        static bool attr_set = false;
-        if (!attr_set)
-        {
-            // dynamic LDS beyond 64 KiB has to be allowed per kernel once
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<SRC>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            attr_set = true;
-        }
+        static LdsGrant grant;
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<SRC>), QUAD_MAX_LDS);
         hipLaunchKernelGGL(gemv_mfma_q4k_kernel<SRC>, grid, block, lds, st, a);
     }
 
@@ -391,13 +385,8 @@ namespace llamql
     template <int SRC>
     void gemv_mfma_q6k_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const Mfma6Args &a)
     {
-        static bool attr_set = false;
-        if (!attr_set)
-        {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_mfma_q6k_kernel<SRC>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            attr_set = true;
-        }
+        static LdsGrant grant;
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q6k_kernel<SRC>), QUAD_MAX_LDS);
         hipLaunchKernelGGL(gemv_mfma_q6k_kernel<SRC>, grid, block, lds, st, a);
     }
 

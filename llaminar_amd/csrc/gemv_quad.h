@@ -728,14 +728,8 @@ namespace llamql
     template <class Q, int M, int U, int SRC>
     inline void gemv_quad_launch_mus(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
-        static bool attr_set = false;
-        if (!attr_set)
-        {
-            // dynamic LDS beyond 64 KiB has to be allowed per kernel once
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            attr_set = true;
-        }
+        static LdsGrant grant;
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC>), QUAD_MAX_LDS);
         hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U, SRC>), grid, block, lds, st, a);
     }
 
@@ -779,13 +773,8 @@ namespace llamql
     inline void gemv_quad_dual_launch_ms(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         auto kernel = &gemv_quad_dual_kernel<QA, quad_unroll<QA>(M), QB, quad_unroll<QB>(M), M, SRC>;
-        static bool attr_set = false;
-        if (!attr_set)
-        {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      160 * 1024);
-            attr_set = true;
-        }
+        static LdsGrant grant;
+        (void)allow_lds(grant, reinterpret_cast<const void *>(kernel), QUAD_MAX_LDS);
         hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
     }
 

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -35,6 +36,28 @@ namespace llamql
         if (e != hipSuccess)
             return fail(fn, "kernel launch failed: %s", hipGetErrorString(e));
         return true;
+    }
+
+    // Dynamic LDS beyond 64 KiB has to be allowed per kernel, once on every device the kernel
+    // runs on.  One LdsGrant per launch site remembers the devices that have been served; the
+    // flags are atomics because several host threads may launch the same kernel.
+    struct LdsGrant
+    {
+        static constexpr int MAX_DEVICES = 64;
+        std::atomic<bool> done[MAX_DEVICES];
+    };
+    inline hipError_t allow_lds(LdsGrant &g, const void *kernel, size_t bytes)
+    {
+        int dev = -1;
+        if (hipGetDevice(&dev) != hipSuccess)
+            dev = -1;
+        const bool tracked = dev >= 0 && dev < LdsGrant::MAX_DEVICES;
+        if (tracked && g.done[dev].load(std::memory_order_acquire))
+            return hipSuccess;
+        const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e == hipSuccess && tracked)
+            g.done[dev].store(true, std::memory_order_release);
+        return e;
     }
 
     // byte offset of the Q6_K factor plane in a prepared matrix of T super-blocks
