@@ -94,7 +94,7 @@ def bench_gemm(args, torch, capi, synth, dev):
 
 
 def bench_moe(args, torch, capi, synth, dev):
-    """MoE expert FFN decode: route, gate/up, SwiGLU+quantise, down, shared expert."""
+    """MoE expert FFN decode: route (+ Q8_1 of the hidden state), gate/up, SwiGLU+quantise, down, shared expert."""
     from llaminar_amd.capi import FMT_IQ3_S
 
     T = args.batch
@@ -124,8 +124,7 @@ def bench_moe(args, torch, capi, synth, dev):
                      "w": torch.ones(T, TOPK + 1, device=dev)})
 
     def step(s):
-        capi.moe_route(s["logits"], TOPK, ids=s["ids"], weights=s["w"])
-        capi.quantize_q8_1(s["x"], out=s["q8"])
+        capi.moe_route_quantize(s["logits"], TOPK, s["x"], s["q8"], ids=s["ids"], weights=s["w"])
         gate, up = capi.moe_gate_up(fmt, table, E + 1, s["ids"], s["q8"], T, TOPK + 1, H, I)
         qa = capi.swiglu_quantize(gate, up)
         capi.moe_down(fmt, table, E + 1, s["ids"], s["w"], qa, s["out"], T, TOPK + 1, H, I, accumulate=False)
@@ -151,7 +150,7 @@ def bench_moe(args, torch, capi, synth, dev):
                     "tokens": T, "weight_bytes_per_step": w_bytes, "tokens_per_s": round(T / (us * 1e-6), 1),
                     "token_sets_rotated": nsets, "distinct_routed_experts_over_sets": distinct,
                     "launch": "hip-graph replay of all token sets' steps"},
-                   {"kernel": "moe step (5 launches)", "bound": "hbm", "achieved": round(value, 1),
+                   {"kernel": "moe step (4 launches)", "bound": "hbm", "achieved": round(value, 1),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None,
                     "bytes_per_launch": w_bytes, "us_per_launch": round(us, 2), "launches_timed": args.steps})
 

@@ -177,6 +177,15 @@ bool llam_ql_moe_route(const float *d_logits, int n_tokens, int n_experts,
                        int top_k, int normalize, int32_t *d_ids,
                        float *d_weights, int device_id, void *stream);
 
+/* llam_ql_moe_route_ex and llam_ql_quantize_q8_1(d_hidden, d_q8, n_tokens, d_model) in one
+ * launch: the hidden state the expert GEMVs read does not depend on the routing, so its
+ * quantiser rides along (same bits as the two calls).  No counterpart in the reference, whose
+ * stage quantises inside the first expert GEMV (MoEExpertComputeStage.cpp:1450-1500). */
+bool llam_ql_moe_route_quantize(const float *d_logits, int n_tokens, int n_experts, int top_k,
+                                int normalize, int32_t *d_ids, float *d_weights, int slot_stride,
+                                const float *d_hidden, int d_model, void *d_q8, int device_id,
+                                void *stream);
+
 /* Same with the slots of a token slot_stride (>= top_k) entries apart in d_ids and
  * d_weights: columns top_k.. are left alone, so a caller can keep always-on experts
  * (the shared expert of MoEExpertComputeStage.cpp:1450-1708, weight 1 or its sigmoid

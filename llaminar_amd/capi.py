@@ -59,6 +59,8 @@ SIGNATURES = {
     "llam_ql_moe_router_logits": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_route_ex": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "llam_ql_moe_route": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "llam_ql_moe_route_quantize": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p,
+                                            c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_moe_gate_up": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                      c_int, c_int, c_int, c_void_p]),
     "llam_ql_swiglu_quantize": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
@@ -277,6 +279,23 @@ def moe_route(logits, top_k: int, normalize: bool = True, stream=None, ids=None,
     assert ids.shape == weights.shape and ids.shape[0] == T and ids.is_contiguous() and weights.is_contiguous()
     _check(load().llam_ql_moe_route_ex(_ptr(logits), T, E, top_k, int(normalize), _ptr(ids), _ptr(weights),
                                        ids.shape[1], _dev(logits), _stream(stream)), "moe_route")
+    return ids, weights
+
+
+def moe_route_quantize(logits, top_k: int, hidden, q8_out, normalize: bool = True, stream=None, ids=None,
+                       weights=None):
+    """moe_route and quantize_q8_1(hidden) in one launch."""
+    import torch
+
+    T, E = logits.shape
+    if ids is None:
+        ids = torch.empty(T, top_k, dtype=torch.int32, device=logits.device)
+        weights = torch.empty(T, top_k, dtype=torch.float32, device=logits.device)
+    assert ids.shape == weights.shape and ids.shape[0] == T and ids.is_contiguous() and weights.is_contiguous()
+    assert hidden.shape[0] == T and hidden.is_contiguous()
+    _check(load().llam_ql_moe_route_quantize(_ptr(logits), T, E, top_k, int(normalize), _ptr(ids), _ptr(weights),
+                                             ids.shape[1], _ptr(hidden), hidden.shape[1], _ptr(q8_out), _dev(logits),
+                                             _stream(stream)), "moe_route_quantize")
     return ids, weights
 
 

@@ -38,11 +38,28 @@ namespace llamql
         return r;
     }
 
+    // Workgroups past the tokens (optional) quantise `q_blocks` 32-element blocks of q_x to Q8_1
+    // with the stand-alone quantiser's arithmetic: the hidden state the expert GEMVs read does
+    // not depend on the routing, so its quantiser rides in the same launch.
     template <int PER>
     __global__ void __launch_bounds__(WAVE)
-        moe_route_kernel(const float *__restrict__ logits, int n_experts, int top_k, int normalize,
-                         int32_t *__restrict__ ids, float *__restrict__ weights, int slot_stride)
+        moe_route_kernel(const float *__restrict__ logits, int n_tokens, int n_experts, int top_k, int normalize,
+                         int32_t *__restrict__ ids, float *__restrict__ weights, int slot_stride,
+                         const float4 *__restrict__ q_x, uint32_t *__restrict__ q_out, long q_blocks)
     {
+        if ((int)blockIdx.x >= n_tokens) // uniform
+        {
+            const long lane_global = (long)((int)blockIdx.x - n_tokens) * WAVE + threadIdx.x;
+            const long blk = lane_global >> 3;
+            if (blk >= q_blocks)
+                return; // whole 8-lane groups leave together
+            const Q8Lane q = q8_1_quantize_lane(q_x[lane_global]);
+            uint32_t *dst = q_out + blk * 9;
+            dst[1 + (lane_global & 7)] = q.packed;
+            if ((lane_global & 7) == 0)
+                dst[0] = q.head;
+            return;
+        }
         const int t = blockIdx.x;
         const int lane = threadIdx.x;
         const float *l = logits + (size_t)t * n_experts;
@@ -511,42 +528,76 @@ extern "C" bool llam_ql_moe_router_logits(const float *d_hidden, const float *d_
     return launched(fn);
 }
 
+namespace llamql
+{
+    namespace
+    {
+        bool moe_route_run(const char *fn, const float *d_logits, int n_tokens, int n_experts, int top_k,
+                           int normalize, int32_t *d_ids, float *d_weights, int slot_stride, const float *d_x,
+                           void *d_q8, long q_blocks, int device_id, void *stream)
+        {
+            if (n_tokens < 0)
+                return fail(fn, "negative n_tokens");
+            if (n_tokens == 0)
+                return true;
+            if (n_experts < 1 || n_experts > WAVE * ROUTE_MAX_PER_LANE)
+                return fail(fn, "n_experts=%d outside 1..%d", n_experts, WAVE * ROUTE_MAX_PER_LANE);
+            if (top_k < 1 || top_k > n_experts || top_k > 64)
+                return fail(fn, "top_k=%d outside 1..min(n_experts,64)", top_k);
+            if (slot_stride < top_k)
+                return fail(fn, "slot_stride=%d smaller than top_k=%d", slot_stride, top_k);
+            if (!d_logits || !d_ids || !d_weights)
+                return fail(fn, "null pointer");
+            if (!set_device(fn, device_id))
+                return false;
+            const long q_wgs = (q_blocks * 8 + WAVE - 1) / WAVE;
+            if ((long)n_tokens + q_wgs > 0x7FFFFFFFl)
+                return fail(fn, "too much work for one launch");
+            const dim3 grid((unsigned)(n_tokens + q_wgs)), block(WAVE);
+            hipStream_t st = as_stream(stream);
+            const float4 *qx = reinterpret_cast<const float4 *>(d_x);
+            uint32_t *qo = static_cast<uint32_t *>(d_q8);
+            const int per = (n_experts + WAVE - 1) / WAVE;
+            if (per <= 4)
+                hipLaunchKernelGGL((moe_route_kernel<4>), grid, block, 0, st, d_logits, n_tokens, n_experts, top_k,
+                                   normalize, d_ids, d_weights, slot_stride, qx, qo, q_blocks);
+            else if (per <= 8)
+                hipLaunchKernelGGL((moe_route_kernel<8>), grid, block, 0, st, d_logits, n_tokens, n_experts, top_k,
+                                   normalize, d_ids, d_weights, slot_stride, qx, qo, q_blocks);
+            else if (per <= 16)
+                hipLaunchKernelGGL((moe_route_kernel<16>), grid, block, 0, st, d_logits, n_tokens, n_experts, top_k,
+                                   normalize, d_ids, d_weights, slot_stride, qx, qo, q_blocks);
+            else
+                hipLaunchKernelGGL((moe_route_kernel<32>), grid, block, 0, st, d_logits, n_tokens, n_experts, top_k,
+                                   normalize, d_ids, d_weights, slot_stride, qx, qo, q_blocks);
+            return launched(fn);
+        }
+    } // namespace
+} // namespace llamql
+
 extern "C" bool llam_ql_moe_route_ex(const float *d_logits, int n_tokens, int n_experts,
                                      int top_k, int normalize, int32_t *d_ids,
                                      float *d_weights, int slot_stride, int device_id, void *stream)
 {
+    return llamql::moe_route_run("llam_ql_moe_route", d_logits, n_tokens, n_experts, top_k, normalize, d_ids, d_weights,
+                                 slot_stride, nullptr, nullptr, 0, device_id, stream);
+}
+
+extern "C" bool llam_ql_moe_route_quantize(const float *d_logits, int n_tokens, int n_experts, int top_k,
+                                           int normalize, int32_t *d_ids, float *d_weights, int slot_stride,
+                                           const float *d_hidden, int d_model, void *d_q8, int device_id,
+                                           void *stream)
+{
     using namespace llamql;
-    static const char *fn = "llam_ql_moe_route";
-    if (n_tokens < 0)
-        return fail(fn, "negative n_tokens");
-    if (n_tokens == 0)
-        return true;
-    if (n_experts < 1 || n_experts > WAVE * ROUTE_MAX_PER_LANE)
-        return fail(fn, "n_experts=%d outside 1..%d", n_experts, WAVE * ROUTE_MAX_PER_LANE);
-    if (top_k < 1 || top_k > n_experts || top_k > 64)
-        return fail(fn, "top_k=%d outside 1..min(n_experts,64)", top_k);
-    if (slot_stride < top_k)
-        return fail(fn, "slot_stride=%d smaller than top_k=%d", slot_stride, top_k);
-    if (!d_logits || !d_ids || !d_weights)
+    static const char *fn = "llam_ql_moe_route_quantize";
+    if (d_model < 32 || (d_model % 32) != 0)
+        return fail(fn, "d_model=%d must be a positive multiple of 32", d_model);
+    if (n_tokens > 0 && (!d_hidden || !d_q8))
         return fail(fn, "null pointer");
-    if (!set_device(fn, device_id))
-        return false;
-    const dim3 grid((unsigned)n_tokens), block(WAVE);
-    hipStream_t st = as_stream(stream);
-    const int per = (n_experts + WAVE - 1) / WAVE;
-    if (per <= 4)
-        hipLaunchKernelGGL((moe_route_kernel<4>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
-                           d_weights, slot_stride);
-    else if (per <= 8)
-        hipLaunchKernelGGL((moe_route_kernel<8>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
-                           d_weights, slot_stride);
-    else if (per <= 16)
-        hipLaunchKernelGGL((moe_route_kernel<16>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
-                           d_weights, slot_stride);
-    else
-        hipLaunchKernelGGL((moe_route_kernel<32>), grid, block, 0, st, d_logits, n_experts, top_k, normalize, d_ids,
-                           d_weights, slot_stride);
-    return launched(fn);
+    if (n_tokens > 0 && (!aligned16(d_hidden) || !aligned4(d_q8)))
+        return fail(fn, "d_hidden must be 16-byte aligned, d_q8 4-byte aligned");
+    return moe_route_run(fn, d_logits, n_tokens, n_experts, top_k, normalize, d_ids, d_weights, slot_stride, d_hidden,
+                         d_q8, (long)(n_tokens > 0 ? n_tokens : 0) * (d_model / 32), device_id, stream);
 }
 
 extern "C" bool llam_ql_moe_route(const float *d_logits, int n_tokens, int n_experts,

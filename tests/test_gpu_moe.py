@@ -161,6 +161,11 @@ def test_expert_ffn_baseline_shape(capi, dev, oracle, T):
 
     ids, w = capi.moe_route(torch.from_numpy(logits).to(dev), k, True)
     qd = capi.quantize_q8_1(xd)
+    # routing and the quantiser of the hidden state in one launch: the bits of the two calls
+    qd2 = torch.zeros_like(qd)
+    ids2, w2 = capi.moe_route_quantize(torch.from_numpy(logits).to(dev), k, xd, qd2)
+    sync()
+    assert torch.equal(ids2, ids) and torch.equal(w2, w) and torch.equal(qd2, qd)
     gate, up = capi.moe_gate_up(fmt, table, n_exp + 1, ids, qd, T, k, hidden, inter)
     q8a = capi.swiglu_quantize(gate, up)
     out = torch.empty((T, hidden), device=dev)
