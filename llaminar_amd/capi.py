@@ -386,7 +386,8 @@ def rope_inv_freq(head_dim: int, theta: float, device=None):
 
 
 def rope_kv_append(qkv, inv_freq, pos, kcache, vcache, n_heads: int, n_kv: int, head_dim: int, stream=None):
-    """qkv [B, >= (n_heads+2 n_kv)*head_dim] fp32, rotated in place; caches [B, n_kv, cap, head_dim] fp16."""
+    """qkv [B, >= (n_heads+2 n_kv)*head_dim] fp32, rotated in place; kcache [B, n_kv, cap, head_dim],
+    vcache [B, n_kv, head_dim, cap] (dimension-major), both fp16."""
     B = qkv.shape[0]
     cap = kcache.shape[2]
     _check(load().llam_dec_rope_kv_append(_ptr(qkv), _ld(qkv), _ptr(inv_freq), _ptr(pos), _ptr(kcache), _ptr(vcache),
@@ -403,11 +404,13 @@ def attention_scratch(B: int, n_heads: int, head_dim: int, cap: int, device):
 
 def attention(q, kcache, vcache, pos, n_heads: int, n_kv: int, head_dim: int, out=None, scratch=None, stream=None,
               q8_out=None):
-    """out [B, n_heads*head_dim] fp32; q8_out (optional) receives the Q8_1 blocks of the same rows."""
+    """out [B, n_heads*head_dim] fp32; q8_out (optional) receives the Q8_1 blocks of the same rows.
+    kcache [B, n_kv, cap, head_dim], vcache [B, n_kv, head_dim, cap] (dimension-major), both fp16."""
     import torch
 
     B = q.shape[0]
     cap = kcache.shape[2]
+    assert tuple(vcache.shape) == (kcache.shape[0], kcache.shape[1], kcache.shape[3], cap), "V cache is [B, n_kv, head_dim, cap]"
     if out is None:
         out = torch.empty(B, n_heads * head_dim, dtype=torch.float32, device=q.device)
     if scratch is None:

@@ -120,7 +120,8 @@ namespace llamql
 
     // ---- rotary embedding + KV append -----------------------------------------------------
     // One workgroup of head_dim/2 threads per (sequence, head); heads n_heads.. are the K
-    // heads, whose workgroups also copy the matching V head.
+    // heads, whose workgroups also copy the matching V head (K cache [ctx_cap][head_dim] per
+    // head, V cache [head_dim][ctx_cap]).
     __global__ void rope_kv_append_kernel(float *__restrict__ qkv, int ld_qkv, const float *__restrict__ inv_freq,
                                           const int32_t *__restrict__ pos, __half *__restrict__ kcache,
                                           __half *__restrict__ vcache, int n_heads, int n_kv, int head_dim,
@@ -149,32 +150,47 @@ namespace llamql
         kcache[at + i] = __float2half_rn(r0);
         kcache[at + i + half_dim] = __float2half_rn(r1);
         const float *vhead = row + (size_t)(n_heads + n_kv + kh) * head_dim;
-        vcache[at + i] = __float2half_rn(vhead[i]);
-        vcache[at + i + half_dim] = __float2half_rn(vhead[i + half_dim]);
+        // V is kept dimension-major, [head_dim][ctx_cap]: the attention kernel reads eight
+        // consecutive positions of one dimension as one 16-byte matrix operand
+        __half *vcol = vcache + ((size_t)b * n_kv + kh) * head_dim * ctx_cap + p;
+        vcol[(size_t)i * ctx_cap] = __float2half_rn(vhead[i]);
+        vcol[(size_t)(i + half_dim) * ctx_cap] = __float2half_rn(vhead[i + half_dim]);
     }
 
     // ---- attention --------------------------------------------------------------------------
     // Workgroup = (chunk of ATT_CHUNK = 128 cache positions, KV head, sequence); its G = n_heads/n_kv
-    // query heads share every K and V row it reads.  Sixteen lanes cover the 128 columns of
-    // a row (8 fp16 = 16 bytes each), so a wavefront takes four positions per pass.
-    //   pass 1: scores s[p][g] = q_g . K[p] / sqrt(d)          -> LDS
+    // query heads share every K and V element it reads.  Each of the four wavefronts takes 32
+    // positions and runs both products on the matrix unit (v_mfma_f32_16x16x32_f16, fp32 sums):
+    //   scores  S[head][pos] = sum_d Q[head][d] K[pos][d]     A = Q rows (heads, padded to 16),
+    //                                                          B = K rows as columns: lane (pos, g)
+    //                                                          holds 8 dims of its position
     //   softmax statistics of the chunk per head: m = max, e = exp(s - m), l = sum e
-    //   pass 2: o_g = sum_p e[p][g] V[p]                       -> partial result per chunk
+    //   output  O[head][d] = sum_pos e[head][pos] V[pos][d]   A = e rows, B = V columns: lane (d, g)
+    //                                                          holds 8 positions of its dim, which
+    //                                                          are contiguous in the V cache's
+    //                                                          [head_dim][ctx_cap] layout
+    // K and V are exact fp16 operands.  The fp32 factors (Q, e) enter as the sum of two fp16 numbers,
+    // high part and remainder, so every product is that of the fp32 value to about 2^-22.
     // A second kernel merges the chunks: o = sum_c o_c exp(m_c - M) / sum_c l_c exp(m_c - M).
     constexpr int ATT_CHUNK = 128;
     constexpr int ATT_THREADS = 256;
     constexpr int ATT_HD = 128;
-    constexpr int ATT_ROWS = (ATT_THREADS / WAVE) * 4; // position rows in flight per workgroup
+    constexpr int ATT_WAVES = ATT_THREADS / WAVE;
+    constexpr int ATT_PER_WAVE = ATT_CHUNK / ATT_WAVES; // 32 positions: two score tiles, one output step
+    constexpr float ATT_P_SCALE = 1024.0f;              // e <= 1 is split after scaling: small weights stay normal fp16
 
-    __device__ __forceinline__ void unpack_row8(const uint4 &raw, float (&v)[8])
+    typedef _Float16 att_v8h __attribute__((ext_vector_type(8)));
+    typedef float att_v4f __attribute__((ext_vector_type(4)));
+
+    // x = hi + lo up to 2^-22 |x|, both fp16 (the remainder is exact in fp32)
+    __device__ __forceinline__ void att_split(const float (&x)[8], att_v8h &hi, att_v8h &lo)
     {
-        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 8; ++j)
         {
-            const float2 f = __half22float2(h[j]);
-            v[2 * j] = f.x;
-            v[2 * j + 1] = f.y;
+            const _Float16 h = (_Float16)x[j];
+            hi[j] = h;
+            lo[j] = (_Float16)(x[j] - (float)h);
         }
     }
 
@@ -185,86 +201,83 @@ namespace llamql
                                  float *__restrict__ part_o, float *__restrict__ part_ml, int n_heads, int n_kv,
                                  int ctx_cap, int n_chunks)
     {
-        // scores [ATT_CHUNK][G], then the partial output rows [ATT_ROWS][G][ATT_HD]
-        extern __shared__ __attribute__((aligned(16))) float att_lds[];
-        float(*s_sc)[G] = reinterpret_cast<float(*)[G]>(att_lds);
-        float(*s_o)[G][ATT_HD] = reinterpret_cast<float(*)[G][ATT_HD]>(att_lds + ATT_CHUNK * G);
+        __shared__ __attribute__((aligned(16))) float s_sc[G][ATT_CHUNK];       // scores, then e
+        __shared__ __attribute__((aligned(16))) float s_o[ATT_WAVES][G][ATT_HD]; // per-wavefront outputs
         const int chunk = blockIdx.x, kh = blockIdx.y, b = blockIdx.z;
         const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
-        const int col = (lane & 15) * 8, prow = lane >> 4;
+        const int n = lane & 15, gq = lane >> 4; // matrix-unit lane: row/column n, k-group gq
         const int last = pos[b] < ctx_cap - 1 ? pos[b] : ctx_cap - 1; // newest position, inclusive
         const int p0 = chunk * ATT_CHUNK;
         const size_t out_base = ((size_t)b * n_heads + (size_t)kh * G) * n_chunks + chunk;
         if (p0 > last)
             return; // no position in this chunk yet: the merge does not read it
         const __half *kbase = kcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
-        const __half *vbase = vcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
+        const __half *vbase = vcache + ((size_t)b * n_kv + kh) * ATT_HD * ctx_cap;
+        const int pw = p0 + wave * ATT_PER_WAVE; // first position of this wavefront
 
-        float qv[G][8];
-        const float scale = 0.08838834764831845f; // 1/sqrt(128)
+        // Every K and V element this wavefront will need is requested before the first use.
+        // K: tile t holds positions pw + 16 t + n, step s the dims 32 s + 8 gq .. + 7.
+        uint4 kraw[2][4];
 #pragma unroll
-        for (int g = 0; g < G; ++g)
+        for (int t = 0; t < 2; ++t)
         {
-            const float *qh = q + (size_t)b * ld_q + (size_t)(kh * G + g) * ATT_HD + col;
-            const float4 a = *reinterpret_cast<const float4 *>(qh);
-            const float4 c = *reinterpret_cast<const float4 *>(qh + 4);
-            qv[g][0] = a.x * scale, qv[g][1] = a.y * scale, qv[g][2] = a.z * scale, qv[g][3] = a.w * scale;
-            qv[g][4] = c.x * scale, qv[g][5] = c.y * scale, qv[g][6] = c.z * scale, qv[g][7] = c.w * scale;
+            const int p = pw + 16 * t + n;
+            const __half *row = kbase + (size_t)(p <= last ? p : last) * ATT_HD + 8 * gq; // rows past the end: weight 0
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                kraw[t][s] = *reinterpret_cast<const uint4 *>(row + 32 * s);
+        }
+        // V: column tile ct holds dims 16 ct + n, positions pw + 8 gq .. + 7 (a group that starts
+        // past the newest position is read at the newest one's group; the mask below clears it)
+        uint4 vraw[8];
+        const int pg = pw + 8 * gq;
+        {
+            const __half *colp = vbase + (size_t)n * ctx_cap + (pg <= last ? pg : (last & ~7));
+#pragma unroll
+            for (int ct = 0; ct < 8; ++ct)
+                vraw[ct] = *reinterpret_cast<const uint4 *>(colp + (size_t)(16 * ct) * ctx_cap);
         }
 
-        // Every row this wavefront will need, K and V, is requested before the first use:
-        // one round trip to memory instead of one per pass over four positions.
-        constexpr int PER_WAVE = ATT_CHUNK / (ATT_THREADS / WAVE); // positions per wavefront
-        constexpr int ITERS = PER_WAVE / 4;
-        uint4 kraw[ITERS], vraw[ITERS];
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it)
+        // Q rows: lane (head n, gq) holds dims 32 s + 8 gq .. + 7, scaled by 1/sqrt(128)
+        att_v8h qhi[4], qlo[4];
         {
-            const int p = p0 + wave * PER_WAVE + it * 4 + prow;
-            const size_t at = (size_t)(p <= last ? p : last) * ATT_HD + col; // rows past the end: weight 0
-            kraw[it] = *reinterpret_cast<const uint4 *>(kbase + at);
-        }
+            const float scale = 0.08838834764831845f;
+            const float *qh = q + (size_t)b * ld_q + (size_t)(kh * G + (n < G ? n : 0)) * ATT_HD + 8 * gq;
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it)
-        {
-            const int p = p0 + wave * PER_WAVE + it * 4 + prow;
-            const size_t at = (size_t)(p <= last ? p : last) * ATT_HD + col;
-            vraw[it] = *reinterpret_cast<const uint4 *>(vbase + at);
+            for (int s = 0; s < 4; ++s)
+            {
+                const float4 a = *reinterpret_cast<const float4 *>(qh + 32 * s);
+                const float4 c = *reinterpret_cast<const float4 *>(qh + 32 * s + 4);
+                const float live = n < G ? scale : 0.0f; // rows past the group's heads are zero
+                const float x[8] = {a.x * live, a.y * live, a.z * live, a.w * live,
+                                    c.x * live, c.y * live, c.z * live, c.w * live};
+                att_split(x, qhi[s], qlo[s]);
+            }
         }
 
-        // pass 1
+        // scores: lane (position n of tile t, gq) receives heads 4 gq .. 4 gq + 3
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it)
+        for (int t = 0; t < 2; ++t)
         {
-            const int pl = wave * PER_WAVE + it * 4 + prow;
+            att_v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+            {
+                const att_v8h kv = __builtin_bit_cast(att_v8h, kraw[t][s]);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qhi[s], kv, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qlo[s], kv, acc, 0, 0, 0);
+            }
+            const int pl = wave * ATT_PER_WAVE + 16 * t + n;
             const bool valid = p0 + pl <= last;
-            float kv[8];
-            unpack_row8(kraw[it], kv);
-            float s[G];
 #pragma unroll
-            for (int g = 0; g < G; ++g)
-            {
-                float a = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    a = fmaf(qv[g][j], kv[j], a);
-                a += dpp_f32<DPP_QUAD_XOR1>(a);
-                a += dpp_f32<DPP_QUAD_XOR2>(a);
-                a += dpp_f32<DPP_ROW_HALF_MIRROR>(a);
-                a += dpp_f32<DPP_ROW_MIRROR>(a);
-                s[g] = valid ? a : -INFINITY;
-            }
-            if ((lane & 15) == 0)
-            {
-#pragma unroll
-                for (int g = 0; g < G; ++g)
-                    s_sc[pl][g] = s[g];
-            }
+            for (int r = 0; r < 4; ++r)
+                if (4 * gq + r < G)
+                    s_sc[4 * gq + r][pl] = valid ? acc[r] : -INFINITY;
         }
         __syncthreads();
 
         // statistics: wavefront w takes heads w, w + 4, ...
-        for (int g = wave; g < G; g += ATT_THREADS / WAVE)
+        for (int g = wave; g < G; g += ATT_WAVES)
         {
             constexpr int PER_LANE = ATT_CHUNK / WAVE;
             float sc[PER_LANE];
@@ -272,7 +285,7 @@ namespace llamql
 #pragma unroll
             for (int k = 0; k < PER_LANE; ++k)
             {
-                sc[k] = s_sc[lane + WAVE * k][g];
+                sc[k] = s_sc[g][lane + WAVE * k];
                 mx = fmaxf(mx, sc[k]);
             }
 #pragma unroll
@@ -283,7 +296,7 @@ namespace llamql
             for (int k = 0; k < PER_LANE; ++k)
             {
                 const float e = expf(sc[k] - mx); // position p0 is valid: mx is finite
-                s_sc[lane + WAVE * k][g] = e;
+                s_sc[g][lane + WAVE * k] = e;
                 l += e;
             }
 #pragma unroll
@@ -297,36 +310,41 @@ namespace llamql
         }
         __syncthreads();
 
-        // pass 2
-        float o[G][8];
-#pragma unroll
-        for (int g = 0; g < G; ++g)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                o[g][j] = 0.0f;
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it)
+        // output: A = e rows, lane (head n, gq) holds positions pw + 8 gq .. + 7
+        att_v8h phi, plo;
         {
-            const int pl = wave * PER_WAVE + it * 4 + prow;
-            float vv[8];
-            unpack_row8(vraw[it], vv);
-#pragma unroll
-            for (int g = 0; g < G; ++g)
-            {
-                const float w = s_sc[pl][g];
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    o[g][j] = fmaf(w, vv[j], o[g][j]);
-            }
+            float x[8];
+            const float4 *src = reinterpret_cast<const float4 *>(&s_sc[n < G ? n : 0][wave * ATT_PER_WAVE + 8 * gq]);
+            const float4 a = src[0], c = src[1];
+            const float live = n < G ? ATT_P_SCALE : 0.0f;
+            x[0] = a.x * live, x[1] = a.y * live, x[2] = a.z * live, x[3] = a.w * live;
+            x[4] = c.x * live, x[5] = c.y * live, x[6] = c.z * live, x[7] = c.w * live;
+            att_split(x, phi, plo);
         }
-        // the sixteen partial rows of the workgroup (four position rows in each of four
-        // wavefronts) meet in LDS; thread t then sums four columns of one head
-#pragma unroll
-        for (int g = 0; g < G; ++g)
+        // V elements of positions past the newest one may be anything, NaN included: clear them
+        uint4 keep;
         {
-            float4 *dst = reinterpret_cast<float4 *>(&s_o[wave * 4 + prow][g][col]);
-            dst[0] = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
-            dst[1] = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
+            const int left = last - pg; // halves 0 .. left of the group are live
+            uint32_t m[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                m[j] = (2 * j <= left ? 0x0000ffffu : 0u) | (2 * j + 1 <= left ? 0xffff0000u : 0u);
+            keep = make_uint4(m[0], m[1], m[2], m[3]);
+        }
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct)
+        {
+            uint4 v = vraw[ct];
+            v.x &= keep.x, v.y &= keep.y, v.z &= keep.z, v.w &= keep.w;
+            const att_v8h vv = __builtin_bit_cast(att_v8h, v);
+            att_v4f o = {0.0f, 0.0f, 0.0f, 0.0f};
+            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi, vv, o, 0, 0, 0);
+            o = __builtin_amdgcn_mfma_f32_16x16x32_f16(plo, vv, o, 0, 0, 0);
+            // lane (dim 16 ct + n, gq) holds heads 4 gq .. 4 gq + 3
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (4 * gq + r < G)
+                    s_o[wave][4 * gq + r][16 * ct + n] = o[r] * (1.0f / ATT_P_SCALE);
         }
         __syncthreads();
         for (int i = threadIdx.x; i < G * (ATT_HD / 4); i += ATT_THREADS)
@@ -334,9 +352,9 @@ namespace llamql
             const int g = i / (ATT_HD / 4), c4 = (i % (ATT_HD / 4)) * 4;
             float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
-            for (int r = 0; r < ATT_ROWS; ++r)
+            for (int w = 0; w < ATT_WAVES; ++w)
             {
-                const float4 v = *reinterpret_cast<const float4 *>(&s_o[r][g][c4]);
+                const float4 v = *reinterpret_cast<const float4 *>(&s_o[w][g][c4]);
                 a.x += v.x, a.y += v.y, a.z += v.z, a.w += v.w;
             }
             *reinterpret_cast<float4 *>(part_o + (out_base + (size_t)g * n_chunks) * ATT_HD + c4) = a;
@@ -348,11 +366,7 @@ namespace llamql
                                   const __half *vc, const int32_t *pos, float *part_o, float *part_ml, int n_heads,
                                   int n_kv, int ctx_cap, int n_chunks)
     {
-        constexpr size_t lds = (size_t)(ATT_CHUNK * G + ATT_ROWS * G * ATT_HD) * sizeof(float);
-        static LdsGrant grant;
-        if (lds > 64 * 1024)
-            (void)allow_lds(grant, reinterpret_cast<const void *>(&attention_partial_kernel<G>), lds);
-        hipLaunchKernelGGL(attention_partial_kernel<G>, grid, dim3(ATT_THREADS), lds, st, q, ld_q, kc, vc, pos, part_o,
+        hipLaunchKernelGGL(attention_partial_kernel<G>, grid, dim3(ATT_THREADS), 0, st, q, ld_q, kc, vc, pos, part_o,
                            part_ml, n_heads, n_kv, ctx_cap, n_chunks);
     }
 
@@ -637,6 +651,8 @@ extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kca
         (d_out && !aligned4(d_out)) || (d_q8_out && !aligned4(d_q8_out)) ||
         !aligned16(d_scratch))
         return fail(fn, "misaligned pointer (q, caches and scratch 16-byte, out 4-byte)");
+    if ((ctx_cap % 8) != 0)
+        return fail(fn, "ctx_cap=%d must be a multiple of 8 (the V cache is read eight positions at a time)", ctx_cap);
     const int n_chunks = (ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
     if (n_chunks > ATT_MAX_CHUNKS || B > 65535)
         return fail(fn, "ctx_cap=%d beyond %d positions, or too many sequences", ctx_cap, ATT_MAX_CHUNKS * ATT_CHUNK);

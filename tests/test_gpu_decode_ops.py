@@ -80,13 +80,13 @@ def test_rope_kv_append(capi, dev, oracle, B, n_heads, n_kv):
     inv = capi.rope_inv_freq(hd, theta, dev)
     assert np.array_equal(inv.cpu().numpy(), oracle.rope_inv_freq(hd, theta))
     kc = torch.zeros(B, n_kv, cap, hd, dtype=torch.float16, device=dev)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(B, n_kv, hd, cap, dtype=torch.float16, device=dev)   # V is kept [head_dim][ctx_cap]
     qd = torch.from_numpy(qkv).to(dev)
     capi.rope_kv_append(qd, inv, torch.from_numpy(pos_h).to(dev), kc, vc, n_heads, n_kv, hd)
     sync()
     got = qd.cpu().numpy()
     kg = kc.cpu().numpy().view(np.uint16)
-    vg = vc.cpu().numpy().view(np.uint16)
+    vg = np.ascontiguousarray(vc.cpu().numpy().view(np.uint16).transpose(0, 1, 3, 2))   # as [cap][hd]
     f = oracle.rope_inv_freq(hd, theta)
     for b in range(B):
         ke = np.zeros((n_kv, cap, hd), np.uint16)
@@ -105,8 +105,9 @@ def test_rope_kv_append(capi, dev, oracle, B, n_heads, n_kv):
 
 
 @pytest.mark.parametrize("B,n_heads,n_kv,cap,positions", [
-    (1, 64, 8, 4224, [4095]), (2, 64, 8, 600, [0, 599]), (3, 8, 2, 300, [127, 128, 255]),
-    (2, 4, 4, 130, [5, 129]), (1, 2, 1, 128, [64])])
+    (1, 64, 8, 4224, [4095]), (2, 64, 8, 600, [0, 599]), (3, 8, 2, 304, [127, 128, 255]),
+    (2, 4, 4, 136, [5, 129]), (1, 2, 1, 128, [64]), (4, 16, 2, 264, [6, 7, 8, 263]),
+    (2, 3, 3, 40, [30, 39])])
 def test_attention_decode(capi, dev, oracle, B, n_heads, n_kv, cap, positions):
     import torch
 
@@ -114,7 +115,10 @@ def test_attention_decode(capi, dev, oracle, B, n_heads, n_kv, cap, positions):
     g = torch.Generator(device=dev)
     g.manual_seed(cap + n_heads)
     kc = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
-    vc = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
+    vc = torch.randn(B, n_kv, hd, cap, device=dev, generator=g).half()
+    for b, p in enumerate(positions):      # what lies past the newest position must not matter, whatever it is
+        kc[b, :, p + 1:] = float("nan")
+        vc[b, :, :, p + 1:] = float("nan")
     q = torch.randn(B, n_heads * hd + 32, device=dev, generator=g) * 1.5
     pos = torch.tensor(positions, dtype=torch.int32, device=dev)
     out = torch.full((B, n_heads * hd + 4), float("nan"), device=dev)
@@ -126,7 +130,8 @@ def test_attention_decode(capi, dev, oracle, B, n_heads, n_kv, cap, positions):
     assert np.array_equal(q8.cpu().numpy().reshape(B, n_heads * hd // 32, 36),
                           oracle.quantize(np.ascontiguousarray(got[:, :n_heads * hd])))
     assert np.isnan(got[:, n_heads * hd:]).all()
-    kh, vh = kc.cpu().numpy().view(np.uint16), vc.cpu().numpy().view(np.uint16)
+    kh = kc.cpu().numpy().view(np.uint16)
+    vh = np.ascontiguousarray(vc.cpu().numpy().view(np.uint16).transpose(0, 1, 3, 2))   # the oracle's [cap][hd]
     qh = q.cpu().numpy()
     for b in range(B):
         exp = oracle.attention_decode(qh[b, :n_heads * hd], kh[b], vh[b], positions[b], n_heads, n_kv, hd)
@@ -141,16 +146,29 @@ def test_attention_follows_the_position_in_memory(capi, dev, oracle):
     g = torch.Generator(device=dev)
     g.manual_seed(3)
     kc = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
-    vc = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
+    vc = torch.randn(B, n_kv, hd, cap, device=dev, generator=g).half()
     q = torch.randn(B, n_heads * hd, device=dev, generator=g)
     pos = torch.zeros(1, dtype=torch.int32, device=dev)
+    v_rows = np.ascontiguousarray(vc.cpu().numpy().view(np.uint16)[0].transpose(0, 2, 1))
     scratch = capi.attention_scratch(B, n_heads, hd, cap, dev)
     for p in (0, 1, 130, 511):
         pos.fill_(p)
         out = capi.attention(q, kc, vc, pos, n_heads, n_kv, hd, scratch=scratch)
         exp = oracle.attention_decode(q.cpu().numpy()[0], kc.cpu().numpy().view(np.uint16)[0],
-                                      vc.cpu().numpy().view(np.uint16)[0], p, n_heads, n_kv, hd)
+                                      v_rows, p, n_heads, n_kv, hd)
         assert close(out.cpu().numpy()[0], exp, 1e-5), p
+
+
+def test_attention_refuses_a_cache_it_cannot_read(capi, dev):
+    import torch
+
+    hd, cap = 128, 132   # not a multiple of 8: a 16-byte group of V positions would straddle two dimensions
+    kc = torch.zeros(1, 1, cap, hd, dtype=torch.float16, device=dev)
+    vc = torch.zeros(1, 1, hd, cap, dtype=torch.float16, device=dev)
+    q = torch.zeros(1, hd, device=dev)
+    pos = torch.zeros(1, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        capi.attention(q, kc, vc, pos, 1, 1, hd)
 
 
 def test_argmax(capi, dev, oracle):

@@ -72,7 +72,8 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
         vc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
     for l in range(shape.n_layers):
         dec.buffer("kcache", l).copy_(torch.from_numpy(kc_h[:, l]).to(dev))
-        dec.buffer("vcache", l).copy_(torch.from_numpy(vc_h[:, l]).to(dev))
+        # the device keeps V dimension-major: [batch][n_kv][head_dim][cap]
+        dec.buffer("vcache", l).copy_(torch.from_numpy(np.ascontiguousarray(vc_h[:, l].transpose(0, 1, 3, 2))).to(dev))
     dec.set_state(ids, pos)
     kc_u, vc_u = kc_h.view(np.uint16).copy(), vc_h.view(np.uint16).copy()
 
@@ -97,6 +98,9 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
                 kg = dec.buffer("kcache", l)[b, :, int(pos[b]) + step].cpu().numpy().astype(np.float32)
                 ke = kc_u[b, l, :, int(pos[b]) + step].view(np.float16).astype(np.float32)
                 assert np.abs(kg - ke).max() <= 2e-2 * max(np.abs(ke).max(), 1.0), (step, b, l)
+                vg = dec.buffer("vcache", l)[b, :, :, int(pos[b]) + step].cpu().numpy().astype(np.float32)
+                ve = vc_u[b, l, :, int(pos[b]) + step].view(np.float16).astype(np.float32)
+                assert np.abs(vg - ve).max() <= 2e-2 * max(np.abs(ve).max(), 1.0), (step, b, l)
         ids = new_ids.copy()   # both sides continue from the device's tokens
     dec.close()
 
@@ -155,6 +159,8 @@ def test_bad_configurations_are_refused(capi, dev):
     assert not L.llam_decoder_create(bad)
     ok = decoder.Config(512, 4, 4, 128, 512, 1000, 1, 16, 9, 1e6, 1e-6, 0)        # batch 9
     assert not L.llam_decoder_create(ok)
+    assert not L.llam_decoder_create(decoder.Config(512, 4, 4, 128, 512, 1000, 1, 12, 1, 1e6, 1e-6, 0))
+    assert b"multiple of 8" in L.llam_decoder_last_error()                        # 12 cache positions
     h = L.llam_decoder_create(decoder.Config(512, 4, 4, 128, 512, 1000, 1, 16, 1, 1e6, 1e-6, 0))
     assert h
     assert not L.llam_decoder_step(h, None) and b"globals not set" in L.llam_decoder_last_error()
