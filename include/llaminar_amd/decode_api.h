@@ -91,6 +91,29 @@ bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kcache, const 
                         float *d_scratch, int B, int n_heads, int n_kv, int head_dim, int ctx_cap,
                         int device_id, void *stream);
 
+/* d_table[b][i] = (cos, sin) of float(d_pos[b]) * d_inv_freq[i], i < head_dim/2, as two
+ * floats each: the rotation of a decode step, which is the same in every layer.  One call
+ * per step serves the llam_dec_rope_attention call of every layer.  d_table holds
+ * B * head_dim floats. */
+bool llam_dec_rope_table(const int32_t *d_pos, const float *d_inv_freq, float *d_table, int B,
+                         int head_dim, int device_id, void *stream);
+
+/* llam_dec_rope_kv_append and llam_dec_attention as one operator, two launches instead of
+ * three: d_qkv is the unrotated row of the fused Q/K/V projection (layout as for
+ * llam_dec_rope_kv_append), d_rope_table what llam_dec_rope_table wrote for the same
+ * d_pos.  Every workgroup of the attention kernel rotates the query heads it serves; the
+ * one whose chunk of the cache holds position d_pos[b] rotates the K head, rounds it and
+ * the V head to fp16, appends both to the caches and attends over them.
+ * Results and cache contents are those of the two calls in sequence, with one difference:
+ * d_qkv is only read (the rotated Q is not written back).  Same limits as llam_dec_attention.
+ * Replaces RoPEStage + KVCacheAppendStage + the decode attention stage
+ * (src/v2/models/qwen/QwenGraphBase.cpp:2691-2790;
+ * src/v2/kernels/cpu/attention/CPUFlashAttentionKernelT.h:507-545). */
+bool llam_dec_rope_attention(const float *d_qkv, int ld_qkv, const float *d_rope_table,
+                             const int32_t *d_pos, void *d_kcache, void *d_vcache, float *d_out,
+                             int ld_out, void *d_q8_out, float *d_scratch, int B, int n_heads,
+                             int n_kv, int head_dim, int ctx_cap, int device_id, void *stream);
+
 /* Scratch bytes llam_dec_argmax needs for its per-workgroup partial results. */
 size_t llam_dec_argmax_scratch_bytes(int B, int n);
 

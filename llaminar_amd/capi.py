@@ -77,6 +77,9 @@ SIGNATURES = {
     "llam_dec_attention_scratch_floats": (c_size_t, [c_int, c_int, c_int, c_int]),
     "llam_dec_attention": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                     c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_dec_rope_table": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_dec_rope_attention": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_dec_argmax_scratch_bytes": (c_size_t, [c_int, c_int]),
     "llam_dec_argmax": (c_bool, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
 }
@@ -418,6 +421,36 @@ def attention(q, kcache, vcache, pos, n_heads: int, n_kv: int, head_dim: int, ou
     _check(load().llam_dec_attention(_ptr(q), _ld(q), _ptr(kcache), _ptr(vcache), _ptr(pos), _ptr(out), _ld(out),
                                      _ptr(q8_out), _ptr(scratch), B, n_heads, n_kv, head_dim, cap, _dev(q),
                                      _stream(stream)), "attention")
+    return out
+
+
+def rope_table(pos, inv_freq, head_dim: int, stream=None):
+    """[B, head_dim/2, 2] fp32: cos and sin of pos[b] * inv_freq[i], for rope_attention."""
+    import torch
+
+    B = pos.shape[0]
+    table = torch.empty(B, head_dim // 2, 2, dtype=torch.float32, device=pos.device)
+    _check(load().llam_dec_rope_table(_ptr(pos), _ptr(inv_freq), _ptr(table), B, head_dim, _dev(pos), _stream(stream)),
+           "rope_table")
+    return table
+
+
+def rope_attention(qkv, table, pos, kcache, vcache, n_heads: int, n_kv: int, head_dim: int, out=None,
+                   scratch=None, stream=None, q8_out=None):
+    """rope_kv_append and attention as one operator; qkv [B, >= (n_heads+2 n_kv)*head_dim] is only read,
+    table = rope_table(pos, inv_freq, head_dim)."""
+    import torch
+
+    B = qkv.shape[0]
+    cap = kcache.shape[2]
+    assert tuple(vcache.shape) == (kcache.shape[0], kcache.shape[1], kcache.shape[3], cap), "V cache is [B, n_kv, head_dim, cap]"
+    if out is None:
+        out = torch.empty(B, n_heads * head_dim, dtype=torch.float32, device=qkv.device)
+    if scratch is None:
+        scratch = attention_scratch(B, n_heads, head_dim, cap, qkv.device)
+    _check(load().llam_dec_rope_attention(_ptr(qkv), _ld(qkv), _ptr(table), _ptr(pos), _ptr(kcache), _ptr(vcache),
+                                          _ptr(out), _ld(out), _ptr(q8_out), _ptr(scratch), B, n_heads, n_kv,
+                                          head_dim, cap, _dev(qkv), _stream(stream)), "rope_attention")
     return out
 
 

@@ -122,6 +122,14 @@ namespace llamql
     // One workgroup of head_dim/2 threads per (sequence, head); heads n_heads.. are the K
     // heads, whose workgroups also copy the matching V head (K cache [ctx_cap][head_dim] per
     // head, V cache [head_dim][ctx_cap]).
+    // (x0, x1) rotated by the angle whose cosine and sine are c and s; every product and sum is
+    // rounded on its own, as in the scalar host code (apply_rope_to_head_scalar)
+    __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float &r0, float &r1)
+    {
+        r0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
+        r1 = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+    }
+
     __global__ void rope_kv_append_kernel(float *__restrict__ qkv, int ld_qkv, const float *__restrict__ inv_freq,
                                           const int32_t *__restrict__ pos, __half *__restrict__ kcache,
                                           __half *__restrict__ vcache, int n_heads, int n_kv, int head_dim,
@@ -135,8 +143,8 @@ namespace llamql
         const float c = cosf(angle), s = sinf(angle);
         float *head = row + (size_t)h * head_dim;
         const float x0 = head[i], x1 = head[i + half_dim];
-        const float r0 = x0 * c - x1 * s;
-        const float r1 = x0 * s + x1 * c;
+        float r0, r1;
+        rope_pair(x0, x1, c, s, r0, r1);
         if (h < n_heads)
         {
             head[i] = r0;
@@ -157,6 +165,15 @@ namespace llamql
         vcol[(size_t)(i + half_dim) * ctx_cap] = __float2half_rn(vhead[i + half_dim]);
     }
 
+    // cos and sin of float(pos[b]) * inv_freq[i]: the same for every layer of a decode step
+    __global__ void rope_table_kernel(const int32_t *__restrict__ pos, const float *__restrict__ inv_freq,
+                                      float2 *__restrict__ table, int half_dim)
+    {
+        const int b = blockIdx.x, i = threadIdx.x;
+        const float angle = (float)pos[b] * inv_freq[i];
+        table[(size_t)b * half_dim + i] = make_float2(cosf(angle), sinf(angle));
+    }
+
     // ---- attention --------------------------------------------------------------------------
     // Workgroup = (chunk of ATT_CHUNK = 128 cache positions, KV head, sequence); its G = n_heads/n_kv
     // query heads share every K and V element it reads.  Each of the four wavefronts takes 32
@@ -170,14 +187,15 @@ namespace llamql
     //                                                          are contiguous in the V cache's
     //                                                          [head_dim][ctx_cap] layout
     // K and V are exact fp16 operands.  The fp32 factors (Q, e) enter as the sum of two fp16 numbers,
-    // high part and remainder, so every product is that of the fp32 value to about 2^-22.
+    // high part and remainder, after a scaling by a power of two that keeps the remainders out of
+    // the subnormal range, so every product is that of the fp32 value to about 2^-22.
     // A second kernel merges the chunks: o = sum_c o_c exp(m_c - M) / sum_c l_c exp(m_c - M).
     constexpr int ATT_CHUNK = 128;
     constexpr int ATT_THREADS = 256;
     constexpr int ATT_HD = 128;
     constexpr int ATT_WAVES = ATT_THREADS / WAVE;
     constexpr int ATT_PER_WAVE = ATT_CHUNK / ATT_WAVES; // 32 positions: two score tiles, one output step
-    constexpr float ATT_P_SCALE = 1024.0f;              // e <= 1 is split after scaling: small weights stay normal fp16
+    constexpr float ATT_P_SCALE = 32768.0f;             // e <= 1 is split after scaling: remainders stay normal fp16
 
     typedef _Float16 att_v8h __attribute__((ext_vector_type(8)));
     typedef float att_v4f __attribute__((ext_vector_type(4)));
@@ -194,15 +212,23 @@ namespace llamql
         }
     }
 
-    template <int G>
+    // ROPE: q is the unrotated output row of the fused Q/K/V projection (Q heads, then K heads,
+    // then V heads).  The workgroup rotates its G query heads itself, and the workgroup whose chunk
+    // holds the new position also rotates that K head, rounds it and the V head to fp16, appends
+    // both to the caches and uses them in place of what the caches held: the work of
+    // rope_kv_append_kernel without its launch.  The cosines and sines come from the table that
+    // rope_table_kernel writes once per decode step (computing them here, in every workgroup of
+    // every layer, cost more than the launch saved).
+    template <int G, bool ROPE>
     __global__ void __launch_bounds__(ATT_THREADS)
-        attention_partial_kernel(const float *__restrict__ q, int ld_q, const __half *__restrict__ kcache,
-                                 const __half *__restrict__ vcache, const int32_t *__restrict__ pos,
-                                 float *__restrict__ part_o, float *__restrict__ part_ml, int n_heads, int n_kv,
-                                 int ctx_cap, int n_chunks)
+        attention_partial_kernel(const float *__restrict__ q, int ld_q, const float2 *__restrict__ rope_table,
+                                 __half *__restrict__ kcache, __half *__restrict__ vcache,
+                                 const int32_t *__restrict__ pos, float *__restrict__ part_o,
+                                 float *__restrict__ part_ml, int n_heads, int n_kv, int ctx_cap, int n_chunks)
     {
         __shared__ __attribute__((aligned(16))) float s_sc[G][ATT_CHUNK];       // scores, then e
-        __shared__ __attribute__((aligned(16))) float s_o[ATT_WAVES][G][ATT_HD]; // per-wavefront outputs
+        __shared__ __attribute__((aligned(16))) float s_o[ATT_WAVES][G][ATT_HD]; // per-wavefront outputs; first the rotated Q
+        __shared__ __attribute__((aligned(16))) __half s_new[2][ATT_HD];         // the appended K and V rows
         const int chunk = blockIdx.x, kh = blockIdx.y, b = blockIdx.z;
         const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6;
         const int n = lane & 15, gq = lane >> 4; // matrix-unit lane: row/column n, k-group gq
@@ -214,6 +240,38 @@ namespace llamql
         const __half *kbase = kcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
         const __half *vbase = vcache + ((size_t)b * n_kv + kh) * ATT_HD * ctx_cap;
         const int pw = p0 + wave * ATT_PER_WAVE; // first position of this wavefront
+
+        // ROPE: the few values of the rotation are requested first: loads return in order, and the
+        // rotation then runs while the K and V loads behind them are in flight
+        constexpr int HALF = ATT_HD / 2;
+        constexpr int Q_PAIRS = (G * HALF + ATT_THREADS - 1) / ATT_THREADS; // head pairs per thread
+        const int ri = threadIdx.x & (HALF - 1);
+        float2 rope_cs = make_float2(1.0f, 0.0f);
+        float rope_x0[Q_PAIRS], rope_x1[Q_PAIRS], new_x0 = 0.0f, new_x1 = 0.0f;
+        int rope_p = -1;
+        bool owner = false;
+        if (ROPE)
+        {
+            rope_p = pos[b];
+            owner = rope_p >= 0 && rope_p < ctx_cap && rope_p / ATT_CHUNK == chunk; // the append is this workgroup's
+            rope_cs = rope_table[(size_t)b * HALF + ri];
+            const float *row = q + (size_t)b * ld_q;
+#pragma unroll
+            for (int k = 0; k < Q_PAIRS; ++k)
+            {
+                const int g = threadIdx.x / HALF + k * (ATT_THREADS / HALF);
+                const float *head = row + (size_t)(kh * G + (g < G ? g : 0)) * ATT_HD;
+                rope_x0[k] = head[ri];
+                rope_x1[k] = head[ri + HALF];
+            }
+            if (owner && threadIdx.x < ATT_HD) // first 64 threads: the K head, next 64: the V head
+            {
+                const float *head = row + (size_t)(n_heads + (threadIdx.x >= HALF ? n_kv : 0) + kh) * ATT_HD;
+                new_x0 = head[ri];
+                new_x1 = head[ri + HALF];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
 
         // Every K and V element this wavefront will need is requested before the first use.
         // K: tile t holds positions pw + 16 t + n, step s the dims 32 s + 8 gq .. + 7.
@@ -238,20 +296,108 @@ namespace llamql
                 vraw[ct] = *reinterpret_cast<const uint4 *>(colp + (size_t)(16 * ct) * ctx_cap);
         }
 
-        // Q rows: lane (head n, gq) holds dims 32 s + 8 gq .. + 7, scaled by 1/sqrt(128)
+        if (ROPE)
+        {
+            __builtin_amdgcn_sched_barrier(0);
+            const int p = rope_p, i = ri;
+            const float c = rope_cs.x, sn = rope_cs.y;
+            float(*s_q)[ATT_HD] = s_o[0];
+#pragma unroll
+            for (int k = 0; k < Q_PAIRS; ++k)
+            {
+                const int g = threadIdx.x / HALF + k * (ATT_THREADS / HALF);
+                if (g < G)
+                    rope_pair(rope_x0[k], rope_x1[k], c, sn, s_q[g][i], s_q[g][i + HALF]);
+            }
+            if (owner && threadIdx.x < ATT_HD)
+            {
+                const bool is_v = threadIdx.x >= HALF;
+                float r0 = new_x0, r1 = new_x1;
+                if (!is_v)
+                    rope_pair(new_x0, new_x1, c, sn, r0, r1);
+                const __half h0 = __float2half_rn(r0), h1 = __float2half_rn(r1);
+                s_new[is_v][i] = h0;
+                s_new[is_v][i + HALF] = h1;
+                if (is_v)
+                {
+                    __half *vcol = vcache + ((size_t)b * n_kv + kh) * ATT_HD * ctx_cap + p;
+                    vcol[(size_t)i * ctx_cap] = h0;
+                    vcol[(size_t)(i + HALF) * ctx_cap] = h1;
+                }
+                else
+                {
+                    __half *krow = kcache + (((size_t)b * n_kv + kh) * ctx_cap + p) * ATT_HD;
+                    krow[i] = h0;
+                    krow[i + HALF] = h1;
+                }
+            }
+            __syncthreads();
+            if (owner)
+            {
+                // the new row replaces what was loaded for its position
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    if (pw + 16 * t + n == p)
+                    {
+#pragma unroll
+                        for (int s = 0; s < 4; ++s)
+                            kraw[t][s] = *reinterpret_cast<const uint4 *>(&s_new[0][32 * s + 8 * gq]);
+                    }
+                const int j = p - pg;
+                if (j >= 0 && j < 8)
+                {
+                    const uint32_t sh = (j & 1) * 16, clear = ~(0xffffu << sh);
+#pragma unroll
+                    for (int ct = 0; ct < 8; ++ct)
+                    {
+                        const uint32_t nv = (uint32_t)__half_as_ushort(s_new[1][16 * ct + n]) << sh;
+                        uint32_t *w = reinterpret_cast<uint32_t *>(&vraw[ct]);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            if (k == (j >> 1))
+                                w[k] = (w[k] & clear) | nv;
+                    }
+                }
+            }
+        }
+
+        // Q rows: lane (head n, gq) holds dims 32 s + 8 gq .. + 7, scaled by 1/sqrt(128) and by the
+        // power of two that brings the head's largest magnitude to [2^14, 2^15): the matrix unit
+        // treats subnormal fp16 operands as zero, and the remainders of values near 0.1 would be
+        // subnormal.  q_down undoes the power of two on the scores, exactly.
         att_v8h qhi[4], qlo[4];
+        float q_down;
         {
             const float scale = 0.08838834764831845f;
-            const float *qh = q + (size_t)b * ld_q + (size_t)(kh * G + (n < G ? n : 0)) * ATT_HD + 8 * gq;
+            const float *qh = ROPE ? &s_o[0][n < G ? n : 0][8 * gq]
+                                   : q + (size_t)b * ld_q + (size_t)(kh * G + (n < G ? n : 0)) * ATT_HD + 8 * gq;
+            const float live = n < G ? scale : 0.0f; // rows past the group's heads are zero
+            float x[4][8];
+            float mx = 0.0f;
 #pragma unroll
             for (int s = 0; s < 4; ++s)
             {
                 const float4 a = *reinterpret_cast<const float4 *>(qh + 32 * s);
                 const float4 c = *reinterpret_cast<const float4 *>(qh + 32 * s + 4);
-                const float live = n < G ? scale : 0.0f; // rows past the group's heads are zero
-                const float x[8] = {a.x * live, a.y * live, a.z * live, a.w * live,
-                                    c.x * live, c.y * live, c.z * live, c.w * live};
-                att_split(x, qhi[s], qlo[s]);
+                x[s][0] = a.x * live, x[s][1] = a.y * live, x[s][2] = a.z * live, x[s][3] = a.w * live;
+                x[s][4] = c.x * live, x[s][5] = c.y * live, x[s][6] = c.z * live, x[s][7] = c.w * live;
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    mx = fmaxf(mx, fabsf(x[s][j]));
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE)); // the head's four lanes agree
+            int sh = 15 - __builtin_amdgcn_frexp_expf(mx); // mx = f 2^e with 0.5 <= f < 1
+            sh = sh > 100 ? 100 : (sh < -100 ? -100 : sh);
+            const float up = ldexpf(1.0f, sh);
+            q_down = ldexpf(1.0f, -sh);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+            {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    x[s][j] *= up;
+                att_split(x[s], qhi[s], qlo[s]);
             }
         }
 
@@ -271,8 +417,11 @@ namespace llamql
             const bool valid = p0 + pl <= last;
 #pragma unroll
             for (int r = 0; r < 4; ++r)
+            {
+                const float down = __shfl(q_down, 4 * gq + r, WAVE); // lane h < 16 holds head h
                 if (4 * gq + r < G)
-                    s_sc[4 * gq + r][pl] = valid ? acc[r] : -INFINITY;
+                    s_sc[4 * gq + r][pl] = valid ? acc[r] * down : -INFINITY;
+            }
         }
         __syncthreads();
 
@@ -362,12 +511,16 @@ namespace llamql
     }
 
     template <int G>
-    void attention_partial_launch(dim3 grid, hipStream_t st, const float *q, int ld_q, const __half *kc,
-                                  const __half *vc, const int32_t *pos, float *part_o, float *part_ml, int n_heads,
-                                  int n_kv, int ctx_cap, int n_chunks)
+    void attention_partial_launch(dim3 grid, hipStream_t st, const float *q, int ld_q, const float2 *inv_freq,
+                                  __half *kc, __half *vc, const int32_t *pos, float *part_o, float *part_ml,
+                                  int n_heads, int n_kv, int ctx_cap, int n_chunks)
     {
-        hipLaunchKernelGGL(attention_partial_kernel<G>, grid, dim3(ATT_THREADS), 0, st, q, ld_q, kc, vc, pos, part_o,
-                           part_ml, n_heads, n_kv, ctx_cap, n_chunks);
+        if (inv_freq)
+            hipLaunchKernelGGL((attention_partial_kernel<G, true>), grid, dim3(ATT_THREADS), 0, st, q, ld_q, inv_freq, kc,
+                               vc, pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
+        else
+            hipLaunchKernelGGL((attention_partial_kernel<G, false>), grid, dim3(ATT_THREADS), 0, st, q, ld_q, inv_freq, kc,
+                               vc, pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks);
     }
 
     // One workgroup of 128 threads per (sequence, head): thread k weighs chunk k, then thread c
@@ -626,56 +779,107 @@ extern "C" size_t llam_dec_attention_scratch_floats(int B, int n_heads, int head
     return (size_t)B * n_heads * chunks * ((size_t)head_dim + 2);
 }
 
+namespace
+{
+    // llam_dec_attention (no table of cosines and sines: d_inv_freq == nullptr, d_q holds rotated query heads) and
+    // llam_dec_rope_attention (d_q is the unrotated Q/K/V row) share everything but the kernel variant.
+    bool attention_run(const char *fn, const float *d_q, int ld_q, const float2 *d_inv_freq, void *d_kcache,
+                       void *d_vcache, const int32_t *d_pos, float *d_out, int ld_out, void *d_q8_out,
+                       float *d_scratch, int B, int n_heads, int n_kv, int head_dim, int ctx_cap, int device_id,
+                       void *stream)
+    {
+        using namespace llamql;
+        if (B < 0 || n_heads < 1 || n_kv < 1 || ctx_cap < 1)
+            return fail(fn, "bad size");
+        if (B == 0)
+            return true;
+        if (head_dim != ATT_HD)
+            return fail(fn, "head_dim=%d: only 128 is built", head_dim);
+        if ((n_heads % n_kv) != 0)
+            return fail(fn, "n_heads=%d not a multiple of n_kv=%d", n_heads, n_kv);
+        const int G = n_heads / n_kv;
+        if (G != 1 && G != 2 && G != 4 && G != 8)
+            return fail(fn, "n_heads/n_kv=%d: only 1, 2, 4 and 8 are built", G);
+        const int width = (d_inv_freq ? n_heads + 2 * n_kv : n_heads) * head_dim;
+        if (ld_q < width || (d_out && ld_out < n_heads * head_dim))
+            return fail(fn, "row strides smaller than the rows");
+        if (!d_q || !d_kcache || !d_vcache || !d_pos || (!d_out && !d_q8_out) || !d_scratch)
+            return fail(fn, "null pointer");
+        if (!aligned16(d_q) || (ld_q % 4) != 0 || !aligned16(d_kcache) || !aligned16(d_vcache) ||
+            (d_out && !aligned4(d_out)) || (d_q8_out && !aligned4(d_q8_out)) || !aligned16(d_scratch))
+            return fail(fn, "misaligned pointer (q, caches and scratch 16-byte, out 4-byte)");
+        if ((ctx_cap % 8) != 0)
+            return fail(fn, "ctx_cap=%d must be a multiple of 8 (the V cache is read eight positions at a time)",
+                        ctx_cap);
+        const int n_chunks = (ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
+        if (n_chunks > ATT_MAX_CHUNKS || B > 65535)
+            return fail(fn, "ctx_cap=%d beyond %d positions, or too many sequences", ctx_cap,
+                        ATT_MAX_CHUNKS * ATT_CHUNK);
+        if (!set_device(fn, device_id))
+            return false;
+        float *part_o = d_scratch;
+        float *part_ml = d_scratch + (size_t)B * n_heads * n_chunks * ATT_HD;
+        __half *kc = static_cast<__half *>(d_kcache);
+        __half *vc = static_cast<__half *>(d_vcache);
+        const dim3 grid(n_chunks, n_kv, B);
+        hipStream_t st = as_stream(stream);
+        switch (G)
+        {
+        case 1: attention_partial_launch<1>(grid, st, d_q, ld_q, d_inv_freq, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
+        case 2: attention_partial_launch<2>(grid, st, d_q, ld_q, d_inv_freq, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
+        case 4: attention_partial_launch<4>(grid, st, d_q, ld_q, d_inv_freq, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
+        default: attention_partial_launch<8>(grid, st, d_q, ld_q, d_inv_freq, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
+        }
+        if (!launched(fn))
+            return false;
+        hipLaunchKernelGGL(attention_merge_kernel, dim3(n_heads, B), dim3(ATT_HD), 0, st, part_o, part_ml, d_pos, d_out,
+                           ld_out, static_cast<uint32_t *>(d_q8_out), n_heads, n_chunks, ctx_cap);
+        return launched(fn);
+    }
+} // namespace
+
 extern "C" bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kcache, const void *d_vcache,
                                    const int32_t *d_pos, float *d_out, int ld_out, void *d_q8_out,
                                    float *d_scratch, int B, int n_heads, int n_kv, int head_dim, int ctx_cap,
                                    int device_id, void *stream)
 {
-    static const char *fn = "llam_dec_attention";
-    if (B < 0 || n_heads < 1 || n_kv < 1 || ctx_cap < 1)
+    // without the table of frequencies the kernel only reads the caches
+    return attention_run("llam_dec_attention", d_q, ld_q, nullptr, const_cast<void *>(d_kcache),
+                         const_cast<void *>(d_vcache), d_pos, d_out, ld_out, d_q8_out, d_scratch, B, n_heads, n_kv,
+                         head_dim, ctx_cap, device_id, stream);
+}
+
+extern "C" bool llam_dec_rope_table(const int32_t *d_pos, const float *d_inv_freq, float *d_table, int B, int head_dim,
+                                    int device_id, void *stream)
+{
+    static const char *fn = "llam_dec_rope_table";
+    if (B < 0 || head_dim < 2 || (head_dim % 2) != 0 || head_dim / 2 > 1024)
         return fail(fn, "bad size");
     if (B == 0)
         return true;
-    if (head_dim != ATT_HD)
-        return fail(fn, "head_dim=%d: only 128 is built", head_dim);
-    if ((n_heads % n_kv) != 0)
-        return fail(fn, "n_heads=%d not a multiple of n_kv=%d", n_heads, n_kv);
-    const int G = n_heads / n_kv;
-    if (G != 1 && G != 2 && G != 4 && G != 8)
-        return fail(fn, "n_heads/n_kv=%d: only 1, 2, 4 and 8 are built", G);
-    if (ld_q < n_heads * head_dim || (d_out && ld_out < n_heads * head_dim))
-        return fail(fn, "row strides smaller than n_heads * head_dim");
-    if (!d_q || !d_kcache || !d_vcache || !d_pos || (!d_out && !d_q8_out) || !d_scratch)
+    if (!d_pos || !d_inv_freq || !d_table)
         return fail(fn, "null pointer");
-    if (!aligned16(d_q) || (ld_q % 4) != 0 || !aligned16(d_kcache) || !aligned16(d_vcache) ||
-        (d_out && !aligned4(d_out)) || (d_q8_out && !aligned4(d_q8_out)) ||
-        !aligned16(d_scratch))
-        return fail(fn, "misaligned pointer (q, caches and scratch 16-byte, out 4-byte)");
-    if ((ctx_cap % 8) != 0)
-        return fail(fn, "ctx_cap=%d must be a multiple of 8 (the V cache is read eight positions at a time)", ctx_cap);
-    const int n_chunks = (ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
-    if (n_chunks > ATT_MAX_CHUNKS || B > 65535)
-        return fail(fn, "ctx_cap=%d beyond %d positions, or too many sequences", ctx_cap, ATT_MAX_CHUNKS * ATT_CHUNK);
+    if (((uintptr_t)d_table & 7) != 0)
+        return fail(fn, "table not 8-byte aligned");
     if (!set_device(fn, device_id))
         return false;
-    float *part_o = d_scratch;
-    float *part_ml = d_scratch + (size_t)B * n_heads * n_chunks * ATT_HD;
-    const __half *kc = static_cast<const __half *>(d_kcache);
-    const __half *vc = static_cast<const __half *>(d_vcache);
-    const dim3 grid(n_chunks, n_kv, B);
-    hipStream_t st = as_stream(stream);
-    switch (G)
-    {
-    case 1: attention_partial_launch<1>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
-    case 2: attention_partial_launch<2>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
-    case 4: attention_partial_launch<4>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
-    default: attention_partial_launch<8>(grid, st, d_q, ld_q, kc, vc, d_pos, part_o, part_ml, n_heads, n_kv, ctx_cap, n_chunks); break;
-    }
-    if (!launched(fn))
-        return false;
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(n_heads, B), dim3(ATT_HD), 0, st, part_o, part_ml, d_pos, d_out,
-                       ld_out, static_cast<uint32_t *>(d_q8_out), n_heads, n_chunks, ctx_cap);
+    hipLaunchKernelGGL(rope_table_kernel, dim3(B), dim3(head_dim / 2), 0, as_stream(stream), d_pos, d_inv_freq,
+                       reinterpret_cast<float2 *>(d_table), head_dim / 2);
     return launched(fn);
+}
+
+extern "C" bool llam_dec_rope_attention(const float *d_qkv, int ld_qkv, const float *d_rope_table, const int32_t *d_pos,
+                                        void *d_kcache, void *d_vcache, float *d_out, int ld_out, void *d_q8_out,
+                                        float *d_scratch, int B, int n_heads, int n_kv, int head_dim, int ctx_cap,
+                                        int device_id, void *stream)
+{
+    static const char *fn = "llam_dec_rope_attention";
+    if (!d_rope_table)
+        return fail(fn, "null pointer");
+    if (((uintptr_t)d_rope_table & 7) != 0)
+        return fail(fn, "table not 8-byte aligned");
+    return attention_run(fn, d_qkv, ld_qkv, reinterpret_cast<const float2 *>(d_rope_table), d_kcache, d_vcache, d_pos,
+                         d_out, ld_out, d_q8_out, d_scratch, B, n_heads, n_kv, head_dim, ctx_cap, device_id, stream);
 }
 
 extern "C" size_t llam_dec_argmax_scratch_bytes(int B, int n)

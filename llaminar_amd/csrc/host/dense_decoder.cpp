@@ -51,7 +51,7 @@ namespace
 
         int32_t *ids = nullptr, *pos = nullptr;
         float *x = nullptr, *delta = nullptr, *qkv = nullptr, *attn = nullptr, *gate = nullptr, *up = nullptr;
-        float *logits = nullptr, *inv_freq = nullptr, *att_scratch = nullptr;
+        float *logits = nullptr, *inv_freq = nullptr, *rope_table = nullptr, *att_scratch = nullptr;
         void *q8_h = nullptr, *q8_attn = nullptr, *q8_act = nullptr, *argmax_scratch = nullptr;
         std::vector<void *> kcache, vcache;
 
@@ -135,6 +135,7 @@ extern "C" void *llam_decoder_create(const llam_decoder_config *c)
               d->alloc(d->attn, (size_t)B * d->qdim() * 4) && d->alloc(d->gate, (size_t)B * F * 4) &&
               d->alloc(d->up, (size_t)B * F * 4) && d->alloc(d->logits, (size_t)B * c->vocab * 4) &&
               d->alloc(d->inv_freq, (size_t)(c->head_dim / 2) * 4) &&
+              d->alloc(d->rope_table, (size_t)B * c->head_dim * 4) &&
               d->alloc(d->att_scratch,
                        llam_dec_attention_scratch_floats(B, c->n_heads, c->head_dim, c->ctx_cap) * 4) &&
               d->alloc(d->q8_h, q8_bytes(B, wide)) && d->alloc(d->q8_attn, q8_bytes(B, d->qdim())) &&
@@ -253,6 +254,9 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
 
     if (!forward(fn, llam_dec_embed_q4k(d->globals.embed_q4k, c.vocab, d->ids, d->x, B, H, H, dev, stream)))
         return false;
+    // the rotation of this step's positions, shared by every layer
+    if (!forward(fn, llam_dec_rope_table(d->pos, d->inv_freq, d->rope_table, B, c.head_dim, dev, stream)))
+        return false;
     for (int l = 0; l < c.n_layers; ++l)
     {
         const llam_decoder_layer &w = d->layers[l];
@@ -266,13 +270,11 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
         qkv[2] = llam_ql_proj{w.wv, d->qkv + QD + KV, KV, ldqkv, w.fmt_v};
         if (!forward(fn, llam_ql_gemv_fused(qkv, 3, d->q8_h, B, H, dev, stream)))
             return false;
-        if (!forward(fn, llam_dec_rope_kv_append(d->qkv, ldqkv, d->inv_freq, d->pos, d->kcache[l], d->vcache[l], B,
-                                                 c.n_heads, c.n_kv, c.head_dim, c.ctx_cap, dev, stream)))
-            return false;
-        // the attention output leaves the merge kernel as Q8_1 blocks: the output projection's
-        // quantiser costs no launch of its own
-        if (!forward(fn, llam_dec_attention(d->qkv, ldqkv, d->kcache[l], d->vcache[l], d->pos, nullptr, 0, d->q8_attn,
-                                            d->att_scratch, B, c.n_heads, c.n_kv, c.head_dim, c.ctx_cap, dev, stream)))
+        // rotary embedding, the cache append and the attention in one operator; its output leaves the
+        // merge kernel as Q8_1 blocks: the output projection's quantiser costs no launch of its own
+        if (!forward(fn, llam_dec_rope_attention(d->qkv, ldqkv, d->rope_table, d->pos, d->kcache[l], d->vcache[l], nullptr,
+                                                 0, d->q8_attn, d->att_scratch, B, c.n_heads, c.n_kv, c.head_dim,
+                                                 c.ctx_cap, dev, stream)))
             return false;
         if (!forward(fn, llam_ql_gemv(w.fmt_o, w.wo, d->q8_attn, d->delta, B, H, QD, H, dev, stream)))
             return false;
