@@ -63,7 +63,7 @@ namespace llamql
             }
             // a following run in the other quad-lane format joins the launch (Q and K with V)
             if constexpr (F::USE_QUAD)
-                if (n >= 1 && n < QUAD_MAX_PROJ && M <= 4 && src.kind != ACT_SRC_SWIGLU)
+                if (n >= 1 && n < QUAD_MAX_PROJ && src.kind != ACT_SRC_SWIGLU)
                 {
                     typedef typename Other<F>::type G;
                     int nb = 0;

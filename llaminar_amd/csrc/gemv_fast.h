@@ -331,6 +331,10 @@ namespace llamql
     // Batches of 5..8 rows on rows of 8 super-blocks or more (the activations of the whole batch
     // and the wavefronts' bounce buffers must fit the 160 KiB of LDS) go to the matrix-unit
     // kernel, in formats that have one.
+    // below this many rows a Q4_K matrix at batch 5..8 stays on the quad-lane kernel (measured on
+    // 5120-column matrices: 1024 rows 10.6 us on the matrix unit, 8192 rows and more faster there)
+    constexpr int MFMA_MIN_ROWS = 4096;
+
     template <class F>
     bool mfma_eligible(int M, int N, int K)
     {
@@ -343,7 +347,9 @@ namespace llamql
             // (any row length works here: long rows are walked in chunks)
             return quad_lds_bytes(M, K / 256) > QUAD_MAX_LDS && Q6KQuad::addressable(N, K / 256);
         else
-            return mfma_max_slices(K / 256) >= 1;
+            // a matrix of few 32-row tiles leaves most compute units idle here: the quad-lane kernel
+            // spreads it over all of them (and shares its launch with a following Q6_K matrix)
+            return mfma_max_slices(K / 256) >= 1 && N >= MFMA_MIN_ROWS;
     }
 
     template <int SRC>
@@ -487,7 +493,7 @@ namespace llamql
     }
 
     // The same over two runs of matrices in two formats (na of FA, then nb of FB; na + nb <=
-    // QUAD_MAX_PROJ), M <= 4, Q8_1 or plain fp32 activations.  The second format starts at a
+    // QUAD_MAX_PROJ), Q8_1 or plain fp32 activations.  The second format starts at a
     // workgroup boundary.
     template <class FA, class FB>
     bool gemv_quad_dual(const char *fn, const QuadProj *pr, int na, int nb, const ActSource &src, int M, int K,

@@ -797,7 +797,11 @@ namespace llamql
         case 1: gemv_quad_dual_launch_m<QA, QB, 1>(src, grid, block, lds, st, a); break;
         case 2: gemv_quad_dual_launch_m<QA, QB, 2>(src, grid, block, lds, st, a); break;
         case 3: gemv_quad_dual_launch_m<QA, QB, 3>(src, grid, block, lds, st, a); break;
-        default: gemv_quad_dual_launch_m<QA, QB, 4>(src, grid, block, lds, st, a); break;
+        case 4: gemv_quad_dual_launch_m<QA, QB, 4>(src, grid, block, lds, st, a); break;
+        case 5: gemv_quad_dual_launch_m<QA, QB, 5>(src, grid, block, lds, st, a); break;
+        case 6: gemv_quad_dual_launch_m<QA, QB, 6>(src, grid, block, lds, st, a); break;
+        case 7: gemv_quad_dual_launch_m<QA, QB, 7>(src, grid, block, lds, st, a); break;
+        default: gemv_quad_dual_launch_m<QA, QB, 8>(src, grid, block, lds, st, a); break;
         }
     }
 

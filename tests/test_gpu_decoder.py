@@ -105,15 +105,17 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
     dec.close()
 
 
-def test_step_replays_as_a_graph(capi, dev):
-    """A captured step replayed three times gives the tokens of three eager steps."""
+@pytest.mark.parametrize("batch", [2, 6])
+def test_step_replays_as_a_graph(capi, dev, batch):
+    """A captured step replayed gives the tokens of eager steps (batch 6: the matrix-unit kernels)."""
     import torch
 
     from llaminar_amd.decoder import DenseDecoder, Shape
 
     shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
-    dec = DenseDecoder(shape, 2, 160, dev, seed=6)
-    ids0, pos0 = np.array([7, 1999], np.int32), np.array([0, 0], np.int32)
+    dec = DenseDecoder(shape, batch, 160, dev, seed=6)
+    ids0 = np.array([7, 1999, 3, 1024, 77, 500][:batch], np.int32)
+    pos0 = np.array([0, 0, 5, 17, 1, 130][:batch], np.int32)
 
     def run(n, graph):
         for l in range(shape.n_layers):

@@ -146,17 +146,18 @@ def test_fused_projections(capi, dev, oracle):
         assert rel_err(got[:, c0:c0 + N], oracle.gemm(fmt, W, K, q8)) <= TOL[fmt] * 1e-2
 
 
-@pytest.mark.parametrize("M", [1, 2, 5, 8])
+@pytest.mark.parametrize("M", [1, 2, 5, 7, 8])
 def test_fused_groups_equal_separate_calls(capi, dev, M):
     """Neighbouring projections of one format share a launch; every output must carry the
-    bits of its own llam_ql_gemv call.  Groups here: five Q4_K (four + one), two Q6_K, an
-    IQ3_S (never grouped), then a Q4_K again; ragged N, a strided output."""
+    bits of its own llam_ql_gemv call.  Groups here: five Q4_K (four + one, the last joined by
+    two Q6_K in a two-format launch), an IQ3_S (never grouped), a Q4_K again, and a Q4_K of
+    4096 rows, which from batch 5 on runs alone on the matrix unit; ragged N, a strided output."""
     import torch
 
     K = 5120
     qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(8, K, 23)).to(dev))
     specs = [(FMT_Q4_K, 700), (FMT_Q4_K, 37), (FMT_Q4_K, 1), (FMT_Q4_K, 2048), (FMT_Q4_K, 129),
-             (FMT_Q6_K, 300), (FMT_Q6_K, 64), (FMT_IQ3_S, 96), (FMT_Q4_K, 250)]
+             (FMT_Q6_K, 300), (FMT_Q6_K, 64), (FMT_IQ3_S, 96), (FMT_Q4_K, 250), (FMT_Q4_K, 4096), (FMT_Q6_K, 40)]
     total = sum(n for _, n in specs)
     out = torch.full((M, total + 5), float("nan"), device=dev)
     projs, singles, col = [], [], 0
