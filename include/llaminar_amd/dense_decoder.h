@@ -17,7 +17,7 @@
  *               down = Wdown Q8_1(silu(Wgate h2) * (Wup h2))
  *   logits = Wlm Q8_1(rmsnorm(x += down) * final_norm) ; ids = argmax(logits) ; pos += 1
  *
- * llam_decoder_step() only enqueues kernels on the given stream (about 12 per layer):
+ * llam_decoder_step() only enqueues kernels on the given stream (9 per layer up to batch 4):
  * no allocation, no synchronisation, no host read of device data.  Token ids and
  * positions live in device memory and are advanced by the step itself, so a step can
  * be captured in a HIP graph once and replayed for every following token.

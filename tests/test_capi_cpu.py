@@ -32,6 +32,21 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(capi.SIGNATURES), "capi.SIGNATURES out of step with the headers"
 
 
+def test_host_library_exports_every_declared_symbol():
+    """dense_decoder.h and weights_io.h are the C ABI of the host library."""
+    from llaminar_amd import capi, decoder
+
+    capi.load()
+    assert decoder.HOST_LIB.exists(), "build the library first: python -m llaminar_amd.build"
+    lib = ctypes.CDLL(str(decoder.HOST_LIB))
+    text = "".join((ROOT / "include" / "llaminar_amd" / h).read_text() for h in ("dense_decoder.h", "weights_io.h"))
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(llam_(?:decoder|gguf|weights|prepared)_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) >= 20, names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/ but not exported by the host library"
+
+
 def test_block_layouts_match_header():
     from llaminar_amd import capi
 
