@@ -46,10 +46,13 @@ namespace llamql
 
     // ---- RMSNorm -------------------------------------------------------------------------
     // One workgroup per row.  Pass 1 adds the delta (when given), stores the new residual
-    // and accumulates the sum of squares in double; pass 2 re-reads the row (the same
-    // thread reads what it wrote), scales it and, eight threads per 32-element block,
-    // quantises it.
+    // and accumulates the sum of squares in double; pass 2 scales the row and, eight
+    // threads per 32-element block, quantises it.  A thread keeps its first NORM_KEEP
+    // float4 of the row and of gamma in registers (rows of up to 8192 values: all of
+    // them), so every global load of the kernel is issued before the reduction and pass 2
+    // waits for no memory; longer rows re-read the rest (the same thread reads what it wrote).
     constexpr int NORM_THREADS = 512;
+    constexpr int NORM_KEEP = 4;
 
     __global__ void __launch_bounds__(NORM_THREADS)
         rmsnorm_q8_1_kernel(float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ gamma,
@@ -62,8 +65,46 @@ namespace llamql
         const float4 *drow = delta ? reinterpret_cast<const float4 *>(delta + (size_t)m * H) : nullptr;
         const float4 *g4 = reinterpret_cast<const float4 *>(gamma);
 
+        float4 keep[NORM_KEEP], dk[NORM_KEEP], gk[NORM_KEEP];
+#pragma unroll
+        for (int t = 0; t < NORM_KEEP; ++t)
+        {
+            const int i = threadIdx.x + t * NORM_THREADS;
+            keep[t] = dk[t] = gk[t] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (i < nvec)
+            {
+                keep[t] = row[i];
+                if (drow)
+                    dk[t] = drow[i];
+                gk[t] = g4[i];
+            }
+        }
+
         double acc = 0.0;
-        for (int i = threadIdx.x; i < nvec; i += NORM_THREADS)
+        auto square = [&acc](const float4 &v) {
+            acc += (double)v.x * (double)v.x;
+            acc += (double)v.y * (double)v.y;
+            acc += (double)v.z * (double)v.z;
+            acc += (double)v.w * (double)v.w;
+        };
+#pragma unroll
+        for (int t = 0; t < NORM_KEEP; ++t)
+        {
+            const int i = threadIdx.x + t * NORM_THREADS;
+            if (i < nvec)
+            {
+                if (drow)
+                {
+                    keep[t].x += dk[t].x;
+                    keep[t].y += dk[t].y;
+                    keep[t].z += dk[t].z;
+                    keep[t].w += dk[t].w;
+                    row[i] = keep[t];
+                }
+                square(keep[t]);
+            }
+        }
+        for (int i = threadIdx.x + NORM_KEEP * NORM_THREADS; i < nvec; i += NORM_THREADS)
         {
             float4 v = row[i];
             if (drow)
@@ -75,10 +116,7 @@ namespace llamql
                 v.w += d.w;
                 row[i] = v;
             }
-            acc += (double)v.x * (double)v.x;
-            acc += (double)v.y * (double)v.y;
-            acc += (double)v.z * (double)v.z;
-            acc += (double)v.w * (double)v.w;
+            square(v);
         }
 #pragma unroll
         for (int off = WAVE / 2; off > 0; off >>= 1)
@@ -96,10 +134,7 @@ namespace llamql
 
         float4 *yrow = y ? reinterpret_cast<float4 *>(y + (size_t)m * H) : nullptr;
         uint32_t *qrow = q8 ? q8 + (size_t)m * (H >> 5) * 9 : nullptr;
-        for (int i = threadIdx.x; i < nvec; i += NORM_THREADS) // whole 8-thread groups stay together
-        {
-            const float4 v = row[i];
-            const float4 g = g4[i];
+        auto emit = [&](int i, const float4 &v, const float4 &g) { // whole 8-thread groups stay together
             float4 o;
             o.x = __fmul_rn(__fmul_rn(v.x, inv), g.x);
             o.y = __fmul_rn(__fmul_rn(v.y, inv), g.y);
@@ -115,7 +150,16 @@ namespace llamql
                 if ((i & 7) == 0)
                     dst[0] = q.head;
             }
+        };
+#pragma unroll
+        for (int t = 0; t < NORM_KEEP; ++t)
+        {
+            const int i = threadIdx.x + t * NORM_THREADS;
+            if (i < nvec)
+                emit(i, keep[t], gk[t]);
         }
+        for (int i = threadIdx.x + NORM_KEEP * NORM_THREADS; i < nvec; i += NORM_THREADS)
+            emit(i, row[i], g4[i]);
     }
 
     // ---- rotary embedding + KV append -----------------------------------------------------
@@ -526,6 +570,7 @@ namespace llamql
     // One workgroup of 128 threads per (sequence, head): thread k weighs chunk k, then thread c
     // sums column c over the chunks that hold positions.
     constexpr int ATT_MAX_CHUNKS = 1024; // 131072 cache positions
+    constexpr int ATT_MERGE_KEEP = 40;   // chunks whose partial outputs a thread holds in registers (5120 positions)
 
     __global__ void __launch_bounds__(ATT_HD)
         attention_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml,
@@ -539,6 +584,14 @@ namespace llamql
         const int last = pos[b] < ctx_cap - 1 ? pos[b] : ctx_cap - 1;
         const int used = last < 0 ? 0 : last / ATT_CHUNK + 1; // chunks that were written
         const size_t base = ((size_t)b * n_heads + h) * n_chunks;
+
+        // The first ATT_MERGE_KEEP chunks' column values are requested before anything is
+        // waited for: they do not depend on the weights, and the kernel is then one memory
+        // latency deep instead of one per few chunks.
+        float po[ATT_MERGE_KEEP];
+#pragma unroll
+        for (int k = 0; k < ATT_MERGE_KEEP; ++k)
+            po[k] = k < used ? part_o[(base + k) * ATT_HD + c] : 0.0f;
 
         float mx = -INFINITY;
         for (int k = c; k < used; k += ATT_HD)
@@ -567,8 +620,12 @@ namespace llamql
         const float L = s_red[0] + s_red[1];
 
         float acc = 0.0f;
+#pragma unroll
+        for (int k = 0; k < ATT_MERGE_KEEP; ++k)
+            if (k < used)
+                acc = fmaf(po[k], s_w[k], acc);
 #pragma unroll 4
-        for (int k = 0; k < used; ++k)
+        for (int k = ATT_MERGE_KEEP; k < used; ++k)
             acc = fmaf(part_o[(base + k) * ATT_HD + c], s_w[k], acc);
         const float val = L > 0.0f ? __fdiv_rn(acc, L) : 0.0f; // pos < 0: nothing attended
         if (out)
