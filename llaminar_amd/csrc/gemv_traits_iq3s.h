@@ -5,11 +5,14 @@
 // g in {1,3,..,15} times db = d*(1+2*nib), signed, then scale = max|v|/127 and
 // w = rne(v/scale).  Because v = +-g*db with one db per sub-block this is the pure
 // integer map  w = +-round(g*127/gmax)  (gmax = largest magnitude in the
-// sub-block; never a tie) with  b_scale = f16((gmax*db)/127).  The kernel keeps
-// the eight possible maps (gmax = 1,3,..,15) applied to the whole 512-entry
-// codebook as lookup tables in LDS, so one ds_read_b32 yields four requantised
-// magnitudes; signs are applied with a byte permute.  HBM traffic stays at the
-// format's 110 B per 256 weights (+2 B alignment padding).
+// sub-block; never a tie) with  b_scale = f16((gmax*db)/127).  Every magnitude is odd,
+// g = 2k+1 with k in 0..7, so for a given gmax the map is an 8-entry byte table: the
+// kernel keeps the codebook in LDS as k-bytes (2 KB; bits 28..30 of an entry hold its
+// largest k, so the largest of eight raw entries carries the sub-block's), finds gmax from the eight entries of a sub-block, fetches
+// that gmax's table (two dwords) and applies it with one byte permute per four weights;
+// signs are applied with a second permute whose selector comes from a 16-entry table.
+// One LDS gather per four weights, none of them dependent on another.  HBM traffic stays
+// at the format's 110 B per 256 weights (+2 B alignment padding).
 //
 // Device layout (llam_ql_prepare_weights): three planes over T = N*K/256
 // super-blocks -- qs [T][64], signs [T][32], meta [T][16] = qh[8] scales[4] d[2]
@@ -24,41 +27,55 @@ namespace llamql
 {
     struct IQ3STables
     {
-        uint32_t req[8 * 512]; // req[gi*512 + idx]: bytes round(g*127/(2*gi+1)) of codebook entry idx
-        uint32_t gmax[128];    // byte idx: largest magnitude in codebook entry idx
+        uint32_t cb[512];   // codebook entry idx as bytes k = g >> 1; bits 28..30: the entry's largest k
+        uint32_t map[8][2]; // map[gi]: bytes round((2k+1)*127/(2*gi+1)) for k = 0..7 (k > gi is never looked up)
+        uint32_t sign[16];  // permute selector for a sign nibble: byte b selects byte b, or b+4 (negated) if bit b is set
+        bool odd;           // every codebook magnitude is odd and at most 15
     };
 
     constexpr IQ3STables make_iq3s_tables()
     {
         IQ3STables t{};
+        t.odd = true;
         for (int idx = 0; idx < 512; ++idx)
         {
             const uint32_t g4 = llam_iq3s_grid[idx];
-            uint32_t mx = 0;
+            uint32_t mx = 0, e = 0;
             for (int b = 0; b < 4; ++b)
             {
                 const uint32_t g = (g4 >> (8 * b)) & 0xFFu;
-                if (g > mx)
-                    mx = g;
+                if ((g & 1u) == 0u || g > 15u)
+                    t.odd = false;
+                const uint32_t k = g >> 1;
+                if (k > mx)
+                    mx = k;
+                e |= k << (8 * b);
             }
-            t.gmax[idx >> 2] |= mx << (8 * (idx & 3));
-            for (int gi = 0; gi < 8; ++gi)
+            t.cb[idx] = e | (mx << 28);
+        }
+        for (int gi = 0; gi < 8; ++gi)
+        {
+            const uint32_t gm = 2u * (uint32_t)gi + 1u;
+            for (int k = 0; k < 8; ++k)
             {
-                const uint32_t gm = 2u * (uint32_t)gi + 1u;
-                uint32_t out = 0;
-                for (int b = 0; b < 4; ++b)
-                {
-                    const uint32_t g = (g4 >> (8 * b)) & 0xFFu;
-                    uint32_t q = (2u * g * 127u + gm) / (2u * gm); // round half up; never exactly half
-                    if (q > 127u)
-                        q = 127u; // entries with g > gm are never looked up
-                    out |= q << (8 * b);
-                }
-                t.req[gi * 512 + idx] = out;
+                const uint32_t g = 2u * (uint32_t)k + 1u;
+                uint32_t q = (2u * g * 127u + gm) / (2u * gm); // round half up; never exactly half
+                if (q > 127u)
+                    q = 127u; // g > gm: never looked up
+                t.map[gi][k >> 2] |= q << (8 * (k & 3));
             }
+        }
+        for (uint32_t sg = 0; sg < 16; ++sg)
+        {
+            uint32_t sel = 0x03020100u;
+            for (int b = 0; b < 4; ++b)
+                if ((sg >> b) & 1u)
+                    sel |= 4u << (8 * b);
+            t.sign[sg] = sel;
         }
         return t;
     }
+    static_assert(make_iq3s_tables().odd, "IQ3_S codebook magnitudes must be odd and at most 15");
 
     static __device__ const IQ3STables g_iq3s_tables = make_iq3s_tables();
 
@@ -69,13 +86,13 @@ namespace llamql
         static constexpr bool USE_QUAD = false;
         static constexpr bool USE_MFMA_BATCH = false;  // matrix-unit kernel for 5..8 activation rows
         static constexpr int FAST_MAX_U = 3;          // load batches in flight in the chunked kernel
-        static constexpr int TABLE_BYTES = (int)sizeof(IQ3STables);
+        static constexpr int TABLE_BYTES = (512 + 16 + 16) * 4; // cb, map, sign
 
         __device__ static void stage_tables(void *lds_tab)
         {
             const uint4 *src = reinterpret_cast<const uint4 *>(&g_iq3s_tables);
             uint4 *dst = static_cast<uint4 *>(lds_tab);
-            constexpr int n = (int)(sizeof(IQ3STables) / 16);
+            constexpr int n = TABLE_BYTES / 16;
             for (int i = threadIdx.x; i < n; i += blockDim.x)
                 dst[i] = src[i];
         }
@@ -118,8 +135,8 @@ namespace llamql
         __device__ __forceinline__ static void decode(const Raw &r, int c, v4i &w0, v4i &w1, int &j,
                                                       float &bscale, float &bmin, const void *tab)
         {
-            const uint32_t *req = static_cast<const uint32_t *>(tab);
-            const uint8_t *gmaxb = reinterpret_cast<const uint8_t *>(req + 8 * 512);
+            const uint32_t *cb = static_cast<const uint32_t *>(tab);
+            const uint2 *maps = reinterpret_cast<const uint2 *>(cb + 512);
 
             // picked with a bit mask: a conditional on two members of r would become a load
             // through a computed address and force arrays of Raw into memory
@@ -135,10 +152,16 @@ namespace llamql
                 const uint32_t qsb = ((l < 4 ? r.qs.x : r.qs.y) >> (8 * (l & 3))) & 0xFFu;
                 idx[l] = qsb | (((qh >> l) & 1u) << 8);
             }
-            uint32_t gm = 0;
+            uint32_t e[8];
 #pragma unroll
             for (int l = 0; l < 8; ++l)
-                gm = max(gm, (uint32_t)gmaxb[idx[l]]);
+                e[l] = cb[idx[l]];
+            uint32_t km = 0;
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+                km = max(km, e[l]); // the field above every k byte decides
+            km >>= 28;
+            const uint32_t gm = 2u * km + 1u;
 
             const float db = d * (1.0f + 2.0f * (float)nib);
             const float amax = (float)gm * db;
@@ -148,18 +171,23 @@ namespace llamql
             if (amax < 1e-6f)
                 scale = 0.0f;
 
-            const uint32_t *rq = req + (gm >> 1) * 512;
+            uint2 mp = maps[km];
+            uint32_t sg_all = r.signs;
+            if (scale == 0.0f) // all-zero sub-block: zero magnitudes, and no sign to apply to them
+            {
+                mp = make_uint2(0u, 0u);
+                sg_all = 0u;
+            }
             int ws[8];
 #pragma unroll
             for (int l = 0; l < 8; ++l)
             {
-                const uint32_t w = rq[idx[l]];
-                const uint32_t sg = (r.signs >> (4 * l)) & 0xFu;
+                const uint32_t w = __builtin_amdgcn_perm(mp.y, mp.x, e[l] & 0x07070707u);
+                const uint32_t sg = (sg_all >> (4 * l)) & 0xFu;
                 // bit k of sg -> bit 0 of byte k, then selector byte k = k (keep) or k+4 (negated)
-                const uint32_t spread = (sg * 0x00204081u) & 0x01010101u;
-                const uint32_t sel = 0x03020100u | (spread << 2);
-                const uint32_t neg = 0x01010100u - w; // bytewise -w: every byte of w is in 1..127
-                ws[l] = (scale != 0.0f) ? (int)__builtin_amdgcn_perm(neg, w, sel) : 0;
+                const uint32_t sel = 0x03020100u | (((sg * 0x00204081u) & 0x01010101u) << 2);
+                const uint32_t neg = 0x01010100u - w; // bytewise -w: every byte of w is in 1..127 (or all are 0)
+                ws[l] = (int)__builtin_amdgcn_perm(neg, w, sel);
             }
             w0 = (v4i){ws[0], ws[1], ws[2], ws[3]};
             w1 = (v4i){ws[4], ws[5], ws[6], ws[7]};
