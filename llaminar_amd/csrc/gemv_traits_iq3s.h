@@ -8,9 +8,9 @@
 // sub-block; never a tie) with  b_scale = f16((gmax*db)/127).  Every magnitude is odd,
 // g = 2k+1 with k in 0..7, so for a given gmax the map is an 8-entry byte table: the
 // kernel keeps the codebook in LDS as k-bytes (2 KB; bits 28..30 of an entry hold its
-// largest k, so the largest of eight raw entries carries the sub-block's), finds gmax from the eight entries of a sub-block, fetches
+// largest k, so the largest of a sub-block's eight raw entries carries gmax), fetches
 // that gmax's table (two dwords) and applies it with one byte permute per four weights;
-// signs are applied with a second permute whose selector comes from a 16-entry table.
+// signs are applied with a second permute whose selector is spread out of the sign nibble.
 // One LDS gather per four weights, none of them dependent on another.  HBM traffic stays
 // at the format's 110 B per 256 weights (+2 B alignment padding).
 //
@@ -29,7 +29,6 @@ namespace llamql
     {
         uint32_t cb[512];   // codebook entry idx as bytes k = g >> 1; bits 28..30: the entry's largest k
         uint32_t map[8][2]; // map[gi]: bytes round((2k+1)*127/(2*gi+1)) for k = 0..7 (k > gi is never looked up)
-        uint32_t sign[16];  // permute selector for a sign nibble: byte b selects byte b, or b+4 (negated) if bit b is set
         bool odd;           // every codebook magnitude is odd and at most 15
     };
 
@@ -65,14 +64,6 @@ namespace llamql
                 t.map[gi][k >> 2] |= q << (8 * (k & 3));
             }
         }
-        for (uint32_t sg = 0; sg < 16; ++sg)
-        {
-            uint32_t sel = 0x03020100u;
-            for (int b = 0; b < 4; ++b)
-                if ((sg >> b) & 1u)
-                    sel |= 4u << (8 * b);
-            t.sign[sg] = sel;
-        }
         return t;
     }
     static_assert(make_iq3s_tables().odd, "IQ3_S codebook magnitudes must be odd and at most 15");
@@ -86,7 +77,7 @@ namespace llamql
         static constexpr bool USE_QUAD = false;
         static constexpr bool USE_MFMA_BATCH = false;  // matrix-unit kernel for 5..8 activation rows
         static constexpr int FAST_MAX_U = 3;          // load batches in flight in the chunked kernel
-        static constexpr int TABLE_BYTES = (512 + 16 + 16) * 4; // cb, map, sign
+        static constexpr int TABLE_BYTES = (512 + 16) * 4; // cb, map
 
         __device__ static void stage_tables(void *lds_tab)
         {
