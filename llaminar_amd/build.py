@@ -12,6 +12,7 @@ Usage: ``python -m llaminar_amd.build``
 from __future__ import annotations
 
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -39,6 +40,49 @@ HIP_FLAGS = [
     f"-I{ROOT / 'include'}",
     f"-I{CSRC}",
 ]
+# Register allocation of every kernel is reported by the compiler and checked below.
+RESOURCE_FLAG = "-Rpass-analysis=kernel-resource-usage"
+
+
+class SpillError(RuntimeError):
+    """A kernel needs per-lane scratch memory (register spills)."""
+
+
+def check_kernel_resources(remarks: str, src_name: str) -> dict[str, dict[str, int]]:
+    """Parse hipcc's kernel-resource-usage remarks and refuse any kernel that spills.
+
+    Several kernels issue their global loads as inline assembly and wait for them by
+    hand many instructions later.  The compiler takes the destination registers of such
+    a load as written at the point of issue.  If it has to spill, it may store such a
+    register to scratch straight after the load instruction (before the data has
+    arrived) and hand the register to another value, for instance an address; the
+    load then lands in that value.  Its own scratch loads and stores also count in
+    vmcnt and shift every hand-written ``s_waitcnt vmcnt(n)``.  The kernels are only
+    correct with zero spills, so a spill fails the build instead of the GPU.
+    """
+    usage: dict[str, dict[str, int]] = {}
+    name = None
+    for line in remarks.splitlines():
+        m = re.search(r"remark: Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            usage[name] = {}
+            continue
+        m = re.search(r"remark:\s+(ScratchSize \[bytes/lane\]|VGPRs Spill|SGPRs Spill|VGPRs|Dynamic Stack): (\S+)", line)
+        if m and name is not None:
+            v = m.group(2)
+            usage[name][m.group(1)] = int(v) if v.isdigit() else int(v == "True")
+    bad = [
+        f"{k}: scratch {u.get('ScratchSize [bytes/lane]', 0)} B/lane, {u.get('VGPRs Spill', 0)} VGPRs spilled"
+        for k, u in usage.items()
+        if u.get("ScratchSize [bytes/lane]", 0) or u.get("VGPRs Spill", 0) or u.get("Dynamic Stack", 0)
+    ]
+    if bad:
+        raise SpillError(
+            f"{src_name}: kernels with register spills are refused (hand-scheduled loads are unsafe "
+            "once the compiler spills):\n  " + "\n  ".join(bad)
+        )
+    return usage
 
 
 def hipcc() -> str:
@@ -70,15 +114,35 @@ def build_host(verbose: bool = True) -> Path:
     return HOST_LIB
 
 
+def _drop_resource_remarks(lines: list[str]) -> list[str]:
+    """Compiler output without the kernel-resource-usage remarks and their source excerpts."""
+    out, skip = [], 0
+    for l in lines:
+        if "[-Rpass-analysis=kernel-resource-usage]" in l:
+            skip = 2 if "Function Name" in l else 0  # the excerpt: source line and caret line
+            continue
+        if skip and (re.match(r"\s*\d+ \|", l) or re.match(r"\s*\|\s*\^", l)):
+            skip -= 1
+            continue
+        skip = 0
+        if re.match(r"In file included from ", l) or re.search(r"\d+ (warning|remark)s? generated", l):
+            continue
+        out.append(l)
+    return out
+
+
 def _compile(src: Path) -> Path:
     obj = OBJDIR / (src.stem + ".o")
-    cmd = [hipcc(), *HIP_FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc(), *HIP_FLAGS, RESOURCE_FLAG, "-c", str(src), "-o", str(obj)]
     if src.suffix == ".cpp":
         cmd.insert(1, "-x")
         cmd.insert(2, "hip")
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    lines = [l for l in proc.stderr.splitlines() if noise not in l]
+    if proc.returncode == 0:
+        check_kernel_resources(proc.stderr, src.name)
+    err = "\n".join(_drop_resource_remarks(lines))
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{err}")
     if err.strip():

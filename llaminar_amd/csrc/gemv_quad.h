@@ -532,6 +532,12 @@ namespace llamql
     template <class Q, int U>
     __device__ __forceinline__ void wait_for(typename Q::Raw &r, int u)
     {
+        // The counts below are the loads issued after step u's: the rest of its chunk and the whole
+        // next chunk.  They hold only while nothing else touches vmcnt in between, which the
+        // build enforces by refusing kernels that spill (scratch traffic counts in vmcnt too,
+        // and a spilled destination register of a load in flight is overwritten when it lands).
+        static_assert(U >= 1 && U <= 4, "wait_for covers chunks of 1..4 steps");
+        static_assert(Q::LOADS * (2 * U - 1) <= 63, "vmcnt is a 6-bit counter");
         // u is a compile-time constant after unrolling
         switch (u)
         {
