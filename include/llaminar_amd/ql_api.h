@@ -127,6 +127,20 @@ bool llam_ql_gemv_f32(uint8_t fmt, const void *d_w, const float *d_x, int ldx, f
 bool llam_ql_gemv_fused_f32(const llam_ql_proj *projs, int num, const float *d_x, int ldx,
                             int M, int K, void *d_q8_scratch, int device_id, void *stream);
 
+/* llam_ql_gemv_f32 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the Q8_1 scratch is a
+ * buffer of LLAM_QL_STATIC_SCRATCH_BYTES built into the library's device image, so the
+ * caller passes inputs and outputs only and the results are the bits of llam_ql_gemv_f32
+ * with a scratch buffer.  It has no counterpart in the reference, whose operators draw
+ * scratch from a caller-bound DeviceWorkspaceManager.
+ * Limits: M * (K/32) * 36 <= LLAM_QL_STATIC_SCRATCH_BYTES (8 rows of K = 32768), otherwise
+ * the call fails with a message.  All calls on one GPU share that GPU's buffer: two calls that
+ * overlap on one GPU (different streams or host threads) race; calls on one stream are
+ * ordered and safe.  Nothing in the buffer needs clearing between calls. */
+#define LLAM_QL_STATIC_SCRATCH_BYTES (8 * (32768 / 32) * 36)
+bool llam_ql_gemv_f32_static(uint8_t fmt, const void *d_w, const float *d_x, int ldx, float *d_y,
+                             int M, int N, int K, int ldy, int device_id, void *stream);
+
 /* d_y = (silu(gate) * up) @ W^T for fp32 gate/up rows of ld_gu floats: the bits of
  * llam_ql_swiglu_quantize followed by llam_ql_gemv, in one launch.  Replaces
  * multiply_tensor_with_fused_swiglu (CPUNativeVNNIGemmKernel.h:325-431: compute_swiglu,

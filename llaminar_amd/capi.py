@@ -47,6 +47,8 @@ SIGNATURES = {
     "llam_ql_gemv_fused": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_gemv_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                   c_int, c_void_p]),
+    "llam_ql_gemv_f32_static": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int,
+                                         c_int, c_void_p]),
     "llam_ql_gemv_fused_f32": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int,
                                         c_void_p]),
     "llam_ql_gemv_swiglu_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
@@ -208,6 +210,16 @@ def gemv_f32(fmt: int, w, x, M: int, N: int, K: int, out=None, q8_scratch=None, 
         out = torch.empty(M, N, dtype=torch.float32, device=w.device)
     _check(load().llam_ql_gemv_f32(fmt, _ptr(w), _ptr(x), _ld(x), _ptr(out), M, N, K, _ld(out), _ptr(q8_scratch),
                                    _dev(w), _stream(stream)), "gemv_f32")
+    return out
+
+
+STATIC_SCRATCH_BYTES = 8 * (32768 // 32) * 36
+
+
+def gemv_f32_static(fmt: int, w, x, M: int, N: int, K: int, out, stream=None):
+    """llam_ql_gemv_f32 with the library's built-in Q8_1 scratch; `out` is caller-provided."""
+    _check(load().llam_ql_gemv_f32_static(fmt, _ptr(w), _ptr(x), _ld(x), _ptr(out), M, N, K, _ld(out), _dev(w),
+                                          _stream(stream)), "gemv_f32_static")
     return out
 
 

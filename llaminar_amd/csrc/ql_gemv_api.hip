@@ -206,6 +206,70 @@ extern "C" bool llam_ql_gemv_f32(uint8_t fmt, const void *d_w, const float *d_x,
                            device_id, stream);
 }
 
+// ---- the entry point that brings its own scratch ----------------------------------------
+// Q8_1 scratch of llam_ql_gemv_f32_static: LLAM_QL_STATIC_SCRATCH_BYTES of device memory that
+// every GPU the library runs on holds from load to exit.  In host code the array's name is
+// only a handle for hipGetSymbolAddress; kernels and copies get the address looked up below.
+static __device__ __align__(256) uint8_t g_q8_static_scratch[LLAM_QL_STATIC_SCRATCH_BYTES];
+
+namespace llamql
+{
+    namespace
+    {
+        // Address of g_q8_static_scratch on the current device (each device has its own copy
+        // at its own address), looked up once per device.
+        void *static_scratch(const char *fn, int device_id)
+        {
+            constexpr int MAX_DEVICES = 64;
+            static std::atomic<void *> ptr[MAX_DEVICES];
+            if (device_id < 0 || device_id >= MAX_DEVICES)
+            {
+                (void)fail(fn, "device_id %d beyond the %d devices the static scratch is tracked for", device_id,
+                           MAX_DEVICES);
+                return nullptr;
+            }
+            void *p = ptr[device_id].load(std::memory_order_acquire);
+            if (p)
+                return p;
+            const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_q8_static_scratch));
+            if (e != hipSuccess || !p)
+            {
+                (void)fail(fn, "hipGetSymbolAddress(scratch) on device %d: %s", device_id, hipGetErrorString(e));
+                return nullptr;
+            }
+            ptr[device_id].store(p, std::memory_order_release); // concurrent first calls find the same address
+            return p;
+        }
+    } // namespace
+} // namespace llamql
+
+extern "C" bool llam_ql_gemv_f32_static(uint8_t fmt, const void *d_w, const float *d_x, int ldx, float *d_y,
+                                        int M, int N, int K, int ldy, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_f32_static";
+    llam_ql_proj p;
+    p.d_w = d_w;
+    p.d_y = d_y;
+    p.N = N;
+    p.ldy = ldy;
+    p.fmt = fmt;
+    if (!check_projections(fn, &p, 1, M, K) || !check_f32(fn, d_x, ldx, K, nullptr))
+        return false;
+    const size_t need = (size_t)M * (size_t)(K / 32) * sizeof(llam_block_q8_1);
+    if (need > (size_t)LLAM_QL_STATIC_SCRATCH_BYTES)
+        return fail(fn, "M=%d rows of K=%d need %zu bytes of Q8_1 scratch, the built-in buffer holds %d", M, K, need,
+                    LLAM_QL_STATIC_SCRATCH_BYTES);
+    if (!set_device(fn, device_id))
+        return false;
+    void *scratch = static_scratch(fn, device_id);
+    if (!scratch)
+        return false;
+    // Every block a call reads from the buffer it has written first: nothing needs clearing.
+    return run_projections(fn, &p, 1, ActSource{ACT_SRC_F32, nullptr, d_x, nullptr, ldx}, M, K, scratch, device_id,
+                           stream);
+}
+
 extern "C" bool llam_ql_gemv_fused_f32(const llam_ql_proj *projs, int num, const float *d_x, int ldx,
                                        int M, int K, void *d_q8_scratch, int device_id, void *stream)
 {
