@@ -150,12 +150,34 @@ bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const float *d_gate,
                              int ldy, void *d_q8_scratch, int device_id, void *stream);
 
 /* Parity hook: the exact per-block int32 sums the GEMV forms, for rows
- * [row0, row0+nrows): d_sums[(m*nrows + r)*(K/32) + kb].  Runs the same integer
- * pipeline as llam_ql_gemv.  (The reference exposes the same quantity only
- * inside its kernels: int_acc in CPUNativeVNNIGemv.h:417-487.) */
+ * [row0, row0+nrows): d_sums[(m*nrows + r)*(K/32) + kb].  The call makes the choices
+ * llam_ql_gemv makes for (fmt, M, N, K) -- quad-lane, matrix-unit, chunked or generic
+ * kernel, K slices, batch splits -- and runs the chosen kernel's block-sum variant: the
+ * same code compiled with the stores of the sums switched on and the fp32 output off.
+ * (The reference exposes the same quantity only inside its kernels: int_acc in
+ * CPUNativeVNNIGemv.h:417-487.)  M * nrows * (K/32) * 4 bytes must stay below 2 GiB. */
 bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,
                              int32_t *d_sums, int M, int N, int K, int row0,
                              int nrows, int device_id, void *stream);
+
+/* What llam_ql_gemv does with a shape: which kernel runs, how the batch and the row are
+ * split.  For tests, tuning and the operator's decode-equivalence guard; the launcher
+ * executes exactly this plan.  (Reference: the dispatch tables behind
+ * rocmGemv_native_vnni_fp32, ROCmNativeVNNIDecodeDispatchGenerated.inc.) */
+#define LLAM_QL_KERNEL_GENERIC 0 /* rows shorter than 5 super-blocks */
+#define LLAM_QL_KERNEL_CHUNKED 1 /* 8 lanes per super-block, whole rows per wavefront */
+#define LLAM_QL_KERNEL_QUAD 2    /* 4 lanes per super-block, runs of rows per wavefront */
+#define LLAM_QL_KERNEL_MFMA 3    /* batches of 5..8 on the matrix unit */
+typedef struct
+{
+    int kernel;            /* LLAM_QL_KERNEL_*, or -1 when the shape cannot be served */
+    int m_first;           /* activation rows of the first launch group (the rest follows alike) */
+    int slice_sb;          /* super-blocks per K slice (one slice = the whole row) */
+    int rows_per_wave;
+    int decode_equivalent; /* 1: every row of the M-row call has the bits of its own M = 1 call */
+} llam_ql_gemv_plan;
+bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int device_id,
+                           llam_ql_gemv_plan *out);
 
 /* ---- P3: prefill GEMM (any M) -------------------------------------------------------
  * Same contract as llam_ql_gemv for many activation rows, on int8 MFMA with
@@ -165,6 +187,15 @@ bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,
  * (src/v2/kernels/rocm/gemm/ROCmQuantisedGemmKernel_native_VNNI.hip:2580-2632). */
 bool llam_ql_gemm(uint8_t fmt, const void *d_w, const void *d_q8, float *d_y,
                   int M, int N, int K, int ldy, int device_id, void *stream);
+
+/* Parity hook of the GEMM: the matrix unit's exact per-block int32 sums of weight rows
+ * [row0, row0+nrows) for all M activation rows, d_sums[(m*nrows + r)*(K/32) + kb], from
+ * the block-sum variant of llam_ql_gemm's kernel (same tiles, same decode, same MFMA).
+ * Counterpart of the reference's int32 accumulators in gemm_2row_native_chunk /
+ * gemm_2row_int8_chunk (CPUNativeVNNIGemv.h:1046-1376). */
+bool llam_ql_gemm_block_sums(uint8_t fmt, const void *d_w, const void *d_q8, int32_t *d_sums,
+                             int M, int N, int K, int row0, int nrows, int device_id,
+                             void *stream);
 
 /* C = beta*C + alpha*T (+ bias per column), the operator's epilogue
  * (CPUNativeVNNIGemmKernel.h:154-214).  beta == 0 overwrites.  T row stride N. */

@@ -55,10 +55,10 @@ def check_kernel_resources(remarks: str, src_name: str) -> dict[str, dict[str, i
     hand many instructions later.  The compiler takes the destination registers of such
     a load as written at the point of issue.  If it has to spill, it may store such a
     register to scratch straight after the load instruction (before the data has
-    arrived) and hand the register to another value, for instance an address; the
-    load then lands in that value.  Its own scratch loads and stores also count in
-    vmcnt and shift every hand-written ``s_waitcnt vmcnt(n)``.  The kernels are only
-    correct with zero spills, so a spill fails the build instead of the GPU.
+    arrived: the spill slot gets stale contents) and hand the register to another
+    value, for instance an address; the load then lands in that value and the kernel
+    reads a wild address.  The kernels are only correct with zero spills, so a spill
+    fails the build instead of the GPU.
     """
     usage: dict[str, dict[str, int]] = {}
     name = None

@@ -30,6 +30,14 @@ class Proj(ctypes.Structure):
     _fields_ = [("d_w", c_void_p), ("d_y", c_void_p), ("N", c_int), ("ldy", c_int), ("fmt", c_uint8)]
 
 
+class GemvPlan(ctypes.Structure):
+    _fields_ = [("kernel", c_int), ("m_first", c_int), ("slice_sb", c_int), ("rows_per_wave", c_int),
+                ("decode_equivalent", c_int)]
+
+
+KERNEL_GENERIC, KERNEL_CHUNKED, KERNEL_QUAD, KERNEL_MFMA = 0, 1, 2, 3
+
+
 class Expert(ctypes.Structure):
     _fields_ = [("d_gate", c_void_p), ("d_up", c_void_p), ("d_down", c_void_p)]
 
@@ -55,7 +63,10 @@ SIGNATURES = {
                                          c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_gemv_block_sums": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                          c_int, c_void_p]),
+    "llam_ql_gemv_describe": (c_bool, [c_uint8, c_int, c_int, c_int, c_int, POINTER(GemvPlan)]),
     "llam_ql_gemm": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemm_block_sums": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                         c_int, c_void_p]),
     "llam_ql_epilogue": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int,
                                   c_void_p]),
     "llam_ql_moe_router_logits": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
@@ -253,6 +264,13 @@ def gemv_block_sums(fmt: int, w, q8, M: int, N: int, K: int, row0: int, nrows: i
     return out
 
 
+def gemv_describe(fmt: int, M: int, N: int, K: int, device_id: int = 0) -> GemvPlan:
+    """The launch plan of llam_ql_gemv for a shape (no GPU work)."""
+    plan = GemvPlan()
+    _check(load().llam_ql_gemv_describe(fmt, M, N, K, device_id, ctypes.byref(plan)), "gemv_describe")
+    return plan
+
+
 def gemm(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None):
     import torch
 
@@ -260,6 +278,15 @@ def gemm(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None):
         out = torch.empty(M, N, dtype=torch.float32, device=w.device)
     _check(load().llam_ql_gemm(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, out.stride(0), _dev(w), _stream(stream)),
            "gemm")
+    return out
+
+
+def gemm_block_sums(fmt: int, w, q8, M: int, N: int, K: int, row0: int, nrows: int, stream=None):
+    import torch
+
+    out = torch.empty(M, nrows, K // 32, dtype=torch.int32, device=w.device)
+    _check(load().llam_ql_gemm_block_sums(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, row0, nrows, _dev(w),
+                                          _stream(stream)), "gemm_block_sums")
     return out
 
 

@@ -48,6 +48,11 @@ namespace llamql
         const uint32_t *q8; // [M][K/32] blocks as dwords
         float *y;
         int M, ldy;
+        // DUMP kernels only: the exact per-block int32 sums of weight rows [row0, row0+nrows) go to
+        // sums[(m * nrows + n - row0) * (K/32) + block]
+        int32_t *sums;
+        int row0, nrows;
+        int tile0; // first 64-row tile of the launch (0 unless DUMP)
     };
 
     template <class F>
@@ -173,7 +178,9 @@ namespace llamql
         __device__ __forceinline__ void finish() {}
     };
 
-    template <class F>
+    // DUMP: also store the matrix unit's results, the exact int32 block sums (the parity hook of
+    // the C-ABI), for a window of weight rows; otherwise the same code.
+    template <class F, bool DUMP = false>
     __global__ void __launch_bounds__(GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
         gemm_kernel(const GemmArgs g)
     {
@@ -197,7 +204,7 @@ namespace llamql
         const int l32 = lane & 31;
         const int lh = lane >> 5;
 
-        const long n0 = (long)blockIdx.x * GEMM_BN;
+        const long n0 = ((long)blockIdx.x + g.tile0) * GEMM_BN;
         const long m0 = (long)blockIdx.y * GEMM_BM;
         const int KB = g.w.SB * 8;
 
@@ -287,6 +294,21 @@ namespace llamql
                 if (kb + 1 < 8)
                     idot[(kb + 1) & 1] = product(kb + 1);
                 const v16i d = idot[kb & 1];
+                if constexpr (DUMP)
+                {
+                    const long n = n0 + ntile * 32 + l32;
+                    const long nn = n - g.row0;
+                    if (n < g.w.N && nn >= 0 && nn < g.nrows)
+                    {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                        {
+                            const long m = m0 + mtile * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                            if (m < g.M)
+                                g.sums[((size_t)m * g.nrows + (size_t)nn) * (size_t)KB + (size_t)sb * 8 + kb] = d[r];
+                        }
+                    }
+                }
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     acc[r] = fmaf((float)d[r], cs[r], acc[r]);
@@ -310,7 +332,7 @@ namespace llamql
 
         // ---- store: lane holds weight row n, 16 tokens -------------------------------------
         const long n = n0 + ntile * 32 + l32;
-        if (n < g.w.N)
+        if (!DUMP && n < g.w.N)
         {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
@@ -339,9 +361,11 @@ namespace llamql
         *dst = v;
     }
 
-    template <class F>
+    // d_sums: the block-sum variant over weight rows [row0, row0+nrows); only the workgroups
+    // whose 64-row tile meets the window are launched.
+    template <class F, bool DUMP = false>
     bool gemm_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int M, int N, int K, int ldy,
-                     hipStream_t st)
+                     hipStream_t st, int32_t *d_sums = nullptr, int row0 = 0, int nrows = 0)
     {
         GemmArgs g;
         g.w = GemvArgs{};
@@ -352,13 +376,18 @@ namespace llamql
         g.y = d_y;
         g.M = M;
         g.ldy = ldy;
+        g.sums = d_sums;
+        g.row0 = row0;
+        g.nrows = nrows;
+        g.tile0 = DUMP ? row0 / GEMM_BN : 0;
+        const int tile_end = DUMP ? (row0 + nrows + GEMM_BN - 1) / GEMM_BN : (N + GEMM_BN - 1) / GEMM_BN;
         constexpr size_t lds = gemm_lds_bytes<F>();
         static LdsGrant grant;
-        const hipError_t e = allow_lds(grant, reinterpret_cast<const void *>(&gemm_kernel<F>), lds);
+        const hipError_t e = allow_lds(grant, reinterpret_cast<const void *>(&gemm_kernel<F, DUMP>), lds);
         if (e != hipSuccess)
             return fail(fn, "cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-        const dim3 grid((unsigned)((N + GEMM_BN - 1) / GEMM_BN), (unsigned)((M + GEMM_BM - 1) / GEMM_BM));
-        hipLaunchKernelGGL((gemm_kernel<F>), grid, dim3(GEMM_THREADS), lds, st, g);
+        const dim3 grid((unsigned)(tile_end - g.tile0), (unsigned)((M + GEMM_BM - 1) / GEMM_BM));
+        hipLaunchKernelGGL((gemm_kernel<F, DUMP>), grid, dim3(GEMM_THREADS), lds, st, g);
         return launched(fn);
     }
 } // namespace llamql
@@ -392,6 +421,36 @@ extern "C" bool llam_ql_gemm(uint8_t fmt, const void *d_w, const void *d_q8, flo
     case LLAM_FMT_Q4_K: return gemm_launch<Q4KTraits>(fn, d_w, d_q8, d_y, M, N, K, ldy, st);
     case LLAM_FMT_Q6_K: return gemm_launch<Q6KTraits>(fn, d_w, d_q8, d_y, M, N, K, ldy, st);
     default: return gemm_launch<IQ3STraits>(fn, d_w, d_q8, d_y, M, N, K, ldy, st);
+    }
+}
+
+extern "C" bool llam_ql_gemm_block_sums(uint8_t fmt, const void *d_w, const void *d_q8, int32_t *d_sums,
+                                        int M, int N, int K, int row0, int nrows, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemm_block_sums";
+    if (fmt != LLAM_FMT_Q4_K && fmt != LLAM_FMT_Q6_K && fmt != LLAM_FMT_IQ3_S)
+        return fail(fn, "unsupported weight format id %d", (int)fmt);
+    if (M < 1 || N < 1 || K < 1 || (K % 256) != 0)
+        return fail(fn, "need M, N >= 1 and K a positive multiple of 256 (M=%d N=%d K=%d)", M, N, K);
+    if (!d_w || !d_q8 || !d_sums)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_w) || !aligned4(d_q8) || !aligned4(d_sums))
+        return fail(fn, "d_w must be 16-byte, d_q8 and d_sums 4-byte aligned");
+    if (row0 < 0 || nrows < 1 || (long)row0 + nrows > N)
+        return fail(fn, "row window [%d,%d) outside [0,%d)", row0, row0 + nrows, N);
+    if ((M + GEMM_BM - 1) / GEMM_BM > 65535)
+        return fail(fn, "M=%d too large for one launch", M);
+    if ((size_t)M * (size_t)nrows * (size_t)(K / 32) * sizeof(int32_t) >= ((size_t)1 << 31))
+        return fail(fn, "M=%d x %d rows x %d blocks of sums exceed 2 GiB", M, nrows, K / 32);
+    if (!set_device(fn, device_id))
+        return false;
+    hipStream_t st = as_stream(stream);
+    switch (fmt)
+    {
+    case LLAM_FMT_Q4_K: return gemm_launch<Q4KTraits, true>(fn, d_w, d_q8, nullptr, M, N, K, 0, st, d_sums, row0, nrows);
+    case LLAM_FMT_Q6_K: return gemm_launch<Q6KTraits, true>(fn, d_w, d_q8, nullptr, M, N, K, 0, st, d_sums, row0, nrows);
+    default: return gemm_launch<IQ3STraits, true>(fn, d_w, d_q8, nullptr, M, N, K, 0, st, d_sums, row0, nrows);
     }
 }
 

@@ -26,6 +26,30 @@ namespace llamql
 
     namespace
     {
+        template <class F>
+        void describe(int M, int N, int K, int device_id, llam_ql_gemv_plan *out)
+        {
+            const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
+            out->kernel = p.kernel;
+            out->m_first = p.m_first;
+            out->slice_sb = p.slice_sb;
+            out->rows_per_wave = p.rows_per_wave;
+            out->decode_equivalent = gemv_decode_equivalent<F>(M, N, K, device_id) ? 1 : 0;
+        }
+    } // namespace
+
+    void gemv_describe(uint8_t fmt, int M, int N, int K, int device_id, llam_ql_gemv_plan *out)
+    {
+        switch (fmt)
+        {
+        case LLAM_FMT_Q4_K: describe<Q4KTraits>(M, N, K, device_id, out); break;
+        case LLAM_FMT_Q6_K: describe<Q6KTraits>(M, N, K, device_id, out); break;
+        default: describe<IQ3STraits>(M, N, K, device_id, out); break;
+        }
+    }
+
+    namespace
+    {
         // the other format with a quad-lane kernel
         template <class F>
         struct Other;

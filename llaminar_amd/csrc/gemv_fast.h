@@ -53,11 +53,14 @@ namespace llamql
         }
     }
 
-    template <class F, int M, int U, bool PARTIAL>
+    // dump_row: with DUMP, where the block sums of this lane's row go (sums + (row - row0) * blocks
+    // per row, null outside the window); the sums of activation row m lie dump_m_stride further
+    template <class F, int M, int U, bool PARTIAL, bool DUMP>
     __device__ __forceinline__ void gemv_fast_chunk(const typename F::Raw (&cur)[U], const typename F::Lane &lc,
                                                     bool odd, int s_base, int nsb, const uint8_t *aq_lane,
                                                     const uint8_t *ads_lane, int m_stride_aq, int m_stride_ads,
-                                                    const void *tab, float (&acc)[M])
+                                                    const void *tab, float (&acc)[M], int32_t *dump_row,
+                                                    size_t dump_m_stride, int dump_sb0)
     {
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -86,6 +89,11 @@ namespace llamql
                 {
                     idot = dot16(a1, w1, dot16(a0, w0, 0));
                 }
+                if constexpr (DUMP)
+                {
+                    if (dump_row)
+                        dump_row[(size_t)m * dump_m_stride + (size_t)(dump_sb0 + s_base + 8 * u) * 8 + lc.j] = idot;
+                }
                 const float cs = sd.x * bscale;
                 acc[m] = fmaf((float)idot, cs, acc[m]);
                 if (F::HAS_MIN)
@@ -94,7 +102,8 @@ namespace llamql
         }
     }
 
-    template <class F, int M, int U>
+    // DUMP: also store the exact int32 block sums (the parity hook); otherwise the same code.
+    template <class F, int M, int U, bool DUMP = false>
     __global__ void __launch_bounds__(GEMV_WAVES *WAVE) gemv_fast_kernel(const GemvArgs a)
     {
         extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
@@ -146,6 +155,13 @@ namespace llamql
 #pragma unroll
             for (int m = 0; m < M; ++m)
                 acc[m] = 0.0f;
+            int32_t *dump_row = nullptr;
+            const size_t dump_m_stride = (size_t)a.nrows * ((size_t)a.SB * 8);
+            if constexpr (DUMP)
+            {
+                if (row >= a.row0 && row < (long)a.row0 + a.nrows)
+                    dump_row = a.sums + (size_t)(row - a.row0) * ((size_t)a.SB * 8);
+            }
 
             for (int ch = 0; ch < nchunks; ++ch)
             {
@@ -182,28 +198,33 @@ namespace llamql
                 const uint8_t *aql = aq_lane0 + ch * (U * 2048);
                 const uint8_t *adl = ads_lane0 + ch * (U * 512);
                 if (ch < nfull)
-                    gemv_fast_chunk<F, M, U, false>(cur, lc, odd, grp + ch * chunk_sb, a.nsb, aql, adl, m_stride_aq,
-                                                    m_stride_ads, tab, acc);
+                    gemv_fast_chunk<F, M, U, false, DUMP>(cur, lc, odd, grp + ch * chunk_sb, a.nsb, aql, adl,
+                                                          m_stride_aq, m_stride_ads, tab, acc, dump_row, dump_m_stride,
+                                                          a.sb0);
                 else
-                    gemv_fast_chunk<F, M, U, true>(cur, lc, odd, grp + ch * chunk_sb, a.nsb, aql, adl, m_stride_aq,
-                                                   m_stride_ads, tab, acc);
+                    gemv_fast_chunk<F, M, U, true, DUMP>(cur, lc, odd, grp + ch * chunk_sb, a.nsb, aql, adl,
+                                                         m_stride_aq, m_stride_ads, tab, acc, dump_row, dump_m_stride,
+                                                         a.sb0);
             }
 
-#pragma unroll
-            for (int m = 0; m < M; ++m)
+            if constexpr (!DUMP) // the block-sum variant has no fp32 output
             {
-                const float total = wave_sum(acc[m]);
-                if (lane == 0)
+#pragma unroll
+                for (int m = 0; m < M; ++m)
                 {
-                    float *dst = a.y + (size_t)m * a.ldy + row;
-                    const float v = a.out_scale * total;
-                    *dst = a.accumulate ? (*dst + v) : v;
+                    const float total = wave_sum(acc[m]);
+                    if (lane == 0)
+                    {
+                        float *dst = a.y + (size_t)m * a.ldy + row;
+                        const float v = a.out_scale * total;
+                        *dst = a.accumulate ? (*dst + v) : v;
+                    }
                 }
             }
         }
     }
 
-    template <class F, int M>
+    template <class F, int M, bool DUMP>
     inline void gemv_fast_launch_u(int U, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
     {
         dim3 block(GEMV_WAVES * WAVE);
@@ -212,30 +233,42 @@ namespace llamql
         {
             switch (U)
             {
-            case 1: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1>), grid, block, lds, st, a); break;
-            case 2: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 2>), grid, block, lds, st, a); break;
-            case 3: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 3>), grid, block, lds, st, a); break;
-            default: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 4>), grid, block, lds, st, a); break;
+            case 1: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1, DUMP>), grid, block, lds, st, a); break;
+            case 2: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 2, DUMP>), grid, block, lds, st, a); break;
+            case 3: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 3, DUMP>), grid, block, lds, st, a); break;
+            default: hipLaunchKernelGGL((gemv_fast_kernel<F, M, 4, DUMP>), grid, block, lds, st, a); break;
             }
         }
         else
         {
             (void)U;
-            hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1>), grid, block, lds, st, a);
+            hipLaunchKernelGGL((gemv_fast_kernel<F, M, 1, DUMP>), grid, block, lds, st, a);
         }
     }
 
-    // M is one of 1,2,3,4,8.
+    // M is one of 1,2,3,4,8.  a.sums set: the block-sum variant of the same kernel.
     template <class F>
     inline void gemv_fast_launch(int M, int U, dim3 grid, size_t lds, hipStream_t st, const GemvArgs &a)
     {
+        if (a.sums)
+        {
+            switch (M)
+            {
+            case 1: gemv_fast_launch_u<F, 1, true>(U, grid, lds, st, a); break;
+            case 2: gemv_fast_launch_u<F, 2, true>(U, grid, lds, st, a); break;
+            case 3: gemv_fast_launch_u<F, 3, true>(U, grid, lds, st, a); break;
+            case 4: gemv_fast_launch_u<F, 4, true>(U, grid, lds, st, a); break;
+            default: gemv_fast_launch_u<F, 8, true>(U, grid, lds, st, a); break;
+            }
+            return;
+        }
         switch (M)
         {
-        case 1: gemv_fast_launch_u<F, 1>(U, grid, lds, st, a); break;
-        case 2: gemv_fast_launch_u<F, 2>(U, grid, lds, st, a); break;
-        case 3: gemv_fast_launch_u<F, 3>(U, grid, lds, st, a); break;
-        case 4: gemv_fast_launch_u<F, 4>(U, grid, lds, st, a); break;
-        default: gemv_fast_launch_u<F, 8>(U, grid, lds, st, a); break;
+        case 1: gemv_fast_launch_u<F, 1, false>(U, grid, lds, st, a); break;
+        case 2: gemv_fast_launch_u<F, 2, false>(U, grid, lds, st, a); break;
+        case 3: gemv_fast_launch_u<F, 3, false>(U, grid, lds, st, a); break;
+        case 4: gemv_fast_launch_u<F, 4, false>(U, grid, lds, st, a); break;
+        default: gemv_fast_launch_u<F, 8, false>(U, grid, lds, st, a); break;
         }
     }
 
@@ -352,19 +385,20 @@ namespace llamql
             return mfma_max_slices(K / 256) >= 1 && N >= MFMA_MIN_ROWS;
     }
 
-    template <int SRC>
+    template <int SRC, bool DUMP = false>
     void gemv_mfma_q4k_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const MfmaArgs &a)
     {
         static LdsGrant grant;
-        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<SRC>), QUAD_MAX_LDS);
-        hipLaunchKernelGGL(gemv_mfma_q4k_kernel<SRC>, grid, block, lds, st, a);
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<SRC, DUMP>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_mfma_q4k_kernel<SRC, DUMP>), grid, block, lds, st, a);
     }
 
     inline bool gemv_mfma_q4k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
-                                     int K, int ldy, int device_id, hipStream_t st)
+                                     int K, int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr,
+                                     int row0 = 0, int nrows = 0)
     {
         const int SB = K / 256;
-        const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id));
+        const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id), d_sums ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES);
         MfmaArgs a;
         a.w = static_cast<const uint8_t *>(d_w);
         a.q8 = static_cast<const uint32_t *>(src.q8);
@@ -377,8 +411,18 @@ namespace llamql
         a.SB = SB;
         a.M = M;
         a.slices = sh.slices;
+        a.sums = d_sums;
+        a.row0 = row0;
+        a.nrows = nrows;
         const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles_per_wg) * WAVE);
         const size_t lds = mfma_lds_bytes(SB, sh.slices * sh.tiles_per_wg);
+        if (d_sums)
+        {
+            if (src.kind != ACT_SRC_Q8)
+                return fail(fn, "block sums are dumped on Q8_1 input");
+            gemv_mfma_q4k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            return launched(fn);
+        }
         switch (src.kind)
         {
         case ACT_SRC_F32: gemv_mfma_q4k_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;
@@ -388,19 +432,21 @@ namespace llamql
         return launched(fn);
     }
 
-    template <int SRC>
+    template <int SRC, bool DUMP = false>
     void gemv_mfma_q6k_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const Mfma6Args &a)
     {
         static LdsGrant grant;
-        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q6k_kernel<SRC>), QUAD_MAX_LDS);
-        hipLaunchKernelGGL(gemv_mfma_q6k_kernel<SRC>, grid, block, lds, st, a);
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q6k_kernel<SRC, DUMP>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_mfma_q6k_kernel<SRC, DUMP>), grid, block, lds, st, a);
     }
 
     inline bool gemv_mfma_q6k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
-                                     int K, int ldy, int device_id, hipStream_t st)
+                                     int K, int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr,
+                                     int row0 = 0, int nrows = 0)
     {
         const int SB = K / 256;
-        const Mfma6Shape sh = gemv_mfma6_shape(N, SB, cu_count(device_id));
+        const Mfma6Shape sh =
+            gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA6_DUMP_COMPUTE : MFMA6_MAX_COMPUTE);
         Mfma6Args a;
         a.w = static_cast<const uint8_t *>(d_w);
         a.q8 = static_cast<const uint32_t *>(src.q8);
@@ -415,8 +461,18 @@ namespace llamql
         a.slices = sh.slices;
         a.tiles = sh.tiles;
         a.chunk = sh.chunk;
+        a.sums = d_sums;
+        a.row0 = row0;
+        a.nrows = nrows;
         const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles + MFMA6_PRODUCERS) * WAVE);
         const size_t lds = mfma6_lds_bytes(SB, sh.chunk, sh.slices * sh.tiles);
+        if (d_sums)
+        {
+            if (src.kind != ACT_SRC_Q8)
+                return fail(fn, "block sums are dumped on Q8_1 input");
+            gemv_mfma_q6k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            return launched(fn);
+        }
         switch (src.kind)
         {
         case ACT_SRC_F32: gemv_mfma_q6k_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;
@@ -429,20 +485,22 @@ namespace llamql
     // The matrix-unit kernel of format F (mfma_eligible<F> has said yes).
     template <class F>
     bool gemv_mfma_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N, int K,
-                          int ldy, int device_id, hipStream_t st)
+                          int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr, int row0 = 0,
+                          int nrows = 0)
     {
         if constexpr (std::is_same<typename F::Quad, Q6KQuad>::value)
-            return gemv_mfma_q6k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st);
+            return gemv_mfma_q6k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
         else
-            return gemv_mfma_q4k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st);
+            return gemv_mfma_q4k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
     }
 
     static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU,
                   "activation source kinds");
 
+    // d_sums (one matrix, Q8_1 input): run the block-sum variant over rows [row0, row0+nrows).
     template <class F>
     bool gemv_quad_multi(const char *fn, const QuadProj *pr, int n, const ActSource &src, int M, int K,
-                         int device_id, hipStream_t st)
+                         int device_id, hipStream_t st, int32_t *d_sums = nullptr, int row0 = 0, int nrows = 0)
     {
         if constexpr (F::USE_QUAD)
         {
@@ -457,6 +515,11 @@ namespace llamql
             a.SB = SB;
             a.nproj = n;
             a.first_b = n;
+            a.sums = d_sums;
+            a.row0 = row0;
+            a.nrows = nrows;
+            if (d_sums && (n != 1 || src.kind != ACT_SRC_Q8))
+                return fail(fn, "block sums are dumped for one matrix on Q8_1 input");
             long waves = 0;
             for (int i = 0; i < QUAD_MAX_PROJ; ++i)
             {
@@ -516,6 +579,8 @@ namespace llamql
             a.SB = SB;
             a.nproj = n;
             a.first_b = na;
+            a.sums = nullptr;
+            a.row0 = a.nrows = 0;
             long cnt[QUAD_MAX_PROJ], waves = 0;
             for (int i = 0; i < QUAD_MAX_PROJ; ++i)
             {
@@ -557,57 +622,137 @@ namespace llamql
         }
     }
 
+    // What the launcher does with a shape: the one place where the kernel, the batch split and
+    // the K slices are decided.  gemv_launch() executes a plan; llam_ql_gemv_describe() reports it.
+    constexpr int GEMV_KERNEL_GENERIC = 0; // gemv_kernel: rows shorter than 5 super-blocks
+    constexpr int GEMV_KERNEL_CHUNKED = 1; // gemv_fast_kernel
+    constexpr int GEMV_KERNEL_QUAD = 2;    // gemv_quad_kernel
+    constexpr int GEMV_KERNEL_MFMA = 3;    // gemv_mfma_q4k_kernel / gemv_mfma_q6k_kernel
+    struct GemvPlan
+    {
+        int kernel;        // GEMV_KERNEL_*; -1: the shape cannot be served
+        int m_first;       // batch rows of the first launch group; the rest (M - m_first > 0) is
+                           // planned and launched the same way after it
+        int slice_sb;      // super-blocks per K slice (generic and chunked kernels; others: the row)
+        int rows_per_wave; // row (batches) a wavefront walks
+        int unroll;        // load batches in flight (chunked kernel)
+        int gshift;        // 8-lane groups per row, log2 (generic and chunked kernels)
+        long grid;
+    };
+
+    template <class F>
+    GemvPlan gemv_plan(int M, int N, int K, int device_id)
+    {
+        const int SB = K / 256;
+        GemvPlan p{};
+        p.m_first = M;
+        p.slice_sb = SB;
+        if constexpr (F::USE_MFMA_BATCH)
+            if (mfma_eligible<F>(M, N, K))
+            {
+                p.kernel = GEMV_KERNEL_MFMA;
+                return p;
+            }
+        // Rows of at least 16 super-blocks in a format with a quad-lane decoder: the
+        // quad kernel, which stages whole activation rows (up to 160 KiB of LDS).
+        if constexpr (F::USE_QUAD)
+            if (SB >= QUAD_STEP_SB && gemv_unroll_override() == 0 && F::Quad::addressable(N, SB))
+            {
+                p.kernel = GEMV_KERNEL_QUAD;
+                if (quad_lds_bytes(M, SB) > QUAD_MAX_LDS)
+                {
+                    if (M == 1)
+                    {
+                        p.kernel = -1; // one activation row does not fit the LDS
+                        return p;
+                    }
+                    p.m_first = M / 2;
+                }
+                const QuadShape sh = gemv_quad_shape(N, SB, cu_count(device_id), F::Quad::max_threads(p.m_first) / WAVE);
+                p.rows_per_wave = sh.rows_per_wave;
+                p.grid = sh.grid;
+                return p;
+            }
+        // batch sizes without a dedicated kernel are run as 4 + (M-4)
+        if (M > 4 && M < 8)
+            p.m_first = 4;
+        // K slices keep the staged activations (+ tables) within 64 KiB of LDS.
+        int slice = (64 * 1024 - F::TABLE_BYTES) / (p.m_first * GEMV_LDS_PER_SB);
+        if (slice > SB)
+            slice = SB;
+        if (slice < 1)
+        {
+            p.kernel = -1;
+            return p;
+        }
+        GemvShape sh = gemv_shape(N, slice, cu_count(device_id));
+        if (gemv_unroll_override() <= 0 && sh.U > F::FAST_MAX_U)
+            sh.U = F::FAST_MAX_U;
+        p.kernel = sh.gshift == 3 ? GEMV_KERNEL_CHUNKED : GEMV_KERNEL_GENERIC;
+        p.slice_sb = slice;
+        p.rows_per_wave = sh.rpw;
+        p.unroll = sh.U;
+        p.gshift = sh.gshift;
+        p.grid = sh.grid;
+        return p;
+    }
+
+    // Whether every activation row of an M-row call gets the bits of its own M = 1 call: the
+    // same kernel walks the same rows and K slices in the same order for both batch sizes.
+    // (The quad-lane kernel picks its rows per wavefront from N and K alone and a batch split
+    // runs the same kernel on each part; the chunked and generic kernels add a lane's
+    // super-blocks in ascending order whatever the unroll, so only the K slicing, which
+    // shrinks with M, can differ; the matrix-unit kernels add blocks in another order.)
+    template <class F>
+    bool gemv_decode_equivalent(int M, int N, int K, int device_id)
+    {
+        const GemvPlan one = gemv_plan<F>(1, N, K, device_id);
+        for (int m0 = 0; m0 < M;)
+        {
+            const GemvPlan p = gemv_plan<F>(M - m0, N, K, device_id);
+            if (p.kernel < 0 || one.kernel < 0 || p.kernel != one.kernel || p.kernel == GEMV_KERNEL_MFMA)
+                return false;
+            if (p.kernel != GEMV_KERNEL_QUAD && (p.slice_sb != one.slice_sb || p.gshift != one.gshift))
+                return false;
+            m0 += p.m_first;
+        }
+        return true;
+    }
+
     // Shared host launcher.  Arguments are validated by the callers; the device
-    // is current.  M is 1..8.
+    // is current.  M is 1..8.  With d_sums the same plan is executed with the chosen kernel's
+    // block-sum variant: the parity hook reads the integer pipeline that serves this
+    // (format, M, N, K).
     template <class F>
     bool gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
                      int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
     {
         const int SB = K / 256;
         const bool dump = d_sums != nullptr;
-        if constexpr (F::USE_MFMA_BATCH)
-            if (!dump && mfma_eligible<F>(M, N, K))
-                return gemv_mfma_launch<F>(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st);
-        // Rows of at least 16 super-blocks in a format with a quad-lane decoder: the
-        // quad kernel, which stages whole activation rows (up to 160 KiB of LDS).
-        if constexpr (F::USE_QUAD)
-        if (!dump && SB >= QUAD_STEP_SB && gemv_unroll_override() == 0 && F::Quad::addressable(N, SB))
+        const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
+        if (p.kernel < 0)
+            return fail(fn, "K=%d is too long for %d activation row(s) in LDS", K, p.m_first);
+        if (p.m_first < M)
         {
-            if (quad_lds_bytes(M, SB) > QUAD_MAX_LDS)
-            {
-                if (M == 1)
-                    return fail(fn, "K=%d is too long for one activation row in LDS", K);
-                const int M0 = M / 2;
-                if (!gemv_launch<F>(fn, d_w, d_q8, d_y, d_sums, M0, N, K, ldy, row0, nrows, device_id, st))
-                    return false;
-                const uint8_t *q8b = static_cast<const uint8_t *>(d_q8) + (size_t)M0 * (K / 32) * 36;
-                return gemv_launch<F>(fn, d_w, q8b, d_y + (size_t)M0 * ldy, nullptr, M - M0, N, K, ldy, row0, nrows,
-                                      device_id, st);
-            }
-            QuadProj one{d_w, d_y, N, ldy};
-            return gemv_quad_multi<F>(fn, &one, 1, act_source_q8(d_q8), M, K, device_id, st);
-        }
-        // batch sizes without a dedicated kernel are run as 4 + (M-4)
-        if (M > 4 && M < 8)
-        {
-            if (!gemv_launch<F>(fn, d_w, d_q8, d_y, d_sums, 4, N, K, ldy, row0, nrows, device_id, st))
+            // the first p.m_first rows now, the others after them
+            if (!gemv_launch<F>(fn, d_w, d_q8, d_y, d_sums, p.m_first, N, K, ldy, row0, nrows, device_id, st))
                 return false;
-            const uint8_t *q8b = static_cast<const uint8_t *>(d_q8) + (size_t)4 * (K / 32) * 36;
-            return gemv_launch<F>(fn, d_w, q8b, d_y ? d_y + (size_t)4 * ldy : nullptr,
-                                  d_sums ? d_sums + (size_t)4 * nrows * (K / 32) : nullptr, M - 4, N, K, ldy, row0,
-                                  nrows, device_id, st);
+            const uint8_t *q8b = static_cast<const uint8_t *>(d_q8) + (size_t)p.m_first * (K / 32) * 36;
+            return gemv_launch<F>(fn, d_w, q8b, d_y ? d_y + (size_t)p.m_first * ldy : nullptr,
+                                  d_sums ? d_sums + (size_t)p.m_first * nrows * (K / 32) : nullptr, M - p.m_first, N,
+                                  K, ldy, row0, nrows, device_id, st);
         }
-        // K slices keep the staged activations (+ tables) within 64 KiB of LDS.
-        int slice = (64 * 1024 - F::TABLE_BYTES) / (M * GEMV_LDS_PER_SB);
-        if (slice > SB)
-            slice = SB;
-        if (slice < 1)
-            return fail(fn, "activation rows do not fit LDS (M=%d)", M);
-        GemvShape sh = gemv_shape(N, slice, cu_count(device_id));
-        if (gemv_unroll_override() <= 0 && sh.U > F::FAST_MAX_U)
-            sh.U = F::FAST_MAX_U;
-
-        for (int sb0 = 0; sb0 < SB; sb0 += slice)
+        if constexpr (F::USE_MFMA_BATCH)
+            if (p.kernel == GEMV_KERNEL_MFMA)
+                return gemv_mfma_launch<F>(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st, d_sums,
+                                           row0, nrows);
+        if constexpr (F::USE_QUAD)
+            if (p.kernel == GEMV_KERNEL_QUAD)
+            {
+                QuadProj one{d_w, d_y, N, ldy};
+                return gemv_quad_multi<F>(fn, &one, 1, act_source_q8(d_q8), M, K, device_id, st, d_sums, row0, nrows);
+            }
+        for (int sb0 = 0; sb0 < SB; sb0 += p.slice_sb)
         {
             GemvArgs a;
             a.w = d_w;
@@ -618,18 +763,18 @@ namespace llamql
             a.N = N;
             a.SB = SB;
             a.sb0 = sb0;
-            a.nsb = (SB - sb0 < slice) ? (SB - sb0) : slice;
-            a.rows_per_wave = sh.rpw;
-            a.gshift = sh.gshift;
+            a.nsb = (SB - sb0 < p.slice_sb) ? (SB - sb0) : p.slice_sb;
+            a.rows_per_wave = p.rows_per_wave;
+            a.gshift = p.gshift;
             a.accumulate = sb0 > 0;
             a.out_scale = 1.0f;
             a.row0 = row0;
             a.nrows = nrows;
             const size_t lds = gemv_lds_bytes<F>(M, a.nsb);
-            if (!dump && sh.gshift == 3)
-                gemv_fast_launch<F>(M, sh.U, dim3((unsigned)sh.grid), lds, st, a);
+            if (p.kernel == GEMV_KERNEL_CHUNKED)
+                gemv_fast_launch<F>(M, p.unroll, dim3((unsigned)p.grid), lds, st, a);
             else
-                gemv_launch_m<F>(M, dump, dim3((unsigned)sh.grid), lds, st, a);
+                gemv_launch_m<F>(M, dump, dim3((unsigned)p.grid), lds, st, a);
             if (!launched(fn))
                 return false;
         }

@@ -31,6 +31,7 @@ namespace llamql
     constexpr int MFMA_TILE_ROWS = 32;
     constexpr int MFMA_MAX_SLICES = 8;
     constexpr int MFMA_MAX_WAVES = 16;     // wavefronts per workgroup
+    constexpr int MFMA_DUMP_WAVES = 8;     // the same for the block-sum variant
     constexpr int MFMA_LOADS = 5;          // vector memory loads per step and lane
     constexpr int MFMA_BOUNCE = 5 * 1024;  // LDS bytes of a wavefront's bounce buffer (320 pieces, 288 used)
 
@@ -48,6 +49,10 @@ namespace llamql
         int M;            // activation rows, 1..8
         int slices;       // wavefronts per 32-row tile (wavefront j walks super-blocks j, j + slices, ..);
                           // a workgroup holds blockDim/64/slices tiles
+        // DUMP kernels only: the exact per-block int32 sums of rows [row0, row0+nrows) go to
+        // sums[(m * nrows + row - row0) * (SB * 8) + block]
+        int32_t *sums;
+        int row0, nrows;
     };
 
     // LDS: per 32-column block 8 activation rows x 32 int8 (16 bytes of padding: neighbouring
@@ -184,8 +189,13 @@ namespace llamql
     }
 
     // SRC: where the activations come from (QUAD_SRC_*): Q8_1 blocks, or fp32 rows quantised here.
-    template <int SRC>
-    __global__ void __launch_bounds__(MFMA_MAX_WAVES *WAVE) gemv_mfma_q4k_kernel(const MfmaArgs a)
+    // DUMP: also store the matrix unit's results, the exact int32 block sums (the parity hook).
+    // Its stores need registers the 16-wavefront workgroup does not have (and the build refuses to
+    // spill): the variant runs in workgroups of at most MFMA_DUMP_WAVES wavefronts, fewer tiles per
+    // workgroup, the same code per tile.
+    template <int SRC, bool DUMP = false>
+    __global__ void __launch_bounds__((DUMP ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES) * WAVE)
+        gemv_mfma_q4k_kernel(const MfmaArgs a)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];
         const int nsb = a.SB;
@@ -250,6 +260,17 @@ namespace llamql
         mfma_keep(bufB);
 
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        // DUMP: byte offset from a.sums of this lane's sums of its first activation row (4 lh); the
+        // following rows lie dump_stride sums further each.  All ones outside the row window.  (The
+        // host keeps the whole dump below 4 GiB.)
+        uint32_t dump_off = 0xFFFFFFFFu;
+        const size_t dump_stride = (size_t)a.nrows * (size_t)nkb;
+        if constexpr (DUMP)
+        {
+            const long rr = row - a.row0;
+            if (row < a.N && rr >= 0 && rr < a.nrows)
+                dump_off = (uint32_t)((((size_t)(4 * lh) * a.nrows + (size_t)rr) * (size_t)nkb) * sizeof(int32_t));
+        }
         v16i zero;
 #pragma unroll
         for (int i = 0; i < 16; ++i)
@@ -311,6 +332,20 @@ namespace llamql
                 const float bs = Q4KQuad::scale_f32(S[j >> 1], j & 1);
                 const float bm = Q4KQuad::min_f32(S[j >> 1], j & 1);
                 const v16i d = idot[j & 1];
+                if constexpr (DUMP)
+                {
+                    if (dump_off != 0xFFFFFFFFu)
+                    {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (4 * lh + i < a.M)
+                            {
+                                // uniform base in scalar registers, one 32-bit lane offset
+                                char *base = reinterpret_cast<char *>(a.sums) + ((size_t)(sb * 8 + j) + (size_t)i * dump_stride) * sizeof(int32_t);
+                                *reinterpret_cast<int32_t *>(base + dump_off) = d[i];
+                            }
+                    }
+                }
                 acc[0] = fmaf((float)d[0], ad.x * bs, acc[0]);
                 acc[0] = fmaf(asd.x, bm, acc[0]);
                 acc[1] = fmaf((float)d[1], ad.y * bs, acc[1]);
@@ -366,8 +401,11 @@ namespace llamql
                 for (int s = 1; s < a.slices; ++s)
                     v += red[((wave + s) * 4 + i) * WAVE + lane];
                 const int m = 4 * lh + i;
-                if (m < a.M && row < a.N)
-                    a.y[(size_t)m * a.ldy + row] = v;
+                if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
+                {
+                    if (m < a.M && row < a.N)
+                        a.y[(size_t)m * a.ldy + row] = v;
+                }
             }
         }
     }
@@ -390,7 +428,7 @@ namespace llamql
     // super-blocks long; tiles per workgroup so that every workgroup of the launch is resident
     // at once (a second round of workgroups would run nearly alone on the chip and cost a
     // workgroup's whole latency again) and the activations are staged less often.
-    inline MfmaShape gemv_mfma_shape(long N, int nsb, int cus)
+    inline MfmaShape gemv_mfma_shape(long N, int nsb, int cus, int max_waves = MFMA_MAX_WAVES)
     {
         const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
         long want = ((long)cus * 12 + tiles - 1) / tiles;
@@ -406,12 +444,12 @@ namespace llamql
         // workgroups a compute unit holds at once: by LDS, and 16 wavefronts at this kernel's registers
         auto resident = [&](int t) {
             const long by_lds = (long)(QUAD_MAX_LDS / mfma_lds_bytes(nsb, t * sh.slices));
-            const long by_waves = MFMA_MAX_WAVES / (t * sh.slices);
+            const long by_waves = max_waves / (t * sh.slices);
             const long r = by_lds < by_waves ? by_lds : by_waves;
             return r < 1 ? 1 : r;
         };
         int t = 1;
-        while (t * 2 * sh.slices <= MFMA_MAX_WAVES && mfma_lds_bytes(nsb, t * 2 * sh.slices) <= QUAD_MAX_LDS &&
+        while (t * 2 * sh.slices <= max_waves && mfma_lds_bytes(nsb, t * 2 * sh.slices) <= QUAD_MAX_LDS &&
                (tiles + t - 1) / t > (long)cus * resident(t))
             t *= 2;
         sh.tiles_per_wg = t;

@@ -33,6 +33,7 @@ namespace llamql
 {
     constexpr int MFMA6_PRODUCERS = 2;     // wavefronts that only stage activations
     constexpr int MFMA6_MAX_COMPUTE = 8;   // compute wavefronts per workgroup
+    constexpr int MFMA6_DUMP_COMPUTE = 6;  // the same for the block-sum variant
     constexpr int MFMA6_LOADS = 8;         // vector memory loads per super-block and lane
     constexpr int MFMA6_QL_STRIDE = 144;   // bounce buffer: bytes between the ql lines of two rows
     constexpr int MFMA6_QH_STRIDE = 80;    // and between their 64 bytes of qh
@@ -53,6 +54,10 @@ namespace llamql
         int slices; // compute wavefronts per 32-row tile
         int tiles;  // tiles per workgroup
         int chunk;  // super-blocks per activation buffer; a multiple of slices when SB > chunk
+        // DUMP kernels only: the exact per-block int32 sums of rows [row0, row0+nrows) go to
+        // sums[(m * nrows + row - row0) * (SB * 8) + block]
+        int32_t *sums;
+        int row0, nrows;
     };
 
     struct Mfma6Raw
@@ -109,8 +114,11 @@ namespace llamql
         return mfma6_act_bytes(nsb, chunk) + (size_t)ncomp * MFMA6_BOUNCE;
     }
 
-    template <int SRC>
-    __global__ void __launch_bounds__((MFMA6_MAX_COMPUTE + MFMA6_PRODUCERS) * WAVE)
+    // DUMP: also store the matrix unit's results, the exact int32 block sums (the parity hook).
+    // Its stores need a few registers more than ten wavefronts leave each lane (and the build
+    // refuses to spill): the variant runs with at most MFMA6_DUMP_COMPUTE compute wavefronts.
+    template <int SRC, bool DUMP = false>
+    __global__ void __launch_bounds__(((DUMP ? MFMA6_DUMP_COMPUTE : MFMA6_MAX_COMPUTE) + MFMA6_PRODUCERS) * WAVE)
         gemv_mfma_q6k_kernel(const Mfma6Args a)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma6_lds[];
@@ -201,6 +209,18 @@ namespace llamql
             mfma6_keep(bufA); // the staging code must not reuse the registers of the loads in flight
             mfma6_keep(bufB);
 
+            // DUMP: byte offset from a.sums of this lane's sums of its first activation row (4 lh); the
+            // following rows lie dump_stride sums further each.  All ones outside the row window.  (The
+            // host keeps the whole dump below 4 GiB.)
+            uint32_t dump_off = 0xFFFFFFFFu;
+            const size_t dump_stride = (size_t)a.nrows * ((size_t)nsb * 8);
+            if constexpr (DUMP)
+            {
+                const long row = tile_row0 + l32;
+                const long rr = row - a.row0;
+                if (row < a.N && rr >= 0 && rr < a.nrows)
+                    dump_off = (uint32_t)((((size_t)(4 * lh) * a.nrows + (size_t)rr) * ((size_t)nsb * 8)) * sizeof(int32_t));
+            }
             v16i zero;
 #pragma unroll
             for (int i = 0; i < 16; ++i)
@@ -272,6 +292,20 @@ namespace llamql
                     const float4 ad = *reinterpret_cast<const float4 *>(sb_sc + j * 16);
                     const v16i dd = idot[j & 1];
                     const float b = bs[j & 1];
+                    if constexpr (DUMP)
+                    {
+                        if (dump_off != 0xFFFFFFFFu)
+                        {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                if (4 * lh + i < a.M)
+                                {
+                                    // uniform base in scalar registers, one 32-bit lane offset
+                                    char *base = reinterpret_cast<char *>(a.sums) + ((size_t)(sb * 8 + j) + (size_t)i * dump_stride) * sizeof(int32_t);
+                                    *reinterpret_cast<int32_t *>(base + dump_off) = dd[i];
+                                }
+                        }
+                    }
                     acc[0] = fmaf((float)dd[0], ad.x * b, acc[0]);
                     acc[1] = fmaf((float)dd[1], ad.y * b, acc[1]);
                     acc[2] = fmaf((float)dd[2], ad.z * b, acc[2]);
@@ -336,8 +370,11 @@ namespace llamql
                     for (int s = 1; s < a.slices; ++s)
                         v += red[((wave + s) * 4 + i) * WAVE + lane];
                     const int m = 4 * (lane >> 5) + i;
-                    if (m < a.M && row < a.N)
-                        a.y[(size_t)m * a.ldy + row] = v;
+                    if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
+                    {
+                        if (m < a.M && row < a.N)
+                            a.y[(size_t)m * a.ldy + row] = v;
+                    }
                 }
             }
         }
@@ -351,14 +388,14 @@ namespace llamql
     // Slices so that a compute unit sees about eight compute wavefronts, five at least (the
     // scales of eight neighbouring super-blocks share a cache line) and each two steps long;
     // tiles per workgroup to fill its compute wavefronts when there are tiles to spare.
-    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus)
+    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus, int max_compute = MFMA6_MAX_COMPUTE)
     {
         const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
-        long want = ((long)cus * MFMA6_MAX_COMPUTE + tiles - 1) / tiles;
+        long want = ((long)cus * max_compute + tiles - 1) / tiles;
         if (want < 5)
             want = 5;
-        if (want > MFMA6_MAX_COMPUTE)
-            want = MFMA6_MAX_COMPUTE;
+        if (want > max_compute)
+            want = max_compute;
         if (want > nsb / 2)
             want = nsb / 2;
         if (want < 1)
@@ -366,7 +403,7 @@ namespace llamql
         Mfma6Shape sh;
         sh.slices = (int)want;
         int t = 1;
-        while ((t * 2) * sh.slices <= MFMA6_MAX_COMPUTE && tiles / (t * 2) >= 2L * cus)
+        while ((t * 2) * sh.slices <= max_compute && tiles / (t * 2) >= 2L * cus)
             t *= 2;
         sh.tiles = t;
         sh.grid = (tiles + t - 1) / t;

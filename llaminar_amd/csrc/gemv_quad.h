@@ -61,6 +61,10 @@ namespace llamql
         int R[QUAD_MAX_PROJ]; // rows per wavefront
         int wave_begin[QUAD_MAX_PROJ];
         int first_b; // nproj in a launch of one format
+        // DUMP kernels only (one matrix): the exact per-block int32 sums of rows [row0, row0+nrows)
+        // go to sums[(m * nrows + row - row0) * (SB * 8) + block]
+        int32_t *sums;
+        int row0, nrows;
     };
 
     // LDS bytes for M activation rows of nsb super-blocks.
@@ -508,7 +512,7 @@ namespace llamql
     template <class Q, int M, int U>
     __device__ __forceinline__ void quad_compute_step(const typename Q::Raw &r, const typename Q::Lane &lc,
                                                       const uint8_t *aq_lane, const uint8_t *ads_lane, int aq_stride,
-                                                      int ads_stride, float (&t)[M])
+                                                      int ads_stride, float (&t)[M], int (&idot)[M][2])
     {
         v4i w[4];
         typename Q::Scale S;
@@ -522,9 +526,9 @@ namespace llamql
             const v4i a2 = *reinterpret_cast<const v4i *>(ap + 2048);
             const v4i a3 = *reinterpret_cast<const v4i *>(ap + 3072);
             const float4 sd = *reinterpret_cast<const float4 *>(ads_lane + m * ads_stride);
-            const int idot0 = dot16(a1, w[1], dot16(a0, w[0], 0));
-            const int idot1 = dot16(a3, w[3], dot16(a2, w[2], 0));
-            t[m] = Q::apply(S, idot0, idot1, sd, 0.0f);
+            idot[m][0] = dot16(a1, w[1], dot16(a0, w[0], 0));
+            idot[m][1] = dot16(a3, w[3], dot16(a2, w[2], 0));
+            t[m] = Q::apply(S, idot[m][0], idot[m][1], sd, 0.0f);
         }
     }
 
@@ -563,7 +567,9 @@ namespace llamql
             }
     }
 
-    template <class Q, int M, int U, int SRC>
+    // DUMP: also store the exact int32 block sums the lanes form (the parity hook of the C-ABI);
+    // everything else is the same code.
+    template <class Q, int M, int U, int SRC, bool DUMP = false>
     __device__ __forceinline__ void quad_body(const QuadArgs &qa, uint8_t *quad_lds, int p, int w_first, int wid_all)
     {
         const int nsb = qa.SB;
@@ -639,10 +645,25 @@ namespace llamql
             const uint8_t *aq_lane = aq + ((sbr >> 4) << 12) + ((sbr & 15) << 6) + (l << 4);
             const uint8_t *ads_lane = ads + (sbr << 6) + (l << 4);
             float t[M];
-            quad_compute_step<Q, M, U>(r, lc, aq_lane, ads_lane, aq_stride, ads_stride, t);
+            int idot[M][2]; // the lane's two exact block sums per activation row
+            quad_compute_step<Q, M, U>(r, lc, aq_lane, ads_lane, aq_stride, ads_stride, t, idot);
 
             const int gb = nsb - first;                       // lane groups still in the current row
             const int ge = total - step * QUAD_STEP_SB;       // lane groups with data at all
+            if constexpr (DUMP)
+            {
+                const long rr = (grp < gb ? row : row + 1) - qa.row0;
+                if (grp < ge && rr >= 0 && rr < qa.nrows)
+                {
+#pragma unroll
+                    for (int m = 0; m < M; ++m)
+                    {
+                        int32_t *dst = qa.sums + ((size_t)m * qa.nrows + (size_t)rr) * ((size_t)nsb * 8) + (size_t)sbr * 8;
+                        dst[Q::block_of(l, 0)] = idot[m][0];
+                        dst[Q::block_of(l, 1)] = idot[m][1];
+                    }
+                }
+            }
             {
                 // one code shape for every step keeps cur/nxt in registers
                 const bool in_cur = grp < gb && grp < ge;
@@ -661,8 +682,11 @@ namespace llamql
                 for (int m = 0; m < M; ++m)
                 {
                     const float tot = wave_sum(cur[m]);
-                    if (lane == 0)
-                        y[(size_t)m * ldy + row] = tot;
+                    if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
+                    {
+                        if (lane == 0)
+                            y[(size_t)m * ldy + row] = tot;
+                    }
                     cur[m] = nxt[m];
                     nxt[m] = 0.0f;
                 }
@@ -703,7 +727,7 @@ namespace llamql
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the run
     }
 
-    template <class Q, int M, int U, int SRC>
+    template <class Q, int M, int U, int SRC, bool DUMP = false>
     __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const QuadArgs qa)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
@@ -711,7 +735,7 @@ namespace llamql
         const int wid_all = (int)blockIdx.x * (int)(blockDim.x >> 6) + wave;
         int p, w_first;
         quad_which(qa, wid_all, p, w_first);
-        quad_body<Q, M, U, SRC>(qa, quad_lds, p, w_first, wid_all);
+        quad_body<Q, M, U, SRC, DUMP>(qa, quad_lds, p, w_first, wid_all);
     }
 
     // Two formats in one launch (Q and K in Q4_K, V in Q6_K): whole workgroups belong to one
@@ -731,17 +755,23 @@ namespace llamql
             quad_body<QB, M, UB, SRC>(qa, quad_lds, p, w_first, wid_all);
     }
 
-    template <class Q, int M, int U, int SRC>
+    template <class Q, int M, int U, int SRC, bool DUMP = false>
     inline void gemv_quad_launch_mus(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         static LdsGrant grant;
-        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC>), QUAD_MAX_LDS);
-        hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U, SRC>), grid, block, lds, st, a);
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC, DUMP>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U, SRC, DUMP>), grid, block, lds, st, a);
     }
 
+    // a.sums set: the block-sum variant of the same kernel (Q8_1 input only)
     template <class Q, int M, int U>
     inline void gemv_quad_launch_mu(int src, dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
+        if (a.sums)
+        {
+            gemv_quad_launch_mus<Q, M, U, QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            return;
+        }
         switch (src)
         {
         case QUAD_SRC_F32: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_F32>(grid, block, lds, st, a); break;

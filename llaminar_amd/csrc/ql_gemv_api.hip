@@ -11,6 +11,7 @@ namespace llamql
                          int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
     bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
                           int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
+    void gemv_describe(uint8_t fmt, int M, int N, int K, int device_id, llam_ql_gemv_plan *out);
     int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const ActSource &src, int M, int K,
                           int device_id, hipStream_t st);
 
@@ -320,7 +321,23 @@ extern "C" bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void
         return fail(fn, "null output");
     if (row0 < 0 || nrows < 1 || (long)row0 + nrows > N)
         return fail(fn, "row window [%d,%d) outside [0,%d)", row0, row0 + nrows, N);
+    if ((size_t)M * (size_t)nrows * (size_t)(K / 32) * sizeof(int32_t) >= ((size_t)1 << 31))
+        return fail(fn, "M=%d x %d rows x %d blocks of sums exceed 2 GiB", M, nrows, K / 32);
     if (!set_device(fn, device_id))
         return false;
     return dispatch(fn, fmt, d_w, d_q8, nullptr, d_sums, M, N, K, 0, row0, nrows, device_id, as_stream(stream));
+}
+
+extern "C" bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int device_id, llam_ql_gemv_plan *out)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_describe";
+    if (!out)
+        return fail(fn, "null output");
+    if (fmt != LLAM_FMT_Q4_K && fmt != LLAM_FMT_Q6_K && fmt != LLAM_FMT_IQ3_S)
+        return fail(fn, "unsupported weight format id %d", (int)fmt);
+    if (M < 1 || M > LLAM_QL_MAX_GEMV_M || N < 1 || K < 1 || (K % 256) != 0)
+        return fail(fn, "bad shape (M=%d N=%d K=%d)", M, N, K);
+    gemv_describe(fmt, M, N, K, device_id, out); // no device call: the unit count falls back to 256
+    return true;
 }

@@ -54,6 +54,23 @@ def test_gemm_rows_equal_gemv(capi, dev, oracle, fmt):
     assert rel_err(yg.cpu().numpy(), yv.cpu().numpy()) <= 2e-6
 
 
+@pytest.mark.parametrize("fmt", list(FMTS.values()), ids=list(FMTS))
+@pytest.mark.parametrize("M,N,K,r0,nr", [(1, 128, 256, 0, 128), (17, 100, 512, 37, 63), (130, 257, 768, 190, 67),
+                                         (300, 200, 2048, 60, 70)])
+def test_block_sums_of_the_gemm_kernel(capi, dev, oracle, fmt, M, N, K, r0, nr):
+    """The matrix unit's per-block results of llam_ql_gemm's own kernel (block-sum variant) are
+    the reference's int32 sums bit for bit: ragged tiles, windows that start and end inside a
+    64-row tile, token tails."""
+    W = synth.weights_numpy(fmt, N, K, 70 + M + N)
+    q8 = oracle.quantize(synth.activations_numpy(M, K, 90 + K))
+    wd = upload_weights(capi, dev, fmt, W)
+    qd = upload_q8(dev, q8)
+    s = capi.gemm_block_sums(fmt, wd, qd, M, N, K, r0, nr)
+    sync()
+    _, sums = oracle.gemm(fmt, W, K, q8, n0=r0, n1=r0 + nr, want_sums=True)
+    assert np.array_equal(s.cpu().numpy(), sums)
+
+
 def test_prefill_config_full_size(capi, dev, oracle):
     """Config 3: M=512, K=5120, N=25600, Q4_K.  Oracle on a window of weight rows for all
     512 tokens; determinism over the whole output."""
@@ -73,8 +90,11 @@ def test_prefill_config_full_size(capi, dev, oracle):
     assert np.array_equal(qd.cpu().numpy().reshape(q8.shape), q8)
     Wh = wd.cpu().numpy()
     for n0 in (0, 12800 - 32, N - 64):
-        C = oracle.gemm(fmt, Wh, K, q8, n0=n0, n1=n0 + 64)
+        C, sums = oracle.gemm(fmt, Wh, K, q8, n0=n0, n1=n0 + 64, want_sums=True)
         assert rel_err(y.cpu().numpy()[:, n0:n0 + 64], C) <= TOL[fmt] * 1e-2
+        s = capi.gemm_block_sums(fmt, wd, qd, M, N, K, n0, 64)
+        sync()
+        assert np.array_equal(s.cpu().numpy(), sums), f"block sums of rows from {n0}"
     assert np.isfinite(y.cpu().numpy()).all()
 
 

@@ -440,3 +440,120 @@ def test_q6k_subscale_pairs_on_the_matrix_unit_bit_exact(capi, dev, oracle):
     sync()
     C = oracle.gemm(FMT_Q6_K, W, K, q8)
     assert np.array_equal(y.cpu().numpy().view(np.uint32), C.view(np.uint32))
+
+
+# ---- the block sums come from the kernel that serves the shape -------------------------------
+# llam_ql_gemv_block_sums executes llam_ql_gemv's launch plan with the chosen kernel's block-sum
+# variant, so each case below pins the integer pipeline of one production kernel; the expected
+# kernel is asserted through llam_ql_gemv_describe so that a change of the dispatch shows up here.
+def _production_cases():
+    from llaminar_amd.capi import KERNEL_CHUNKED as CH, KERNEL_GENERIC as GE, KERNEL_MFMA as MF, KERNEL_QUAD as QU
+
+    return [
+        ("q4k_quad_m1", FMT_Q4_K, 777, 5120, 1, QU),
+        ("q4k_quad_m4_row_ends_inside_steps", FMT_Q4_K, 1030, 4352, 4, QU),
+        ("q4k_quad_batch_split_m5", FMT_Q4_K, 100, 25600, 5, QU),
+        ("q6k_quad_m1", FMT_Q6_K, 1024, 5120, 1, QU),
+        ("q6k_quad_m8", FMT_Q6_K, 700, 5120, 8, QU),
+        ("q6k_quad_m4_long_rows", FMT_Q6_K, 64, 25600, 4, QU),
+        ("q4k_mfma_m8", FMT_Q4_K, 4100, 5120, 8, MF),
+        ("q4k_mfma_m5", FMT_Q4_K, 4096, 4096, 5, MF),
+        ("q6k_mfma_m8_chunked_row", FMT_Q6_K, 200, 25600, 8, MF),
+        ("q6k_mfma_m7_short_last_chunk", FMT_Q6_K, 70, 17408, 7, MF),
+        ("iq3s_chunked_m1", FMT_IQ3_S, 1000, 5120, 1, CH),
+        ("iq3s_chunked_m8", FMT_IQ3_S, 300, 5120, 8, CH),
+        ("iq3s_k_sliced_m4", FMT_IQ3_S, 50, 25600, 4, CH),
+        ("q4k_chunked_m3", FMT_Q4_K, 500, 2048, 3, CH),
+        ("q6k_chunked_m6_batch_split", FMT_Q6_K, 90, 3072, 6, CH),
+        ("q6k_generic_m2", FMT_Q6_K, 100, 512, 2, GE),
+        ("iq3s_generic_m1", FMT_IQ3_S, 33, 1024, 1, GE),
+    ]
+
+
+@pytest.mark.parametrize("case", _production_cases(), ids=[c[0] for c in _production_cases()])
+def test_block_sums_of_the_production_kernels(capi, dev, oracle, case):
+    name, fmt, N, K, M, kernel = case
+    print(f"[block sums] {name}: fmt {fmt} N={N} K={K} M={M}", flush=True)
+    plan = capi.gemv_describe(fmt, M, N, K)
+    assert plan.kernel == kernel, f"{name}: the dispatcher now picks kernel {plan.kernel}"
+    W = synth.weights_numpy(fmt, N, K, 1000 + N + M)
+    q8 = oracle.quantize(synth.activations_numpy(M, K, 2000 + K))
+    wd = upload_weights(capi, dev, fmt, W)
+    qd = upload_q8(dev, q8)
+    y = capi.gemv(fmt, wd, qd, M, N, K)
+    windows = [(0, min(N, 40)), (max(0, N - 33), N)] + ([(N // 2 - 7, N // 2 + 30)] if N > 200 else [])
+    for r0, r1 in windows:
+        s = capi.gemv_block_sums(fmt, wd, qd, M, N, K, r0, r1 - r0)
+        sync()
+        C, sums = oracle.gemm(fmt, W, K, q8, n0=r0, n1=r1, want_sums=True)
+        assert np.array_equal(s.cpu().numpy(), sums), f"{name}: block sums of rows [{r0},{r1}) differ"
+        assert rel_err(y.cpu().numpy()[:, r0:r1], C) <= TOL[fmt] * 1e-2
+
+
+def test_config1_q4k_5120x5120(capi, dev, oracle):
+    """BASELINE config 1: one Q4_K GEMV, N = K = 5120, batch 1.  Block sums of the quad-lane
+    kernel on row windows, fp32 over ALL rows against the oracle, bitwise repeatability, and the
+    fp32-input entry point (quantiser inside the kernel) with the same bits."""
+    import torch
+
+    fmt, N, K = FMT_Q4_K, 5120, 5120
+    assert capi.gemv_describe(fmt, 1, N, K).kernel == capi.KERNEL_QUAD
+    W = synth.weights_numpy(fmt, N, K, 20240)
+    x = synth.activations_numpy(1, K, 20241)
+    q8 = oracle.quantize(x)
+    wd = upload_weights(capi, dev, fmt, W)
+    xd = torch.from_numpy(x).to(dev)
+    qd = capi.quantize_q8_1(xd)
+    sync()
+    assert np.array_equal(qd.cpu().numpy().reshape(q8.shape), q8), "Q8_1 bytes differ from the oracle"
+    y = capi.gemv(fmt, wd, qd, 1, N, K)
+    y_again = capi.gemv(fmt, wd, qd, 1, N, K)
+    y_f32 = capi.gemv_f32(fmt, wd, xd, 1, N, K)
+    sync()
+    C = oracle.gemm(fmt, W, K, q8)
+    assert rel_err(y.cpu().numpy(), C) <= TOL[fmt] * 1e-2
+    assert torch.equal(y, y_again) and torch.equal(y, y_f32)
+    for r0 in (0, 2537, N - 64):
+        s = capi.gemv_block_sums(fmt, wd, qd, 1, N, K, r0, 64)
+        sync()
+        _, sums = oracle.gemm(fmt, W, K, q8, n0=r0, n1=r0 + 64, want_sums=True)
+        assert np.array_equal(s.cpu().numpy(), sums), f"rows from {r0}"
+    # doubling the activations doubles d of every Q8_1 block and leaves the quants alone:
+    # the output doubles exactly (a size-independent check of the whole row range)
+    y2 = capi.gemv_f32(fmt, wd, 2.0 * xd, 1, N, K)
+    sync()
+    assert torch.equal(y2, 2.0 * y)
+
+
+@pytest.mark.parametrize("M", [1, 8])
+def test_lm_head_shape_q6k_152064x5120(capi, dev, oracle, M):
+    """The lm_head of config 5 at full size: oracle on row windows at both ends and in the
+    middle (block sums bit-exact, fp32 close), properties over all 152064 rows."""
+    import torch
+
+    fmt, N, K = FMT_Q6_K, 152064, 5120
+    raw = synth.weights_torch(fmt, N, K, 777, dev)
+    wd = capi.prepare_weights(fmt, raw, N, K)
+    x = synth.activations_numpy(8, K, 778)
+    q8 = oracle.quantize(x)
+    qd = upload_q8(dev, q8[:M])
+    y = capi.gemv(fmt, wd, qd, M, N, K)
+    y_again = capi.gemv(fmt, wd, qd, M, N, K)
+    sync()
+    assert torch.equal(y, y_again)
+    assert bool(torch.isfinite(y).all())
+    bb = 210 * (K // 256)
+    for r0 in (0, 76000, N - 48):
+        Wh = raw[r0 * bb:(r0 + 48) * bb].cpu().numpy().reshape(48, K // 256, 210)
+        s = capi.gemv_block_sums(fmt, wd, qd, M, N, K, r0, 48)
+        sync()
+        C, sums = oracle.gemm(fmt, Wh, K, q8[:M], want_sums=True)
+        assert np.array_equal(s.cpu().numpy(), sums), f"rows from {r0}"
+        assert rel_err(y.cpu().numpy()[:, r0:r0 + 48], C) <= TOL[fmt] * 1e-2
+    if M == 8:
+        # a batch row has the bits of its single-row call (Q6_K rows of this length stay on
+        # the quad-lane kernel at every batch size)
+        assert capi.gemv_describe(fmt, 8, N, K).decode_equivalent == 1
+        y1 = capi.gemv(fmt, wd, upload_q8(dev, q8[5:6]), 1, N, K)
+        sync()
+        assert torch.equal(y[5], y1[0])
