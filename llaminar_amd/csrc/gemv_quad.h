@@ -14,10 +14,14 @@
 // super-blocks (K >= 4096) so that a step touches at most two rows.
 //
 // Loads run U steps ahead in two alternating register buffers.  Activations (Q8_1)
-// are staged once per workgroup in LDS, laid out so that each of a lane's reads is a
-// conflict-free ds_read_b128:
-//   quants  [m][sb/16][part 0..3][sb%16][l][16 B]   part = 2*(block&1) + half
-//   scales  [m][sb][l]{f32 d, f32 sum*d of block 2l ; same of block 2l+1}
+// are staged once per workgroup in LDS, 320 bytes per super-block and activation row:
+//   [m][sb]{ part 0..3: [l][16 B of quants]   part = 2*(first|second block of the lane) + half
+//            [l]{f32 d, f32 sum*d of the lane's first block ; same of its second} }
+// so a lane reads its five 16-byte pieces at fixed offsets from ONE address (the super-block
+// of a lane changes by 16 modulo the row length from step to step) and the 16 lanes served
+// together fall into different banks.  The Q8_1 blocks are asked for BEFORE the first weight
+// chunks: a wavefront's loads return in issue order, and activations queued behind 14 KB of
+// weights would hold up the staging, the barrier and with them the first product.
 //
 // Per block: idot exact; acc = fma(float(idot), f32(a.d)*b_scale, acc);
 // acc = fma(float(a.sum)*f32(a.d), b_min, acc) -- the reference's arithmetic
@@ -68,10 +72,10 @@ namespace llamql
     };
 
     // LDS bytes for M activation rows of nsb super-blocks.
+    constexpr int QUAD_SB_LDS = 320; // LDS bytes per super-block and activation row
     inline size_t quad_lds_bytes(int M, int nsb)
     {
-        const size_t chunks = (size_t)(nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
-        return (size_t)M * (chunks * 4096 + (size_t)nsb * 64);
+        return (size_t)M * (size_t)nsb * QUAD_SB_LDS;
     }
 
     // One thread per Q8_1 block.  Block j of a super-block goes to the quad lane that
@@ -95,11 +99,70 @@ namespace llamql
                 const int sb = kb >> 3, j = kb & 7;
                 int l, odd;
                 Q::owner(j, l, odd);
-                *reinterpret_cast<float2 *>(ads + m * ads_stride + sb * 64 + l * 16 + odd * 8) =
-                    make_float2(d, (float)(int16_t)(v[0] >> 16) * d);
-                uint8_t *base = aq + m * aq_stride + (sb >> 4) * 4096 + (odd * 2) * 1024 + (sb & 15) * 64 + l * 16;
-                *reinterpret_cast<uint4 *>(base) = make_uint4(v[1], v[2], v[3], v[4]);
-                *reinterpret_cast<uint4 *>(base + 1024) = make_uint4(v[5], v[6], v[7], v[8]);
+                uint8_t *base = aq + m * aq_stride + sb * QUAD_SB_LDS + l * 16;
+                *reinterpret_cast<float2 *>(base + 256 + odd * 8) = make_float2(d, (float)(int16_t)(v[0] >> 16) * d);
+                *reinterpret_cast<uint4 *>(base + (odd * 2) * 64) = make_uint4(v[1], v[2], v[3], v[4]);
+                *reinterpret_cast<uint4 *>(base + (odd * 2 + 1) * 64) = make_uint4(v[5], v[6], v[7], v[8]);
+            }
+        }
+    }
+
+    // Q8_1 blocks fetched ahead of the weights.  A wavefront's loads return in the order they
+    // were issued: activations asked for after the first weight chunks would arrive behind
+    // them, and the staging (and the barrier after it) would wait for 18 KB of weights per
+    // wavefront first.  Here every thread asks for up to QUAD_ACT_PASSES blocks before the
+    // weight loads go out and waits for exactly those (the weights stay in flight).  The loads
+    // are assembly so that the kernel decides where they are waited for; they are never
+    // predicated (threads without a block re-read the last one).
+    constexpr int QUAD_ACT_PASSES = 2;
+    struct QuadActRaw
+    {
+        v4i lo, hi;
+        int tail;
+    };
+    __device__ __forceinline__ void quad_act_issue(QuadActRaw (&r)[QUAD_ACT_PASSES], const uint32_t *q8, int total)
+    {
+#pragma unroll
+        for (int p = 0; p < QUAD_ACT_PASSES; ++p)
+        {
+            int idx = (int)threadIdx.x + p * (int)blockDim.x;
+            idx = idx < total ? idx : total - 1;
+            const uint32_t *src = q8 + (size_t)idx * 9;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r[p].lo) : "v"(src));
+            asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=&v"(r[p].hi) : "v"(src));
+            asm volatile("global_load_dword %0, %1, off offset:32" : "=&v"(r[p].tail) : "v"(src));
+        }
+    }
+    // until at most NEWER vector memory operations issued after the activation loads are pending
+    template <int NEWER>
+    __device__ __forceinline__ void quad_act_wait(QuadActRaw (&r)[QUAD_ACT_PASSES])
+    {
+        static_assert(NEWER <= 63, "vmcnt is a 6-bit counter");
+#pragma unroll
+        for (int p = 0; p < QUAD_ACT_PASSES; ++p)
+            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r[p].lo), "+v"(r[p].hi), "+v"(r[p].tail) : "n"(NEWER));
+    }
+    template <class Q>
+    __device__ __forceinline__ void quad_act_store(const QuadActRaw (&r)[QUAD_ACT_PASSES], int nsb, int total,
+                                                   uint8_t *aq, int aq_stride)
+    {
+        const int nkb = nsb * 8;
+#pragma unroll
+        for (int p = 0; p < QUAD_ACT_PASSES; ++p)
+        {
+            const int idx = (int)threadIdx.x + p * (int)blockDim.x;
+            if (idx < total)
+            {
+                const int m = idx / nkb, kb = idx - m * nkb;
+                const uint32_t head = (uint32_t)r[p].lo.x;
+                const float d = h2f((uint16_t)(head & 0xFFFFu));
+                const int sb = kb >> 3, j = kb & 7;
+                int l, odd;
+                Q::owner(j, l, odd);
+                uint8_t *base = aq + m * aq_stride + sb * QUAD_SB_LDS + l * 16;
+                *reinterpret_cast<float2 *>(base + 256 + odd * 8) = make_float2(d, (float)(int16_t)(head >> 16) * d);
+                *reinterpret_cast<v4i *>(base + (odd * 2) * 64) = (v4i){r[p].lo.y, r[p].lo.z, r[p].lo.w, r[p].hi.x};
+                *reinterpret_cast<v4i *>(base + (odd * 2 + 1) * 64) = (v4i){r[p].hi.y, r[p].hi.z, r[p].hi.w, r[p].tail};
             }
         }
     }
@@ -142,15 +205,14 @@ namespace llamql
                     const int sb = kb >> 3, j = kb & 7;
                     int l, odd;
                     Q::owner(j, l, odd);
+                    uint8_t *base = aq + m * aq_stride + sb * QUAD_SB_LDS + l * 16;
                     if (sub == 0)
                     {
                         const float d = h2f((uint16_t)(q.head & 0xFFFFu));
-                        *reinterpret_cast<float2 *>(ads + m * ads_stride + sb * 64 + l * 16 + odd * 8) =
+                        *reinterpret_cast<float2 *>(base + 256 + odd * 8) =
                             make_float2(d, (float)(int16_t)(q.head >> 16) * d);
                     }
-                    uint8_t *base = aq + m * aq_stride + (sb >> 4) * 4096 + (odd * 2 + (sub >> 2)) * 1024 +
-                                    (sb & 15) * 64 + l * 16 + (sub & 3) * 4;
-                    *reinterpret_cast<uint32_t *>(base) = q.packed;
+                    *reinterpret_cast<uint32_t *>(base + (odd * 2 + (sub >> 2)) * 64 + (sub & 3) * 4) = q.packed;
                 }
             }
         }
@@ -522,12 +584,12 @@ namespace llamql
         {
             const uint8_t *ap = aq_lane + m * aq_stride;
             const v4i a0 = *reinterpret_cast<const v4i *>(ap);
-            const v4i a1 = *reinterpret_cast<const v4i *>(ap + 1024);
-            const v4i a2 = *reinterpret_cast<const v4i *>(ap + 2048);
-            const v4i a3 = *reinterpret_cast<const v4i *>(ap + 3072);
-            const float4 sd = *reinterpret_cast<const float4 *>(ads_lane + m * ads_stride);
-            idot[m][0] = dot16(a1, w[1], dot16(a0, w[0], 0));
-            idot[m][1] = dot16(a3, w[3], dot16(a2, w[2], 0));
+            const v4i a1 = *reinterpret_cast<const v4i *>(ap + 64);
+            const v4i a2 = *reinterpret_cast<const v4i *>(ap + 128);
+            const v4i a3 = *reinterpret_cast<const v4i *>(ap + 192);
+            const float4 sd = *reinterpret_cast<const float4 *>(ap + 256);
+            idot[m][0] = dot16(a1, w[1], dot16z(a0, w[0]));
+            idot[m][1] = dot16(a3, w[3], dot16z(a2, w[2]));
             t[m] = Q::apply(S, idot[m][0], idot[m][1], sd, 0.0f);
         }
     }
@@ -573,10 +635,10 @@ namespace llamql
     __device__ __forceinline__ void quad_body(const QuadArgs &qa, uint8_t *quad_lds, int p, int w_first, int wid_all)
     {
         const int nsb = qa.SB;
-        const int aq_stride = ((nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB) * 4096;
-        const int ads_stride = nsb * 64;
+        const int aq_stride = nsb * QUAD_SB_LDS;
+        const int ads_stride = 0;
         uint8_t *aq = quad_lds;
-        uint8_t *ads = quad_lds + M * aq_stride;
+        uint8_t *ads = quad_lds;
 
         const int lane = threadIdx.x & (WAVE - 1);
         const int l = lane & 3;
@@ -613,13 +675,27 @@ namespace llamql
         };
 
         typename Q::Raw bufA[U], bufB[U];
-        load_chunk(bufA); // two chunks in flight while the activations are staged
-        load_chunk(bufB);
-
         if constexpr (SRC == QUAD_SRC_Q8)
-            quad_stage_q8<Q, M>(qa.q8, nsb, aq, ads, aq_stride, ads_stride);
+        {
+            // activations first (they return first), then two chunks of weights, which stay in
+            // flight while the activations are staged
+            const int total_blk = M * nsb * 8;
+            QuadActRaw ar[QUAD_ACT_PASSES];
+            quad_act_issue(ar, qa.q8, total_blk);
+            load_chunk(bufA);
+            load_chunk(bufB);
+            quad_act_wait<2 * U * Q::LOADS>(ar);
+            if (total_blk <= QUAD_ACT_PASSES * (int)blockDim.x) // uniform
+                quad_act_store<Q>(ar, nsb, total_blk, aq, aq_stride);
+            else
+                quad_stage_q8<Q, M>(qa.q8, nsb, aq, ads, aq_stride, ads_stride); // more blocks than the prefetch holds
+        }
         else
+        {
+            load_chunk(bufA); // two chunks in flight while the activations are quantised and staged
+            load_chunk(bufB);
             quad_stage_f32<Q, M, SRC>(qa.x, qa.x2, qa.ldx, nsb, aq, ads, aq_stride, ads_stride);
+        }
         __syncthreads();
         // the staging code above must not reuse the registers of the loads in flight
 #pragma unroll
@@ -629,24 +705,23 @@ namespace llamql
             Q::keep(bufB[u]);
         }
 
-        float cur[M], nxt[M];
+        float cur[M]; // this lane's share of the row being walked
 #pragma unroll
         for (int m = 0; m < M; ++m)
-            cur[m] = nxt[m] = 0.0f;
+            cur[m] = 0.0f;
 
         int first = 0;  // super-block (inside its row) that lane group 0 handles in this step
         long row = r0;  // row `cur` belongs to
         int step = 0;
 
         auto compute_step = [&](const typename Q::Raw &r) {
-            int sbr = first + grp;
-            if (sbr >= nsb)
-                sbr -= nsb;
-            const uint8_t *aq_lane = aq + ((sbr >> 4) << 12) + ((sbr & 15) << 6) + (l << 4);
-            const uint8_t *ads_lane = ads + (sbr << 6) + (l << 4);
+            // super-block of this lane inside its row: (first + grp) mod nsb (first < nsb, grp < 16 <= nsb)
+            const uint32_t x = (uint32_t)(first + grp);
+            const uint32_t sbr = min(x, x - (uint32_t)nsb);
+            const uint8_t *aq_lane = aq + sbr * QUAD_SB_LDS + (l << 4);
             float t[M];
             int idot[M][2]; // the lane's two exact block sums per activation row
-            quad_compute_step<Q, M, U>(r, lc, aq_lane, ads_lane, aq_stride, ads_stride, t, idot);
+            quad_compute_step<Q, M, U>(r, lc, aq_lane, aq_lane, aq_stride, ads_stride, t, idot);
 
             const int gb = nsb - first;                       // lane groups still in the current row
             const int ge = total - step * QUAD_STEP_SB;       // lane groups with data at all
@@ -664,37 +739,38 @@ namespace llamql
                     }
                 }
             }
+            if (ge < QUAD_STEP_SB) // the last step of the run: lane groups past its end hold nothing
             {
-                // one code shape for every step keeps cur/nxt in registers
-                const bool in_cur = grp < gb && grp < ge;
-                const bool in_nxt = grp >= gb && grp < ge;
 #pragma unroll
                 for (int m = 0; m < M; ++m)
-                {
-                    cur[m] += in_cur ? t[m] : 0.0f;
-                    nxt[m] += in_nxt ? t[m] : 0.0f;
-                }
+                    t[m] = grp < ge ? t[m] : 0.0f;
             }
             if (gb <= QUAD_STEP_SB)
             {
-                // the current row ends in this step
+                // the current row ends in this step: lane groups below gb finish it, the others
+                // start the next one
+                const bool fin = grp < gb;
 #pragma unroll
                 for (int m = 0; m < M; ++m)
                 {
-                    const float tot = wave_sum(cur[m]);
+                    const float tot = wave_sum(cur[m] + (fin ? t[m] : 0.0f));
                     if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
                     {
                         if (lane == 0)
                             y[(size_t)m * ldy + row] = tot;
                     }
-                    cur[m] = nxt[m];
-                    nxt[m] = 0.0f;
+                    cur[m] = fin ? 0.0f : t[m];
                 }
                 ++row;
                 first = QUAD_STEP_SB - gb;
             }
             else
+            {
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                    cur[m] += t[m];
                 first += QUAD_STEP_SB;
+            }
             ++step;
         };
 
@@ -786,8 +862,8 @@ namespace llamql
     {
         switch (M)
         {
-        case 1: gemv_quad_launch_mu<Q, 1, Q::LOADS <= 3 ? 3 : 2>(src, grid, block, lds, st, a); break;
-        case 2: gemv_quad_launch_mu<Q, 2, Q::LOADS <= 3 ? 3 : 2>(src, grid, block, lds, st, a); break;
+        case 1: gemv_quad_launch_mu<Q, 1, 2>(src, grid, block, lds, st, a); break;
+        case 2: gemv_quad_launch_mu<Q, 2, 2>(src, grid, block, lds, st, a); break;
         case 3: gemv_quad_launch_mu<Q, 3, 2>(src, grid, block, lds, st, a); break;
         case 4: gemv_quad_launch_mu<Q, 4, 2>(src, grid, block, lds, st, a); break;
         // (formats with many loads per step run out of registers at two steps per chunk)
@@ -802,7 +878,7 @@ namespace llamql
     template <class Q>
     constexpr int quad_unroll(int M)
     {
-        return M <= 2 ? (Q::LOADS <= 3 ? 3 : 2) : M <= 4 ? 2 : (Q::LOADS <= 3 ? 2 : 1);
+        return M <= 4 ? 2 : (Q::LOADS <= 3 ? 2 : 1);
     }
 
     template <class QA, class QB, int M, int SRC>

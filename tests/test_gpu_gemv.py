@@ -459,7 +459,7 @@ def _production_cases():
         ("q4k_mfma_m8", FMT_Q4_K, 4100, 5120, 8, MF),
         ("q4k_mfma_m5", FMT_Q4_K, 4096, 4096, 5, MF),
         ("q6k_mfma_m8_chunked_row", FMT_Q6_K, 200, 25600, 8, MF),
-        ("q6k_mfma_m7_short_last_chunk", FMT_Q6_K, 70, 17408, 7, MF),
+        ("q6k_mfma_m8_short_last_chunk", FMT_Q6_K, 70, 17408, 8, MF),
         ("iq3s_chunked_m1", FMT_IQ3_S, 1000, 5120, 1, CH),
         ("iq3s_chunked_m8", FMT_IQ3_S, 300, 5120, 8, CH),
         ("iq3s_k_sliced_m4", FMT_IQ3_S, 50, 25600, 4, CH),
