@@ -544,8 +544,11 @@ namespace llamql
             if (nw < 1)
                 nw = 1;
             const long grid = (waves + nw - 1) / nw;
-            gemv_quad_launch<typename F::Quad>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE),
-                                               quad_lds_bytes(M, SB), st, a);
+            size_t lds = quad_lds_bytes(M, SB);
+            a.ring = M == 1 && !d_sums && lds + (size_t)nw * QUAD_RING_BYTES <= QUAD_MAX_LDS;
+            if (a.ring)
+                lds += (size_t)nw * QUAD_RING_BYTES;
+            gemv_quad_launch<typename F::Quad>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
             return launched(fn);
         }
         else
@@ -611,8 +614,11 @@ namespace llamql
             if (at > 0x7FFFFFFFL / WAVE)
                 return fail(fn, "too many rows for one launch");
             const long grid = (at + nw - 1) / nw;
-            gemv_quad_dual_launch<QA, QB>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE),
-                                          quad_lds_bytes(M, SB), st, a);
+            size_t lds = quad_lds_bytes(M, SB);
+            a.ring = M == 1 && lds + (size_t)nw * QUAD_RING_BYTES <= QUAD_MAX_LDS;
+            if (a.ring)
+                lds += (size_t)nw * QUAD_RING_BYTES;
+            gemv_quad_dual_launch<QA, QB>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
             return launched(fn);
         }
         else

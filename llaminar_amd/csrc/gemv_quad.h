@@ -69,10 +69,21 @@ namespace llamql
         // go to sums[(m * nrows + row - row0) * (SB * 8) + block]
         int32_t *sums;
         int row0, nrows;
+        // single activation row: the launch reserves QUAD_RING_BYTES of LDS per wavefront behind
+        // the activations and the kernel runs in QUAD_MODE_RING
+        int ring;
     };
 
     // LDS bytes for M activation rows of nsb super-blocks.
     constexpr int QUAD_SB_LDS = 320; // LDS bytes per super-block and activation row
+    // Single activation row (QUAD_MODE_RING): finished rows park their 64 per-lane partial sums in a
+    // per-wavefront LDS ring and are reduced 16 rows at a time (lane = (row, quarter): 16 values each,
+    // then two exchanges inside the quad), so the loop carries no reduction chain and the row
+    // sums leave as 64-byte stores.  The additions are associated exactly as wave_sum() does it
+    // (pairs, quads, eights, sixteens, then (r0+r1)+(r2+r3)): the same bits either way.
+    constexpr int QUAD_RING_ROWS = 16;
+    constexpr int QUAD_RING_STRIDE = 68; // floats per parked row: 64 + 4 so neighbouring rows start 4 banks apart
+    constexpr size_t QUAD_RING_BYTES = (size_t)QUAD_RING_ROWS * QUAD_RING_STRIDE * 4;
     inline size_t quad_lds_bytes(int M, int nsb)
     {
         return (size_t)M * (size_t)nsb * QUAD_SB_LDS;
@@ -616,6 +627,15 @@ namespace llamql
     }
 
     // which matrix the wavefront works on, and the first wavefront of that matrix
+    // orders the LDS traffic of one wavefront as seen by the compiler; the hardware runs a
+    // wavefront's LDS instructions in order, so no instruction is needed
+    __device__ __forceinline__ void wave_lds_sync()
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
     __device__ __forceinline__ void quad_which(const QuadArgs &qa, int wid_all, int &p, int &w_first)
     {
         p = 0;
@@ -629,11 +649,14 @@ namespace llamql
             }
     }
 
-    // DUMP: also store the exact int32 block sums the lanes form (the parity hook of the C-ABI);
+    // MODE: QUAD_MODE_DUMP also stores the exact int32 block sums the lanes form (the parity hook of
+    // the C-ABI) and no fp32 output; QUAD_MODE_RING reduces finished rows through the LDS ring;
     // everything else is the same code.
-    template <class Q, int M, int U, int SRC, bool DUMP = false>
+    constexpr int QUAD_MODE_PLAIN = 0, QUAD_MODE_DUMP = 1, QUAD_MODE_RING = 2;
+    template <class Q, int M, int U, int SRC, int MODE = QUAD_MODE_PLAIN>
     __device__ __forceinline__ void quad_body(const QuadArgs &qa, uint8_t *quad_lds, int p, int w_first, int wid_all)
     {
+        constexpr bool DUMP = MODE == QUAD_MODE_DUMP, DEFER = MODE == QUAD_MODE_RING;
         const int nsb = qa.SB;
         const int aq_stride = nsb * QUAD_SB_LDS;
         const int ads_stride = 0;
@@ -714,6 +737,28 @@ namespace llamql
         long row = r0;  // row `cur` belongs to
         int step = 0;
 
+        float *ring = reinterpret_cast<float *>(quad_lds + (size_t)M * aq_stride) +
+                      (size_t)(threadIdx.x >> 6) * (QUAD_RING_ROWS * QUAD_RING_STRIDE * M);
+        int slot = 0; // parked rows: row - slot .. row - 1
+        auto flush_ring = [&]() {
+            wave_lds_sync(); // the wavefront's writes are in the ring (its LDS instructions run in order)
+            const int r = lane >> 2, q = lane & 3;
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+            {
+                const float4 *src = reinterpret_cast<const float4 *>(ring + (r * M + m) * QUAD_RING_STRIDE + q * 16);
+                const float4 v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
+                float sum = ((v0.x + v0.y) + (v0.z + v0.w)) + ((v1.x + v1.y) + (v1.z + v1.w));
+                sum += ((v2.x + v2.y) + (v2.z + v2.w)) + ((v3.x + v3.y) + (v3.z + v3.w));
+                sum += dpp_f32<DPP_QUAD_XOR1>(sum);
+                sum += dpp_f32<DPP_QUAD_XOR2>(sum);
+                if (q == 0 && r < slot)
+                    y[(size_t)m * ldy + (row - slot + r)] = sum;
+            }
+            wave_lds_sync(); // reads done before the ring is written again
+            slot = 0;
+        };
+
         auto compute_step = [&](const typename Q::Raw &r) {
             // super-block of this lane inside its row: (first + grp) mod nsb (first < nsb, grp < 16 <= nsb)
             const uint32_t x = (uint32_t)(first + grp);
@@ -750,18 +795,34 @@ namespace llamql
                 // the current row ends in this step: lane groups below gb finish it, the others
                 // start the next one
                 const bool fin = grp < gb;
-#pragma unroll
-                for (int m = 0; m < M; ++m)
+                if constexpr (DEFER)
                 {
-                    const float tot = wave_sum(cur[m] + (fin ? t[m] : 0.0f));
-                    if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
+#pragma unroll
+                    for (int m = 0; m < M; ++m)
                     {
-                        if (lane == 0)
-                            y[(size_t)m * ldy + row] = tot;
+                        ring[(slot * M + m) * QUAD_RING_STRIDE + lane] = cur[m] + (fin ? t[m] : 0.0f);
+                        cur[m] = fin ? 0.0f : t[m];
                     }
-                    cur[m] = fin ? 0.0f : t[m];
+                    ++slot;
+                    ++row;
+                    if (slot == QUAD_RING_ROWS) // uniform
+                        flush_ring();
                 }
-                ++row;
+                else
+                {
+#pragma unroll
+                    for (int m = 0; m < M; ++m)
+                    {
+                        const float tot = wave_sum(cur[m] + (fin ? t[m] : 0.0f));
+                        if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
+                        {
+                            if (lane == 0)
+                                y[(size_t)m * ldy + row] = tot;
+                        }
+                        cur[m] = fin ? 0.0f : t[m];
+                    }
+                    ++row;
+                }
                 first = QUAD_STEP_SB - gb;
             }
             else
@@ -801,9 +862,14 @@ namespace llamql
             load_chunk(bufB);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the run
+        if constexpr (DEFER)
+        {
+            if (slot > 0) // uniform
+                flush_ring();
+        }
     }
 
-    template <class Q, int M, int U, int SRC, bool DUMP = false>
+    template <class Q, int M, int U, int SRC, int MODE = QUAD_MODE_PLAIN>
     __global__ void __launch_bounds__(Q::max_threads(M)) gemv_quad_kernel(const QuadArgs qa)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t quad_lds[];
@@ -811,12 +877,12 @@ namespace llamql
         const int wid_all = (int)blockIdx.x * (int)(blockDim.x >> 6) + wave;
         int p, w_first;
         quad_which(qa, wid_all, p, w_first);
-        quad_body<Q, M, U, SRC, DUMP>(qa, quad_lds, p, w_first, wid_all);
+        quad_body<Q, M, U, SRC, MODE>(qa, quad_lds, p, w_first, wid_all);
     }
 
     // Two formats in one launch (Q and K in Q4_K, V in Q6_K): whole workgroups belong to one
     // format, so the branch is uniform per workgroup.
-    template <class QA, int UA, class QB, int UB, int M, int SRC>
+    template <class QA, int UA, class QB, int UB, int M, int SRC, int MODE = QUAD_MODE_PLAIN>
     __global__ void __launch_bounds__(QA::max_threads(M) < QB::max_threads(M) ? QA::max_threads(M) : QB::max_threads(M))
         gemv_quad_dual_kernel(const QuadArgs qa)
     {
@@ -826,17 +892,17 @@ namespace llamql
         int p, w_first;
         quad_which(qa, wid_all, p, w_first);
         if (p < qa.first_b)
-            quad_body<QA, M, UA, SRC>(qa, quad_lds, p, w_first, wid_all);
+            quad_body<QA, M, UA, SRC, MODE>(qa, quad_lds, p, w_first, wid_all);
         else
-            quad_body<QB, M, UB, SRC>(qa, quad_lds, p, w_first, wid_all);
+            quad_body<QB, M, UB, SRC, MODE>(qa, quad_lds, p, w_first, wid_all);
     }
 
-    template <class Q, int M, int U, int SRC, bool DUMP = false>
+    template <class Q, int M, int U, int SRC, int MODE = QUAD_MODE_PLAIN>
     inline void gemv_quad_launch_mus(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         static LdsGrant grant;
-        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC, DUMP>), QUAD_MAX_LDS);
-        hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U, SRC, DUMP>), grid, block, lds, st, a);
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC, MODE>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U, SRC, MODE>), grid, block, lds, st, a);
     }
 
     // a.sums set: the block-sum variant of the same kernel (Q8_1 input only)
@@ -845,8 +911,21 @@ namespace llamql
     {
         if (a.sums)
         {
-            gemv_quad_launch_mus<Q, M, U, QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            gemv_quad_launch_mus<Q, M, U, QUAD_SRC_Q8, QUAD_MODE_DUMP>(grid, block, lds, st, a);
             return;
+        }
+        if constexpr (M == 1)
+        {
+            if (a.ring)
+            {
+                switch (src)
+                {
+                case QUAD_SRC_F32: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_F32, QUAD_MODE_RING>(grid, block, lds, st, a); break;
+                case QUAD_SRC_SWIGLU: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_SWIGLU, QUAD_MODE_RING>(grid, block, lds, st, a); break;
+                default: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_Q8, QUAD_MODE_RING>(grid, block, lds, st, a); break;
+                }
+                return;
+            }
         }
         switch (src)
         {
@@ -856,13 +935,24 @@ namespace llamql
         }
     }
 
+    // Steps per load chunk (two chunks are in flight).  Measured on 5120..25600-column matrices:
+    // a single activation row is fastest with ONE step per chunk (4.6 KB in flight per wavefront;
+    // deeper queues only lengthen the memory system's own queues) unless rows are long (64
+    // super-blocks and more), where a wavefront holds few rows and two steps pay.
+    constexpr int QUAD_LONG_ROW_SB = 64;
+
     template <class Q>
     inline void gemv_quad_launch(int M, int src, dim3 grid, dim3 block, size_t lds, hipStream_t st,
                                  const QuadArgs &a)
     {
         switch (M)
         {
-        case 1: gemv_quad_launch_mu<Q, 1, 2>(src, grid, block, lds, st, a); break;
+        case 1:
+            if (a.SB >= QUAD_LONG_ROW_SB)
+                gemv_quad_launch_mu<Q, 1, 2>(src, grid, block, lds, st, a);
+            else
+                gemv_quad_launch_mu<Q, 1, 1>(src, grid, block, lds, st, a);
+            break;
         case 2: gemv_quad_launch_mu<Q, 2, 2>(src, grid, block, lds, st, a); break;
         case 3: gemv_quad_launch_mu<Q, 3, 2>(src, grid, block, lds, st, a); break;
         case 4: gemv_quad_launch_mu<Q, 4, 2>(src, grid, block, lds, st, a); break;
@@ -878,12 +968,23 @@ namespace llamql
     template <class Q>
     constexpr int quad_unroll(int M)
     {
-        return M <= 4 ? 2 : (Q::LOADS <= 3 ? 2 : 1);
+        return M == 1 ? 1 : M <= 4 ? 2 : (Q::LOADS <= 3 ? 2 : 1);
     }
 
     template <class QA, class QB, int M, int SRC>
     inline void gemv_quad_dual_launch_ms(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
+        if constexpr (M == 1)
+        {
+            if (a.ring)
+            {
+                auto kernel = &gemv_quad_dual_kernel<QA, quad_unroll<QA>(M), QB, quad_unroll<QB>(M), M, SRC, QUAD_MODE_RING>;
+                static LdsGrant grant;
+                (void)allow_lds(grant, reinterpret_cast<const void *>(kernel), QUAD_MAX_LDS);
+                hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+                return;
+            }
+        }
         auto kernel = &gemv_quad_dual_kernel<QA, quad_unroll<QA>(M), QB, quad_unroll<QB>(M), M, SRC>;
         static LdsGrant grant;
         (void)allow_lds(grant, reinterpret_cast<const void *>(kernel), QUAD_MAX_LDS);
