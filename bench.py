@@ -123,11 +123,31 @@ def bench_moe(args, torch, capi, synth, dev):
                      "ids": torch.full((T, TOPK + 1), E, dtype=torch.int32, device=dev),
                      "w": torch.ones(T, TOPK + 1, device=dev)})
 
+    # Batches sort the (token, slot) pairs by expert on the device and read every distinct
+    # expert's matrices once (6 launches); a single token has nothing to group (4 launches).
+    # (measured: per-slot launches 100 us at 16 tokens against 104 grouped; 172 against 153 at 32; 316 against 217 at 64)
+    path = args.moe_path if args.moe_path != "auto" else ("grouped" if T >= 32 else "slots")
+    S = TOPK + 1
+    for s_ in sets:
+        s_["group"] = torch.empty(int(capi.load().llam_ql_moe_group_bytes(T, S)), dtype=torch.uint8, device=dev)
+        s_["gate"] = torch.empty(T * S, I, device=dev)
+        s_["up"] = torch.empty(T * S, I, device=dev)
+        s_["pair_out"] = torch.empty(T * S, H, device=dev)
+
     def step(s):
         capi.moe_route_quantize(s["logits"], TOPK, s["x"], s["q8"], ids=s["ids"], weights=s["w"])
-        gate, up = capi.moe_gate_up(fmt, table, E + 1, s["ids"], s["q8"], T, TOPK + 1, H, I)
+        if path == "slots":
+            gate, up = capi.moe_gate_up(fmt, table, E + 1, s["ids"], s["q8"], T, S, H, I)
+        else:
+            capi.moe_group(s["ids"], E + 1, group=s["group"])
+            gate, up = capi.moe_gate_up_grouped(fmt, table, E + 1, s["group"], s["q8"], T, S, H, I, gate=s["gate"],
+                                                up=s["up"])
         qa = capi.swiglu_quantize(gate, up)
-        capi.moe_down(fmt, table, E + 1, s["ids"], s["w"], qa, s["out"], T, TOPK + 1, H, I, accumulate=False)
+        if path == "grouped":
+            capi.moe_down_grouped(fmt, table, E + 1, s["group"], s["ids"], s["w"], qa, s["pair_out"], s["out"], T, S,
+                                  H, I)
+        else:
+            capi.moe_down(fmt, table, E + 1, s["ids"], s["w"], qa, s["out"], T, S, H, I, accumulate=False)
 
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -141,18 +161,26 @@ def bench_moe(args, torch, capi, synth, dev):
         reps = max(1, (args.steps + nsets - 1) // nsets)
         us = _time_launches(torch, stream, lambda i: gr.replay(), reps, 2) / nsets
         distinct = len(set(int(v) for s_ in sets for v in s_["ids"][:, :TOPK].flatten().tolist()))
+        per_set = [len(set(int(v) for v in s_["ids"].flatten().tolist())) for s_ in sets]
     blk = 112  # device bytes per IQ3_S super-block
-    w_bytes = (TOPK + 1) * T * 3 * I * (H // 256) * blk  # every token slot streams its expert's three matrices
+    per_expert = 3 * I * (H // 256) * blk
+    slot_bytes = S * T * per_expert                       # every token slot streams its expert's matrices
+    distinct_bytes = sum(per_set) / nsets * per_expert    # every distinct expert of a step once (incl. the shared one)
+    # algorithmic bytes: the distinct experts a step touches (a single token touches S of them)
+    w_bytes = distinct_bytes
     value = w_bytes / (us * 1e-6) / 1e9
+    launches = {"slots": 4, "grouped-gate-up": 5, "grouped": 6}[path]
     return _common(args, "MoE expert FFN decode effective GB/s", round(value, 1), "GB/s", round(us * 1e-3, 5), "int8",
                    {"workload": "MoE expert FFN decode: hidden 2048, 256 routed experts + 1 shared, top-8, expert "
                                 "intermediate 512, IQ3_S, %d token(s); route, quantise, gate/up, SwiGLU + quantise, down; shared expert in a ninth slot" % T,
-                    "tokens": T, "weight_bytes_per_step": w_bytes, "tokens_per_s": round(T / (us * 1e-6), 1),
+                    "tokens": T, "weight_bytes_per_step": round(w_bytes), "slot_bytes_per_step": slot_bytes,
+                    "distinct_experts_per_step": round(sum(per_set) / nsets, 1),
+                    "tokens_per_s": round(T / (us * 1e-6), 1), "path": path,
                     "token_sets_rotated": nsets, "distinct_routed_experts_over_sets": distinct,
                     "launch": "hip-graph replay of all token sets' steps"},
-                   {"kernel": "moe step (4 launches)", "bound": "hbm", "achieved": round(value, 1),
+                   {"kernel": "moe step (%d launches)" % launches, "bound": "hbm", "achieved": round(value, 1),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None,
-                    "bytes_per_launch": w_bytes, "us_per_launch": round(us, 2), "launches_timed": args.steps})
+                    "bytes_per_launch": round(w_bytes), "us_per_launch": round(us, 2), "launches_timed": args.steps})
 
 
 def bench_gemv(args, torch, capi, synth, dev):
@@ -304,6 +332,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--moe-path", choices=["auto", "slots", "grouped-gate-up", "grouped"], default="auto",
+                    help="moe workload: per-slot launches, or tokens grouped by expert (gate/up only, or down as well)")
     ap.add_argument("--workload", choices=["layer", "gemm", "moe", "gemv", "decode"], default="layer",
                     help="layer: the headline decode-layer step (default); gemm: prefill int8 GEMM 512x25600x5120 Q4_K; "
                          "moe: 256-expert top-8 IQ3_S expert FFN decode; gemv: single GEMVs of every format and layer shape")

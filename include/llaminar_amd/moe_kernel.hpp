@@ -35,6 +35,14 @@ namespace llaminar_amd
         int stride() const { return slot_stride ? slot_stride : top_k; }
     };
 
+    // Host-side routing result (reference: MoERoutingResult, src/v2/kernels/IMoEKernel.h:37-42).
+    struct MoERoutingResult
+    {
+        std::vector<int> expert_indices;   // [seq_len * top_k]
+        std::vector<float> expert_weights; // [seq_len * top_k]
+        std::vector<float> router_logits;  // [seq_len * num_experts] probabilities after the softmax
+    };
+
     // Reason of the calling thread's last failed MI355MoEKernel call.
     const char *moe_kernel_last_error();
 
@@ -74,6 +82,34 @@ namespace llaminar_amd
                                const DeviceTensor *gate_weights, int d_model, int num_experts, int top_k,
                                bool normalize_weights);
 
+        // IMoEKernel::route (IMoEKernel.h:84-90): the same routing with the result on the host.
+        // hidden and gate_weights are device pointers; the call waits for the stream (the result
+        // is host memory by its interface).
+        bool route(const float *hidden, const float *gate_weights, int seq_len, int d_model, int num_experts,
+                   int top_k, bool normalize_weights, MoERoutingResult &result);
+        // IMoEKernel::weightedAdd (IMoEKernel.h:189-195): output[i] += weight * input[i], device buffers.
+        bool weightedAdd(float *output, const float *input, float weight, int count);
+
+        // ---- single-token grouped projections from host or fp32 device routing ------------------
+        // (IMoEKernel.h:452-575)  FromTable: expert_ids / expert_weights are HOST arrays of the
+        // num_active slots, uploaded as per-call metadata.  FromRouting: routing_indices /
+        // routing_weights are DEVICE tensors of top_k fp32 values.  gate_outputs / up_outputs:
+        // one contiguous [slots x intermediate] device buffer; output [1 x d_model], overwritten.
+        bool groupedExpertGateUpDecodeFromTable(const DeviceTensor *input, const int *expert_ids,
+                                                int descriptor_table_id, int num_active, float *gate_outputs,
+                                                float *up_outputs, int d_model, int intermediate);
+        bool groupedExpertGateUpDecodeFromRouting(const DeviceTensor *input, const float *routing_indices,
+                                                  int descriptor_table_id, int top_k, float *gate_outputs,
+                                                  float *up_outputs, int d_model, int intermediate);
+        bool groupedExpertDownDecodeFromTable(const float *gate_tensors, const float *up_tensors,
+                                              const int *expert_ids, const float *expert_weights,
+                                              int descriptor_table_id, int num_active, DeviceTensor *output,
+                                              int d_model, int intermediate);
+        bool groupedExpertDownDecodeFromRouting(const float *gate_tensors, const float *up_tensors,
+                                                const float *routing_indices, const float *routing_weights,
+                                                int descriptor_table_id, int top_k, DeviceTensor *output, int d_model,
+                                                int intermediate);
+
         // ---- grouped projections (IMoEKernel.h:508-620) ------------------------------------------
         // input [n_tokens x d_model] fp32; gate_outputs / up_outputs [n_tokens*slots x intermediate].
         bool groupedExpertGateUpDecodeFromRuntime(DeviceMoELayerRuntime *runtime_layer, const DeviceTensor *input,
@@ -106,6 +142,11 @@ namespace llaminar_amd
         const Table *table(const char *fn, int id, bool want_down, int d_model, int intermediate) const;
         int add_table(const char *fn, const DeviceQuantMatrixDesc *a, const DeviceQuantMatrixDesc *b,
                       const DeviceQuantMatrixDesc *c, int num_experts, int d_model, int intermediate);
+        bool gate_up_ids(const char *fn, const DeviceTensor *input, const int32_t *d_ids, uint8_t *scratch_after_ids,
+                         size_t scratch_left, const Table *t, int slots, float *gate_outputs, float *up_outputs);
+        bool down_ids(const char *fn, const float *gate_tensors, const float *up_tensors, const int32_t *d_ids,
+                      const float *d_weights, uint8_t *scratch, size_t scratch_left, const Table *t, int slots,
+                      DeviceTensor *output);
         struct Scratch
         {
             uint8_t *p = nullptr;

@@ -280,7 +280,7 @@ bool llam_ql_swiglu_quantize(const float *d_gate, const float *d_up,
 /* Down GEMVs and weighted accumulation:
  *   d_out[t*hidden + h] (+)= sum_s d_weights[t*top_k+s] * (W_down[e_s][h,:] . q8_act[t,s])
  * Slots are added in ascending s; accumulate != 0 adds onto d_out, else
- * overwrites.  Replaces multiply_fused_expert_down + vec_axpy
+ * overwrites (a token all of whose slots are skipped gets zeros).  Replaces multiply_fused_expert_down + vec_axpy
  * (MoEExpertComputeStage.cpp:1664-1673); counterpart of
  * groupedExpertDownDecode* (IMoEKernel.h:378-643). */
 bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts,
@@ -288,6 +288,45 @@ bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts,
                       const void *d_q8_act, float *d_out, int n_tokens,
                       int top_k, int hidden, int inter, int accumulate,
                       int device_id, void *stream);
+
+/* ---- batches: tokens grouped by expert ---------------------------------------------------
+ * With several tokens the same expert is usually picked more than once (16 tokens x 8 slots
+ * of 256 experts hit about 100 distinct ones, and an always-on shared expert serves all 16).
+ * llam_ql_moe_group sorts the (token, slot) pairs by expert id on the device (stable; ids
+ * outside [0, n_experts) are left out) into a caller-provided workspace of
+ * llam_ql_moe_group_bytes(); the _grouped launches then read every distinct expert's matrices
+ * once per chunk of two of its tokens (four from 512 pairs on).  Outputs are the bits of the
+ * ungrouped launches.  At most 4096 pairs per call.  Replaces the per-expert bucketing of
+ * MoEExpertComputeStage::execute (MoEExpertComputeStage.cpp:884-979: gatherTokenBatch,
+ * multiply_fused_tensor with m = tokens of the expert, scatterAddWeighted); device counterpart
+ * IMoEKernel::groupTokensByExpertDevice (src/v2/kernels/IMoEKernel.h:737) and
+ * moe_grouped_prefill (src/v2/kernels/rocm/gemm/ROCmMoEGroupedPrefillKernels.hip:1465).
+ * d_ids [n_tokens x slot_stride] as written by llam_ql_moe_route_ex (every column is a slot). */
+size_t llam_ql_moe_group_bytes(int n_tokens, int slot_stride);
+bool llam_ql_moe_group(const int32_t *d_ids, int n_tokens, int slot_stride, int n_experts,
+                       void *d_group, int device_id, void *stream);
+/* llam_ql_moe_gate_up over the grouped pairs: same outputs, same layout
+ * (d_gate_out[(t*slot_stride+s)*inter + i]). */
+bool llam_ql_moe_gate_up_grouped(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                                 const void *d_group, const void *d_q8, float *d_gate_out,
+                                 float *d_up_out, int n_tokens, int slot_stride, int hidden,
+                                 int inter, int device_id, void *stream);
+/* llam_ql_moe_down over the grouped pairs: the down products of every pair go to
+ * d_pair_out [n_tokens*slot_stride x hidden] (scratch), then a token's live slots are added
+ * in ascending order with their routing weights -- the order and arithmetic of
+ * llam_ql_moe_down, the same bits.  A token without a live slot gets zeros when
+ * accumulate == 0. */
+bool llam_ql_moe_down_grouped(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                              const void *d_group, const int32_t *d_ids, const float *d_weights,
+                              const void *d_q8_act, float *d_pair_out, float *d_out, int n_tokens,
+                              int slot_stride, int hidden, int inter, int accumulate,
+                              int device_id, void *stream);
+
+/* Expert ids from a device tensor that holds them as fp32 values (the reference's routing_indices
+ * tensors of groupedExpert*DecodeFromRouting, src/v2/kernels/IMoEKernel.h:480-575): truncation
+ * toward zero; NaN, negative and out-of-range values become -1, which every launch skips. */
+bool llam_ql_moe_ids_from_f32(const float *d_indices, int32_t *d_ids, int n, int device_id,
+                              void *stream);
 
 /* Shared expert: d_out[t,:] += g_t * d_shared[t,:] with
  * g_t = sigmoid(dot(d_gate_inp, d_hidden[t,:])), or g_t = 1 when d_gate_inp is

@@ -79,6 +79,13 @@ SIGNATURES = {
     "llam_ql_swiglu_quantize": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                   c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_group_bytes": (c_size_t, [c_int, c_int]),
+    "llam_ql_moe_group": (c_bool, [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
+    "llam_ql_moe_gate_up_grouped": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                             c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_down_grouped": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_ids_from_f32": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "llam_ql_shared_expert_add": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     # decode_api.h
     "llam_dec_embed_q4k": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
@@ -379,6 +386,38 @@ def moe_down(fmt: int, table, n_experts: int, ids, weights, q8_act, out, n_token
     _check(load().llam_ql_moe_down(fmt, _ptr(table), n_experts, _ptr(ids), _ptr(weights), _ptr(q8_act), _ptr(out),
                                    n_tokens, top_k, hidden, inter, int(accumulate), _dev(out), _stream(stream)),
            "moe_down")
+    return out
+
+
+def moe_group(ids, n_experts: int, group=None, stream=None):
+    """Sort the (token, slot) pairs of ids [T, S] by expert on the device -> workspace tensor."""
+    import torch
+
+    T, S = ids.shape
+    if group is None:
+        group = torch.empty(int(load().llam_ql_moe_group_bytes(T, S)), dtype=torch.uint8, device=ids.device)
+    _check(load().llam_ql_moe_group(_ptr(ids), T, S, n_experts, _ptr(group), _dev(ids), _stream(stream)), "moe_group")
+    return group
+
+
+def moe_gate_up_grouped(fmt: int, table, n_experts: int, group, q8, n_tokens: int, slots: int, hidden: int, inter: int,
+                        gate=None, up=None, stream=None):
+    import torch
+
+    if gate is None:
+        gate = torch.empty(n_tokens * slots, inter, dtype=torch.float32, device=q8.device)
+        up = torch.empty_like(gate)
+    _check(load().llam_ql_moe_gate_up_grouped(fmt, _ptr(table), n_experts, _ptr(group), _ptr(q8), _ptr(gate), _ptr(up),
+                                              n_tokens, slots, hidden, inter, _dev(q8), _stream(stream)),
+           "moe_gate_up_grouped")
+    return gate, up
+
+
+def moe_down_grouped(fmt: int, table, n_experts: int, group, ids, weights, q8_act, pair_out, out, n_tokens: int,
+                     slots: int, hidden: int, inter: int, accumulate: bool = False, stream=None):
+    _check(load().llam_ql_moe_down_grouped(fmt, _ptr(table), n_experts, _ptr(group), _ptr(ids), _ptr(weights),
+                                           _ptr(q8_act), _ptr(pair_out), _ptr(out), n_tokens, slots, hidden, inter,
+                                           int(accumulate), _dev(out), _stream(stream)), "moe_down_grouped")
     return out
 
 

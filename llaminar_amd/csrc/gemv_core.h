@@ -53,18 +53,24 @@ namespace llamql
         int accumulate;     // add onto y instead of overwriting
         float out_scale;    // y (+)= out_scale * (row dot); 1 for plain GEMV
         int row0, nrows;    // DUMP only: rows [row0,row0+nrows) of the matrix
+        // Optional gather of the batch rows (MoE token groups): batch row m takes the activation
+        // row pairs[m] / pair_div of q8 and writes output row pairs[m] of y.  Null: row m both.
+        const int32_t *pairs;
+        int pair_div;
     };
 
     // Stage `nkb` Q8_1 blocks of each of M activation rows into LDS.
     template <class F, int M>
     __device__ __forceinline__ void stage_q8(const uint32_t *__restrict__ q8, int KB_total, int kb0, int nkb,
-                                             uint32_t *aq, float *ad, float *asd)
+                                             uint32_t *aq, float *ad, float *asd, const int32_t *pairs = nullptr,
+                                             int pair_div = 1)
     {
         const int ndw = nkb * 9;
         constexpr int U = 8; // loads in flight per thread
         for (int m = 0; m < M; ++m)
         {
-            const uint32_t *src = q8 + ((size_t)m * KB_total + kb0) * 9;
+            const size_t arow = pairs ? (size_t)(pairs[m] / pair_div) : (size_t)m;
+            const uint32_t *src = q8 + (arow * KB_total + kb0) * 9;
             for (int base = 0; base < ndw; base += U * (int)blockDim.x)
             {
                 uint32_t v[U];
@@ -171,7 +177,7 @@ namespace llamql
 
         if (F::TABLE_BYTES > 0)
             F::stage_tables(tab);
-        stage_q8<F, M>(a.q8, a.SB * 8, a.sb0 * 8, nkb, aq, ad, asd);
+        stage_q8<F, M>(a.q8, a.SB * 8, a.sb0 * 8, nkb, aq, ad, asd, a.pairs, a.pair_div);
         __syncthreads();
 
         for (int r = 0; r < a.rows_per_wave; ++r)
@@ -263,7 +269,8 @@ namespace llamql
                     const float total = segment_sum(acc[m], a.gshift);
                     if (row_ok && (lane & (8 * G - 1)) == 0)
                     {
-                        float *dst = a.y + (size_t)m * a.ldy + row;
+                        const size_t orow = a.pairs ? (size_t)a.pairs[m] : (size_t)m;
+                        float *dst = a.y + orow * a.ldy + row;
                         const float v = a.out_scale * total;
                         *dst = a.accumulate ? (*dst + v) : v;
                     }

@@ -776,6 +776,8 @@ namespace llamql
             a.out_scale = 1.0f;
             a.row0 = row0;
             a.nrows = nrows;
+            a.pairs = nullptr;
+            a.pair_div = 1;
             const size_t lds = gemv_lds_bytes<F>(M, a.nsb);
             if (p.kernel == GEMV_KERNEL_CHUNKED)
                 gemv_fast_launch<F>(M, p.unroll, dim3((unsigned)p.grid), lds, st, a);

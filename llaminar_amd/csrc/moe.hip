@@ -209,6 +209,8 @@ namespace llamql
         a.out_scale = 1.0f;
         a.row0 = 0;
         a.nrows = 0;
+        a.pairs = nullptr;
+        a.pair_div = 1;
         gemv_body<F, 1, 1, false>(a, (long)blockIdx.x, lds);
     }
 
@@ -243,9 +245,20 @@ namespace llamql
             a.out_scale = m.weights[slot];
             a.row0 = 0;
             a.nrows = 0;
+            a.pairs = nullptr;
+            a.pair_div = 1;
             gemv_body<F, 1, 1, false>(a, (long)blockIdx.x, lds);
             first = false;
             __syncthreads(); // LDS is restaged by the next slot
+        }
+        if (first)
+        {
+            // accumulate == 0 and no live slot: the token's output is zero, not what the buffer held
+            const int gsh = m.gshift;
+            const int rows_per_wg = GEMV_WAVES * (8 >> gsh) * m.rows_per_wave;
+            const long r0 = (long)blockIdx.x * rows_per_wg;
+            for (long r = r0 + threadIdx.x; r < r0 + rows_per_wg && r < m.hidden; r += blockDim.x)
+                m.out0[(size_t)t * m.hidden + r] = 0.0f;
         }
     }
 
@@ -378,12 +391,298 @@ namespace llamql
                 else
                     y = y + v;
             }
-            if (row < m.hidden && (lane & (8 * G - 1)) == 0 && !(first && m.accumulate == 0))
+            // (a token without a live slot: y is 0, which overwrites when accumulate == 0)
+            if (row < m.hidden && (lane & (8 * G - 1)) == 0)
             {
                 float *dst = m.out0 + (size_t)t * m.hidden + row;
                 *dst = m.accumulate ? (*dst + y) : y;
             }
         }
+    }
+
+
+    // ---- token grouping by expert ---------------------------------------------------------
+    // Batches: the (token, slot) pairs sorted by expert id, so that the grouped launches read
+    // every distinct expert's matrices once per chunk of four of its tokens
+    // (MoEExpertComputeStage::execute buckets the same way on the host,
+    // src/v2/execution/compute_stages/stages/MoEExpertComputeStage.cpp:884-979; device
+    // counterpart IMoEKernel::groupTokensByExpertDevice, src/v2/kernels/IMoEKernel.h:737).
+    // Workspace, int32, P = n_tokens * slot_stride:
+    //   [0] segments  [1] valid pairs  [2] chunks  [3] pairs per chunk
+    //   seg_expert[P]  seg_begin[P+1]  pair_sorted[P]  chunk_expert[P]  chunk_begin[P]  chunk_count[P]
+    // A segment is the run of one expert's pairs in pair_sorted (stable: ascending pair index);
+    // a chunk is up to moe_chunk_size(P) consecutive pairs of a segment, the unit of work of the grouped
+    // launches.  Pairs with an id outside [0, n_experts) are left out.
+    constexpr int MOE_GROUP_THREADS = 1024;
+    constexpr int MOE_GROUP_MAX_PAIRS = 4096;
+    constexpr int MOE_GROUP_MAX_EXPERTS = 2 * MOE_GROUP_THREADS; // two experts per thread
+    // Tokens of one expert that share a workgroup's pass over its matrix.  Measured on the
+    // 256-expert IQ3_S shape: four pay from about 500 pairs on (64 tokens: 217 against 247 us
+    // per step); below that the larger register footprint of the four-row body costs more than
+    // the second read of the few experts with more than two tokens saves (16 tokens: 107
+    // against 104 us).
+    constexpr int MOE_CHUNK_MAX = 4;
+    __host__ __device__ inline int moe_chunk_size(int P) { return P >= 512 ? 4 : 2; }
+    struct MoEGroupView
+    {
+        int32_t *head, *seg_expert, *seg_begin, *pair_sorted, *chunk_expert, *chunk_begin, *chunk_count;
+    };
+    __host__ __device__ inline MoEGroupView moe_group_view(void *ws, int P)
+    {
+        int32_t *w = static_cast<int32_t *>(ws);
+        MoEGroupView g;
+        g.head = w;
+        g.seg_expert = w + 4;
+        g.seg_begin = g.seg_expert + P;
+        g.pair_sorted = g.seg_begin + (P + 1);
+        g.chunk_expert = g.pair_sorted + P;
+        g.chunk_begin = g.chunk_expert + P;
+        g.chunk_count = g.chunk_begin + P;
+        return g;
+    }
+    __host__ __device__ inline size_t moe_group_bytes(int P) { return ((size_t)(4 + 6 * (size_t)P + 1) * 4 + 15) & ~(size_t)15; }
+
+    // exclusive sums of three counters over the workgroup's threads, and the totals
+    struct Int3
+    {
+        int a, b, c;
+    };
+    __device__ __forceinline__ Int3 block_exclusive_scan3(Int3 v, Int3 &total, int (*wave_sums)[3])
+    {
+        const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+        Int3 inc = v;
+#pragma unroll
+        for (int off = 1; off < WAVE; off <<= 1)
+        {
+            const int a = __shfl_up(inc.a, off), b = __shfl_up(inc.b, off), c = __shfl_up(inc.c, off);
+            if (lane >= off)
+            {
+                inc.a += a;
+                inc.b += b;
+                inc.c += c;
+            }
+        }
+        if (lane == WAVE - 1)
+        {
+            wave_sums[wave][0] = inc.a;
+            wave_sums[wave][1] = inc.b;
+            wave_sums[wave][2] = inc.c;
+        }
+        __syncthreads();
+        Int3 base{0, 0, 0};
+        total = Int3{0, 0, 0};
+        for (int w = 0; w < nwaves; ++w)
+        {
+            if (w < wave)
+            {
+                base.a += wave_sums[w][0];
+                base.b += wave_sums[w][1];
+                base.c += wave_sums[w][2];
+            }
+            total.a += wave_sums[w][0];
+            total.b += wave_sums[w][1];
+            total.c += wave_sums[w][2];
+        }
+        return Int3{base.a + inc.a - v.a, base.b + inc.b - v.b, base.c + inc.c - v.c};
+    }
+
+    __global__ void __launch_bounds__(MOE_GROUP_THREADS)
+        moe_group_kernel(const int32_t *__restrict__ ids, int P, int n_experts, void *ws)
+    {
+        extern __shared__ int32_t grp_se[]; // expert of every pair (INT_MAX: left out), padded to a multiple of 4
+        __shared__ int hist[MOE_GROUP_MAX_EXPERTS];
+        __shared__ int wave_sums[MOE_GROUP_THREADS / WAVE][3];
+        const MoEGroupView g = moe_group_view(ws, P);
+        const int tid = threadIdx.x;
+        for (int e = tid; e < MOE_GROUP_MAX_EXPERTS; e += blockDim.x)
+            hist[e] = 0;
+        __syncthreads();
+        const int P4 = (P + 3) & ~3;
+        for (int p = tid; p < P4; p += blockDim.x)
+        {
+            const int e = p < P ? ids[p] : -1;
+            const bool ok = e >= 0 && e < n_experts;
+            grp_se[p] = ok ? e : 0x7FFFFFFF;
+            if (ok)
+                atomicAdd(&hist[e], 1); // integer: the counts do not depend on the order
+        }
+        __syncthreads();
+        // thread i owns experts 2i and 2i+1: pairs, non-empty experts and chunks before them
+        const int c0 = hist[2 * tid], c1 = hist[2 * tid + 1];
+        const int MOE_CHUNK = moe_chunk_size(P);
+        const int k0 = (c0 + MOE_CHUNK - 1) / MOE_CHUNK, k1 = (c1 + MOE_CHUNK - 1) / MOE_CHUNK;
+        Int3 total;
+        const Int3 ex = block_exclusive_scan3(Int3{c0 + c1, (c0 > 0) + (c1 > 0), k0 + k1}, total, wave_sums);
+        __syncthreads(); // everybody has read its counts: hist becomes the experts' offsets
+        hist[2 * tid] = ex.a;
+        hist[2 * tid + 1] = ex.a + c0;
+        auto emit = [&](int e, int cnt, int seg, int begin, int chunk) {
+            g.seg_expert[seg] = e;
+            g.seg_begin[seg] = begin;
+            for (int j = 0; j * MOE_CHUNK < cnt; ++j)
+            {
+                g.chunk_expert[chunk + j] = e;
+                g.chunk_begin[chunk + j] = begin + j * MOE_CHUNK;
+                g.chunk_count[chunk + j] = cnt - j * MOE_CHUNK < MOE_CHUNK ? cnt - j * MOE_CHUNK : MOE_CHUNK;
+            }
+        };
+        if (c0 > 0)
+            emit(2 * tid, c0, ex.b, ex.a, ex.c);
+        if (c1 > 0)
+            emit(2 * tid + 1, c1, ex.b + (c0 > 0), ex.a + c0, ex.c + k0);
+        if (tid == 0)
+        {
+            g.head[0] = total.b;
+            g.head[1] = total.a;
+            g.head[2] = total.c;
+            g.head[3] = MOE_CHUNK;
+            g.seg_begin[total.b] = total.a;
+        }
+        __syncthreads();
+        // stable place of every pair: its expert's offset plus the earlier pairs of that expert
+        for (int p = tid; p < P; p += blockDim.x)
+        {
+            const int e = grp_se[p];
+            if (e == 0x7FFFFFFF)
+                continue;
+            int same = 0;
+            const int4 *v = reinterpret_cast<const int4 *>(grp_se);
+            const int full = p >> 2;
+            for (int q = 0; q < full; ++q)
+            {
+                const int4 x = v[q];
+                same += (x.x == e) + (x.y == e) + (x.z == e) + (x.w == e);
+            }
+            for (int q = full * 4; q < p; ++q)
+                same += grp_se[q] == e;
+            g.pair_sorted[hist[e] + same] = p;
+        }
+    }
+
+    // One chunk of the grouped launches: the expert's matrix (gate, up or down) against the
+    // chunk's 1..MOE_CHUNK tokens, through the generic GEMV body with its batch rows gathered
+    // through the sorted pair list.  Every output row carries the bits of the ungrouped launch:
+    // a batch row's arithmetic does not depend on the batch it rides in.
+    template <class F, int MAXM>
+    __device__ __forceinline__ void moe_chunk_body(GemvArgs &a, const MoEGroupView &g, int chunk, uint32_t *lds)
+    {
+        a.pairs = g.pair_sorted + g.chunk_begin[chunk];
+        const int n = g.chunk_count[chunk]; // uniform
+        if constexpr (MAXM >= 4)
+        {
+            if (n == 4)
+            {
+                gemv_body<F, 4, 1, false>(a, (long)blockIdx.x, lds);
+                return;
+            }
+            if (n == 3)
+            {
+                gemv_body<F, 3, 1, false>(a, (long)blockIdx.x, lds);
+                return;
+            }
+        }
+        if (n == 2)
+            gemv_body<F, 2, 1, false>(a, (long)blockIdx.x, lds);
+        else
+            gemv_body<F, 1, 1, false>(a, (long)blockIdx.x, lds);
+    }
+
+    // grid: (workgroups per matrix, chunks (upper bound), 2 = gate|up)
+    template <class F, int MAXM>
+    __global__ void __launch_bounds__(GEMV_WAVES *WAVE) moe_gate_up_grouped_kernel(const MoEArgs m, void *ws, int P)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+        const MoEGroupView g = moe_group_view(ws, P);
+        const int chunk = blockIdx.y;
+        if (chunk >= g.head[2])
+            return; // uniform
+        const int e = g.chunk_expert[chunk];
+        GemvArgs a;
+        a.w = blockIdx.z == 0 ? m.experts[e].d_gate : m.experts[e].d_up;
+        if (!a.w)
+            return; // an expert whose matrices live elsewhere (uniform)
+        a.q8 = m.q8;
+        a.y = blockIdx.z == 0 ? m.out0 : m.out1;
+        a.sums = nullptr;
+        a.ldy = m.inter;
+        a.N = m.inter;
+        a.SB = m.hidden / 256;
+        a.sb0 = 0;
+        a.nsb = a.SB;
+        a.rows_per_wave = m.rows_per_wave;
+        a.gshift = m.gshift;
+        a.accumulate = 0;
+        a.out_scale = 1.0f;
+        a.row0 = 0;
+        a.nrows = 0;
+        a.pair_div = m.top_k; // pair = token * slot_stride + slot
+        moe_chunk_body<F, MAXM>(a, g, chunk, lds);
+    }
+
+    // Down projection of one chunk into per-pair rows: pair_out[pair][:] = W_down[e] . act[pair]
+    // (unweighted; moe_pair_reduce_kernel adds a token's slots).  grid: (workgroups per matrix, chunks)
+    template <class F, int MAXM>
+    __global__ void __launch_bounds__(GEMV_WAVES *WAVE) moe_down_grouped_kernel(const MoEArgs m, void *ws, int P)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+        const MoEGroupView g = moe_group_view(ws, P);
+        const int chunk = blockIdx.y;
+        if (chunk >= g.head[2])
+            return;
+        const int e = g.chunk_expert[chunk];
+        GemvArgs a;
+        a.w = m.experts[e].d_down;
+        if (!a.w)
+            return;
+        a.q8 = m.q8;  // Q8_1 activations, one row per pair
+        a.y = m.out1; // [P x hidden]
+        a.sums = nullptr;
+        a.ldy = m.hidden;
+        a.N = m.hidden;
+        a.SB = m.inter / 256;
+        a.sb0 = 0;
+        a.nsb = a.SB;
+        a.rows_per_wave = m.rows_per_wave;
+        a.gshift = m.gshift;
+        a.accumulate = 0;
+        a.out_scale = 1.0f;
+        a.row0 = 0;
+        a.nrows = 0;
+        a.pair_div = 1;
+        moe_chunk_body<F, MAXM>(a, g, chunk, lds);
+    }
+
+    // out[t][h] (+)= sum over the token's live slots, ascending, of weight * pair_out[pair][h]:
+    // the arithmetic and order of moe_down_kernel, so the same bits.  A token without a live
+    // slot gets zeros when accumulate == 0.
+    __global__ void __launch_bounds__(256)
+        moe_pair_reduce_kernel(const float *__restrict__ pair_out, const int32_t *__restrict__ ids,
+                               const float *__restrict__ weights, const llam_ql_expert *__restrict__ experts,
+                               int n_experts, float *__restrict__ out, int slots, int hidden, int accumulate)
+    {
+        const int t = blockIdx.y;
+        const int h = blockIdx.x * blockDim.x + threadIdx.x;
+        if (h >= hidden)
+            return;
+        float y = 0.0f;
+        bool first = accumulate == 0;
+        for (int s = 0; s < slots; ++s)
+        {
+            const int pair = t * slots + s;
+            const int e = ids[pair];
+            if (e < 0 || e >= n_experts || !experts[e].d_down)
+                continue;
+            const float v = weights[pair] * pair_out[(size_t)pair * hidden + h];
+            if (first)
+            {
+                y = v;
+                first = false;
+            }
+            else
+                y = y + v;
+        }
+        float *dst = out + (size_t)t * hidden + h;
+        *dst = accumulate ? (*dst + y) : y;
     }
 
     // ---- SwiGLU + Q8_1 ---------------------------------------------------------------
@@ -408,6 +707,20 @@ namespace llamql
         dst[1 + sub] = q.packed;
         if (sub == 0)
             dst[0] = q.head;
+    }
+
+    // ---- fp32 routing indices -> int32 ids ----------------------------------------------------
+    // The reference's device routing tensors hold expert indices as fp32 values
+    // (IMoEKernel::groupedExpert*DecodeFromRouting, src/v2/kernels/IMoEKernel.h:480-575).
+    __global__ void __launch_bounds__(256)
+        moe_ids_from_f32_kernel(const float *__restrict__ src, int32_t *__restrict__ dst, int n)
+    {
+        const int i = blockIdx.x * blockDim.x + threadIdx.x;
+        if (i < n)
+        {
+            const float v = src[i];
+            dst[i] = (v >= 0.0f && v < 2147483520.0f) ? (int32_t)v : -1; // NaN, negative, huge: no expert
+        }
     }
 
     // ---- shared expert gate -----------------------------------------------------------
@@ -669,6 +982,153 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     return launched(fn);
 }
 
+
+extern "C" size_t llam_ql_moe_group_bytes(int n_tokens, int slot_stride)
+{
+    if (n_tokens < 1 || slot_stride < 1)
+        return 0;
+    return llamql::moe_group_bytes(n_tokens * slot_stride);
+}
+
+extern "C" bool llam_ql_moe_group(const int32_t *d_ids, int n_tokens, int slot_stride, int n_experts, void *d_group,
+                                  int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_group";
+    if (n_tokens < 1 || slot_stride < 1 || n_experts < 1)
+        return fail(fn, "need n_tokens, slot_stride, n_experts >= 1 (%d, %d, %d)", n_tokens, slot_stride, n_experts);
+    const long P = (long)n_tokens * slot_stride;
+    if (P > MOE_GROUP_MAX_PAIRS)
+        return fail(fn, "%ld (token, slot) pairs: at most %d are grouped in one call", P, MOE_GROUP_MAX_PAIRS);
+    if (!d_ids || !d_group)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_group))
+        return fail(fn, "d_group must be 16-byte aligned");
+    if (!set_device(fn, device_id))
+        return false;
+    if (n_experts > MOE_GROUP_MAX_EXPERTS)
+        return fail(fn, "n_experts=%d: at most %d experts are grouped", n_experts, MOE_GROUP_MAX_EXPERTS);
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(MOE_GROUP_THREADS), (size_t)((P + 3) & ~3L) * 4,
+                       as_stream(stream), d_ids, (int)P, n_experts, d_group);
+    return launched(fn);
+}
+
+namespace llamql
+{
+    namespace
+    {
+        template <class F>
+        bool moe_grouped_launch(const char *fn, bool down, const MoEArgs &m, void *ws, int P, dim3 grid, hipStream_t st)
+        {
+            const int nsb = (down ? m.inter : m.hidden) / 256;
+            const size_t lds = gemv_lds_bytes<F>(4, nsb);
+            if (lds > 64 * 1024)
+                return fail(fn, "%s=%d too large for one LDS stage of four tokens", down ? "inter" : "hidden",
+                            down ? m.inter : m.hidden);
+            const dim3 block(GEMV_WAVES * WAVE);
+            const bool four = moe_chunk_size(P) > 2; // the chunk size llam_ql_moe_group used for P pairs
+            if (down && four)
+                hipLaunchKernelGGL((moe_down_grouped_kernel<F, 4>), grid, block, lds, st, m, ws, P);
+            else if (down)
+                hipLaunchKernelGGL((moe_down_grouped_kernel<F, 2>), grid, block, lds, st, m, ws, P);
+            else if (four)
+                hipLaunchKernelGGL((moe_gate_up_grouped_kernel<F, 4>), grid, block, lds, st, m, ws, P);
+            else
+                hipLaunchKernelGGL((moe_gate_up_grouped_kernel<F, 2>), grid, block, lds, st, m, ws, P);
+            return launched(fn);
+        }
+    } // namespace
+} // namespace llamql
+
+extern "C" bool llam_ql_moe_gate_up_grouped(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                                            const void *d_group, const void *d_q8, float *d_gate_out,
+                                            float *d_up_out, int n_tokens, int slot_stride, int hidden, int inter,
+                                            int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_gate_up_grouped";
+    if (!check_moe(fn, fmt, n_tokens, n_experts, slot_stride, hidden, inter))
+        return false;
+    const long P = (long)n_tokens * slot_stride;
+    if (P > MOE_GROUP_MAX_PAIRS)
+        return fail(fn, "%ld (token, slot) pairs: at most %d are grouped", P, MOE_GROUP_MAX_PAIRS);
+    if (!d_experts || !d_group || !d_q8 || !d_gate_out || !d_up_out)
+        return fail(fn, "null pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    MoEArgs m;
+    m.experts = d_experts;
+    m.ids = nullptr;
+    m.weights = nullptr;
+    m.q8 = static_cast<const uint32_t *>(d_q8);
+    m.out0 = d_gate_out;
+    m.out1 = d_up_out;
+    m.n_experts = n_experts;
+    m.top_k = slot_stride;
+    m.hidden = hidden;
+    m.inter = inter;
+    m.accumulate = 0;
+    long gx;
+    moe_shape(inter, hidden / 256, P * 2, device_id, m.gshift, m.rows_per_wave, gx);
+    const dim3 grid((unsigned)gx, (unsigned)P, 2); // one chunk per workgroup row; P bounds their number
+    void *ws = const_cast<void *>(d_group);
+    hipStream_t st = as_stream(stream);
+    switch (fmt)
+    {
+    case LLAM_FMT_Q4_K: return moe_grouped_launch<Q4KTraits>(fn, false, m, ws, (int)P, grid, st);
+    case LLAM_FMT_Q6_K: return moe_grouped_launch<Q6KTraits>(fn, false, m, ws, (int)P, grid, st);
+    default: return moe_grouped_launch<IQ3STraits>(fn, false, m, ws, (int)P, grid, st);
+    }
+}
+
+extern "C" bool llam_ql_moe_down_grouped(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                                         const void *d_group, const int32_t *d_ids, const float *d_weights,
+                                         const void *d_q8_act, float *d_pair_out, float *d_out, int n_tokens,
+                                         int slot_stride, int hidden, int inter, int accumulate, int device_id,
+                                         void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_down_grouped";
+    if (!check_moe(fn, fmt, n_tokens, n_experts, slot_stride, hidden, inter))
+        return false;
+    const long P = (long)n_tokens * slot_stride;
+    if (P > MOE_GROUP_MAX_PAIRS)
+        return fail(fn, "%ld (token, slot) pairs: at most %d are grouped", P, MOE_GROUP_MAX_PAIRS);
+    if (!d_experts || !d_group || !d_ids || !d_weights || !d_q8_act || !d_pair_out || !d_out)
+        return fail(fn, "null pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    MoEArgs m;
+    m.experts = d_experts;
+    m.ids = d_ids;
+    m.weights = d_weights;
+    m.q8 = static_cast<const uint32_t *>(d_q8_act);
+    m.out0 = d_out;
+    m.out1 = d_pair_out;
+    m.n_experts = n_experts;
+    m.top_k = slot_stride;
+    m.hidden = hidden;
+    m.inter = inter;
+    m.accumulate = accumulate;
+    long gx;
+    moe_shape(hidden, inter / 256, P, device_id, m.gshift, m.rows_per_wave, gx);
+    const dim3 grid((unsigned)gx, (unsigned)P);
+    void *ws = const_cast<void *>(d_group);
+    hipStream_t st = as_stream(stream);
+    bool ok;
+    switch (fmt)
+    {
+    case LLAM_FMT_Q4_K: ok = moe_grouped_launch<Q4KTraits>(fn, true, m, ws, (int)P, grid, st); break;
+    case LLAM_FMT_Q6_K: ok = moe_grouped_launch<Q6KTraits>(fn, true, m, ws, (int)P, grid, st); break;
+    default: ok = moe_grouped_launch<IQ3STraits>(fn, true, m, ws, (int)P, grid, st); break;
+    }
+    if (!ok)
+        return false;
+    hipLaunchKernelGGL(moe_pair_reduce_kernel, dim3((unsigned)((hidden + 255) / 256), (unsigned)n_tokens), dim3(256), 0,
+                       st, d_pair_out, d_ids, d_weights, d_experts, n_experts, d_out, slot_stride, hidden, accumulate);
+    return launched(fn);
+}
+
 extern "C" bool llam_ql_swiglu_quantize(const float *d_gate, const float *d_up,
                                         float *d_act_out, void *d_q8_out, int rows,
                                         int inter, int device_id, void *stream)
@@ -732,6 +1192,23 @@ extern "C" bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts, i
     case LLAM_FMT_Q6_K: return moe_down_launch<Q6KTraits>(fn, m, grid, block, st);
     default: return moe_down_launch<IQ3STraits>(fn, m, grid, block, st);
     }
+}
+
+extern "C" bool llam_ql_moe_ids_from_f32(const float *d_indices, int32_t *d_ids, int n, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_ids_from_f32";
+    if (n < 0)
+        return fail(fn, "negative count");
+    if (n == 0)
+        return true;
+    if (!d_indices || !d_ids)
+        return fail(fn, "null pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(moe_ids_from_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       d_indices, d_ids, n);
+    return launched(fn);
 }
 
 extern "C" bool llam_ql_shared_expert_add(float *d_out, const float *d_shared,

@@ -136,7 +136,8 @@ static void test_host_logic()
     CHECK(MI355MoEKernel::getWorkspaceRequirements(0, 9, 2048, 512, 256) == 0);
     const size_t ws = MI355MoEKernel::getWorkspaceRequirements(1, 9, 2048, 512, 256);
     // logits 1 KiB, Q8_1 hidden 2304 B, gate and up 18 KiB each, Q8_1 activations 5184 B, each rounded to 256
-    CHECK(ws == 1024 + 2304 + 2 * 18432 + 5376);
+    // logits, Q8_1 hidden, gate and up rows, Q8_1 SwiGLU, pair table, per-pair down rows, ids and weights
+    CHECK(ws == 1024 + 2304 + 2 * 18432 + 5376 + 256 + 73728 + 2 * 256);
     DeviceQuantMatrixDesc d[2];
     CHECK(k.uploadGroupedExpertDownDescriptorTable(nullptr, 2, 512, 256) == -1);
     CHECK(k.uploadGroupedExpertDownDescriptorTable(d, 2, 500, 256) == -1 && contains(moe_kernel_last_error(), "bad shape"));
@@ -275,6 +276,61 @@ static void test_decode(uint8_t fmt, int T)
     }
     CHECK(rel_err(out3, ref3) <= 1e-5f);
 
+    // IMoEKernel::route: the same routing with the result on the host, probabilities included
+    {
+        MoERoutingResult rr;
+        CHECK(k.route(d_hidden.p, d_gate_w.p, T, D, E, TOPK, true, rr));
+        CHECK(rr.expert_indices.size() == (size_t)T * TOPK && rr.router_logits.size() == (size_t)T * E);
+        for (int t = 0; t < T; ++t)
+        {
+            for (int s = 0; s < TOPK; ++s)
+            {
+                CHECK(rr.expert_indices[(size_t)t * TOPK + s] == oids[(size_t)t * TOPK + s]);
+                CHECK(std::fabs(rr.expert_weights[(size_t)t * TOPK + s] - ow[(size_t)t * TOPK + s]) <= 1e-5f);
+            }
+            for (int e = 0; e < E; ++e)
+                CHECK(std::fabs(rr.router_logits[(size_t)t * E + e] - probs[(size_t)t * E + e]) <= 1e-5f);
+        }
+    }
+
+    // single-token calls driven by host ids (FromTable) and by fp32 device routing tensors
+    // (FromRouting): the bits of the FromRuntime calls on token 0
+    {
+        std::vector<int> hid(SLOTS);
+        std::vector<float> hw(SLOTS), fidx(SLOTS);
+        for (int s = 0; s < SLOTS; ++s)
+        {
+            hid[s] = ids[s];
+            hw[s] = w[s];
+            fidx[s] = (float)ids[s];
+        }
+        DevBuf<float> d_fidx(fidx), d_fw(hw), g1((size_t)SLOTS * I), u1((size_t)SLOTS * I), g2((size_t)SLOTS * I),
+            u2((size_t)SLOTS * I), o1(D), o2(D), o0(D), g0((size_t)SLOTS * I), u0((size_t)SLOTS * I);
+        DevBuf<int32_t> d_ids0(std::vector<int32_t>(ids.begin(), ids.begin() + SLOTS));
+        DeviceMoELayerRuntime rt0;
+        rt0.topk_expert_ids = d_ids0.p;
+        rt0.topk_weights = d_fw.p;
+        rt0.slot_stride = SLOTS;
+        DeviceTensor th0(d_hidden.p, 1, D), to0(o0.p, 1, D), to1(o1.p, 1, D), to2b(o2.p, 1, D);
+        CHECK(k.groupedExpertGateUpDecodeFromRuntime(&rt0, &th0, tg, SLOTS, g0.p, u0.p, D, I));
+        CHECK(k.groupedExpertDownDecodeFromRuntime(g0.p, u0.p, &rt0, td, SLOTS, &to0, D, I));
+        CHECK(k.groupedExpertGateUpDecodeFromTable(&th0, hid.data(), tg, SLOTS, g1.p, u1.p, D, I));
+        CHECK(k.groupedExpertDownDecodeFromTable(g1.p, u1.p, hid.data(), hw.data(), td, SLOTS, &to1, D, I));
+        CHECK(k.groupedExpertGateUpDecodeFromRouting(&th0, d_fidx.p, tg, SLOTS, g2.p, u2.p, D, I));
+        CHECK(k.groupedExpertDownDecodeFromRouting(g2.p, u2.p, d_fidx.p, d_fw.p, td, SLOTS, &to2b, D, I));
+        const std::vector<float> a0 = o0.download(), a1 = o1.download(), a2 = o2.download();
+        CHECK(memcmp(a0.data(), a1.data(), a0.size() * 4) == 0);
+        CHECK(memcmp(a0.data(), a2.data(), a0.size() * 4) == 0);
+        CHECK(memcmp(a0.data(), out.data(), a0.size() * 4) == 0); // token 0 of the batch
+        // weightedAdd: o1 += 0.25 * o2
+        CHECK(k.weightedAdd(o1.p, o2.p, 0.25f, D));
+        const std::vector<float> a3 = o1.download();
+        float worst = 0.0f;
+        for (int c = 0; c < D; ++c)
+            worst = std::max(worst, std::fabs(a3[c] - (a1[c] + 0.25f * a2[c])));
+        CHECK(worst <= 1e-6f * std::max(1.0f, std::fabs(a1[0])) + 1e-5f);
+    }
+
     // errors keep their reason
     CHECK(!k.groupedExpertDecodeFromRuntime(&rt, &th, td, td, SLOTS, &to, D, I));
     CHECK(contains(moe_kernel_last_error(), "holds no gate/up"));
@@ -291,6 +347,7 @@ int main(int argc, char **argv)
         test_decode(LLAM_FMT_Q4_K, 1);
         test_decode(LLAM_FMT_Q4_K, 5);
         test_decode(LLAM_FMT_IQ3_S, 3);
+        test_decode(LLAM_FMT_IQ3_S, 100); // 300 (token, slot) pairs: the fused sequence groups tokens by expert
     }
     printf("%d checks, %d failed\n%s\n", g_checks, g_failed, g_failed ? "FAILED" : "PASSED");
     return g_failed ? 1 : 0;

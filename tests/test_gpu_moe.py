@@ -208,6 +208,111 @@ def test_expert_ffn_baseline_shape(capi, dev, oracle, T):
     assert rel_err(out.cpu().numpy(), want) <= 1e-3
 
 
+def test_token_without_live_slot_gets_zeros(capi, dev):
+    """accumulate == 0 overwrites: a token whose ids are all out of range (or whose experts
+    live elsewhere) must end up zero, not keep what the buffer held (both down kernels and the
+    grouped path); with accumulate != 0 its row is left alone."""
+    import torch
+
+    fmt, n_exp, T = FMT_Q4_K, 3, 3
+    for hidden, inter, k in ((256, 256, 2), (512, 2304, 2)):  # multi-slot kernel / slot-by-slot kernel
+        host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 7)
+        ids = torch.tensor([[0, 2], [9, -1], [1, 9]], dtype=torch.int32, device=dev)
+        w = torch.full((T, k), 0.5, device=dev)
+        q8a = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(T * k, inter, 3)).to(dev))
+        out = torch.full((T, hidden), 7.0, device=dev)
+        capi.moe_down(fmt, table, n_exp, ids, w, q8a, out, T, k, hidden, inter, accumulate=False)
+        acc = torch.full((T, hidden), 7.0, device=dev)
+        capi.moe_down(fmt, table, n_exp, ids, w, q8a, acc, T, k, hidden, inter, accumulate=True)
+        grp = capi.moe_group(ids, n_exp)
+        pair_out = torch.full((T * k, hidden), float("nan"), device=dev)
+        out_g = torch.full((T, hidden), 7.0, device=dev)
+        capi.moe_down_grouped(fmt, table, n_exp, grp, ids, w, q8a, pair_out, out_g, T, k, hidden, inter)
+        sync()
+        assert float(out[1].abs().max()) == 0.0 and float(out[0].abs().max()) > 0.0
+        assert float((acc[1] - 7.0).abs().max()) == 0.0
+        assert torch.equal(out_g, out)
+
+
+def test_group_tokens_by_expert(capi, dev):
+    """The device-side sort of (token, slot) pairs by expert against numpy's stable argsort:
+    segment table, order inside a segment, ids out of range left out."""
+    import torch
+
+    rng = np.random.default_rng(21)
+    for T, S, E in ((1, 9, 257), (16, 9, 257), (5, 3, 4), (64, 9, 257), (7, 1, 2)):
+        ids = rng.integers(-1, E + 2, size=(T, S)).astype(np.int32)  # -1, E and E+1 are invalid
+        g = capi.moe_group(torch.from_numpy(ids).to(dev), E)
+        sync()
+        P = T * S
+        w = g.cpu().numpy().view(np.int32)
+        flat = ids.reshape(-1)
+        valid = np.flatnonzero((flat >= 0) & (flat < E))
+        order = valid[np.argsort(flat[valid], kind="stable")]
+        experts = np.unique(flat[valid])
+        n_seg, n_valid = int(w[0]), int(w[1])
+        assert n_valid == len(valid) and n_seg == len(experts)
+        seg_expert, seg_begin, pair_sorted = w[4:4 + P], w[4 + P:4 + 2 * P + 1], w[4 + 2 * P + 1:4 + 3 * P + 1]
+        assert np.array_equal(seg_expert[:n_seg], experts)
+        assert np.array_equal(pair_sorted[:n_valid], order)
+        begins = np.searchsorted(flat[order], experts)
+        assert np.array_equal(seg_begin[:n_seg], begins) and seg_begin[n_seg] == n_valid
+        # chunks: every segment cut into runs of at most `per` pairs (2 below 512 pairs, else 4), in segment order
+        per = 4 if P >= 512 else 2
+        assert int(w[3]) == per
+        c0 = 4 + 3 * P + 1
+        chunk_expert, chunk_begin, chunk_count = w[c0:c0 + P], w[c0 + P:c0 + 2 * P], w[c0 + 2 * P:c0 + 3 * P]
+        want = []
+        ends = list(begins[1:]) + [n_valid]
+        for e, b, en in zip(experts, begins, ends):
+            for j in range(b, en, per):
+                want.append((e, j, min(per, en - j)))
+        assert int(w[2]) == len(want)
+        got = list(zip(chunk_expert[:len(want)].tolist(), chunk_begin[:len(want)].tolist(), chunk_count[:len(want)].tolist()))
+        assert got == [(int(e), int(b), int(c)) for e, b, c in want]
+
+
+@pytest.mark.parametrize("fmt", list(FMTS.values()), ids=list(FMTS))
+def test_grouped_launches_equal_ungrouped(capi, dev, fmt):
+    """Tokens grouped by expert: every gate/up row and every token output carries the bits of
+    the ungrouped launches (12 tokens on 5 experts + an always-on slot: segments of 1..12 tokens,
+    an expert missing from the table, an id out of range)."""
+    import torch
+
+    n_exp, hidden, inter, k, T = 6, 1024, 512, 3, 12
+    host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 60)
+    tab = table.clone()
+    tab.view(torch.int64).view(n_exp, 3)[4] = 0      # expert 4 lives elsewhere: null matrices
+    rng = np.random.default_rng(9)
+    ids = rng.integers(0, n_exp - 1, size=(T, k + 1)).astype(np.int32)
+    ids[:, k] = n_exp - 1                             # the always-on expert in the extra slot
+    ids[3, 1] = 77                                    # out of range
+    idd = torch.from_numpy(ids).to(dev)
+    w = torch.from_numpy(rng.random((T, k + 1)).astype(np.float32)).to(dev)
+    qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(T, hidden, 4)).to(dev))
+    S = k + 1
+    gate = torch.full((T * S, inter), 3.0, device=dev)
+    up = torch.full((T * S, inter), 3.0, device=dev)
+    lib = capi.load()
+    assert lib.llam_ql_moe_gate_up(fmt, tab.data_ptr(), n_exp, idd.data_ptr(), qd.data_ptr(), gate.data_ptr(),
+                                   up.data_ptr(), T, S, hidden, inter, 0, None)
+    grp = capi.moe_group(idd, n_exp)
+    gate_g = torch.full((T * S, inter), 3.0, device=dev)
+    up_g = torch.full((T * S, inter), 3.0, device=dev)
+    capi.moe_gate_up_grouped(fmt, tab, n_exp, grp, qd, T, S, hidden, inter, gate=gate_g, up=up_g)
+    sync()
+    assert torch.equal(gate_g, gate) and torch.equal(up_g, up)
+    q8a = capi.swiglu_quantize(gate, up)
+    out = torch.full((T, hidden), float("nan"), device=dev)
+    capi.moe_down(fmt, tab, n_exp, idd, w, q8a, out, T, S, hidden, inter, accumulate=False)
+    out_g = torch.full((T, hidden), float("nan"), device=dev)
+    pair_out = torch.empty((T * S, hidden), device=dev)
+    capi.moe_down_grouped(fmt, tab, n_exp, grp, idd, w, q8a, pair_out, out_g, T, S, hidden, inter)
+    sync()
+    assert torch.equal(out_g, out)
+    assert bool(torch.isfinite(out).all())
+
+
 def test_shared_expert_gate(capi, dev):
     import torch
 
