@@ -58,8 +58,7 @@ namespace llamql
     template <class F>
     constexpr size_t gemm_lds_bytes()
     {
-        return (size_t)(GEMM_BM + GEMM_BN) * GEMM_STRIDE + (size_t)2 * 8 * (GEMM_SM + GEMM_SN) * sizeof(float) +
-               F::TABLE_BYTES;
+        return (size_t)(GEMM_BM + GEMM_BN) * GEMM_STRIDE + (size_t)2 * 8 * (GEMM_SM + GEMM_SN) * sizeof(float);
     }
 
     // Two adjacent Q8_1 blocks (72 bytes, 4-byte aligned) of one token, fetched with loads
@@ -191,7 +190,7 @@ namespace llamql
         float *asd = ad + 8 * GEMM_SM;                  // [8][SM]
         float *bs = asd + 8 * GEMM_SM;                  // [8][SN]
         float *bm = bs + 8 * GEMM_SN;                   // [8][SN]
-        void *tab = bm + 8 * GEMM_SN;
+        void *tab = format_tables_lds<F>(); // static LDS beside the dynamic tiles
 
         if (F::TABLE_BYTES > 0)
             F::stage_tables(tab);

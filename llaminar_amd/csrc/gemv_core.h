@@ -59,6 +59,21 @@ namespace llamql
         int pair_div;
     };
 
+    // The format's decode tables (IQ3_S: codebook, maps, sign masks) live in STATIC LDS: their
+    // address is a link-time constant, so every table look-up is a ds_read with an immediate
+    // offset instead of an address addition.  Null for formats without tables.
+    template <class F>
+    __device__ __forceinline__ void *format_tables_lds()
+    {
+        if constexpr (F::TABLE_BYTES > 0)
+        {
+            __shared__ __attribute__((aligned(16))) uint8_t format_tables[F::TABLE_BYTES];
+            return format_tables;
+        }
+        else
+            return nullptr;
+    }
+
     // Stage `nkb` Q8_1 blocks of each of M activation rows into LDS.
     template <class F, int M>
     __device__ __forceinline__ void stage_q8(const uint32_t *__restrict__ q8, int KB_total, int kb0, int nkb,
@@ -144,7 +159,7 @@ namespace llamql
         uint32_t *aq = lds;                                      // M * nkb * 8 dwords
         float *ad = reinterpret_cast<float *>(aq + M * nkb * 8); // M * nkb
         float *asd = ad + M * nkb;                               // M * nkb
-        void *tab = asd + M * nkb;                               // F::TABLE_BYTES
+        void *tab = format_tables_lds<F>();
 
         const int lane = threadIdx.x & (WAVE - 1);
         const int wave = threadIdx.x >> 6;
@@ -317,7 +332,7 @@ namespace llamql
     template <class F>
     inline size_t gemv_lds_bytes(int M, int nsb)
     {
-        return (size_t)M * nsb * GEMV_LDS_PER_SB + F::TABLE_BYTES;
+        return (size_t)M * nsb * GEMV_LDS_PER_SB; // dynamic part; F::TABLE_BYTES more are static
     }
 
 } // namespace llamql

@@ -22,6 +22,7 @@
 #include "gemv_quad.h"
 #include "gemv_mfma.h"
 #include "gemv_mfma_q6k.h"
+#include <atomic>
 #include <type_traits>
 
 namespace llamql
@@ -110,7 +111,7 @@ namespace llamql
         const int nkb = a.nsb * 8;
         uint32_t *aq = lds;                                          // M * nkb * 8 dwords
         float2 *ads = reinterpret_cast<float2 *>(aq + M * nkb * 8);  // M * nkb
-        void *tab = ads + M * nkb;                                   // F::TABLE_BYTES
+        void *tab = format_tables_lds<F>();
 
         const int lane = threadIdx.x & (WAVE - 1);
         const int wave = threadIdx.x >> 6;
@@ -272,6 +273,66 @@ namespace llamql
         }
     }
 
+    // Wavefronts of gemv_fast_kernel<F, M, U> a compute unit holds at once, as far as registers
+    // allow (asked of the runtime once per instantiation; the LDS limit is the caller's).
+    template <class F, int M, int U>
+    inline int gemv_fast_resident_waves_mu()
+    {
+        static std::atomic<int> cached{0};
+        int w = cached.load(std::memory_order_relaxed);
+        if (w == 0)
+        {
+            int blocks = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, gemv_fast_kernel<F, M, U, false>,
+                                                             GEMV_WAVES * WAVE, 0) != hipSuccess ||
+                blocks < 1)
+            {
+                (void)hipGetLastError();
+                blocks = 32 / GEMV_WAVES;
+            }
+            w = blocks * GEMV_WAVES;
+            cached.store(w, std::memory_order_relaxed);
+        }
+        return w;
+    }
+
+    template <class F, int M>
+    inline int gemv_fast_resident_waves_m(int U)
+    {
+        if constexpr (F::FAST_MAX_U >= 4)
+        {
+            switch (U)
+            {
+            case 1: return gemv_fast_resident_waves_mu<F, M, 1>();
+            case 2: return gemv_fast_resident_waves_mu<F, M, 2>();
+            case 3: return gemv_fast_resident_waves_mu<F, M, 3>();
+            default: return gemv_fast_resident_waves_mu<F, M, 4>();
+            }
+        }
+        else
+            return gemv_fast_resident_waves_mu<F, M, 1>();
+    }
+
+    // M is one of 1,2,3,4,8; lds: dynamic LDS of a workgroup.
+    template <class F>
+    inline int gemv_fast_resident_waves(int M, int U, size_t lds)
+    {
+        int w;
+        switch (M)
+        {
+        case 1: w = gemv_fast_resident_waves_m<F, 1>(U); break;
+        case 2: w = gemv_fast_resident_waves_m<F, 2>(U); break;
+        case 3: w = gemv_fast_resident_waves_m<F, 3>(U); break;
+        case 4: w = gemv_fast_resident_waves_m<F, 4>(U); break;
+        default: w = gemv_fast_resident_waves_m<F, 8>(U); break;
+        }
+        const size_t per_wg = lds + F::TABLE_BYTES + 256;
+        const long by_lds = (long)(160 * 1024 / per_wg) * GEMV_WAVES;
+        if (by_lds < w)
+            w = (int)by_lds;
+        return w < GEMV_WAVES ? GEMV_WAVES : w;
+    }
+
     int gemv_unroll_override();
     // Launch shape for N rows of nsb super-blocks (one LDS slice) on a device with
     // `cus` compute units.  Rows are dealt to workgroups so that every compute unit
@@ -282,7 +343,10 @@ namespace llamql
         long grid;
     };
 
-    inline GemvShape gemv_shape(long N, int nsb, int cus)
+    // max_u: deepest unroll the format builds; resident(U): wavefronts of the kernel with that
+    // unroll a compute unit holds at once.
+    template <class Resident>
+    inline GemvShape gemv_shape(long N, int nsb, int cus, int max_u, Resident resident)
     {
         GemvShape sh;
         sh.gshift = 3;
@@ -309,6 +373,12 @@ namespace llamql
         }
         if (gemv_unroll_override() > 0)
             sh.U = gemv_unroll_override() > 4 ? 4 : gemv_unroll_override();
+        else if (sh.U > max_u)
+            sh.U = max_u;
+        int cap = sh.gshift == 3 ? resident(sh.U) : 32; // wavefronts a compute unit holds
+        if (cap > 32)
+            cap = 32;
+        const int floor_waves = cap < 16 ? cap : 16;
 
         // rows (in units of R) each compute unit must cover
         const long units = (N + R - 1) / R;
@@ -316,19 +386,20 @@ namespace llamql
         int rpw = gemv_rows_per_wave_override();
         if (rpw <= 0)
         {
-            // candidates: 1..8 row batches per wavefront; cost = padded work per CU, with
-            // at least 16 wavefronts per CU when there is enough work, at most 32
+            // candidates: row batches per wavefront; cost = padded work per CU, with at least
+            // 16 wavefronts per CU when there is enough work (and they fit), at most what a
+            // compute unit holds at once: a second round runs at a fraction of the occupancy
             double best_cost = 1e30;
             rpw = 1;
-            for (int cand = 1; cand <= 8; ++cand)
+            for (int cand = 1; cand <= 64; ++cand)
             {
                 const long wg_units = (long)GEMV_WAVES * cand;
                 const long wgs_per_cu = (per_cu + wg_units - 1) / wg_units;
                 double cost = (double)(wgs_per_cu * wg_units) / (double)per_cu;
                 const long waves = wgs_per_cu * GEMV_WAVES;
-                if (waves > 32)
-                    cost *= 1.0 + 0.05 * (double)((waves + 31) / 32 - 1); // extra rounds: restaging + tail
-                if (waves < 16 && per_cu >= 16)
+                if (waves > cap)
+                    cost *= 1.0 + 0.25 * (double)((waves + cap - 1) / cap - 1); // extra rounds: restaging + tail
+                if (waves < floor_waves && per_cu >= floor_waves)
                     cost *= 1.25; // too little memory-level parallelism
                 if (cost < best_cost - 1e-9)
                 {
@@ -691,9 +762,10 @@ namespace llamql
             p.kernel = -1;
             return p;
         }
-        GemvShape sh = gemv_shape(N, slice, cu_count(device_id));
-        if (gemv_unroll_override() <= 0 && sh.U > F::FAST_MAX_U)
-            sh.U = F::FAST_MAX_U;
+        const int m_first = p.m_first;
+        const GemvShape sh = gemv_shape(N, slice, cu_count(device_id), F::FAST_MAX_U, [=](int U) {
+            return gemv_fast_resident_waves<F>(m_first, U, gemv_lds_bytes<F>(m_first, slice));
+        });
         p.kernel = sh.gshift == 3 ? GEMV_KERNEL_CHUNKED : GEMV_KERNEL_GENERIC;
         p.slice_sb = slice;
         p.rows_per_wave = sh.rpw;

@@ -279,7 +279,7 @@ namespace llamql
         uint32_t *aq = lds;
         float *ad = reinterpret_cast<float *>(aq + nkb_all * 8);
         float *asd = ad + nkb_all;
-        void *tab = asd + nkb_all;
+        void *tab = format_tables_lds<F>();
 
         const int lane = threadIdx.x & (WAVE - 1);
         const int wave = threadIdx.x >> 6;
@@ -796,8 +796,8 @@ namespace llamql
             if (nsb <= 8 && m.top_k <= 12)
             {
                 const int S = m.top_k <= 4 ? 4 : (m.top_k <= 8 ? 8 : 12);
-                const size_t lds = (size_t)m.top_k * nsb * GEMV_LDS_PER_SB + F::TABLE_BYTES;
-                if (lds <= 64 * 1024)
+                const size_t lds = (size_t)m.top_k * nsb * GEMV_LDS_PER_SB;
+                if (lds + F::TABLE_BYTES <= 64 * 1024)
                 {
                     if (S == 4)
                         hipLaunchKernelGGL((moe_down_multi_kernel<F, 4>), grid, block, lds, st, m);
@@ -809,7 +809,7 @@ namespace llamql
                 }
             }
             const size_t lds = gemv_lds_bytes<F>(1, nsb);
-            if (lds > 64 * 1024)
+            if (lds + F::TABLE_BYTES > 64 * 1024)
                 return fail(fn, "inter=%d too large for one LDS stage", m.inter);
             hipLaunchKernelGGL((moe_down_kernel<F>), grid, block, lds, st, m);
             return launched(fn);
@@ -957,7 +957,7 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     case LLAM_FMT_Q4_K:
     {
         const size_t lds = gemv_lds_bytes<Q4KTraits>(1, hidden / 256);
-        if (lds > 64 * 1024)
+        if (lds + Q4KTraits::TABLE_BYTES > 64 * 1024)
             return fail(fn, "hidden=%d too large for one LDS stage", hidden);
         hipLaunchKernelGGL((moe_gate_up_kernel<Q4KTraits>), grid, block, lds, st, m);
         break;
@@ -965,7 +965,7 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     case LLAM_FMT_Q6_K:
     {
         const size_t lds = gemv_lds_bytes<Q6KTraits>(1, hidden / 256);
-        if (lds > 64 * 1024)
+        if (lds + Q6KTraits::TABLE_BYTES > 64 * 1024)
             return fail(fn, "hidden=%d too large for one LDS stage", hidden);
         hipLaunchKernelGGL((moe_gate_up_kernel<Q6KTraits>), grid, block, lds, st, m);
         break;
@@ -973,7 +973,7 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     default:
     {
         const size_t lds = gemv_lds_bytes<IQ3STraits>(1, hidden / 256);
-        if (lds > 64 * 1024)
+        if (lds + IQ3STraits::TABLE_BYTES > 64 * 1024)
             return fail(fn, "hidden=%d too large for one LDS stage", hidden);
         hipLaunchKernelGGL((moe_gate_up_kernel<IQ3STraits>), grid, block, lds, st, m);
         break;
@@ -1022,7 +1022,7 @@ namespace llamql
         {
             const int nsb = (down ? m.inter : m.hidden) / 256;
             const size_t lds = gemv_lds_bytes<F>(4, nsb);
-            if (lds > 64 * 1024)
+            if (lds + F::TABLE_BYTES > 64 * 1024)
                 return fail(fn, "%s=%d too large for one LDS stage of four tokens", down ? "inter" : "hidden",
                             down ? m.inter : m.hidden);
             const dim3 block(GEMV_WAVES * WAVE);

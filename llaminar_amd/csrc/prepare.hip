@@ -6,9 +6,11 @@
 //   Q6_K  : planes ql [T][128] | qh [T][64] | scales [T][16] | d [T] fp16      (T*210 B)
 //           | pad to 16 | factors [T][8] x 4 B (q6k_block_code, ql_device.h)    (T*32 B)
 //   IQ3_S : planes qs [T][64] | signs [T][32] | meta [T][16]                   (T*112 B)
-//           meta = qh[8] scales[4] d[2] pad[2]
+//           meta = qh[8] scales[4] d[2] hints[2]: two bits per 32-element block, which of the
+//           requantisation maps the block needs (its largest codebook magnitude; iq3s_gmax_hint)
 // with T = N*K/256 super-blocks in row-major order.  Raw Q6_K / IQ3_S blocks are
 // 210 / 110 bytes, i.e. only 2-byte aligned, so the copy works in halfwords.
+#include "gemv_traits_iq3s.h"
 #include "ql_device.h"
 #include "ql_host.h"
 
@@ -55,7 +57,7 @@ namespace llamql
     __global__ void __launch_bounds__(256)
         prepare_iq3s_kernel(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst, size_t T)
     {
-        // 56 halfwords are written per block (55 copied + 1 zero pad)
+        // 56 halfwords are written per block (55 copied + the gmax hints in place of padding)
         const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
         if (i >= T * 56)
             return;
@@ -65,7 +67,11 @@ namespace llamql
         size_t o;
         if (u == 55)
         {
-            o = T * 48 + t * 8 + 7; // pad
+            o = T * 48 + t * 8 + 7; // hints: block j in bits 2j, 2j+1
+            const uint8_t *blk = reinterpret_cast<const uint8_t *>(src + t * 55); // d[2] qs[64] qh[8] signs[32] scales[4]
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                v |= (uint16_t)(iq3s_gmax_hint(blk + 2 + 8 * j, blk[66 + j]) << (2 * j));
         }
         else
         {

@@ -55,6 +55,7 @@ class Oracle:
         L.qlo_moe_route.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
         L.qlo_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_void_p]
         L.qlo_check_div127.restype = ctypes.c_long
+        L.qlo_check_div127_all_significands.restype = ctypes.c_long
         L.qlo_check_q6k_factor.restype = ctypes.c_long
         L.qlo_check_q6k_factor.argtypes = [c_int]
         L.qlo_dequant_row_q4k.argtypes = [c_void_p, c_int, c_void_p]
@@ -149,6 +150,9 @@ class Oracle:
 
     def check_div127(self) -> int:
         return int(self.L.qlo_check_div127())
+
+    def check_div127_all_significands(self) -> int:
+        return int(self.L.qlo_check_div127_all_significands())
 
     def check_q6k_factor(self, ulps: int) -> int:
         return int(self.L.qlo_check_q6k_factor(ulps))

@@ -468,6 +468,36 @@ long qlo_check_div127(void)
     return bad;
 }
 
+/* The same correction step for EVERY finite x: the result of the sequence depends on the
+ * significand of x only (each operation scales with x by an exact power of two as long as
+ * nothing leaves the normal range), so all 2^23 significands at two exponents far from the
+ * ends of the range cover every x between 2^-100 and 2^100.  Used by the IQ3_S block scale
+ * (gmax * d * (1 + 2 nib)) / 127 of the GPU decoder. */
+long qlo_check_div127_all_significands(void)
+{
+    const float c = 0x1.020408p-7f;
+    long bad = 0;
+    for (int pass = 0; pass < 2; ++pass)
+    {
+        const uint32_t expo = pass == 0 ? 127u : 127u - 20u;
+        for (uint32_t m = 0; m < (1u << 23); ++m)
+        {
+            const uint32_t bits = (expo << 23) | m;
+            float x;
+            memcpy(&x, &bits, 4);
+            const float want = x / 127.0f;
+            const float q0 = x * c;
+            const float r = fmaf(-q0, 127.0f, x);
+            const float got = fmaf(r, c, q0);
+            uint32_t a, b;
+            memcpy(&a, &want, 4);
+            memcpy(&b, &got, 4);
+            bad += a != b;
+        }
+    }
+    return bad;
+}
+
 /* nearbyint(s * 32512 / (msc * 32)) for |s| <= msc <= 128 (the 8.8 factor of the smaller
  * sub-scale) against rint of one Newton step on s * 1016 * r, for EVERY r within `ulps`
  * units in the last place of the correctly rounded 1/msc (the GPU's reciprocal instruction

@@ -98,6 +98,7 @@ void qlo_swiglu(const float *gate, const float *up, int n, float *out);
 /* Exhaustive checks of division-free forms used by the GPU kernels: number of inputs on
  * which they differ from the reference's divisions (0 expected).                          */
 long qlo_check_div127(void);
+long qlo_check_div127_all_significands(void);
 long qlo_check_q6k_factor(int ulps);
 
 /* ---- decode-step operators (decode_oracle.c) ------------------------------------- */

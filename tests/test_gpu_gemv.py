@@ -9,6 +9,7 @@ from tests.helpers import FMTS, TOL, rel_err, sync, upload_q8, upload_weights
 
 pytestmark = pytest.mark.gpu
 
+GOLDEN_PATH = __import__("pathlib").Path(__file__).resolve().parent / "golden" / "ql_goldens.npz"
 GOLD = {FMT_Q4_K: "q4k", FMT_Q6_K: "q6k", FMT_IQ3_S: "iq3s"}
 
 
@@ -291,7 +292,17 @@ def test_prepare_moves_every_byte(capi, dev, oracle, fmt):
         assert np.array_equal(meta[:, 0:8], B[:, 66:74])
         assert np.array_equal(meta[:, 8:12], B[:, 106:110])
         assert np.array_equal(meta[:, 12:14], B[:, 0:2])
-        assert not meta[:, 14:].any()
+        # the two spare bytes carry the gmax hints: two bits per 32-element block, 7 - k for the
+        # block's largest codebook magnitude 2k+1 when k >= 5, else 3
+        grid = np.load(GOLDEN_PATH, allow_pickle=False)["iq3s_grid"].astype(np.uint32).reshape(-1)[:512]
+        kmax = np.max(np.stack([(grid >> (8 * b)) & 0xFF for b in range(4)]), axis=0) >> 1
+        hints = meta[:, 14].astype(np.uint32) | (meta[:, 15].astype(np.uint32) << 8)
+        for t in range(T):
+            qs, qh = B[t, 2:66].astype(np.uint32), B[t, 66:74].astype(np.uint32)
+            for j in range(8):
+                idx = qs[8 * j:8 * j + 8] | (((qh[j] >> np.arange(8)) & 1) << 8)
+                k = int(kmax[idx].max())
+                assert (int(hints[t]) >> (2 * j)) & 3 == (7 - k if k >= 5 else 3), (t, j)
 
 
 def test_error_paths(capi, dev):

@@ -142,6 +142,8 @@ def test_division_free_forms_of_the_q6k_factors(oracle):
     x/127 for every fp16 d and max sub-scale, and rne(s*1016/msc) for every (s, msc) with any
     reciprocal within 4 units in the last place of the true one."""
     assert oracle.check_div127() == 0
+    # every fp32 significand: the IQ3_S block scale divides d * (odd products up to 465) by 127
+    assert oracle.check_div127_all_significands() == 0
     for ulps in (0, 1, 4):
         assert oracle.check_q6k_factor(ulps) == 0
 
