@@ -50,18 +50,23 @@ namespace llamql
 
     namespace
     {
-        // the other format with a quad-lane kernel
+        // the format that can share a quad-lane launch with F (Q and K in Q4_K with V in Q6_K)
         template <class F>
-        struct Other;
+        struct Other
+        {
+            static constexpr bool exists = false;
+        };
         template <>
         struct Other<Q4KTraits>
         {
+            static constexpr bool exists = true;
             typedef Q6KTraits type;
             static constexpr uint8_t fmt = LLAM_FMT_Q6_K;
         };
         template <>
         struct Other<Q6KTraits>
         {
+            static constexpr bool exists = true;
             typedef Q4KTraits type;
             static constexpr uint8_t fmt = LLAM_FMT_Q4_K;
         };
@@ -86,7 +91,7 @@ namespace llamql
                 ++n;
             }
             // a following run in the other quad-lane format joins the launch (Q and K with V)
-            if constexpr (F::USE_QUAD)
+            if constexpr (F::USE_QUAD && Other<F>::exists)
                 if (n >= 1 && n < QUAD_MAX_PROJ && src.kind != ACT_SRC_SWIGLU)
                 {
                     typedef typename Other<F>::type G;
@@ -119,6 +124,7 @@ namespace llamql
         {
         case LLAM_FMT_Q4_K: return group_launch<Q4KTraits>(fn, projs, num, src, M, K, device_id, st);
         case LLAM_FMT_Q6_K: return group_launch<Q6KTraits>(fn, projs, num, src, M, K, device_id, st);
+        case LLAM_FMT_IQ3_S: return group_launch<IQ3STraits>(fn, projs, num, src, M, K, device_id, st);
         default: return 0;
         }
     }

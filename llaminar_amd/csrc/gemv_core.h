@@ -27,7 +27,7 @@
 //   static void unit_of(int j, int q, int &c, int &p)   LDS slot of dword q of block j
 //   static Raw  load(const GemvArgs&, long row, int sb, int c)
 //   static void decode(const Raw&, int c, v4i &w0, v4i &w1, int &j, float &bscale, float &bmin, const void *tab)
-//   static constexpr int TABLE_BYTES; static void stage_tables(void *lds_tab)
+//   static constexpr int TABLE_BYTES; static void *tables_lds(); static void stage_tables(void *lds_tab)
 #pragma once
 
 #include "ql_device.h"
@@ -65,13 +65,7 @@ namespace llamql
     template <class F>
     __device__ __forceinline__ void *format_tables_lds()
     {
-        if constexpr (F::TABLE_BYTES > 0)
-        {
-            __shared__ __attribute__((aligned(16))) uint8_t format_tables[F::TABLE_BYTES];
-            return format_tables;
-        }
-        else
-            return nullptr;
+        return F::tables_lds();
     }
 
     // Stage `nkb` Q8_1 blocks of each of M activation rows into LDS.

@@ -428,7 +428,7 @@ namespace llamql
     {
         if constexpr (F::USE_QUAD)
             return K / 256 >= QUAD_STEP_SB && gemv_unroll_override() == 0 && F::Quad::addressable(N, K / 256) &&
-                   quad_lds_bytes(M, K / 256) <= QUAD_MAX_LDS;
+                   quad_lds_bytes(M, K / 256) + F::Quad::STATIC_LDS <= QUAD_MAX_LDS;
         else
             return false;
     }
@@ -599,7 +599,7 @@ namespace llamql
                 a.y[i] = pr[j].y;
                 a.N[i] = pr[j].N;
                 a.ldy[i] = pr[j].ldy;
-                a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves).rows_per_wave;
+                a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves, F::Quad::RESIDENT_WAVES).rows_per_wave;
                 a.wave_begin[i] = (int)waves;
                 if (i < n)
                     waves += ((long)pr[j].N + a.R[i] - 1) / a.R[i];
@@ -616,7 +616,7 @@ namespace llamql
                 nw = 1;
             const long grid = (waves + nw - 1) / nw;
             size_t lds = quad_lds_bytes(M, SB);
-            a.ring = M == 1 && !d_sums && lds + (size_t)nw * QUAD_RING_BYTES <= QUAD_MAX_LDS;
+            a.ring = M == 1 && !d_sums && lds + (size_t)nw * QUAD_RING_BYTES + F::Quad::STATIC_LDS <= QUAD_MAX_LDS;
             if (a.ring)
                 lds += (size_t)nw * QUAD_RING_BYTES;
             gemv_quad_launch<typename F::Quad>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
@@ -736,7 +736,7 @@ namespace llamql
             if (SB >= QUAD_STEP_SB && gemv_unroll_override() == 0 && F::Quad::addressable(N, SB))
             {
                 p.kernel = GEMV_KERNEL_QUAD;
-                if (quad_lds_bytes(M, SB) > QUAD_MAX_LDS)
+                if (quad_lds_bytes(M, SB) + F::Quad::STATIC_LDS > QUAD_MAX_LDS)
                 {
                     if (M == 1)
                     {
@@ -745,7 +745,8 @@ namespace llamql
                     }
                     p.m_first = M / 2;
                 }
-                const QuadShape sh = gemv_quad_shape(N, SB, cu_count(device_id), F::Quad::max_threads(p.m_first) / WAVE);
+                const QuadShape sh = gemv_quad_shape(N, SB, cu_count(device_id), F::Quad::max_threads(p.m_first) / WAVE,
+                                                     F::Quad::RESIDENT_WAVES);
                 p.rows_per_wave = sh.rows_per_wave;
                 p.grid = sh.grid;
                 return p;

@@ -237,6 +237,9 @@ namespace llamql
     struct Q4KQuad
     {
         static constexpr int SB_BYTES = 144;
+        static constexpr int STATIC_LDS = 0;     // bytes of static LDS (decode tables) beside the activations
+        static constexpr int RESIDENT_WAVES = 8; // wavefronts per compute unit the launch shape aims at
+        __device__ __forceinline__ static void stage() {}
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         // workgroup size bound: one activation row leaves room for 16 wavefronts of 128 registers
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
@@ -425,6 +428,9 @@ namespace llamql
         typedef unsigned short v2s __attribute__((ext_vector_type(2)));
         typedef int v2i_ __attribute__((ext_vector_type(2)));
         static constexpr int LOADS = 5;
+        static constexpr int STATIC_LDS = 0;
+        static constexpr int RESIDENT_WAVES = 8;
+        __device__ __forceinline__ static void stage() {}
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
         static bool addressable(long N, int SB) { return (double)N * SB * 128.0 < 4.0e9; }
 
@@ -719,6 +725,7 @@ namespace llamql
             load_chunk(bufB);
             quad_stage_f32<Q, M, SRC>(qa.x, qa.x2, qa.ldx, nsb, aq, ads, aq_stride, ads_stride);
         }
+        Q::stage(); // the format's decode tables, if it has any
         __syncthreads();
         // the staging code above must not reuse the registers of the loads in flight
 #pragma unroll
@@ -901,7 +908,8 @@ namespace llamql
     inline void gemv_quad_launch_mus(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
         static LdsGrant grant;
-        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC, MODE>), QUAD_MAX_LDS);
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_quad_kernel<Q, M, U, SRC, MODE>),
+                        QUAD_MAX_LDS - Q::STATIC_LDS);
         hipLaunchKernelGGL((gemv_quad_kernel<Q, M, U, SRC, MODE>), grid, block, lds, st, a);
     }
 
@@ -1031,20 +1039,23 @@ namespace llamql
         int waves, rows_per_wave;
         long grid;
     };
-    inline QuadShape gemv_quad_shape(long N, int nsb, int cus, int max_waves)
+    // resident: wavefronts a compute unit should hold at once (8 for the memory-bound decoders:
+    // two per SIMD unit; 16 for the arithmetic-bound one)
+    inline QuadShape gemv_quad_shape(long N, int nsb, int cus, int max_waves, int resident = 8)
     {
         const int rpw_override = gemv_rows_per_wave_override();
         // the search below costs a microsecond or two: remember the last answers
         struct Memo
         {
             long N;
-            int nsb, cus, max_waves, rpw;
+            int nsb, cus, max_waves, resident, rpw;
             QuadShape sh;
         };
         thread_local Memo memo[16] = {};
         thread_local int memo_next = 0;
         for (const Memo &e : memo)
-            if (e.N == N && e.nsb == nsb && e.cus == cus && e.max_waves == max_waves && e.rpw == rpw_override)
+            if (e.N == N && e.nsb == nsb && e.cus == cus && e.max_waves == max_waves && e.resident == resident &&
+                e.rpw == rpw_override)
                 return e.sh;
         int best_R = 1;
         long best_wpc = 1;
@@ -1056,14 +1067,17 @@ namespace llamql
             const long steps = ((long)R * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
             const long waves = (N + R - 1) / R;
             const long wpc = (waves + cus - 1) / cus; // wavefronts on the busiest compute unit
-            // at most 8 wavefronts of the widest variant fit a compute unit at once
-            const long rounds = (wpc + 7) / 8;
-            const long per_simd = rounds > 1 ? 2 * rounds : (wpc + 3) / 4;
+            // at most `resident` wavefronts of the widest variant fit a compute unit at once
+            const long rounds = (wpc + resident - 1) / resident;
+            const long per_simd = rounds > 1 ? (resident / 4) * rounds : (wpc + 3) / 4;
             double cost = (double)(per_simd * steps) / ((double)N * nsb / cus / (4.0 * QUAD_STEP_SB));
             if (wpc < 4)
                 cost *= 1.0 + 0.25 * (double)(4 - wpc); // too few loads in flight
-            else if (wpc < 8)
+            else if (resident <= 8 && wpc < 8)
                 cost *= 1.10;                           // one wavefront cannot keep a SIMD unit busy
+            if (resident > 8 && wpc <= 4)
+                cost *= 1.28; // arithmetic-bound decoder: a lone wavefront leaves its SIMD unit idle
+                              // while it waits (measured: 24.3 against 19.2 us at two per unit)
             if (steps < 4)
                 cost *= 1.0 + 0.10 * (double)(4 - steps); // short runs do not amortise their start
             if (cost < best_cost - 1e-9)
@@ -1084,7 +1098,7 @@ namespace llamql
             nw = waves;
         sh.waves = (int)(nw < 1 ? 1 : nw);
         sh.grid = (waves + sh.waves - 1) / sh.waves;
-        memo[memo_next] = Memo{N, nsb, cus, max_waves, rpw_override, sh};
+        memo[memo_next] = Memo{N, nsb, cus, max_waves, resident, rpw_override, sh};
         memo_next = (memo_next + 1) % 16;
         return sh;
     }

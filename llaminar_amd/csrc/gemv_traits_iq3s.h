@@ -1,4 +1,5 @@
-// IQ3_S x Q8_1 decode GEMV for gfx950: format traits for the shared skeleton.
+// IQ3_S x Q8_1 decode GEMV for gfx950: format traits for the shared skeleton and the
+// quad-lane decoder.
 //
 // The reference's CPU path REQUANTISES every 32-element IQ3_S sub-block to int8
 // at pack time (src/v2/tensors/SIMDHelpers.h:8612-8768): codebook magnitudes
@@ -6,23 +7,29 @@
 // w = rne(v/scale).  Because v = +-g*db with one db per sub-block this is the pure
 // integer map  w = +-round(g*127/gmax)  (gmax = largest magnitude in the
 // sub-block; never a tie) with  b_scale = f16((gmax*db)/127).  Every magnitude is odd,
-// g = 2k+1 with k in 0..7, so for a given gmax the map is an 8-entry byte table.  The kernel
-// keeps in LDS (4.6 KB): the codebook as k-bytes (2 KB), the eight maps, and a 256-entry table
-// that turns eight sign bits into two byte masks; a sub-block costs eight codebook gathers,
-// one map fetch and four sign-mask gathers, and per four weights one v_perm_b32 (map), one
-// subtraction (bytewise negation: every magnitude is 1..127) and one v_bfi_b32 (signs).
-// Which map a sub-block needs -- its gmax -- is worked out when the weights are prepared and
-// kept as a two-bit hint per sub-block in the two spare bytes of the super-block's meta
-// record: 0, 1, 2 mean gmax 15, 13, 11 (93 %, 6 % and 1 % of sub-blocks with uniform codebook
-// indices); 3 means "smaller": those few look their entries' maxima up in a byte table.  HBM
+// g = 2k+1 with k in 0..7, so for a given gmax the map is an 8-entry byte table.  The kernels
+// keep in (static) LDS, 4.6 KB: the codebook as k-bytes (2 KB), the maps, and a 256-entry
+// table that turns eight sign bits into two byte masks; a sub-block costs eight codebook
+// gathers, one map fetch and four sign-mask gathers, and per four weights one v_perm_b32
+// (map), one subtraction (bytewise negation: every magnitude is 1..127) and one v_bfi_b32
+// (signs).
+//
+// What a sub-block needs beyond its bytes is worked out when the weights are prepared and kept
+// as a two-bit hint per sub-block in the two spare bytes of the super-block's meta record:
+// 0, 1, 2 mean "regular, gmax 15, 13, 11" (93 %, 6 % and 1 % of sub-blocks with uniform
+// codebook indices), where regular says that the scale is an ordinary fp16 number, so that the
+// decoder needs no test for zero, overflow, subnormal or non-finite scales; 3 means "anything
+// else": those few take the general path (maxima from a byte table, every special case).  HBM
 // traffic stays at the format's 110 B per 256 weights (+2 B alignment padding, which now
 // carries the hints).
 //
 // Device layout (llam_ql_prepare_weights): three planes over T = N*K/256
 // super-blocks -- qs [T][64], signs [T][32], meta [T][16] = qh[8] scales[4] d[2]
-// hints[2].  Lane c of an 8-lane group owns sub-block c.
+// hints[2].  In the shared skeleton lane c of an 8-lane group owns sub-block c; in the
+// quad-lane kernel lane l of a quad owns sub-blocks 2l and 2l+1.
 #pragma once
 #include "gemv_core.h"
+#include "gemv_quad.h"
 #include <cstddef>
 
 #define LLAM_IQ3S_GRID_QUALIFIER static constexpr
@@ -32,12 +39,16 @@ namespace llamql
 {
     struct IQ3STables
     {
-        uint32_t cb[512];    // codebook entry idx as bytes k = g >> 1
-        uint8_t cbmax[512];  // the entry's largest k
-        uint32_t map[8][2];  // map[gi]: bytes round((2k+1)*127/(2*gi+1)) for k = 0..7 (k > gi is never looked up)
+        uint32_t cb[512];     // codebook entry idx as bytes k = g >> 1
+        uint8_t cbmax[512];   // the entry's largest k
+        uint32_t map[10][2];  // map[7 - gi]: bytes round((2k+1)*127/(2*gi+1)) for k = 0..7 (k > gi is never
+                              // looked up); map[8], map[9]: zeros (an all-zero sub-block)
         uint32_t sgn[256][2]; // eight sign bits -> 0xFF bytes where the bit is set: elements 0-3, 4-7
-        bool odd;            // every codebook magnitude is odd and at most 15
+        bool odd;             // every codebook magnitude is odd and at most 15
     };
+    constexpr int IQ3S_TABLE_BYTES = 2048 + 512 + 80 + 2048;
+    constexpr int IQ3S_OFF_CBMAX = 2048, IQ3S_OFF_MAP = 2560, IQ3S_OFF_SGN = 2640;
+    constexpr uint32_t IQ3S_MAP_ZERO = 8; // index of the all-zero map
 
     constexpr IQ3STables make_iq3s_tables()
     {
@@ -69,7 +80,7 @@ namespace llamql
                 uint32_t q = (2u * g * 127u + gm) / (2u * gm); // round half up; never exactly half
                 if (q > 127u)
                     q = 127u; // g > gm: never looked up
-                t.map[gi][k >> 2] |= q << (8 * (k & 3));
+                t.map[7 - gi][k >> 2] |= q << (8 * (k & 3));
             }
         }
         for (int s8 = 0; s8 < 256; ++s8)
@@ -79,22 +90,28 @@ namespace llamql
         return t;
     }
     static_assert(make_iq3s_tables().odd, "IQ3_S codebook magnitudes must be odd and at most 15");
+    static_assert(offsetof(IQ3STables, cbmax) == IQ3S_OFF_CBMAX && offsetof(IQ3STables, map) == IQ3S_OFF_MAP &&
+                      offsetof(IQ3STables, sgn) == IQ3S_OFF_SGN && offsetof(IQ3STables, odd) == IQ3S_TABLE_BYTES &&
+                      IQ3S_TABLE_BYTES % 16 == 0,
+                  "table offsets the decoder assumes");
 
     static __device__ const IQ3STables g_iq3s_tables = make_iq3s_tables();
 
-    // The gmax hint of a sub-block (two bits): the largest k of its eight codebook entries as
-    // 7 - k for k = 7, 6, 5, and 3 for anything smaller.
-    constexpr uint32_t IQ3S_HINT_OTHER = 3;
-    __device__ __forceinline__ uint32_t iq3s_gmax_hint(const uint8_t *qs8, uint32_t qh)
+    // The tables' place in LDS: a static array, so that its address is a link-time constant and
+    // every look-up is a ds_read with an immediate offset.  Every kernel that decodes IQ3_S
+    // fills it (iq3s_stage_tables) before its first barrier.
+    __device__ __forceinline__ uint8_t *iq3s_tables_lds()
     {
-        uint32_t mx = 0;
-#pragma unroll
-        for (int l = 0; l < 8; ++l)
-        {
-            const uint32_t k = g_iq3s_tables.cbmax[qs8[l] | (((qh >> l) & 1u) << 8)];
-            mx = k > mx ? k : mx;
-        }
-        return mx >= 5u ? 7u - mx : IQ3S_HINT_OTHER;
+        __shared__ __attribute__((aligned(16))) uint8_t iq3s_tables[IQ3S_TABLE_BYTES];
+        return iq3s_tables;
+    }
+    __device__ __forceinline__ void iq3s_stage_tables()
+    {
+        const uint4 *src = reinterpret_cast<const uint4 *>(&g_iq3s_tables);
+        uint4 *dst = reinterpret_cast<uint4 *>(iq3s_tables_lds());
+        constexpr int n = IQ3S_TABLE_BYTES / 16;
+        for (int i = threadIdx.x; i < n; i += blockDim.x)
+            dst[i] = src[i];
     }
 
     // (byte N of x) << sh in one instruction (sub-dword addressing of the operand).  sh is a
@@ -114,26 +131,243 @@ namespace llamql
         return r;
     }
 
+    // The general scale of a sub-block whose largest codebook byte is km: amax = gmax * (d * (1 + 2 nib))
+    // is exact in fp32 (11 x 5 x 4 bits), so is d * (gmax * (1 + 2 nib)).  Returns the scale before
+    // its fp16 rounding; 0 for a sub-block the packer treats as all zero.
+    __device__ __forceinline__ float iq3s_scale_general(float d, uint32_t km, uint32_t nib)
+    {
+        const float amax = d * (float)((2u * km + 1u) * (2u * nib + 1u));
+        float scale = div_by_127(amax);
+        if (scale > 65504.0f)
+            scale = 65504.0f;
+        if (amax < 1e-6f)
+            scale = 0.0f;
+        return scale;
+    }
+
+    // The hint of a sub-block (two bits), worked out when the weights are prepared.
+    constexpr uint32_t IQ3S_HINT_OTHER = 3;
+    __device__ __forceinline__ uint32_t iq3s_block_hint(const uint8_t *qs8, uint32_t qh, uint32_t nib, float d)
+    {
+        uint32_t mx = 0;
+#pragma unroll
+        for (int l = 0; l < 8; ++l)
+        {
+            const uint32_t k = g_iq3s_tables.cbmax[qs8[l] | (((qh >> l) & 1u) << 8)];
+            mx = k > mx ? k : mx;
+        }
+        if (mx < 5u)
+            return IQ3S_HINT_OTHER;
+        // regular: a positive scale inside the normal fp16 range (which excludes zeros, clamped,
+        // subnormal-after-rounding and non-finite scales; a NaN fails both comparisons)
+        const float scale = iq3s_scale_general(d, mx, nib);
+        const bool regular = scale >= 6.103515625e-05f && scale < 65504.0f;
+        return regular ? 7u - mx : IQ3S_HINT_OTHER;
+    }
+
+    // One 32-element sub-block to int8 weights and its scale.
+    //   qs: the eight low index bytes; qh: bit l is the ninth bit of index l (bits above 7 are ignored);
+    //   nib: the 4-bit sub-block scale; hint: see above; signs: the 32 sign bits; d: the super-block scale
+    __device__ __forceinline__ void iq3s_decode_block(const uint2 qs, const uint32_t qh, const uint32_t nib,
+                                                      const uint32_t hint, const float d, const uint32_t signs,
+                                                      v4i &w0, v4i &w1, float &bscale)
+    {
+        const uint8_t *tab = iq3s_tables_lds();
+
+        // byte offsets of the eight codebook entries: (qs byte l) * 4 + (bit l of qh) * 1024
+        uint32_t off[8];
+        {
+            const uint32_t two = 2u;
+            const uint32_t a[8] = {byte_shl<0>(qs.x, two), byte_shl<1>(qs.x, two), byte_shl<2>(qs.x, two),
+                                   byte_shl<3>(qs.x, two), byte_shl<0>(qs.y, two), byte_shl<1>(qs.y, two),
+                                   byte_shl<2>(qs.y, two), byte_shl<3>(qs.y, two)};
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+                off[l] = ((qh << (10 - l)) & 0x400u) | a[l]; // v_lshlrev_b32 + v_and_or_b32
+        }
+        uint32_t e[8];
+#pragma unroll
+        for (int l = 0; l < 8; ++l)
+            e[l] = *reinterpret_cast<const uint32_t *>(tab + off[l]);
+
+        // regular sub-block: gmax = 15 - 2 hint; scale = f16(d * gmax * (1 + 2 nib) / 127), finite,
+        // not zero and a normal fp16 number, so nearest-even is the packer's rounding
+        uint32_t mi = hint; // which map
+        uint32_t sg_all = signs;
+        {
+            const float amax = d * (float)((15u - 2u * hint) * (2u * nib + 1u));
+            const float c = 0x1.020408p-7f;
+            const float q0 = amax * c;
+            const float q1 = fmaf(fmaf(-q0, 127.0f, amax), c, q0); // div_by_127 of a finite non-zero value
+            bscale = __half2float(__float2half_rn(q1));
+        }
+        if (__builtin_expect(hint == IQ3S_HINT_OTHER, 0))
+        {
+            // 3 in 10000 with uniform indices: largest magnitude 9 or less, or a special scale
+            uint32_t km = 0;
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+                km = max(km, (uint32_t)tab[IQ3S_OFF_CBMAX + (off[l] >> 2)]);
+            const float scale = iq3s_scale_general(d, km, nib);
+            bscale = f16_round_packer(scale);
+            mi = 7u - km;
+            if (scale == 0.0f) // all-zero sub-block: zero magnitudes, and no sign to apply to them
+            {
+                mi = IQ3S_MAP_ZERO;
+                sg_all = 0u;
+            }
+        }
+        const uint2 mp = *reinterpret_cast<const uint2 *>(tab + IQ3S_OFF_MAP + mi * 8u);
+
+        int ws[8];
+        {
+            const uint8_t *sgb = tab + IQ3S_OFF_SGN;
+            const uint32_t three = 3u;
+            // byte masks of elements 8p..8p+3 (x) and 8p+4..8p+7 (y)
+            const uint2 sm[4] = {*reinterpret_cast<const uint2 *>(sgb + byte_shl<0>(sg_all, three)),
+                                 *reinterpret_cast<const uint2 *>(sgb + byte_shl<1>(sg_all, three)),
+                                 *reinterpret_cast<const uint2 *>(sgb + byte_shl<2>(sg_all, three)),
+                                 *reinterpret_cast<const uint2 *>(sgb + byte_shl<3>(sg_all, three))};
+#pragma unroll
+            for (int l = 0; l < 8; ++l)
+            {
+                const uint32_t w = __builtin_amdgcn_perm(mp.y, mp.x, e[l]);
+                const uint32_t neg = 0x01010100u - w; // bytewise -w: every byte of w is in 1..127 (or all are 0)
+                const uint32_t mask = (l & 1) ? sm[l >> 1].y : sm[l >> 1].x;
+                ws[l] = (int)((neg & mask) | (w & ~mask)); // v_bfi_b32
+            }
+        }
+        w0 = (v4i){ws[0], ws[1], ws[2], ws[3]};
+        w1 = (v4i){ws[4], ws[5], ws[6], ws[7]};
+    }
+
+    // ---- quad-lane decoder -------------------------------------------------------------
+    // Lane l of a quad decodes sub-blocks 2l and 2l+1: 16 bytes of qs, 8 of signs, and the
+    // super-block's meta record (the four lanes ask for the same 16 bytes).  Weight addresses
+    // are 32-bit offsets from the plane bases.
+    struct IQ3SQuad
+    {
+        typedef int v2i_ __attribute__((ext_vector_type(2)));
+        static constexpr int LOADS = 3;
+        static constexpr int STATIC_LDS = IQ3S_TABLE_BYTES;
+        // 16 wavefronts of 128 registers for a single activation row
+        static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
+        // the decoder is arithmetic-bound: a compute unit should hold 16 wavefronts
+        static constexpr int RESIDENT_WAVES = 16;
+        static bool addressable(long N, int SB) { return (double)N * SB * 64.0 < 4.0e9; }
+        __device__ __forceinline__ static void stage() { iq3s_stage_tables(); }
+
+        struct Raw
+        {
+            v4i qs, meta;
+            v2i_ sg;
+        };
+        struct Lane
+        {
+            uint32_t l;
+            uint32_t qh_sel; // v_perm selector: qh bytes 2l and 2l+1 of {meta.x, meta.y} into bits 0-7 and 16-23
+        };
+        struct Scale
+        {
+            float bs0, bs1;
+        };
+        struct Cursor
+        {
+            const uint8_t *qs, *sg, *meta; // plane bases (uniform)
+            uint32_t t, first;             // this lane's super-block index: current, and the one read
+                                           // instead past the end of the run
+        };
+
+        __device__ __forceinline__ static Lane lane_consts(int l)
+        {
+            Lane c;
+            c.l = (uint32_t)l;
+            const uint32_t b = 2u * (uint32_t)l;
+            c.qh_sel = b | (0x0Cu << 8) | ((b + 1u) << 16) | (0x0Cu << 24);
+            return c;
+        }
+        __device__ __forceinline__ static void owner(int j, int &l, int &which)
+        {
+            l = j >> 1;
+            which = j & 1;
+        }
+        __device__ __forceinline__ static int block_of(int l, int which) { return 2 * l + which; }
+
+        __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, size_t t_safe, const Lane &)
+        {
+            const size_t T = (size_t)a.N * a.SB;
+            Cursor c;
+            c.qs = static_cast<const uint8_t *>(a.w);
+            c.sg = c.qs + T * 64;
+            c.meta = c.qs + T * 96;
+            c.t = (uint32_t)t;
+            c.first = (uint32_t)t_safe;
+            return c;
+        }
+        __device__ __forceinline__ static void advance(Cursor &c, int steps) { c.t += (uint32_t)(steps * QUAD_STEP_SB); }
+        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, int step, bool valid)
+        {
+            load_index(r, c, lc, valid ? c.t + (uint32_t)(step * QUAD_STEP_SB) : c.first);
+        }
+        __device__ __forceinline__ static void load_at(Raw &r, const Cursor &c, const Lane &lc, int sb_off)
+        {
+            load_index(r, c, lc, c.t + (uint32_t)sb_off);
+        }
+        // Loads issued as assembly so that the kernel decides where they are waited for.
+        __device__ __forceinline__ static void load_index(Raw &r, const Cursor &c, const Lane &lc, uint32_t t)
+        {
+            const uint32_t oqs = t * 64u + lc.l * 16u, osg = t * 32u + lc.l * 8u, om = t * 16u;
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qs) : "v"(oqs), "s"(c.qs));
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.meta) : "v"(om), "s"(c.meta));
+            asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(r.sg) : "v"(osg), "s"(c.sg));
+        }
+        __device__ __forceinline__ static void keep(Raw &r)
+        {
+            asm volatile("" : "+v"(r.qs), "+v"(r.meta), "+v"(r.sg));
+        }
+        template <int NEWER>
+        __device__ __forceinline__ static void wait(Raw &r)
+        {
+            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r.qs), "+v"(r.meta), "+v"(r.sg) : "n"(NEWER));
+        }
+
+        // w[0], w[1]: elements 0-15, 16-31 of sub-block 2l; w[2], w[3]: of sub-block 2l+1.
+        __device__ __forceinline__ static void decode(const Raw &r, const Lane &lc, v4i (&w)[4], Scale &S)
+        {
+            const uint32_t qh2 = __builtin_amdgcn_perm((uint32_t)r.meta.y, (uint32_t)r.meta.x, lc.qh_sel);
+            const uint32_t nibs = ((uint32_t)r.meta.z >> (8u * lc.l)); // scales[l]: low nibble 2l, high nibble 2l+1
+            const uint32_t hints = ((uint32_t)r.meta.w >> (16u + 4u * lc.l));
+            const float d = h2f((uint16_t)((uint32_t)r.meta.w & 0xFFFFu));
+            iq3s_decode_block(make_uint2((uint32_t)r.qs.x, (uint32_t)r.qs.y), qh2, nibs & 0xFu, hints & 3u, d,
+                              (uint32_t)r.sg.x, w[0], w[1], S.bs0);
+            iq3s_decode_block(make_uint2((uint32_t)r.qs.z, (uint32_t)r.qs.w), qh2 >> 16, (nibs >> 4) & 0xFu,
+                              (hints >> 2) & 3u, d, (uint32_t)r.sg.y, w[2], w[3], S.bs1);
+        }
+
+        __device__ __forceinline__ static float scale_f32(const Scale &S, int i) { return i ? S.bs1 : S.bs0; }
+        __device__ __forceinline__ static float min_f32(const Scale &, int) { return 0.0f; }
+
+        // the format has no block minimum
+        __device__ __forceinline__ static float apply(const Scale &S, int idot0, int idot1, const float4 sd, float acc)
+        {
+            acc = fmaf((float)idot0, sd.x * S.bs0, acc);
+            acc = fmaf((float)idot1, sd.z * S.bs1, acc);
+            return acc;
+        }
+    };
+
     struct IQ3STraits
     {
         static constexpr bool PAIR = false;
         static constexpr bool HAS_MIN = false;
-        static constexpr bool USE_QUAD = false;
+        static constexpr bool USE_QUAD = true;         // quad-lane kernel for rows of >= 16 super-blocks
         static constexpr bool USE_MFMA_BATCH = false;  // matrix-unit kernel for 5..8 activation rows
+        typedef IQ3SQuad Quad;
         static constexpr int FAST_MAX_U = 3;          // load batches in flight in the chunked kernel
-        static constexpr int TABLE_BYTES = 2048 + 512 + 64 + 2048; // cb, cbmax, map, sgn
+        static constexpr int TABLE_BYTES = IQ3S_TABLE_BYTES;
 
-        __device__ static void stage_tables(void *lds_tab)
-        {
-            static_assert(offsetof(IQ3STables, cbmax) == 2048 && offsetof(IQ3STables, map) == 2560 &&
-                              offsetof(IQ3STables, sgn) == 2624 && offsetof(IQ3STables, odd) == TABLE_BYTES,
-                          "table offsets the decoder assumes");
-            const uint4 *src = reinterpret_cast<const uint4 *>(&g_iq3s_tables);
-            uint4 *dst = static_cast<uint4 *>(lds_tab);
-            constexpr int n = TABLE_BYTES / 16;
-            for (int i = threadIdx.x; i < n; i += blockDim.x)
-                dst[i] = src[i];
-        }
+        __device__ static void *tables_lds() { return iq3s_tables_lds(); }
+        __device__ static void stage_tables(void *) { iq3s_stage_tables(); }
 
         struct Raw // no padding between members: arrays of it stay in registers
         {
@@ -171,85 +405,17 @@ namespace llamql
         }
 
         __device__ __forceinline__ static void decode(const Raw &r, int c, v4i &w0, v4i &w1, int &j,
-                                                      float &bscale, float &bmin, const void *tab)
+                                                      float &bscale, float &bmin, const void *)
         {
-            const uint32_t *cb = static_cast<const uint32_t *>(tab);
-            const uint8_t *cbmax = static_cast<const uint8_t *>(tab) + 2048;
-            const uint2 *maps = reinterpret_cast<const uint2 *>(static_cast<const uint8_t *>(tab) + 2560);
-            const uint2 *sgn = reinterpret_cast<const uint2 *>(static_cast<const uint8_t *>(tab) + 2624);
-
             // picked with a bit mask: a conditional on two members of r would become a load
             // through a computed address and force arrays of Raw into memory
             const uint32_t m4 = (uint32_t)0 - (uint32_t)((c >> 2) & 1);
-            const uint32_t qh = ((((r.meta.y & m4) | (r.meta.x & ~m4))) >> (8 * (c & 3))) & 0xFFu;
+            const uint32_t qh = (((r.meta.y & m4) | (r.meta.x & ~m4))) >> (8 * (c & 3));
             const uint32_t nib = (r.meta.z >> (4 * c)) & 0xFu; // scales[c/2], low nibble for even c
             const float d = h2f((uint16_t)(r.meta.w & 0xFFFFu));
             const uint32_t hint = (r.meta.w >> (16 + 2 * c)) & 3u;
-
-            // byte offsets of the eight codebook entries: (qs byte l) * 4 + (bit l of qh) * 1024
-            const uint8_t *cbb = static_cast<const uint8_t *>(tab);
-            uint32_t off[8];
-            {
-                const uint32_t two = 2u;
-                const uint32_t a0 = byte_shl<0>(r.qs.x, two), a1 = byte_shl<1>(r.qs.x, two), a2 = byte_shl<2>(r.qs.x, two),
-                               a3 = byte_shl<3>(r.qs.x, two), a4 = byte_shl<0>(r.qs.y, two), a5 = byte_shl<1>(r.qs.y, two),
-                               a6 = byte_shl<2>(r.qs.y, two), a7 = byte_shl<3>(r.qs.y, two);
-                const uint32_t a[8] = {a0, a1, a2, a3, a4, a5, a6, a7};
-#pragma unroll
-                for (int l = 0; l < 8; ++l)
-                    off[l] = (((qh >> l) & 1u) << 10) | a[l]; // v_bfe_u32 + v_lshl_or_b32
-            }
-            uint32_t e[8];
-#pragma unroll
-            for (int l = 0; l < 8; ++l)
-                e[l] = *reinterpret_cast<const uint32_t *>(cbb + off[l]);
-            uint32_t km = 7u - hint;
-            if (__builtin_expect(hint == IQ3S_HINT_OTHER, 0))
-            {
-                // a sub-block whose largest magnitude is 9 or less (3 in 10000 with uniform indices)
-                km = 0;
-#pragma unroll
-                for (int l = 0; l < 8; ++l)
-                    km = max(km, (uint32_t)cbmax[off[l] >> 2]);
-            }
-
-            // amax = gmax * (d * (1 + 2 nib)) is exact in fp32 (11 x 5 x 4 bits), so is d * (gmax * (1 + 2 nib))
-            const float amax = d * (float)((2u * km + 1u) * (2u * nib + 1u));
-            float scale = div_by_127(amax);
-            if (scale > 65504.0f)
-                scale = 65504.0f;
-            if (amax < 1e-6f)
-                scale = 0.0f;
-
-            uint2 mp = maps[km];
-            uint32_t sg_all = r.signs;
-            if (scale == 0.0f) // all-zero sub-block: zero magnitudes, and no sign to apply to them
-            {
-                mp = make_uint2(0u, 0u);
-                sg_all = 0u;
-            }
-            int ws[8];
-            {
-                const uint8_t *sgb = reinterpret_cast<const uint8_t *>(sgn);
-                const uint32_t three = 3u;
-                // byte masks of elements 8p..8p+3 (x) and 8p+4..8p+7 (y)
-                const uint2 sm[4] = {*reinterpret_cast<const uint2 *>(sgb + byte_shl<0>(sg_all, three)),
-                                     *reinterpret_cast<const uint2 *>(sgb + byte_shl<1>(sg_all, three)),
-                                     *reinterpret_cast<const uint2 *>(sgb + byte_shl<2>(sg_all, three)),
-                                     *reinterpret_cast<const uint2 *>(sgb + byte_shl<3>(sg_all, three))};
-#pragma unroll
-                for (int l = 0; l < 8; ++l)
-                {
-                    const uint32_t w = __builtin_amdgcn_perm(mp.y, mp.x, e[l]);
-                    const uint32_t neg = 0x01010100u - w; // bytewise -w: every byte of w is in 1..127 (or all are 0)
-                    const uint32_t mask = (l & 1) ? sm[l >> 1].y : sm[l >> 1].x;
-                    ws[l] = (int)((neg & mask) | (w & ~mask)); // v_bfi_b32
-                }
-            }
-            w0 = (v4i){ws[0], ws[1], ws[2], ws[3]};
-            w1 = (v4i){ws[4], ws[5], ws[6], ws[7]};
+            iq3s_decode_block(r.qs, qh, nib, hint, d, r.signs, w0, w1, bscale);
             j = c;
-            bscale = f16_round_packer(scale);
             bmin = 0.0f;
         }
 

@@ -25,6 +25,7 @@ namespace llamql
         typedef Q4KQuad Quad;
         static constexpr int FAST_MAX_U = 4;          // load batches in flight in the chunked kernel
         static constexpr int TABLE_BYTES = 0;
+        __device__ static void *tables_lds() { return nullptr; }
         __device__ static void stage_tables(void *) {}
 
         struct Raw

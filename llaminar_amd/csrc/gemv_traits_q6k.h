@@ -54,6 +54,7 @@ namespace llamql
         typedef Q6KQuad Quad;
         static constexpr int FAST_MAX_U = 1;          // load batches in flight in the chunked kernel
         static constexpr int TABLE_BYTES = 0;
+        __device__ static void *tables_lds() { return nullptr; }
         __device__ static void stage_tables(void *) {}
 
         struct Raw

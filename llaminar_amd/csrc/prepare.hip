@@ -7,7 +7,8 @@
 //           | pad to 16 | factors [T][8] x 4 B (q6k_block_code, ql_device.h)    (T*32 B)
 //   IQ3_S : planes qs [T][64] | signs [T][32] | meta [T][16]                   (T*112 B)
 //           meta = qh[8] scales[4] d[2] hints[2]: two bits per 32-element block, which of the
-//           requantisation maps the block needs (its largest codebook magnitude; iq3s_gmax_hint)
+//           requantisation maps the block needs (its largest codebook magnitude) when its scale is
+//           an ordinary fp16 number, else "take the general path" (iq3s_block_hint)
 // with T = N*K/256 super-blocks in row-major order.  Raw Q6_K / IQ3_S blocks are
 // 210 / 110 bytes, i.e. only 2-byte aligned, so the copy works in halfwords.
 #include "gemv_traits_iq3s.h"
@@ -69,9 +70,13 @@ namespace llamql
         {
             o = T * 48 + t * 8 + 7; // hints: block j in bits 2j, 2j+1
             const uint8_t *blk = reinterpret_cast<const uint8_t *>(src + t * 55); // d[2] qs[64] qh[8] signs[32] scales[4]
+            const float d = h2f((uint16_t)(blk[0] | (blk[1] << 8)));
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                v |= (uint16_t)(iq3s_gmax_hint(blk + 2 + 8 * j, blk[66 + j]) << (2 * j));
+            {
+                const uint32_t nib = ((uint32_t)blk[106 + (j >> 1)] >> (4 * (j & 1))) & 0xFu;
+                v |= (uint16_t)(iq3s_block_hint(blk + 2 + 8 * j, blk[66 + j], nib, d) << (2 * j));
+            }
         }
         else
         {

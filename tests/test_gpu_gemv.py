@@ -151,14 +151,14 @@ def test_fused_projections(capi, dev, oracle):
 def test_fused_groups_equal_separate_calls(capi, dev, M):
     """Neighbouring projections of one format share a launch; every output must carry the
     bits of its own llam_ql_gemv call.  Groups here: five Q4_K (four + one, the last joined by
-    two Q6_K in a two-format launch), an IQ3_S (never grouped), a Q4_K again, and a Q4_K of
+    two Q6_K in a two-format launch), two IQ3_S (one launch), a Q4_K again, and a Q4_K of
     4096 rows, which from batch 5 on runs alone on the matrix unit; ragged N, a strided output."""
     import torch
 
     K = 5120
     qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(8, K, 23)).to(dev))
     specs = [(FMT_Q4_K, 700), (FMT_Q4_K, 37), (FMT_Q4_K, 1), (FMT_Q4_K, 2048), (FMT_Q4_K, 129),
-             (FMT_Q6_K, 300), (FMT_Q6_K, 64), (FMT_IQ3_S, 96), (FMT_Q4_K, 250), (FMT_Q4_K, 4096), (FMT_Q6_K, 40)]
+             (FMT_Q6_K, 300), (FMT_Q6_K, 64), (FMT_IQ3_S, 96), (FMT_IQ3_S, 33), (FMT_Q4_K, 250), (FMT_Q4_K, 4096), (FMT_Q6_K, 40)]
     total = sum(n for _, n in specs)
     out = torch.full((M, total + 5), float("nan"), device=dev)
     projs, singles, col = [], [], 0
@@ -177,8 +177,8 @@ def test_fused_groups_equal_separate_calls(capi, dev, M):
 @pytest.mark.parametrize("M", [1, 3, 8])
 def test_fp32_input_equals_quantise_then_gemv(capi, dev, M):
     """llam_ql_gemv_f32 / _fused_f32 / _swiglu_f32 quantise inside the kernel: bits of the
-    two-step path, for kernels that quantise themselves (Q4_K, Q6_K, K >= 4096), for the ones
-    that need the scratch buffer (IQ3_S, short K), with padded input rows, and with tiny
+    two-step path, for kernels that quantise themselves (K >= 4096), for the ones
+    that need the scratch buffer (short K), with padded input rows, and with tiny
     and zero blocks in the input."""
     import torch
 
@@ -204,15 +204,15 @@ def test_fp32_input_equals_quantise_then_gemv(capi, dev, M):
             ref = capi.gemv(fmt, wd, qd, M, N, K)
             ref_s = capi.gemv(fmt, wd, qa, M, N, K)
             # with a scratch buffer the library picks the cheaper way; without one the kernel
-            # has to quantise for itself, which IQ3_S and short rows cannot
-            for sc in (scratch, None) if (fmt != FMT_IQ3_S and K >= 4096) else (scratch,):
+            # has to quantise for itself, which short rows cannot
+            for sc in (scratch, None) if K >= 4096 else (scratch,):
                 assert torch.equal(capi.gemv_f32(fmt, wd, x, M, N, K, q8_scratch=sc), ref), (K, fmt, "f32")
                 assert torch.equal(capi.gemv_swiglu_f32(fmt, wd, g, x, M, N, K, q8_scratch=sc), ref_s), (K, fmt)
             col += N
         if K >= 4096:
-            capi.gemv_fused_f32(projs[:3], x, M, K)  # no scratch: one launch per format group
+            capi.gemv_fused_f32(projs[:4], x, M, K)  # no scratch: one launch per format group
             col = 0
-            for (fmt, N), (_, wd, _) in zip(specs[:3], projs[:3]):
+            for (fmt, N), (_, wd, _) in zip(specs[:4], projs[:4]):
                 assert torch.equal(out[:, col:col + N], capi.gemv(fmt, wd, qd, M, N, K)), (K, fmt, "fused/self")
                 col += N
             out.fill_(float("nan"))
@@ -292,17 +292,23 @@ def test_prepare_moves_every_byte(capi, dev, oracle, fmt):
         assert np.array_equal(meta[:, 0:8], B[:, 66:74])
         assert np.array_equal(meta[:, 8:12], B[:, 106:110])
         assert np.array_equal(meta[:, 12:14], B[:, 0:2])
-        # the two spare bytes carry the gmax hints: two bits per 32-element block, 7 - k for the
-        # block's largest codebook magnitude 2k+1 when k >= 5, else 3
+        # the two spare bytes carry the hints: two bits per 32-element block, 7 - k for the block's
+        # largest codebook magnitude 2k+1 when k >= 5 and the block's scale is an ordinary fp16
+        # number (normal, below the clamp), else 3
         grid = np.load(GOLDEN_PATH, allow_pickle=False)["iq3s_grid"].astype(np.uint32).reshape(-1)[:512]
         kmax = np.max(np.stack([(grid >> (8 * b)) & 0xFF for b in range(4)]), axis=0) >> 1
         hints = meta[:, 14].astype(np.uint32) | (meta[:, 15].astype(np.uint32) << 8)
         for t in range(T):
             qs, qh = B[t, 2:66].astype(np.uint32), B[t, 66:74].astype(np.uint32)
+            d = np.float32(B[t, 0:2].view(np.float16)[0])
             for j in range(8):
                 idx = qs[8 * j:8 * j + 8] | (((qh[j] >> np.arange(8)) & 1) << 8)
                 k = int(kmax[idx].max())
-                assert (int(hints[t]) >> (2 * j)) & 3 == (7 - k if k >= 5 else 3), (t, j)
+                nib = (int(B[t, 106 + (j >> 1)]) >> (4 * (j & 1))) & 15
+                with np.errstate(all="ignore"):
+                    scale = np.float32(d * np.float32((2 * k + 1) * (2 * nib + 1))) / np.float32(127.0)
+                regular = bool(scale >= np.float32(6.103515625e-05)) and bool(scale < np.float32(65504.0))
+                assert (int(hints[t]) >> (2 * j)) & 3 == (7 - k if k >= 5 and regular else 3), (t, j)
 
 
 def test_error_paths(capi, dev):
@@ -471,9 +477,12 @@ def _production_cases():
         ("q4k_mfma_m5", FMT_Q4_K, 4096, 4096, 5, MF),
         ("q6k_mfma_m8_chunked_row", FMT_Q6_K, 200, 25600, 8, MF),
         ("q6k_mfma_m8_short_last_chunk", FMT_Q6_K, 70, 17408, 8, MF),
-        ("iq3s_chunked_m1", FMT_IQ3_S, 1000, 5120, 1, CH),
-        ("iq3s_chunked_m8", FMT_IQ3_S, 300, 5120, 8, CH),
-        ("iq3s_k_sliced_m4", FMT_IQ3_S, 50, 25600, 4, CH),
+        ("iq3s_quad_m1", FMT_IQ3_S, 1000, 5120, 1, QU),
+        ("iq3s_quad_m8", FMT_IQ3_S, 300, 5120, 8, QU),
+        ("iq3s_quad_m4_long_rows", FMT_IQ3_S, 50, 25600, 4, QU),
+        ("iq3s_quad_m3_row_ends_inside_steps", FMT_IQ3_S, 515, 4352, 3, QU),
+        ("iq3s_chunked_m1", FMT_IQ3_S, 1000, 3072, 1, CH),
+        ("iq3s_chunked_m8", FMT_IQ3_S, 300, 2048, 8, CH),
         ("q4k_chunked_m3", FMT_Q4_K, 500, 2048, 3, CH),
         ("q6k_chunked_m6_batch_split", FMT_Q6_K, 90, 3072, 6, CH),
         ("q6k_generic_m2", FMT_Q6_K, 100, 512, 2, GE),
