@@ -21,6 +21,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import subprocess
 import sys
 import time
@@ -31,10 +32,19 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# runs of this script (profiles/gemv_q4k_25600x5120_batch1_pmc.txt): (36157.8 KiB x 2.000 +
-# 114.9 KiB x 1.000), the factors being what the same counters read for a plain 256 MiB kernel.
-DOMINANT_TRAFFIC_BYTES = 74168832
+DOMINANT_PROFILE = ROOT / "profiles" / "gemv_q4k_25600x5120_batch1_pmc.txt"
+
+
+def dominant_traffic_bytes():
+    """HBM bytes per launch of the dominant kernel as measured with rocprofv3 --pmc (FETCH_SIZE and
+    WRITE_SIZE runs of this script, scaled by what the same counters read for a plain copy
+    kernel): the `traffic_bytes_per_launch = N` line of the committed profile summary.  None
+    when the summary is missing."""
+    try:
+        m = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", DOMINANT_PROFILE.read_text(), re.M)
+    except OSError:
+        return None
+    return int(m.group(1)) if m else None
 
 HIDDEN, QDIM, KVDIM, FFN = 5120, 8192, 1024, 25600
 
@@ -347,6 +357,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true",
                     help="layer workload at batch 1: skip the short run of the 64-layer decode step")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="layer workload at batch 1: skip the short runs of the prefill GEMM and the MoE decode")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 256 MiB read + 256 MiB write elementwise kernel a few times, so a rocprofv3 --pmc run of this "
                          "command records FETCH_SIZE / WRITE_SIZE for a kernel of known traffic")
@@ -543,13 +555,14 @@ def main():
             "launch": "eager" if graphs is None else "hip-graph replay",
         },
         "roofline": {
-            "kernel": "gemv_quad_kernel<Q4KQuad,1,3,0> N=25600 K=5120",
+            "kernel": "gemv_quad_kernel<Q4KQuad, 1 activation row, 1 step per load chunk, Q8_1 input, row sums "
+                      "through the LDS ring> N=25600 K=5120",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": DOMINANT_TRAFFIC_BYTES,
+            "traffic": dominant_traffic_bytes(),
             "bytes_per_launch": k_bytes,
             "us_per_launch": round(k_us, 3),
             "launches_timed": reps,
@@ -559,7 +572,7 @@ def main():
     if M == 1 and not args.no_decode:
         # the metric's second figure: tokens per second of the whole 64-layer decode step at
         # batch 1 (the `decode` workload, a shorter run of it), reported beside the headline
-        del layers, graphs, group
+        layers = graphs = group = None
         torch.cuda.empty_cache()
         try:
             sub = argparse.Namespace(**vars(args))
@@ -572,6 +585,44 @@ def main():
                 "steps": sub.steps, "workload": "bench.py --workload decode"}
         except Exception as e:  # noqa: BLE001 - the headline figure must still be reported
             out["config"]["decode_step"] = {"error": str(e)[:200]}
+    if M == 1 and not args.no_extras:
+        # the other configurations of the baseline, short runs of their own workloads, each with
+        # its own roofline fraction: the prefill GEMM (int8 matrix-unit peak) and the MoE expert
+        # FFN decode at 1 and 16 tokens (HBM peak over the distinct experts' bytes)
+        layers = graphs = group = mats = None
+        torch.cuda.empty_cache()
+
+        def brief(d, extra):
+            r = d["roofline"]
+            o = {"value": d["value"], "unit": d["unit"], "us_per_step": round(d["ms_per_step"] * 1e3, 2),
+                 "roofline": {"bound": r["bound"], "achieved": r["achieved"], "peak": r["peak"], "unit": r["unit"],
+                              "frac": r["frac"]}}
+            o.update(extra)
+            return o
+
+        try:
+            sub = argparse.Namespace(**vars(args))
+            sub.workload, sub.batch, sub.steps, sub.warmup = "gemm", 512, 20, 3
+            d = bench_gemm(sub, torch, capi, synth, dev)
+            out["config"]["prefill_gemm"] = brief(d, {"M": 512, "N": FFN, "K": HIDDEN, "fmt": "Q4_K",
+                                                      "workload": "bench.py --workload gemm"})
+        except Exception as e:  # noqa: BLE001
+            out["config"]["prefill_gemm"] = {"error": str(e)[:200]}
+        torch.cuda.empty_cache()
+        moe = []
+        for tokens in (1, 16):
+            try:
+                sub = argparse.Namespace(**vars(args))
+                sub.workload, sub.batch, sub.steps, sub.warmup = "moe", tokens, 128, 4
+                d = bench_moe(sub, torch, capi, synth, dev)
+                moe.append(brief(d, {"tokens": tokens, "path": d["config"]["path"],
+                                     "distinct_experts_per_step": d["config"]["distinct_experts_per_step"],
+                                     "tokens_per_s": d["config"]["tokens_per_s"],
+                                     "workload": "bench.py --workload moe --batch %d" % tokens}))
+            except Exception as e:  # noqa: BLE001
+                moe.append({"tokens": tokens, "error": str(e)[:200]})
+            torch.cuda.empty_cache()
+        out["config"]["moe_decode"] = moe
     print(json.dumps(out))
 
 

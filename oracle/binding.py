@@ -56,6 +56,8 @@ class Oracle:
         L.qlo_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_void_p]
         L.qlo_check_div127.restype = ctypes.c_long
         L.qlo_check_div127_all_significands.restype = ctypes.c_long
+        L.qlo_stream_triad.restype = ctypes.c_double
+        L.qlo_stream_triad.argtypes = [c_void_p, c_void_p, c_void_p, ctypes.c_long, c_int]
         L.qlo_check_q6k_factor.restype = ctypes.c_long
         L.qlo_check_q6k_factor.argtypes = [c_int]
         L.qlo_dequant_row_q4k.argtypes = [c_void_p, c_int, c_void_p]
@@ -147,6 +149,12 @@ class Oracle:
         probs = np.zeros((T, E), np.float32)
         self.L.qlo_moe_route(_p(logits), T, E, top_k, int(normalize), _p(ids), _p(w), _p(probs))
         return ids, w, probs
+
+    def stream_triad_gbs(self, mib_per_array: int = 256, reps: int = 5) -> float:
+        """Host DRAM bandwidth (STREAM triad, every OpenMP thread), GB/s."""
+        n = mib_per_array * (1 << 20) // 8
+        a, b, c = np.zeros(n), np.ones(n), np.full(n, 2.0)
+        return float(self.L.qlo_stream_triad(_p(a), _p(b), _p(c), n, reps)) / 1e9
 
     def check_div127(self) -> int:
         return int(self.L.qlo_check_div127())

@@ -37,6 +37,32 @@ def cpu_flags() -> set:
     return set()
 
 
+def cpu_topology() -> dict:
+    """Sockets, physical cores and logical CPUs of this host, from /proc/cpuinfo."""
+    cores, sockets, logical, model = set(), set(), 0, ""
+    phys = core = None
+    try:
+        for line in open("/proc/cpuinfo"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "processor":
+                logical += 1
+                phys = core = None
+            elif key == "model name" and not model:
+                model = val
+            elif key == "physical id":
+                phys = val
+                sockets.add(val)
+            elif key == "core id":
+                core = val
+            if phys is not None and core is not None:
+                cores.add((phys, core))
+    except OSError:
+        pass
+    return {"sockets": len(sockets) or None, "physical_cores": len(cores) or None, "logical_cpus": logical or None,
+            "model": model}
+
+
 def main():
     N, K, fmt = 25600, 5120, FMT_Q4_K
     budget_s = float(os.environ.get("QL_CPU_BASELINE_SECONDS", "12"))
@@ -95,11 +121,20 @@ def main():
         kind = "port"
         detail = f"scalar C restatement on {rows} of {N} rows, OpenMP over rows"
     med = float(np.median(times))
+    del flush
+    try:
+        stream_gbs = round(o.stream_triad_gbs(), 1)
+    except Exception:  # noqa: BLE001 - an older oracle library without the routine
+        stream_gbs = None
+    topo = cpu_topology()
     print(json.dumps({
         "value": nbytes / med / 1e9,
         "unit": "GB/s",
         "cores": threads,
         "kind": kind,
+        "host": topo,
+        "host_dram_stream_triad_gbs": stream_gbs,
+        "frac_of_host_dram": (round(nbytes / med / 1e9 / stream_gbs, 3) if stream_gbs else None),
         "sample": f"Q4_K GEMV N={N} K={K} batch 1, {len(times)} timed calls with the caches flushed before each "
                   f"(median {med * 1e3:.3f} ms, min {min(times) * 1e3:.3f} ms), {detail}",
     }))

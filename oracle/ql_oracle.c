@@ -8,6 +8,7 @@
 #include "ql_oracle.h"
 
 #include <math.h>
+#include <omp.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -528,4 +529,28 @@ long qlo_check_q6k_factor(int ulps)
         }
     }
     return bad;
+}
+
+
+/* Host memory bandwidth for the CPU baseline's context: the triad a[i] = b[i] + s * c[i] over
+ * three arrays of n doubles with every OpenMP thread, `reps` passes, best pass.  Returns bytes per
+ * second counting 24 bytes per element (the STREAM convention: no write-allocate traffic), as
+ * the reference's performance harness reports beside its GEMV figures
+ * (tests/v2/performance/kernels/cpu/native_vnni/Perf__CPUNativeVNNI_GEMV.cpp:120-177). */
+double qlo_stream_triad(double *a, const double *b, const double *c, long n, int reps)
+{
+    double best = 0.0;
+    for (int r = 0; r < reps; ++r) {
+        const double t0 = omp_get_wtime();
+#pragma omp parallel for schedule(static)
+        for (long i = 0; i < n; ++i)
+            a[i] = b[i] + 3.0 * c[i];
+        const double dt = omp_get_wtime() - t0;
+        if (dt > 0.0) {
+            const double bw = 24.0 * (double)n / dt;
+            if (bw > best)
+                best = bw;
+        }
+    }
+    return best;
 }

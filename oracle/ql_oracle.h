@@ -112,6 +112,9 @@ void qlo_attention_decode(const float *q, const uint16_t *kcache, const uint16_t
                           int n_heads, int n_kv, int head_dim, int ctx_cap);
 int qlo_argmax(const float *x, int n);
 
+/* STREAM triad over three arrays of n doubles, all OpenMP threads; bytes per second of the best of `reps` passes */
+double qlo_stream_triad(double *a, const double *b, const double *c, long n, int reps);
+
 #ifdef __cplusplus
 }
 #endif
