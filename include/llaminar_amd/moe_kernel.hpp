@@ -57,6 +57,16 @@ namespace llaminar_amd
         bool supports_device(int device_idx) const { return device_idx == device_id_; }
         void setGPUStream(void *stream) { stream_ = stream; }
         bool isValid() const { return valid_; }
+        // nothing of its own to snapshot: the expert matrices belong to their GEMM operators
+        // (kernels/rocm/moe/ROCmMoEKernel.h:387-390)
+        KernelSnapshotInfo getKernelSnapshotInfo() const
+        {
+            KernelSnapshotInfo info;
+            info.kernel_name = "MoE";
+            info.kernel_description = "pass-through";
+            info.is_passthrough = true;
+            return info;
+        }
 
         // ---- workspace -----------------------------------------------------------------
         // Bytes the decode methods need for n_tokens tokens of `slots` expert slots each:

@@ -66,6 +66,55 @@ namespace llaminar_amd
     // Reason of the calling thread's last failed operator or registry call.
     const char *quant_gemm_last_error();
 
+    // Prepared weights outside an operator: what detachWeights() hands over, cloneWeights()
+    // copies and attachWeights() takes (the reference's transferable packed weights,
+    // kernels/IPackedWeights.h:62-130: format, shape, size, deep copy).  Device memory in the
+    // prepared layout of llam_ql_prepare_weights, owned (freed with the object) or kept alive
+    // by a shared owner.
+    class MI355PackedWeights
+    {
+    public:
+        ~MI355PackedWeights();
+        MI355PackedWeights(const MI355PackedWeights &) = delete;
+        MI355PackedWeights &operator=(const MI355PackedWeights &) = delete;
+
+        uint8_t format() const { return fmt_; } // llam_weight_format
+        int N() const { return n_; }
+        int K() const { return k_; }
+        int device() const { return device_id_; }
+        size_t sizeBytes() const { return bytes_; }
+        const void *data() const { return d_; }
+        // Deep copy on the same device (stream-ordered copy, synchronised before it returns);
+        // null when the allocation or the copy fails.
+        std::unique_ptr<MI355PackedWeights> clone(void *stream = nullptr) const;
+
+    private:
+        friend class MI355QuantGemmKernel;
+        MI355PackedWeights() = default;
+        uint8_t fmt_ = 0;
+        int n_ = 0, k_ = 0, device_id_ = 0;
+        size_t bytes_ = 0;
+        const void *d_ = nullptr;
+        void *owned_ = nullptr;
+        std::shared_ptr<void> keepalive_;
+    };
+
+    // What a snapshot tool may record around one call of the operator: the buffers and scalars
+    // by name (tensors/KernelSnapshotInfo.h:249-300; kernels/rocm/gemm/ROCmQuantisedGemmKernel.cpp:5049-5059).
+    struct KernelBufferDesc
+    {
+        const char *name;
+        const char *description;
+        const char *dtype; // "FP32", "INT8", "INT32"
+    };
+    struct KernelSnapshotInfo
+    {
+        const char *kernel_name = "";
+        const char *kernel_description = "";
+        std::vector<KernelBufferDesc> inputs, outputs, weights, scalars;
+        bool is_passthrough = false; // nothing to snapshot
+    };
+
     class MI355QuantGemmKernel
     {
     public:
@@ -96,6 +145,16 @@ namespace llaminar_amd
         bool hasWeights() const { return valid_ && (d_weights_ || host_gguf_); }
         void releaseWeights();
         size_t packedWeightBytes() const;
+        // Weight hand-over (TensorKernels.h:1335-1394).  detachWeights: the operator gives its
+        // prepared weights away and has none until attachWeights (hasWeights() is false, every
+        // multiply fails); cloneWeights: a deep copy, the operator keeps its own; attachWeights:
+        // takes weights of the same format, shape and device in place of whatever it held,
+        // false (and the argument destroyed) on a mismatch.  Host GGUF bytes that have not been
+        // uploaded yet are prepared first.
+        std::unique_ptr<MI355PackedWeights> detachWeights();
+        std::unique_ptr<MI355PackedWeights> cloneWeights();
+        bool attachWeights(std::unique_ptr<MI355PackedWeights> weights);
+        KernelSnapshotInfo getKernelSnapshotInfo() const;
         uint8_t codebookId() const { return fmt_; }
         int get_n() const { return N_; }
         int get_k() const { return K_; }

@@ -116,7 +116,132 @@ namespace llaminar_amd
 
     size_t MI355QuantGemmKernel::packedWeightBytes() const
     {
-        return valid_ ? llam_ql_prepared_bytes(fmt_, N_, K_) : 0;
+        return (valid_ && (d_weights_ || host_gguf_)) ? llam_ql_prepared_bytes(fmt_, N_, K_) : 0;
+    }
+
+    // ---- weight hand-over ----------------------------------------------------------
+
+    MI355PackedWeights::~MI355PackedWeights()
+    {
+        if (owned_)
+        {
+            (void)hipSetDevice(device_id_);
+            (void)hipFree(owned_);
+        }
+    }
+
+    std::unique_ptr<MI355PackedWeights> MI355PackedWeights::clone(void *stream) const
+    {
+        static const char *fn = "MI355PackedWeights::clone";
+        if (!d_ || bytes_ == 0)
+        {
+            fail(fn, "no weights to copy");
+            return nullptr;
+        }
+        if (hipSetDevice(device_id_) != hipSuccess)
+        {
+            fail(fn, "no HIP device %d", device_id_);
+            return nullptr;
+        }
+        void *copy = nullptr;
+        if (hipMalloc(&copy, bytes_) != hipSuccess)
+        {
+            (void)hipGetLastError();
+            fail(fn, "device allocation of %zu bytes failed", bytes_);
+            return nullptr;
+        }
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        if (hipMemcpyAsync(copy, d_, bytes_, hipMemcpyDeviceToDevice, st) != hipSuccess ||
+            hipStreamSynchronize(st) != hipSuccess)
+        {
+            (void)hipGetLastError();
+            (void)hipFree(copy);
+            fail(fn, "device copy of %zu bytes failed", bytes_);
+            return nullptr;
+        }
+        std::unique_ptr<MI355PackedWeights> w(new MI355PackedWeights());
+        w->fmt_ = fmt_;
+        w->n_ = n_;
+        w->k_ = k_;
+        w->device_id_ = device_id_;
+        w->bytes_ = bytes_;
+        w->d_ = copy;
+        w->owned_ = copy;
+        return w;
+    }
+
+    std::unique_ptr<MI355PackedWeights> MI355QuantGemmKernel::detachWeights()
+    {
+        if (!ready("detachWeights"))
+            return nullptr;
+        std::lock_guard<std::mutex> lock(prepare_mutex_);
+        std::unique_ptr<MI355PackedWeights> w(new MI355PackedWeights());
+        w->fmt_ = fmt_;
+        w->n_ = N_;
+        w->k_ = K_;
+        w->device_id_ = device_id_;
+        w->bytes_ = llam_ql_prepared_bytes(fmt_, N_, K_);
+        w->d_ = d_weights_;
+        w->owned_ = d_owned_;
+        w->keepalive_ = std::move(lifetime_owner_);
+        d_owned_ = nullptr;
+        d_weights_ = nullptr;
+        lifetime_owner_.reset();
+        return w; // valid_ stays: the shape is known, attachWeights() makes the operator usable again
+    }
+
+    std::unique_ptr<MI355PackedWeights> MI355QuantGemmKernel::cloneWeights()
+    {
+        if (!ready("cloneWeights"))
+            return nullptr;
+        MI355PackedWeights view;
+        view.fmt_ = fmt_;
+        view.n_ = N_;
+        view.k_ = K_;
+        view.device_id_ = device_id_;
+        view.bytes_ = llam_ql_prepared_bytes(fmt_, N_, K_);
+        view.d_ = d_weights_; // not owned: the view frees nothing
+        return view.clone(stream_);
+    }
+
+    bool MI355QuantGemmKernel::attachWeights(std::unique_ptr<MI355PackedWeights> weights)
+    {
+        static const char *fn = "attachWeights";
+        if (!valid_)
+            return fail(fn, "operator is not valid");
+        if (!weights || !weights->d_)
+            return fail(fn, "null weights");
+        if (weights->fmt_ != fmt_ || weights->n_ != N_ || weights->k_ != K_ || weights->device_id_ != device_id_)
+            return fail(fn, "weights are format %d [%d x %d] on device %d, the operator is format %d [%d x %d] on device %d",
+                        (int)weights->fmt_, weights->n_, weights->k_, weights->device_id_, (int)fmt_, N_, K_, device_id_);
+        std::lock_guard<std::mutex> lock(prepare_mutex_);
+        if (d_owned_)
+        {
+            (void)hipSetDevice(device_id_);
+            (void)hipFree(d_owned_);
+        }
+        d_owned_ = weights->owned_;
+        d_weights_ = weights->d_;
+        lifetime_owner_ = std::move(weights->keepalive_);
+        host_gguf_ = nullptr;
+        weights->owned_ = nullptr; // ownership moved
+        weights->d_ = nullptr;
+        return true;
+    }
+
+    KernelSnapshotInfo MI355QuantGemmKernel::getKernelSnapshotInfo() const
+    {
+        KernelSnapshotInfo info;
+        info.kernel_name = "GEMM";
+        info.kernel_description = "block-quantized linear projection: C = alpha * A @ W^T + beta * C (+ bias)";
+        info.inputs = {{"A", "input activations [m, k]", "FP32"}};
+        info.weights = {{"B", "quantized weight matrix [n, k] (GGUF blocks in the prepared device layout)", "INT8"}};
+        info.outputs = {{"C", "output matrix [m, n]", "FP32"}};
+        info.scalars = {{"N", "output features", "INT32"},
+                        {"K", "input features", "INT32"},
+                        {"rocm_device_id", "HIP device ID", "INT32"},
+                        {"weights_converted", "whether the weights are on the device in the prepared layout", "INT32"}};
+        return info;
     }
 
     // Upload the GGUF bytes and bring them into the prepared layout.  The staging copy
@@ -125,7 +250,7 @@ namespace llaminar_amd
     {
         static const char *fn = "prepareWeights";
         std::lock_guard<std::mutex> lock(prepare_mutex_);
-        if (!valid_ || d_weights_)
+        if (!valid_ || d_weights_ || !host_gguf_) // nothing to upload (also after detachWeights)
             return;
         if (hipSetDevice(device_id_) != hipSuccess)
         {
@@ -410,10 +535,22 @@ namespace llaminar_amd
         DeviceWorkspace *workspace)
     {
         static const char *fn = "multiply_fused_verifier_rows_decode_equivalent";
-        // Rows are bit-identical to the m == 1 result while the activations of all rows
-        // fit the GEMV's LDS staging in one piece: 320 bytes per 256 columns and row.
-        if (m < 1 || m > 4 || (size_t)m * (size_t)(k / 256) * 320 > 64 * 1024)
-            return fail(fn, "m=%d k=%d is outside the decode-equivalent range", m, k);
+        // A row is bit-identical to its m == 1 result when the launcher serves both batch sizes
+        // with the same kernel on the same row partition and K slices: asked of the launcher
+        // itself, per projection (llam_ql_gemv_describe reports the plan llam_ql_gemv executes).
+        if (m < 1 || m > 4)
+            return fail(fn, "m=%d is outside the decode-equivalent range 1..4", m);
+        for (const auto &p : projections)
+        {
+            if (!p.kernel)
+                return fail(fn, "null projection kernel");
+            llam_ql_gemv_plan plan;
+            if (!forward(fn, llam_ql_gemv_describe(p.kernel->fmt_, m, p.n, k, device_id_, &plan)))
+                return false;
+            if (!plan.decode_equivalent)
+                return fail(fn, "m=%d n=%d k=%d (format %d) is not served like m=1: rows would differ in the last bits",
+                            m, p.n, k, (int)p.kernel->fmt_);
+        }
         return multiply_fused_tensor(input, projections, m, k, workspace);
     }
 

@@ -369,6 +369,59 @@ static void test_multiply_tensor(uint8_t fmt)
     HIP_OK(hipDeviceSynchronize());
 }
 
+// detachWeights / cloneWeights / attachWeights (TensorKernels.h:1335-1394) and the snapshot
+// description: a clone attached to another operator of the same shape computes the donor's
+// result bit for bit; a detached operator has no weights and fails until they come back.
+static void test_weight_handover(uint8_t fmt)
+{
+    const std::string name = std::string("WeightHandover_") + fmt_name(fmt);
+    begin(name.c_str());
+    const int N = 96, K = 1024, m = 2;
+    auto wa = make_weights(fmt, N, K, 61), wb = make_weights(fmt, N, K, 62);
+    MI355QuantGemmKernel a(fmt, wa.data(), N, K, 0), b(fmt, wb.data(), N, K, 0);
+    auto x = make_floats((size_t)m * K, 63);
+    DevBuf<float> dX(x), dA((size_t)m * N), dB((size_t)m * N);
+    DeviceTensor X(dX.p, m, K), CA(dA.p, m, N), CB(dB.p, m, N);
+    CHECK(a.multiply_tensor(&X, &CA, m, N, K));
+    CHECK(b.multiply_tensor(&X, &CB, m, N, K));
+    const auto ya = dA.download();
+    CHECK(ya != dB.download());
+
+    auto copy = a.cloneWeights();
+    CHECK(copy && copy->format() == fmt && copy->N() == N && copy->K() == K && copy->device() == 0);
+    CHECK(copy && copy->sizeBytes() == a.packedWeightBytes() && copy->data() != nullptr);
+    CHECK(a.hasWeights()); // the donor keeps its own
+    CHECK(b.attachWeights(std::move(copy)));
+    CHECK(b.multiply_tensor(&X, &CB, m, N, K));
+    CHECK(dB.download() == ya);
+
+    auto taken = a.detachWeights();
+    CHECK(taken && taken->sizeBytes() == llam_ql_prepared_bytes(fmt, N, K));
+    CHECK(!a.hasWeights() && a.packedWeightBytes() == 0);
+    CHECK(!a.multiply_tensor(&X, &CA, m, N, K)); // no weights: fails, does not crash
+    CHECK(strstr(quant_gemm_last_error(), "weights") != nullptr);
+    auto second = taken ? taken->clone() : nullptr; // a copy of a detached payload
+    CHECK(second != nullptr);
+    CHECK(a.attachWeights(std::move(taken)));
+    CHECK(a.hasWeights());
+    CHECK(a.multiply_tensor(&X, &CA, m, N, K));
+    CHECK(dA.download() == ya);
+
+    // a payload of another shape or format is refused
+    auto wz = make_weights(fmt, 64, 256, 64);
+    MI355QuantGemmKernel z(fmt, wz.data(), 64, 256, 0);
+    CHECK(!z.attachWeights(std::move(second)));
+    CHECK(!z.attachWeights(nullptr));
+
+    const KernelSnapshotInfo info = a.getKernelSnapshotInfo();
+    CHECK(std::string(info.kernel_name) == "GEMM" && !info.is_passthrough);
+    CHECK(info.inputs.size() == 1 && std::string(info.inputs[0].name) == "A");
+    CHECK(info.weights.size() == 1 && std::string(info.weights[0].name) == "B");
+    CHECK(info.outputs.size() == 1 && std::string(info.outputs[0].name) == "C");
+    CHECK(info.scalars.size() == 4 && std::string(info.scalars[3].name) == "weights_converted");
+    HIP_OK(hipDeviceSynchronize());
+}
+
 static void test_fused_and_verifier_rows(uint8_t fmt)
 {
     const std::string name = std::string("FusedProjections_") + fmt_name(fmt);
@@ -402,6 +455,33 @@ static void test_fused_and_verifier_rows(uint8_t fmt)
     }
     CHECK(same);
     CHECK(!q.multiply_fused_verifier_rows_decode_equivalent(&A, projs, 5, K));
+
+    // the down projection's row length (K = 25600) at three and four rows: accepted, and every
+    // row carries the bits of the single-row call
+    {
+        const int KL = 25600, NL = 48;
+        auto wl = make_weights(fmt, NL, KL, 27);
+        MI355QuantGemmKernel dl(fmt, wl.data(), NL, KL, 0);
+        auto al = make_floats((size_t)4 * KL, 28);
+        DevBuf<float> dAl(al), dCl((size_t)4 * NL);
+        DeviceTensor Al(dAl.p, 4, KL), Cl(dCl.p, 4, NL);
+        std::vector<P> one_proj = {P(&dl, &Cl, NL, nullptr, "down")};
+        for (int mm = 3; mm <= 4; ++mm)
+        {
+            CHECK(dl.multiply_fused_verifier_rows_decode_equivalent(&Al, one_proj, mm, KL));
+            auto got = dCl.download();
+            bool eq = true;
+            for (int r = 0; r < mm; ++r)
+            {
+                DevBuf<float> d1(NL);
+                DeviceTensor A1(dAl.p + (size_t)r * KL, 1, KL), C1(d1.p, 1, NL);
+                CHECK(dl.multiply_tensor(&A1, &C1, 1, NL, KL));
+                auto one = d1.download();
+                eq = eq && memcmp(one.data(), got.data() + (size_t)r * NL, NL * sizeof(float)) == 0;
+            }
+            CHECK(eq);
+        }
+    }
 
     // a projection with a bias takes the per-projection route
     std::vector<P> with_bias = {P(&q, &Q, Nq), P(&kk, &Kt, Nk, &B, "k")};
@@ -570,6 +650,7 @@ int main(int argc, char **argv)
         {
             test_multiply_tensor(fmt);
             test_fused_and_verifier_rows(fmt);
+            test_weight_handover(fmt);
             test_precomputed_q8_1(fmt);
             test_swiglu_and_expert_down(fmt);
         }

@@ -365,6 +365,34 @@ def test_q4k_long_rows_all_batches(capi, dev, oracle, N, K):
         lib.llam_ql_reset_gemv_tuning()
 
 
+@pytest.mark.parametrize("fmt", [FMT_Q4_K, FMT_Q6_K, FMT_IQ3_S], ids=["q4_k", "q6_k", "iq3_s"])
+@pytest.mark.parametrize("N,K", [(100, 512), (33, 1024), (300, 2048), (257, 3840), (64, 4096), (40, 25600)],
+                         ids=["generic_k512", "generic_k1024", "chunked_k2048", "chunked_k3840", "quad_k4096",
+                              "quad_k25600"])
+def test_rows_of_small_batches_equal_the_single_row_call(capi, dev, fmt, N, K):
+    """What the operator's decode-equivalent verifier rows rely on: for up to four activation
+    rows the launcher reports decode_equivalent (same kernel, row partition and K slices as the
+    single-row call) and every row of the batch carries the bits of its own single-row call --
+    on the generic, the chunked and the quad-lane kernel, all formats, K = 25600 included."""
+    import torch
+
+    W = synth.weights_torch(fmt, N, K, 400 + N, dev)
+    wd = capi.prepare_weights(fmt, W, N, K)
+    qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(4, K, 401 + K)).to(dev))
+    rb = (K // 32) * 36
+    one = [capi.gemv(fmt, wd, qd[m * rb:(m + 1) * rb], 1, N, K) for m in range(4)]
+    for M in (2, 3, 4):
+        plan = capi.gemv_describe(fmt, M, N, K)
+        assert plan.decode_equivalent == 1, (M, plan.kernel, plan.slice_sb)
+        y = capi.gemv(fmt, wd, qd, M, N, K)
+        sync()
+        for m in range(M):
+            assert torch.equal(y[m], one[m][0]), (M, m)
+    # five and more rows of a large Q4_K matrix go to the matrix unit, which adds blocks in another order
+    if fmt == FMT_Q4_K:
+        assert capi.gemv_describe(fmt, 8, 8192, 5120).decode_equivalent == 0
+
+
 @pytest.mark.parametrize("N,K", [(19, 25600), (70, 17408), (33, 30720)])
 def test_q6k_long_rows_large_batches(capi, dev, oracle, N, K):
     """Q6_K rows too long for eight activation rows in LDS: batches the quad-lane kernel would
