@@ -258,6 +258,8 @@ def bench_decode(args, torch, capi, synth, dev):
             with torch.cuda.graph(graph, stream=stream):
                 dec.step(stream)
         run = (lambda: graph.replay()) if graph is not None else (lambda: dec.step(stream))
+        if graph is not None:
+            dec.advance(max(args.warmup - 1, 1) + args.steps)  # replays do not pass through dec.step()
         for _ in range(max(args.warmup - 1, 1)):
             run()
         torch.cuda.synchronize()

@@ -80,8 +80,19 @@ bool llam_decoder_set_globals(void *dec, const llam_decoder_globals *g);
  * synchronously.  The cache must hold positions 0..pos-1 already (llam_decoder_buffer). */
 bool llam_decoder_set_state(void *dec, const int32_t *h_ids, const int32_t *h_pos);
 
-/* One token for every sequence; see the file comment. */
+/* One token for every sequence; see the file comment.  Fails, enqueuing nothing, when a
+ * sequence has reached ctx_cap: the handle counts, on the host, the position llam_decoder_set_state
+ * gave plus one per call (the device advances its own copy), so the check costs no
+ * synchronisation. */
 bool llam_decoder_step(void *dec, void *stream);
+
+/* Steps that may still run before the furthest sequence reaches ctx_cap, by that host count. */
+int llam_decoder_steps_left(void *dec);
+
+/* Replays of a captured step do not pass through llam_decoder_step: a caller that replays a
+ * graph of the step reports the replays here (before launching them), which advances the host
+ * count by n and fails, changing nothing, when fewer than n steps are left. */
+bool llam_decoder_advance(void *dec, int n);
 
 /* Device buffers, for filling caches, reading results and parity checks:
  *   "ids" int32[batch], "pos" int32[batch], "logits" fp32[batch][vocab], "x" fp32[batch][hidden]

@@ -58,7 +58,10 @@ void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll);
 void llam_ql_reset_gemv_tuning(void);
 
 /* ---- P1: activation quantiser --------------------------------------------------
- * fp32 [M x K] (row stride K) -> llam_block_q8_1 [M x K/32].  K % 32 == 0.
+ * fp32 [M x K] (row stride K) -> llam_block_q8_1 [M x ceil(K/32)].  d_x 16-byte aligned when
+ * K % 32 == 0 (every shape the GEMV and GEMM entry points take), 4-byte aligned otherwise: a row's
+ * partial last block then follows the reference's scalar quantiser (round half away from zero,
+ * software fp16 conversion, zero padding; src/v2/tensors/SIMDHelpers.h:4554-4596).
  * Replaces simd::quantize_single_block / quantize_two_blocks_avx512 and
  * quantize_activations_to_q8_1 (src/v2/tensors/SIMDHelpers.h:4716-4959,
  * src/v2/kernels/cpu/native_vnni/CPUNativeVNNIGemv.h:2000-2036); device-side

@@ -168,14 +168,14 @@ def _dev(t) -> int:
 # ---------------------------------------------------------------------------
 
 def quantize_q8_1(x, out=None, stream=None):
-    """fp32 [M,K] (or [K]) on the GPU -> uint8 tensor of M*(K/32) 36-byte Q8_1 blocks."""
+    """fp32 [M,K] (or [K]) on the GPU -> uint8 tensor of M*ceil(K/32) 36-byte Q8_1 blocks."""
     import torch
 
     x2 = x.reshape(1, -1) if x.dim() == 1 else x
     M, K = x2.shape
     assert x2.dtype == torch.float32 and x2.is_contiguous() and x2.is_cuda
     if out is None:
-        out = torch.empty(M * (K // 32) * 36, dtype=torch.uint8, device=x.device)
+        out = torch.empty(M * ((K + 31) // 32) * 36, dtype=torch.uint8, device=x.device)
     _check(load().llam_ql_quantize_q8_1(_ptr(x2), _ptr(out), M, K, _dev(x2), _stream(stream)), "quantize_q8_1")
     return out
 

@@ -50,6 +50,7 @@ namespace
         size_t owned_bytes = 0;
 
         int32_t *ids = nullptr, *pos = nullptr;
+        int host_max_pos = 0; // the furthest sequence's position as the host counts it
         float *x = nullptr, *delta = nullptr, *qkv = nullptr, *attn = nullptr, *gate = nullptr, *up = nullptr;
         float *logits = nullptr, *inv_freq = nullptr, *rope_table = nullptr, *att_scratch = nullptr;
         void *q8_h = nullptr, *q8_attn = nullptr, *q8_act = nullptr, *argmax_scratch = nullptr;
@@ -208,6 +209,30 @@ extern "C" bool llam_decoder_set_state(void *dec, const int32_t *h_ids, const in
         hipMemcpy(d->ids, h_ids, (size_t)d->cfg.batch * 4, hipMemcpyHostToDevice) != hipSuccess ||
         hipMemcpy(d->pos, h_pos, (size_t)d->cfg.batch * 4, hipMemcpyHostToDevice) != hipSuccess)
         return fail("set_state", "upload failed");
+    d->host_max_pos = 0;
+    for (int b = 0; b < d->cfg.batch; ++b)
+        d->host_max_pos = h_pos[b] > d->host_max_pos ? h_pos[b] : d->host_max_pos;
+    return true;
+}
+
+extern "C" int llam_decoder_steps_left(void *dec)
+{
+    Decoder *d = static_cast<Decoder *>(dec);
+    if (!d)
+        return 0;
+    const int left = d->cfg.ctx_cap - d->host_max_pos;
+    return left > 0 ? left : 0;
+}
+
+extern "C" bool llam_decoder_advance(void *dec, int n)
+{
+    Decoder *d = static_cast<Decoder *>(dec);
+    if (!d || n < 0)
+        return fail("advance", "bad argument");
+    if (n > llam_decoder_steps_left(dec))
+        return fail("advance", "context full: %d step(s) asked for, %d left of ctx_cap=%d", n,
+                    llam_decoder_steps_left(dec), d->cfg.ctx_cap);
+    d->host_max_pos += n;
     return true;
 }
 
@@ -251,6 +276,9 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
     const llam_decoder_config &c = d->cfg;
     const int B = c.batch, H = c.hidden, F = c.ffn, dev = c.device_id;
     const int QD = d->qdim(), KV = d->kvdim(), ldqkv = QD + 2 * KV;
+    // a position at ctx_cap would neither be appended to the cache nor attended to
+    if (d->host_max_pos >= c.ctx_cap)
+        return fail(fn, "context full: a sequence is at position %d of ctx_cap=%d", d->host_max_pos, c.ctx_cap);
 
     if (!forward(fn, llam_dec_embed_q4k(d->globals.embed_q4k, c.vocab, d->ids, d->x, B, H, H, dev, stream)))
         return false;
@@ -297,6 +325,8 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
     if (!forward(fn, llam_ql_gemv(d->globals.fmt_lm_head, d->globals.lm_head, d->q8_h, d->logits, B, c.vocab, H,
                                   c.vocab, dev, stream)))
         return false;
-    return forward(fn, llam_dec_argmax(d->logits, c.vocab, c.vocab, B, d->ids, d->pos, d->argmax_scratch, dev,
-                                       stream));
+    if (!forward(fn, llam_dec_argmax(d->logits, c.vocab, c.vocab, B, d->ids, d->pos, d->argmax_scratch, dev, stream)))
+        return false;
+    d->host_max_pos += 1; // (a call recorded under stream capture counts too: the count errs on the safe side)
+    return true;
 }

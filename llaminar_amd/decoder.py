@@ -50,6 +50,10 @@ def load() -> ctypes.CDLL:
         L.llam_decoder_set_state.argtypes = [c_void_p, c_void_p, c_void_p]
         L.llam_decoder_step.restype = c_bool
         L.llam_decoder_step.argtypes = [c_void_p, c_void_p]
+        L.llam_decoder_steps_left.restype = c_int
+        L.llam_decoder_steps_left.argtypes = [c_void_p]
+        L.llam_decoder_advance.restype = c_bool
+        L.llam_decoder_advance.argtypes = [c_void_p, c_int]
         L.llam_decoder_buffer.restype = c_void_p
         L.llam_decoder_buffer.argtypes = [c_void_p, c_char_p, c_int]
         L.llam_decoder_device_bytes.restype = c_size_t
@@ -189,6 +193,15 @@ class DenseDecoder:
 
     def step(self, stream=None):
         if not self.L.llam_decoder_step(self.h, capi._stream(stream)):
+            raise capi.QLError(self.L.llam_decoder_last_error().decode())
+
+    def steps_left(self) -> int:
+        """Steps before the furthest sequence reaches the end of the cache (the host's count)."""
+        return int(self.L.llam_decoder_steps_left(self.h))
+
+    def advance(self, n: int):
+        """Report n replays of a captured step (they do not pass through step())."""
+        if not self.L.llam_decoder_advance(self.h, n):
             raise capi.QLError(self.L.llam_decoder_last_error().decode())
 
     def device_bytes(self) -> int:

@@ -66,8 +66,10 @@ def test_argument_validation_and_error_text():
     buf = np.zeros(4096, np.uint8)
     p = buf.ctypes.data
     p16 = p + (-p % 16)
-    assert not lib.llam_ql_quantize_q8_1(p16, p16, 1, 33, 0, None)
-    assert "multiple of 32" in capi.last_error() and "llam_ql_quantize_q8_1" in capi.last_error()
+    assert not lib.llam_ql_quantize_q8_1(p16 + 4, p16, 1, 64, 0, None)
+    assert "16-byte aligned" in capi.last_error() and "llam_ql_quantize_q8_1" in capi.last_error()
+    assert not lib.llam_ql_quantize_q8_1(p16 + 2, p16, 1, 33, 0, None)
+    assert "4-byte aligned" in capi.last_error()
     assert not lib.llam_ql_gemv(capi.FMT_Q4_K, p16, p16, p16, 9, 4, 256, 4, 0, None)
     assert "M=9" in capi.last_error()
     assert not lib.llam_ql_gemv(capi.FMT_Q4_K, p16, p16, p16, 1, 4, 100, 4, 0, None)

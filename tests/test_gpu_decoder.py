@@ -105,6 +105,86 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
     dec.close()
 
 
+def test_batch_eight_against_numpy_walk(capi, dev, oracle):
+    """One step at batch 8 (the matrix-unit GEMV kernels, the batched attention and sampler)
+    against the numpy walk, sequence by sequence: logits, greedy token and the appended K row."""
+    import torch
+
+    from llaminar_amd.decoder import DenseDecoder, Shape
+
+    batch = 8
+    shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
+    cap, start = 64, 20
+    dec = DenseDecoder(shape, batch, cap, dev, seed=9, keep_raw=True, d_lo=0.002, d_hi=0.004, norm_scale=1.0)
+    ref = NumpyDecoder(oracle, shape, dec.raw, cap)
+    rng = np.random.default_rng(2)
+    ids = rng.integers(0, shape.vocab, batch).astype(np.int32)
+    pos = (start + 3 * np.arange(batch)).astype(np.int32)
+    kc_h = np.zeros((batch, shape.n_layers, shape.n_kv, cap, 128), np.float16)
+    vc_h = np.zeros_like(kc_h)
+    for b in range(batch):
+        kc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
+        vc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
+    for l in range(shape.n_layers):
+        dec.buffer("kcache", l).copy_(torch.from_numpy(kc_h[:, l]).to(dev))
+        dec.buffer("vcache", l).copy_(torch.from_numpy(np.ascontiguousarray(vc_h[:, l].transpose(0, 1, 3, 2))).to(dev))
+    dec.set_state(ids, pos)
+    kc_u, vc_u = kc_h.view(np.uint16).copy(), vc_h.view(np.uint16).copy()
+    dec.step()
+    sync()
+    logits = dec.buffer("logits").cpu().numpy()
+    new_ids = dec.buffer("ids").cpu().numpy()
+    assert dec.buffer("pos").cpu().tolist() == [int(p) + 1 for p in pos]
+    for b in range(batch):
+        exp = ref.step(int(ids[b]), int(pos[b]), kc_u[b], vc_u[b])
+        scale = np.abs(exp).max()
+        assert np.abs(logits[b] - exp).max() <= 5e-3 * scale, b
+        assert new_ids[b] == int(np.argmax(logits[b]))
+        top2 = np.sort(exp)[-2:]
+        if top2[1] - top2[0] > 2 * 5e-3 * scale:
+            assert new_ids[b] == int(np.argmax(exp)), b
+        for l in range(shape.n_layers):
+            kg = dec.buffer("kcache", l)[b, :, int(pos[b])].cpu().numpy().astype(np.float32)
+            ke = kc_u[b, l, :, int(pos[b])].view(np.float16).astype(np.float32)
+            assert np.abs(kg - ke).max() <= 2e-2 * max(np.abs(ke).max(), 1.0), (b, l)
+    dec.close()
+
+
+def test_a_full_context_is_reported(capi, dev):
+    """The last position of the cache can still be decoded; the step after it fails with a clear
+    error and enqueues nothing (ids, positions and logits keep their values); replays of a
+    captured step are accounted through advance()."""
+    from llaminar_amd.decoder import DenseDecoder, Shape
+
+    shape = Shape(hidden=1024, n_heads=8, n_kv=2, head_dim=128, ffn=1024, vocab=512, n_layers=1)
+    cap = 16
+    dec = DenseDecoder(shape, 2, cap, dev, seed=3)
+    dec.set_state([5, 6], [cap - 3, cap - 1])          # the furthest sequence sits on the last position
+    assert dec.steps_left() == 1
+    dec.step()
+    sync()
+    assert dec.buffer("pos").cpu().tolist() == [cap - 2, cap]
+    assert dec.steps_left() == 0
+    ids = dec.buffer("ids").cpu().tolist()
+    logits = dec.buffer("logits").clone()
+    with pytest.raises(capi.QLError, match="context full"):
+        dec.step()
+    sync()
+    assert dec.buffer("pos").cpu().tolist() == [cap - 2, cap] and dec.buffer("ids").cpu().tolist() == ids
+    import torch
+
+    assert torch.equal(dec.buffer("logits"), logits)
+    with pytest.raises(capi.QLError, match="context full"):
+        dec.advance(1)
+    dec.set_state([1, 2], [0, 3])
+    assert dec.steps_left() == cap - 3
+    dec.advance(cap - 4)
+    assert dec.steps_left() == 1
+    with pytest.raises(capi.QLError, match="outside"):
+        dec.set_state([1, 2], [0, cap])
+    dec.close()
+
+
 @pytest.mark.parametrize("batch", [2, 6])
 def test_step_replays_as_a_graph(capi, dev, batch):
     """A captured step replayed gives the tokens of eager steps (batch 6: the matrix-unit kernels)."""

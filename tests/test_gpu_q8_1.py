@@ -16,7 +16,7 @@ def _gpu_quantize(capi, dev, x):
     q = capi.quantize_q8_1(xd)
     sync()
     M, K = x.shape
-    return q.cpu().numpy().reshape(M, K // 32, 36)
+    return q.cpu().numpy().reshape(M, (K + 31) // 32, 36)
 
 
 def test_golden_blocks(capi, dev, golden):
@@ -39,6 +39,26 @@ def test_random_rows_bit_exact(capi, dev, oracle, M, K, scale):
     if K >= 96:
         x[M - 1, 32:64] = 1e-11
     assert np.array_equal(_gpu_quantize(capi, dev, x), oracle.quantize(x))
+
+
+@pytest.mark.parametrize("M,K", [(1, 1), (1, 31), (3, 33), (2, 48), (5, 100), (1, 5121), (4, 5151)])
+def test_partial_last_block_bit_exact(capi, dev, oracle, M, K):
+    """Rows whose length is not a multiple of 32: the last block of a row holds K % 32 values and
+    follows the reference's scalar quantiser (round half away from zero, software fp16, zero
+    padding), the full blocks before it the SIMD one.  Row 0 is built so that x * id lands on
+    exact .5 ties in both kinds of block (amax 127 makes d = id = 1): the two roundings differ there."""
+    x = synth.activations_numpy(M, K, 3000 + M + K)
+    ties = (np.arange(K) % 32).astype(np.float32) - 15.5     # -15.5 .. 15.5
+    x[0] = ties
+    x[0, (np.arange(K) % 32) == 0] = 127.0                    # every block's amax
+    if K > 32 * 2 and M > 1:
+        x[1, 32 * ((K - 1) // 32):] = 1e-11                   # a partial block below the zero threshold
+        x[M - 1, 32 * ((K - 1) // 32):] *= np.float32(1e-7)   # its d is an fp16 subnormal (truncated)
+    want = oracle.quantize(x)
+    got = _gpu_quantize(capi, dev, x)
+    assert np.array_equal(got, want)
+    tail = K % 32
+    assert (got[:, -1, 4 + tail:] == 0).all()                 # zero padding
 
 
 def test_prefill_size_bit_exact(capi, dev, oracle):
@@ -65,6 +85,7 @@ def test_empty_and_errors(capi, dev):
     assert lib.llam_ql_quantize_q8_1(None, None, 0, 5120, 0, None)
     x = torch.zeros(64, device=dev)
     out = torch.zeros(72, dtype=torch.uint8, device=dev)
-    assert not lib.llam_ql_quantize_q8_1(x.data_ptr(), out.data_ptr(), 1, 48, 0, None)
+    assert not lib.llam_ql_quantize_q8_1(x.data_ptr() + 4, out.data_ptr(), 1, 32, 0, None)
+    assert "16-byte aligned" in capi.last_error()
     assert not lib.llam_ql_quantize_q8_1(x.data_ptr(), out.data_ptr(), 1, 64, 99, None)
     assert "device_id" in capi.last_error()
