@@ -85,6 +85,96 @@ def check_kernel_resources(remarks: str, src_name: str) -> dict[str, dict[str, i
     return usage
 
 
+class InFlightRegisterError(RuntimeError):
+    """Compiler-generated code touches the destination register of a hand-issued load before its wait."""
+
+
+_VREG = re.compile(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]")
+_ASM_LOAD = re.compile(r"^\s*(global_load_\w+|buffer_load_\w+)\s+(v\d+|v\[\d+:\d+\])\s*,")
+_VMEM = re.compile(r"^\s*(global_|buffer_|flat_|scratch_)(load|store|atomic)")
+_VMCNT = re.compile(r"vmcnt\((\d+)\)")
+
+
+def _vregs(text: str) -> set[int]:
+    regs: set[int] = set()
+    for m in _VREG.finditer(text):
+        if m.group(1) is not None:
+            regs.add(int(m.group(1)))
+        else:
+            regs.update(range(int(m.group(2)), int(m.group(3)) + 1))
+    return regs
+
+
+def check_inflight_registers(asm: str, src_name: str) -> int:
+    """Scan the device assembly for the second way the hand-scheduled loads can break.
+
+    The kernels issue global loads inside inline assembly and wait for them (s_waitcnt
+    vmcnt, also inline assembly) many instructions later.  To the compiler the destination
+    registers hold their values from the point of issue, so besides spilling them it may
+    COPY them (a phi move at a loop entry, a move into another allocation) or reuse them
+    while the data is still on its way: the copy reads stale contents, or the load lands in
+    whatever lives in the register by then.  This pass walks every function in program
+    order, keeps the queue of vector memory operations that vmcnt counts (hand-issued loads
+    with their destination registers, everything else as a placeholder), retires entries at
+    each s_waitcnt vmcnt(N), and reports any instruction that names a register of a
+    hand-issued load still in the queue.  Straight-line bookkeeping: the queue is emptied
+    where control cannot fall through (s_branch, s_endpgm, s_setpc), so the pass can miss a
+    hazard across a jump but does not invent one.  Returns the number of hand-issued loads
+    it followed.
+    """
+    findings: list[str] = []
+    followed = 0
+    func = "?"
+    queue: list[set[int] | None] = []  # oldest first; None: an operation whose registers the compiler tracks
+    in_asm = False
+    for raw_line in asm.splitlines():
+        line = raw_line.split(";")[0].rstrip() if not raw_line.lstrip().startswith(";;#") else raw_line.strip()
+        if line.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if line.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        m = re.match(r"^([A-Za-z_][\w$.]*):", line)
+        if m and not line.startswith(".L"):
+            func, queue = m.group(1), []
+            continue
+        text = line.strip()
+        if not text or text.startswith(".") or text.endswith(":"):
+            continue
+        if text.startswith("s_waitcnt"):
+            w = _VMCNT.search(text)
+            if w:
+                keep = int(w.group(1))
+                queue = queue[len(queue) - keep:] if keep and keep < len(queue) else ([] if keep == 0 else queue)
+            continue
+        if re.match(r"^(s_branch|s_endpgm|s_setpc_b64)\b", text):
+            queue = []
+            continue
+        touched = _vregs(text)
+        load = _ASM_LOAD.match(text) if in_asm else None
+        pending = set().union(*[q for q in queue if q]) if queue else set()
+        if load:
+            dst = _vregs(load.group(2))
+            hit = (touched - dst) & pending or (dst & pending)
+            if hit:
+                findings.append(f"{func}: '{text}' uses v{sorted(hit)[0]} while a hand-issued load into it is in flight")
+            queue.append(dst)
+            followed += 1
+            continue
+        hit = touched & pending
+        if hit:
+            findings.append(f"{func}: '{text}' touches v{sorted(hit)[0]} before the wait for the hand-issued load into it")
+        if _VMEM.match(text):
+            queue.append(None)
+    if findings:
+        shown = "\n  ".join(findings[:12]) + ("" if len(findings) <= 12 else f"\n  ... and {len(findings) - 12} more")
+        raise InFlightRegisterError(
+            f"{src_name}: registers of hand-issued loads are touched before their s_waitcnt "
+            f"(the data has not arrived; see check_inflight_registers):\n  {shown}")
+    return followed
+
+
 def hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not Path(exe).exists():
@@ -133,7 +223,8 @@ def _drop_resource_remarks(lines: list[str]) -> list[str]:
 
 def _compile(src: Path) -> Path:
     obj = OBJDIR / (src.stem + ".o")
-    cmd = [hipcc(), *HIP_FLAGS, RESOURCE_FLAG, "-c", str(src), "-o", str(obj)]
+    # -save-temps leaves the device assembly beside the object file for check_inflight_registers
+    cmd = [hipcc(), *HIP_FLAGS, RESOURCE_FLAG, "-save-temps=obj", "-c", str(src), "-o", str(obj)]
     if src.suffix == ".cpp":
         cmd.insert(1, "-x")
         cmd.insert(2, "hip")
@@ -142,6 +233,8 @@ def _compile(src: Path) -> Path:
     lines = [l for l in proc.stderr.splitlines() if noise not in l]
     if proc.returncode == 0:
         check_kernel_resources(proc.stderr, src.name)
+        for asm_file in OBJDIR.glob(f"{src.stem}-hip-amdgcn-*.s"):
+            check_inflight_registers(asm_file.read_text(), src.name)
     err = "\n".join(_drop_resource_remarks(lines))
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{err}")

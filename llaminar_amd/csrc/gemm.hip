@@ -8,8 +8,9 @@
 // (K depth 32 = exactly one Q8_1 block, zero accumulator input), so it is the
 // same exact integer the reference forms with vpdpbusd
 // (CPUNativeVNNIGemv.h:1046-1231); the per-block rescale is fp32 work: the scale
-// products a_d[m] * b_scale[n] of a block, a rank-1 matrix, come from one
-// v_mfma_f32_32x32x2f32 (exact), convert and multiply-add per output element stay on
+// products a_d[m] * b_scale[n] of a block, a rank-1 matrix, come from the matrix unit too
+// (v_mfma_f32_32x32x1_2b_f32: two blocks per instruction, exact), convert and multiply-add per
+// output element stay on
 // the vector unit (two operations against 64 int8 MFMA operations: this, not the int8
 // rate of the matrix unit, bounds the kernel), and the rank-1 min term goes through
 // another v_mfma_f32_32x32x2f32 straight into the accumulator.
@@ -32,6 +33,7 @@
 namespace llamql
 {
     typedef float v16f __attribute__((ext_vector_type(16)));
+    typedef float v32f __attribute__((ext_vector_type(32)));
 
     constexpr int GEMM_BM = 128;        // tokens per workgroup
     constexpr int GEMM_BN = 64;         // weight rows per workgroup
@@ -186,7 +188,7 @@ namespace llamql
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         uint8_t *Al = smem;                             // [BM][STRIDE] activations int8
         uint8_t *Wl = Al + GEMM_BM * GEMM_STRIDE;       // [BN][STRIDE] weights int8
-        float *ad = reinterpret_cast<float *>(Wl + GEMM_BN * GEMM_STRIDE); // [8][SM] a_d / 2
+        float *ad = reinterpret_cast<float *>(Wl + GEMM_BN * GEMM_STRIDE); // [8][SM] a_d
         float *asd = ad + 8 * GEMM_SM;                  // [8][SM]
         float *bs = asd + 8 * GEMM_SM;                  // [8][SN]
         float *bm = bs + 8 * GEMM_SN;                   // [8][SN]
@@ -224,6 +226,34 @@ namespace llamql
             areg.load(asrc + (size_t)sb * 72);
         };
 
+        // One K step's staging: registers -> LDS (weights as int8 [row][k] + scales, activations
+        // beside them), then the next step's global data is asked for, to travel while this one
+        // is multiplied (the last step re-reads itself: every issued load is consumed, none is
+        // conditional).
+        auto stage = [&](int sb) {
+            __syncthreads(); // previous step's LDS reads (and the table staging) are done
+            pf.store(Wl, bs, bm, tab);
+            areg.wait();
+            {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                {
+                    const uint32_t h = areg.dword(9 * i);
+                    const float d = h2f((uint16_t)(h & 0xFFFFu));
+                    const int kb = 2 * ap + i;
+                    ad[kb * GEMM_SM + am] = d;
+                    asd[kb * GEMM_SM + am] = (float)(int16_t)(h >> 16) * d;
+                    v4i *dst = reinterpret_cast<v4i *>(Al + am * GEMM_STRIDE + kb * 32);
+                    dst[0] = (v4i){(int)areg.dword(9 * i + 1), (int)areg.dword(9 * i + 2), (int)areg.dword(9 * i + 3),
+                                   (int)areg.dword(9 * i + 4)};
+                    dst[1] = (v4i){(int)areg.dword(9 * i + 5), (int)areg.dword(9 * i + 6), (int)areg.dword(9 * i + 7),
+                                   (int)areg.dword(9 * i + 8)};
+                }
+            }
+            __syncthreads();
+            issue(sb + 1 < g.w.SB ? sb + 1 : sb);
+        };
+
         v16f acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r)
@@ -232,67 +262,60 @@ namespace llamql
         issue(0);
         for (int sb = 0; sb < g.w.SB; ++sb)
         {
-            __syncthreads(); // previous step's LDS reads (and the table staging) are done
-
-            // ---- registers -> LDS: weights as int8 [row][k] + scales, activations beside them
-            pf.store(Wl, bs, bm, tab);
-            areg.wait();
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-            {
-                const uint32_t h = areg.dword(9 * i);
-                const float d = h2f((uint16_t)(h & 0xFFFFu));
-                const int kb = 2 * ap + i;
-                ad[kb * GEMM_SM + am] = 0.5f * d; // halved for the depth-2 scale product below
-                asd[kb * GEMM_SM + am] = (float)(int16_t)(h >> 16) * d;
-                v4i *dst = reinterpret_cast<v4i *>(Al + am * GEMM_STRIDE + kb * 32);
-                dst[0] = (v4i){(int)areg.dword(9 * i + 1), (int)areg.dword(9 * i + 2), (int)areg.dword(9 * i + 3),
-                               (int)areg.dword(9 * i + 4)};
-                dst[1] = (v4i){(int)areg.dword(9 * i + 5), (int)areg.dword(9 * i + 6), (int)areg.dword(9 * i + 7),
-                               (int)areg.dword(9 * i + 8)};
-            }
-            __syncthreads();
-
-            // ---- next step's global data travels while this one is multiplied (the last
-            //      step re-reads itself: every issued load is consumed, none is conditional)
-            issue(sb + 1 < g.w.SB ? sb + 1 : sb);
+            stage(sb);
 
             // ---- multiply ------------------------------------------------------------------
-            // 8 block products per step.  The MFMA of product kb+1 is issued before product kb
-            // is rescaled, so the matrix unit and the VALU work side by side: the results
-            // alternate between two register sets.
+            // 8 block products per step; the other wavefronts of the SIMD unit keep the vector
+            // unit busy while this one waits for the matrix unit.
             const uint8_t *wrow = Wl + (ntile * 32 + l32) * GEMM_STRIDE + lh * 16;
             const uint8_t *arow = Al + (mtile * 32 + l32) * GEMM_STRIDE + lh * 16;
             v16i zero;
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 zero[r] = 0;
-            v16f zerof;
+            v32f zero2f;
+#pragma unroll
+            for (int r = 0; r < 32; ++r)
+                zero2f[r] = 0.0f;
+            v16f zero1f;
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                zerof[r] = 0.0f;
+                zero1f[r] = 0.0f;
             auto product = [&](int kb) {
                 const v4i bw = *reinterpret_cast<const v4i *>(wrow + kb * 32);
                 const v4i aa = *reinterpret_cast<const v4i *>(arow + kb * 32);
                 return __builtin_amdgcn_mfma_i32_32x32x32_i8(aa, bw, zero, 0, 0, 0);
             };
             // The scale products a_d[m] * b_scale[n] of a block are a rank-1 matrix: the matrix
-            // unit forms them in the layout of the block sums instead of 16 multiplies per lane.
-            // Its depth of 2 adds (a_d/2) * b_scale twice: exact, both factors are fp16 values.
+            // unit forms them in the layout of the block sums instead of 16 multiplies per lane,
+            // two blocks per instruction (v_mfma_f32_32x32x1_2b_f32: lane half lh supplies block
+            // kb + lh, results 0-15 belong to block kb, 16-31 to block kb + 1).  Exact: both
+            // factors are fp16 values.
             auto scales = [&](int kb) {
-                const float av = ad[kb * GEMM_SM + mtile * 32 + l32]; // a_d / 2
-                const float bv = bs[kb * GEMM_SN + ntile * 32 + l32];
-                return __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, zerof, 0, 0, 0);
+                const float av = ad[(kb + lh) * GEMM_SM + mtile * 32 + l32];
+                const float bv = bs[(kb + lh) * GEMM_SN + ntile * 32 + l32];
+                return __builtin_amdgcn_mfma_f32_32x32x1f32(av, bv, zero2f, 0, 0, 0);
             };
-            v16i idot[2];
-            idot[0] = product(0);
-            v16f cs = scales(0);
+            // Formats whose prefetch registers leave no room for two blocks' scale products form
+            // them one block at a time (v_mfma_f32_32x32x2_f32 adds (a_d/2) * b_scale twice: exact).
+            auto scales1 = [&](int kb) {
+                const float av = 0.5f * ad[kb * GEMM_SM + mtile * 32 + l32];
+                const float bv = bs[kb * GEMM_SN + ntile * 32 + l32];
+                return __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, zero1f, 0, 0, 0);
+            };
+            v32f cs;
+            v16f cs1;
+            if constexpr (F::GEMM_PAIR_SCALES)
+                cs = scales(0);
+            else
+                cs1 = scales1(0);
 #pragma unroll
             for (int kb = 0; kb < 8; ++kb)
             {
-                if (kb + 1 < 8)
-                    idot[(kb + 1) & 1] = product(kb + 1);
-                const v16i d = idot[kb & 1];
+                // (one set of result registers: with the scale products held as well, a second
+                // set would not fit the 128 registers that four wavefronts per SIMD unit leave;
+                // the other wavefronts cover the product's latency)
+                const v16i d = product(kb);
                 if constexpr (DUMP)
                 {
                     const long n = n0 + ntile * 32 + l32;
@@ -310,10 +333,18 @@ namespace llamql
                 }
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    acc[r] = fmaf((float)d[r], cs[r], acc[r]);
+                    acc[r] = fmaf((float)d[r], F::GEMM_PAIR_SCALES ? cs[16 * (kb & 1) + r] : cs1[r], acc[r]);
                 __builtin_amdgcn_sched_barrier(0);
-                if (kb + 1 < 8)
-                    cs = scales(kb + 1); // the other wavefronts of the unit cover its latency
+                if constexpr (F::GEMM_PAIR_SCALES)
+                {
+                    if ((kb & 1) && kb + 1 < 8)
+                        cs = scales(kb + 1); // the other wavefronts of the unit cover its latency
+                }
+                else
+                {
+                    if (kb + 1 < 8)
+                        cs1 = scales1(kb + 1);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 if (F::HAS_MIN && (kb & 1))
                 {

@@ -361,6 +361,7 @@ namespace llamql
         static constexpr bool PAIR = false;
         static constexpr bool HAS_MIN = false;
         static constexpr bool USE_QUAD = true;         // quad-lane kernel for rows of >= 16 super-blocks
+        static constexpr bool GEMM_PAIR_SCALES = true;   // prefill GEMM: scale products of two blocks per matrix instruction
         static constexpr bool USE_MFMA_BATCH = false;  // matrix-unit kernel for 5..8 activation rows
         typedef IQ3SQuad Quad;
         static constexpr int FAST_MAX_U = 3;          // load batches in flight in the chunked kernel

@@ -21,6 +21,7 @@ namespace llamql
         static constexpr bool PAIR = true;
         static constexpr bool HAS_MIN = true;
         static constexpr bool USE_QUAD = true;        // quad-lane kernel for rows of >= 16 super-blocks
+        static constexpr bool GEMM_PAIR_SCALES = true;   // prefill GEMM: scale products of two blocks per matrix instruction
         static constexpr bool USE_MFMA_BATCH = true;  // matrix-unit kernel for 5..8 activation rows
         typedef Q4KQuad Quad;
         static constexpr int FAST_MAX_U = 4;          // load batches in flight in the chunked kernel

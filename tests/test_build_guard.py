@@ -46,3 +46,112 @@ def test_remarks_do_not_reach_the_build_log():
 
 def test_compile_command_asks_for_the_remarks():
     assert b.RESOURCE_FLAG == "-Rpass-analysis=kernel-resource-usage"
+
+
+# ---- the second check: registers of hand-issued loads touched before their wait ----------
+
+_PROLOGUE = """\
+\t.text
+_ZN6llamql4demoEv:
+\ts_load_dwordx2 s[0:1], s[4:5], 0x0
+"""
+
+
+def _asm(body: str) -> str:
+    return _PROLOGUE + body + "\ts_endpgm\n"
+
+
+def test_inflight_check_accepts_use_after_wait():
+    from llaminar_amd.build import check_inflight_registers
+
+    asm = _asm("""\
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[8:11], v[2:3], off
+\t;;#ASMEND
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[12:15], v[2:3], off offset:16
+\t;;#ASMEND
+\tv_add_u32_e32 v20, v21, v22
+\t;;#ASMSTART
+\ts_waitcnt vmcnt(1)
+\t;;#ASMEND
+\tv_and_b32_e32 v4, 0xf0f0f0f, v8
+\t;;#ASMSTART
+\ts_waitcnt vmcnt(0)
+\t;;#ASMEND
+\tv_and_b32_e32 v5, 0xf0f0f0f, v12
+""")
+    assert check_inflight_registers(asm, "demo.hip") == 2
+
+
+def test_inflight_check_refuses_a_copy_before_the_wait():
+    from llaminar_amd.build import InFlightRegisterError, check_inflight_registers
+
+    asm = _asm("""\
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[8:11], v[2:3], off
+\t;;#ASMEND
+\tv_mov_b64_e32 v[20:21], v[8:9]
+\t;;#ASMSTART
+\ts_waitcnt vmcnt(0)
+\t;;#ASMEND
+""")
+    with pytest.raises(InFlightRegisterError, match="v8"):
+        check_inflight_registers(asm, "demo.hip")
+
+
+def test_inflight_check_refuses_partial_wait_and_reuse_as_address():
+    from llaminar_amd.build import InFlightRegisterError, check_inflight_registers
+
+    # vmcnt(1) retires the older load only: the newer one's registers are still in flight
+    asm = _asm("""\
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[8:11], v[2:3], off
+\t;;#ASMEND
+\t;;#ASMSTART
+\tglobal_load_dwordx2 v[12:13], v[2:3], off offset:16
+\t;;#ASMEND
+\t;;#ASMSTART
+\ts_waitcnt vmcnt(1)
+\t;;#ASMEND
+\tv_add_u32_e32 v4, v8, v12
+""")
+    with pytest.raises(InFlightRegisterError, match="v12"):
+        check_inflight_registers(asm, "demo.hip")
+    # the destination of a load in flight handed out as an address of the next load
+    asm = _asm("""\
+\t;;#ASMSTART
+\tglobal_load_dwordx2 v[8:9], v[2:3], off
+\t;;#ASMEND
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[16:19], v[8:9], off
+\t;;#ASMEND
+""")
+    with pytest.raises(InFlightRegisterError, match="in flight"):
+        check_inflight_registers(asm, "demo.hip")
+
+
+def test_inflight_check_counts_other_memory_operations_and_resets_at_jumps():
+    from llaminar_amd.build import check_inflight_registers
+
+    # a compiler-issued store after the load is one more entry of vmcnt: vmcnt(1) then means
+    # "the hand-issued load has landed"; after an unconditional branch nothing is assumed in flight
+    asm = _asm("""\
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[8:11], v[2:3], off
+\t;;#ASMEND
+\tglobal_store_dword v[30:31], v32, off
+\t;;#ASMSTART
+\ts_waitcnt vmcnt(1)
+\t;;#ASMEND
+\tv_mov_b32_e32 v4, v8
+\t;;#ASMSTART
+\tglobal_load_dwordx4 v[12:15], v[2:3], off
+\t;;#ASMEND
+\ts_branch .LBB0_2
+.LBB0_1:
+\tv_mov_b32_e32 v5, v12
+.LBB0_2:
+\ts_waitcnt vmcnt(0)
+""")
+    assert check_inflight_registers(asm, "demo.hip") == 2

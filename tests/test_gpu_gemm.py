@@ -71,6 +71,34 @@ def test_block_sums_of_the_gemm_kernel(capi, dev, oracle, fmt, M, N, K, r0, nr):
     assert np.array_equal(s.cpu().numpy(), sums)
 
 
+@pytest.mark.parametrize("fmt", list(FMTS.values()), ids=list(FMTS))
+def test_more_tiles_than_the_chip_holds(capi, dev, oracle, fmt):
+    """More tiles than the chip holds at once, with a sparsely filled last round of workgroups
+    (580 tiles of 128 x 64 on 512 workgroup slots), ragged in both directions (130 tokens: the
+    second token tile holds two; 18550 rows: the last row tile holds 54): every output element
+    written exactly once and equal to the oracle's."""
+    import torch
+
+    M, N, K = 130, 18550, 512
+    W = synth.weights_numpy(fmt, N, K, 4242)
+    q8 = oracle.quantize(synth.activations_numpy(M, K, 4243))
+    wd = upload_weights(capi, dev, fmt, W)
+    qd = upload_q8(dev, q8)
+    y = torch.full((M, N), float("nan"), device=dev)
+    capi.gemm(fmt, wd, qd, M, N, K, out=y)
+    sync()
+    got = y.cpu().numpy()
+    assert np.isfinite(got).all()
+    C = oracle.gemm(fmt, W, K, q8)
+    assert rel_err(got, C) <= TOL[fmt] * 1e-2
+    # the worst single element, too: a misplaced tile would hide in a norm
+    assert np.abs(got - C).max() <= 1e-4 * np.abs(C).max()
+    y2 = torch.full((M, N), float("nan"), device=dev)
+    capi.gemm(fmt, wd, qd, M, N, K, out=y2)
+    sync()
+    assert torch.equal(y, y2)
+
+
 def test_prefill_config_full_size(capi, dev, oracle):
     """Config 3: M=512, K=5120, N=25600, Q4_K.  Oracle on a window of weight rows for all
     512 tokens; determinism over the whole output."""
