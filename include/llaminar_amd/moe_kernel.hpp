@@ -99,6 +99,16 @@ namespace llaminar_amd
                    int top_k, bool normalize_weights, MoERoutingResult &result);
         // IMoEKernel::weightedAdd (IMoEKernel.h:189-195): output[i] += weight * input[i], device buffers.
         bool weightedAdd(float *output, const float *input, float weight, int count);
+        // The other device helpers of the interface (IMoEKernel.h:92-171), all over device
+        // pointers, enqueued on the operator's stream.  token_indices are device int32; num_rows
+        // bounds them (rows of `hidden` / `output`).
+        bool gatherTokenBatch(const float *hidden, float *batch_buffer, const int *token_indices, int num_tokens,
+                              int d_model, int num_rows);
+        bool scatterAddWeighted(float *output, const float *expert_output, const int *token_indices,
+                                const float *weights, int num_tokens, int d_model, int num_rows);
+        bool sharedExpertGate(const float *input, const float *gate_inp, float *shared_output, int seq_len,
+                              int d_model);
+        bool swiGLU(float *gate, const float *up, int count);
 
         // ---- single-token grouped projections from host or fp32 device routing ------------------
         // (IMoEKernel.h:452-575)  FromTable: expert_ids / expert_weights are HOST arrays of the

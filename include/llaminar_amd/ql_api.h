@@ -341,6 +341,26 @@ bool llam_ql_shared_expert_add(float *d_out, const float *d_shared,
                                int n_tokens, int d_model, int device_id,
                                void *stream);
 
+/* The remaining device helpers of the MoE operator interface (src/v2/kernels/IMoEKernel.h:92-171;
+ * CPU forms in src/v2/kernels/cpu/moe/CPUMoEKernel.cpp:133-202), for callers that batch tokens
+ * per expert themselves:
+ *   shared_expert_gate    d_shared[t,:] *= sigmoid(dot(d_gate_inp, d_hidden[t,:]))     (sharedExpertGate)
+ *   gather_rows           d_batch[i,:] = d_hidden[d_token_indices[i],:]                (gatherTokenBatch)
+ *   scatter_add_weighted  d_output[d_token_indices[i],:] += d_weights[i] * d_expert_output[i,:], rows
+ *                         taken in ascending i, so repeated indices add up in order   (scatterAddWeighted)
+ *   swiglu_inplace        d_gate[i] = silu(d_gate[i]) * d_up[i]                        (swiGLU)
+ * n_rows bounds the token indices: an index outside [0, n_rows) reads as a row of zeros
+ * (gather) or is skipped (scatter). */
+bool llam_ql_shared_expert_gate(float *d_shared, const float *d_hidden, const float *d_gate_inp,
+                                int n_tokens, int d_model, int device_id, void *stream);
+bool llam_ql_moe_gather_rows(const float *d_hidden, float *d_batch, const int32_t *d_token_indices,
+                             int num_tokens, int n_rows, int d_model, int device_id, void *stream);
+bool llam_ql_moe_scatter_add_weighted(float *d_output, const float *d_expert_output,
+                                      const int32_t *d_token_indices, const float *d_weights,
+                                      int num_tokens, int n_rows, int d_model, int device_id,
+                                      void *stream);
+bool llam_ql_swiglu_inplace(float *d_gate, const float *d_up, long count, int device_id, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

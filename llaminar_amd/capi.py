@@ -87,6 +87,11 @@ SIGNATURES = {
                                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_ids_from_f32": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "llam_ql_shared_expert_add": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_shared_expert_gate": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_gather_rows": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_scatter_add_weighted": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                                  c_void_p]),
+    "llam_ql_swiglu_inplace": (c_bool, [c_void_p, c_void_p, ctypes.c_long, c_int, c_void_p]),
     # decode_api.h
     "llam_dec_embed_q4k": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_dec_rmsnorm_q8_1": (c_bool, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int,

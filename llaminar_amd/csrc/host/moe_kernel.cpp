@@ -405,6 +405,44 @@ namespace llaminar_amd
         return true;
     }
 
+    bool MI355MoEKernel::gatherTokenBatch(const float *hidden, float *batch_buffer, const int *token_indices,
+                                          int num_tokens, int d_model, int num_rows)
+    {
+        static const char *fn = "gatherTokenBatch";
+        if (!valid_)
+            return fail(fn, "operator is not valid");
+        return forward(fn, llam_ql_moe_gather_rows(hidden, batch_buffer, token_indices, num_tokens, num_rows, d_model,
+                                                   device_id_, stream_));
+    }
+
+    bool MI355MoEKernel::scatterAddWeighted(float *output, const float *expert_output, const int *token_indices,
+                                            const float *weights, int num_tokens, int d_model, int num_rows)
+    {
+        static const char *fn = "scatterAddWeighted";
+        if (!valid_)
+            return fail(fn, "operator is not valid");
+        return forward(fn, llam_ql_moe_scatter_add_weighted(output, expert_output, token_indices, weights, num_tokens,
+                                                            num_rows, d_model, device_id_, stream_));
+    }
+
+    bool MI355MoEKernel::sharedExpertGate(const float *input, const float *gate_inp, float *shared_output, int seq_len,
+                                          int d_model)
+    {
+        static const char *fn = "sharedExpertGate";
+        if (!valid_)
+            return fail(fn, "operator is not valid");
+        return forward(fn, llam_ql_shared_expert_gate(shared_output, input, gate_inp, seq_len, d_model, device_id_,
+                                                      stream_));
+    }
+
+    bool MI355MoEKernel::swiGLU(float *gate, const float *up, int count)
+    {
+        static const char *fn = "swiGLU";
+        if (!valid_)
+            return fail(fn, "operator is not valid");
+        return forward(fn, llam_ql_swiglu_inplace(gate, up, count, device_id_, stream_));
+    }
+
     bool MI355MoEKernel::weightedAdd(float *output, const float *input, float weight, int count)
     {
         static const char *fn = "weightedAdd";

@@ -754,6 +754,84 @@ namespace llamql
             out[(size_t)t * d_model + i] += gate * shared[(size_t)t * d_model + i];
     }
 
+    // shared[t,:] *= sigmoid(dot(gate_inp, hidden[t,:])) in place (IMoEKernel::sharedExpertGate,
+    // kernels/cpu/moe/CPUMoEKernel.cpp:162-197).  One workgroup per token.
+    __global__ void __launch_bounds__(256)
+        shared_expert_gate_kernel(float *__restrict__ shared, const float *__restrict__ hidden,
+                                  const float *__restrict__ gate_inp, int d_model)
+    {
+        __shared__ float s_part[256];
+        const int t = blockIdx.x;
+        const float *x = hidden + (size_t)t * d_model;
+        float part = 0.0f;
+        for (int i = threadIdx.x; i < d_model; i += blockDim.x)
+            part = fmaf(gate_inp[i], x[i], part);
+        s_part[threadIdx.x] = part;
+        __syncthreads();
+        for (int off = 128; off > 0; off >>= 1)
+        {
+            if ((int)threadIdx.x < off)
+                s_part[threadIdx.x] += s_part[threadIdx.x + off];
+            __syncthreads();
+        }
+        const float gate = __fdiv_rn(1.0f, 1.0f + expf(-s_part[0]));
+        for (int i = threadIdx.x; i < d_model; i += blockDim.x)
+            shared[(size_t)t * d_model + i] *= gate;
+    }
+
+    // batch[i,:] = hidden[idx[i],:] (IMoEKernel::gatherTokenBatch, CPUMoEKernel.cpp:133-144);
+    // rows whose index is outside [0, n_rows) are filled with zeros.
+    __global__ void __launch_bounds__(256)
+        moe_gather_rows_kernel(const float *__restrict__ hidden, float *__restrict__ batch,
+                               const int32_t *__restrict__ idx, int n_rows, int d_model)
+    {
+        const int i = blockIdx.x;
+        const int src = idx[i];
+        const bool ok = src >= 0 && src < n_rows;
+        for (int c = threadIdx.x; c < d_model; c += blockDim.x)
+            batch[(size_t)i * d_model + c] = ok ? hidden[(size_t)src * d_model + c] : 0.0f;
+    }
+
+    // out[idx[i],:] += w[i] * expert_out[i,:] (IMoEKernel::scatterAddWeighted, CPUMoEKernel.cpp:146-160).
+    // One workgroup per COLUMN block walks the batch rows in ascending order, so rows that name
+    // the same token are added one after the other, as the reference's loop adds them.
+    __global__ void __launch_bounds__(256)
+        moe_scatter_add_weighted_kernel(float *__restrict__ out, const float *__restrict__ expert_out,
+                                        const int32_t *__restrict__ idx, const float *__restrict__ w, int num_tokens,
+                                        int n_rows, int d_model)
+    {
+        const int c = blockIdx.x * blockDim.x + threadIdx.x;
+        if (c >= d_model)
+            return;
+        for (int i = 0; i < num_tokens; ++i)
+        {
+            const int dst = idx[i];
+            if (dst < 0 || dst >= n_rows)
+                continue;
+            float *o = out + (size_t)dst * d_model + c;
+            *o = fmaf(w[i], expert_out[(size_t)i * d_model + c], *o);
+        }
+    }
+
+    // gate[i] = silu(gate[i]) * up[i] in place (IMoEKernel::swiGLU, CPUMoEKernel.cpp:199-202), four
+    // values per thread with the arithmetic of swiglu4.
+    __global__ void __launch_bounds__(256)
+        swiglu_inplace_kernel(float *__restrict__ gate, const float *__restrict__ up, long n4, long n)
+    {
+        const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+        if (i < n4)
+        {
+            float4 *g = reinterpret_cast<float4 *>(gate) + i;
+            *g = swiglu4(*g, reinterpret_cast<const float4 *>(up)[i]);
+        }
+        else if (i < n4 + (n - 4 * n4)) // the last n % 4 values, one thread each
+        {
+            const long e = 4 * n4 + (i - n4);
+            const float4 v = swiglu4(make_float4(gate[e], 0.f, 0.f, 0.f), make_float4(up[e], 0.f, 0.f, 0.f));
+            gate[e] = v.x;
+        }
+    }
+
     namespace
     {
         // matrices: how many [N x SB] matrices the launch walks (slots x tokens x gate|up).
@@ -1227,5 +1305,84 @@ extern "C" bool llam_ql_shared_expert_add(float *d_out, const float *d_shared,
         return false;
     hipLaunchKernelGGL(shared_expert_add_kernel, dim3((unsigned)n_tokens), dim3(256), 0, as_stream(stream),
                        d_out, d_shared, d_hidden, d_gate_inp, d_model);
+    return launched(fn);
+}
+
+extern "C" bool llam_ql_shared_expert_gate(float *d_shared, const float *d_hidden, const float *d_gate_inp,
+                                           int n_tokens, int d_model, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_shared_expert_gate";
+    if (n_tokens < 0 || d_model < 0)
+        return fail(fn, "negative size");
+    if (n_tokens == 0 || d_model == 0)
+        return true;
+    if (!d_shared || !d_hidden || !d_gate_inp)
+        return fail(fn, "null pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(shared_expert_gate_kernel, dim3((unsigned)n_tokens), dim3(256), 0, as_stream(stream), d_shared,
+                       d_hidden, d_gate_inp, d_model);
+    return launched(fn);
+}
+
+extern "C" bool llam_ql_moe_gather_rows(const float *d_hidden, float *d_batch, const int32_t *d_token_indices,
+                                        int num_tokens, int n_rows, int d_model, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_gather_rows";
+    if (num_tokens < 0 || n_rows < 0 || d_model < 0)
+        return fail(fn, "negative size");
+    if (num_tokens == 0 || d_model == 0)
+        return true;
+    if (!d_hidden || !d_batch || !d_token_indices)
+        return fail(fn, "null pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(moe_gather_rows_kernel, dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream), d_hidden,
+                       d_batch, d_token_indices, n_rows, d_model);
+    return launched(fn);
+}
+
+extern "C" bool llam_ql_moe_scatter_add_weighted(float *d_output, const float *d_expert_output,
+                                                 const int32_t *d_token_indices, const float *d_weights,
+                                                 int num_tokens, int n_rows, int d_model, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_scatter_add_weighted";
+    if (num_tokens < 0 || n_rows < 0 || d_model < 0)
+        return fail(fn, "negative size");
+    if (num_tokens == 0 || d_model == 0)
+        return true;
+    if (!d_output || !d_expert_output || !d_token_indices || !d_weights)
+        return fail(fn, "null pointer");
+    if (!set_device(fn, device_id))
+        return false;
+    hipLaunchKernelGGL(moe_scatter_add_weighted_kernel, dim3((unsigned)((d_model + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), d_output, d_expert_output, d_token_indices, d_weights, num_tokens, n_rows,
+                       d_model);
+    return launched(fn);
+}
+
+extern "C" bool llam_ql_swiglu_inplace(float *d_gate, const float *d_up, long count, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_swiglu_inplace";
+    if (count < 0)
+        return fail(fn, "negative size");
+    if (count == 0)
+        return true;
+    if (!d_gate || !d_up)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_gate) || !aligned16(d_up))
+        return fail(fn, "d_gate and d_up must be 16-byte aligned");
+    if (!set_device(fn, device_id))
+        return false;
+    const long n4 = count / 4, work = n4 + (count - 4 * n4);
+    const long grid = (work + 255) / 256;
+    if (grid > 0x7FFFFFFFL)
+        return fail(fn, "count too large for one launch");
+    hipLaunchKernelGGL(swiglu_inplace_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream), d_gate, d_up, n4,
+                       count);
     return launched(fn);
 }

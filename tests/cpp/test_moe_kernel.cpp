@@ -329,6 +329,24 @@ static void test_decode(uint8_t fmt, int T)
         for (int c = 0; c < D; ++c)
             worst = std::max(worst, std::fabs(a3[c] - (a1[c] + 0.25f * a2[c])));
         CHECK(worst <= 1e-6f * std::max(1.0f, std::fabs(a1[0])) + 1e-5f);
+
+        // the token-batching helpers of the interface: gather two rows of o0's buffer (one token
+        // here, so index 0 twice), scatter them back with weights, gate and SwiGLU in place
+        const std::vector<int> idx = {0, 0};
+        const std::vector<float> ws = {0.5f, 0.25f};
+        DevBuf<int> d_idx(idx);
+        DevBuf<float> d_ws(ws), d_batch((size_t)2 * D);
+        CHECK(k.gatherTokenBatch(o0.p, d_batch.p, d_idx.p, 2, D, 1));
+        const std::vector<float> gb = d_batch.download();
+        CHECK(memcmp(gb.data(), a0.data(), D * 4) == 0 && memcmp(gb.data() + D, a0.data(), D * 4) == 0);
+        CHECK(k.scatterAddWeighted(o2.p, d_batch.p, d_idx.p, d_ws.p, 2, D, 1));
+        const std::vector<float> a4 = o2.download();
+        worst = 0.0f;
+        for (int c = 0; c < D; ++c)
+            worst = std::max(worst, std::fabs(a4[c] - (a2[c] + 0.75f * a0[c])));
+        CHECK(worst <= 1e-5f * std::max(1.0f, std::fabs(a2[0])) + 1e-5f);
+        CHECK(!k.gatherTokenBatch(nullptr, d_batch.p, d_idx.p, 2, D, 1));
+        CHECK(contains(moe_kernel_last_error(), "null pointer"));
     }
 
     // errors keep their reason

@@ -328,3 +328,62 @@ def test_shared_expert_gate(capi, dev):
     gate = 1.0 / (1.0 + np.exp(-(h.astype(np.float64) @ gi.astype(np.float64))))
     want = out + gate[:, None] * sh
     assert np.allclose(od.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+
+
+def test_token_batching_helpers(capi, dev, oracle):
+    """The remaining device helpers of the MoE operator interface: gather of token rows into an
+    expert's batch (exact copy, rows with a bad index read as zeros), weighted scatter-add back
+    (rows taken in order, so a token listed twice gets both contributions; bad indices skipped),
+    the shared expert's sigmoid gate in place, and SwiGLU in place (the restatement's values,
+    any count: the last count % 4 values take the scalar path)."""
+    import torch
+
+    lib = capi.load()
+    rng = np.random.default_rng(6)
+    T, D = 7, 2048
+    hidden = rng.standard_normal((T, D)).astype(np.float32)
+    idx = np.array([3, 0, 6, 3, -1, 7, 2], dtype=np.int32)       # 3 twice, two indices out of range
+    hd = torch.from_numpy(hidden).to(dev)
+    idx_d = torch.from_numpy(idx).to(dev)
+    batch = torch.full((len(idx), D), float("nan"), device=dev)
+    assert lib.llam_ql_moe_gather_rows(hd.data_ptr(), batch.data_ptr(), idx_d.data_ptr(), len(idx), T, D, 0, None), \
+        capi.last_error()
+    sync()
+    want = np.stack([hidden[i] if 0 <= i < T else np.zeros(D, np.float32) for i in idx])
+    assert np.array_equal(batch.cpu().numpy(), want)
+
+    expert_out = rng.standard_normal((len(idx), D)).astype(np.float32)
+    w = rng.uniform(0.1, 1.0, len(idx)).astype(np.float32)
+    out0 = rng.standard_normal((T, D)).astype(np.float32)
+    out = torch.from_numpy(out0.copy()).to(dev)
+    assert lib.llam_ql_moe_scatter_add_weighted(out.data_ptr(), torch.from_numpy(expert_out).to(dev).data_ptr(),
+                                                idx_d.data_ptr(), torch.from_numpy(w).to(dev).data_ptr(), len(idx), T,
+                                                D, 0, None), capi.last_error()
+    sync()
+    want = out0.astype(np.float64)
+    for i, t in enumerate(idx):
+        if 0 <= t < T:
+            want[t] += np.float64(w[i]) * expert_out[i]
+    assert np.allclose(out.cpu().numpy(), want, rtol=1e-6, atol=1e-6)
+    assert np.array_equal(out.cpu().numpy()[[1, 4, 5]], out0[[1, 4, 5]])   # tokens no row names are untouched
+
+    sh = rng.standard_normal((T, D)).astype(np.float32)
+    gi = (rng.standard_normal(D) * 0.05).astype(np.float32)
+    shd = torch.from_numpy(sh.copy()).to(dev)
+    assert lib.llam_ql_shared_expert_gate(shd.data_ptr(), hd.data_ptr(), torch.from_numpy(gi).to(dev).data_ptr(), T, D,
+                                          0, None), capi.last_error()
+    sync()
+    gate = 1.0 / (1.0 + np.exp(-(hidden.astype(np.float64) @ gi.astype(np.float64))))
+    assert np.allclose(shd.cpu().numpy(), gate[:, None] * sh, rtol=1e-5, atol=1e-6)
+
+    for count in (4096, 1027, 3):
+        g = (rng.standard_normal(count) * 3).astype(np.float32)
+        u = rng.standard_normal(count).astype(np.float32)
+        gd = torch.from_numpy(g.copy()).to(dev)
+        assert lib.llam_ql_swiglu_inplace(gd.data_ptr(), torch.from_numpy(u).to(dev).data_ptr(), count, 0, None), \
+            capi.last_error()
+        sync()
+        ref = oracle.swiglu(g, u)
+        assert np.allclose(gd.cpu().numpy(), ref, rtol=2e-6, atol=1e-7), count
+    assert not lib.llam_ql_swiglu_inplace(gd.data_ptr() + 4, gd.data_ptr(), 8, 0, None)
+    assert "aligned" in capi.last_error()
