@@ -663,7 +663,10 @@ namespace llamql
                 a.y[i] = pr[j].y;
                 a.N[i] = pr[j].N;
                 a.ldy[i] = pr[j].ldy;
-                a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves).rows_per_wave;
+                // every matrix keeps the rows per wavefront of its own single launch
+                const int resident = j < na ? QA::RESIDENT_WAVES : QB::RESIDENT_WAVES;
+                const int own_max = (j < na ? mta : mtb) / WAVE;
+                a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, own_max, resident).rows_per_wave;
                 cnt[i] = i < n ? ((long)pr[j].N + a.R[i] - 1) / a.R[i] : 0;
                 waves += cnt[i];
             }

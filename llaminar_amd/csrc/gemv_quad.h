@@ -238,7 +238,10 @@ namespace llamql
     {
         static constexpr int SB_BYTES = 144;
         static constexpr int STATIC_LDS = 0;     // bytes of static LDS (decode tables) beside the activations
-        static constexpr int RESIDENT_WAVES = 8; // wavefronts per compute unit the launch shape aims at
+        // wavefronts per compute unit the launch shape may use in one round; with 16 the shape
+        // search also avoids a lone wavefront per SIMD unit (measured on 5120 x 8192: 7.5 us with
+        // seven wavefronts per compute unit against 8.2 us with four)
+        static constexpr int RESIDENT_WAVES = 16;
         __device__ __forceinline__ static void stage() {}
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         // workgroup size bound: one activation row leaves room for 16 wavefronts of 128 registers
@@ -429,7 +432,7 @@ namespace llamql
         typedef int v2i_ __attribute__((ext_vector_type(2)));
         static constexpr int LOADS = 5;
         static constexpr int STATIC_LDS = 0;
-        static constexpr int RESIDENT_WAVES = 8;
+        static constexpr int RESIDENT_WAVES = 16; // (5120 x 25600: 25.9 us with seven wavefronts per compute unit, 27.4 with four)
         __device__ __forceinline__ static void stage() {}
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
         static bool addressable(long N, int SB) { return (double)N * SB * 128.0 < 4.0e9; }
