@@ -56,6 +56,9 @@ int llam_ql_abi_version(void);
  * kernel would be used.  Values <= 0 restore the built-in choice.  Not thread-safe. */
 void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll);
 void llam_ql_reset_gemv_tuning(void);
+/* The same for the matrix-unit kernels of batches 5..8: rows of weight per tile, 16..32;
+ * any other value restores the built-in choice.  No counterpart in the reference. */
+void llam_ql_set_batch_tile_rows(int tile_rows);
 
 /* ---- P1: activation quantiser --------------------------------------------------
  * fp32 [M x K] (row stride K) -> llam_block_q8_1 [M x ceil(K/32)].  d_x 16-byte aligned when

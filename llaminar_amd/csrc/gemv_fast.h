@@ -482,6 +482,7 @@ namespace llamql
         a.SB = SB;
         a.M = M;
         a.slices = sh.slices;
+        a.tile_rows = sh.tile_rows;
         a.sums = d_sums;
         a.row0 = row0;
         a.nrows = nrows;
@@ -531,6 +532,7 @@ namespace llamql
         a.M = M;
         a.slices = sh.slices;
         a.tiles = sh.tiles;
+        a.tile_rows = sh.tile_rows;
         a.chunk = sh.chunk;
         a.sums = d_sums;
         a.row0 = row0;
@@ -600,9 +602,11 @@ namespace llamql
                 a.N[i] = pr[j].N;
                 a.ldy[i] = pr[j].ldy;
                 a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves, F::Quad::RESIDENT_WAVES).rows_per_wave;
+                a.TW[i] = (int)(((long)pr[j].N + a.R[i] - 1) / a.R[i]);
+                a.rows_min[i] = pr[j].N / a.TW[i];
                 a.wave_begin[i] = (int)waves;
                 if (i < n)
-                    waves += ((long)pr[j].N + a.R[i] - 1) / a.R[i];
+                    waves += a.TW[i];
             }
             if (waves > 0x7FFFFFFFL / WAVE)
                 return fail(fn, "too many rows for one launch");
@@ -667,7 +671,9 @@ namespace llamql
                 const int resident = j < na ? QA::RESIDENT_WAVES : QB::RESIDENT_WAVES;
                 const int own_max = (j < na ? mta : mtb) / WAVE;
                 a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, own_max, resident).rows_per_wave;
-                cnt[i] = i < n ? ((long)pr[j].N + a.R[i] - 1) / a.R[i] : 0;
+                a.TW[i] = (int)(((long)pr[j].N + a.R[i] - 1) / a.R[i]);
+                a.rows_min[i] = pr[j].N / a.TW[i];
+                cnt[i] = i < n ? a.TW[i] : 0;
                 waves += cnt[i];
             }
             const long wpc = (waves + cus - 1) / cus;

@@ -28,7 +28,8 @@
 
 namespace llamql
 {
-    constexpr int MFMA_TILE_ROWS = 32;
+    constexpr int MFMA_TILE_ROWS = 32;     // rows of a full tile (columns of the matrix instruction)
+    constexpr int MFMA_MIN_TILE_ROWS = 16; // shortest tile the launch shapes consider
     constexpr int MFMA_MAX_SLICES = 8;
     constexpr int MFMA_MAX_WAVES = 16;     // wavefronts per workgroup
     constexpr int MFMA_DUMP_WAVES = 8;     // the same for the block-sum variant
@@ -47,8 +48,10 @@ namespace llamql
         int N;
         int SB;           // super-blocks per weight row
         int M;            // activation rows, 1..8
-        int slices;       // wavefronts per 32-row tile (wavefront j walks super-blocks j, j + slices, ..);
+        int slices;       // wavefronts per tile (wavefront j walks super-blocks j, j + slices, ..);
                           // a workgroup holds blockDim/64/slices tiles
+        int tile_rows;    // weight rows of a tile, 1..32: fewer than 32 leave columns of the matrix
+                          // instruction unused, and let the tiles of a launch fill every compute unit
         // DUMP kernels only: the exact per-block int32 sums of rows [row0, row0+nrows) go to
         // sums[(m * nrows + row - row0) * (SB * 8) + block]
         int32_t *sums;
@@ -215,15 +218,17 @@ namespace llamql
         // super-blocks (144 bytes each) is asked for by two wavefronts of the workgroup at the
         // same time and crosses the fabric once
         const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
-        const long tile_row0 = ((long)blockIdx.x * tiles_per_wg + tile_local) * MFMA_TILE_ROWS;
+        const long tile_row0 = ((long)blockIdx.x * tiles_per_wg + tile_local) * a.tile_rows;
         const long row = tile_row0 + l32;
+        const bool row_ok = l32 < a.tile_rows && row < a.N;
         const int last_step = nsteps > 0 ? nsteps - 1 : 0;
 
         // piece p = lane + 64 i of the step: 16 bytes at offset 16 (p % 9) of row p / 9.  Rows
-        // past the end of the matrix (and the 32 pieces past the tile) re-read the last row.
+        // past the end of the tile or of the matrix (and the 32 pieces past row 31) re-read the
+        // last row.
         const long base_row = tile_row0 < a.N ? tile_row0 : a.N - 1;
-        const int max_local = (int)(a.N - 1 - base_row) < MFMA_TILE_ROWS - 1 ? (int)(a.N - 1 - base_row)
-                                                                             : MFMA_TILE_ROWS - 1;
+        const int max_local = (int)(a.N - 1 - base_row) < a.tile_rows - 1 ? (int)(a.N - 1 - base_row)
+                                                                          : a.tile_rows - 1;
         uint32_t off[5];
 #pragma unroll
         for (int i = 0; i < 5; ++i)
@@ -268,7 +273,7 @@ namespace llamql
         if constexpr (DUMP)
         {
             const long rr = row - a.row0;
-            if (row < a.N && rr >= 0 && rr < a.nrows)
+            if (row_ok && rr >= 0 && rr < a.nrows)
                 dump_off = (uint32_t)((((size_t)(4 * lh) * a.nrows + (size_t)rr) * (size_t)nkb) * sizeof(int32_t));
         }
         v16i zero;
@@ -403,7 +408,7 @@ namespace llamql
                 const int m = 4 * lh + i;
                 if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
                 {
-                    if (m < a.M && row < a.N)
+                    if (m < a.M && row_ok)
                         a.y[(size_t)m * a.ldy + row] = v;
                 }
             }
@@ -412,7 +417,7 @@ namespace llamql
 
     struct MfmaShape
     {
-        int slices, tiles_per_wg;
+        int slices, tiles_per_wg, tile_rows;
         long grid;
     };
     // Most slices the LDS of a compute unit leaves room for (0: the row is too long for this kernel).
@@ -424,13 +429,15 @@ namespace llamql
         const size_t fit = (QUAD_MAX_LDS - act) / MFMA_BOUNCE;
         return fit < (size_t)MFMA_MAX_SLICES ? (int)fit : MFMA_MAX_SLICES;
     }
-    // Slices so that a compute unit sees about a dozen wavefronts, each at least two
-    // super-blocks long; tiles per workgroup so that every workgroup of the launch is resident
-    // at once (a second round of workgroups would run nearly alone on the chip and cost a
-    // workgroup's whole latency again) and the activations are staged less often.
-    inline MfmaShape gemv_mfma_shape(long N, int nsb, int cus, int max_waves = MFMA_MAX_WAVES)
+    int gemv_mfma_tile_rows_override();
+    // The launch for tiles of `tile_rows` rows.  Slices so that a compute unit sees about a dozen
+    // wavefronts, each at least two super-blocks long; tiles per workgroup so that every workgroup
+    // of the launch is resident at once (a second round of workgroups would run nearly alone on
+    // the chip and cost a workgroup's whole latency again) and the activations are staged less
+    // often.
+    inline MfmaShape gemv_mfma_shape_of(long N, int nsb, int cus, int max_waves, int tile_rows)
     {
-        const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
+        const long tiles = (N + tile_rows - 1) / tile_rows;
         long want = ((long)cus * 12 + tiles - 1) / tiles;
         if (want > mfma_max_slices(nsb))
             want = mfma_max_slices(nsb);
@@ -439,6 +446,7 @@ namespace llamql
         if (want < 1)
             want = 1;
         MfmaShape sh;
+        sh.tile_rows = tile_rows;
         const int per_slice = (int)((nsb + want - 1) / want);
         sh.slices = (nsb + per_slice - 1) / per_slice;
         // workgroups a compute unit holds at once: by LDS, and 16 wavefronts at this kernel's registers
@@ -455,5 +463,29 @@ namespace llamql
         sh.tiles_per_wg = t;
         sh.grid = (tiles + t - 1) / t;
         return sh;
+    }
+    // Tiles of 32 rows use every column of the matrix instruction, but their count rarely fits
+    // the chip: 25600 rows are 800 tiles, 200 workgroups of four, and 56 compute units idle while
+    // the others walk 128 rows each.  A compute unit's time goes with the rows it streams, so the
+    // tile height that leaves the busiest compute unit the fewest rows wins; ties go to the
+    // taller tile.
+    inline MfmaShape gemv_mfma_shape(long N, int nsb, int cus, int max_waves = MFMA_MAX_WAVES)
+    {
+        const int forced = gemv_mfma_tile_rows_override();
+        MfmaShape best;
+        long best_cost = -1;
+        for (int tr = MFMA_TILE_ROWS; tr >= MFMA_MIN_TILE_ROWS; --tr)
+        {
+            if (forced > 0 && tr != forced)
+                continue;
+            const MfmaShape sh = gemv_mfma_shape_of(N, nsb, cus, max_waves, tr);
+            const long cost = ((sh.grid + cus - 1) / cus) * sh.tiles_per_wg * tr; // rows of the busiest compute unit
+            if (best_cost < 0 || cost * 20 < best_cost * 19) // a shorter tile has to win 5 %
+            {
+                best = sh;
+                best_cost = cost;
+            }
+        }
+        return best;
     }
 } // namespace llamql

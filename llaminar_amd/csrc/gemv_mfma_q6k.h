@@ -51,7 +51,8 @@ namespace llamql
         int N;
         int SB;     // super-blocks per weight row
         int M;      // activation rows, 1..8
-        int slices; // compute wavefronts per 32-row tile
+        int slices; // compute wavefronts per tile
+        int tile_rows; // weight rows of a tile, 1..32 (gemv_mfma.h)
         int tiles;  // tiles per workgroup
         int chunk;  // super-blocks per activation buffer; a multiple of slices when SB > chunk
         // DUMP kernels only: the exact per-block int32 sums of rows [row0, row0+nrows) go to
@@ -165,11 +166,11 @@ namespace llamql
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
             const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
             const int last_step = nsteps > 0 ? nsteps - 1 : 0;
-            const long tile_row0 = ((long)blockIdx.x * a.tiles + tile_local) * MFMA_TILE_ROWS;
+            const long tile_row0 = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows;
             const size_t T = (size_t)a.N * nsb;
-            // rows past the end of the matrix re-read the last one
+            // rows past the end of the tile or of the matrix re-read the last one
             auto sb_index = [&](int local_row) {
-                const long r = tile_row0 + local_row;
+                const long r = tile_row0 + (local_row < a.tile_rows ? local_row : a.tile_rows - 1);
                 return (uint32_t)((r < a.N ? r : a.N - 1) * nsb);
             };
             Mfma6Off off;
@@ -218,7 +219,7 @@ namespace llamql
             {
                 const long row = tile_row0 + l32;
                 const long rr = row - a.row0;
-                if (row < a.N && rr >= 0 && rr < a.nrows)
+                if (l32 < a.tile_rows && row < a.N && rr >= 0 && rr < a.nrows)
                     dump_off = (uint32_t)((((size_t)(4 * lh) * a.nrows + (size_t)rr) * ((size_t)nsb * 8)) * sizeof(int32_t));
             }
             v16i zero;
@@ -360,8 +361,8 @@ namespace llamql
         if (wave < ncomp)
         {
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
-            const long row = ((long)blockIdx.x * a.tiles + tile_local) * MFMA_TILE_ROWS + (lane & 31);
-            if (slice == 0)
+            const long row = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows + (lane & 31);
+            if (slice == 0 && (lane & 31) < a.tile_rows)
             {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
@@ -382,15 +383,16 @@ namespace llamql
 
     struct Mfma6Shape
     {
-        int slices, tiles, chunk;
+        int slices, tiles, chunk, tile_rows;
         long grid;
     };
-    // Slices so that a compute unit sees about eight compute wavefronts, five at least (the
-    // scales of eight neighbouring super-blocks share a cache line) and each two steps long;
-    // tiles per workgroup to fill its compute wavefronts when there are tiles to spare.
-    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus, int max_compute = MFMA6_MAX_COMPUTE)
+    // The launch for tiles of `tile_rows` rows.  Slices so that a compute unit sees about eight
+    // compute wavefronts, five at least (the scales of eight neighbouring super-blocks share a
+    // cache line) and each two steps long; tiles per workgroup to fill its compute wavefronts
+    // when there are tiles to spare.
+    inline Mfma6Shape gemv_mfma6_shape_of(long N, int nsb, int cus, int max_compute, int tile_rows)
     {
-        const long tiles = (N + MFMA_TILE_ROWS - 1) / MFMA_TILE_ROWS;
+        const long tiles = (N + tile_rows - 1) / tile_rows;
         long want = ((long)cus * max_compute + tiles - 1) / tiles;
         if (want < 5)
             want = 5;
@@ -401,6 +403,7 @@ namespace llamql
         if (want < 1)
             want = 1;
         Mfma6Shape sh;
+        sh.tile_rows = tile_rows;
         sh.slices = (int)want;
         int t = 1;
         while ((t * 2) * sh.slices <= max_compute && tiles / (t * 2) >= 2L * cus)
@@ -418,5 +421,26 @@ namespace llamql
             sh.chunk = (fit / sh.slices) * sh.slices;
         }
         return sh;
+    }
+    // The tile height that leaves the busiest compute unit the fewest rows (gemv_mfma_shape):
+    // 5120 rows are 160 full tiles, and 256 tiles of 20 rows.
+    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus, int max_compute = MFMA6_MAX_COMPUTE)
+    {
+        const int forced = gemv_mfma_tile_rows_override();
+        Mfma6Shape best;
+        long best_cost = -1;
+        for (int tr = MFMA_TILE_ROWS; tr >= MFMA_MIN_TILE_ROWS; --tr)
+        {
+            if (forced > 0 && tr != forced)
+                continue;
+            const Mfma6Shape sh = gemv_mfma6_shape_of(N, nsb, cus, max_compute, tr);
+            const long cost = ((sh.grid + cus - 1) / cus) * sh.tiles * tr;
+            if (best_cost < 0 || cost * 20 < best_cost * 19) // a shorter tile has to win 5 %
+            {
+                best = sh;
+                best_cost = cost;
+            }
+        }
+        return best;
     }
 } // namespace llamql

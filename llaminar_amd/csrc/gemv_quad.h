@@ -62,7 +62,12 @@ namespace llamql
         float *y[QUAD_MAX_PROJ];
         int N[QUAD_MAX_PROJ];
         int ldy[QUAD_MAX_PROJ];
-        int R[QUAD_MAX_PROJ]; // rows per wavefront
+        int R[QUAD_MAX_PROJ]; // rows per wavefront (the most any wavefront of the matrix walks)
+        // The rows of a matrix are dealt round robin: wavefront j of its TW walks rows j, j + TW, ..
+        // (rows_min of them, one more for the first N - rows_min * TW wavefronts).  At any moment
+        // the wavefronts of the launch then read rows that lie close together in memory.
+        int TW[QUAD_MAX_PROJ];
+        int rows_min[QUAD_MAX_PROJ];
         int wave_begin[QUAD_MAX_PROJ];
         int first_b; // nproj in a launch of one format
         // DUMP kernels only (one matrix): the exact per-block int32 sums of rows [row0, row0+nrows)
@@ -299,15 +304,26 @@ namespace llamql
             c.first = static_cast<const uint8_t *>(a.w) + t_safe * SB_BYTES;
             return c;
         }
-        __device__ __forceinline__ static void advance(Cursor &c, int steps)
+        // What a lane's position moves by from one step to the next (uniform): the step's
+        // super-blocks, and `jump` more when the lane's next super-block lies in the next row.
+        struct Stride
         {
-            c.p += (size_t)steps * (QUAD_STEP_SB * SB_BYTES);
+            size_t plain, cross;
+        };
+        __device__ __forceinline__ static Stride stride(uint32_t jump)
+        {
+            Stride st;
+            st.plain = (size_t)QUAD_STEP_SB * SB_BYTES;
+            st.cross = ((size_t)QUAD_STEP_SB + jump) * SB_BYTES;
+            return st;
         }
-        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, int step, bool valid)
+        __device__ __forceinline__ static void next(Cursor &c, bool cross, const Stride &st)
         {
-            const uint8_t *p = c.p + (size_t)step * (QUAD_STEP_SB * SB_BYTES);
-            if (!valid)
-                p = c.first;
+            c.p += cross ? st.cross : st.plain;
+        }
+        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, bool valid)
+        {
+            const uint8_t *p = valid ? c.p : c.first;
             load(r, p, p + lc.byte_off);
         }
         // super-block sb_off after the cursor's
@@ -485,12 +501,27 @@ namespace llamql
             c.first = (uint32_t)t_safe;
             return c;
         }
-        __device__ __forceinline__ static void advance(Cursor &c, int steps) { c.t += (uint32_t)(steps * QUAD_STEP_SB); }
+        // super-blocks a lane moves by per step, without and with a row crossing (Q4KQuad::Stride)
+        struct Stride
+        {
+            uint32_t plain, cross;
+        };
+        __device__ __forceinline__ static Stride stride(uint32_t jump)
+        {
+            Stride st;
+            st.plain = (uint32_t)QUAD_STEP_SB;
+            st.cross = (uint32_t)QUAD_STEP_SB + jump;
+            return st;
+        }
+        __device__ __forceinline__ static void next(Cursor &c, bool cross, const Stride &st)
+        {
+            c.t += cross ? st.cross : st.plain;
+        }
         __device__ __forceinline__ static int block_of(int l, int which) { return 4 * (l >> 1) + (l & 1) + 2 * which; }
 
-        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, int step, bool valid)
+        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, bool valid)
         {
-            load_index(r, c, lc, valid ? c.t + (uint32_t)(step * QUAD_STEP_SB) : c.first);
+            load_index(r, c, lc, valid ? c.t : c.first);
         }
         __device__ __forceinline__ static void load_at(Raw &r, const Cursor &c, const Lane &lc, int sb_off)
         {
@@ -685,24 +716,33 @@ namespace llamql
         const int ldy = qa.ldy[p];
         const int R = qa.R[p];
 
-        // rows [r0, r1) of this wavefront: one run of `total` super-blocks
-        const long r0 = (long)(wid_all - w_first) * R;
-        long r1 = r0 + R;
-        if (r1 > a.N)
-            r1 = a.N;
-        const int total = r1 > r0 ? (int)(r1 - r0) * nsb : 0; // wavefronts past the last row idle
+        // Rows j, j + TW, .. of this wavefront, walked as ONE run of `total` super-blocks: position
+        // s of the run is super-block s % nsb of the wavefront's row number s / nsb.
+        const long TW = qa.TW[p];
+        const long j = wid_all - w_first;
+        const long with_more = (long)a.N - (long)qa.rows_min[p] * TW; // wavefronts that walk a row more
+        const int nrows = j < TW ? qa.rows_min[p] + (j < with_more ? 1 : 0) : 0; // wavefronts past the last idle
+        const int total = nrows * nsb;
         const int nsteps = (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
 
-        const size_t t0 = (size_t)(total > 0 ? r0 : 0) * nsb + grp;
-        // this lane's last valid super-block of the run (for an idle wavefront: of row 0)
-        const int last_step = total > grp ? (total - 1 - grp) / QUAD_STEP_SB : 0;
-        typename Q::Cursor wc = Q::cursor(a, t0, t0 + (size_t)last_step * QUAD_STEP_SB, lc);
+        // this lane's first super-block; past the end of the run it re-reads its super-block of
+        // the wavefront's last row (an idle wavefront: of row 0)
+        const size_t t0 = (size_t)(nrows > 0 ? j : 0) * nsb + grp;
+        const size_t t_safe = (size_t)(nrows > 0 ? j + (long)(nrows - 1) * TW : 0) * nsb + grp;
+        typename Q::Cursor wc = Q::cursor(a, t0, t_safe, lc);
+        const typename Q::Stride stride = Q::stride((uint32_t)((TW - 1) * nsb));
         int ld_step = 0;
+        int ld_sbr = grp; // where in its row the lane's next load lies (grp < 16 <= nsb)
         auto load_chunk = [&](typename Q::Raw(&buf)[U]) {
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                Q::load(buf[u], wc, lc, u, (ld_step + u) * QUAD_STEP_SB + grp < total);
-            Q::advance(wc, U);
+            {
+                Q::load(buf[u], wc, lc, (ld_step + u) * QUAD_STEP_SB + grp < total);
+                ld_sbr += QUAD_STEP_SB;
+                const bool cross = ld_sbr >= nsb; // the next step's super-block belongs to the next row
+                ld_sbr -= cross ? nsb : 0;
+                Q::next(wc, cross, stride);
+            }
             ld_step += U;
         };
 
@@ -744,7 +784,7 @@ namespace llamql
             cur[m] = 0.0f;
 
         int first = 0;  // super-block (inside its row) that lane group 0 handles in this step
-        long row = r0;  // row `cur` belongs to
+        int row = 0;    // row `cur` belongs to, counted along the run: row j + row * TW of the matrix
         int step = 0;
 
         float *ring = reinterpret_cast<float *>(quad_lds + (size_t)M * aq_stride) +
@@ -763,7 +803,7 @@ namespace llamql
                 sum += dpp_f32<DPP_QUAD_XOR1>(sum);
                 sum += dpp_f32<DPP_QUAD_XOR2>(sum);
                 if (q == 0 && r < slot)
-                    y[(size_t)m * ldy + (row - slot + r)] = sum;
+                    y[(size_t)m * ldy + (size_t)(j + (long)(row - slot + r) * TW)] = sum;
             }
             wave_lds_sync(); // reads done before the ring is written again
             slot = 0;
@@ -782,7 +822,7 @@ namespace llamql
             const int ge = total - step * QUAD_STEP_SB;       // lane groups with data at all
             if constexpr (DUMP)
             {
-                const long rr = (grp < gb ? row : row + 1) - qa.row0;
+                const long rr = j + (long)(grp < gb ? row : row + 1) * TW - qa.row0;
                 if (grp < ge && rr >= 0 && rr < qa.nrows)
                 {
 #pragma unroll
@@ -827,7 +867,7 @@ namespace llamql
                         if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
                         {
                             if (lane == 0)
-                                y[(size_t)m * ldy + row] = tot;
+                                y[(size_t)m * ldy + (size_t)(j + (long)row * TW)] = tot;
                         }
                         cur[m] = fin ? 0.0f : t[m];
                     }

@@ -304,10 +304,25 @@ namespace llamql
             c.first = (uint32_t)t_safe;
             return c;
         }
-        __device__ __forceinline__ static void advance(Cursor &c, int steps) { c.t += (uint32_t)(steps * QUAD_STEP_SB); }
-        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, int step, bool valid)
+        // super-blocks a lane moves by per step, without and with a row crossing (Q4KQuad::Stride)
+        struct Stride
         {
-            load_index(r, c, lc, valid ? c.t + (uint32_t)(step * QUAD_STEP_SB) : c.first);
+            uint32_t plain, cross;
+        };
+        __device__ __forceinline__ static Stride stride(uint32_t jump)
+        {
+            Stride st;
+            st.plain = (uint32_t)QUAD_STEP_SB;
+            st.cross = (uint32_t)QUAD_STEP_SB + jump;
+            return st;
+        }
+        __device__ __forceinline__ static void next(Cursor &c, bool cross, const Stride &st)
+        {
+            c.t += cross ? st.cross : st.plain;
+        }
+        __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, bool valid)
+        {
+            load_index(r, c, lc, valid ? c.t : c.first);
         }
         __device__ __forceinline__ static void load_at(Raw &r, const Cursor &c, const Lane &lc, int sb_off)
         {

@@ -9,9 +9,11 @@ namespace llamql
     {
         int g_rows_per_wave = 0;
         int g_unroll = 0;
+        int g_mfma_tile_rows = 0;
     }
     int gemv_rows_per_wave_override() { return g_rows_per_wave; }
     int gemv_unroll_override() { return g_unroll; }
+    int gemv_mfma_tile_rows_override() { return g_mfma_tile_rows; }
 } // namespace llamql
 
 extern "C" void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll)
@@ -23,4 +25,8 @@ extern "C" void llam_ql_reset_gemv_tuning(void)
 {
     llamql::g_rows_per_wave = 0;
     llamql::g_unroll = 0;
+}
+extern "C" void llam_ql_set_batch_tile_rows(int tile_rows)
+{
+    llamql::g_mfma_tile_rows = tile_rows >= 16 && tile_rows <= 32 ? tile_rows : 0;
 }
