@@ -570,6 +570,11 @@ namespace llamql
     static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU,
                   "activation source kinds");
 
+    // Wavefronts that share the N rows of a matrix when none walks more than R.  (Rows are dealt
+    // round robin, so any count would do; a count rounded up to a whole number per compute unit
+    // measured no faster.)
+    inline int quad_wavefronts(long N, int R, int) { return (int)((N + R - 1) / R); }
+
     // d_sums (one matrix, Q8_1 input): run the block-sum variant over rows [row0, row0+nrows).
     template <class F>
     bool gemv_quad_multi(const char *fn, const QuadProj *pr, int n, const ActSource &src, int M, int K,
@@ -602,7 +607,7 @@ namespace llamql
                 a.N[i] = pr[j].N;
                 a.ldy[i] = pr[j].ldy;
                 a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, max_waves, F::Quad::RESIDENT_WAVES).rows_per_wave;
-                a.TW[i] = (int)(((long)pr[j].N + a.R[i] - 1) / a.R[i]);
+                a.TW[i] = quad_wavefronts(pr[j].N, a.R[i], cus);
                 a.rows_min[i] = pr[j].N / a.TW[i];
                 a.wave_begin[i] = (int)waves;
                 if (i < n)
@@ -671,7 +676,7 @@ namespace llamql
                 const int resident = j < na ? QA::RESIDENT_WAVES : QB::RESIDENT_WAVES;
                 const int own_max = (j < na ? mta : mtb) / WAVE;
                 a.R[i] = gemv_quad_shape(pr[j].N, SB, cus, own_max, resident).rows_per_wave;
-                a.TW[i] = (int)(((long)pr[j].N + a.R[i] - 1) / a.R[i]);
+                a.TW[i] = quad_wavefronts(pr[j].N, a.R[i], cus);
                 a.rows_min[i] = pr[j].N / a.TW[i];
                 cnt[i] = i < n ? a.TW[i] : 0;
                 waves += cnt[i];

@@ -448,7 +448,9 @@ namespace llamql
         typedef int v2i_ __attribute__((ext_vector_type(2)));
         static constexpr int LOADS = 5;
         static constexpr int STATIC_LDS = 0;
-        static constexpr int RESIDENT_WAVES = 16; // (5120 x 25600: 25.9 us with seven wavefronts per compute unit, 27.4 with four)
+        // arithmetic keeps a lone wavefront per SIMD unit busy here (5120 x 25600: 24.3 us with four
+        // wavefronts per compute unit, 25.7 with seven)
+        static constexpr int RESIDENT_WAVES = 8;
         __device__ __forceinline__ static void stage() {}
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
         static bool addressable(long N, int SB) { return (double)N * SB * 128.0 < 4.0e9; }
