@@ -336,7 +336,48 @@ def bench_decode(args, torch, capi, synth, dev):
     return out
 
 
-OTHER_WORKLOADS = {"gemm": bench_gemm, "moe": bench_moe, "gemv": bench_gemv, "decode": bench_decode}
+def bench_read_order(args, torch, capi, synth, dev):
+    """What the order of a GEMV's reads is worth on its own: read-only kernels over 25600 x 5120 Q4_K-sized buffers
+    (73.7 MB each, eight rotated so nothing is served from a previous launch), no arithmetic."""
+    lib = capi.load()
+    N, K = FFN, HIDDEN
+    nbytes = N * (K // 256) * 144
+    bufs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(8)]
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = torch.cuda.Stream()
+    # (label, pattern, rows per wavefront, wavefronts per workgroup, depth, workgroups)
+    cases = [("quad-lane loads, 13 contiguous rows per wavefront, 2 steps in flight", 0, 13, 8, 2, 0),
+             ("quad-lane loads, rows dealt round robin, 2 steps in flight", 1, 13, 8, 2, 0),
+             ("quad-lane loads, contiguous rows, 1 step in flight", 0, 13, 8, 1, 0),
+             ("quad-lane loads, round robin, 1 step in flight", 1, 13, 8, 1, 0),
+             ("quad-lane loads, contiguous rows, 4 steps in flight", 0, 13, 8, 4, 0),
+             ("quad-lane loads, round robin, 4 steps in flight", 1, 13, 8, 4, 0),
+             ("quad-lane loads, 7 contiguous rows, 16 wavefronts, 1 step in flight", 0, 7, 16, 1, 0),
+             ("quad-lane loads, 7 rows round robin, 16 wavefronts, 1 step in flight", 1, 7, 16, 1, 0),
+             ("1 KB stream, region per wavefront, 256 x 1024 threads, 3 loads in flight", 2, 0, 16, 3, 256),
+             ("1 KB stream, grid-stride, 256 x 1024 threads, 3 loads in flight", 3, 0, 16, 3, 256),
+             ("1 KB stream, region per wavefront, 256 x 1024 threads, 6 loads in flight", 2, 0, 16, 6, 256),
+             ("1 KB stream, grid-stride, 256 x 1024 threads, 6 loads in flight", 3, 0, 16, 6, 256),
+             ("1 KB stream, grid-stride, 256 x 1024 threads, 9 loads in flight", 3, 0, 16, 9, 256)]
+    rows = []
+    with torch.cuda.stream(stream):
+        for label, pattern, rpw, wpw, depth, wgs in cases:
+            def launch(i):
+                ok = lib.llam_ql_read_probe(bufs[i % 8].data_ptr(), N, K, pattern, rpw, wpw, depth, wgs,
+                                            sink.data_ptr(), 0, stream.cuda_stream)
+                assert ok, capi.last_error()
+            us = min(_time_launches(torch, stream, launch, args.steps, 20) for _ in range(3))
+            rows.append({"pattern": label, "us": round(us, 2), "frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+    best = min(rows, key=lambda r: r["us"])
+    gbs = round(nbytes / (best["us"] * 1e-6) / 1e9, 1)
+    return _common(args, "read-only stream GB/s by order of reads", gbs, "GB/s", round(best["us"] * 1e-3, 5), "u8",
+                   {"workload": "read-only probes over 25600 x 5120 Q4_K-sized buffers (73.7 MB), 8 rotated", "patterns": rows},
+                   {"kernel": best["pattern"], "bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": best["frac"], "traffic": None, "us_per_launch": best["us"], "launches_timed": args.steps})
+
+
+OTHER_WORKLOADS = {"gemm": bench_gemm, "moe": bench_moe, "gemv": bench_gemv, "decode": bench_decode,
+                   "read-order": bench_read_order}
 
 
 def parse():
@@ -346,9 +387,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--moe-path", choices=["auto", "slots", "grouped-gate-up", "grouped"], default="auto",
                     help="moe workload: per-slot launches, or tokens grouped by expert (gate/up only, or down as well)")
-    ap.add_argument("--workload", choices=["layer", "gemm", "moe", "gemv", "decode"], default="layer",
+    ap.add_argument("--workload", choices=["layer", "gemm", "moe", "gemv", "decode", "read-order"], default="layer",
                     help="layer: the headline decode-layer step (default); gemm: prefill int8 GEMM 512x25600x5120 Q4_K; "
-                         "moe: 256-expert top-8 IQ3_S expert FFN decode; gemv: single GEMVs of every format and layer shape")
+                         "moe: 256-expert top-8 IQ3_S expert FFN decode; gemv: single GEMVs of every format and layer shape; "
+                         "read-order: read-only probes of the GEMV's load stream in several orders")
     ap.add_argument("--batch", type=int, default=1, help="activation rows / tokens per step")
     ap.add_argument("--layers", type=int, default=4, help="distinct weight sets rotated through")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")

@@ -60,6 +60,24 @@ void llam_ql_reset_gemv_tuning(void);
  * any other value restores the built-in choice.  No counterpart in the reference. */
 void llam_ql_set_batch_tile_rows(int tile_rows);
 
+/* Read-only probe for measurements: streams the N * (K/256) * 144 bytes of a Q4_K-sized
+ * buffer once and computes nothing, in the order a decode GEMV would read them.  No
+ * counterpart in the reference.
+ *   ROWS_*: the quad-lane kernel's loads (4 lanes per super-block, 3 x 16 bytes per lane and
+ *     step), N rows shared by ceil(N / rows_per_wave) wavefronts, each with its rows
+ *     contiguous or dealt round robin; depth = steps in flight per wavefront (1, 2, 4);
+ *     `workgroups` is ignored.
+ *   STREAM_*: 1 KB per load instruction, `workgroups` workgroups, a region per wavefront or
+ *     grid-stride; depth = loads in flight per lane (3, 6, 9); rows_per_wave is ignored.
+ * d_sink: one int the kernels may write. */
+#define LLAM_QL_PROBE_ROWS_CONTIGUOUS 0
+#define LLAM_QL_PROBE_ROWS_ROUND_ROBIN 1
+#define LLAM_QL_PROBE_STREAM_REGION 2
+#define LLAM_QL_PROBE_STREAM_GRID_STRIDE 3
+bool llam_ql_read_probe(const void *d_buf, int N, int K, int pattern, int rows_per_wave,
+                        int waves_per_wg, int depth, int workgroups, int *d_sink, int device_id,
+                        void *stream);
+
 /* ---- P1: activation quantiser --------------------------------------------------
  * fp32 [M x K] (row stride K) -> llam_block_q8_1 [M x ceil(K/32)].  d_x 16-byte aligned when
  * K % 32 == 0 (every shape the GEMV and GEMM entry points take), 4-byte aligned otherwise: a row's

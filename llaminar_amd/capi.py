@@ -49,6 +49,7 @@ SIGNATURES = {
     "llam_ql_set_gemv_tuning": (None, [c_int, c_int]),
     "llam_ql_reset_gemv_tuning": (None, []),
     "llam_ql_set_batch_tile_rows": (None, [c_int]),
+    "llam_ql_read_probe": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_quantize_q8_1": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_prepared_bytes": (c_size_t, [c_uint8, c_int, c_int]),
     "llam_ql_prepare_weights": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
