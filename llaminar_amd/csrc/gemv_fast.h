@@ -625,9 +625,11 @@ namespace llamql
                 nw = 1;
             const long grid = (waves + nw - 1) / nw;
             size_t lds = quad_lds_bytes(M, SB);
-            a.ring = M == 1 && !d_sums && lds + (size_t)nw * QUAD_RING_BYTES + F::Quad::STATIC_LDS <= QUAD_MAX_LDS;
+            // (the ring must not cost a compute unit one of the workgroups it would hold at once)
+            a.ring = M <= QUAD_RING_MAX_M && !d_sums &&
+                     (size_t)wgs_per_cu * (lds + (size_t)nw * M * QUAD_RING_BYTES + F::Quad::STATIC_LDS) <= QUAD_MAX_LDS;
             if (a.ring)
-                lds += (size_t)nw * QUAD_RING_BYTES;
+                lds += (size_t)nw * M * QUAD_RING_BYTES;
             gemv_quad_launch<typename F::Quad>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
             return launched(fn);
         }
@@ -700,9 +702,10 @@ namespace llamql
                 return fail(fn, "too many rows for one launch");
             const long grid = (at + nw - 1) / nw;
             size_t lds = quad_lds_bytes(M, SB);
-            a.ring = M == 1 && lds + (size_t)nw * QUAD_RING_BYTES <= QUAD_MAX_LDS;
+            a.ring = M <= QUAD_RING_MAX_M &&
+                     (size_t)wgs_per_cu * (lds + (size_t)nw * M * QUAD_RING_BYTES) <= QUAD_MAX_LDS;
             if (a.ring)
-                lds += (size_t)nw * QUAD_RING_BYTES;
+                lds += (size_t)nw * M * QUAD_RING_BYTES;
             gemv_quad_dual_launch<QA, QB>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
             return launched(fn);
         }

@@ -74,8 +74,8 @@ namespace llamql
         // go to sums[(m * nrows + row - row0) * (SB * 8) + block]
         int32_t *sums;
         int row0, nrows;
-        // single activation row: the launch reserves QUAD_RING_BYTES of LDS per wavefront behind
-        // the activations and the kernel runs in QUAD_MODE_RING
+        // up to QUAD_RING_MAX_M activation rows: the launch reserves QUAD_RING_BYTES of LDS per
+        // wavefront and row behind the activations and the kernel runs in QUAD_MODE_RING
         int ring;
     };
 
@@ -88,7 +88,8 @@ namespace llamql
     // (pairs, quads, eights, sixteens, then (r0+r1)+(r2+r3)): the same bits either way.
     constexpr int QUAD_RING_ROWS = 16;
     constexpr int QUAD_RING_STRIDE = 68; // floats per parked row: 64 + 4 so neighbouring rows start 4 banks apart
-    constexpr size_t QUAD_RING_BYTES = (size_t)QUAD_RING_ROWS * QUAD_RING_STRIDE * 4;
+    constexpr size_t QUAD_RING_BYTES = (size_t)QUAD_RING_ROWS * QUAD_RING_STRIDE * 4; // per wavefront and activation row
+    constexpr int QUAD_RING_MAX_M = 4; // batches that may run in QUAD_MODE_RING (where the LDS has the room)
     inline size_t quad_lds_bytes(int M, int nsb)
     {
         return (size_t)M * (size_t)nsb * QUAD_SB_LDS;
@@ -967,7 +968,7 @@ namespace llamql
             gemv_quad_launch_mus<Q, M, U, QUAD_SRC_Q8, QUAD_MODE_DUMP>(grid, block, lds, st, a);
             return;
         }
-        if constexpr (M == 1)
+        if constexpr (M <= QUAD_RING_MAX_M)
         {
             if (a.ring)
             {
@@ -1027,7 +1028,7 @@ namespace llamql
     template <class QA, class QB, int M, int SRC>
     inline void gemv_quad_dual_launch_ms(dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
-        if constexpr (M == 1)
+        if constexpr (M <= QUAD_RING_MAX_M)
         {
             if (a.ring)
             {
