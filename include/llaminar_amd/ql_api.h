@@ -184,6 +184,32 @@ bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,
                              int32_t *d_sums, int M, int N, int K, int row0,
                              int nrows, int device_id, void *stream);
 
+/* d_y[m, n] += dot(W[n, :], x[m, :]): llam_ql_gemv whose row sums are added (one fp32 add each) to
+ * what d_y holds -- the residual add in front of the next norm (fused_residual_rmsnorm_row_*,
+ * RMSNormPrimitives.cpp:1491-1562) done by the projection that produces the delta, with the bits of
+ * llam_ql_gemv followed by that add.  Served where llam_ql_gemv_accumulate_supported says so
+ * (a single quad-lane launch that reduces its rows in LDS); elsewhere the call fails and the
+ * caller keeps the delta in a buffer of its own. */
+bool llam_ql_gemv_accumulate_supported(uint8_t fmt, int M, int N, int K, int device_id);
+bool llam_ql_gemv_accumulate(uint8_t fmt, const void *d_w, const void *d_q8, float *d_y, int M,
+                             int N, int K, int ldy, int device_id, void *stream);
+
+/* RMSNorm, Q8_1 quantiser and the projections of the normalised row in the projections' own
+ * launches: every workgroup normalises and quantises the M rows for itself (rows of a few
+ * thousand floats), which saves the norm's launch.
+ *     v = d_x[m] (+ d_delta[m] when d_delta is given; then d_x_out[m] = v, d_x is not written)
+ *     y = (v * (1/rms)) * gamma,  rms = sqrt(float(sum_sq / K) + eps), sum_sq in double
+ *     projections of the Q8_1 blocks of y, as llam_ql_gemv_fused
+ * with the bits of llam_dec_rmsnorm_q8_1 followed by llam_ql_gemv_fused (the fused form of
+ * CPURMSNormKernelT<FP32>::apply_with_residual_add, CPURMSNormKernelT.h:300-322, in front of the
+ * activation quantiser).  Rows of d_x, d_delta and d_x_out are K floats apart.  Served where
+ * llam_ql_gemv_fused_rmsnorm_supported says so (M <= 4, rows the quad-lane kernel takes);
+ * elsewhere the call fails and the norm and the projections run as two calls. */
+bool llam_ql_gemv_fused_rmsnorm_supported(const llam_ql_proj *projs, int num, int M, int K);
+bool llam_ql_gemv_fused_rmsnorm(const llam_ql_proj *projs, int num, const float *d_x,
+                                const float *d_delta, const float *d_gamma, float eps,
+                                float *d_x_out, int M, int K, int device_id, void *stream);
+
 /* What llam_ql_gemv does with a shape: which kernel runs, how the batch and the row are
  * split.  For tests, tuning and the operator's decode-equivalence guard; the launcher
  * executes exactly this plan.  (Reference: the dispatch tables behind

@@ -59,6 +59,11 @@ SIGNATURES = {
                                   c_int, c_void_p]),
     "llam_ql_gemv_f32_static": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int,
                                          c_int, c_void_p]),
+    "llam_ql_gemv_accumulate_supported": (c_bool, [c_uint8, c_int, c_int, c_int, c_int]),
+    "llam_ql_gemv_accumulate": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv_fused_rmsnorm_supported": (c_bool, [POINTER(Proj), c_int, c_int, c_int]),
+    "llam_ql_gemv_fused_rmsnorm": (c_bool, [POINTER(Proj), c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
+                                            c_int, c_int, c_void_p]),
     "llam_ql_gemv_fused_f32": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int,
                                         c_void_p]),
     "llam_ql_gemv_swiglu_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
@@ -255,6 +260,35 @@ def gemv_fused_f32(projs, x, M: int, K: int, q8_scratch=None, stream=None):
         arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], _ld(out), fmt)
     _check(load().llam_ql_gemv_fused_f32(arr, len(projs), _ptr(x), _ld(x), M, K, _ptr(q8_scratch), _dev(x),
                                          _stream(stream)), "gemv_fused_f32")
+
+
+def gemv_accumulate_supported(fmt: int, M: int, N: int, K: int, device: int = 0) -> bool:
+    return bool(load().llam_ql_gemv_accumulate_supported(fmt, M, N, K, device))
+
+
+def gemv_accumulate(fmt: int, w, q8, M: int, N: int, K: int, out, stream=None):
+    """out[M,N] += Q8_1 activations times W^T, inside the GEMV's launch."""
+    _check(load().llam_ql_gemv_accumulate(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, _ld(out), _dev(w),
+                                          _stream(stream)), "gemv_accumulate")
+    return out
+
+
+def _proj_array(projs):
+    arr = (Proj * len(projs))()
+    for i, (fmt, w, out) in enumerate(projs):
+        arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], _ld(out), fmt)
+    return arr
+
+
+def gemv_fused_rmsnorm_supported(projs, M: int, K: int) -> bool:
+    """Whether every projection of the list (fmt, w, out[M,N]) can run the norm inside its own kernel."""
+    return bool(load().llam_ql_gemv_fused_rmsnorm_supported(_proj_array(projs), len(projs), M, K))
+
+
+def gemv_fused_rmsnorm(projs, x, delta, gamma, eps: float, x_out, M: int, K: int, stream=None):
+    """projs: list of (fmt, w, out[M,N]) on RMSNorm(x (+ delta)) * gamma; x + delta goes to x_out."""
+    _check(load().llam_ql_gemv_fused_rmsnorm(_proj_array(projs), len(projs), _ptr(x), _ptr(delta), _ptr(gamma), eps,
+                                             _ptr(x_out), M, K, _dev(x), _stream(stream)), "gemv_fused_rmsnorm")
 
 
 def gemv_swiglu_f32(fmt: int, w, gate, up, M: int, N: int, K: int, out=None, q8_scratch=None, stream=None):

@@ -112,6 +112,51 @@ namespace llamql
         }
     } // namespace
 
+    // Whether a projection of this shape can take its activations from the norm fused into the
+    // quad-lane kernel (ACT_SRC_RMSNORM).
+    bool gemv_norm_fusable(uint8_t fmt, int M, int N, int K)
+    {
+        if (M < 1 || M > QUAD_NORM_MAX_M)
+            return false;
+        switch (fmt)
+        {
+        case LLAM_FMT_Q4_K: return quad_eligible<Q4KTraits>(M, N, K) && quad_lds_bytes(M, K / 256) + QUAD_NORM_LDS <= QUAD_MAX_LDS;
+        case LLAM_FMT_Q6_K: return quad_eligible<Q6KTraits>(M, N, K) && quad_lds_bytes(M, K / 256) + QUAD_NORM_LDS <= QUAD_MAX_LDS;
+        case LLAM_FMT_IQ3_S:
+            return quad_eligible<IQ3STraits>(M, N, K) &&
+                   quad_lds_bytes(M, K / 256) + QUAD_NORM_LDS + IQ3STraits::Quad::STATIC_LDS <= QUAD_MAX_LDS;
+        default: return false;
+        }
+    }
+
+    namespace
+    {
+        template <class F>
+        bool accumulate_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int M, int N, int K,
+                               int ldy, int device_id, hipStream_t st, bool query)
+        {
+            const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
+            if (p.kernel != GEMV_KERNEL_QUAD || p.m_first < M)
+                return query ? false : fail(fn, "M=%d N=%d K=%d: not a single quad-lane launch", M, N, K);
+            const QuadProj pr{d_w, d_y, N, ldy};
+            return gemv_quad_multi<F>(fn, &pr, 1, act_source_q8(d_q8), M, K, device_id, st, nullptr, 0, 0,
+                                      query ? QUAD_ACC_QUERY : QUAD_ACC_LAUNCH);
+        }
+    } // namespace
+
+    // y += W a in the GEMV's own launch (query: only whether the shape's launch can do that).
+    bool gemv_accumulate(const char *fn, uint8_t fmt, const void *d_w, const void *d_q8, float *d_y, int M, int N,
+                         int K, int ldy, int device_id, hipStream_t st, bool query)
+    {
+        switch (fmt)
+        {
+        case LLAM_FMT_Q4_K: return accumulate_launch<Q4KTraits>(fn, d_w, d_q8, d_y, M, N, K, ldy, device_id, st, query);
+        case LLAM_FMT_Q6_K: return accumulate_launch<Q6KTraits>(fn, d_w, d_q8, d_y, M, N, K, ldy, device_id, st, query);
+        case LLAM_FMT_IQ3_S: return accumulate_launch<IQ3STraits>(fn, d_w, d_q8, d_y, M, N, K, ldy, device_id, st, query);
+        default: return false;
+        }
+    }
+
     // Launches the longest run of projections at the head of `projs` (same format, all fit
     // for the quad-lane kernel) as ONE kernel.  Returns how many it covered, 0 when the
     // first projection has to go through its own launch on Q8_1 input, -1 on error.

@@ -567,7 +567,8 @@ namespace llamql
             return gemv_mfma_q4k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
     }
 
-    static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU,
+    static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU &&
+                      ACT_SRC_RMSNORM == QUAD_SRC_RMSNORM,
                   "activation source kinds");
 
     // Wavefronts that share the N rows of a matrix when none walks more than R.  (Rows are dealt
@@ -576,9 +577,14 @@ namespace llamql
     inline int quad_wavefronts(long N, int R, int) { return (int)((N + R - 1) / R); }
 
     // d_sums (one matrix, Q8_1 input): run the block-sum variant over rows [row0, row0+nrows).
+    // accumulate (one matrix): QUAD_ACC_LAUNCH adds the row sums to what the output holds, which the
+    // kernel can do where it reduces rows through the ring and a wavefront's rows fit one flush;
+    // QUAD_ACC_QUERY only answers whether this launch could (no launch, no error text).
+    constexpr int QUAD_ACC_NONE = 0, QUAD_ACC_LAUNCH = 1, QUAD_ACC_QUERY = 2;
     template <class F>
     bool gemv_quad_multi(const char *fn, const QuadProj *pr, int n, const ActSource &src, int M, int K,
-                         int device_id, hipStream_t st, int32_t *d_sums = nullptr, int row0 = 0, int nrows = 0)
+                         int device_id, hipStream_t st, int32_t *d_sums = nullptr, int row0 = 0, int nrows = 0,
+                         int accumulate = QUAD_ACC_NONE)
     {
         if constexpr (F::USE_QUAD)
         {
@@ -590,6 +596,10 @@ namespace llamql
             a.x = src.x;
             a.x2 = src.x2;
             a.ldx = src.ldx;
+            a.gamma = src.gamma;
+            a.x_out = src.x_out;
+            a.eps = src.eps;
+            a.norm_lds = 0;
             a.SB = SB;
             a.nproj = n;
             a.first_b = n;
@@ -625,11 +635,29 @@ namespace llamql
                 nw = 1;
             const long grid = (waves + nw - 1) / nw;
             size_t lds = quad_lds_bytes(M, SB);
+            const size_t norm = src.kind == ACT_SRC_RMSNORM ? QUAD_NORM_LDS : 0;
+            if (norm && M > QUAD_NORM_MAX_M)
+                return fail(fn, "the fused norm serves batches of 1..%d", QUAD_NORM_MAX_M);
             // (the ring must not cost a compute unit one of the workgroups it would hold at once)
             a.ring = M <= QUAD_RING_MAX_M && !d_sums &&
-                     (size_t)wgs_per_cu * (lds + (size_t)nw * M * QUAD_RING_BYTES + F::Quad::STATIC_LDS) <= QUAD_MAX_LDS;
+                     (size_t)wgs_per_cu * (lds + norm + (size_t)nw * M * QUAD_RING_BYTES + F::Quad::STATIC_LDS) <=
+                         QUAD_MAX_LDS;
             if (a.ring)
                 lds += (size_t)nw * M * QUAD_RING_BYTES;
+            a.norm_lds = (int)lds;
+            lds += norm;
+            if (lds + F::Quad::STATIC_LDS > QUAD_MAX_LDS)
+                return fail(fn, "K=%d: %d activation row(s) and the norm's scratch do not fit the LDS", K, M);
+            a.accumulate = 0;
+            if (accumulate != QUAD_ACC_NONE)
+            {
+                const bool can = n == 1 && a.ring && a.R[0] <= QUAD_RING_ROWS;
+                if (accumulate == QUAD_ACC_QUERY)
+                    return can;
+                if (!can)
+                    return fail(fn, "M=%d N=%d K=%d: this launch cannot add to its output", M, pr[0].N, K);
+                a.accumulate = 1;
+            }
             gemv_quad_launch<typename F::Quad>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
             return launched(fn);
         }
@@ -661,11 +689,16 @@ namespace llamql
             a.x = src.x;
             a.x2 = src.x2;
             a.ldx = src.ldx;
+            a.gamma = src.gamma;
+            a.x_out = src.x_out;
+            a.eps = src.eps;
+            a.norm_lds = 0;
             a.SB = SB;
             a.nproj = n;
             a.first_b = na;
             a.sums = nullptr;
             a.row0 = a.nrows = 0;
+            a.accumulate = 0;
             long cnt[QUAD_MAX_PROJ], waves = 0;
             for (int i = 0; i < QUAD_MAX_PROJ; ++i)
             {
@@ -702,10 +735,17 @@ namespace llamql
                 return fail(fn, "too many rows for one launch");
             const long grid = (at + nw - 1) / nw;
             size_t lds = quad_lds_bytes(M, SB);
+            const size_t norm = src.kind == ACT_SRC_RMSNORM ? QUAD_NORM_LDS : 0;
+            if (norm && M > QUAD_NORM_MAX_M)
+                return fail(fn, "the fused norm serves batches of 1..%d", QUAD_NORM_MAX_M);
             a.ring = M <= QUAD_RING_MAX_M &&
-                     (size_t)wgs_per_cu * (lds + (size_t)nw * M * QUAD_RING_BYTES) <= QUAD_MAX_LDS;
+                     (size_t)wgs_per_cu * (lds + norm + (size_t)nw * M * QUAD_RING_BYTES) <= QUAD_MAX_LDS;
             if (a.ring)
                 lds += (size_t)nw * M * QUAD_RING_BYTES;
+            a.norm_lds = (int)lds;
+            lds += norm;
+            if (lds > QUAD_MAX_LDS)
+                return fail(fn, "K=%d: %d activation row(s) and the norm's scratch do not fit the LDS", K, M);
             gemv_quad_dual_launch<QA, QB>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
             return launched(fn);
         }

@@ -43,6 +43,11 @@ namespace llamql
     constexpr int QUAD_SRC_Q8 = 0;     // Q8_1 blocks
     constexpr int QUAD_SRC_F32 = 1;    // fp32 rows
     constexpr int QUAD_SRC_SWIGLU = 2; // silu(gate) * up of two fp32 inputs
+    constexpr int QUAD_SRC_RMSNORM = 3; // RMSNorm of fp32 residual rows (+ delta), batches of 1..QUAD_NORM_MAX_M
+    // (every workgroup normalises and quantises all rows again: measured against a norm launch of
+    // its own, 3.4 us, that pays for a single row of 5120 and no longer for four)
+    constexpr int QUAD_NORM_MAX_M = 1;
+    constexpr int QUAD_NORM_LDS = 8 * 8 * QUAD_NORM_MAX_M; // LDS bytes of the norm's partial sums
 
     // One launch: up to QUAD_MAX_PROJ weight matrices of one row length against the same
     // activations (projections that share an input: Q, K and V; gate and up).  The
@@ -56,6 +61,13 @@ namespace llamql
         const float *x;     // fp32 activations, M rows of ldx floats (QUAD_SRC_F32); the gate
         const float *x2;    // rows for QUAD_SRC_SWIGLU, whose up rows are x2
         int ldx;
+        // QUAD_SRC_RMSNORM: x are the residual rows, x2 the delta rows added first (or null), gamma the
+        // norm's weights; workgroup 0 stores x + delta to x_out (when there is a delta).  The
+        // partial sums of squares live in QUAD_NORM_LDS bytes of LDS at byte offset norm_lds.
+        const float *gamma;
+        float *x_out;
+        float eps;
+        int norm_lds;
         int SB;             // super-blocks per weight row
         int nproj;
         const void *w[QUAD_MAX_PROJ];
@@ -77,6 +89,9 @@ namespace llamql
         // up to QUAD_RING_MAX_M activation rows: the launch reserves QUAD_RING_BYTES of LDS per
         // wavefront and row behind the activations and the kernel runs in QUAD_MODE_RING
         int ring;
+        // QUAD_MODE_RING only, wavefronts of at most QUAD_RING_ROWS rows: the row sums are ADDED to what
+        // y holds (y += W a: the residual add of the next norm done by the projection that feeds it)
+        int accumulate;
     };
 
     // LDS bytes for M activation rows of nsb super-blocks.
@@ -184,6 +199,24 @@ namespace llamql
         }
     }
 
+    // One lane's share (float4 number i of the row) of a quantised 32-element block into the
+    // activation row at aq_row, in the layout the decoder Q reads.
+    template <class Q>
+    __device__ __forceinline__ void quad_store_q8_lane(const Q8Lane q, int i, uint8_t *aq_row)
+    {
+        const int kb = i >> 3, sub = i & 7;
+        const int sb = kb >> 3, j = kb & 7;
+        int l, odd;
+        Q::owner(j, l, odd);
+        uint8_t *base = aq_row + sb * QUAD_SB_LDS + l * 16;
+        if (sub == 0)
+        {
+            const float d = h2f((uint16_t)(q.head & 0xFFFFu));
+            *reinterpret_cast<float2 *>(base + 256 + odd * 8) = make_float2(d, (float)(int16_t)(q.head >> 16) * d);
+        }
+        *reinterpret_cast<uint32_t *>(base + (odd * 2 + (sub >> 2)) * 64 + (sub & 3) * 4) = q.packed;
+    }
+
     // The same from fp32 rows (SRC = QUAD_SRC_F32) or from silu(x) * x2 (QUAD_SRC_SWIGLU):
     // eight neighbouring threads quantise one 32-element block.
     template <class Q, int M, int SRC>
@@ -217,21 +250,159 @@ namespace llamql
                         break;
                     if constexpr (SRC == QUAD_SRC_SWIGLU)
                         v[u] = swiglu4(v[u], v2[u]);
-                    const Q8Lane q = q8_1_quantize_lane(v[u]);
-                    const int kb = i >> 3, sub = i & 7;
-                    const int sb = kb >> 3, j = kb & 7;
-                    int l, odd;
-                    Q::owner(j, l, odd);
-                    uint8_t *base = aq + m * aq_stride + sb * QUAD_SB_LDS + l * 16;
-                    if (sub == 0)
-                    {
-                        const float d = h2f((uint16_t)(q.head & 0xFFFFu));
-                        *reinterpret_cast<float2 *>(base + 256 + odd * 8) =
-                            make_float2(d, (float)(int16_t)(q.head >> 16) * d);
-                    }
-                    *reinterpret_cast<uint32_t *>(base + (odd * 2 + (sub >> 2)) * 64 + (sub & 3) * 4) = q.packed;
+                    quad_store_q8_lane<Q>(q8_1_quantize_lane(v[u]), i, aq + m * aq_stride);
                 }
             }
+        }
+    }
+
+    // RMSNorm of the residual rows in front of the quantiser (QUAD_SRC_RMSNORM), with the bits of the
+    // stand-alone operator (rmsnorm_q8_1_kernel: 512 threads, thread t sums the squares of float4
+    // t, t + 512, .. in double, the 64 lanes of a wavefront are added as a butterfly, the eight
+    // wavefronts in order).  Here the threads of the workgroup play those 512 "virtual threads",
+    // every workgroup of the launch for itself.  Workgroups of 512 threads and more on rows of up to
+    // 8192 values keep a virtual thread's values and weights in registers between the sum and the
+    // scaling (all loads are issued before the sum, nothing is read twice); the others play the
+    // virtual threads in turn, whole wavefronts at a time, and read the row again from the caches.
+    // Contains a workgroup barrier.
+    template <class Q, int M>
+    __device__ __forceinline__ void quad_stage_rmsnorm(const QuadArgs &qa, int nsb, uint8_t *aq, int aq_stride,
+                                                       uint8_t *quad_lds)
+    {
+        constexpr int VT = 512; // threads of the stand-alone kernel
+        constexpr int KEEP = 4; // float4 of a virtual thread kept in registers
+        const int H = nsb * 256, nvec = nsb * 64;
+        double *s_part = reinterpret_cast<double *>(quad_lds + qa.norm_lds); // [M][8]
+        // (the workgroup that stores x + delta: a variant that added a workgroup without rows for it
+        // measured the same)
+        const bool writer = blockIdx.x == 0 && qa.x2 != nullptr && qa.x_out != nullptr;
+        const float4 *g4 = reinterpret_cast<const float4 *>(qa.gamma);
+        auto add4 = [](float4 v, const float4 d) {
+            v.x += d.x;
+            v.y += d.y;
+            v.z += d.z;
+            v.w += d.w;
+            return v;
+        };
+        auto row_value = [&](int m, int i) {
+            const float4 v = reinterpret_cast<const float4 *>(qa.x + (size_t)m * qa.ldx)[i];
+            return qa.x2 ? add4(v, reinterpret_cast<const float4 *>(qa.x2 + (size_t)m * qa.ldx)[i]) : v;
+        };
+        auto square = [](double &acc, const float4 v) {
+            acc += (double)v.x * (double)v.x;
+            acc += (double)v.y * (double)v.y;
+            acc += (double)v.z * (double)v.z;
+            acc += (double)v.w * (double)v.w;
+        };
+        auto butterfly = [](double acc) {
+#pragma unroll
+            for (int off = WAVE / 2; off > 0; off >>= 1)
+                acc += __shfl_xor(acc, off, WAVE);
+            return acc;
+        };
+        auto inverse_rms = [&](int m) {
+            double sum_sq = 0.0;
+#pragma unroll
+            for (int w = 0; w < VT / WAVE; ++w)
+                sum_sq += s_part[m * 8 + w];
+            const float rms = __fsqrt_rn(__fadd_rn((float)(sum_sq / (double)H), qa.eps));
+            return __fdiv_rn(1.0f, rms);
+        };
+        auto emit = [&](int m, int i, const float4 v, const float4 g, float inv) {
+            float4 o;
+            o.x = __fmul_rn(__fmul_rn(v.x, inv), g.x);
+            o.y = __fmul_rn(__fmul_rn(v.y, inv), g.y);
+            o.z = __fmul_rn(__fmul_rn(v.z, inv), g.z);
+            o.w = __fmul_rn(__fmul_rn(v.w, inv), g.w);
+            quad_store_q8_lane<Q>(q8_1_quantize_lane(o), i, aq + m * aq_stride);
+        };
+
+        if ((int)blockDim.x >= VT && nvec <= KEEP * VT) // uniform
+        {
+            const int vt = threadIdx.x;
+            float4 keep[M][KEEP], gk[KEEP];
+            if (vt < VT) // whole wavefronts
+            {
+                // every load first (one branch around all loads of the delta), then the additions
+                float4 dk[M][KEEP];
+#pragma unroll
+                for (int k = 0; k < KEEP; ++k)
+                {
+                    const int i = min(vt + k * VT, nvec - 1);
+                    gk[k] = g4[i];
+#pragma unroll
+                    for (int m = 0; m < M; ++m)
+                        keep[m][k] = reinterpret_cast<const float4 *>(qa.x + (size_t)m * qa.ldx)[i];
+                }
+                if (qa.x2) // uniform
+                {
+#pragma unroll
+                    for (int k = 0; k < KEEP; ++k)
+#pragma unroll
+                        for (int m = 0; m < M; ++m)
+                            dk[m][k] = reinterpret_cast<const float4 *>(qa.x2 + (size_t)m * qa.ldx)[min(vt + k * VT, nvec - 1)];
+#pragma unroll
+                    for (int k = 0; k < KEEP; ++k)
+#pragma unroll
+                        for (int m = 0; m < M; ++m)
+                            keep[m][k] = add4(keep[m][k], dk[m][k]);
+                }
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                {
+                    double acc = 0.0;
+#pragma unroll
+                    for (int k = 0; k < KEEP; ++k)
+                        if (vt + k * VT < nvec)
+                        {
+                            if (writer)
+                                reinterpret_cast<float4 *>(qa.x_out + (size_t)m * qa.ldx)[vt + k * VT] = keep[m][k];
+                            square(acc, keep[m][k]);
+                        }
+                    acc = butterfly(acc);
+                    if ((vt & (WAVE - 1)) == 0)
+                        s_part[m * 8 + (vt >> 6)] = acc;
+                }
+            }
+            __syncthreads();
+            if (vt < VT)
+            {
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                {
+                    const float inv = inverse_rms(m);
+#pragma unroll
+                    for (int k = 0; k < KEEP; ++k)
+                        if (vt + k * VT < nvec) // whole 8-thread groups stay together (nvec is a multiple of 64)
+                            emit(m, vt + k * VT, keep[m][k], gk[k], inv);
+                }
+            }
+            return;
+        }
+
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+            for (int vt = threadIdx.x; vt < VT; vt += (int)blockDim.x) // uniform per wavefront
+            {
+                double acc = 0.0;
+                for (int i = vt; i < nvec; i += VT)
+                {
+                    const float4 v = row_value(m, i);
+                    if (writer)
+                        reinterpret_cast<float4 *>(qa.x_out + (size_t)m * qa.ldx)[i] = v;
+                    square(acc, v);
+                }
+                acc = butterfly(acc);
+                if ((vt & (WAVE - 1)) == 0)
+                    s_part[m * 8 + (vt >> 6)] = acc;
+            }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+        {
+            const float inv = inverse_rms(m);
+            for (int i = threadIdx.x; i < nvec; i += (int)blockDim.x) // whole 8-thread groups stay together
+                emit(m, i, row_value(m, i), g4[i], inv);
         }
     }
 
@@ -769,7 +940,10 @@ namespace llamql
         {
             load_chunk(bufA); // two chunks in flight while the activations are quantised and staged
             load_chunk(bufB);
-            quad_stage_f32<Q, M, SRC>(qa.x, qa.x2, qa.ldx, nsb, aq, ads, aq_stride, ads_stride);
+            if constexpr (SRC == QUAD_SRC_RMSNORM)
+                quad_stage_rmsnorm<Q, M>(qa, nsb, aq, aq_stride, quad_lds);
+            else
+                quad_stage_f32<Q, M, SRC>(qa.x, qa.x2, qa.ldx, nsb, aq, ads, aq_stride, ads_stride);
         }
         Q::stage(); // the format's decode tables, if it has any
         __syncthreads();
@@ -793,6 +967,21 @@ namespace llamql
         float *ring = reinterpret_cast<float *>(quad_lds + (size_t)M * aq_stride) +
                       (size_t)(threadIdx.x >> 6) * (QUAD_RING_ROWS * QUAD_RING_STRIDE * M);
         int slot = 0; // parked rows: row - slot .. row - 1
+        // accumulate: what y holds for this lane's row of the (only) flush, requested now and long
+        // there by the time the run ends
+        float held[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+            held[m] = 0.0f;
+        if constexpr (DEFER)
+        {
+            if (qa.accumulate && (lane >> 2) < nrows)
+            {
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                    held[m] = y[(size_t)m * ldy + (size_t)(j + (long)(lane >> 2) * TW)];
+            }
+        }
         auto flush_ring = [&]() {
             wave_lds_sync(); // the wavefront's writes are in the ring (its LDS instructions run in order)
             const int r = lane >> 2, q = lane & 3;
@@ -806,7 +995,7 @@ namespace llamql
                 sum += dpp_f32<DPP_QUAD_XOR1>(sum);
                 sum += dpp_f32<DPP_QUAD_XOR2>(sum);
                 if (q == 0 && r < slot)
-                    y[(size_t)m * ldy + (size_t)(j + (long)(row - slot + r) * TW)] = sum;
+                    y[(size_t)m * ldy + (size_t)(j + (long)(row - slot + r) * TW)] = qa.accumulate ? held[m] + sum : sum;
             }
             wave_lds_sync(); // reads done before the ring is written again
             slot = 0;
@@ -972,6 +1161,12 @@ namespace llamql
         {
             if (a.ring)
             {
+                if constexpr (M <= QUAD_NORM_MAX_M)
+                    if (src == QUAD_SRC_RMSNORM)
+                    {
+                        gemv_quad_launch_mus<Q, M, U, QUAD_SRC_RMSNORM, QUAD_MODE_RING>(grid, block, lds, st, a);
+                        return;
+                    }
                 switch (src)
                 {
                 case QUAD_SRC_F32: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_F32, QUAD_MODE_RING>(grid, block, lds, st, a); break;
@@ -981,6 +1176,12 @@ namespace llamql
                 return;
             }
         }
+        if constexpr (M <= QUAD_NORM_MAX_M)
+            if (src == QUAD_SRC_RMSNORM)
+            {
+                gemv_quad_launch_mus<Q, M, U, QUAD_SRC_RMSNORM>(grid, block, lds, st, a);
+                return;
+            }
         switch (src)
         {
         case QUAD_SRC_F32: gemv_quad_launch_mus<Q, M, U, QUAD_SRC_F32>(grid, block, lds, st, a); break;
@@ -1048,6 +1249,12 @@ namespace llamql
     template <class QA, class QB, int M>
     inline void gemv_quad_dual_launch_m(int src, dim3 grid, dim3 block, size_t lds, hipStream_t st, const QuadArgs &a)
     {
+        if constexpr (M <= QUAD_NORM_MAX_M)
+            if (src == QUAD_SRC_RMSNORM)
+            {
+                gemv_quad_dual_launch_ms<QA, QB, M, QUAD_SRC_RMSNORM>(grid, block, lds, st, a);
+                return;
+            }
         if (src == QUAD_SRC_F32)
             gemv_quad_dual_launch_ms<QA, QB, M, QUAD_SRC_F32>(grid, block, lds, st, a);
         else

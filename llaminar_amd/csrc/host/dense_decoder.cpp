@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <utility>
 #include <vector>
 
 #include "llaminar_amd/decode_api.h"
@@ -51,7 +52,7 @@ namespace
 
         int32_t *ids = nullptr, *pos = nullptr;
         int host_max_pos = 0; // the furthest sequence's position as the host counts it
-        float *x = nullptr, *delta = nullptr, *qkv = nullptr, *attn = nullptr, *gate = nullptr, *up = nullptr;
+        float *x = nullptr, *x_alt = nullptr, *delta = nullptr, *qkv = nullptr, *attn = nullptr, *gate = nullptr, *up = nullptr;
         float *logits = nullptr, *inv_freq = nullptr, *rope_table = nullptr, *att_scratch = nullptr;
         void *q8_h = nullptr, *q8_attn = nullptr, *q8_act = nullptr, *argmax_scratch = nullptr;
         std::vector<void *> kcache, vcache;
@@ -131,7 +132,8 @@ extern "C" void *llam_decoder_create(const llam_decoder_config *c)
     const int B = c->batch, H = c->hidden, F = c->ffn;
     const int wide = H > d->qdim() ? H : d->qdim();
     bool ok = d->alloc(d->ids, (size_t)B * 4) && d->alloc(d->pos, (size_t)B * 4) &&
-              d->alloc(d->x, (size_t)B * H * 4) && d->alloc(d->delta, (size_t)B * H * 4) &&
+              d->alloc(d->x, (size_t)B * H * 4) && d->alloc(d->x_alt, (size_t)B * H * 4) &&
+              d->alloc(d->delta, (size_t)B * H * 4) &&
               d->alloc(d->qkv, (size_t)B * (d->qdim() + 2 * d->kvdim()) * 4) &&
               d->alloc(d->attn, (size_t)B * d->qdim() * 4) && d->alloc(d->gate, (size_t)B * F * 4) &&
               d->alloc(d->up, (size_t)B * F * 4) && d->alloc(d->logits, (size_t)B * c->vocab * 4) &&
@@ -285,18 +287,49 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
     // the rotation of this step's positions, shared by every layer
     if (!forward(fn, llam_dec_rope_table(d->pos, d->inv_freq, d->rope_table, B, c.head_dim, dev, stream)))
         return false;
+    // The residual stream: the rows in `res`, and `pending`, a delta still to be added to them (or null).
+    // A projection that can add its result to its output (llam_ql_gemv_accumulate) updates `res`
+    // itself and leaves nothing pending; otherwise its result waits in d->delta for the next norm.
+    // Where the projections' kernels can run the norm themselves (llam_ql_gemv_fused_rmsnorm: no
+    // launch for the norm) a pending delta is added into the other of the two buffers, elsewhere the
+    // norm updates `res` in place.
+    float *res = d->x, *spare = d->x_alt;
+    const float *pending = nullptr;
+    auto norm_and_project = [&](const llam_ql_proj *projs, int num, const float *gamma) {
+        if (llam_ql_gemv_fused_rmsnorm_supported(projs, num, B, H))
+        {
+            if (!forward(fn, llam_ql_gemv_fused_rmsnorm(projs, num, res, pending, gamma, c.rms_eps, spare, B, H, dev,
+                                                        stream)))
+                return false;
+            if (pending)
+                std::swap(res, spare);
+        }
+        else
+        {
+            if (!forward(fn, llam_dec_rmsnorm_q8_1(res, pending, gamma, c.rms_eps, nullptr, d->q8_h, B, H, dev, stream)))
+                return false;
+            if (!forward(fn, llam_ql_gemv_fused(projs, num, d->q8_h, B, H, dev, stream)))
+                return false;
+        }
+        pending = nullptr;
+        return true;
+    };
+    // res += W q8 where the launch can, else delta = W q8 and pending
+    auto project_into_residual = [&](uint8_t fmt, const void *w, const void *q8, int K) {
+        if (llam_ql_gemv_accumulate_supported(fmt, B, H, K, dev))
+            return forward(fn, llam_ql_gemv_accumulate(fmt, w, q8, res, B, H, K, H, dev, stream));
+        pending = d->delta;
+        return forward(fn, llam_ql_gemv(fmt, w, q8, d->delta, B, H, K, H, dev, stream));
+    };
     for (int l = 0; l < c.n_layers; ++l)
     {
         const llam_decoder_layer &w = d->layers[l];
         // attention half
-        if (!forward(fn, llam_dec_rmsnorm_q8_1(d->x, l ? d->delta : nullptr, w.attn_norm, c.rms_eps, nullptr, d->q8_h,
-                                               B, H, dev, stream)))
-            return false;
         llam_ql_proj qkv[3];
         qkv[0] = llam_ql_proj{w.wq, d->qkv, QD, ldqkv, w.fmt_q};
         qkv[1] = llam_ql_proj{w.wk, d->qkv + QD, KV, ldqkv, w.fmt_k};
         qkv[2] = llam_ql_proj{w.wv, d->qkv + QD + KV, KV, ldqkv, w.fmt_v};
-        if (!forward(fn, llam_ql_gemv_fused(qkv, 3, d->q8_h, B, H, dev, stream)))
+        if (!norm_and_project(qkv, 3, w.attn_norm))
             return false;
         // rotary embedding, the cache append and the attention in one operator; its output leaves the
         // merge kernel as Q8_1 blocks: the output projection's quantiser costs no launch of its own
@@ -304,22 +337,32 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
                                                  0, d->q8_attn, d->att_scratch, B, c.n_heads, c.n_kv, c.head_dim,
                                                  c.ctx_cap, dev, stream)))
             return false;
-        if (!forward(fn, llam_ql_gemv(w.fmt_o, w.wo, d->q8_attn, d->delta, B, H, QD, H, dev, stream)))
+        if (!project_into_residual(w.fmt_o, w.wo, d->q8_attn, QD))
             return false;
         // feed-forward half
-        if (!forward(fn, llam_dec_rmsnorm_q8_1(d->x, d->delta, w.ffn_norm, c.rms_eps, nullptr, d->q8_h, B, H, dev,
-                                               stream)))
-            return false;
         llam_ql_proj gu[2];
         gu[0] = llam_ql_proj{w.wgate, d->gate, F, F, w.fmt_gate};
         gu[1] = llam_ql_proj{w.wup, d->up, F, F, w.fmt_up};
-        if (!forward(fn, llam_ql_gemv_fused(gu, 2, d->q8_h, B, H, dev, stream)))
+        if (!norm_and_project(gu, 2, w.ffn_norm))
             return false;
-        if (!forward(fn, llam_ql_gemv_swiglu_f32(w.fmt_down, w.wdown, d->gate, d->up, F, d->delta, B, H, F, H,
-                                                 d->q8_act, dev, stream)))
-            return false;
+        if (llam_ql_gemv_accumulate_supported(w.fmt_down, B, H, F, dev))
+        {
+            // SwiGLU and its quantiser as a launch of their own (rows this long are not quantised
+            // again by every workgroup of the projection), then res += W_down act
+            if (!forward(fn, llam_ql_swiglu_quantize(d->gate, d->up, nullptr, d->q8_act, B, F, dev, stream)))
+                return false;
+            if (!project_into_residual(w.fmt_down, w.wdown, d->q8_act, F))
+                return false;
+        }
+        else
+        {
+            if (!forward(fn, llam_ql_gemv_swiglu_f32(w.fmt_down, w.wdown, d->gate, d->up, F, d->delta, B, H, F, H,
+                                                     d->q8_act, dev, stream)))
+                return false;
+            pending = d->delta;
+        }
     }
-    if (!forward(fn, llam_dec_rmsnorm_q8_1(d->x, d->delta, d->globals.final_norm, c.rms_eps, nullptr, d->q8_h, B, H,
+    if (!forward(fn, llam_dec_rmsnorm_q8_1(res, pending, d->globals.final_norm, c.rms_eps, nullptr, d->q8_h, B, H,
                                            dev, stream)))
         return false;
     if (!forward(fn, llam_ql_gemv(d->globals.fmt_lm_head, d->globals.lm_head, d->q8_h, d->logits, B, c.vocab, H,

@@ -12,6 +12,9 @@ namespace llamql
     bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
                           int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
     void gemv_describe(uint8_t fmt, int M, int N, int K, int device_id, llam_ql_gemv_plan *out);
+    bool gemv_norm_fusable(uint8_t fmt, int M, int N, int K);
+    bool gemv_accumulate(const char *fn, uint8_t fmt, const void *d_w, const void *d_q8, float *d_y, int M, int N,
+                         int K, int ldy, int device_id, hipStream_t st, bool query);
     int gemv_group_launch(const char *fn, const llam_ql_proj *projs, int num, const ActSource &src, int M, int K,
                           int device_id, hipStream_t st);
 
@@ -307,6 +310,79 @@ extern "C" bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const floa
         return false;
     return run_projections(fn, &p, 1, ActSource{ACT_SRC_SWIGLU, nullptr, d_gate, d_up, ld_gu}, M, K, d_q8_scratch,
                            device_id, stream);
+}
+
+extern "C" bool llam_ql_gemv_accumulate_supported(uint8_t fmt, int M, int N, int K, int device_id)
+{
+    using namespace llamql;
+    if ((fmt != LLAM_FMT_Q4_K && fmt != LLAM_FMT_Q6_K && fmt != LLAM_FMT_IQ3_S) || M < 1 || M > LLAM_QL_MAX_GEMV_M ||
+        N < 1 || K < 256 || (K % 256) != 0)
+        return false;
+    return gemv_accumulate("llam_ql_gemv_accumulate_supported", fmt, nullptr, nullptr, nullptr, M, N, K, N, device_id,
+                           nullptr, true);
+}
+
+extern "C" bool llam_ql_gemv_accumulate(uint8_t fmt, const void *d_w, const void *d_q8, float *d_y, int M, int N,
+                                        int K, int ldy, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_accumulate";
+    if (!check_common(fn, fmt, d_w, d_q8, M, N, K))
+        return false;
+    if (!d_y)
+        return fail(fn, "null output");
+    if (ldy < N)
+        return fail(fn, "ldy=%d smaller than N=%d", ldy, N);
+    if (!set_device(fn, device_id))
+        return false;
+    return gemv_accumulate(fn, fmt, d_w, d_q8, d_y, M, N, K, ldy, device_id, as_stream(stream), false);
+}
+
+extern "C" bool llam_ql_gemv_fused_rmsnorm_supported(const llam_ql_proj *projs, int num, int M, int K)
+{
+    using namespace llamql;
+    if (!projs || num < 1 || num > LLAM_QL_MAX_FUSED || K < 256 || (K % 256) != 0)
+        return false;
+    for (int i = 0; i < num; ++i)
+        if (projs[i].N < 1 || !gemv_norm_fusable(projs[i].fmt, M, projs[i].N, K))
+            return false;
+    return true;
+}
+
+extern "C" bool llam_ql_gemv_fused_rmsnorm(const llam_ql_proj *projs, int num, const float *d_x, const float *d_delta,
+                                           const float *d_gamma, float eps, float *d_x_out, int M, int K,
+                                           int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_fused_rmsnorm";
+    if (!check_projections(fn, projs, num, M, K))
+        return false;
+    if (num == 0)
+        return fail(fn, "no projection: the norm runs inside their kernels");
+    if (!check_f32(fn, d_x, K, K, nullptr))
+        return false;
+    if (!d_gamma || !aligned16(d_gamma))
+        return fail(fn, "gamma must be a 16-byte aligned device pointer");
+    if (d_delta && (!aligned16(d_delta) || !d_x_out || !aligned16(d_x_out) || d_x_out == d_x))
+        return fail(fn, "with a delta, x + delta goes to d_x_out: 16-byte aligned and not d_x itself");
+    if (!llam_ql_gemv_fused_rmsnorm_supported(projs, num, M, K))
+        return fail(fn, "M=%d K=%d: not every projection's kernel can fuse the norm (ask "
+                        "llam_ql_gemv_fused_rmsnorm_supported; otherwise norm and projections run as two calls)",
+                    M, K);
+    if (!set_device(fn, device_id))
+        return false;
+    ActSource src{ACT_SRC_RMSNORM, nullptr, d_x, d_delta, K};
+    src.gamma = d_gamma;
+    src.eps = eps;
+    src.x_out = d_delta ? d_x_out : nullptr;
+    for (int i = 0; i < num;)
+    {
+        const int took = gemv_group_launch(fn, projs + i, num - i, src, M, K, device_id, as_stream(stream));
+        if (took <= 0)
+            return took < 0 ? false : fail(fn, "projection %d found no fused launch", i);
+        i += took;
+    }
+    return true;
 }
 
 extern "C" bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,

@@ -72,14 +72,19 @@ namespace llamql
 
     // The activations of a decode GEMV: Q8_1 blocks, or fp32 rows that the kernel quantises
     // itself (plain, or silu(x) * x2 first).
-    constexpr int ACT_SRC_Q8 = 0, ACT_SRC_F32 = 1, ACT_SRC_SWIGLU = 2;
+    // ACT_SRC_RMSNORM: the residual rows x (+ delta), RMS-normalised and scaled by gamma.
+    constexpr int ACT_SRC_Q8 = 0, ACT_SRC_F32 = 1, ACT_SRC_SWIGLU = 2, ACT_SRC_RMSNORM = 3;
     struct ActSource
     {
         int kind;        // ACT_SRC_*
         const void *q8;  // ACT_SRC_Q8: [M][K/32] blocks
-        const float *x;  // ACT_SRC_F32: rows of ldx floats; the gate rows for ACT_SRC_SWIGLU
-        const float *x2; // ACT_SRC_SWIGLU: the up rows
+        const float *x;  // ACT_SRC_F32: rows of ldx floats; the gate rows for ACT_SRC_SWIGLU; the
+                         // residual rows for ACT_SRC_RMSNORM
+        const float *x2; // ACT_SRC_SWIGLU: the up rows; ACT_SRC_RMSNORM: the delta rows to add first, or null
         int ldx;
+        const float *gamma = nullptr; // ACT_SRC_RMSNORM: K weights of the norm
+        float eps = 0.0f;
+        float *x_out = nullptr;       // ACT_SRC_RMSNORM with a delta: where x + delta goes (not x itself)
     };
     inline ActSource act_source_q8(const void *d_q8) { return ActSource{ACT_SRC_Q8, d_q8, nullptr, nullptr, 0}; }
 } // namespace llamql

@@ -605,3 +605,102 @@ def test_lm_head_shape_q6k_152064x5120(capi, dev, oracle, M):
         y1 = capi.gemv(fmt, wd, upload_q8(dev, q8[5:6]), 1, N, K)
         sync()
         assert torch.equal(y[5], y1[0])
+
+
+# (formats, Ns) of the projections, K, M: the decoder's two uses (Q and K in Q4_K with V in Q6_K; gate and up),
+# a format with decode tables, matrices whose workgroups are smaller than the norm's 512 threads, rows too long
+# for the registers
+_NORM_CASES = [
+    ((FMT_Q4_K, FMT_Q4_K, FMT_Q6_K), (8192, 1024, 1024), 5120, 1),
+    ((FMT_Q4_K, FMT_Q4_K), (25600, 25600), 5120, 1),
+    ((FMT_Q4_K, FMT_Q4_K, FMT_Q6_K), (2048, 512, 512), 4096, 1),
+    ((FMT_Q4_K, FMT_Q4_K), (6400, 6400), 8192, 1),
+    ((FMT_IQ3_S,), (4096,), 5120, 1),
+    ((FMT_Q6_K,), (384,), 8192, 1),
+    ((FMT_Q4_K,), (3000,), 12800, 1),
+]
+
+
+@pytest.mark.parametrize("fmts,Ns,K,M", _NORM_CASES)
+def test_norm_inside_the_projections_equals_norm_then_projections(capi, dev, fmts, Ns, K, M):
+    """llam_ql_gemv_fused_rmsnorm against llam_dec_rmsnorm_q8_1 followed by llam_ql_gemv_fused: the same bits in
+    every output and in the updated residual, with and without a delta, whatever the workgroup size of the launch."""
+    import torch
+
+    rng = np.random.default_rng(K + M + sum(Ns))
+    x = torch.from_numpy((rng.standard_normal((M, K)) * rng.uniform(0.05, 20, (M, 1))).astype(np.float32)).to(dev)
+    d = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(dev)
+    g = torch.from_numpy(rng.uniform(0.2, 2.0, K).astype(np.float32)).to(dev)
+    ws = [capi.prepare_weights(f, synth.weights_torch(f, N, K, 300 + i, dev), N, K) for i, (f, N) in enumerate(zip(fmts, Ns))]
+    for delta in (None, d):
+        sep = [torch.full((M, N), 3.0, device=dev) for N in Ns]
+        fus = [torch.full((M, N), 5.0, device=dev) for N in Ns]
+        projs_sep = [(f, w, o) for f, w, o in zip(fmts, ws, sep)]
+        projs_fus = [(f, w, o) for f, w, o in zip(fmts, ws, fus)]
+        assert capi.gemv_fused_rmsnorm_supported(projs_fus, M, K)
+        x_sep = x.clone()
+        _, q8 = capi.rmsnorm_q8_1(x_sep, g, 1e-6, delta=delta, want_y=False)
+        capi.gemv_fused(projs_sep, q8, M, K)
+        x_in = x.clone()
+        x_out = torch.full((M, K), 9.0, device=dev)
+        capi.gemv_fused_rmsnorm(projs_fus, x_in, delta, g, 1e-6, x_out if delta is not None else None, M, K)
+        sync()
+        for a, b in zip(sep, fus):
+            assert torch.equal(a, b)
+        assert torch.equal(x_in, x)                      # the input rows are read only
+        if delta is not None:
+            assert torch.equal(x_out, x_sep)             # x + delta, as the stand-alone norm leaves it
+        else:
+            assert (x_out == 9.0).all()                  # no delta: nothing to store
+
+
+def test_norm_inside_the_projections_is_refused_where_no_kernel_fuses_it(capi, dev):
+    import torch
+
+    K = 5120
+    w = capi.prepare_weights(FMT_Q4_K, synth.weights_torch(FMT_Q4_K, 8192, K, 1, dev), 8192, K)
+    x = torch.randn(8, K, device=dev)
+    g = torch.ones(K, device=dev)
+    out = torch.empty(8, 8192, device=dev)
+    for M in (2, 8):                                                               # one row only
+        assert not capi.gemv_fused_rmsnorm_supported([(FMT_Q4_K, w, out[:M])], M, K)
+        with pytest.raises(capi.QLError):
+            capi.gemv_fused_rmsnorm([(FMT_Q4_K, w, out[:M])], x[:M], None, g, 1e-6, None, M, K)
+    small = torch.empty(1, 64, device=dev)
+    w2 = capi.prepare_weights(FMT_Q4_K, synth.weights_torch(FMT_Q4_K, 64, 1024, 2, dev), 64, 1024)
+    assert not capi.gemv_fused_rmsnorm_supported([(FMT_Q4_K, w2, small)], 1, 1024)  # rows too short for the quad-lane kernel
+    with pytest.raises(capi.QLError):                                              # x + delta must not land on x
+        capi.gemv_fused_rmsnorm([(FMT_Q4_K, w, out[:1])], x[:1], x[1:2], g, 1e-6, x[:1], 1, K)
+
+
+@pytest.mark.parametrize("fmt,N,K,M", [(FMT_Q4_K, 5120, 8192, 1), (FMT_Q6_K, 5120, 25600, 1), (FMT_IQ3_S, 4096, 5120, 1),
+                                       (FMT_Q4_K, 5120, 8192, 2), (FMT_Q6_K, 1000, 4096, 1)])
+def test_accumulating_launch_equals_gemv_then_add(capi, dev, fmt, N, K, M):
+    """llam_ql_gemv_accumulate: y += W a inside the launch has the bits of llam_ql_gemv followed by one fp32 add."""
+    import torch
+
+    assert capi.gemv_accumulate_supported(fmt, M, N, K)
+    w = capi.prepare_weights(fmt, synth.weights_torch(fmt, N, K, 77, dev), N, K)
+    x = torch.randn(M, K, device=dev, generator=torch.Generator(device=dev).manual_seed(N + K))
+    q8 = capi.quantize_q8_1(x)
+    y0 = torch.randn(M, N + 8, device=dev)                 # a residual with a row stride of its own
+    delta = capi.gemv(fmt, w, q8, M, N, K)
+    got = y0.clone()
+    capi.gemv_accumulate(fmt, w, q8, M, N, K, got[:, :N])
+    sync()
+    assert torch.equal(got[:, :N], y0[:, :N] + delta)
+    assert torch.equal(got[:, N:], y0[:, N:])
+
+
+def test_accumulating_launch_is_refused_where_the_kernel_cannot(capi, dev):
+    import torch
+
+    # the lm_head shape: a wavefront walks more rows than one flush of the ring holds; batch 8: the matrix unit;
+    # short rows: not the quad-lane kernel
+    for fmt, M, N, K in ((FMT_Q6_K, 1, 152064, 5120), (FMT_Q4_K, 8, 25600, 5120), (FMT_Q4_K, 1, 512, 1024)):
+        assert not capi.gemv_accumulate_supported(fmt, M, N, K)
+    N, K = 512, 1024
+    w = capi.prepare_weights(FMT_Q4_K, synth.weights_torch(FMT_Q4_K, N, K, 5, dev), N, K)
+    q8 = capi.quantize_q8_1(torch.randn(1, K, device=dev))
+    with pytest.raises(capi.QLError):
+        capi.gemv_accumulate(FMT_Q4_K, w, q8, 1, N, K, torch.zeros(1, N, device=dev))
