@@ -135,8 +135,8 @@ def bench_moe(args, torch, capi, synth, dev):
 
     # Batches sort the (token, slot) pairs by expert on the device and read every distinct
     # expert's matrices once (6 launches); a single token has nothing to group (4 launches).
-    # (measured: per-slot launches 100 us at 16 tokens against 104 grouped; 172 against 153 at 32; 316 against 217 at 64)
-    path = args.moe_path if args.moe_path != "auto" else ("grouped" if T >= 32 else "slots")
+    # (measured: per-slot launches 67 us at 16 tokens, 107 against 135 grouped at 32, 184 against 201 at 64, 334 against 296 at 128)
+    path = args.moe_path if args.moe_path != "auto" else ("grouped" if T * (TOPK + 1) >= 768 else "slots")
     S = TOPK + 1
     for s_ in sets:
         s_["group"] = torch.empty(int(capi.load().llam_ql_moe_group_bytes(T, S)), dtype=torch.uint8, device=dev)

@@ -214,6 +214,245 @@ namespace llamql
         gemv_body<F, 1, 1, false>(a, (long)blockIdx.x, lds);
     }
 
+    // ---- the same with the quad-lane decoders (gemv_quad.h) ---------------------------------
+    // Expert rows are short (2..16 super-blocks): a wavefront step of 16 super-blocks covers 16 / nsb
+    // WHOLE rows, so a lane's product is final after one step and a segmented sum over the
+    // 4 nsb lanes of a row ends it -- no run across rows, no ring.  A lane decodes two 32-element
+    // blocks of a super-block with the format's quad-lane decoder (per super-block work shared by
+    // four lanes instead of repeated by eight), loads are issued as in the quad-lane GEMV (two
+    // steps in flight).  nsb: a power of two, 2..16.
+    constexpr int MOE_QUAD_WAVES = 8;
+
+    // sum over the 4 << nsb_log2 lanes of a row (nsb_log2 = 1..4); every lane gets the total
+    __device__ __forceinline__ float moe_quad_row_sum(float v, int nsb_log2) { return segment_sum(v, nsb_log2 - 1); }
+
+    // One wavefront step: decode, dot with the activation row at `aq` (quad-lane layout), this lane's share.
+    template <class Q>
+    __device__ __forceinline__ float moe_quad_step(const typename Q::Raw &r, const typename Q::Lane &lc,
+                                                   const uint8_t *aq_lane)
+    {
+        v4i w[4];
+        typename Q::Scale S;
+        Q::decode(r, lc, w, S);
+        const v4i a0 = *reinterpret_cast<const v4i *>(aq_lane);
+        const v4i a1 = *reinterpret_cast<const v4i *>(aq_lane + 64);
+        const v4i a2 = *reinterpret_cast<const v4i *>(aq_lane + 128);
+        const v4i a3 = *reinterpret_cast<const v4i *>(aq_lane + 192);
+        const float4 sd = *reinterpret_cast<const float4 *>(aq_lane + 256);
+        const int i0 = dot16(a1, w[1], dot16z(a0, w[0]));
+        const int i1 = dot16(a3, w[3], dot16z(a2, w[2]));
+        return Q::apply(S, i0, i1, sd, 0.0f);
+    }
+
+    // grid: (workgroups per matrix, n_tokens*top_k, 2 = gate|up), MOE_QUAD_WAVES wavefronts;
+    // m.rows_per_wave: STEPS per wavefront, m.gshift: log2(nsb)
+    template <class Q>
+    __global__ void __launch_bounds__(MOE_QUAD_WAVES *WAVE) moe_gate_up_quad_kernel(const MoEArgs m)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t moe_quad_lds[];
+        const int slot = blockIdx.y;
+        const int t = slot / m.top_k;
+        const int e = m.ids[slot];
+        if (e < 0 || e >= m.n_experts)
+            return; // uniform for the workgroup; outputs of a bad id stay untouched
+        GemvArgs a;
+        a.w = blockIdx.z == 0 ? m.experts[e].d_gate : m.experts[e].d_up;
+        if (!a.w)
+            return; // an expert whose matrices live elsewhere: skipped like a bad id (uniform)
+        const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
+        a.N = m.inter;
+        a.SB = nsb;
+        float *y = (blockIdx.z == 0 ? m.out0 : m.out1) + (size_t)slot * m.inter;
+
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int l = lane & 3, grp = lane >> 2;
+        const typename Q::Lane lc = Q::lane_consts(l);
+        const int total = m.inter * nsb;                       // super-blocks of the matrix
+        const int step0 = ((int)blockIdx.x * MOE_QUAD_WAVES + wave) * m.rows_per_wave;
+        const int nsteps = min(m.rows_per_wave, max(0, (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB - step0));
+        // loads are never predicated: past the end a lane re-reads its first super-block
+        const size_t t0 = (size_t)min(step0 * QUAD_STEP_SB + grp, total - 1);
+        typename Q::Cursor wc = Q::cursor(a, t0, t0, lc);
+        const typename Q::Stride stride = Q::stride(0);
+        int ld_step = 0;
+        auto issue = [&](typename Q::Raw &buf) {
+            Q::load(buf, wc, lc, ld_step < nsteps && (step0 + ld_step) * QUAD_STEP_SB + grp < total);
+            Q::next(wc, false, stride);
+            ++ld_step;
+        };
+        typename Q::Raw bufA, bufB;
+        issue(bufA);
+        issue(bufB);
+        quad_stage_q8<Q, 1>(m.q8 + (size_t)t * (m.hidden / 32) * 9, nsb, moe_quad_lds, moe_quad_lds, 0, 0);
+        Q::stage();
+        __syncthreads();
+        Q::keep(bufA);
+        Q::keep(bufB);
+
+        const uint8_t *aq_lane = moe_quad_lds + (grp & (nsb - 1)) * QUAD_SB_LDS + (l << 4);
+        const int seg_mask = (4 << nsb_log2) - 1;
+        int step = 0;
+        auto compute = [&](const typename Q::Raw &buf) {
+            const int sb = (step0 + step) * QUAD_STEP_SB + grp;
+            float v = moe_quad_step<Q>(buf, lc, aq_lane);
+            v = sb < total ? v : 0.0f;
+            const float tot = moe_quad_row_sum(v, nsb_log2);
+            if (sb < total && (lane & seg_mask) == 0)
+                y[sb >> nsb_log2] = tot;
+            ++step;
+        };
+        for (int c0 = 0; c0 < nsteps; c0 += 2)
+        {
+            Q::template wait<Q::LOADS>(bufA);
+            if (step < nsteps) // uniform
+                compute(bufA);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufA);
+            Q::template wait<Q::LOADS>(bufB);
+            if (step < nsteps)
+                compute(bufB);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufB);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end
+        Q::keep(bufA);
+        Q::keep(bufB);
+    }
+
+    // Down projection of one token's slots with the quad-lane decoder: a wavefront walks its steps
+    // (16 / nsb whole rows each) slot after slot, so a row's slots are added in ascending order by
+    // the one lane that writes it (moe_down_kernel's arithmetic).  The live slots (good id, matrix
+    // present) are listed in LDS; two (step, slot) items are in flight per wavefront.
+    // grid: (workgroups per matrix, n_tokens); m.rows_per_wave: steps per wavefront, m.gshift: log2(nsb).
+    struct MoEQuadSlot
+    {
+        const void *w;
+        float weight;
+        int slot; // within the token
+    };
+    constexpr int MOE_QUAD_MAX_SLOTS = 16;
+
+    template <class Q>
+    __global__ void __launch_bounds__(MOE_QUAD_WAVES *WAVE) moe_down_quad_kernel(const MoEArgs m)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t moe_quad_lds[];
+        __shared__ MoEQuadSlot live[MOE_QUAD_MAX_SLOTS];
+        __shared__ int n_live_s;
+        const int t = blockIdx.y;
+        const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int l = lane & 3, grp = lane >> 2;
+        const typename Q::Lane lc = Q::lane_consts(l);
+        const int total = m.hidden * nsb; // super-blocks of one down matrix
+        const int step0 = ((int)blockIdx.x * MOE_QUAD_WAVES + wave) * m.rows_per_wave;
+        const int nsteps = min(m.rows_per_wave, max(0, (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB - step0));
+
+        if (threadIdx.x == 0)
+        {
+            int n = 0;
+            for (int s = 0; s < m.top_k; ++s)
+            {
+                const int e = m.ids[t * m.top_k + s];
+                const void *w = (e >= 0 && e < m.n_experts) ? m.experts[e].d_down : nullptr;
+                if (w) // a bad id, or an expert whose matrices live elsewhere, is skipped
+                {
+                    live[n].w = w;
+                    live[n].weight = m.weights[t * m.top_k + s];
+                    live[n].slot = s;
+                    ++n;
+                }
+            }
+            n_live_s = n;
+        }
+        __syncthreads();
+        const int n_live = n_live_s;
+        if (n_live == 0) // uniform
+        {
+            if (m.accumulate == 0) // no live slot: the token's output is zero, not what the buffer held
+            {
+                const long r0 = (long)blockIdx.x * MOE_QUAD_WAVES * m.rows_per_wave * (QUAD_STEP_SB >> nsb_log2);
+                const long r1 = r0 + (long)MOE_QUAD_WAVES * m.rows_per_wave * (QUAD_STEP_SB >> nsb_log2);
+                for (long r = r0 + threadIdx.x; r < r1 && r < m.hidden; r += blockDim.x)
+                    m.out0[(size_t)t * m.hidden + r] = 0.0f;
+            }
+            return;
+        }
+
+        GemvArgs a; // weight addressing only
+        a.N = m.hidden;
+        a.SB = nsb;
+        int ld_step = 0, ld_k = 0;
+        // loads are never predicated: past the end a lane re-reads its first super-block of the slot
+        auto issue = [&](typename Q::Raw &buf) {
+            const uint64_t wp = (uint64_t)live[ld_k].w;
+            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)wp);
+            const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(wp >> 32));
+            a.w = reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
+            const int st = ld_step < nsteps ? ld_step : 0;
+            const size_t ti = (size_t)min((step0 + st) * QUAD_STEP_SB + grp, total - 1);
+            const typename Q::Cursor wc = Q::cursor(a, ti, ti, lc);
+            Q::load(buf, wc, lc, true);
+            if (++ld_k == n_live)
+            {
+                ld_k = 0;
+                ++ld_step;
+            }
+        };
+        typename Q::Raw bufA, bufB;
+        issue(bufA);
+        issue(bufB);
+        // the token's slots form one long activation row: slot s at super-blocks s * nsb ..
+        quad_stage_q8<Q, 1>(m.q8 + (size_t)t * m.top_k * (m.inter / 32) * 9, nsb * m.top_k, moe_quad_lds, moe_quad_lds,
+                            0, 0);
+        Q::stage();
+        __syncthreads();
+        Q::keep(bufA);
+        Q::keep(bufB);
+
+        const uint8_t *aq_lane = moe_quad_lds + (grp & (nsb - 1)) * QUAD_SB_LDS + (l << 4);
+        const int seg_mask = (4 << nsb_log2) - 1;
+        const int n_items = nsteps * n_live;
+        int item = 0, step = 0, k = 0;
+        float y = 0.0f;
+        auto compute = [&](const typename Q::Raw &buf) {
+            const int sb = (step0 + step) * QUAD_STEP_SB + grp;
+            const int slot = live[k].slot;
+            float v = moe_quad_step<Q>(buf, lc, aq_lane + (size_t)slot * nsb * QUAD_SB_LDS);
+            v = sb < total ? v : 0.0f;
+            const float val = live[k].weight * moe_quad_row_sum(v, nsb_log2);
+            y = k == 0 ? val : y + val; // the first live slot starts the sum
+            if (++k == n_live)
+            {
+                if (sb < total && (lane & seg_mask) == 0)
+                {
+                    float *dst = m.out0 + (size_t)t * m.hidden + (sb >> nsb_log2);
+                    *dst = m.accumulate ? (*dst + y) : y;
+                }
+                k = 0;
+                ++step;
+            }
+            ++item;
+        };
+        for (int c0 = 0; c0 < n_items; c0 += 2)
+        {
+            Q::template wait<Q::LOADS>(bufA);
+            if (item < n_items) // uniform
+                compute(bufA);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufA);
+            Q::template wait<Q::LOADS>(bufB);
+            if (item < n_items)
+                compute(bufB);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufB);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end
+        Q::keep(bufA);
+        Q::keep(bufB);
+    }
+
     // grid: (workgroups per matrix, n_tokens).  Slots are walked in ascending
     // order inside the workgroup, so each output element is accumulated by one
     // lane in a fixed order.
@@ -852,6 +1091,16 @@ namespace llamql
             grid_x = ((long)N + rows_per_wg - 1) / rows_per_wg;
         }
 
+        // rows the short-row quad-lane kernels take: 2, 4, 8 or 16 super-blocks
+        bool moe_quad_rows(int nsb) { return nsb >= 2 && nsb <= QUAD_STEP_SB && (nsb & (nsb - 1)) == 0; }
+        int moe_log2(int v)
+        {
+            int l = 0;
+            while ((1 << l) < v)
+                ++l;
+            return l;
+        }
+
         bool check_moe(const char *fn, uint8_t fmt, int n_tokens, int n_experts, int top_k, int hidden, int inter)
         {
             if (fmt != LLAM_FMT_Q4_K && fmt != LLAM_FMT_Q6_K && fmt != LLAM_FMT_IQ3_S)
@@ -1025,11 +1274,29 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     m.hidden = hidden;
     m.inter = inter;
     m.accumulate = 0;
+    hipStream_t st = as_stream(stream);
+    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(hidden / 256) && IQ3STraits::Quad::addressable(inter, hidden / 256))
+    {
+        // the quad-lane decoder on short rows: steps per wavefront so that a compute unit sees a few
+        // workgroups, each long enough to be worth its staging
+        typedef IQ3STraits::Quad Q;
+        const int nsb = hidden / 256;
+        const long steps = ((long)inter * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+        const long all_steps = steps * n_tokens * top_k * 2;
+        int spw = 2;
+        while (spw < 8 && all_steps / ((long)cu_count(device_id) * MOE_QUAD_WAVES * 2) >= 2 * spw)
+            spw *= 2;
+        m.rows_per_wave = spw;
+        m.gshift = moe_log2(nsb);
+        const long gx = (steps + (long)MOE_QUAD_WAVES * spw - 1) / ((long)MOE_QUAD_WAVES * spw);
+        const dim3 grid((unsigned)gx, (unsigned)(n_tokens * top_k), 2);
+        hipLaunchKernelGGL((moe_gate_up_quad_kernel<Q>), grid, dim3(MOE_QUAD_WAVES * WAVE), (size_t)nsb * QUAD_SB_LDS, st, m);
+        return launched(fn);
+    }
     long gx;
     moe_shape(inter, hidden / 256, (long)n_tokens * top_k * 2, device_id, m.gshift, m.rows_per_wave, gx);
     const dim3 grid((unsigned)gx, (unsigned)(n_tokens * top_k), 2);
     const dim3 block(GEMV_WAVES * WAVE);
-    hipStream_t st = as_stream(stream);
     switch (fmt)
     {
     case LLAM_FMT_Q4_K:
@@ -1259,11 +1526,33 @@ extern "C" bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts, i
     m.hidden = hidden;
     m.inter = inter;
     m.accumulate = accumulate;
+    hipStream_t st = as_stream(stream);
+    // (with little work per compute unit the launch is a chain of memory round trips: there the kernel that
+    // has the loads of all slots of a row in flight at once is faster -- 1 token 24.1 against 26.9 us per step,
+    // 4 tokens 35.3 against 37.1, 8 tokens 54.9 against 47.5, 16 tokens 78.9 against 67.0)
+    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(inter / 256) && top_k <= MOE_QUAD_MAX_SLOTS &&
+        IQ3STraits::Quad::addressable(hidden, inter / 256) &&
+        (long)hidden * (inter / 256) / QUAD_STEP_SB * n_tokens * top_k >= 48L * cu_count(device_id))
+    {
+        // the quad-lane decoder on short rows: workgroups of a step or more per wavefront, at least
+        // two of them per compute unit
+        typedef IQ3STraits::Quad Q;
+        const int nsb = inter / 256;
+        const long steps = ((long)hidden * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+        int spw = 1;
+        while (spw < 8 && steps * n_tokens / ((long)cu_count(device_id) * MOE_QUAD_WAVES * 2) >= 2 * spw)
+            spw *= 2;
+        m.rows_per_wave = spw;
+        m.gshift = moe_log2(nsb);
+        const long gx = (steps + (long)MOE_QUAD_WAVES * spw - 1) / ((long)MOE_QUAD_WAVES * spw);
+        hipLaunchKernelGGL((moe_down_quad_kernel<Q>), dim3((unsigned)gx, (unsigned)n_tokens), dim3(MOE_QUAD_WAVES * WAVE),
+                           (size_t)top_k * nsb * QUAD_SB_LDS, st, m);
+        return launched(fn);
+    }
     long gx;
     moe_shape(hidden, inter / 256, (long)n_tokens, device_id, m.gshift, m.rows_per_wave, gx);
     const dim3 grid((unsigned)gx, (unsigned)n_tokens);
     const dim3 block(GEMV_WAVES * WAVE);
-    hipStream_t st = as_stream(stream);
     switch (fmt)
     {
     case LLAM_FMT_Q4_K: return moe_down_launch<Q4KTraits>(fn, m, grid, block, st);
