@@ -728,8 +728,9 @@ namespace llamql
         // ">> 8, keep the low byte" is "take the high byte".
         __device__ __forceinline__ static int requant4(uint32_t q, v2s ff, v2s cc)
         {
-            const uint32_t e = q & 0x00FF00FFu;
-            const uint32_t o = (q >> 8) & 0x00FF00FFu;
+            // bytes 0, 2 and bytes 1, 3 of q, each widened to 16 bits: one byte permute apiece
+            const uint32_t e = __builtin_amdgcn_perm(0u, q, 0x0C020C00u);
+            const uint32_t o = __builtin_amdgcn_perm(0u, q, 0x0C030C01u);
             const v2s re = __builtin_bit_cast(v2s, e) * ff + cc;
             const v2s ro = __builtin_bit_cast(v2s, o) * ff + cc;
             return (int)__builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, ro), __builtin_bit_cast(uint32_t, re),
