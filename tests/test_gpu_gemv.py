@@ -704,3 +704,50 @@ def test_accumulating_launch_is_refused_where_the_kernel_cannot(capi, dev):
     q8 = capi.quantize_q8_1(torch.randn(1, K, device=dev))
     with pytest.raises(capi.QLError):
         capi.gemv_accumulate(FMT_Q4_K, w, q8, 1, N, K, torch.zeros(1, N, device=dev))
+
+
+def test_read_probe_runs_and_checks_its_arguments(capi, dev):
+    """The read-only probes behind bench.py --workload read-order: every pattern runs on a small buffer (they read
+    inside N * K/256 * 144 bytes and write nothing), bad arguments are refused."""
+    import torch
+
+    lib = capi.load()
+    N, K = 96, 4096
+    buf = torch.randint(0, 256, (N * (K // 256) * 144 + 64,), dtype=torch.uint8, device=dev)
+    guard = buf[-64:].clone()
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    for pattern, rpw, depth, wgs in ((0, 3, 2, 0), (1, 3, 1, 0), (1, 5, 4, 0), (2, 0, 3, 4), (3, 0, 6, 4), (3, 0, 9, 2)):
+        assert lib.llam_ql_read_probe(buf.data_ptr(), N, K, pattern, rpw, 4, depth, wgs, sink.data_ptr(), 0, None), capi.last_error()
+    sync()
+    assert torch.equal(buf[-64:], guard) and int(sink[0]) in (0, 1)
+    for args in ((buf.data_ptr(), N, K, 7, 3, 4, 2, 0), (buf.data_ptr(), N, K, 0, 3, 4, 3, 0), (buf.data_ptr(), N, 1024, 0, 3, 4, 2, 0),
+                 (buf.data_ptr(), N, K, 2, 0, 4, 3, 0), (0, N, K, 0, 3, 4, 2, 0), (buf.data_ptr(), N, K, 0, 3, 17, 2, 0)):
+        assert not lib.llam_ql_read_probe(*args, sink.data_ptr(), 0, None)
+
+
+@pytest.mark.parametrize("fmt,N,K", [(FMT_Q4_K, 8192 + 40, 5120), (FMT_Q6_K, 1000, 25600)])
+def test_batch_tile_heights_agree(capi, dev, oracle, fmt, N, K):
+    """The matrix-unit kernels of batches 5..8 with tiles of 16..32 weight rows (llam_ql_set_batch_tile_rows): every
+    height against the CPU restatement on a row window, and the exact block sums of the kernel that serves the
+    shape unchanged by the height (rows that do not fill the last tile included)."""
+    import torch
+
+    M = 8
+    lib = capi.load()
+    assert capi.gemv_describe(fmt, M, N, K).kernel == 3
+    W = synth.weights_numpy(fmt, N, K, 31)
+    w = capi.prepare_weights(fmt, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
+    x = synth.activations_numpy(M, K, 6)
+    q8 = capi.quantize_q8_1(torch.from_numpy(x).to(dev))
+    rows = slice(N - 70, N)
+    exp, exp_sums = oracle.gemm(fmt, W[rows], K, oracle.quantize(x), want_sums=True)
+    try:
+        for tr in (0, 32, 27, 20, 16):
+            lib.llam_ql_set_batch_tile_rows(tr)
+            y = capi.gemv(fmt, w, q8, M, N, K)
+            s = capi.gemv_block_sums(fmt, w, q8, M, N, K, N - 70, 70)
+            sync()
+            assert rel_err(y.cpu().numpy()[:, rows], exp) <= TOL[fmt] * 1e-2, tr
+            assert np.array_equal(s.cpu().numpy(), exp_sums), tr   # bit-exact whatever the tile height
+    finally:
+        lib.llam_ql_set_batch_tile_rows(0)
