@@ -8,11 +8,14 @@
 // integer map  w = +-round(g*127/gmax)  (gmax = largest magnitude in the
 // sub-block; never a tie) with  b_scale = f16((gmax*db)/127).  Every magnitude is odd,
 // g = 2k+1 with k in 0..7, so for a given gmax the map is an 8-entry byte table.  The kernels
-// keep in (static) LDS, 4.6 KB: the codebook as k-bytes (2 KB), the maps, and a 256-entry
-// table that turns eight sign bits into two byte masks; a sub-block costs eight codebook
-// gathers, one map fetch and four sign-mask gathers, and per four weights one v_perm_b32
-// (map), one subtraction (bytewise negation: every magnitude is 1..127) and one v_bfi_b32
-// (signs).
+// keep in (static) LDS, 4.9 KB: the codebook as k-bytes (2 KB), the maps, a 256-entry
+// table that turns eight sign bits into two byte masks, and the 48 products (15 - 2 hint) *
+// (1 + 2 nib) as floats; a sub-block costs eight codebook gathers, one map fetch, four sign-mask
+// gathers and one scale fetch, and per four weights one v_perm_b32 (map), one subtraction
+// (bytewise negation: every magnitude is 1..127) and one v_bfi_b32 (signs).  (Signs through one
+// v_xad_u32, (w ^ mask) + ones, need the masks' 0x01 bytes from the table as well: eight vector
+// instructions fewer per sub-block and 16-byte gathers for 8-byte ones, 5 % slower -- the LDS
+// is as busy as the vector unit here.)
 //
 // What a sub-block needs beyond its bytes is worked out when the weights are prepared and kept
 // as a two-bit hint per sub-block in the two spare bytes of the super-block's meta record:
@@ -44,10 +47,11 @@ namespace llamql
         uint32_t map[10][2];  // map[7 - gi]: bytes round((2k+1)*127/(2*gi+1)) for k = 0..7 (k > gi is never
                               // looked up); map[8], map[9]: zeros (an all-zero sub-block)
         uint32_t sgn[256][2]; // eight sign bits -> 0xFF bytes where the bit is set: elements 0-3, 4-7
+        float gmul[4][16];    // [hint][nib]: (15 - 2 hint) * (1 + 2 nib), what d is multiplied by in a regular sub-block
         bool odd;             // every codebook magnitude is odd and at most 15
     };
-    constexpr int IQ3S_TABLE_BYTES = 2048 + 512 + 80 + 2048;
-    constexpr int IQ3S_OFF_CBMAX = 2048, IQ3S_OFF_MAP = 2560, IQ3S_OFF_SGN = 2640;
+    constexpr int IQ3S_TABLE_BYTES = 2048 + 512 + 80 + 2048 + 256;
+    constexpr int IQ3S_OFF_CBMAX = 2048, IQ3S_OFF_MAP = 2560, IQ3S_OFF_SGN = 2640, IQ3S_OFF_GMUL = 4688;
     constexpr uint32_t IQ3S_MAP_ZERO = 8; // index of the all-zero map
 
     constexpr IQ3STables make_iq3s_tables()
@@ -87,11 +91,15 @@ namespace llamql
             for (int b = 0; b < 8; ++b)
                 if (s8 & (1 << b))
                     t.sgn[s8][b >> 2] |= 0xFFu << (8 * (b & 3));
+        for (int h = 0; h < 3; ++h)
+            for (int nib = 0; nib < 16; ++nib)
+                t.gmul[h][nib] = (float)((15 - 2 * h) * (1 + 2 * nib));
         return t;
     }
     static_assert(make_iq3s_tables().odd, "IQ3_S codebook magnitudes must be odd and at most 15");
     static_assert(offsetof(IQ3STables, cbmax) == IQ3S_OFF_CBMAX && offsetof(IQ3STables, map) == IQ3S_OFF_MAP &&
-                      offsetof(IQ3STables, sgn) == IQ3S_OFF_SGN && offsetof(IQ3STables, odd) == IQ3S_TABLE_BYTES &&
+                      offsetof(IQ3STables, sgn) == IQ3S_OFF_SGN && offsetof(IQ3STables, gmul) == IQ3S_OFF_GMUL &&
+                      offsetof(IQ3STables, odd) == IQ3S_TABLE_BYTES &&
                       IQ3S_TABLE_BYTES % 16 == 0,
                   "table offsets the decoder assumes");
 
@@ -174,16 +182,28 @@ namespace llamql
     {
         const uint8_t *tab = iq3s_tables_lds();
 
-        // byte offsets of the eight codebook entries: (qs byte l) * 4 + (bit l of qh) * 1024
+        // Byte offsets of the eight codebook entries: (qs byte l) * 4 + (bit l of qh) * 1024, that is
+        // low byte (b << 2) & 0xFC and high byte (b >> 6) | bit << 2.  Four at a time: the dword of
+        // index bytes rotated right by six holds, in byte l, the two top bits of index byte l at the
+        // bottom and the six low bits of index byte l + 1 above them; four bits of qh times a constant
+        // with one bit per byte land on bit 2 of bytes 0..3 (the shifted copies of the four bits do
+        // not overlap: nothing carries).  One v_perm_b32 per offset then picks its two bytes: 6 + 4
+        // instructions per dword where shifting and merging each offset by itself took 12.
         uint32_t off[8];
-        {
-            const uint32_t two = 2u;
-            const uint32_t a[8] = {byte_shl<0>(qs.x, two), byte_shl<1>(qs.x, two), byte_shl<2>(qs.x, two),
-                                   byte_shl<3>(qs.x, two), byte_shl<0>(qs.y, two), byte_shl<1>(qs.y, two),
-                                   byte_shl<2>(qs.y, two), byte_shl<3>(qs.y, two)};
 #pragma unroll
-            for (int l = 0; l < 8; ++l)
-                off[l] = ((qh << (10 - l)) & 0x400u) | a[l]; // v_lshlrev_b32 + v_and_or_b32
+        for (int h = 0; h < 2; ++h)
+        {
+            const uint32_t q = h ? qs.y : qs.x;
+            const uint32_t rot = __builtin_amdgcn_alignbit(q, q, 6);
+            const uint32_t lo = rot & 0xFCFCFCFCu;  // byte l: (index byte (l + 1) & 3) << 2, truncated
+            const uint32_t top = rot & 0x03030303u; // byte l: (index byte l) >> 6
+            const uint32_t nib4 = h ? (qh >> 4) & 0xFu : qh & 0xFu;
+            const uint32_t spread = __umul24(nib4, (1u << 2) | (1u << 9) | (1u << 16) | (1u << 23)); // bit l -> bit 8 l + 2
+            const uint32_t hi = (spread & 0x04040404u) | top;
+            off[4 * h + 0] = __builtin_amdgcn_perm(hi, lo, 0x0C0C0403u);
+            off[4 * h + 1] = __builtin_amdgcn_perm(hi, lo, 0x0C0C0500u);
+            off[4 * h + 2] = __builtin_amdgcn_perm(hi, lo, 0x0C0C0601u);
+            off[4 * h + 3] = __builtin_amdgcn_perm(hi, lo, 0x0C0C0702u);
         }
         uint32_t e[8];
 #pragma unroll
@@ -195,7 +215,8 @@ namespace llamql
         uint32_t mi = hint; // which map
         uint32_t sg_all = signs;
         {
-            const float amax = d * (float)((15u - 2u * hint) * (2u * nib + 1u));
+            // (15 - 2 hint) * (1 + 2 nib) as a float from a 64-entry table: three instructions for seven
+            const float amax = d * *reinterpret_cast<const float *>(tab + IQ3S_OFF_GMUL + ((hint << 6) | (nib << 2)));
             const float c = 0x1.020408p-7f;
             const float q0 = amax * c;
             const float q1 = fmaf(fmaf(-q0, 127.0f, amax), c, q0); // div_by_127 of a finite non-zero value
