@@ -191,6 +191,30 @@ namespace llamql
         }
     }
 
+    // The same layout from blocks fetched ahead (quad_act_issue: block idx = m * nkb + kb of whole rows).
+    constexpr int MFMA_ACT_PASSES = 3; // eight rows of 5120 over eight wavefronts
+    __device__ __forceinline__ void mfma_act_store(const QuadActRaw (&r)[MFMA_ACT_PASSES], int nkb, int total, uint8_t *aq,
+                                                   float *asc)
+    {
+#pragma unroll
+        for (int p = 0; p < MFMA_ACT_PASSES; ++p)
+        {
+            const int idx = (int)threadIdx.x + p * (int)blockDim.x;
+            if (idx < total)
+            {
+                const int m = idx / nkb, kb = idx - m * nkb;
+                const uint32_t head = (uint32_t)r[p].lo.x;
+                const float d = h2f((uint16_t)(head & 0xFFFFu));
+                uint4 *dst = reinterpret_cast<uint4 *>(aq + (size_t)kb * MFMA_AQ_STRIDE + m * 32);
+                dst[0] = make_uint4((uint32_t)r[p].lo.y, (uint32_t)r[p].lo.z, (uint32_t)r[p].lo.w, (uint32_t)r[p].hi.x);
+                dst[1] = make_uint4((uint32_t)r[p].hi.y, (uint32_t)r[p].hi.z, (uint32_t)r[p].hi.w, (uint32_t)r[p].tail);
+                float *sc = asc + (size_t)kb * 16 + (m >> 2) * 8 + (m & 3);
+                sc[0] = d;
+                sc[4] = (float)(int16_t)(head >> 16) * d;
+            }
+        }
+    }
+
     // SRC: where the activations come from (QUAD_SRC_*): Q8_1 blocks, or fp32 rows quantised here.
     // DUMP: also store the matrix unit's results, the exact int32 block sums (the parity hook).
     // Its stores need registers the 16-wavefront workgroup does not have (and the build refuses to
@@ -255,11 +279,29 @@ namespace llamql
             mfma_load(r, reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo), off);
         };
         MfmaRaw bufA, bufB;
-        issue(bufA, 0);
-        issue(bufB, 1);
-
         // ---- activations into LDS ------------------------------------------------------------
-        mfma_stage_acts<SRC>(a.q8, a.x, a.x2, a.ldx, a.M, nkb, 0, nkb, aq, asc, (int)threadIdx.x, (int)blockDim.x);
+        if constexpr (SRC == QUAD_SRC_Q8)
+        {
+            // Q8_1 blocks are asked for BEFORE the weights and waited for by themselves (a wavefront's
+            // loads return in issue order: behind two steps of weights per wavefront, 100 KB and more
+            // per compute unit, the staging and its barrier would wait for all of those first)
+            const int total = a.M * nkb;
+            QuadActRaw ar[MFMA_ACT_PASSES];
+            quad_act_issue(ar, a.q8, total);
+            issue(bufA, 0);
+            issue(bufB, 1);
+            quad_act_wait<2 * MFMA_LOADS>(ar);
+            if (total <= MFMA_ACT_PASSES * (int)blockDim.x) // uniform
+                mfma_act_store(ar, nkb, total, aq, asc);
+            else
+                mfma_stage_acts<SRC>(a.q8, a.x, a.x2, a.ldx, a.M, nkb, 0, nkb, aq, asc, (int)threadIdx.x, (int)blockDim.x);
+        }
+        else
+        {
+            issue(bufA, 0);
+            issue(bufB, 1);
+            mfma_stage_acts<SRC>(a.q8, a.x, a.x2, a.ldx, a.M, nkb, 0, nkb, aq, asc, (int)threadIdx.x, (int)blockDim.x);
+        }
         __syncthreads();
         mfma_keep(bufA); // the staging code must not reuse the registers of the loads in flight
         mfma_keep(bufB);

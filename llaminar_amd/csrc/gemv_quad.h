@@ -152,10 +152,11 @@ namespace llamql
         v4i lo, hi;
         int tail;
     };
-    __device__ __forceinline__ void quad_act_issue(QuadActRaw (&r)[QUAD_ACT_PASSES], const uint32_t *q8, int total)
+    template <int PASSES>
+    __device__ __forceinline__ void quad_act_issue(QuadActRaw (&r)[PASSES], const uint32_t *q8, int total)
     {
 #pragma unroll
-        for (int p = 0; p < QUAD_ACT_PASSES; ++p)
+        for (int p = 0; p < PASSES; ++p)
         {
             int idx = (int)threadIdx.x + p * (int)blockDim.x;
             idx = idx < total ? idx : total - 1;
@@ -166,12 +167,12 @@ namespace llamql
         }
     }
     // until at most NEWER vector memory operations issued after the activation loads are pending
-    template <int NEWER>
-    __device__ __forceinline__ void quad_act_wait(QuadActRaw (&r)[QUAD_ACT_PASSES])
+    template <int NEWER, int PASSES>
+    __device__ __forceinline__ void quad_act_wait(QuadActRaw (&r)[PASSES])
     {
         static_assert(NEWER <= 63, "vmcnt is a 6-bit counter");
 #pragma unroll
-        for (int p = 0; p < QUAD_ACT_PASSES; ++p)
+        for (int p = 0; p < PASSES; ++p)
             asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r[p].lo), "+v"(r[p].hi), "+v"(r[p].tail) : "n"(NEWER));
     }
     template <class Q>
