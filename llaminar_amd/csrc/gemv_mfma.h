@@ -192,7 +192,7 @@ namespace llamql
     }
 
     // The same layout from blocks fetched ahead (quad_act_issue: block idx = m * nkb + kb of whole rows).
-    constexpr int MFMA_ACT_PASSES = 3; // eight rows of 5120 over eight wavefronts
+    constexpr int MFMA_ACT_PASSES = 4; // eight rows of 8192 over eight wavefronts
     __device__ __forceinline__ void mfma_act_store(const QuadActRaw (&r)[MFMA_ACT_PASSES], int nkb, int total, uint8_t *aq,
                                                    float *asc)
     {
