@@ -469,36 +469,53 @@ namespace llamql
         }
         __syncthreads();
 
-        // statistics: wavefront w takes heads w, w + 4, ...
-        for (int g = wave; g < G; g += ATT_WAVES)
+        // statistics: wavefront w takes heads w, w + 4, ..., all of them side by side (their reductions are
+        // chains of dependent cross-lane steps: one after the other they were a tenth of the kernel)
         {
             constexpr int PER_LANE = ATT_CHUNK / WAVE;
-            float sc[PER_LANE];
-            float mx = -INFINITY;
+            constexpr int HEADS = (G + ATT_WAVES - 1) / ATT_WAVES; // heads per wavefront
+            float sc[HEADS][PER_LANE], mx[HEADS], l[HEADS];
 #pragma unroll
-            for (int k = 0; k < PER_LANE; ++k)
+            for (int h = 0; h < HEADS; ++h)
             {
-                sc[k] = s_sc[g][lane + WAVE * k];
-                mx = fmaxf(mx, sc[k]);
+                const int g = wave + ATT_WAVES * h;
+                mx[h] = -INFINITY;
+#pragma unroll
+                for (int k = 0; k < PER_LANE; ++k)
+                {
+                    sc[h][k] = s_sc[g < G ? g : 0][lane + WAVE * k];
+                    mx[h] = fmaxf(mx[h], sc[h][k]);
+                }
             }
 #pragma unroll
-            for (int off = WAVE / 2; off > 0; off >>= 1)
-                mx = fmaxf(mx, __shfl_xor(mx, off, WAVE));
-            float l = 0.0f;
+            for (int h = 0; h < HEADS; ++h)
+                mx[h] = wave_max(mx[h]);
 #pragma unroll
-            for (int k = 0; k < PER_LANE; ++k)
+            for (int h = 0; h < HEADS; ++h)
             {
-                const float e = expf(sc[k] - mx); // position p0 is valid: mx is finite
-                s_sc[g][lane + WAVE * k] = e;
-                l += e;
+                const int g = wave + ATT_WAVES * h;
+                l[h] = 0.0f;
+#pragma unroll
+                for (int k = 0; k < PER_LANE; ++k)
+                {
+                    const float e = expf(sc[h][k] - mx[h]); // position p0 is valid: mx is finite
+                    if (g < G)
+                        s_sc[g][lane + WAVE * k] = e;
+                    l[h] += e;
+                }
             }
 #pragma unroll
-            for (int off = WAVE / 2; off > 0; off >>= 1)
-                l += __shfl_xor(l, off, WAVE);
-            if (lane == 0)
+            for (int h = 0; h < HEADS; ++h)
+                l[h] = wave_sum(l[h]);
+#pragma unroll
+            for (int h = 0; h < HEADS; ++h)
             {
-                part_ml[(out_base + (size_t)g * n_chunks) * 2 + 0] = mx;
-                part_ml[(out_base + (size_t)g * n_chunks) * 2 + 1] = l;
+                const int g = wave + ATT_WAVES * h;
+                if (lane == 0 && g < G)
+                {
+                    part_ml[(out_base + (size_t)g * n_chunks) * 2 + 0] = mx[h];
+                    part_ml[(out_base + (size_t)g * n_chunks) * 2 + 1] = l[h];
+                }
             }
         }
         __syncthreads();
@@ -596,9 +613,7 @@ namespace llamql
         float mx = -INFINITY;
         for (int k = c; k < used; k += ATT_HD)
             mx = fmaxf(mx, part_ml[(base + k) * 2]);
-#pragma unroll
-        for (int off = WAVE / 2; off > 0; off >>= 1)
-            mx = fmaxf(mx, __shfl_xor(mx, off, WAVE));
+        mx = wave_max(mx);
         if ((c & (WAVE - 1)) == 0)
             s_red[c >> 6] = mx;
         __syncthreads();
@@ -611,9 +626,7 @@ namespace llamql
             s_w[k] = w;
             l = fmaf(part_ml[(base + k) * 2 + 1], w, l);
         }
-#pragma unroll
-        for (int off = WAVE / 2; off > 0; off >>= 1)
-            l += __shfl_xor(l, off, WAVE);
+        l = wave_sum(l);
         if ((c & (WAVE - 1)) == 0)
             s_red[c >> 6] = l;
         __syncthreads();

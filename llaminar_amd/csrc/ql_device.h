@@ -147,6 +147,21 @@ namespace llamql
         return (r0 + r1) + (r2 + r3);
     }
 
+    // Maximum over the 64 lanes of a wavefront; every lane returns it.
+    __device__ __forceinline__ float wave_max(float v)
+    {
+        v = fmaxf(v, dpp_f32<DPP_QUAD_XOR1>(v));
+        v = fmaxf(v, dpp_f32<DPP_QUAD_XOR2>(v));
+        v = fmaxf(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v));
+        v = fmaxf(v, dpp_f32<DPP_ROW_MIRROR>(v));
+        const int b = __float_as_int(v);
+        const float r0 = __int_as_float(__builtin_amdgcn_readlane(b, 0));
+        const float r1 = __int_as_float(__builtin_amdgcn_readlane(b, 16));
+        const float r2 = __int_as_float(__builtin_amdgcn_readlane(b, 32));
+        const float r3 = __int_as_float(__builtin_amdgcn_readlane(b, 48));
+        return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+    }
+
     // ---- Q8_1 quantiser, one lane's share ---------------------------------------------
     // Eight neighbouring lanes (lane & 7 = 0..7) own one 32-element block, four values
     // each; all eight must be active.  Arithmetic of the reference's quantiser
