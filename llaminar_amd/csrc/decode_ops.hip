@@ -118,9 +118,7 @@ namespace llamql
             }
             square(v);
         }
-#pragma unroll
-        for (int off = WAVE / 2; off > 0; off >>= 1)
-            acc += __shfl_xor(acc, off, WAVE);
+        acc = wave_sum(acc);
         if ((threadIdx.x & (WAVE - 1)) == 0)
             s_part[threadIdx.x >> 6] = acc;
         __syncthreads();

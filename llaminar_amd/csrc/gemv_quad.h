@@ -295,12 +295,7 @@ namespace llamql
             acc += (double)v.z * (double)v.z;
             acc += (double)v.w * (double)v.w;
         };
-        auto butterfly = [](double acc) {
-#pragma unroll
-            for (int off = WAVE / 2; off > 0; off >>= 1)
-                acc += __shfl_xor(acc, off, WAVE);
-            return acc;
-        };
+        auto butterfly = [](double acc) { return wave_sum(acc); }; // the stand-alone norm's reduction
         auto inverse_rms = [&](int m) {
             double sum_sq = 0.0;
 #pragma unroll

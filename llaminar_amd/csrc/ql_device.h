@@ -147,6 +147,30 @@ namespace llamql
         return (r0 + r1) + (r2 + r3);
     }
 
+    // The same for a double (two 32-bit halves travel per step); every lane returns the total.
+    template <int CTRL>
+    __device__ __forceinline__ double dpp_f64(double v)
+    {
+        const long long b = __double_as_longlong(v);
+        const int lo = dpp_i32<CTRL>((int)(b & 0xFFFFFFFFLL)), hi = dpp_i32<CTRL>((int)(b >> 32));
+        return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+    }
+    __device__ __forceinline__ double wave_sum(double v)
+    {
+        v += dpp_f64<DPP_QUAD_XOR1>(v);
+        v += dpp_f64<DPP_QUAD_XOR2>(v);
+        v += dpp_f64<DPP_ROW_HALF_MIRROR>(v);
+        v += dpp_f64<DPP_ROW_MIRROR>(v);
+        const long long b = __double_as_longlong(v);
+        const int lo = (int)(b & 0xFFFFFFFFLL), hi = (int)(b >> 32);
+        auto row = [&](int lane) {
+            const unsigned int l = (unsigned int)__builtin_amdgcn_readlane(lo, lane);
+            const int h = __builtin_amdgcn_readlane(hi, lane);
+            return __longlong_as_double(((long long)h << 32) | l);
+        };
+        return (row(0) + row(16)) + (row(32) + row(48));
+    }
+
     // Maximum over the 64 lanes of a wavefront; every lane returns it.
     __device__ __forceinline__ float wave_max(float v)
     {
