@@ -234,15 +234,16 @@ def bench_decode(args, torch, capi, synth, dev):
     B = args.batch
     shape = Shape(n_layers=args.decode_layers)
     ctx = args.context
-    cap = (ctx + args.steps + args.warmup + 8 + 7) // 8 * 8   # the attention kernel reads V eight positions at a time
+    cap = (ctx + args.steps + args.warmup + 8 + 31) // 32 * 32   # the caches are kept in tiles of 16 and 32 positions
     t_build = time.perf_counter()
     dec = DenseDecoder(shape, B, cap, dev, seed=11, keep_prepared=True)
     g = torch.Generator(device=dev)
     g.manual_seed(3)
     for l in range(shape.n_layers):   # a cache as `ctx - 1` earlier tokens would have left it
         k, v = dec.buffer("kcache", l), dec.buffer("vcache", l)
-        k[:, :, : ctx - 1].copy_(torch.randn(B, shape.n_kv, ctx - 1, shape.head_dim, device=dev, generator=g))
-        v[:, :, :, : ctx - 1].copy_(torch.randn(B, shape.n_kv, shape.head_dim, ctx - 1, device=dev, generator=g))
+        # (random values: the tiles' order inside the caches does not matter to what the step costs)
+        k.copy_(torch.randn(B, shape.n_kv, cap, shape.head_dim, device=dev, generator=g))
+        v.copy_(torch.randn(B, shape.n_kv, cap, shape.head_dim, device=dev, generator=g))
     ids0 = torch.randint(0, shape.vocab, (B,), generator=torch.Generator().manual_seed(5)).numpy()
     dec.set_state(ids0, [ctx - 1] * B)
     torch.cuda.synchronize()

@@ -57,11 +57,15 @@ void llam_dec_rope_inv_freq(int head_dim, float theta, float *h_inv_freq);
  * Pairs (i, i + head_dim/2) of every Q and K head are rotated by
  * angle = float(pos) * inv_freq[i] (apply_rope_to_head_scalar,
  * RoPEPrimitives.cpp:180-203).  Q is rotated in place; rotated K and V are rounded
- * to fp16 (nearest even) into the caches at position d_pos[b].  Cache layouts:
- * K [B][n_kv][ctx_cap][head_dim] (a position's row is contiguous), V dimension-major
- * [B][n_kv][head_dim][ctx_cap] (eight consecutive positions of one dimension are one
- * 16-byte matrix operand of llam_dec_attention).  0 <= d_pos[b] < ctx_cap is the
- * caller's duty (a position outside is not written).
+ * to fp16 (nearest even) into the caches at position d_pos[b].  Cache layouts: per
+ * (sequence, KV head) a slice of ctx_cap * head_dim fp16 values, [B][n_kv] slices, tiled
+ * for the matrix operands of llam_dec_attention so that each of its load instructions
+ * reads one contiguous kilobyte (head_dim a multiple of 16, ctx_cap of 32):
+ *   K: element (p, d) at (p/16)*16*head_dim + (d/8)*128 + (p%16)*8 + d%8
+ *      (tiles of 16 positions; a 16-byte piece = 8 dims of one position)
+ *   V: element (p, d) at (p/32)*32*head_dim + (d/16)*512 + ((p/8)%4)*128 + (d%16)*8 + p%8
+ *      (tiles of 32 positions; a 16-byte piece = 8 positions of one dim).
+ * 0 <= d_pos[b] < ctx_cap is the caller's duty (a position outside is not written).
  * Replaces RoPEStage + KVCacheAppendStage for decode
  * (src/v2/models/qwen/QwenGraphBase.cpp:2691-2736, 2738-2790). */
 bool llam_dec_rope_kv_append(float *d_qkv, int ld_qkv, const float *d_inv_freq,
@@ -85,7 +89,7 @@ size_t llam_dec_attention_scratch_floats(int B, int n_heads, int head_dim, int c
  * unit in fp16 x fp16 -> fp32: K and V are exact operands, the fp32 factors (q / sqrt(d),
  * the softmax weights) enter as the sum of two fp16 numbers, i.e. to about 2^-22;
  * |q| / sqrt(head_dim) must stay below the fp16 range (65504).
- * head_dim == 128, n_heads / n_kv in {1, 2, 4, 8}, ctx_cap a multiple of 8. */
+ * head_dim == 128, n_heads / n_kv in {1, 2, 4, 8}, ctx_cap a multiple of 32. */
 bool llam_dec_attention(const float *d_q, int ld_q, const void *d_kcache, const void *d_vcache,
                         const int32_t *d_pos, float *d_out, int ld_out, void *d_q8_out,
                         float *d_scratch, int B, int n_heads, int n_kv, int head_dim, int ctx_cap,

@@ -45,7 +45,7 @@ typedef struct
     int ffn;       /* feed-forward width, multiple of 256 */
     int vocab;
     int n_layers;
-    int ctx_cap;   /* KV-cache positions per sequence, a multiple of 8 */
+    int ctx_cap;   /* KV-cache positions per sequence, a multiple of 32 */
     int batch;     /* sequences decoded together, 1..8 */
     float rope_theta;
     float rms_eps;
@@ -97,8 +97,8 @@ bool llam_decoder_advance(void *dec, int n);
 /* Device buffers, for filling caches, reading results and parity checks:
  *   "ids" int32[batch], "pos" int32[batch], "logits" fp32[batch][vocab], "x" fp32[batch][hidden]
  *   (the residual stream as the last step left it, before the final add of "delta"),
- *   "delta" fp32[batch][hidden], "kcache" fp16[batch][n_kv][ctx_cap][head_dim] and
- *   "vcache" fp16[batch][n_kv][head_dim][ctx_cap] of `layer`. */
+ *   "delta" fp32[batch][hidden], "kcache" and "vcache" fp16[batch][n_kv][ctx_cap * head_dim] of `layer`,
+ *   each (sequence, head) slice in the tiles llam_dec_rope_kv_append documents. */
 void *llam_decoder_buffer(void *dec, const char *name, int layer);
 
 /* Bytes of device memory the handle owns. */

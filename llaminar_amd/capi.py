@@ -507,9 +507,45 @@ def rope_inv_freq(head_dim: int, theta: float, device=None):
     return t.to(device) if device is not None else t
 
 
+def kcache_tiled(k):
+    """[..., cap, head_dim] position-major values -> the K cache's tiles (same shape, same values):
+    [cap/16][head_dim/8][16 positions][8 dims] per (sequence, head)."""
+    *lead, cap, hd = k.shape
+    assert cap % 32 == 0 and hd % 16 == 0, "cap a multiple of 32, head_dim of 16"
+    t = k.reshape(*lead, cap // 16, 16, hd // 8, 8)
+    n = len(lead)
+    return t.permute(*range(n), n, n + 2, n + 1, n + 3).reshape(*lead, cap, hd).contiguous()
+
+
+def kcache_logical(k):
+    """The inverse of kcache_tiled."""
+    *lead, cap, hd = k.shape
+    t = k.reshape(*lead, cap // 16, hd // 8, 16, 8)
+    n = len(lead)
+    return t.permute(*range(n), n, n + 2, n + 1, n + 3).reshape(*lead, cap, hd).contiguous()
+
+
+def vcache_tiled(v):
+    """[..., cap, head_dim] position-major values -> the V cache's tiles (same shape, same values):
+    [cap/32][head_dim/16][4 groups of 8 positions][16 dims][8 positions] per (sequence, head)."""
+    *lead, cap, hd = v.shape
+    assert cap % 32 == 0 and hd % 16 == 0, "cap a multiple of 32, head_dim of 16"
+    t = v.reshape(*lead, cap // 32, 4, 8, hd // 16, 16)   # p32, group, p8, d16 tile, d
+    n = len(lead)
+    return t.permute(*range(n), n, n + 3, n + 1, n + 4, n + 2).reshape(*lead, cap, hd).contiguous()
+
+
+def vcache_logical(v):
+    """The inverse of vcache_tiled."""
+    *lead, cap, hd = v.shape
+    t = v.reshape(*lead, cap // 32, hd // 16, 4, 16, 8)   # p32, d16 tile, group, d, p8
+    n = len(lead)
+    return t.permute(*range(n), n, n + 2, n + 4, n + 1, n + 3).reshape(*lead, cap, hd).contiguous()
+
+
 def rope_kv_append(qkv, inv_freq, pos, kcache, vcache, n_heads: int, n_kv: int, head_dim: int, stream=None):
-    """qkv [B, >= (n_heads+2 n_kv)*head_dim] fp32, rotated in place; kcache [B, n_kv, cap, head_dim],
-    vcache [B, n_kv, head_dim, cap] (dimension-major), both fp16."""
+    """qkv [B, >= (n_heads+2 n_kv)*head_dim] fp32, rotated in place; kcache and vcache [B, n_kv, cap, head_dim]
+    fp16 in the tiles of kcache_tiled / vcache_tiled."""
     B = qkv.shape[0]
     cap = kcache.shape[2]
     _check(load().llam_dec_rope_kv_append(_ptr(qkv), _ld(qkv), _ptr(inv_freq), _ptr(pos), _ptr(kcache), _ptr(vcache),
@@ -527,12 +563,12 @@ def attention_scratch(B: int, n_heads: int, head_dim: int, cap: int, device):
 def attention(q, kcache, vcache, pos, n_heads: int, n_kv: int, head_dim: int, out=None, scratch=None, stream=None,
               q8_out=None):
     """out [B, n_heads*head_dim] fp32; q8_out (optional) receives the Q8_1 blocks of the same rows.
-    kcache [B, n_kv, cap, head_dim], vcache [B, n_kv, head_dim, cap] (dimension-major), both fp16."""
+    kcache and vcache [B, n_kv, cap, head_dim] fp16 in the tiles of kcache_tiled / vcache_tiled."""
     import torch
 
     B = q.shape[0]
     cap = kcache.shape[2]
-    assert tuple(vcache.shape) == (kcache.shape[0], kcache.shape[1], kcache.shape[3], cap), "V cache is [B, n_kv, head_dim, cap]"
+    assert tuple(vcache.shape) == tuple(kcache.shape), "both caches are [B, n_kv, cap, head_dim]"
     if out is None:
         out = torch.empty(B, n_heads * head_dim, dtype=torch.float32, device=q.device)
     if scratch is None:
@@ -562,7 +598,7 @@ def rope_attention(qkv, table, pos, kcache, vcache, n_heads: int, n_kv: int, hea
 
     B = qkv.shape[0]
     cap = kcache.shape[2]
-    assert tuple(vcache.shape) == (kcache.shape[0], kcache.shape[1], kcache.shape[3], cap), "V cache is [B, n_kv, head_dim, cap]"
+    assert tuple(vcache.shape) == tuple(kcache.shape), "both caches are [B, n_kv, cap, head_dim]"
     if out is None:
         out = torch.empty(B, n_heads * head_dim, dtype=torch.float32, device=qkv.device)
     if scratch is None:

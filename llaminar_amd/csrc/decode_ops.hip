@@ -160,10 +160,28 @@ namespace llamql
             emit(i, row[i], g4[i]);
     }
 
+    // ---- the caches' tiles ---------------------------------------------------------------
+    // Both caches hold, per (sequence, KV head), ctx_cap x head_dim fp16 values in tiles laid out for
+    // the attention kernel's matrix operands, so that every load instruction of a wavefront (64
+    // lanes x 16 bytes) reads ONE contiguous kilobyte instead of 64 pieces of 16 bytes:
+    //   K: tiles of 16 positions, [position / 16][dim / 8][position % 16][dim % 8]
+    //      (a lane's operand: 8 dims of one position; 16 neighbouring lanes: 16 positions)
+    //   V: tiles of 32 positions, [position / 32][dim / 16][(position / 8) % 4][dim % 16][position % 8]
+    //      (a lane's operand: 8 positions of one dim; 16 neighbouring lanes: 16 dims)
+    // Element offsets inside the (sequence, head) slice; head_dim a multiple of 16, ctx_cap of 32.
+    __host__ __device__ inline size_t kv_k_offset(int p, int d, int head_dim)
+    {
+        return (size_t)(p >> 4) * (size_t)(16 * head_dim) + (size_t)(d >> 3) * 128 + (size_t)(p & 15) * 8 + (size_t)(d & 7);
+    }
+    __host__ __device__ inline size_t kv_v_offset(int p, int d, int head_dim)
+    {
+        return (size_t)(p >> 5) * (size_t)(32 * head_dim) + (size_t)(d >> 4) * 512 + (size_t)((p >> 3) & 3) * 128 +
+               (size_t)(d & 15) * 8 + (size_t)(p & 7);
+    }
+
     // ---- rotary embedding + KV append -----------------------------------------------------
     // One workgroup of head_dim/2 threads per (sequence, head); heads n_heads.. are the K
-    // heads, whose workgroups also copy the matching V head (K cache [ctx_cap][head_dim] per
-    // head, V cache [head_dim][ctx_cap]).
+    // heads, whose workgroups also copy the matching V head.
     // (x0, x1) rotated by the angle whose cosine and sine are c and s; every product and sum is
     // rounded on its own, as in the scalar host code (apply_rope_to_head_scalar)
     __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float &r0, float &r1)
@@ -196,15 +214,12 @@ namespace llamql
         if (p < 0 || p >= ctx_cap)
             return;
         const int kh = h - n_heads;
-        const size_t at = (((size_t)b * n_kv + kh) * ctx_cap + p) * head_dim;
-        kcache[at + i] = __float2half_rn(r0);
-        kcache[at + i + half_dim] = __float2half_rn(r1);
+        const size_t slice = ((size_t)b * n_kv + kh) * (size_t)ctx_cap * head_dim;
+        kcache[slice + kv_k_offset(p, i, head_dim)] = __float2half_rn(r0);
+        kcache[slice + kv_k_offset(p, i + half_dim, head_dim)] = __float2half_rn(r1);
         const float *vhead = row + (size_t)(n_heads + n_kv + kh) * head_dim;
-        // V is kept dimension-major, [head_dim][ctx_cap]: the attention kernel reads eight
-        // consecutive positions of one dimension as one 16-byte matrix operand
-        __half *vcol = vcache + ((size_t)b * n_kv + kh) * head_dim * ctx_cap + p;
-        vcol[(size_t)i * ctx_cap] = __float2half_rn(vhead[i]);
-        vcol[(size_t)(i + half_dim) * ctx_cap] = __float2half_rn(vhead[i + half_dim]);
+        vcache[slice + kv_v_offset(p, i, head_dim)] = __float2half_rn(vhead[i]);
+        vcache[slice + kv_v_offset(p, i + half_dim, head_dim)] = __float2half_rn(vhead[i + half_dim]);
     }
 
     // cos and sin of float(pos[b]) * inv_freq[i]: the same for every layer of a decode step
@@ -227,7 +242,7 @@ namespace llamql
     //   output  O[head][d] = sum_pos e[head][pos] V[pos][d]   A = e rows, B = V columns: lane (d, g)
     //                                                          holds 8 positions of its dim, which
     //                                                          are contiguous in the V cache's
-    //                                                          [head_dim][ctx_cap] layout
+    //                                                          tiles (kv_v_offset)
     // K and V are exact fp16 operands.  The fp32 factors (Q, e) enter as the sum of two fp16 numbers,
     // high part and remainder, after a scaling by a power of two that keeps the remainders out of
     // the subnormal range, so every product is that of the fp32 value to about 2^-22.
@@ -280,7 +295,7 @@ namespace llamql
         if (p0 > last)
             return; // no position in this chunk yet: the merge does not read it
         const __half *kbase = kcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
-        const __half *vbase = vcache + ((size_t)b * n_kv + kh) * ATT_HD * ctx_cap;
+        const __half *vbase = vcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
         const int pw = p0 + wave * ATT_PER_WAVE; // first position of this wavefront
 
         // ROPE: the few values of the rotation are requested first: loads return in order, and the
@@ -322,20 +337,20 @@ namespace llamql
         for (int t = 0; t < 2; ++t)
         {
             const int p = pw + 16 * t + n;
-            const __half *row = kbase + (size_t)(p <= last ? p : last) * ATT_HD + 8 * gq; // rows past the end: weight 0
+            const __half *row = kbase + kv_k_offset(p <= last ? p : last, 8 * gq, ATT_HD); // rows past the end: weight 0
 #pragma unroll
             for (int s = 0; s < 4; ++s)
-                kraw[t][s] = *reinterpret_cast<const uint4 *>(row + 32 * s);
+                kraw[t][s] = *reinterpret_cast<const uint4 *>(row + 512 * s); // dims 32 s further: four 8-dim groups of 128 values
         }
         // V: column tile ct holds dims 16 ct + n, positions pw + 8 gq .. + 7 (a group that starts
         // past the newest position is read at the newest one's group; the mask below clears it)
         uint4 vraw[8];
         const int pg = pw + 8 * gq;
         {
-            const __half *colp = vbase + (size_t)n * ctx_cap + (pg <= last ? pg : (last & ~7));
+            const __half *colp = vbase + kv_v_offset(pg <= last ? pg : (last & ~7), n, ATT_HD);
 #pragma unroll
             for (int ct = 0; ct < 8; ++ct)
-                vraw[ct] = *reinterpret_cast<const uint4 *>(colp + (size_t)(16 * ct) * ctx_cap);
+                vraw[ct] = *reinterpret_cast<const uint4 *>(colp + 512 * ct); // dims 16 ct further
         }
 
         if (ROPE)
@@ -362,15 +377,15 @@ namespace llamql
                 s_new[is_v][i + HALF] = h1;
                 if (is_v)
                 {
-                    __half *vcol = vcache + ((size_t)b * n_kv + kh) * ATT_HD * ctx_cap + p;
-                    vcol[(size_t)i * ctx_cap] = h0;
-                    vcol[(size_t)(i + HALF) * ctx_cap] = h1;
+                    __half *vhead = vcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
+                    vhead[kv_v_offset(p, i, ATT_HD)] = h0;
+                    vhead[kv_v_offset(p, i + HALF, ATT_HD)] = h1;
                 }
                 else
                 {
-                    __half *krow = kcache + (((size_t)b * n_kv + kh) * ctx_cap + p) * ATT_HD;
-                    krow[i] = h0;
-                    krow[i + HALF] = h1;
+                    __half *khead = kcache + ((size_t)b * n_kv + kh) * ctx_cap * ATT_HD;
+                    khead[kv_k_offset(p, i, ATT_HD)] = h0;
+                    khead[kv_k_offset(p, i + HALF, ATT_HD)] = h1;
                 }
             }
             __syncthreads();
@@ -825,8 +840,10 @@ extern "C" bool llam_dec_rope_kv_append(float *d_qkv, int ld_qkv, const float *d
         return fail(fn, "bad size");
     if (B == 0)
         return true;
-    if ((head_dim % 2) != 0 || head_dim / 2 > 1024)
-        return fail(fn, "head_dim=%d must be even and at most 2048", head_dim);
+    if ((head_dim % 16) != 0 || head_dim / 2 > 1024)
+        return fail(fn, "head_dim=%d must be a multiple of 16 and at most 2048", head_dim);
+    if ((ctx_cap % 32) != 0)
+        return fail(fn, "ctx_cap=%d must be a multiple of 32 (the caches are kept in tiles of 16 and 32 positions)", ctx_cap);
     if (ld_qkv < (n_heads + 2 * n_kv) * head_dim)
         return fail(fn, "ld_qkv=%d smaller than (n_heads + 2 n_kv) * head_dim", ld_qkv);
     if (!d_qkv || !d_inv_freq || !d_pos || !d_kcache || !d_vcache)
@@ -876,8 +893,8 @@ namespace
         if (!aligned16(d_q) || (ld_q % 4) != 0 || !aligned16(d_kcache) || !aligned16(d_vcache) ||
             (d_out && !aligned4(d_out)) || (d_q8_out && !aligned4(d_q8_out)) || !aligned16(d_scratch))
             return fail(fn, "misaligned pointer (q, caches and scratch 16-byte, out 4-byte)");
-        if ((ctx_cap % 8) != 0)
-            return fail(fn, "ctx_cap=%d must be a multiple of 8 (the V cache is read eight positions at a time)",
+        if ((ctx_cap % 32) != 0)
+            return fail(fn, "ctx_cap=%d must be a multiple of 32 (the caches are kept in tiles of 16 and 32 positions)",
                         ctx_cap);
         const int n_chunks = (ctx_cap + ATT_CHUNK - 1) / ATT_CHUNK;
         if (n_chunks > ATT_MAX_CHUNKS || B > 65535)

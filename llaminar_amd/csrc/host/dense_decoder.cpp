@@ -109,9 +109,9 @@ extern "C" void *llam_decoder_create(const llam_decoder_config *c)
         return nullptr;
     }
     if (c->batch < 1 || c->batch > LLAM_QL_MAX_GEMV_M || c->n_layers < 1 || c->vocab < 1 || c->ctx_cap < 1 ||
-        (c->ctx_cap % 8) != 0)
+        (c->ctx_cap % 32) != 0)
     {
-        fail("create", "batch=%d (1..%d), n_layers=%d, vocab=%d, ctx_cap=%d (a multiple of 8)", c->batch, LLAM_QL_MAX_GEMV_M, c->n_layers,
+        fail("create", "batch=%d (1..%d), n_layers=%d, vocab=%d, ctx_cap=%d (a multiple of 32)", c->batch, LLAM_QL_MAX_GEMV_M, c->n_layers,
              c->vocab, c->ctx_cap);
         return nullptr;
     }

@@ -175,7 +175,7 @@ class DenseDecoder:
         shapes = {"ids": ((B,), torch.int32), "pos": ((B,), torch.int32), "logits": ((B, s.vocab), torch.float32),
                   "x": ((B, s.hidden), torch.float32), "delta": ((B, s.hidden), torch.float32),
                   "kcache": ((B, s.n_kv, self.ctx_cap, s.head_dim), torch.float16),
-                  "vcache": ((B, s.n_kv, s.head_dim, self.ctx_cap), torch.float16)}   # dimension-major
+                  "vcache": ((B, s.n_kv, self.ctx_cap, s.head_dim), torch.float16)}   # both in tiles (capi.kcache_tiled, vcache_tiled)
         shp, dt = shapes[name]
         n = 1
         for v in shp:

@@ -71,7 +71,7 @@ def test_rmsnorm_q8_1(capi, dev, oracle, M, H):
 def test_rope_kv_append(capi, dev, oracle, B, n_heads, n_kv):
     import torch
 
-    hd, cap, theta = 128, 40, 1e6
+    hd, cap, theta = 128, 64, 1e6
     rng = np.random.default_rng(B + n_heads)
     width = (n_heads + 2 * n_kv) * hd
     qkv = rng.standard_normal((B, width + 16)).astype(np.float32)
@@ -79,14 +79,14 @@ def test_rope_kv_append(capi, dev, oracle, B, n_heads, n_kv):
     pos_h[0] = cap - 1
     inv = capi.rope_inv_freq(hd, theta, dev)
     assert np.array_equal(inv.cpu().numpy(), oracle.rope_inv_freq(hd, theta))
-    kc = torch.zeros(B, n_kv, cap, hd, dtype=torch.float16, device=dev)
-    vc = torch.zeros(B, n_kv, hd, cap, dtype=torch.float16, device=dev)   # V is kept [head_dim][ctx_cap]
+    kc = torch.zeros(B, n_kv, cap, hd, dtype=torch.float16, device=dev)   # both caches are kept in tiles
+    vc = torch.zeros(B, n_kv, cap, hd, dtype=torch.float16, device=dev)
     qd = torch.from_numpy(qkv).to(dev)
     capi.rope_kv_append(qd, inv, torch.from_numpy(pos_h).to(dev), kc, vc, n_heads, n_kv, hd)
     sync()
     got = qd.cpu().numpy()
-    kg = kc.cpu().numpy().view(np.uint16)
-    vg = np.ascontiguousarray(vc.cpu().numpy().view(np.uint16).transpose(0, 1, 3, 2))   # as [cap][hd]
+    kg = capi.kcache_logical(kc).cpu().numpy().view(np.uint16)   # as [cap][hd]
+    vg = capi.vcache_logical(vc).cpu().numpy().view(np.uint16)
     f = oracle.rope_inv_freq(hd, theta)
     for b in range(B):
         ke = np.zeros((n_kv, cap, hd), np.uint16)
@@ -105,20 +105,21 @@ def test_rope_kv_append(capi, dev, oracle, B, n_heads, n_kv):
 
 
 @pytest.mark.parametrize("B,n_heads,n_kv,cap,positions", [
-    (1, 64, 8, 4224, [4095]), (2, 64, 8, 600, [0, 599]), (3, 8, 2, 304, [127, 128, 255]),
-    (2, 4, 4, 136, [5, 129]), (1, 2, 1, 128, [64]), (4, 16, 2, 264, [6, 7, 8, 263]),
-    (2, 3, 3, 40, [30, 39])])
+    (1, 64, 8, 4224, [4095]), (2, 64, 8, 608, [0, 607]), (3, 8, 2, 320, [127, 128, 255]),
+    (2, 4, 4, 160, [5, 129]), (1, 2, 1, 128, [64]), (4, 16, 2, 288, [6, 7, 8, 287]),
+    (2, 3, 3, 64, [30, 63])])
 def test_attention_decode(capi, dev, oracle, B, n_heads, n_kv, cap, positions):
     import torch
 
     hd = 128
     g = torch.Generator(device=dev)
     g.manual_seed(cap + n_heads)
-    kc = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
-    vc = torch.randn(B, n_kv, hd, cap, device=dev, generator=g).half()
+    kl = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()   # position-major values
+    vl = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
     for b, p in enumerate(positions):      # what lies past the newest position must not matter, whatever it is
-        kc[b, :, p + 1:] = float("nan")
-        vc[b, :, :, p + 1:] = float("nan")
+        kl[b, :, p + 1:] = float("nan")
+        vl[b, :, p + 1:] = float("nan")
+    kc, vc = capi.kcache_tiled(kl), capi.vcache_tiled(vl)                # as the device keeps them
     q = torch.randn(B, n_heads * hd + 32, device=dev, generator=g) * 1.5
     pos = torch.tensor(positions, dtype=torch.int32, device=dev)
     out = torch.full((B, n_heads * hd + 4), float("nan"), device=dev)
@@ -130,8 +131,8 @@ def test_attention_decode(capi, dev, oracle, B, n_heads, n_kv, cap, positions):
     assert np.array_equal(q8.cpu().numpy().reshape(B, n_heads * hd // 32, 36),
                           oracle.quantize(np.ascontiguousarray(got[:, :n_heads * hd])))
     assert np.isnan(got[:, n_heads * hd:]).all()
-    kh = kc.cpu().numpy().view(np.uint16)
-    vh = np.ascontiguousarray(vc.cpu().numpy().view(np.uint16).transpose(0, 1, 3, 2))   # the oracle's [cap][hd]
+    kh = kl.cpu().numpy().view(np.uint16)   # the oracle's [cap][hd]
+    vh = vl.cpu().numpy().view(np.uint16)
     qh = q.cpu().numpy()
     for b in range(B):
         exp = oracle.attention_decode(qh[b, :n_heads * hd], kh[b], vh[b], positions[b], n_heads, n_kv, hd)
@@ -145,23 +146,24 @@ def test_attention_follows_the_position_in_memory(capi, dev, oracle):
     B, n_heads, n_kv, hd, cap = 1, 8, 1, 128, 512
     g = torch.Generator(device=dev)
     g.manual_seed(3)
-    kc = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
-    vc = torch.randn(B, n_kv, hd, cap, device=dev, generator=g).half()
+    kl = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
+    vl = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
+    kc, vc = capi.kcache_tiled(kl), capi.vcache_tiled(vl)
     q = torch.randn(B, n_heads * hd, device=dev, generator=g)
     pos = torch.zeros(1, dtype=torch.int32, device=dev)
-    v_rows = np.ascontiguousarray(vc.cpu().numpy().view(np.uint16)[0].transpose(0, 2, 1))
+    v_rows = vl.cpu().numpy().view(np.uint16)[0]
     scratch = capi.attention_scratch(B, n_heads, hd, cap, dev)
     for p in (0, 1, 130, 511):
         pos.fill_(p)
         out = capi.attention(q, kc, vc, pos, n_heads, n_kv, hd, scratch=scratch)
-        exp = oracle.attention_decode(q.cpu().numpy()[0], kc.cpu().numpy().view(np.uint16)[0],
+        exp = oracle.attention_decode(q.cpu().numpy()[0], kl.cpu().numpy().view(np.uint16)[0],
                                       v_rows, p, n_heads, n_kv, hd)
         assert close(out.cpu().numpy()[0], exp, 1e-5), p
 
 
 @pytest.mark.parametrize("B,n_heads,n_kv,cap,positions", [
-    (1, 64, 8, 4224, [4095]), (8, 64, 8, 520, [0, 1, 127, 128, 255, 256, 300, 519]), (3, 8, 2, 304, [7, 8, 303]),
-    (2, 4, 4, 136, [5, 129]), (2, 2, 1, 128, [64, 127]), (2, 3, 3, 40, [0, 39])])
+    (1, 64, 8, 4224, [4095]), (8, 64, 8, 544, [0, 1, 127, 128, 255, 256, 300, 543]), (3, 8, 2, 320, [7, 8, 319]),
+    (2, 4, 4, 160, [5, 129]), (2, 2, 1, 128, [64, 127]), (2, 3, 3, 64, [0, 63])])
 def test_rope_attention_is_append_then_attention(capi, dev, oracle, B, n_heads, n_kv, cap, positions):
     """The fused operator leaves the outputs and the caches that the two separate calls leave."""
     import torch
@@ -169,11 +171,12 @@ def test_rope_attention_is_append_then_attention(capi, dev, oracle, B, n_heads, 
     hd = 128
     g = torch.Generator(device=dev)
     g.manual_seed(cap + n_heads + 1)
-    kc = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
-    vc = torch.randn(B, n_kv, hd, cap, device=dev, generator=g).half()
+    kl = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
+    vl = torch.randn(B, n_kv, cap, hd, device=dev, generator=g).half()
     for b, p in enumerate(positions):      # the slot of the new token and everything after it: anything at all
-        kc[b, :, p:] = float("nan")
-        vc[b, :, :, p:] = float("nan")
+        kl[b, :, p:] = float("nan")
+        vl[b, :, p:] = float("nan")
+    kc, vc = capi.kcache_tiled(kl), capi.vcache_tiled(vl)
     width = (n_heads + 2 * n_kv) * hd
     qkv = torch.randn(B, width + 8, device=dev, generator=g) * 1.5
     pos = torch.tensor(positions, dtype=torch.int32, device=dev)
@@ -205,8 +208,8 @@ def test_rope_attention_is_append_then_attention(capi, dev, oracle, B, n_heads, 
     # K value on an fp16 tie may round the other way on the host; test_rope_kv_append bounds that)
     f = oracle.rope_inv_freq(hd, 1e6)
     qh = qkv.cpu().numpy()
-    kh = kc2.cpu().numpy().view(np.uint16)
-    vh = np.ascontiguousarray(vc2.cpu().numpy().view(np.uint16).transpose(0, 1, 3, 2))
+    kh = capi.kcache_logical(kc2).cpu().numpy().view(np.uint16)
+    vh = capi.vcache_logical(vc2).cpu().numpy().view(np.uint16)
     got = out2.cpu().numpy()
     for b in range(B):
         rot = oracle.rope_kv_append(qh[b, :width], f, positions[b], kh[b].copy(), vh[b].copy(), n_heads, n_kv, hd)
@@ -217,12 +220,12 @@ def test_rope_attention_is_append_then_attention(capi, dev, oracle, B, n_heads, 
 def test_attention_refuses_a_cache_it_cannot_read(capi, dev):
     import torch
 
-    hd, cap = 128, 132   # not a multiple of 8: a 16-byte group of V positions would straddle two dimensions
+    hd, cap = 128, 136   # not a multiple of 32: the caches are kept in tiles of 16 and 32 positions
     kc = torch.zeros(1, 1, cap, hd, dtype=torch.float16, device=dev)
-    vc = torch.zeros(1, 1, hd, cap, dtype=torch.float16, device=dev)
+    vc = torch.zeros(1, 1, cap, hd, dtype=torch.float16, device=dev)
     q = torch.zeros(1, hd, device=dev)
     pos = torch.zeros(1, dtype=torch.int32, device=dev)
-    with pytest.raises(RuntimeError, match="multiple of 8"):
+    with pytest.raises(RuntimeError, match="multiple of 32"):
         capi.attention(q, kc, vc, pos, 1, 1, hd)
 
 

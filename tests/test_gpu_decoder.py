@@ -71,9 +71,9 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
         kc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
         vc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
     for l in range(shape.n_layers):
-        dec.buffer("kcache", l).copy_(torch.from_numpy(kc_h[:, l]).to(dev))
-        # the device keeps V dimension-major: [batch][n_kv][head_dim][cap]
-        dec.buffer("vcache", l).copy_(torch.from_numpy(np.ascontiguousarray(vc_h[:, l].transpose(0, 1, 3, 2))).to(dev))
+        # the device keeps both caches in tiles
+        dec.buffer("kcache", l).copy_(capi.kcache_tiled(torch.from_numpy(kc_h[:, l])).to(dev))
+        dec.buffer("vcache", l).copy_(capi.vcache_tiled(torch.from_numpy(vc_h[:, l])).to(dev))
     dec.set_state(ids, pos)
     kc_u, vc_u = kc_h.view(np.uint16).copy(), vc_h.view(np.uint16).copy()
 
@@ -95,10 +95,10 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
                 assert new_ids[b] == int(np.argmax(exp)), (step, b)
             # the appended K/V rows: fp16 of nearly equal fp32 values
             for l in range(shape.n_layers):
-                kg = dec.buffer("kcache", l)[b, :, int(pos[b]) + step].cpu().numpy().astype(np.float32)
+                kg = capi.kcache_logical(dec.buffer("kcache", l))[b, :, int(pos[b]) + step].cpu().numpy().astype(np.float32)
                 ke = kc_u[b, l, :, int(pos[b]) + step].view(np.float16).astype(np.float32)
                 assert np.abs(kg - ke).max() <= 2e-2 * max(np.abs(ke).max(), 1.0), (step, b, l)
-                vg = dec.buffer("vcache", l)[b, :, :, int(pos[b]) + step].cpu().numpy().astype(np.float32)
+                vg = capi.vcache_logical(dec.buffer("vcache", l))[b, :, int(pos[b]) + step].cpu().numpy().astype(np.float32)
                 ve = vc_u[b, l, :, int(pos[b]) + step].view(np.float16).astype(np.float32)
                 assert np.abs(vg - ve).max() <= 2e-2 * max(np.abs(ve).max(), 1.0), (step, b, l)
         ids = new_ids.copy()   # both sides continue from the device's tokens
@@ -126,8 +126,8 @@ def test_batch_eight_against_numpy_walk(capi, dev, oracle):
         kc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
         vc_h[b, :, :, :pos[b]] = rng.standard_normal((shape.n_layers, shape.n_kv, pos[b], 128)).astype(np.float16)
     for l in range(shape.n_layers):
-        dec.buffer("kcache", l).copy_(torch.from_numpy(kc_h[:, l]).to(dev))
-        dec.buffer("vcache", l).copy_(torch.from_numpy(np.ascontiguousarray(vc_h[:, l].transpose(0, 1, 3, 2))).to(dev))
+        dec.buffer("kcache", l).copy_(capi.kcache_tiled(torch.from_numpy(kc_h[:, l])).to(dev))
+        dec.buffer("vcache", l).copy_(capi.vcache_tiled(torch.from_numpy(vc_h[:, l])).to(dev))
     dec.set_state(ids, pos)
     kc_u, vc_u = kc_h.view(np.uint16).copy(), vc_h.view(np.uint16).copy()
     dec.step()
@@ -144,7 +144,7 @@ def test_batch_eight_against_numpy_walk(capi, dev, oracle):
         if top2[1] - top2[0] > 2 * 5e-3 * scale:
             assert new_ids[b] == int(np.argmax(exp)), b
         for l in range(shape.n_layers):
-            kg = dec.buffer("kcache", l)[b, :, int(pos[b])].cpu().numpy().astype(np.float32)
+            kg = capi.kcache_logical(dec.buffer("kcache", l))[b, :, int(pos[b])].cpu().numpy().astype(np.float32)
             ke = kc_u[b, l, :, int(pos[b])].view(np.float16).astype(np.float32)
             assert np.abs(kg - ke).max() <= 2e-2 * max(np.abs(ke).max(), 1.0), (b, l)
     dec.close()
@@ -157,7 +157,7 @@ def test_a_full_context_is_reported(capi, dev):
     from llaminar_amd.decoder import DenseDecoder, Shape
 
     shape = Shape(hidden=1024, n_heads=8, n_kv=2, head_dim=128, ffn=1024, vocab=512, n_layers=1)
-    cap = 16
+    cap = 32
     dec = DenseDecoder(shape, 2, cap, dev, seed=3)
     dec.set_state([5, 6], [cap - 3, cap - 1])          # the furthest sequence sits on the last position
     assert dec.steps_left() == 1
@@ -234,16 +234,16 @@ def test_bad_configurations_are_refused(capi, dev):
     from llaminar_amd import decoder
 
     L = decoder.load()
-    bad = decoder.Config(5000, 64, 8, 128, 25600, 1000, 1, 16, 1, 1e6, 1e-6, 0)  # hidden not a multiple of 256
+    bad = decoder.Config(5000, 64, 8, 128, 25600, 1000, 1, 32, 1, 1e6, 1e-6, 0)  # hidden not a multiple of 256
     assert not L.llam_decoder_create(bad)
     assert b"multiples of 256" in L.llam_decoder_last_error()
-    bad = decoder.Config(512, 6, 4, 128, 512, 1000, 1, 16, 1, 1e6, 1e-6, 0)       # 6 heads on 4 KV heads
+    bad = decoder.Config(512, 6, 4, 128, 512, 1000, 1, 32, 1, 1e6, 1e-6, 0)       # 6 heads on 4 KV heads
     assert not L.llam_decoder_create(bad)
-    ok = decoder.Config(512, 4, 4, 128, 512, 1000, 1, 16, 9, 1e6, 1e-6, 0)        # batch 9
+    ok = decoder.Config(512, 4, 4, 128, 512, 1000, 1, 32, 9, 1e6, 1e-6, 0)        # batch 9
     assert not L.llam_decoder_create(ok)
-    assert not L.llam_decoder_create(decoder.Config(512, 4, 4, 128, 512, 1000, 1, 12, 1, 1e6, 1e-6, 0))
-    assert b"multiple of 8" in L.llam_decoder_last_error()                        # 12 cache positions
-    h = L.llam_decoder_create(decoder.Config(512, 4, 4, 128, 512, 1000, 1, 16, 1, 1e6, 1e-6, 0))
+    assert not L.llam_decoder_create(decoder.Config(512, 4, 4, 128, 512, 1000, 1, 24, 1, 1e6, 1e-6, 0))
+    assert b"multiple of 32" in L.llam_decoder_last_error()                       # 24 cache positions
+    h = L.llam_decoder_create(decoder.Config(512, 4, 4, 128, 512, 1000, 1, 32, 1, 1e6, 1e-6, 0))
     assert h
     assert not L.llam_decoder_step(h, None) and b"globals not set" in L.llam_decoder_last_error()
     L.llam_decoder_destroy(h)
