@@ -116,3 +116,26 @@ def test_synthetic_generators_are_seeded_and_in_range():
         d = a[:, :, off:off + 2].copy().view(np.float16).astype(np.float32)
         assert d.min() >= 0.000999 and d.max() <= 0.02
     assert synth.gemv_bytes(capi.FMT_Q4_K, 25600, 5120) == 25600 * 20 * 144 + 160 * 36 + 25600 * 4
+
+
+def test_cache_tiles_follow_the_documented_offsets():
+    """capi.kcache_tiled / vcache_tiled (the host-side views of the KV caches) against the element offsets
+    include/llaminar_amd/decode_api.h gives for llam_dec_rope_kv_append, and their inverses."""
+    import torch
+
+    from llaminar_amd import capi
+
+    cap, hd = 96, 128
+    x = torch.arange(2 * 3 * cap * hd, dtype=torch.float32).reshape(2, 3, cap, hd)
+    kt, vt = capi.kcache_tiled(x), capi.vcache_tiled(x)
+    assert kt.shape == x.shape and vt.shape == x.shape
+    assert torch.equal(capi.kcache_logical(kt), x) and torch.equal(capi.vcache_logical(vt), x)
+    kf, vf = kt.reshape(2, 3, -1), vt.reshape(2, 3, -1)
+    rng = np.random.default_rng(0)
+    for _ in range(3000):
+        p, d = int(rng.integers(cap)), int(rng.integers(hd))
+        k_off = (p // 16) * 16 * hd + (d // 8) * 128 + (p % 16) * 8 + d % 8
+        v_off = (p // 32) * 32 * hd + (d // 16) * 512 + ((p // 8) % 4) * 128 + (d % 16) * 8 + p % 8
+        assert kf[1, 2, k_off] == x[1, 2, p, d] and vf[0, 1, v_off] == x[0, 1, p, d]
+    with pytest.raises(AssertionError):
+        capi.kcache_tiled(torch.zeros(1, 1, 40, 128))   # capacities are multiples of 32
