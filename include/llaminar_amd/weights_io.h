@@ -58,7 +58,7 @@ const char *llam_gguf_meta_str(const void *gguf, const char *key);
 /* ---- prepared-weights container --------------------------------------------------- */
 
 #define LLAM_PREPARED_MAGIC 0x5750514Cu /* "LQPW" */
-#define LLAM_PREPARED_VERSION 1u
+#define LLAM_PREPARED_VERSION 2u
 
 typedef struct
 {

@@ -163,6 +163,7 @@ namespace llamql
         {
             // ---- compute wavefronts --------------------------------------------------------------
             const int l32 = lane & 31, lh = lane >> 5;
+            const uint32_t lh_second = lh ? Q6K_CODE_BIG1 : 0u; // the record bit that says this lane's sub-scale is the larger one
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
             const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
             const int last_step = nsteps > 0 ? nsteps - 1 : 0;
@@ -266,9 +267,8 @@ namespace llamql
                 // bits 2s, 2s+1 of qh piece n; sub-scales 8n + 2s and 8n + 2s + 1
                 auto product = [&](int j, float &bscale) {
                     const int n = j >> 2, s = j & 3;
-                    int f0, f1;
-                    q6k_block_decode(rec[q6k_code_pos(j)], f0, f1, bscale);
-                    const int f = lh ? f1 : f0; // this lane's 16 elements share one sub-scale
+                    int f; // this lane's 16 elements share one sub-scale
+                    q6k_block_factor(rec[q6k_code_pos(j)], lh_second, f, bscale);
                     const unsigned short fu = (unsigned short)f, ku = (unsigned short)(128 - 32 * f);
                     const Q6KQuad::v2s ff = {fu, fu}, cc = {ku, ku};
                     const v4i lo = ql[2 * n + (s & 1)], hi = qh[n];

@@ -52,10 +52,12 @@ namespace llamql
     // sub-scale's factor is +-1016; the record keeps the other one:
     //   bits  0..11  f of the smaller sub-scale (two's complement)
     //   bit   12     the larger sub-scale is the second one (ties: the first)
-    //   bit   13     the larger sub-scale is negative
-    //   bit   14     both sub-scales are zero (weights and scale are zero)
+    //   bits 13..14  the sign of the larger sub-scale as a two-bit two's complement number: +1, -1, or
+    //                0 when both sub-scales are zero (weights and scale are zero) -- times 1016 it is
+    //                the larger one's factor
     //   bits 16..31  the block scale as fp16 bits
-    constexpr uint32_t Q6K_CODE_BIG1 = 1u << 12, Q6K_CODE_NEG = 1u << 13, Q6K_CODE_ZERO = 1u << 14;
+    constexpr uint32_t Q6K_CODE_BIG1 = 1u << 12, Q6K_CODE_SIGN_SHIFT = 13;
+    constexpr uint32_t Q6K_CODE_POS = 1u << Q6K_CODE_SIGN_SHIFT, Q6K_CODE_NEG = 3u << Q6K_CODE_SIGN_SHIFT;
 
     __device__ __forceinline__ uint32_t q6k_block_code(int s0, int s1, float d)
     {
@@ -63,7 +65,7 @@ namespace llamql
         const bool big0 = a0 >= a1;
         const int msc = big0 ? a0 : a1;
         if (msc == 0)
-            return Q6K_CODE_ZERO;
+            return 0u;
         const int s_small = big0 ? s1 : s0, s_big = big0 ? s0 : s1;
         const float fm = (float)msc;
         // rne(s_small * 1016 / msc) without a division: the quotient has a denominator of at most
@@ -75,17 +77,26 @@ namespace llamql
         const float q0 = num * r;
         const int f_small = (int)rintf(fmaf(fmaf(-fm, q0, num), r, q0));
         const float bscale = f16_round_packer(div_by_127(d * fm * 32.0f));
-        return ((uint32_t)f_small & 0xFFFu) | (big0 ? 0u : Q6K_CODE_BIG1) | (s_big < 0 ? Q6K_CODE_NEG : 0u) |
+        return ((uint32_t)f_small & 0xFFFu) | (big0 ? 0u : Q6K_CODE_BIG1) | (s_big < 0 ? Q6K_CODE_NEG : Q6K_CODE_POS) |
                ((uint32_t)__half_as_ushort(__float2half_rn(bscale)) << 16); // bscale is an fp16 value: exact
     }
     // the two 8.8 factors and the block scale of a record
     __device__ __forceinline__ void q6k_block_decode(uint32_t c, int &f0, int &f1, float &bscale)
     {
         const int fs = __builtin_amdgcn_sbfe((int)c, 0u, 12u);
-        const int fb = (c & Q6K_CODE_ZERO) ? 0 : ((c & Q6K_CODE_NEG) ? -1016 : 1016);
+        const int fb = __builtin_amdgcn_sbfe((int)c, Q6K_CODE_SIGN_SHIFT, 2u) * 1016;
         const bool big1 = (c & Q6K_CODE_BIG1) != 0;
         f0 = big1 ? fs : fb;
         f1 = big1 ? fb : fs;
+        bscale = h2f((uint16_t)(c >> 16));
+    }
+    // the factor of one of the two sub-scales (second: 0 or Q6K_CODE_BIG1, the lane's constant) and the
+    // block scale: what a lane needs that requantises 16 elements of a block
+    __device__ __forceinline__ void q6k_block_factor(uint32_t c, uint32_t second, int &f, float &bscale)
+    {
+        const int fs = __builtin_amdgcn_sbfe((int)c, 0u, 12u);
+        const int fb = __builtin_amdgcn_sbfe((int)c, Q6K_CODE_SIGN_SHIFT, 2u) * 1016;
+        f = (c & Q6K_CODE_BIG1) == second ? fb : fs;
         bscale = h2f((uint16_t)(c >> 16));
     }
     // where the record of block j sits among the eight of its super-block: the two blocks a

@@ -277,14 +277,14 @@ def test_prepare_moves_every_byte(capi, dev, oracle, fmt):
                 msc = max(abs(s0), abs(s1))
                 assert (c >> 16) == int(sc_h[j]), (t, j)
                 if msc == 0:
-                    assert (c & 0xFFFF) == 1 << 14
+                    assert (c & 0xFFFF) == 0
                     continue
                 big1 = abs(s1) > abs(s0)
                 small, big = (s0, s1) if big1 else (s1, s0)
                 fs = c & 0xFFF
                 fs -= 4096 if fs & 0x800 else 0
                 assert fs == rne_div(small * 1016, msc) and bool(c & (1 << 12)) == big1
-                assert bool(c & (1 << 13)) == (big < 0) and not c & (1 << 14)
+                assert (c >> 13) & 3 == (3 if big < 0 else 1)   # the larger sub-scale's sign: -1 or +1 in two bits
     else:
         assert np.array_equal(P[:T * 64].reshape(T, 64), B[:, 2:66])
         assert np.array_equal(P[T * 64:T * 96].reshape(T, 32), B[:, 74:106])

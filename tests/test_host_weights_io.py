@@ -168,7 +168,7 @@ def test_checksum_and_container_header(wio, capi):
         nbytes = capi_cpu.llam_ql_prepared_bytes(fmt, N, K)
         payload = rng.integers(0, 256, nbytes, dtype=np.uint8)
         hdr = wio.header_build(fmt, N, K, payload)
-        assert (hdr.magic, hdr.version, hdr.fmt, hdr.N, hdr.K) == (0x5750514C, 1, fmt, N, K)
+        assert (hdr.magic, hdr.version, hdr.fmt, hdr.N, hdr.K) == (0x5750514C, 2, fmt, N, K)
         assert (hdr.block_bytes, hdr.prepared_bytes, hdr.gguf_bytes) == (block, nbytes, N * 2 * block)
         assert hdr.checksum == wio.checksum(payload)
         blob = np.concatenate([np.frombuffer(bytes(hdr), np.uint8), payload])
