@@ -236,7 +236,7 @@ def bench_decode(args, torch, capi, synth, dev):
     ctx = args.context
     cap = (ctx + args.steps + args.warmup + 8 + 31) // 32 * 32   # the caches are kept in tiles of 16 and 32 positions
     t_build = time.perf_counter()
-    dec = DenseDecoder(shape, B, cap, dev, seed=11, keep_prepared=True)
+    dec = DenseDecoder(shape, B, cap, dev, seed=11, keep_prepared=True, batch_planes=False if args.no_batch_planes else None)
     g = torch.Generator(device=dev)
     g.manual_seed(3)
     for l in range(shape.n_layers):   # a cache as `ctx - 1` earlier tokens would have left it
@@ -320,7 +320,7 @@ def bench_decode(args, torch, capi, synth, dev):
     cfg = {"workload": "end-to-end greedy decode step, random-init %d-layer dense model (hidden 5120, 64x128 heads, "
                        "8 KV heads, ffn 25600; Q4_K projections, Q6_K V/down/lm_head 5120->152064, Q4_K embedding), "
                        "RMSNorm, RoPE theta 1e6, fp16 KV cache at context %d, batch %d" % (shape.n_layers, ctx, B),
-           "batch": B, "context": ctx, "layers": shape.n_layers,
+           "batch": B, "context": ctx, "layers": shape.n_layers, "batch_planes": bool(dec.planed),
            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kv_bytes,
            "linear_only_ms": round(ms_lin, 4), "gemv_share_of_step": round(ms_lin / ms, 4),
            "hbm_bound_tokens_per_s": round(B * HBM_PEAK_GBS * 1e9 / (wbytes + kv_bytes), 1),
@@ -399,6 +399,8 @@ def parse():
     ap.add_argument("--decode-layers", type=int, default=64, help="decode workload: layers of the model")
     ap.add_argument("--separate-quantise", action="store_true",
                     help="layer workload: quantiser kernels of their own instead of the fp32-input GEMV calls")
+    ap.add_argument("--no-batch-planes", action="store_true",
+                    help="batches of 5..8: decode the Q6_K down projection (and lm_head) per launch instead of reading int8 batch planes")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true",
                     help="layer workload at batch 1: skip the short run of the 64-layer decode step")
@@ -437,12 +439,16 @@ def main():
              ("o", HIDDEN, QDIM, FMT_Q4_K), ("gate", FFN, HIDDEN, FMT_Q4_K), ("up", FFN, HIDDEN, FMT_Q4_K),
              ("down", HIDDEN, FFN, FMT_Q6_K)]
     layers = []
+    planes = []   # kept alive with the weights
     for l in range(args.layers):
         w = {}
         for i, (name, N, K, fmt) in enumerate(projs):
             raw = synth.weights_torch(fmt, N, K, 1000 * l + i, dev)
             w[name] = capi.prepare_weights(fmt, raw, N, K)
             del raw
+            # batches of 5..8 rows: the down projection reads its weights from an int8 batch plane
+            if M >= 5 and name == "down" and not args.no_batch_planes:
+                planes.append(capi.attach_batch_plane(fmt, w[name], N, K))
         layers.append(w)
     torch.cuda.synchronize()
 
@@ -597,6 +603,7 @@ def main():
             "bytes_per_step": bytes_per_step,
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
             "distinct_weight_sets": args.layers,
+            "batch_planes": bool(planes),   # the Q6_K down projection read from its int8 batch plane (batches of 5..8)
             "launch": "eager" if graphs is None else "hip-graph replay",
         },
         "roofline": {

@@ -49,6 +49,9 @@ SIGNATURES = {
     "llam_ql_set_gemv_tuning": (None, [c_int, c_int]),
     "llam_ql_reset_gemv_tuning": (None, []),
     "llam_ql_set_batch_tile_rows": (None, [c_int]),
+    "llam_ql_batch_plane_bytes": (c_size_t, [c_uint8, c_int, c_int]),
+    "llam_ql_build_batch_plane": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_attach_batch_plane": (c_bool, [c_void_p, c_void_p, c_int, c_int]),
     "llam_ql_read_probe": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_quantize_q8_1": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_prepared_bytes": (c_size_t, [c_uint8, c_int, c_int]),
@@ -207,6 +210,30 @@ def prepare_weights(fmt: int, gguf, N: int, K: int, stream=None):
     _check(load().llam_ql_prepare_weights(fmt, _ptr(gguf), _ptr(out), N, K, _dev(gguf), _stream(stream)),
            "prepare_weights")
     return out
+
+
+def batch_plane_bytes(fmt: int, N: int, K: int) -> int:
+    """Size of the optional int8 batch plane of a prepared matrix; 0 where the shape has none."""
+    return int(load().llam_ql_batch_plane_bytes(fmt, N, K))
+
+
+def attach_batch_plane(fmt: int, w, N: int, K: int, stream=None):
+    """Builds the batch plane of the prepared matrix `w` and attaches it: batches of 5..8 rows then read the
+    ready-made int8 weights.  Returns the plane (keep it alive as long as `w` is used, then detach_batch_plane),
+    or None where the format or shape has no plane."""
+    import torch
+
+    nbytes = batch_plane_bytes(fmt, N, K)
+    if nbytes == 0:
+        return None
+    plane = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    _check(load().llam_ql_build_batch_plane(fmt, _ptr(w), _ptr(plane), N, K, _dev(w), _stream(stream)), "build_batch_plane")
+    _check(load().llam_ql_attach_batch_plane(_ptr(w), _ptr(plane), N, K), "attach_batch_plane")
+    return plane
+
+
+def detach_batch_plane(w):
+    _check(load().llam_ql_attach_batch_plane(_ptr(w), None, 0, 0), "attach_batch_plane")
 
 
 def gemv(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None):

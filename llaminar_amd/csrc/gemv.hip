@@ -77,7 +77,7 @@ namespace llamql
         {
             // batches that go to the matrix-unit kernel launch one matrix at a time
             if constexpr (F::USE_MFMA_BATCH)
-                if (mfma_eligible<F>(M, projs[0].N, K))
+                if (mfma_eligible<F>(M, projs[0].N, K) || batch_plane_for<F>(projs[0].d_w, M, projs[0].N, K))
                     return gemv_mfma_launch<F>(fn, projs[0].d_w, src, projs[0].d_y, M, projs[0].N, K, projs[0].ldy,
                                                 device_id, st)
                                ? 1
@@ -85,7 +85,8 @@ namespace llamql
             QuadProj pr[QUAD_MAX_PROJ];
             int n = 0;
             while (n < num && n < QUAD_MAX_PROJ && projs[n].fmt == projs[0].fmt &&
-                   quad_eligible<F>(M, projs[n].N, K) && !mfma_eligible<F>(M, projs[n].N, K))
+                   quad_eligible<F>(M, projs[n].N, K) && !mfma_eligible<F>(M, projs[n].N, K) &&
+                   !batch_plane_for<F>(projs[n].d_w, M, projs[n].N, K))
             {
                 pr[n] = QuadProj{projs[n].d_w, projs[n].d_y, projs[n].N, projs[n].ldy};
                 ++n;
@@ -97,7 +98,8 @@ namespace llamql
                     typedef typename Other<F>::type G;
                     int nb = 0;
                     while (n + nb < num && n + nb < QUAD_MAX_PROJ && projs[n + nb].fmt == Other<F>::fmt &&
-                           quad_eligible<G>(M, projs[n + nb].N, K) && !mfma_eligible<G>(M, projs[n + nb].N, K))
+                           quad_eligible<G>(M, projs[n + nb].N, K) && !mfma_eligible<G>(M, projs[n + nb].N, K) &&
+                           !batch_plane_for<G>(projs[n + nb].d_w, M, projs[n + nb].N, K))
                     {
                         pr[n + nb] = QuadProj{projs[n + nb].d_w, projs[n + nb].d_y, projs[n + nb].N, projs[n + nb].ldy};
                         ++nb;
@@ -136,7 +138,8 @@ namespace llamql
                                int ldy, int device_id, hipStream_t st, bool query)
         {
             const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
-            if (p.kernel != GEMV_KERNEL_QUAD || p.m_first < M)
+            // (a batch that has the matrix's batch plane to read goes to the matrix-unit kernel)
+            if (p.kernel != GEMV_KERNEL_QUAD || p.m_first < M || batch_plane_for<F>(d_w, M, N, K))
                 return query ? false : fail(fn, "M=%d N=%d K=%d: not a single quad-lane launch", M, N, K);
             const QuadProj pr{d_w, d_y, N, ldy};
             return gemv_quad_multi<F>(fn, &pr, 1, act_source_q8(d_q8), M, K, device_id, st, nullptr, 0, 0,
@@ -174,3 +177,103 @@ namespace llamql
         }
     }
 } // namespace llamql
+
+// ---- the Q6_K batch plane ---------------------------------------------------------------------
+namespace llamql
+{
+    // Thread (row, super-block, block j, half h) writes the 16 requantised elements 16h..16h+15 of
+    // block j of the row -- what lane (row, h) of gemv_mfma_q6k_kernel hands the matrix unit --
+    // and, for h = 0, the block's scale.  Rows past N (the last group's padding) are zeros.
+    __global__ void __launch_bounds__(256) build_q6k_plane_kernel(const uint8_t *prepared, uint8_t *plane, long N, int nsb)
+    {
+        const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        const size_t rows = q6k_plane_groups(N) * 4;
+        if (idx >= rows * (size_t)nsb * 16)
+            return;
+        const int h = (int)(idx & 1), j = (int)((idx >> 1) & 7);
+        const size_t rs = idx >> 4; // row * nsb + sb
+        const size_t row = rs / (size_t)nsb;
+        const int sb = (int)(rs - row * (size_t)nsb);
+        const size_t cell = (row >> 2) * (size_t)nsb + (size_t)sb; // the group's super-block
+        v4i *dst = reinterpret_cast<v4i *>(plane + (cell * 8 + (size_t)j) * 128 + (row & 3) * 32 + 16 * h);
+        uint16_t *dsc = reinterpret_cast<uint16_t *>(plane + q6k_plane_scales_offset(N, nsb) + cell * 64 + (row & 3) * 16) + j;
+        if ((long)row >= N)
+        {
+            *dst = (v4i){0, 0, 0, 0};
+            if (h == 0)
+                *dsc = 0;
+            return;
+        }
+        const size_t T = (size_t)N * (size_t)nsb, t = row * (size_t)nsb + (size_t)sb;
+        const int n = j >> 2, s = j & 3;
+        const v4i lo = *reinterpret_cast<const v4i *>(prepared + t * 128 + 64 * n + 32 * (s & 1) + 16 * h);
+        const v4i hi = *reinterpret_cast<const v4i *>(prepared + T * 128 + t * 64 + 32 * n + 16 * h);
+        const uint32_t rec = *reinterpret_cast<const uint32_t *>(prepared + q6k_factors_offset(T) + t * 32 + 4 * q6k_code_pos(j));
+        int f;
+        float bscale;
+        q6k_block_factor(rec, h ? Q6K_CODE_BIG1 : 0u, f, bscale);
+        const unsigned short fu = (unsigned short)f, ku = (unsigned short)(128 - 32 * f);
+        const Q6KQuad::v2s ff = {fu, fu}, cc = {ku, ku};
+        const uint32_t k4 = 0x0F0F0F0Fu, k2 = 0x03030303u;
+        auto q4 = [&](int l, int hq) {
+            const uint32_t nib = (s >= 2 ? (uint32_t)l >> 4 : (uint32_t)l) & k4;
+            const uint32_t q = nib | ((((uint32_t)hq >> (2 * s)) & k2) << 4);
+            return Q6KQuad::requant4(q, ff, cc);
+        };
+        *dst = (v4i){q4(lo.x, hi.x), q4(lo.y, hi.y), q4(lo.z, hi.z), q4(lo.w, hi.w)};
+        if (h == 0)
+            *dsc = (uint16_t)(rec >> 16);
+    }
+
+    // A plane exists for Q6_K rows of eight super-blocks and more, as the matrix-unit kernels ask.
+    static bool batch_plane_shape(uint8_t fmt, int N, int K)
+    {
+        return fmt == LLAM_FMT_Q6_K && N >= 1 && K >= 2048 && K % 256 == 0 &&
+               q6k_plane_bytes(N, K / 256) < ((size_t)1 << 32); // the kernel's lane offsets are 32-bit
+    }
+} // namespace llamql
+
+extern "C" size_t llam_ql_batch_plane_bytes(uint8_t fmt, int N, int K)
+{
+    return llamql::batch_plane_shape(fmt, N, K) ? llamql::q6k_plane_bytes(N, K / 256) : 0;
+}
+
+extern "C" bool llam_ql_build_batch_plane(uint8_t fmt, const void *d_prepared, void *d_plane, int N, int K,
+                                          int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_build_batch_plane";
+    if (!batch_plane_shape(fmt, N, K))
+        return fail(fn, "no batch plane for format %d, N=%d, K=%d (llam_ql_batch_plane_bytes is 0)", (int)fmt, N, K);
+    if (!d_prepared || !d_plane)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_prepared) || !aligned16(d_plane))
+        return fail(fn, "d_prepared and d_plane must be 16-byte aligned");
+    if (!set_device(fn, device_id))
+        return false;
+    const int nsb = K / 256;
+    const size_t items = q6k_plane_groups(N) * 4 * (size_t)nsb * 16;
+    const size_t grid = (items + 255) / 256;
+    if (grid > 0x7FFFFFFFull)
+        return fail(fn, "matrix too large (N=%d K=%d)", N, K);
+    hipLaunchKernelGGL(build_q6k_plane_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint8_t *>(d_prepared), static_cast<uint8_t *>(d_plane), (long)N, nsb);
+    return launched(fn);
+}
+
+extern "C" bool llam_ql_attach_batch_plane(const void *d_prepared, const void *d_plane, int N, int K)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_attach_batch_plane";
+    if (!d_prepared)
+        return fail(fn, "null d_prepared");
+    if (d_plane)
+    {
+        if (!batch_plane_shape(LLAM_FMT_Q6_K, N, K))
+            return fail(fn, "no batch plane for N=%d, K=%d", N, K);
+        if (!aligned16(d_plane))
+            return fail(fn, "d_plane must be 16-byte aligned");
+    }
+    batch_plane_attach(d_prepared, d_plane, N, K);
+    return true;
+}

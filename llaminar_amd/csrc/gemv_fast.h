@@ -512,15 +512,27 @@ namespace llamql
         hipLaunchKernelGGL((gemv_mfma_q6k_kernel<SRC, DUMP>), grid, block, lds, st, a);
     }
 
+    template <int SRC>
+    void gemv_mfma_q6k_plane_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const Mfma6Args &a)
+    {
+        static LdsGrant grant;
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q6k_plane_kernel<SRC>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_mfma_q6k_plane_kernel<SRC>), grid, block, lds, st, a);
+    }
+
     inline bool gemv_mfma_q6k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
                                      int K, int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr,
                                      int row0 = 0, int nrows = 0)
     {
         const int SB = K / 256;
+        // the matrix's batch plane if one is attached (the block-sum variant decodes the weights itself)
+        const uint8_t *plane = d_sums ? nullptr : batch_plane_of(d_w, N, K);
         const Mfma6Shape sh =
-            gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA6_DUMP_COMPUTE : MFMA6_MAX_COMPUTE);
+            gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA6_DUMP_COMPUTE : plane ? MFMA6_PLANE_COMPUTE : MFMA6_MAX_COMPUTE,
+                             plane != nullptr);
         Mfma6Args a;
         a.w = static_cast<const uint8_t *>(d_w);
+        a.plane = plane;
         a.q8 = static_cast<const uint32_t *>(src.q8);
         a.x = src.x;
         a.x2 = src.x2;
@@ -537,13 +549,23 @@ namespace llamql
         a.sums = d_sums;
         a.row0 = row0;
         a.nrows = nrows;
-        const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles + MFMA6_PRODUCERS) * WAVE);
-        const size_t lds = mfma6_lds_bytes(SB, sh.chunk, sh.slices * sh.tiles);
+        const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles + (plane ? MFMA6_PLANE_PRODUCERS : MFMA6_PRODUCERS)) * WAVE);
+        const size_t lds = plane ? mfma6_act_bytes(SB, sh.chunk) : mfma6_lds_bytes(SB, sh.chunk, sh.slices * sh.tiles);
         if (d_sums)
         {
             if (src.kind != ACT_SRC_Q8)
                 return fail(fn, "block sums are dumped on Q8_1 input");
             gemv_mfma_q6k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            return launched(fn);
+        }
+        if (plane)
+        {
+            switch (src.kind)
+            {
+            case ACT_SRC_F32: gemv_mfma_q6k_plane_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;
+            case ACT_SRC_SWIGLU: gemv_mfma_q6k_plane_launch_src<QUAD_SRC_SWIGLU>(grid, block, lds, st, a); break;
+            default: gemv_mfma_q6k_plane_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a); break;
+            }
             return launched(fn);
         }
         switch (src.kind)
@@ -555,7 +577,18 @@ namespace llamql
         return launched(fn);
     }
 
-    // The matrix-unit kernel of format F (mfma_eligible<F> has said yes).
+    // The batch plane attached to a Q6_K matrix, for a batch the plane kernel takes (5..8 rows,
+    // no tuning override in force), else null.
+    template <class F>
+    const uint8_t *batch_plane_for(const void *d_w, int M, int N, int K)
+    {
+        if constexpr (F::USE_MFMA_BATCH && std::is_same<typename F::Quad, Q6KQuad>::value)
+            if (M >= 5 && M <= 8 && gemv_unroll_override() == 0 && gemv_rows_per_wave_override() == 0)
+                return batch_plane_of(d_w, N, K);
+        return nullptr;
+    }
+
+    // The matrix-unit kernel of format F (mfma_eligible<F> or batch_plane_for<F> has said yes).
     template <class F>
     bool gemv_mfma_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N, int K,
                           int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr, int row0 = 0,
@@ -865,6 +898,9 @@ namespace llamql
     {
         const int SB = K / 256;
         const bool dump = d_sums != nullptr;
+        if constexpr (F::USE_MFMA_BATCH)
+            if (!dump && batch_plane_for<F>(d_w, M, N, K))
+                return gemv_mfma_launch<F>(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st);
         const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
         if (p.kernel < 0)
             return fail(fn, "K=%d is too long for %d activation row(s) in LDS", K, p.m_first);

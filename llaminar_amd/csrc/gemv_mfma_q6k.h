@@ -42,6 +42,7 @@ namespace llamql
     struct Mfma6Args
     {
         const uint8_t *w;   // prepared Q6_K planes: ql | qh | scales | d over all N*SB super-blocks
+        const uint8_t *plane; // PLANE kernels: the matrix's batch plane (q6k_plane_bytes), w is not read
         const uint32_t *q8; // Q8_1 activations as dwords (QUAD_SRC_Q8)
         const float *x;     // fp32 rows (QUAD_SRC_F32); the gate rows for QUAD_SRC_SWIGLU
         const float *x2;    // the up rows for QUAD_SRC_SWIGLU
@@ -85,6 +86,42 @@ namespace llamql
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qh1) : "v"(o.qh[1]), "s"(p.qh));
         asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.fc0) : "v"(o.fc), "s"(p.fc));
         asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(r.fc1) : "v"(o.fc), "s"(p.fc));
+    }
+    // The same for the batch plane: the eight blocks of this lane's row, ready as operands, and
+    // the row's eight block scales.
+    constexpr int MFMA6_PLANE_LOADS = 9;
+    constexpr int MFMA6_PLANE_PRODUCERS = 2; // wavefronts that only stage activations there (4: 33.8 against 34.5 us at batch 8, 31.4 against 30.4 us at batch 5)
+    constexpr int MFMA6_PLANE_COMPUTE = 8; // compute wavefronts per workgroup of the plane kernel (12: 39.9 us, 14: 38.9 us against 34.7 us at 5120 x 25600)
+    struct Mfma6PlaneRaw
+    {
+        v4i w0, w1, w2, w3, w4, w5, w6, w7, sc;
+    };
+    __device__ __forceinline__ void mfma6_plane_load(Mfma6PlaneRaw &r, const uint8_t *pw, const uint8_t *ps, uint32_t ow,
+                                                     uint32_t os)
+    {
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.w0) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:128" : "=&v"(r.w1) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:256" : "=&v"(r.w2) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:384" : "=&v"(r.w3) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:512" : "=&v"(r.w4) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:640" : "=&v"(r.w5) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:768" : "=&v"(r.w6) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:896" : "=&v"(r.w7) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.sc) : "v"(os), "s"(ps));
+    }
+    __device__ __forceinline__ void mfma6_keep(Mfma6PlaneRaw &r)
+    {
+        asm volatile(""
+                     : "+v"(r.w0), "+v"(r.w1), "+v"(r.w2), "+v"(r.w3), "+v"(r.w4), "+v"(r.w5), "+v"(r.w6), "+v"(r.w7),
+                       "+v"(r.sc));
+    }
+    template <int NEWER>
+    __device__ __forceinline__ void mfma6_wait(Mfma6PlaneRaw &r)
+    {
+        asm volatile("s_waitcnt vmcnt(%9)"
+                     : "+v"(r.w0), "+v"(r.w1), "+v"(r.w2), "+v"(r.w3), "+v"(r.w4), "+v"(r.w5), "+v"(r.w6), "+v"(r.w7),
+                       "+v"(r.sc)
+                     : "n"(NEWER));
     }
     __device__ __forceinline__ void mfma6_keep(Mfma6Raw &r)
     {
@@ -381,6 +418,181 @@ namespace llamql
         }
     }
 
+    // The same product from the matrix's batch plane (q6k_plane_bytes): the int8 weights and
+    // block scales that the kernel above works out per launch are read ready-made, 272 bytes per
+    // super-block and row against 224, and nothing is left to decode.  Lane (n, h) loads the
+    // 16 bytes of elements 16h..16h+15 of every block of its row straight into the B operand
+    // (eight lanes read one 128-byte line of the plane; a group's super-block is 1 KB in one
+    // place), so there is no bounce buffer either.  Same block sums, same scales, same order of
+    // the fp32 operations: the results are those of gemv_mfma_q6k_kernel bit for bit.
+    template <int SRC>
+    __global__ void __launch_bounds__((MFMA6_PLANE_COMPUTE + MFMA6_PLANE_PRODUCERS) * WAVE) gemv_mfma_q6k_plane_kernel(const Mfma6Args a)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t mfma6_lds[];
+        const int nsb = a.SB;
+        const int nph = (nsb + a.chunk - 1) / a.chunk; // activation chunks
+        const size_t buf_bytes = mfma_act_bytes(a.chunk);
+        const int ncomp = a.slices * a.tiles; // compute wavefronts
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+
+        auto buf_aq = [&](int ph) { return mfma6_lds + (size_t)(ph & 1) * buf_bytes; };
+        auto buf_asc = [&](int ph) {
+            return reinterpret_cast<float *>(mfma6_lds + (size_t)(ph & 1) * buf_bytes + (size_t)a.chunk * 8 * MFMA_AQ_STRIDE);
+        };
+        auto stage = [&](int ph, int tid, int nthreads, auto un) {
+            const int c0 = ph * a.chunk;
+            const int c1 = c0 + a.chunk < nsb ? c0 + a.chunk : nsb;
+            mfma_stage_acts<SRC, decltype(un)::value>(a.q8, a.x, a.x2, a.ldx, a.M, nsb * 8, c0 * 8, (c1 - c0) * 8,
+                                                      buf_aq(ph), buf_asc(ph), tid, nthreads);
+        };
+        typedef std::integral_constant<int, 3> Together;
+        typedef std::integral_constant<int, 8> Alone;
+
+        if (wave >= ncomp)
+        {
+            stage(0, (int)threadIdx.x, (int)blockDim.x, Together());
+            __syncthreads();
+            for (int ph = 0; ph + 1 < nph; ++ph)
+            {
+                stage(ph + 1, (int)threadIdx.x - ncomp * WAVE, MFMA6_PLANE_PRODUCERS * WAVE, Alone());
+                __syncthreads();
+            }
+        }
+        else
+        {
+            const int l32 = lane & 31, lh = lane >> 5;
+            const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
+            const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
+            const int last_step = nsteps > 0 ? nsteps - 1 : 0;
+            const long tile_row0 = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows;
+            // rows past the end of the tile or of the matrix re-read the last one
+            const long r_tile = tile_row0 + (l32 < a.tile_rows ? l32 : a.tile_rows - 1);
+            const long row = r_tile < a.N ? r_tile : a.N - 1;
+            const uint32_t grp = (uint32_t)(row >> 2) * (uint32_t)nsb; // the group's first super-block
+            const uint32_t off_w = grp * 1024u + (uint32_t)(row & 3) * 32u + 16u * (uint32_t)lh;
+            const uint32_t off_s = grp * 64u + (uint32_t)(row & 3) * 16u;
+            const uint8_t *scales = a.plane + q6k_plane_scales_offset(a.N, nsb);
+
+            // loads are never predicated: past its last step a lane re-reads that step
+            auto issue = [&](Mfma6PlaneRaw &r, int step) {
+                const uint32_t sb = nsteps > 0 ? (uint32_t)(slice + (step < last_step ? step : last_step) * a.slices) : 0u;
+                auto uniform = [](const uint8_t *p) {
+                    const uint64_t b = (uint64_t)p;
+                    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+                    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+                    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
+                };
+                mfma6_plane_load(r, uniform(a.plane + (size_t)sb * 1024), uniform(scales + (size_t)sb * 64), off_w, off_s);
+            };
+            Mfma6PlaneRaw bufA, bufB;
+            issue(bufA, 0);
+            issue(bufB, 1);
+            stage(0, (int)threadIdx.x, (int)blockDim.x, Together()); // while the first weights are in flight
+            __syncthreads();
+            mfma6_keep(bufA); // the staging code must not reuse the registers of the loads in flight
+            mfma6_keep(bufB);
+
+            v16i zero;
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                zero[i] = 0;
+            const int a_lane = (l32 & 7) * 32 + lh * 16; // rows beyond the batch: any row, result unused
+            int step = 0, cur_ph = 0;
+
+            auto compute = [&](const Mfma6PlaneRaw &r) {
+                const int sb = slice + step * a.slices;
+                const int ph = sb / a.chunk;
+                while (cur_ph < ph) // uniform: wait until the chunk this step needs has been staged
+                {
+                    mfma6_barrier();
+                    ++cur_ph;
+                }
+                const int kb0 = (sb - ph * a.chunk) * 8;
+                const uint8_t *ab = buf_aq(ph) + (size_t)kb0 * MFMA_AQ_STRIDE + a_lane;
+                const float *sb_sc = buf_asc(ph) + (size_t)kb0 * 16 + lh * 8;
+                const v4i wv[8] = {r.w0, r.w1, r.w2, r.w3, r.w4, r.w5, r.w6, r.w7};
+                const uint32_t sc[4] = {(uint32_t)r.sc.x, (uint32_t)r.sc.y, (uint32_t)r.sc.z, (uint32_t)r.sc.w};
+                auto product = [&](int j) {
+                    const v4i av = *reinterpret_cast<const v4i *>(ab + j * MFMA_AQ_STRIDE);
+                    return __builtin_amdgcn_mfma_i32_32x32x32_i8(av, wv[j], zero, 0, 0, 0);
+                };
+                // the product of block j+1 is issued before block j is rescaled
+                v16i idot[2];
+                idot[0] = product(0);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                {
+                    if (j + 1 < 8)
+                        idot[(j + 1) & 1] = product(j + 1);
+                    const float4 ad = *reinterpret_cast<const float4 *>(sb_sc + j * 16);
+                    const v16i dd = idot[j & 1];
+                    const float b = h2f((uint16_t)(sc[j >> 1] >> (16 * (j & 1))));
+                    acc[0] = fmaf((float)dd[0], ad.x * b, acc[0]);
+                    acc[1] = fmaf((float)dd[1], ad.y * b, acc[1]);
+                    acc[2] = fmaf((float)dd[2], ad.z * b, acc[2]);
+                    acc[3] = fmaf((float)dd[3], ad.w * b, acc[3]);
+                }
+                ++step;
+            };
+
+            // Two register buffers alternate; each is reloaded, two steps ahead, once its step has
+            // been computed from it (three buffers, 155 registers: 35.4 against 34.4 us).  Every buffer is waited for, also past the end: a register
+            // whose load is still in flight must not look free to the compiler.
+            for (int c0 = 0; c0 < nsteps; c0 += 2)
+            {
+                mfma6_wait<MFMA6_PLANE_LOADS>(bufA);
+                if (step < nsteps) // uniform
+                    compute(bufA);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufA, c0 + 2);
+                mfma6_wait<MFMA6_PLANE_LOADS>(bufB);
+                if (step < nsteps)
+                    compute(bufB);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufB, c0 + 3);
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end
+            mfma6_keep(bufA);
+            mfma6_keep(bufB);
+            while (cur_ph < nph - 1) // the barriers of chunks this wavefront had no part in
+            {
+                mfma6_barrier();
+                ++cur_ph;
+            }
+        }
+
+        // ---- partial sums of the slices, added in slice order -------------------------------------
+        __syncthreads(); // every wavefront is done with the activations
+        float *red = reinterpret_cast<float *>(mfma6_lds); // [compute wavefront][4][64]
+        if (wave < ncomp)
+        {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                red[(wave * 4 + i) * WAVE + lane] = acc[i];
+        }
+        __syncthreads();
+        if (wave < ncomp)
+        {
+            const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
+            const long row = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows + (lane & 31);
+            if (slice == 0 && (lane & 31) < a.tile_rows)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    float v = acc[i];
+                    for (int s = 1; s < a.slices; ++s)
+                        v += red[((wave + s) * 4 + i) * WAVE + lane];
+                    const int m = 4 * (lane >> 5) + i;
+                    if (m < a.M && row < a.N)
+                        a.y[(size_t)m * a.ldy + row] = v;
+                }
+            }
+        }
+    }
+
     struct Mfma6Shape
     {
         int slices, tiles, chunk, tile_rows;
@@ -390,7 +602,7 @@ namespace llamql
     // compute wavefronts, five at least (the scales of eight neighbouring super-blocks share a
     // cache line) and each two steps long; tiles per workgroup to fill its compute wavefronts
     // when there are tiles to spare.
-    inline Mfma6Shape gemv_mfma6_shape_of(long N, int nsb, int cus, int max_compute, int tile_rows)
+    inline Mfma6Shape gemv_mfma6_shape_of(long N, int nsb, int cus, int max_compute, int tile_rows, bool plane = false)
     {
         const long tiles = (N + tile_rows - 1) / tile_rows;
         long want = ((long)cus * max_compute + tiles - 1) / tiles;
@@ -412,7 +624,7 @@ namespace llamql
         sh.grid = (tiles + t - 1) / t;
         // one buffer if the whole row fits beside the bounce buffers and leaves half the LDS
         // free, else two buffers of a whole number of rounds of the slices
-        const size_t bounce = (size_t)sh.slices * t * MFMA6_BOUNCE;
+        const size_t bounce = plane ? 0 : (size_t)sh.slices * t * MFMA6_BOUNCE; // the plane kernel has no bounce buffers
         if (mfma_act_bytes(nsb) * 2 + bounce <= QUAD_MAX_LDS)
             sh.chunk = nsb;
         else
@@ -424,7 +636,7 @@ namespace llamql
     }
     // The tile height that leaves the busiest compute unit the fewest rows (gemv_mfma_shape):
     // 5120 rows are 160 full tiles, and 256 tiles of 20 rows.
-    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus, int max_compute = MFMA6_MAX_COMPUTE)
+    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus, int max_compute = MFMA6_MAX_COMPUTE, bool plane = false)
     {
         const int forced = gemv_mfma_tile_rows_override();
         Mfma6Shape best;
@@ -433,7 +645,7 @@ namespace llamql
         {
             if (forced > 0 && tr != forced)
                 continue;
-            const Mfma6Shape sh = gemv_mfma6_shape_of(N, nsb, cus, max_compute, tr);
+            const Mfma6Shape sh = gemv_mfma6_shape_of(N, nsb, cus, max_compute, tr, plane);
             const long cost = ((sh.grid + cus - 1) / cus) * sh.tiles * tr;
             if (best_cost < 0 || cost * 20 < best_cost * 19) // a shorter tile has to win 5 %
             {

@@ -62,8 +62,21 @@ namespace llamql
 
     // byte offset of the Q6_K factor plane in a prepared matrix of T super-blocks
     __host__ __device__ inline size_t q6k_factors_offset(size_t T) { return (T * 210 + 15) & ~(size_t)15; }
+    // The Q6_K batch plane: the weights of a matrix already requantised to int8, in the order the
+    // matrix unit takes them, beside the 16-bit scales of their blocks.  Rows go in groups of
+    // four: group g = row / 4 holds, per super-block, eight 128-byte lines (one per 32-column
+    // block: the 32 bytes of its four rows one after the other), then, in a second plane, the
+    // eight fp16 block scales of each of its rows.
+    __host__ __device__ inline size_t q6k_plane_groups(long N) { return (size_t)((N + 3) / 4); }
+    __host__ __device__ inline size_t q6k_plane_scales_offset(long N, int nsb) { return q6k_plane_groups(N) * (size_t)nsb * 1024; }
+    __host__ __device__ inline size_t q6k_plane_bytes(long N, int nsb) { return q6k_plane_groups(N) * (size_t)nsb * (1024 + 64); }
     inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
     inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
+    // Batch planes attached to prepared matrices (llam_ql_attach_batch_plane): the plane of the
+    // matrix at d_w if one is attached for this shape, else null.
+    const uint8_t *batch_plane_of(const void *d_w, int N, int K);
+    void batch_plane_attach(const void *d_w, const void *d_plane, int N, int K); // null plane: detach
 
     // Number of compute units of the current device (cached per device).
     int cu_count(int device_id);

@@ -95,7 +95,8 @@ class DenseDecoder:
     bytes (device tensors) when keep_raw is set, for the CPU check."""
 
     def __init__(self, shape: Shape, batch: int, ctx_cap: int, device, seed: int = 0, keep_raw: bool = False,
-                 d_lo: float = 0.001, d_hi: float = 0.02, keep_prepared: bool = False, norm_scale: float | None = None):
+                 d_lo: float = 0.001, d_hi: float = 0.02, keep_prepared: bool = False, norm_scale: float | None = None,
+                 batch_planes: bool | None = None):
         import torch
 
         self.shape, self.batch, self.ctx_cap, self.device = shape, batch, ctx_cap, device
@@ -108,6 +109,11 @@ class DenseDecoder:
         self.keep = []   # device tensors the handle borrows
         self.raw = {} if keep_raw else None
         self.prepared = {} if keep_prepared else None   # name -> prepared weight tensor
+        # Q6_K matrices of many rows (down, lm_head) get an int8 batch plane where the batch is 5..8 rows:
+        # their launches then read ready-made int8 weights (capi.attach_batch_plane); same results
+        if batch_planes is None:
+            batch_planes = batch >= 5
+        self.planed = []   # prepared tensors with a plane attached
         g = torch.Generator(device=device)
         g.manual_seed(seed)
 
@@ -129,6 +135,11 @@ class DenseDecoder:
             raw = synth.weights_torch(fmt, n, k, sd, device, d_lo=d_lo, d_hi=d_hi)
             w = capi.prepare_weights(fmt, raw, n, k) if prepare else raw
             self.keep.append(w)
+            if prepare and batch_planes and fmt == FMT_Q6_K and n >= 4096:
+                plane = capi.attach_batch_plane(fmt, w, n, k)
+                if plane is not None:
+                    self.keep.append(plane)
+                    self.planed.append(w)
             if keep_raw:
                 self.raw[name] = raw
             if keep_prepared:
@@ -157,6 +168,9 @@ class DenseDecoder:
         if self.h:
             self.L.llam_decoder_destroy(self.h)
             self.h = None
+        for w in self.planed:
+            capi.detach_batch_plane(w)
+        self.planed = []
 
     def __del__(self):
         try:

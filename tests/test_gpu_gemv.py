@@ -751,3 +751,90 @@ def test_batch_tile_heights_agree(capi, dev, oracle, fmt, N, K):
             assert np.array_equal(s.cpu().numpy(), exp_sums), tr   # bit-exact whatever the tile height
     finally:
         lib.llam_ql_set_batch_tile_rows(0)
+
+
+# ---- the Q6_K batch plane (llam_ql_build_batch_plane / llam_ql_attach_batch_plane) -----------------------------
+def _plane_rows(plane: np.ndarray, N: int, nsb: int):
+    """The plane's int8 weights as [rows][nsb][256] and fp16 scale bits as [rows][nsb][8], rows = 4 ceil(N / 4):
+    group g = row / 4 keeps, per super-block, eight 128-byte lines (block j: its four rows' 32 bytes in turn), and
+    in a second plane the rows' eight scales."""
+    G = (N + 3) // 4
+    w = plane[:G * nsb * 1024].reshape(G, nsb, 8, 4, 32).transpose(0, 3, 1, 2, 4).reshape(G * 4, nsb, 256)
+    s = plane[G * nsb * 1024:].view(np.uint16).reshape(G, nsb, 4, 8).transpose(0, 2, 1, 3).reshape(G * 4, nsb, 8)
+    return w.view(np.int8), s
+
+
+@pytest.mark.parametrize("N,K", [(37, 2048), (8, 5120), (130, 25600)])
+def test_batch_plane_holds_the_requantised_weights(capi, dev, oracle, N, K):
+    """The plane is the reference's packed Q6_K matrix: every int8 weight and every fp16 block scale equals the CPU
+    restatement's (subblocks), rows that pad the last group of four are zero."""
+    import torch
+
+    nsb = K // 256
+    W = synth.weights_numpy(FMT_Q6_K, N, K, 5 + N)
+    w = capi.prepare_weights(FMT_Q6_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
+    assert capi.batch_plane_bytes(FMT_Q6_K, N, K) == ((N + 3) // 4) * nsb * 1088
+    plane = capi.attach_batch_plane(FMT_Q6_K, w, N, K)
+    try:
+        sync()
+        got_w, got_s = _plane_rows(plane.cpu().numpy(), N, nsb)
+        for r in range(N):
+            for t in range(nsb):
+                ew, es, _ = oracle.subblocks(FMT_Q6_K, W[r, t])
+                assert np.array_equal(got_w[r, t], ew), (r, t)
+                assert np.array_equal(got_s[r, t], es), (r, t)
+        assert not got_w[N:].any() and not got_s[N:].any()
+    finally:
+        capi.detach_batch_plane(w)
+
+
+def test_batch_plane_launches_match(capi, dev, oracle):
+    """Batches of 5..8 rows with a plane attached: bit-identical to the launch without one where that is the
+    matrix-unit kernel as well (K = 25600, batches the quad-lane kernel cannot hold), within the format's tolerance
+    of the CPU restatement everywhere (K = 5120 and batch 5 of K = 25600 leave the quad-lane kernel for it);
+    batches of 1..4 do not look at the plane; detaching restores the old launch."""
+    import torch
+
+    for N, K in ((1030, 25600), (4100, 5120), (50, 2048)):
+        W = synth.weights_numpy(FMT_Q6_K, N, K, 77 + N)
+        w = capi.prepare_weights(FMT_Q6_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
+        x = synth.activations_numpy(8, K, 9)
+        q8 = capi.quantize_q8_1(torch.from_numpy(x).to(dev))
+        rows = slice(max(N - 70, 0), N)
+        exp, _ = oracle.gemm(FMT_Q6_K, W[rows], K, oracle.quantize(x), want_sums=True)
+        before = {M: capi.gemv(FMT_Q6_K, w, q8, M, N, K).clone() for M in (1, 4, 5, 7, 8)}
+        plane = capi.attach_batch_plane(FMT_Q6_K, w, N, K)
+        assert plane is not None
+        try:
+            for M in (1, 4, 5, 7, 8):
+                y = capi.gemv(FMT_Q6_K, w, q8, M, N, K)
+                sync()
+                assert rel_err(y.cpu().numpy()[:, rows], exp[:M]) <= TOL[FMT_Q6_K] * 1e-2, (N, K, M)
+                if M <= 4 or capi.gemv_describe(FMT_Q6_K, M, N, K).kernel == 3:
+                    assert torch.equal(y, before[M]), (N, K, M)
+            # fp32 input quantised inside the launch takes the plane too
+            xf = torch.from_numpy(x).to(dev)
+            scratch = torch.empty(8 * (K // 32) * 36, dtype=torch.uint8, device=dev)
+            y = capi.gemv_f32(FMT_Q6_K, w, xf, 8, N, K, q8_scratch=scratch)
+            sync()
+            assert rel_err(y.cpu().numpy()[:, rows], exp) <= TOL[FMT_Q6_K] * 1e-2
+        finally:
+            capi.detach_batch_plane(w)
+        y = capi.gemv(FMT_Q6_K, w, q8, 8, N, K)
+        sync()
+        assert torch.equal(y, before[8])
+
+
+def test_batch_plane_refusals(capi, dev):
+    import torch
+
+    lib = capi.load()
+    assert capi.batch_plane_bytes(FMT_Q4_K, 5120, 25600) == 0       # Q6_K only
+    assert capi.batch_plane_bytes(FMT_Q6_K, 5120, 1024) == 0        # rows of eight super-blocks and more
+    assert capi.batch_plane_bytes(FMT_Q6_K, 5120, 25600) == 1280 * 100 * 1088
+    buf = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    assert not lib.llam_ql_build_batch_plane(FMT_Q4_K, buf.data_ptr(), buf.data_ptr(), 4, 2048, 0, None)
+    assert not lib.llam_ql_build_batch_plane(FMT_Q6_K, None, buf.data_ptr(), 4, 2048, 0, None)
+    assert not lib.llam_ql_attach_batch_plane(None, buf.data_ptr(), 4, 2048)
+    assert not lib.llam_ql_attach_batch_plane(buf.data_ptr(), buf.data_ptr(), 4, 1024)
+    assert lib.llam_ql_attach_batch_plane(buf.data_ptr(), None, 0, 0)   # detaching what was never attached is fine
