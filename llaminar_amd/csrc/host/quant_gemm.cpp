@@ -102,6 +102,7 @@ namespace llaminar_amd
     void MI355QuantGemmKernel::releaseWeights()
     {
         std::lock_guard<std::mutex> lock(prepare_mutex_);
+        drop_plane_locked();
         if (d_owned_)
         {
             (void)hipSetDevice(device_id_);
@@ -175,6 +176,7 @@ namespace llaminar_amd
         if (!ready("detachWeights"))
             return nullptr;
         std::lock_guard<std::mutex> lock(prepare_mutex_);
+        drop_plane_locked(); // the plane belongs to this operator, not to the weights handed over
         std::unique_ptr<MI355PackedWeights> w(new MI355PackedWeights());
         w->fmt_ = fmt_;
         w->n_ = N_;
@@ -215,6 +217,7 @@ namespace llaminar_amd
             return fail(fn, "weights are format %d [%d x %d] on device %d, the operator is format %d [%d x %d] on device %d",
                         (int)weights->fmt_, weights->n_, weights->k_, weights->device_id_, (int)fmt_, N_, K_, device_id_);
         std::lock_guard<std::mutex> lock(prepare_mutex_);
+        drop_plane_locked();
         if (d_owned_)
         {
             (void)hipSetDevice(device_id_);
@@ -293,6 +296,50 @@ namespace llaminar_amd
         out.k = K_;
         out.blocks_per_row = (uint32_t)(K_ / 32);
         out.codebook_id = fmt_;
+        return true;
+    }
+
+    // ---- batch plane ----------------------------------------------------------------
+
+    void MI355QuantGemmKernel::drop_plane_locked()
+    {
+        if (!d_plane_)
+            return;
+        (void)llam_ql_attach_batch_plane(d_weights_, nullptr, 0, 0);
+        (void)hipSetDevice(device_id_);
+        (void)hipFree(d_plane_); // waits for the launches that read it
+        d_plane_ = nullptr;
+    }
+
+    void MI355QuantGemmKernel::dropBatchPlane()
+    {
+        std::lock_guard<std::mutex> lock(prepare_mutex_);
+        drop_plane_locked();
+    }
+
+    bool MI355QuantGemmKernel::enableBatchPlane()
+    {
+        static const char *fn = "enableBatchPlane";
+        if (!ready(fn))
+            return false;
+        std::lock_guard<std::mutex> lock(prepare_mutex_);
+        if (d_plane_)
+            return true;
+        const size_t bytes = llam_ql_batch_plane_bytes(fmt_, N_, K_);
+        if (bytes == 0)
+            return fail(fn, "format %d [%d x %d] has no batch plane", (int)fmt_, N_, K_);
+        void *p = nullptr;
+        if (hipSetDevice(device_id_) != hipSuccess || hipMalloc(&p, bytes) != hipSuccess)
+            return fail(fn, "hipMalloc of %zu bytes failed", bytes);
+        // built before it is attached: a launch on another stream must not find a half-written plane
+        if (!llam_ql_build_batch_plane(fmt_, d_weights_, p, N_, K_, device_id_, stream_) ||
+            hipStreamSynchronize(static_cast<hipStream_t>(stream_)) != hipSuccess ||
+            !llam_ql_attach_batch_plane(d_weights_, p, N_, K_))
+        {
+            (void)hipFree(p);
+            return fail(fn, "%s", llam_ql_last_error());
+        }
+        d_plane_ = p;
         return true;
     }
 

@@ -372,6 +372,49 @@ static void test_multiply_tensor(uint8_t fmt)
 // detachWeights / cloneWeights / attachWeights (TensorKernels.h:1335-1394) and the snapshot
 // description: a clone attached to another operator of the same shape computes the donor's
 // result bit for bit; a detached operator has no weights and fails until they come back.
+// enableBatchPlane: a Q6_K operator reads its int8 batch plane for batches of 5..8 rows; the
+// result is within tolerance of the CPU restatement, batches of 1..4 do not change, the plane
+// goes away with the weights, and the other formats have none.
+static void test_batch_plane()
+{
+    begin("BatchPlane");
+    const int N = 136, K = 4096;
+    auto w = make_weights(LLAM_FMT_Q6_K, N, K, 91);
+    MI355QuantGemmKernel k(LLAM_FMT_Q6_K, w.data(), N, K, 0);
+    auto a = make_floats((size_t)8 * K, 92);
+    DevBuf<float> dA(a), d4((size_t)4 * N), d8((size_t)8 * N);
+    DeviceTensor A(dA.p, 8, K), C4(d4.p, 4, N), C8(d8.p, 8, N);
+    CHECK(k.multiply_tensor(&A, &C4, 4, N, K));
+    CHECK(k.multiply_tensor(&A, &C8, 8, N, K));
+    const auto y4 = d4.download();
+    const auto ref = oracle_product(LLAM_FMT_Q6_K, w, N, K, a.data(), 8);
+    CHECK(rel_err(d8.download(), ref) <= TOL);
+
+    CHECK(!k.hasBatchPlane() && k.batchPlaneBytes() == 0);
+    CHECK(k.enableBatchPlane());
+    CHECK(k.hasBatchPlane() && k.batchPlaneBytes() == llam_ql_batch_plane_bytes(LLAM_FMT_Q6_K, N, K));
+    CHECK(k.enableBatchPlane()); // idempotent
+    CHECK(k.multiply_tensor(&A, &C8, 8, N, K));
+    const float e = rel_err(d8.download(), ref);
+    printf("    m=8 from the plane: max rel err %.3g\n", e);
+    CHECK(e <= TOL);
+    CHECK(k.multiply_tensor(&A, &C4, 4, N, K));
+    CHECK(d4.download() == y4); // batches of 1..4 never read the plane
+
+    auto taken = k.detachWeights(); // the plane does not travel with the weights
+    CHECK(taken && !k.hasBatchPlane());
+    CHECK(k.attachWeights(std::move(taken)));
+    CHECK(k.multiply_tensor(&A, &C8, 8, N, K));
+    CHECK(rel_err(d8.download(), ref) <= TOL);
+    CHECK(k.enableBatchPlane());
+    k.dropBatchPlane();
+    CHECK(!k.hasBatchPlane());
+
+    auto w4 = make_weights(LLAM_FMT_Q4_K, N, K, 93);
+    MI355QuantGemmKernel k4(LLAM_FMT_Q4_K, w4.data(), N, K, 0);
+    CHECK(!k4.enableBatchPlane() && contains(quant_gemm_last_error(), "no batch plane"));
+}
+
 static void test_weight_handover(uint8_t fmt)
 {
     const std::string name = std::string("WeightHandover_") + fmt_name(fmt);
@@ -654,6 +697,7 @@ int main(int argc, char **argv)
             test_precomputed_q8_1(fmt);
             test_swiglu_and_expert_down(fmt);
         }
+        test_batch_plane();
         test_workspace_and_preuploaded();
         test_registry_end_to_end();
     }
