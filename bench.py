@@ -400,7 +400,7 @@ def parse():
     ap.add_argument("--separate-quantise", action="store_true",
                     help="layer workload: quantiser kernels of their own instead of the fp32-input GEMV calls")
     ap.add_argument("--no-batch-planes", action="store_true",
-                    help="batches of 5..8: decode the Q6_K down projection (and lm_head) per launch instead of reading int8 batch planes")
+                    help="batches of 5..8: no batch planes beside the prepared matrices (llam_ql_attach_batch_plane)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true",
                     help="layer workload at batch 1: skip the short run of the 64-layer decode step")
@@ -446,8 +446,8 @@ def main():
             raw = synth.weights_torch(fmt, N, K, 1000 * l + i, dev)
             w[name] = capi.prepare_weights(fmt, raw, N, K)
             del raw
-            # batches of 5..8 rows: the down projection reads its weights from an int8 batch plane
-            if M >= 5 and name == "down" and not args.no_batch_planes:
+            # batches of 5..8 rows: the projections of 4096 rows and more read their weights from batch planes
+            if M >= 5 and N >= 4096 and not args.no_batch_planes and capi.batch_plane_bytes(fmt, N, K) > 0:
                 planes.append(capi.attach_batch_plane(fmt, w[name], N, K))
         layers.append(w)
     torch.cuda.synchronize()
@@ -603,7 +603,7 @@ def main():
             "bytes_per_step": bytes_per_step,
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
             "distinct_weight_sets": args.layers,
-            "batch_planes": bool(planes),   # the Q6_K down projection read from its int8 batch plane (batches of 5..8)
+            "batch_planes": len(planes) // max(args.layers, 1),   # projections per layer read from batch planes (batches of 5..8)
             "launch": "eager" if graphs is None else "hip-graph replay",
         },
         "roofline": {

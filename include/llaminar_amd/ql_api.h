@@ -60,24 +60,29 @@ void llam_ql_reset_gemv_tuning(void);
  * any other value restores the built-in choice.  No counterpart in the reference. */
 void llam_ql_set_batch_tile_rows(int tile_rows);
 
-/* Batch plane of a prepared Q6_K matrix: its weights requantised to int8 once (the 8.8
- * requantisation of packWeightsCPUNativeVNNI's Q6_K branch, SIMDHelpers.h:12023-12204, which
- * the decode kernels otherwise repeat on every launch) and laid out as the matrix unit takes
- * them, 272 bytes per super-block and row.  Optional and separate from the prepared matrix: a
- * caller that decodes batches of 5..8 rows trades this memory for the time of the
- * requantisation.  While a plane is attached, llam_ql_gemv and the launches built on it read
- * it for batches of 5..8 rows wherever they use the matrix-unit kernel for Q6_K (rows too
- * long for the quad-lane kernel's batch); results are bit-identical with and without.  No
- * counterpart in the reference (its packed matrix IS int8; here int8 is the optional copy).
+/* Batch plane of a prepared matrix: an optional second copy for callers that decode batches of
+ * 5..8 rows, laid out as the matrix unit takes its operands (rows in groups of four, a 128-byte
+ * line per group and block), separate from the prepared matrix.
+ *   Q6_K: the weights requantised to int8 once (the 8.8 requantisation of
+ *     packWeightsCPUNativeVNNI's Q6_K branch, SIMDHelpers.h:12023-12204, which the decode
+ *     kernels otherwise repeat on every launch) beside their fp16 block scales, 272 bytes per
+ *     super-block and row; rows of eight super-blocks and more.  While attached, every batch
+ *     of 5..8 rows of that matrix runs on the matrix-unit kernel and reads the plane.
+ *   Q4_K: the 144 bytes of every super-block regrouped, not changed; shapes whose batches of
+ *     5..8 go to the matrix-unit kernel (4096 rows and more).  The kernel then finds a lane's
+ *     operands at one address and needs no LDS bounce.
+ * Results are bit-identical to the matrix-unit kernels without a plane.  The reference's packed
+ * matrix is int8 in operand order to begin with; here that is the optional copy, and
+ * llam_ql_gemv_describe and the block-sum hooks describe the launch without one.
  *   llam_ql_batch_plane_bytes: size of the plane, 0 if the format or shape has none.
  *   llam_ql_build_batch_plane: fills d_plane (16-byte aligned) from the prepared matrix.
- *   llam_ql_attach_batch_plane: d_plane != NULL attaches it to d_prepared (same N, K as built),
- *     NULL detaches.  Detach before either buffer is freed.  Thread-safe; launches in flight
- *     keep reading the plane they were given. */
+ *   llam_ql_attach_batch_plane: d_plane != NULL attaches it to d_prepared (fmt, N, K as built),
+ *     NULL detaches (fmt, N, K ignored).  Detach before either buffer is freed.  Thread-safe;
+ *     launches in flight keep reading the plane they were given. */
 size_t llam_ql_batch_plane_bytes(uint8_t fmt, int N, int K);
 bool llam_ql_build_batch_plane(uint8_t fmt, const void* d_prepared, void* d_plane, int N, int K,
                                int device_id, void* stream);
-bool llam_ql_attach_batch_plane(const void* d_prepared, const void* d_plane, int N, int K);
+bool llam_ql_attach_batch_plane(uint8_t fmt, const void* d_prepared, const void* d_plane, int N, int K);
 
 /* Read-only probe for measurements: streams the N * (K/256) * 144 bytes of a Q4_K-sized
  * buffer once and computes nothing, in the order a decode GEMV would read them.  No

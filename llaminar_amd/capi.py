@@ -51,7 +51,7 @@ SIGNATURES = {
     "llam_ql_set_batch_tile_rows": (None, [c_int]),
     "llam_ql_batch_plane_bytes": (c_size_t, [c_uint8, c_int, c_int]),
     "llam_ql_build_batch_plane": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
-    "llam_ql_attach_batch_plane": (c_bool, [c_void_p, c_void_p, c_int, c_int]),
+    "llam_ql_attach_batch_plane": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int]),
     "llam_ql_read_probe": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_quantize_q8_1": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_prepared_bytes": (c_size_t, [c_uint8, c_int, c_int]),
@@ -228,12 +228,12 @@ def attach_batch_plane(fmt: int, w, N: int, K: int, stream=None):
         return None
     plane = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
     _check(load().llam_ql_build_batch_plane(fmt, _ptr(w), _ptr(plane), N, K, _dev(w), _stream(stream)), "build_batch_plane")
-    _check(load().llam_ql_attach_batch_plane(_ptr(w), _ptr(plane), N, K), "attach_batch_plane")
+    _check(load().llam_ql_attach_batch_plane(fmt, _ptr(w), _ptr(plane), N, K), "attach_batch_plane")
     return plane
 
 
 def detach_batch_plane(w):
-    _check(load().llam_ql_attach_batch_plane(_ptr(w), None, 0, 0), "attach_batch_plane")
+    _check(load().llam_ql_attach_batch_plane(0, _ptr(w), None, 0, 0), "attach_batch_plane")
 
 
 def gemv(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None):

@@ -225,17 +225,49 @@ namespace llamql
             *dsc = (uint16_t)(rec >> 16);
     }
 
-    // A plane exists for Q6_K rows of eight super-blocks and more, as the matrix-unit kernels ask.
+    // One thread per 16-byte piece of a super-block: piece 0, the head, goes to the heads plane,
+    // piece 1 + 2c + h is half h of group c.  Rows past N (the last group's padding) are zeros.
+    __global__ void __launch_bounds__(256) build_q4k_plane_kernel(const uint8_t *prepared, uint8_t *plane, long N, int nsb)
+    {
+        const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        const size_t rows = q6k_plane_groups(N) * 4;
+        if (idx >= rows * (size_t)nsb * 9)
+            return;
+        const size_t rs = idx / 9; // row * nsb + sb
+        const int piece = (int)(idx - rs * 9);
+        const size_t row = rs / (size_t)nsb;
+        const int sb = (int)(rs - row * (size_t)nsb);
+        const size_t cell = (row >> 2) * (size_t)nsb + (size_t)sb; // the group's super-block
+        v4i v = {0, 0, 0, 0};
+        if ((long)row < N)
+            v = *reinterpret_cast<const v4i *>(prepared + rs * 144 + piece * 16);
+        uint8_t *dst = piece == 0 ? plane + q4k_plane_heads_offset(N, nsb) + cell * 64 + (row & 3) * 16
+                                  : plane + (cell * 4 + (size_t)((piece - 1) >> 1)) * 128 + (row & 3) * 32 + 16 * ((piece - 1) & 1);
+        *reinterpret_cast<v4i *>(dst) = v;
+    }
+
+    // A plane exists for Q6_K rows of eight super-blocks and more, and for the Q4_K shapes whose
+    // batches of 5..8 go to the matrix-unit kernel.
     static bool batch_plane_shape(uint8_t fmt, int N, int K)
     {
-        return fmt == LLAM_FMT_Q6_K && N >= 1 && K >= 2048 && K % 256 == 0 &&
-               q6k_plane_bytes(N, K / 256) < ((size_t)1 << 32); // the kernel's lane offsets are 32-bit
+        if (N < 1 || K < 2048 || K % 256 != 0)
+            return false;
+        // (the kernels' lane offsets are 32-bit)
+        if (fmt == LLAM_FMT_Q6_K)
+            return q6k_plane_bytes(N, K / 256) < ((size_t)1 << 32);
+        if (fmt == LLAM_FMT_Q4_K)
+            return mfma_eligible<Q4KTraits>(8, N, K) && q4k_plane_bytes(N, K / 256) < ((size_t)1 << 32);
+        return false;
+    }
+    static size_t batch_plane_size(uint8_t fmt, int N, int K)
+    {
+        return fmt == LLAM_FMT_Q6_K ? q6k_plane_bytes(N, K / 256) : q4k_plane_bytes(N, K / 256);
     }
 } // namespace llamql
 
 extern "C" size_t llam_ql_batch_plane_bytes(uint8_t fmt, int N, int K)
 {
-    return llamql::batch_plane_shape(fmt, N, K) ? llamql::q6k_plane_bytes(N, K / 256) : 0;
+    return llamql::batch_plane_shape(fmt, N, K) ? llamql::batch_plane_size(fmt, N, K) : 0;
 }
 
 extern "C" bool llam_ql_build_batch_plane(uint8_t fmt, const void *d_prepared, void *d_plane, int N, int K,
@@ -252,16 +284,20 @@ extern "C" bool llam_ql_build_batch_plane(uint8_t fmt, const void *d_prepared, v
     if (!set_device(fn, device_id))
         return false;
     const int nsb = K / 256;
-    const size_t items = q6k_plane_groups(N) * 4 * (size_t)nsb * 16;
+    const size_t items = q6k_plane_groups(N) * 4 * (size_t)nsb * (fmt == LLAM_FMT_Q6_K ? 16 : 9);
     const size_t grid = (items + 255) / 256;
     if (grid > 0x7FFFFFFFull)
         return fail(fn, "matrix too large (N=%d K=%d)", N, K);
-    hipLaunchKernelGGL(build_q6k_plane_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream),
-                       static_cast<const uint8_t *>(d_prepared), static_cast<uint8_t *>(d_plane), (long)N, nsb);
+    if (fmt == LLAM_FMT_Q6_K)
+        hipLaunchKernelGGL(build_q6k_plane_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream),
+                           static_cast<const uint8_t *>(d_prepared), static_cast<uint8_t *>(d_plane), (long)N, nsb);
+    else
+        hipLaunchKernelGGL(build_q4k_plane_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream),
+                           static_cast<const uint8_t *>(d_prepared), static_cast<uint8_t *>(d_plane), (long)N, nsb);
     return launched(fn);
 }
 
-extern "C" bool llam_ql_attach_batch_plane(const void *d_prepared, const void *d_plane, int N, int K)
+extern "C" bool llam_ql_attach_batch_plane(uint8_t fmt, const void *d_prepared, const void *d_plane, int N, int K)
 {
     using namespace llamql;
     static const char *fn = "llam_ql_attach_batch_plane";
@@ -269,11 +305,11 @@ extern "C" bool llam_ql_attach_batch_plane(const void *d_prepared, const void *d
         return fail(fn, "null d_prepared");
     if (d_plane)
     {
-        if (!batch_plane_shape(LLAM_FMT_Q6_K, N, K))
-            return fail(fn, "no batch plane for N=%d, K=%d", N, K);
+        if (!batch_plane_shape(fmt, N, K))
+            return fail(fn, "no batch plane for format %d, N=%d, K=%d", (int)fmt, N, K);
         if (!aligned16(d_plane))
             return fail(fn, "d_plane must be 16-byte aligned");
     }
-    batch_plane_attach(d_prepared, d_plane, N, K);
+    batch_plane_attach(fmt, d_prepared, d_plane, N, K);
     return true;
 }

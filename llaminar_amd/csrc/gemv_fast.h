@@ -456,12 +456,12 @@ namespace llamql
             return mfma_max_slices(K / 256) >= 1 && N >= MFMA_MIN_ROWS;
     }
 
-    template <int SRC, bool DUMP = false>
+    template <int SRC, bool DUMP = false, bool PLANE = false>
     void gemv_mfma_q4k_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const MfmaArgs &a)
     {
         static LdsGrant grant;
-        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<SRC, DUMP>), QUAD_MAX_LDS);
-        hipLaunchKernelGGL((gemv_mfma_q4k_kernel<SRC, DUMP>), grid, block, lds, st, a);
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<SRC, DUMP, PLANE>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_mfma_q4k_kernel<SRC, DUMP, PLANE>), grid, block, lds, st, a);
     }
 
     inline bool gemv_mfma_q4k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
@@ -472,6 +472,8 @@ namespace llamql
         const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id), d_sums ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES);
         MfmaArgs a;
         a.w = static_cast<const uint8_t *>(d_w);
+        // the matrix's batch plane if one is attached (the block-sum variant reads the prepared matrix)
+        a.plane = d_sums ? nullptr : batch_plane_of(LLAM_FMT_Q4_K, d_w, N, K);
         a.q8 = static_cast<const uint32_t *>(src.q8);
         a.x = src.x;
         a.x2 = src.x2;
@@ -487,12 +489,22 @@ namespace llamql
         a.row0 = row0;
         a.nrows = nrows;
         const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles_per_wg) * WAVE);
-        const size_t lds = mfma_lds_bytes(SB, sh.slices * sh.tiles_per_wg);
+        const size_t lds = a.plane ? mfma_act_bytes(SB) : mfma_lds_bytes(SB, sh.slices * sh.tiles_per_wg);
         if (d_sums)
         {
             if (src.kind != ACT_SRC_Q8)
                 return fail(fn, "block sums are dumped on Q8_1 input");
             gemv_mfma_q4k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            return launched(fn);
+        }
+        if (a.plane)
+        {
+            switch (src.kind)
+            {
+            case ACT_SRC_F32: gemv_mfma_q4k_launch_src<QUAD_SRC_F32, false, true>(grid, block, lds, st, a); break;
+            case ACT_SRC_SWIGLU: gemv_mfma_q4k_launch_src<QUAD_SRC_SWIGLU, false, true>(grid, block, lds, st, a); break;
+            default: gemv_mfma_q4k_launch_src<QUAD_SRC_Q8, false, true>(grid, block, lds, st, a); break;
+            }
             return launched(fn);
         }
         switch (src.kind)
@@ -526,7 +538,7 @@ namespace llamql
     {
         const int SB = K / 256;
         // the matrix's batch plane if one is attached (the block-sum variant decodes the weights itself)
-        const uint8_t *plane = d_sums ? nullptr : batch_plane_of(d_w, N, K);
+        const uint8_t *plane = d_sums ? nullptr : batch_plane_of(LLAM_FMT_Q6_K, d_w, N, K);
         const Mfma6Shape sh =
             gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA6_DUMP_COMPUTE : plane ? MFMA6_PLANE_COMPUTE : MFMA6_MAX_COMPUTE,
                              plane != nullptr);
@@ -577,14 +589,20 @@ namespace llamql
         return launched(fn);
     }
 
-    // The batch plane attached to a Q6_K matrix, for a batch the plane kernel takes (5..8 rows,
-    // no tuning override in force), else null.
+    // The batch plane attached to a matrix, for a batch the plane kernels take (5..8 rows, no
+    // tuning override in force), else null.  Q6_K: wherever a plane is attached; Q4_K: where the
+    // batch goes to the matrix-unit kernel anyway.
     template <class F>
     const uint8_t *batch_plane_for(const void *d_w, int M, int N, int K)
     {
-        if constexpr (F::USE_MFMA_BATCH && std::is_same<typename F::Quad, Q6KQuad>::value)
+        if constexpr (F::USE_MFMA_BATCH)
             if (M >= 5 && M <= 8 && gemv_unroll_override() == 0 && gemv_rows_per_wave_override() == 0)
-                return batch_plane_of(d_w, N, K);
+            {
+                if constexpr (std::is_same<typename F::Quad, Q6KQuad>::value)
+                    return batch_plane_of(LLAM_FMT_Q6_K, d_w, N, K);
+                else
+                    return mfma_eligible<F>(M, N, K) ? batch_plane_of(LLAM_FMT_Q4_K, d_w, N, K) : nullptr;
+            }
         return nullptr;
     }
 

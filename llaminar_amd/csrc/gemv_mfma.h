@@ -25,6 +25,7 @@
 #pragma once
 #include "gemv_core.h"
 #include "gemv_quad.h"
+#include <type_traits>
 
 namespace llamql
 {
@@ -39,6 +40,7 @@ namespace llamql
     struct MfmaArgs
     {
         const uint8_t *w;   // Q4_K super-blocks, row-major
+        const uint8_t *plane; // PLANE kernels: the matrix's batch plane (q4k_plane_bytes), w is not read
         const uint32_t *q8; // Q8_1 activations as dwords (9 per block), M rows (QUAD_SRC_Q8)
         const float *x;     // fp32 rows of ldx floats (QUAD_SRC_F32); the gate rows for QUAD_SRC_SWIGLU
         const float *x2;    // the up rows for QUAD_SRC_SWIGLU
@@ -90,6 +92,34 @@ namespace llamql
     {
         asm volatile("s_waitcnt vmcnt(%5)"
                      : "+v"(r.c0), "+v"(r.c1), "+v"(r.c2), "+v"(r.c3), "+v"(r.c4)
+                     : "n"(NEWER));
+    }
+    // The same bytes from the matrix's batch plane, where they lie in the order the lanes take
+    // them: the head of this lane's row's super-block (d, dmin, scales) and its half of the four
+    // 32-byte groups.
+    constexpr int MFMA_PLANE_LOADS = 5;
+    struct MfmaPlaneRaw
+    {
+        v4i head, q0, q1, q2, q3;
+    };
+    __device__ __forceinline__ void mfma_plane_load(MfmaPlaneRaw &r, const uint8_t *pw, const uint8_t *ph, uint32_t ow,
+                                                    uint32_t oh)
+    {
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.head) : "v"(oh), "s"(ph));
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.q0) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:128" : "=&v"(r.q1) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:256" : "=&v"(r.q2) : "v"(ow), "s"(pw));
+        asm volatile("global_load_dwordx4 %0, %1, %2 offset:384" : "=&v"(r.q3) : "v"(ow), "s"(pw));
+    }
+    __device__ __forceinline__ void mfma_keep(MfmaPlaneRaw &r)
+    {
+        asm volatile("" : "+v"(r.head), "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3));
+    }
+    template <int NEWER>
+    __device__ __forceinline__ void mfma_wait(MfmaPlaneRaw &r)
+    {
+        asm volatile("s_waitcnt vmcnt(%5)"
+                     : "+v"(r.head), "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3)
                      : "n"(NEWER));
     }
     // orders the LDS traffic of one wavefront as seen by the compiler; the hardware runs a
@@ -220,10 +250,17 @@ namespace llamql
     // Its stores need registers the 16-wavefront workgroup does not have (and the build refuses to
     // spill): the variant runs in workgroups of at most MFMA_DUMP_WAVES wavefronts, fewer tiles per
     // workgroup, the same code per tile.
-    template <int SRC, bool DUMP = false>
+    // PLANE: the weights come from the matrix's batch plane (ql_host.h: the super-blocks' bytes
+    // regrouped so that lane (row, h) finds its operands at one address, 128-byte lines shared by
+    // four rows): no bounce buffer, a step is computed straight from the registers its loads
+    // filled.  Same decode, same products, same order: bit-identical results.
+    template <int SRC, bool DUMP = false, bool PLANE = false>
     __global__ void __launch_bounds__((DUMP ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES) * WAVE)
         gemv_mfma_q4k_kernel(const MfmaArgs a)
     {
+        static_assert(!(DUMP && PLANE), "the block-sum variant reads the prepared matrix");
+        typedef typename std::conditional<PLANE, MfmaPlaneRaw, MfmaRaw>::type Raw;
+        constexpr int LOADS = PLANE ? MFMA_PLANE_LOADS : MFMA_LOADS;
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];
         const int nsb = a.SB;
         const int nkb = nsb * 8;
@@ -271,14 +308,27 @@ namespace llamql
         const uint8_t *bounce_rdq = bounce_rd + 16 + 16 * lh;        // its half of every group
 
         // loads are never predicated: past the end of the slice a lane re-reads its last block
-        auto issue = [&](MfmaRaw &r, int step) {
-            const int sb = nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0;
-            const uint64_t b = (uint64_t)(tile_base + (size_t)sb * 144);
+        // PLANE: this lane's row (past the tile or the matrix: the last one), its group's first
+        // super-block and its byte offsets in the two planes
+        const long prow = base_row + (l32 < max_local ? l32 : max_local);
+        const uint32_t pgrp = (uint32_t)(prow >> 2) * (uint32_t)nsb;
+        const uint32_t poff_w = pgrp * 512u + (uint32_t)(prow & 3) * 32u + 16u * (uint32_t)lh;
+        const uint32_t poff_h = pgrp * 64u + (uint32_t)(prow & 3) * 16u;
+        auto uniform = [](const uint8_t *p) {
+            const uint64_t b = (uint64_t)p;
             const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
             const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
-            mfma_load(r, reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo), off);
+            return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
         };
-        MfmaRaw bufA, bufB;
+        auto issue = [&](Raw &r, int step) {
+            const int sb = nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0;
+            if constexpr (PLANE)
+                mfma_plane_load(r, uniform(a.plane + (size_t)sb * 512),
+                                uniform(a.plane + q4k_plane_heads_offset(a.N, nsb) + (size_t)sb * 64), poff_w, poff_h);
+            else
+                mfma_load(r, uniform(tile_base + (size_t)sb * 144), off);
+        };
+        Raw bufA, bufB;
         // ---- activations into LDS ------------------------------------------------------------
         if constexpr (SRC == QUAD_SRC_Q8)
         {
@@ -290,7 +340,7 @@ namespace llamql
             quad_act_issue(ar, a.q8, total);
             issue(bufA, 0);
             issue(bufB, 1);
-            quad_act_wait<2 * MFMA_LOADS>(ar);
+            quad_act_wait<2 * LOADS>(ar);
             if (total <= MFMA_ACT_PASSES * (int)blockDim.x) // uniform
                 mfma_act_store(ar, nkb, total, aq, asc);
             else
@@ -337,13 +387,10 @@ namespace llamql
             mfma_wave_sync();
         };
 
-        auto compute = [&]() {
+        // this lane's operands: the head of its row's super-block and its half of the four groups
+        auto compute = [&](const v4i head, const v4i q0, const v4i q1, const v4i q2, const v4i q3) {
             const int sb = slice + step * a.slices;
-            // this lane's operands: the head of its row's super-block and its half of the four groups
-            const v4i head = *reinterpret_cast<const v4i *>(bounce_rd);
-            const v4i q[4] = {*reinterpret_cast<const v4i *>(bounce_rdq), *reinterpret_cast<const v4i *>(bounce_rdq + 32),
-                              *reinterpret_cast<const v4i *>(bounce_rdq + 64),
-                              *reinterpret_cast<const v4i *>(bounce_rdq + 96)};
+            const v4i q[4] = {q0, q1, q2, q3};
             Q4KQuad::Scale S[4];
             Q4KQuad::decode_scales(head, Q4KQuad::lane_consts(0), S[0]);
             Q4KQuad::decode_scales(head, Q4KQuad::lane_consts(1), S[1]);
@@ -409,24 +456,46 @@ namespace llamql
         // pieces are in LDS, before the step is computed.  Every buffer is waited for, also past
         // the end of the slice: a register whose load is still in flight must not look free to
         // the compiler.
+        auto compute_lds = [&]() {
+            compute(*reinterpret_cast<const v4i *>(bounce_rd), *reinterpret_cast<const v4i *>(bounce_rdq),
+                    *reinterpret_cast<const v4i *>(bounce_rdq + 32), *reinterpret_cast<const v4i *>(bounce_rdq + 64),
+                    *reinterpret_cast<const v4i *>(bounce_rdq + 96));
+        };
         for (int c0 = 0; c0 < nsteps; c0 += 2)
         {
-            mfma_wait<MFMA_LOADS>(bufA);
-            if (step < nsteps) // uniform
-                stage(bufA);
-            __builtin_amdgcn_sched_barrier(0);
-            issue(bufA, c0 + 2);
-            if (step < nsteps)
-                compute();
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_wait<MFMA_LOADS>(bufB);
-            if (step < nsteps)
-                stage(bufB);
-            __builtin_amdgcn_sched_barrier(0);
-            issue(bufB, c0 + 3);
-            if (step < nsteps)
-                compute();
-            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (PLANE)
+            {
+                // a buffer is reloaded once its step has been computed from it
+                mfma_wait<LOADS>(bufA);
+                if (step < nsteps) // uniform
+                    compute(bufA.head, bufA.q0, bufA.q1, bufA.q2, bufA.q3);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufA, c0 + 2);
+                mfma_wait<LOADS>(bufB);
+                if (step < nsteps)
+                    compute(bufB.head, bufB.q0, bufB.q1, bufB.q2, bufB.q3);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufB, c0 + 3);
+            }
+            else
+            {
+                mfma_wait<LOADS>(bufA);
+                if (step < nsteps) // uniform
+                    stage(bufA);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufA, c0 + 2);
+                if (step < nsteps)
+                    compute_lds();
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_wait<LOADS>(bufB);
+                if (step < nsteps)
+                    stage(bufB);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(bufB, c0 + 3);
+                if (step < nsteps)
+                    compute_lds();
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end of the slice
         mfma_keep(bufA);

@@ -305,7 +305,7 @@ namespace llaminar_amd
     {
         if (!d_plane_)
             return;
-        (void)llam_ql_attach_batch_plane(d_weights_, nullptr, 0, 0);
+        (void)llam_ql_attach_batch_plane(fmt_, d_weights_, nullptr, 0, 0);
         (void)hipSetDevice(device_id_);
         (void)hipFree(d_plane_); // waits for the launches that read it
         d_plane_ = nullptr;
@@ -334,7 +334,7 @@ namespace llaminar_amd
         // built before it is attached: a launch on another stream must not find a half-written plane
         if (!llam_ql_build_batch_plane(fmt_, d_weights_, p, N_, K_, device_id_, stream_) ||
             hipStreamSynchronize(static_cast<hipStream_t>(stream_)) != hipSuccess ||
-            !llam_ql_attach_batch_plane(d_weights_, p, N_, K_))
+            !llam_ql_attach_batch_plane(fmt_, d_weights_, p, N_, K_))
         {
             (void)hipFree(p);
             return fail(fn, "%s", llam_ql_last_error());

@@ -52,25 +52,26 @@ namespace llamql
         {
             const uint8_t *plane;
             int N, K;
+            uint8_t fmt;
         };
         std::mutex g_plane_mu;
         std::unordered_map<const void *, BatchPlane> g_planes;
     } // namespace
 
-    const uint8_t *batch_plane_of(const void *d_w, int N, int K)
+    const uint8_t *batch_plane_of(uint8_t fmt, const void *d_w, int N, int K)
     {
         std::lock_guard<std::mutex> lock(g_plane_mu);
         if (g_planes.empty())
             return nullptr;
         const auto it = g_planes.find(d_w);
-        return it != g_planes.end() && it->second.N == N && it->second.K == K ? it->second.plane : nullptr;
+        return it != g_planes.end() && it->second.N == N && it->second.K == K && it->second.fmt == fmt ? it->second.plane : nullptr;
     }
 
-    void batch_plane_attach(const void *d_w, const void *d_plane, int N, int K)
+    void batch_plane_attach(uint8_t fmt, const void *d_w, const void *d_plane, int N, int K)
     {
         std::lock_guard<std::mutex> lock(g_plane_mu);
         if (d_plane)
-            g_planes[d_w] = BatchPlane{static_cast<const uint8_t *>(d_plane), N, K};
+            g_planes[d_w] = BatchPlane{static_cast<const uint8_t *>(d_plane), N, K, fmt};
         else
             g_planes.erase(d_w);
     }

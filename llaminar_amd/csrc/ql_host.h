@@ -70,13 +70,19 @@ namespace llamql
     __host__ __device__ inline size_t q6k_plane_groups(long N) { return (size_t)((N + 3) / 4); }
     __host__ __device__ inline size_t q6k_plane_scales_offset(long N, int nsb) { return q6k_plane_groups(N) * (size_t)nsb * 1024; }
     __host__ __device__ inline size_t q6k_plane_bytes(long N, int nsb) { return q6k_plane_groups(N) * (size_t)nsb * (1024 + 64); }
+    // The Q4_K batch plane: the 144 bytes of every super-block regrouped, not changed.  Rows in
+    // groups of four; per group and super-block four 128-byte lines (one per 32-byte group of
+    // quants: the four rows' 32 bytes in turn), then, in a second plane, the rows' 16-byte heads
+    // (d, dmin, scales).
+    __host__ __device__ inline size_t q4k_plane_heads_offset(long N, int nsb) { return q6k_plane_groups(N) * (size_t)nsb * 512; }
+    __host__ __device__ inline size_t q4k_plane_bytes(long N, int nsb) { return q6k_plane_groups(N) * (size_t)nsb * (512 + 64); }
     inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
     inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
     // Batch planes attached to prepared matrices (llam_ql_attach_batch_plane): the plane of the
     // matrix at d_w if one is attached for this shape, else null.
-    const uint8_t *batch_plane_of(const void *d_w, int N, int K);
-    void batch_plane_attach(const void *d_w, const void *d_plane, int N, int K); // null plane: detach
+    const uint8_t *batch_plane_of(uint8_t fmt, const void *d_w, int N, int K);
+    void batch_plane_attach(uint8_t fmt, const void *d_w, const void *d_plane, int N, int K); // null plane: detach
 
     // Number of compute units of the current device (cached per device).
     int cu_count(int device_id);

@@ -109,8 +109,9 @@ class DenseDecoder:
         self.keep = []   # device tensors the handle borrows
         self.raw = {} if keep_raw else None
         self.prepared = {} if keep_prepared else None   # name -> prepared weight tensor
-        # Q6_K matrices of many rows (down, lm_head) get an int8 batch plane where the batch is 5..8 rows:
-        # their launches then read ready-made int8 weights (capi.attach_batch_plane); same results
+        # Matrices of 4096 rows and more get a batch plane where the batch is 5..8 rows (capi.attach_batch_plane):
+        # Q6_K ones (down, lm_head) an int8 copy, Q4_K ones (Q, O, gate, up) their bytes in the matrix unit's
+        # operand order; same results, less work per launch
         if batch_planes is None:
             batch_planes = batch >= 5
         self.planed = []   # prepared tensors with a plane attached
@@ -135,7 +136,7 @@ class DenseDecoder:
             raw = synth.weights_torch(fmt, n, k, sd, device, d_lo=d_lo, d_hi=d_hi)
             w = capi.prepare_weights(fmt, raw, n, k) if prepare else raw
             self.keep.append(w)
-            if prepare and batch_planes and fmt == FMT_Q6_K and n >= 4096:
+            if prepare and batch_planes and n >= 4096 and capi.batch_plane_bytes(fmt, n, k) > 0:
                 plane = capi.attach_batch_plane(fmt, w, n, k)
                 if plane is not None:
                     self.keep.append(plane)

@@ -765,7 +765,7 @@ def _plane_rows(plane: np.ndarray, N: int, nsb: int):
 
 
 @pytest.mark.parametrize("N,K", [(37, 2048), (8, 5120), (130, 25600)])
-def test_batch_plane_holds_the_requantised_weights(capi, dev, oracle, N, K):
+def test_q6k_batch_plane_holds_the_requantised_weights(capi, dev, oracle, N, K):
     """The plane is the reference's packed Q6_K matrix: every int8 weight and every fp16 block scale equals the CPU
     restatement's (subblocks), rows that pad the last group of four are zero."""
     import torch
@@ -788,7 +788,7 @@ def test_batch_plane_holds_the_requantised_weights(capi, dev, oracle, N, K):
         capi.detach_batch_plane(w)
 
 
-def test_batch_plane_launches_match(capi, dev, oracle):
+def test_q6k_batch_plane_launches_match(capi, dev, oracle):
     """Batches of 5..8 rows with a plane attached: bit-identical to the launch without one where that is the
     matrix-unit kernel as well (K = 25600, batches the quad-lane kernel cannot hold), within the format's tolerance
     of the CPU restatement everywhere (K = 5120 and batch 5 of K = 25600 leave the quad-lane kernel for it);
@@ -829,12 +829,71 @@ def test_batch_plane_refusals(capi, dev):
     import torch
 
     lib = capi.load()
-    assert capi.batch_plane_bytes(FMT_Q4_K, 5120, 25600) == 0       # Q6_K only
+    assert capi.batch_plane_bytes(FMT_IQ3_S, 5120, 25600) == 0      # Q4_K and Q6_K only
+    assert capi.batch_plane_bytes(FMT_Q4_K, 1024, 5120) == 0        # Q4_K: where batches go to the matrix unit
+    assert capi.batch_plane_bytes(FMT_Q4_K, 25600, 5120) == 6400 * 20 * 576
     assert capi.batch_plane_bytes(FMT_Q6_K, 5120, 1024) == 0        # rows of eight super-blocks and more
     assert capi.batch_plane_bytes(FMT_Q6_K, 5120, 25600) == 1280 * 100 * 1088
     buf = torch.zeros(4096, dtype=torch.uint8, device=dev)
-    assert not lib.llam_ql_build_batch_plane(FMT_Q4_K, buf.data_ptr(), buf.data_ptr(), 4, 2048, 0, None)
+    assert not lib.llam_ql_build_batch_plane(FMT_Q4_K, buf.data_ptr(), buf.data_ptr(), 4, 2048, 0, None)   # too few rows
     assert not lib.llam_ql_build_batch_plane(FMT_Q6_K, None, buf.data_ptr(), 4, 2048, 0, None)
-    assert not lib.llam_ql_attach_batch_plane(None, buf.data_ptr(), 4, 2048)
-    assert not lib.llam_ql_attach_batch_plane(buf.data_ptr(), buf.data_ptr(), 4, 1024)
-    assert lib.llam_ql_attach_batch_plane(buf.data_ptr(), None, 0, 0)   # detaching what was never attached is fine
+    assert not lib.llam_ql_attach_batch_plane(FMT_Q6_K, None, buf.data_ptr(), 4, 2048)
+    assert not lib.llam_ql_attach_batch_plane(FMT_Q6_K, buf.data_ptr(), buf.data_ptr(), 4, 1024)
+    assert not lib.llam_ql_attach_batch_plane(FMT_IQ3_S, buf.data_ptr(), buf.data_ptr(), 4096, 5120)
+    assert lib.llam_ql_attach_batch_plane(0, buf.data_ptr(), None, 0, 0)   # detaching what was never attached is fine
+
+
+def test_q4k_batch_plane_is_the_prepared_matrix_regrouped(capi, dev):
+    """The Q4_K plane holds the bytes of the super-blocks, not new ones: per group of four rows and super-block four
+    128-byte lines (the rows' two 16-byte halves of one 32-byte group of quants each), then the rows' heads."""
+    import torch
+
+    N, K = 4098, 2048   # a last group of two rows
+    nsb = K // 256
+    W = synth.weights_numpy(FMT_Q4_K, N, K, 3)           # [N][nsb][144]
+    w = capi.prepare_weights(FMT_Q4_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
+    G = (N + 3) // 4
+    assert capi.batch_plane_bytes(FMT_Q4_K, N, K) == G * nsb * 576
+    plane = capi.attach_batch_plane(FMT_Q4_K, w, N, K)
+    try:
+        sync()
+        p = plane.cpu().numpy()
+        pad = np.zeros((G * 4, nsb, 144), np.uint8)
+        pad[:N] = W.reshape(N, nsb, 144)
+        quants = pad[:, :, 16:].reshape(G, 4, nsb, 4, 32).transpose(0, 2, 3, 1, 4)   # [g][sb][group of quants][row][32]
+        heads = pad[:, :, :16].reshape(G, 4, nsb, 16).transpose(0, 2, 1, 3)          # [g][sb][row][16]
+        assert np.array_equal(p[:G * nsb * 512], quants.reshape(-1))
+        assert np.array_equal(p[G * nsb * 512:], heads.reshape(-1))
+    finally:
+        capi.detach_batch_plane(w)
+
+
+def test_q4k_batch_plane_launches_match(capi, dev, oracle):
+    """Q4_K batches of 5..8 with a plane attached: the matrix-unit kernel's results bit for bit, close to the CPU
+    restatement; rows that do not fill the last tile or group included; fp32 and SwiGLU input as well."""
+    import torch
+
+    for N, K in ((4100, 5120), (4097, 8192)):
+        W = synth.weights_numpy(FMT_Q4_K, N, K, 21 + N)
+        w = capi.prepare_weights(FMT_Q4_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
+        x = synth.activations_numpy(8, K, 4)
+        xd = torch.from_numpy(x).to(dev)
+        q8 = capi.quantize_q8_1(xd)
+        rows = slice(N - 70, N)
+        exp, _ = oracle.gemm(FMT_Q4_K, W[rows], K, oracle.quantize(x), want_sums=True)
+        scratch = torch.empty(8 * (K // 32) * 36, dtype=torch.uint8, device=dev)
+        before = {M: capi.gemv(FMT_Q4_K, w, q8, M, N, K).clone() for M in (4, 5, 6, 8)}
+        before_f32 = capi.gemv_f32(FMT_Q4_K, w, xd, 8, N, K, q8_scratch=scratch).clone()
+        assert capi.gemv_describe(FMT_Q4_K, 5, N, K).kernel == 3
+        plane = capi.attach_batch_plane(FMT_Q4_K, w, N, K)
+        try:
+            for M in (4, 5, 6, 8):
+                y = capi.gemv(FMT_Q4_K, w, q8, M, N, K)
+                sync()
+                assert torch.equal(y, before[M]), (N, K, M)
+                assert rel_err(y.cpu().numpy()[:, rows], exp[:M]) <= TOL[FMT_Q4_K] * 1e-2
+            y = capi.gemv_f32(FMT_Q4_K, w, xd, 8, N, K, q8_scratch=scratch)
+            sync()
+            assert torch.equal(y, before_f32)
+        finally:
+            capi.detach_batch_plane(w)
