@@ -637,6 +637,19 @@ def main():
                 "steps": sub.steps, "workload": "bench.py --workload decode"}
         except Exception as e:  # noqa: BLE001 - the headline figure must still be reported
             out["config"]["decode_step"] = {"error": str(e)[:200]}
+    if M == 1 and not args.no_decode and not args.no_extras:
+        # the same step for eight sequences at once (the matrix-unit kernels and, unless --no-batch-planes, the
+        # batch planes beside the prepared matrices)
+        torch.cuda.empty_cache()
+        try:
+            sub = argparse.Namespace(**vars(args))
+            sub.steps, sub.warmup, sub.batch = 24, 4, 8
+            d = bench_decode(sub, torch, capi, synth, dev)
+            out["config"]["decode_step_batch8"] = {
+                "tokens_per_s": d["value"], "ms_per_step": d["ms_per_step"], "batch_planes": d["config"]["batch_planes"],
+                "steps": sub.steps, "workload": "bench.py --workload decode --batch 8"}
+        except Exception as e:  # noqa: BLE001
+            out["config"]["decode_step_batch8"] = {"error": str(e)[:200]}
     if M == 1 and not args.no_extras:
         # the other configurations of the baseline, short runs of their own workloads, each with
         # its own roofline fraction: the prefill GEMM (int8 matrix-unit peak) and the MoE expert
