@@ -74,7 +74,8 @@ void llam_ql_set_batch_tile_rows(int tile_rows);
  * Results are bit-identical to the matrix-unit kernels without a plane.  The reference's packed
  * matrix is int8 in operand order to begin with; here that is the optional copy, and
  * llam_ql_gemv_describe and the block-sum hooks describe the launch without one.
- *   llam_ql_batch_plane_bytes: size of the plane, 0 if the format or shape has none.
+ *   llam_ql_batch_plane_bytes: size of the plane, 0 if the format or shape has none (Q4_K: also
+ *     while llam_ql_set_gemv_tuning overrides are in force, which keep batches off the matrix unit).
  *   llam_ql_build_batch_plane: fills d_plane (16-byte aligned) from the prepared matrix.
  *   llam_ql_attach_batch_plane: d_plane != NULL attaches it to d_prepared (fmt, N, K as built),
  *     NULL detaches (fmt, N, K ignored).  Detach before either buffer is freed.  Thread-safe;
