@@ -205,6 +205,10 @@ def bench_gemv(args, torch, capi, synth, dev):
         for N, K in ((FFN, HIDDEN), (HIDDEN, FFN), (QDIM, HIDDEN), (HIDDEN, QDIM), (KVDIM, HIDDEN)):
             nmat = max(2, min(8, int(600e6 // synth.gemv_bytes(fmt, N, K, 1)) + 1))
             mats = [capi.prepare_weights(fmt, synth.weights_torch(fmt, N, K, 70 + i, dev), N, K) for i in range(nmat)]
+            # batches of 5..8: with the matrices' batch planes where the shape has them (--no-batch-planes: without)
+            planes = []
+            if M >= 5 and N >= 4096 and not args.no_batch_planes and capi.batch_plane_bytes(fmt, N, K) > 0:
+                planes = [capi.attach_batch_plane(fmt, w, N, K) for w in mats]
             x = torch.randn(M, K, device=dev)
             q8 = capi.quantize_q8_1(x)
             y = torch.empty(M, N, device=dev)
@@ -214,7 +218,11 @@ def bench_gemv(args, torch, capi, synth, dev):
             b = synth.gemv_bytes(fmt, N, K, M)
             rows.append({"fmt": names[fmt], "N": N, "K": K, "M": M, "us": round(us, 2),
                          "GBps": round(b / (us * 1e-6) / 1e9, 1), "frac": round(b / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
-            del mats
+            if planes:
+                rows[-1]["batch_plane"] = True
+                for w in mats:
+                    capi.detach_batch_plane(w)
+            del mats, planes
     head = rows[0]
     return _common(args, "GEMV effective GB/s per shape", head["GBps"], "GB/s", round(head["us"] * 1e-3, 5), "int8",
                    {"workload": "single decode GEMVs, batch %d, all formats x layer shapes" % M, "shapes": rows},
