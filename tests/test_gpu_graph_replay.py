@@ -82,3 +82,53 @@ def test_decode_step_graph_replays_match_eager(capi, dev):
             capi.gemv(FMT_Q4_K, wo, q8o, 1, d_model, d_model)
             torch.cuda.synchronize()
     assert np.isfinite(y.cpu().numpy()).all()
+
+
+def test_batch_plane_launches_replay(capi, dev):
+    """Batches of eight rows on matrices with batch planes attached, captured once: the plane is looked up when the
+    launch is recorded, every replay equals the eager result, and detaching afterwards does not disturb the graph
+    (it keeps the plane it was given; the buffers stay alive here)."""
+    M, H, F = 8, 2048, 4096
+    mk = lambda fmt, N, K, seed: capi.prepare_weights(
+        fmt, torch.from_numpy(synth.weights_numpy(fmt, N, K, seed).reshape(-1)).to(dev), N, K)
+    wu, wd = mk(FMT_Q4_K, F, H, 11), mk(FMT_Q6_K, F, H, 12)
+    planes = [capi.attach_batch_plane(FMT_Q4_K, wu, F, H), capi.attach_batch_plane(FMT_Q6_K, wd, F, H)]
+    assert all(p is not None for p in planes)
+    x = torch.empty(M, H, device=dev)
+    q8 = torch.empty(M * (H // 32) * 36, dtype=torch.uint8, device=dev)
+    a, b = torch.empty(M, F, device=dev), torch.empty(M, F, device=dev)
+
+    def step(stream):
+        s = stream.cuda_stream
+        capi.quantize_q8_1(x, out=q8, stream=s)
+        capi.gemv(FMT_Q4_K, wu, q8, M, F, H, out=a, stream=s)
+        capi.gemv(FMT_Q6_K, wd, q8, M, F, H, out=b, stream=s)
+
+    inputs = [torch.from_numpy(synth.activations_numpy(M, H, 200 + i)).to(dev) for i in range(3)]
+    stream = torch.cuda.Stream()
+    eager = []
+    try:
+        with torch.cuda.stream(stream):
+            for inp in inputs:
+                x.copy_(inp)
+                step(stream)
+                stream.synchronize()
+                eager.append((a.clone(), b.clone()))
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                step(stream)
+        torch.cuda.synchronize()
+    finally:
+        capi.detach_batch_plane(wu)
+        capi.detach_batch_plane(wd)
+    for rep in range(2):
+        for i, inp in enumerate(inputs):
+            x.copy_(inp)
+            a.fill_(float("nan"))
+            b.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(a, eager[i][0]) and torch.equal(b, eager[i][1]), (rep, i)
+            capi.gemv(FMT_Q6_K, wd, q8, M, F, H)   # eager work between the replays, now without a plane
+            torch.cuda.synchronize()
