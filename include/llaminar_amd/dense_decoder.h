@@ -58,6 +58,9 @@ typedef struct
     uint8_t fmt_q, fmt_k, fmt_v, fmt_o, fmt_gate, fmt_up, fmt_down;
     const float *attn_norm; /* [hidden] */
     const float *ffn_norm;  /* [hidden] */
+    /* optional batch planes of the seven matrices (llam_ql_build_batch_plane), read by batches of
+     * 5..8 sequences; NULL = none */
+    const void *plane_q, *plane_k, *plane_v, *plane_o, *plane_gate, *plane_up, *plane_down;
 } llam_decoder_layer;
 
 typedef struct
@@ -66,6 +69,7 @@ typedef struct
     const float *final_norm; /* [hidden] */
     const void *lm_head;     /* prepared weights [vocab x hidden] */
     uint8_t fmt_lm_head;
+    const void *plane_lm_head; /* optional batch plane of lm_head, or NULL */
 } llam_decoder_globals;
 
 /* Allocates the activation buffers, the KV caches (2 * n_layers * batch * n_kv * ctx_cap *
@@ -96,8 +100,9 @@ bool llam_decoder_advance(void *dec, int n);
 
 /* Device buffers, for filling caches, reading results and parity checks:
  *   "ids" int32[batch], "pos" int32[batch], "logits" fp32[batch][vocab], "x" fp32[batch][hidden]
- *   (the residual stream as the last step left it, before the final add of "delta"),
- *   "delta" fp32[batch][hidden], "kcache" and "vcache" fp16[batch][n_kv][ctx_cap * head_dim] of `layer`,
+ *   (the residual stream as the last step left it: every layer's outputs added, the input of the
+ *   final norm; before the first step, the buffer the embedding will fill),
+ *   "kcache" and "vcache" fp16[batch][n_kv][ctx_cap * head_dim] of `layer`,
  *   each (sequence, head) slice in the tiles llam_dec_rope_kv_append documents. */
 void *llam_decoder_buffer(void *dec, const char *name, int layer);
 

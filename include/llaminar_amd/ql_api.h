@@ -56,52 +56,30 @@ int llam_ql_abi_version(void);
  * kernel would be used.  Values <= 0 restore the built-in choice.  Not thread-safe. */
 void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll);
 void llam_ql_reset_gemv_tuning(void);
-/* The same for the matrix-unit kernels of batches 5..8: rows of weight per tile, 16..32;
- * any other value restores the built-in choice.  No counterpart in the reference. */
-void llam_ql_set_batch_tile_rows(int tile_rows);
-
 /* Batch plane of a prepared matrix: an optional second copy for callers that decode batches of
  * 5..8 rows, laid out as the matrix unit takes its operands (rows in groups of four, a 128-byte
  * line per group and block), separate from the prepared matrix.
  *   Q6_K: the weights requantised to int8 once (the 8.8 requantisation of
  *     packWeightsCPUNativeVNNI's Q6_K branch, SIMDHelpers.h:12023-12204, which the decode
  *     kernels otherwise repeat on every launch) beside their fp16 block scales, 272 bytes per
- *     super-block and row; rows of eight super-blocks and more.  While attached, every batch
- *     of 5..8 rows of that matrix runs on the matrix-unit kernel and reads the plane.
+ *     super-block and row; rows of eight super-blocks and more.  A batch of 5..8 rows of that
+ *     matrix launched with its plane runs on the matrix-unit plane kernel.
  *   Q4_K: the 144 bytes of every super-block regrouped, not changed; shapes whose batches of
  *     5..8 go to the matrix-unit kernel (4096 rows and more).  The kernel then finds a lane's
  *     operands at one address and needs no LDS bounce.
  * Results are bit-identical to the matrix-unit kernels without a plane.  The reference's packed
- * matrix is int8 in operand order to begin with; here that is the optional copy, and
- * llam_ql_gemv_describe and the block-sum hooks describe the launch without one.
+ * matrix is int8 in operand order to begin with; here that is the optional copy.
  *   llam_ql_batch_plane_bytes: size of the plane, 0 if the format or shape has none (Q4_K: also
  *     while llam_ql_set_gemv_tuning overrides are in force, which keep batches off the matrix unit).
  *   llam_ql_build_batch_plane: fills d_plane (16-byte aligned) from the prepared matrix.
- *   llam_ql_attach_batch_plane: d_plane != NULL attaches it to d_prepared (fmt, N, K as built),
- *     NULL detaches (fmt, N, K ignored).  Detach before either buffer is freed.  Thread-safe;
- *     launches in flight keep reading the plane they were given. */
+ * The caller owns the plane and hands it to every launch that may use it: the d_plane argument
+ * of llam_ql_gemv_plane, llam_ql_gemv_swiglu_f32 and llam_ql_gemv_block_sums, the d_plane field
+ * of llam_ql_proj.  NULL means "no plane" everywhere; a plane is only read by batches of 5..8
+ * rows.  The library keeps no record of planes: a plane handed to a launch must be the one built
+ * from the d_w of the same launch, and both must stay alive until the launch has finished. */
 size_t llam_ql_batch_plane_bytes(uint8_t fmt, int N, int K);
 bool llam_ql_build_batch_plane(uint8_t fmt, const void* d_prepared, void* d_plane, int N, int K,
                                int device_id, void* stream);
-bool llam_ql_attach_batch_plane(uint8_t fmt, const void* d_prepared, const void* d_plane, int N, int K);
-
-/* Read-only probe for measurements: streams the N * (K/256) * 144 bytes of a Q4_K-sized
- * buffer once and computes nothing, in the order a decode GEMV would read them.  No
- * counterpart in the reference.
- *   ROWS_*: the quad-lane kernel's loads (4 lanes per super-block, 3 x 16 bytes per lane and
- *     step), N rows shared by ceil(N / rows_per_wave) wavefronts, each with its rows
- *     contiguous or dealt round robin; depth = steps in flight per wavefront (1, 2, 4);
- *     `workgroups` is ignored.
- *   STREAM_*: 1 KB per load instruction, `workgroups` workgroups, a region per wavefront or
- *     grid-stride; depth = loads in flight per lane (3, 6, 9); rows_per_wave is ignored.
- * d_sink: one int the kernels may write. */
-#define LLAM_QL_PROBE_ROWS_CONTIGUOUS 0
-#define LLAM_QL_PROBE_ROWS_ROUND_ROBIN 1
-#define LLAM_QL_PROBE_STREAM_REGION 2
-#define LLAM_QL_PROBE_STREAM_GRID_STRIDE 3
-bool llam_ql_read_probe(const void *d_buf, int N, int K, int pattern, int rows_per_wave,
-                        int waves_per_wg, int depth, int workgroups, int *d_sink, int device_id,
-                        void *stream);
 
 /* ---- P1: activation quantiser --------------------------------------------------
  * fp32 [M x K] (row stride K) -> llam_block_q8_1 [M x ceil(K/32)].  d_x 16-byte aligned when
@@ -141,6 +119,10 @@ bool llam_ql_prepare_weights(uint8_t fmt, const void *d_gguf, void *d_prepared,
  * (ROCmGemvKernel_native_VNNI.hip:5228). */
 bool llam_ql_gemv(uint8_t fmt, const void *d_w, const void *d_q8, float *d_y,
                   int M, int N, int K, int ldy, int device_id, void *stream);
+/* The same with the matrix's batch plane (llam_ql_build_batch_plane; NULL: llam_ql_gemv): batches
+ * of 5..8 rows read the plane instead of d_w, smaller batches ignore it. */
+bool llam_ql_gemv_plane(uint8_t fmt, const void *d_w, const void *d_plane, const void *d_q8,
+                        float *d_y, int M, int N, int K, int ldy, int device_id, void *stream);
 
 /* One projection of a fused launch (reference: FusedGemvDesc,
  * CPUNativeVNNIGemv.h:3782-3881 / TensorProjectionDesc, TensorKernels.h:601). */
@@ -151,6 +133,7 @@ typedef struct
     int N;
     int ldy;
     uint8_t fmt;
+    const void *d_plane; /* the matrix's batch plane (llam_ql_build_batch_plane), or NULL */
 } llam_ql_proj;
 
 /* Several projections of ONE quantised input in one launch (QKV, gate+up,
@@ -193,8 +176,8 @@ bool llam_ql_gemv_f32_static(uint8_t fmt, const void *d_w, const float *d_x, int
 /* d_y = (silu(gate) * up) @ W^T for fp32 gate/up rows of ld_gu floats: the bits of
  * llam_ql_swiglu_quantize followed by llam_ql_gemv, in one launch.  Replaces
  * multiply_tensor_with_fused_swiglu (CPUNativeVNNIGemmKernel.h:325-431: compute_swiglu,
- * then the quantising GEMV).  d_q8_scratch as above. */
-bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const float *d_gate,
+ * then the quantising GEMV).  d_q8_scratch as above; d_plane: the matrix's batch plane or NULL. */
+bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const void *d_plane, const float *d_gate,
                              const float *d_up, int ld_gu, float *d_y, int M, int N, int K,
                              int ldy, void *d_q8_scratch, int device_id, void *stream);
 
@@ -204,8 +187,10 @@ bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const float *d_gate,
  * kernel, K slices, batch splits -- and runs the chosen kernel's block-sum variant: the
  * same code compiled with the stores of the sums switched on and the fp32 output off.
  * (The reference exposes the same quantity only inside its kernels: int_acc in
- * CPUNativeVNNIGemv.h:417-487.)  M * nrows * (K/32) * 4 bytes must stay below 2 GiB. */
-bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,
+ * CPUNativeVNNIGemv.h:417-487.)  d_plane: the batch plane the launch to be checked would get, or
+ * NULL -- with a plane and a batch it serves, the plane kernel's block-sum variant runs.
+ * M * nrows * (K/32) * 4 bytes must stay below 2 GiB. */
+bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_plane, const void *d_q8,
                              int32_t *d_sums, int M, int N, int K, int row0,
                              int nrows, int device_id, void *stream);
 
@@ -228,15 +213,16 @@ bool llam_ql_gemv_accumulate(uint8_t fmt, const void *d_w, const void *d_q8, flo
  * with the bits of llam_dec_rmsnorm_q8_1 followed by llam_ql_gemv_fused (the fused form of
  * CPURMSNormKernelT<FP32>::apply_with_residual_add, CPURMSNormKernelT.h:300-322, in front of the
  * activation quantiser).  Rows of d_x, d_delta and d_x_out are K floats apart.  Served where
- * llam_ql_gemv_fused_rmsnorm_supported says so (M <= 4, rows the quad-lane kernel takes);
- * elsewhere the call fails and the norm and the projections run as two calls. */
+ * llam_ql_gemv_fused_rmsnorm_supported says so (single rows, M == 1, of shapes the quad-lane
+ * kernel takes); elsewhere the call fails and the norm and the projections run as two calls.
+ * d_x_out must not overlap d_x or d_delta. */
 bool llam_ql_gemv_fused_rmsnorm_supported(const llam_ql_proj *projs, int num, int M, int K);
 bool llam_ql_gemv_fused_rmsnorm(const llam_ql_proj *projs, int num, const float *d_x,
                                 const float *d_delta, const float *d_gamma, float eps,
                                 float *d_x_out, int M, int K, int device_id, void *stream);
 
-/* What llam_ql_gemv does with a shape: which kernel runs, how the batch and the row are
- * split.  For tests, tuning and the operator's decode-equivalence guard; the launcher
+/* What llam_ql_gemv (has_plane == 0) or a launch that brings the matrix's batch plane
+ * (has_plane != 0) does with a shape: which kernel runs, how the batch and the row are split.  For tests, tuning and the operator's decode-equivalence guard; the launcher
  * executes exactly this plan.  (Reference: the dispatch tables behind
  * rocmGemv_native_vnni_fp32, ROCmNativeVNNIDecodeDispatchGenerated.inc.) */
 #define LLAM_QL_KERNEL_GENERIC 0 /* rows shorter than 5 super-blocks */
@@ -251,7 +237,7 @@ typedef struct
     int rows_per_wave;
     int decode_equivalent; /* 1: every row of the M-row call has the bits of its own M = 1 call */
 } llam_ql_gemv_plan;
-bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int device_id,
+bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int has_plane, int device_id,
                            llam_ql_gemv_plan *out);
 
 /* ---- P3: prefill GEMM (any M) -------------------------------------------------------
@@ -402,6 +388,16 @@ bool llam_ql_moe_down_grouped(uint8_t fmt, const llam_ql_expert *d_experts, int 
  * toward zero; NaN, negative and out-of-range values become -1, which every launch skips. */
 bool llam_ql_moe_ids_from_f32(const float *d_indices, int32_t *d_ids, int n, int device_id,
                               void *stream);
+
+/* The other direction, and what else IMoEKernel::decodeRouteSelect publishes beside the runtime
+ * top-k state (src/v2/kernels/IMoEKernel.h:245-258, write_legacy_outputs / update_runtime_histogram;
+ * src/v2/kernels/rocm/moe/ROCmMoEKernel.cpp:2956-3019): for every token t and slot s < top_k,
+ *   d_indices_f32[t*top_k+s] = float(d_ids[t*slot_stride+s]),  d_weights_f32[t*top_k+s] = d_weights[t*slot_stride+s],
+ *   d_histogram[id] += 1 for ids inside [0, n_experts)   (uint64 counts, integer atomics).
+ * Each of the three outputs may be NULL. */
+bool llam_ql_moe_publish_routing(const int32_t *d_ids, const float *d_weights, int n_tokens, int top_k,
+                                 int slot_stride, float *d_indices_f32, float *d_weights_f32,
+                                 uint64_t *d_histogram, int n_experts, int device_id, void *stream);
 
 /* Shared expert: d_out[t,:] += g_t * d_shared[t,:] with
  * g_t = sigmoid(dot(d_gate_inp, d_hidden[t,:])), or g_t = 1 when d_gate_inp is

@@ -145,10 +145,10 @@ namespace llaminar_amd
         bool hasWeights() const { return valid_ && (d_weights_ || host_gguf_); }
         void releaseWeights();
         size_t packedWeightBytes() const;
-        // Optional int8 batch plane of a Q6_K matrix (ql_api.h, llam_ql_build_batch_plane): built
-        // once, owned by the operator and attached to its prepared weights, so that batches of
-        // 5..8 rows read ready-made int8 weights; dropped with the weights (release, detach,
-        // attach).  The reference's packed matrix is int8 to begin with and has no such switch.
+        // Optional batch plane of the matrix (ql_api.h, llam_ql_build_batch_plane): built once,
+        // owned by the operator and handed to every launch it makes, so that batches of 5..8
+        // rows read weights laid out for the matrix unit (Q6_K: ready-made int8); dropped with
+        // the weights (release, detach, attach).  The reference's packed matrix is int8 to begin with and has no such switch.
         // False (with the reason in last_error) where the format or shape has no plane.
         bool enableBatchPlane();
         bool hasBatchPlane() const { return d_plane_ != nullptr; }
@@ -251,7 +251,7 @@ namespace llaminar_amd
         const void *host_gguf_ = nullptr;
         const void *d_weights_ = nullptr;
         void *d_owned_ = nullptr;
-        void *d_plane_ = nullptr; // the batch plane attached to d_weights_
+        void *d_plane_ = nullptr; // the batch plane built from d_weights_
         void drop_plane_locked();
         std::shared_ptr<void> lifetime_owner_;
         void *stream_ = nullptr;

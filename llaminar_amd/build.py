@@ -221,8 +221,17 @@ def _drop_resource_remarks(lines: list[str]) -> list[str]:
     return out
 
 
-def _compile(src: Path) -> Path:
+def _headers_mtime() -> float:
+    files = list(CSRC.glob("*.h")) + list((ROOT / "include" / "llaminar_amd").glob("*.h*"))
+    return max(f.stat().st_mtime for f in files)
+
+
+def _compile(src: Path, force: bool = True) -> Path:
     obj = OBJDIR / (src.stem + ".o")
+    # without force an object newer than its source and every header is kept (it passed the checks below
+    # when it was made)
+    if not force and obj.exists() and obj.stat().st_mtime >= max(src.stat().st_mtime, _headers_mtime()):
+        return obj
     # -save-temps leaves the device assembly beside the object file for check_inflight_registers
     cmd = [hipcc(), *HIP_FLAGS, RESOURCE_FLAG, "-save-temps=obj", "-c", str(src), "-o", str(obj)]
     if src.suffix == ".cpp":
@@ -253,7 +262,7 @@ def build(force: bool = True, verbose: bool = True) -> Path:
     if verbose:
         print(f"[llaminar_amd.build] hipcc {ARCH}: {len(srcs)} sources", flush=True)
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
-        objs = list(pool.map(_compile, srcs))
+        objs = list(pool.map(lambda src: _compile(src, force), srcs))
     cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
@@ -265,4 +274,4 @@ def build(force: bool = True, verbose: bool = True) -> Path:
 
 
 if __name__ == "__main__":
-    build(force=True)
+    build(force="--incremental" not in sys.argv)

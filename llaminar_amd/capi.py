@@ -27,7 +27,8 @@ class QLError(RuntimeError):
 
 
 class Proj(ctypes.Structure):
-    _fields_ = [("d_w", c_void_p), ("d_y", c_void_p), ("N", c_int), ("ldy", c_int), ("fmt", c_uint8)]
+    _fields_ = [("d_w", c_void_p), ("d_y", c_void_p), ("N", c_int), ("ldy", c_int), ("fmt", c_uint8),
+                ("d_plane", c_void_p)]
 
 
 class GemvPlan(ctypes.Structure):
@@ -48,15 +49,14 @@ SIGNATURES = {
     "llam_ql_abi_version": (c_int, []),
     "llam_ql_set_gemv_tuning": (None, [c_int, c_int]),
     "llam_ql_reset_gemv_tuning": (None, []),
-    "llam_ql_set_batch_tile_rows": (None, [c_int]),
     "llam_ql_batch_plane_bytes": (c_size_t, [c_uint8, c_int, c_int]),
     "llam_ql_build_batch_plane": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
-    "llam_ql_attach_batch_plane": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int]),
-    "llam_ql_read_probe": (c_bool, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_quantize_q8_1": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_prepared_bytes": (c_size_t, [c_uint8, c_int, c_int]),
     "llam_ql_prepare_weights": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_gemv": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv_plane": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                    c_void_p]),
     "llam_ql_gemv_fused": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_gemv_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                   c_int, c_void_p]),
@@ -69,11 +69,11 @@ SIGNATURES = {
                                             c_int, c_int, c_void_p]),
     "llam_ql_gemv_fused_f32": (c_bool, [POINTER(Proj), c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_int,
                                         c_void_p]),
-    "llam_ql_gemv_swiglu_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
-                                         c_int, c_void_p, c_int, c_void_p]),
-    "llam_ql_gemv_block_sums": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                         c_int, c_void_p]),
-    "llam_ql_gemv_describe": (c_bool, [c_uint8, c_int, c_int, c_int, c_int, POINTER(GemvPlan)]),
+    "llam_ql_gemv_swiglu_f32": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
+                                         c_int, c_int, c_void_p, c_int, c_void_p]),
+    "llam_ql_gemv_block_sums": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                         c_int, c_int, c_void_p]),
+    "llam_ql_gemv_describe": (c_bool, [c_uint8, c_int, c_int, c_int, c_int, c_int, POINTER(GemvPlan)]),
     "llam_ql_gemm": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_gemm_block_sums": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                          c_int, c_void_p]),
@@ -96,6 +96,8 @@ SIGNATURES = {
     "llam_ql_moe_down_grouped": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_ids_from_f32": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "llam_ql_moe_publish_routing": (c_bool, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                             c_int, c_int, c_void_p]),
     "llam_ql_shared_expert_add": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_shared_expert_gate": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_gather_rows": (c_bool, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
@@ -217,10 +219,11 @@ def batch_plane_bytes(fmt: int, N: int, K: int) -> int:
     return int(load().llam_ql_batch_plane_bytes(fmt, N, K))
 
 
-def attach_batch_plane(fmt: int, w, N: int, K: int, stream=None):
-    """Builds the batch plane of the prepared matrix `w` and attaches it: batches of 5..8 rows then read the
-    ready-made int8 weights.  Returns the plane (keep it alive as long as `w` is used, then detach_batch_plane),
-    or None where the format or shape has no plane."""
+def build_batch_plane(fmt: int, w, N: int, K: int, stream=None):
+    """Builds the batch plane of the prepared matrix `w`: hand it to the launches of that matrix (`plane=`)
+    and batches of 5..8 rows read weights laid out for the matrix unit.  Returns the plane, finished (the
+    building stream is waited for, so a launch on any stream may read it), or None where the format or shape
+    has no plane.  The caller keeps it alive as long as launches use it."""
     import torch
 
     nbytes = batch_plane_bytes(fmt, N, K)
@@ -228,29 +231,35 @@ def attach_batch_plane(fmt: int, w, N: int, K: int, stream=None):
         return None
     plane = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
     _check(load().llam_ql_build_batch_plane(fmt, _ptr(w), _ptr(plane), N, K, _dev(w), _stream(stream)), "build_batch_plane")
-    _check(load().llam_ql_attach_batch_plane(fmt, _ptr(w), _ptr(plane), N, K), "attach_batch_plane")
+    (stream if stream is not None and not isinstance(stream, int) else torch.cuda.current_stream()).synchronize()
     return plane
 
 
-def detach_batch_plane(w):
-    _check(load().llam_ql_attach_batch_plane(0, _ptr(w), None, 0, 0), "attach_batch_plane")
+def _proj(p):
+    """(fmt, w, out[M,N]) or (fmt, w, out[M,N], plane) -> Proj."""
+    fmt, w, out = p[0], p[1], p[2]
+    plane = p[3] if len(p) > 3 else None
+    return Proj(_ptr(w), _ptr(out), out.shape[-1], out.stride(0) if out.dim() == 2 else out.shape[-1], fmt, _ptr(plane))
 
 
-def gemv(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None):
+def gemv(fmt: int, w, q8, M: int, N: int, K: int, out=None, stream=None, plane=None):
+    """out[M,N] from Q8_1 activations; `plane`: the matrix's batch plane (build_batch_plane) or None."""
     import torch
 
     if out is None:
         out = torch.empty(M, N, dtype=torch.float32, device=w.device)
-    _check(load().llam_ql_gemv(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, out.stride(0) if out.dim() == 2 else N,
-                               _dev(w), _stream(stream)), "gemv")
+    ldy = out.stride(0) if out.dim() == 2 else N
+    if plane is None:
+        _check(load().llam_ql_gemv(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, ldy, _dev(w), _stream(stream)), "gemv")
+    else:
+        _check(load().llam_ql_gemv_plane(fmt, _ptr(w), _ptr(plane), _ptr(q8), _ptr(out), M, N, K, ldy, _dev(w),
+                                         _stream(stream)), "gemv_plane")
     return out
 
 
 def gemv_fused(projs, q8, M: int, K: int, stream=None):
-    """projs: list of (fmt, w, out[M,N]) sharing one quantised input."""
-    arr = (Proj * len(projs))()
-    for i, (fmt, w, out) in enumerate(projs):
-        arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], out.stride(0) if out.dim() == 2 else out.shape[-1], fmt)
+    """projs: list of (fmt, w, out[M,N]) or (fmt, w, out[M,N], plane) sharing one quantised input."""
+    arr = _proj_array(projs)
     dev = _dev(q8)
     _check(load().llam_ql_gemv_fused(arr, len(projs), _ptr(q8), M, K, dev, _stream(stream)), "gemv_fused")
 
@@ -281,10 +290,8 @@ def gemv_f32_static(fmt: int, w, x, M: int, N: int, K: int, out, stream=None):
 
 
 def gemv_fused_f32(projs, x, M: int, K: int, q8_scratch=None, stream=None):
-    """projs: list of (fmt, w, out[M,N]) sharing the fp32 input x[M,K]."""
-    arr = (Proj * len(projs))()
-    for i, (fmt, w, out) in enumerate(projs):
-        arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], _ld(out), fmt)
+    """projs: list of (fmt, w, out[M,N]) or (fmt, w, out[M,N], plane) sharing the fp32 input x[M,K]."""
+    arr = _proj_array(projs)
     _check(load().llam_ql_gemv_fused_f32(arr, len(projs), _ptr(x), _ld(x), M, K, _ptr(q8_scratch), _dev(x),
                                          _stream(stream)), "gemv_fused_f32")
 
@@ -302,8 +309,8 @@ def gemv_accumulate(fmt: int, w, q8, M: int, N: int, K: int, out, stream=None):
 
 def _proj_array(projs):
     arr = (Proj * len(projs))()
-    for i, (fmt, w, out) in enumerate(projs):
-        arr[i] = Proj(_ptr(w), _ptr(out), out.shape[-1], _ld(out), fmt)
+    for i, p in enumerate(projs):
+        arr[i] = _proj(p)
     return arr
 
 
@@ -318,31 +325,33 @@ def gemv_fused_rmsnorm(projs, x, delta, gamma, eps: float, x_out, M: int, K: int
                                              _ptr(x_out), M, K, _dev(x), _stream(stream)), "gemv_fused_rmsnorm")
 
 
-def gemv_swiglu_f32(fmt: int, w, gate, up, M: int, N: int, K: int, out=None, q8_scratch=None, stream=None):
+def gemv_swiglu_f32(fmt: int, w, gate, up, M: int, N: int, K: int, out=None, q8_scratch=None, stream=None,
+                    plane=None):
     """out[M,N] = (silu(gate) * up)[M,K] @ W^T."""
     import torch
 
     if out is None:
         out = torch.empty(M, N, dtype=torch.float32, device=w.device)
     assert _ld(gate) == _ld(up)
-    _check(load().llam_ql_gemv_swiglu_f32(fmt, _ptr(w), _ptr(gate), _ptr(up), _ld(gate), _ptr(out), M, N, K, _ld(out),
+    _check(load().llam_ql_gemv_swiglu_f32(fmt, _ptr(w), _ptr(plane), _ptr(gate), _ptr(up), _ld(gate), _ptr(out), M, N, K, _ld(out),
                                           _ptr(q8_scratch), _dev(w), _stream(stream)), "gemv_swiglu_f32")
     return out
 
 
-def gemv_block_sums(fmt: int, w, q8, M: int, N: int, K: int, row0: int, nrows: int, stream=None):
+def gemv_block_sums(fmt: int, w, q8, M: int, N: int, K: int, row0: int, nrows: int, stream=None, plane=None):
+    """The exact int32 block sums of the kernel a launch with these arguments (plane included) runs."""
     import torch
 
     out = torch.empty(M, nrows, K // 32, dtype=torch.int32, device=w.device)
-    _check(load().llam_ql_gemv_block_sums(fmt, _ptr(w), _ptr(q8), _ptr(out), M, N, K, row0, nrows, _dev(w),
+    _check(load().llam_ql_gemv_block_sums(fmt, _ptr(w), _ptr(plane), _ptr(q8), _ptr(out), M, N, K, row0, nrows, _dev(w),
                                           _stream(stream)), "gemv_block_sums")
     return out
 
 
-def gemv_describe(fmt: int, M: int, N: int, K: int, device_id: int = 0) -> GemvPlan:
-    """The launch plan of llam_ql_gemv for a shape (no GPU work)."""
+def gemv_describe(fmt: int, M: int, N: int, K: int, device_id: int = 0, has_plane: bool = False) -> GemvPlan:
+    """The launch plan for a shape, without or with the matrix's batch plane (no GPU work)."""
     plan = GemvPlan()
-    _check(load().llam_ql_gemv_describe(fmt, M, N, K, device_id, ctypes.byref(plan)), "gemv_describe")
+    _check(load().llam_ql_gemv_describe(fmt, M, N, K, int(has_plane), device_id, ctypes.byref(plan)), "gemv_describe")
     return plan
 
 

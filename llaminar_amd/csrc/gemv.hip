@@ -6,29 +6,43 @@
 
 namespace llamql
 {
-    bool q4k_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                         int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
+    bool q4k_gemv_launch(const char *fn, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                         int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id,
+                         hipStream_t st)
     {
-        return gemv_launch<Q4KTraits>(fn, d_w, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
+        return gemv_launch<Q4KTraits>(fn, d_w, d_plane, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
     }
 
-    bool q6k_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                         int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
+    bool q6k_gemv_launch(const char *fn, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                         int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id,
+                         hipStream_t st)
     {
-        return gemv_launch<Q6KTraits>(fn, d_w, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
+        return gemv_launch<Q6KTraits>(fn, d_w, d_plane, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
     }
 
-    bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                          int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
+    bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                         int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id,
+                         hipStream_t st)
     {
-        return gemv_launch<IQ3STraits>(fn, d_w, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
+        return gemv_launch<IQ3STraits>(fn, d_w, d_plane, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
     }
 
     namespace
     {
         template <class F>
-        void describe(int M, int N, int K, int device_id, llam_ql_gemv_plan *out)
+        void describe(int M, int N, int K, bool has_plane, int device_id, llam_ql_gemv_plan *out)
         {
+            // a batch the caller's batch plane serves runs on the matrix-unit plane kernel whatever
+            // the plan for the matrix alone says
+            if (has_plane && batch_plane_usable<F>(M, N, K))
+            {
+                out->kernel = GEMV_KERNEL_MFMA;
+                out->m_first = M;
+                out->slice_sb = K / 256;
+                out->rows_per_wave = 0;
+                out->decode_equivalent = 0;
+                return;
+            }
             const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
             out->kernel = p.kernel;
             out->m_first = p.m_first;
@@ -38,13 +52,13 @@ namespace llamql
         }
     } // namespace
 
-    void gemv_describe(uint8_t fmt, int M, int N, int K, int device_id, llam_ql_gemv_plan *out)
+    void gemv_describe(uint8_t fmt, int M, int N, int K, bool has_plane, int device_id, llam_ql_gemv_plan *out)
     {
         switch (fmt)
         {
-        case LLAM_FMT_Q4_K: describe<Q4KTraits>(M, N, K, device_id, out); break;
-        case LLAM_FMT_Q6_K: describe<Q6KTraits>(M, N, K, device_id, out); break;
-        default: describe<IQ3STraits>(M, N, K, device_id, out); break;
+        case LLAM_FMT_Q4_K: describe<Q4KTraits>(M, N, K, has_plane, device_id, out); break;
+        case LLAM_FMT_Q6_K: describe<Q6KTraits>(M, N, K, has_plane, device_id, out); break;
+        default: describe<IQ3STraits>(M, N, K, has_plane, device_id, out); break;
         }
     }
 
@@ -77,16 +91,16 @@ namespace llamql
         {
             // batches that go to the matrix-unit kernel launch one matrix at a time
             if constexpr (F::USE_MFMA_BATCH)
-                if (mfma_eligible<F>(M, projs[0].N, K) || batch_plane_for<F>(projs[0].d_w, M, projs[0].N, K))
-                    return gemv_mfma_launch<F>(fn, projs[0].d_w, src, projs[0].d_y, M, projs[0].N, K, projs[0].ldy,
-                                                device_id, st)
+                if (mfma_eligible<F>(M, projs[0].N, K) || batch_plane_for<F>(projs[0].d_plane, M, projs[0].N, K))
+                    return gemv_mfma_launch<F>(fn, projs[0].d_w, batch_plane_for<F>(projs[0].d_plane, M, projs[0].N, K), src,
+                                                projs[0].d_y, M, projs[0].N, K, projs[0].ldy, device_id, st)
                                ? 1
                                : -1;
             QuadProj pr[QUAD_MAX_PROJ];
             int n = 0;
             while (n < num && n < QUAD_MAX_PROJ && projs[n].fmt == projs[0].fmt &&
                    quad_eligible<F>(M, projs[n].N, K) && !mfma_eligible<F>(M, projs[n].N, K) &&
-                   !batch_plane_for<F>(projs[n].d_w, M, projs[n].N, K))
+                   !batch_plane_for<F>(projs[n].d_plane, M, projs[n].N, K))
             {
                 pr[n] = QuadProj{projs[n].d_w, projs[n].d_y, projs[n].N, projs[n].ldy};
                 ++n;
@@ -99,7 +113,7 @@ namespace llamql
                     int nb = 0;
                     while (n + nb < num && n + nb < QUAD_MAX_PROJ && projs[n + nb].fmt == Other<F>::fmt &&
                            quad_eligible<G>(M, projs[n + nb].N, K) && !mfma_eligible<G>(M, projs[n + nb].N, K) &&
-                           !batch_plane_for<G>(projs[n + nb].d_w, M, projs[n + nb].N, K))
+                           !batch_plane_for<G>(projs[n + nb].d_plane, M, projs[n + nb].N, K))
                     {
                         pr[n + nb] = QuadProj{projs[n + nb].d_w, projs[n + nb].d_y, projs[n + nb].N, projs[n + nb].ldy};
                         ++nb;
@@ -138,8 +152,7 @@ namespace llamql
                                int ldy, int device_id, hipStream_t st, bool query)
         {
             const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
-            // (a batch that has the matrix's batch plane to read goes to the matrix-unit kernel)
-            if (p.kernel != GEMV_KERNEL_QUAD || p.m_first < M || batch_plane_for<F>(d_w, M, N, K))
+            if (p.kernel != GEMV_KERNEL_QUAD || p.m_first < M)
                 return query ? false : fail(fn, "M=%d N=%d K=%d: not a single quad-lane launch", M, N, K);
             const QuadProj pr{d_w, d_y, N, ldy};
             return gemv_quad_multi<F>(fn, &pr, 1, act_source_q8(d_q8), M, K, device_id, st, nullptr, 0, 0,
@@ -295,21 +308,4 @@ extern "C" bool llam_ql_build_batch_plane(uint8_t fmt, const void *d_prepared, v
         hipLaunchKernelGGL(build_q4k_plane_kernel, dim3((unsigned)grid), dim3(256), 0, as_stream(stream),
                            static_cast<const uint8_t *>(d_prepared), static_cast<uint8_t *>(d_plane), (long)N, nsb);
     return launched(fn);
-}
-
-extern "C" bool llam_ql_attach_batch_plane(uint8_t fmt, const void *d_prepared, const void *d_plane, int N, int K)
-{
-    using namespace llamql;
-    static const char *fn = "llam_ql_attach_batch_plane";
-    if (!d_prepared)
-        return fail(fn, "null d_prepared");
-    if (d_plane)
-    {
-        if (!batch_plane_shape(fmt, N, K))
-            return fail(fn, "no batch plane for format %d, N=%d, K=%d", (int)fmt, N, K);
-        if (!aligned16(d_plane))
-            return fail(fn, "d_plane must be 16-byte aligned");
-    }
-    batch_plane_attach(fmt, d_prepared, d_plane, N, K);
-    return true;
 }

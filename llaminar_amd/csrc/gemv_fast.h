@@ -464,16 +464,17 @@ namespace llamql
         hipLaunchKernelGGL((gemv_mfma_q4k_kernel<SRC, DUMP, PLANE>), grid, block, lds, st, a);
     }
 
-    inline bool gemv_mfma_q4k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
-                                     int K, int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr,
-                                     int row0 = 0, int nrows = 0)
+    // d_plane: the matrix's batch plane (q4k_plane_bytes) or null; with one, the kernel reads it
+    // instead of the prepared matrix, the block-sum variant included.
+    inline bool gemv_mfma_q4k_launch(const char *fn, const void *d_w, const void *d_plane, const ActSource &src,
+                                     float *d_y, int M, int N, int K, int ldy, int device_id, hipStream_t st,
+                                     int32_t *d_sums = nullptr, int row0 = 0, int nrows = 0)
     {
         const int SB = K / 256;
         const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id), d_sums ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES);
         MfmaArgs a;
         a.w = static_cast<const uint8_t *>(d_w);
-        // the matrix's batch plane if one is attached (the block-sum variant reads the prepared matrix)
-        a.plane = d_sums ? nullptr : batch_plane_of(LLAM_FMT_Q4_K, d_w, N, K);
+        a.plane = static_cast<const uint8_t *>(d_plane);
         a.q8 = static_cast<const uint32_t *>(src.q8);
         a.x = src.x;
         a.x2 = src.x2;
@@ -494,7 +495,10 @@ namespace llamql
         {
             if (src.kind != ACT_SRC_Q8)
                 return fail(fn, "block sums are dumped on Q8_1 input");
-            gemv_mfma_q4k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            if (a.plane)
+                gemv_mfma_q4k_launch_src<QUAD_SRC_Q8, true, true>(grid, block, lds, st, a);
+            else
+                gemv_mfma_q4k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
             return launched(fn);
         }
         if (a.plane)
@@ -524,23 +528,24 @@ namespace llamql
         hipLaunchKernelGGL((gemv_mfma_q6k_kernel<SRC, DUMP>), grid, block, lds, st, a);
     }
 
-    template <int SRC>
+    template <int SRC, bool DUMP = false>
     void gemv_mfma_q6k_plane_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const Mfma6Args &a)
     {
         static LdsGrant grant;
-        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q6k_plane_kernel<SRC>), QUAD_MAX_LDS);
-        hipLaunchKernelGGL((gemv_mfma_q6k_plane_kernel<SRC>), grid, block, lds, st, a);
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q6k_plane_kernel<SRC, DUMP>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_mfma_q6k_plane_kernel<SRC, DUMP>), grid, block, lds, st, a);
     }
 
-    inline bool gemv_mfma_q6k_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N,
-                                     int K, int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr,
-                                     int row0 = 0, int nrows = 0)
+    // d_plane: the matrix's batch plane (q6k_plane_bytes) or null; with one, the plane kernel runs,
+    // also as the block-sum variant.
+    inline bool gemv_mfma_q6k_launch(const char *fn, const void *d_w, const void *d_plane, const ActSource &src,
+                                     float *d_y, int M, int N, int K, int ldy, int device_id, hipStream_t st,
+                                     int32_t *d_sums = nullptr, int row0 = 0, int nrows = 0)
     {
         const int SB = K / 256;
-        // the matrix's batch plane if one is attached (the block-sum variant decodes the weights itself)
-        const uint8_t *plane = d_sums ? nullptr : batch_plane_of(LLAM_FMT_Q6_K, d_w, N, K);
+        const uint8_t *plane = static_cast<const uint8_t *>(d_plane);
         const Mfma6Shape sh =
-            gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA6_DUMP_COMPUTE : plane ? MFMA6_PLANE_COMPUTE : MFMA6_MAX_COMPUTE,
+            gemv_mfma6_shape(N, SB, cu_count(device_id), plane ? MFMA6_PLANE_COMPUTE : d_sums ? MFMA6_DUMP_COMPUTE : MFMA6_MAX_COMPUTE,
                              plane != nullptr);
         Mfma6Args a;
         a.w = static_cast<const uint8_t *>(d_w);
@@ -567,7 +572,10 @@ namespace llamql
         {
             if (src.kind != ACT_SRC_Q8)
                 return fail(fn, "block sums are dumped on Q8_1 input");
-            gemv_mfma_q6k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            if (plane)
+                gemv_mfma_q6k_plane_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            else
+                gemv_mfma_q6k_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
             return launched(fn);
         }
         if (plane)
@@ -589,33 +597,39 @@ namespace llamql
         return launched(fn);
     }
 
-    // The batch plane attached to a matrix, for a batch the plane kernels take (5..8 rows, no
-    // tuning override in force), else null.  Q6_K: wherever a plane is attached; Q4_K: where the
-    // batch goes to the matrix-unit kernel anyway.
+    // Whether a batch of M rows of this matrix is served from its batch plane when the caller
+    // brings one: 5..8 rows, no tuning override in force; Q6_K: rows of eight super-blocks and
+    // more, Q4_K: where the batch goes to the matrix-unit kernel anyway.
     template <class F>
-    const uint8_t *batch_plane_for(const void *d_w, int M, int N, int K)
+    bool batch_plane_usable(int M, int N, int K)
     {
         if constexpr (F::USE_MFMA_BATCH)
             if (M >= 5 && M <= 8 && gemv_unroll_override() == 0 && gemv_rows_per_wave_override() == 0)
             {
                 if constexpr (std::is_same<typename F::Quad, Q6KQuad>::value)
-                    return batch_plane_of(LLAM_FMT_Q6_K, d_w, N, K);
+                    return K / 256 >= 8 && q6k_plane_bytes(N, K / 256) < ((size_t)1 << 32);
                 else
-                    return mfma_eligible<F>(M, N, K) ? batch_plane_of(LLAM_FMT_Q4_K, d_w, N, K) : nullptr;
+                    return mfma_eligible<F>(M, N, K) && q4k_plane_bytes(N, K / 256) < ((size_t)1 << 32);
             }
-        return nullptr;
+        return false;
+    }
+    // The plane a launch reads: d_plane where it is usable, else null.
+    template <class F>
+    const void *batch_plane_for(const void *d_plane, int M, int N, int K)
+    {
+        return d_plane && batch_plane_usable<F>(M, N, K) ? d_plane : nullptr;
     }
 
     // The matrix-unit kernel of format F (mfma_eligible<F> or batch_plane_for<F> has said yes).
     template <class F>
-    bool gemv_mfma_launch(const char *fn, const void *d_w, const ActSource &src, float *d_y, int M, int N, int K,
-                          int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr, int row0 = 0,
-                          int nrows = 0)
+    bool gemv_mfma_launch(const char *fn, const void *d_w, const void *d_plane, const ActSource &src, float *d_y,
+                          int M, int N, int K, int ldy, int device_id, hipStream_t st, int32_t *d_sums = nullptr,
+                          int row0 = 0, int nrows = 0)
     {
         if constexpr (std::is_same<typename F::Quad, Q6KQuad>::value)
-            return gemv_mfma_q6k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
+            return gemv_mfma_q6k_launch(fn, d_w, d_plane, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
         else
-            return gemv_mfma_q4k_launch(fn, d_w, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
+            return gemv_mfma_q4k_launch(fn, d_w, d_plane, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
     }
 
     static_assert(ACT_SRC_Q8 == QUAD_SRC_Q8 && ACT_SRC_F32 == QUAD_SRC_F32 && ACT_SRC_SWIGLU == QUAD_SRC_SWIGLU &&
@@ -910,32 +924,35 @@ namespace llamql
     // is current.  M is 1..8.  With d_sums the same plan is executed with the chosen kernel's
     // block-sum variant: the parity hook reads the integer pipeline that serves this
     // (format, M, N, K).
+    // d_plane: the matrix's batch plane or null; a batch it serves goes to the plane kernel
+    // whatever the plan says for the matrix alone.
     template <class F>
-    bool gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                     int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
+    bool gemv_launch(const char *fn, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                     int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
     {
         const int SB = K / 256;
         const bool dump = d_sums != nullptr;
         if constexpr (F::USE_MFMA_BATCH)
-            if (!dump && batch_plane_for<F>(d_w, M, N, K))
-                return gemv_mfma_launch<F>(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st);
+            if (const void *plane = batch_plane_for<F>(d_plane, M, N, K))
+                return gemv_mfma_launch<F>(fn, d_w, plane, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st,
+                                           d_sums, row0, nrows);
         const GemvPlan p = gemv_plan<F>(M, N, K, device_id);
         if (p.kernel < 0)
             return fail(fn, "K=%d is too long for %d activation row(s) in LDS", K, p.m_first);
         if (p.m_first < M)
         {
             // the first p.m_first rows now, the others after them
-            if (!gemv_launch<F>(fn, d_w, d_q8, d_y, d_sums, p.m_first, N, K, ldy, row0, nrows, device_id, st))
+            if (!gemv_launch<F>(fn, d_w, nullptr, d_q8, d_y, d_sums, p.m_first, N, K, ldy, row0, nrows, device_id, st))
                 return false;
             const uint8_t *q8b = static_cast<const uint8_t *>(d_q8) + (size_t)p.m_first * (K / 32) * 36;
-            return gemv_launch<F>(fn, d_w, q8b, d_y ? d_y + (size_t)p.m_first * ldy : nullptr,
+            return gemv_launch<F>(fn, d_w, nullptr, q8b, d_y ? d_y + (size_t)p.m_first * ldy : nullptr,
                                   d_sums ? d_sums + (size_t)p.m_first * nrows * (K / 32) : nullptr, M - p.m_first, N,
                                   K, ldy, row0, nrows, device_id, st);
         }
         if constexpr (F::USE_MFMA_BATCH)
             if (p.kernel == GEMV_KERNEL_MFMA)
-                return gemv_mfma_launch<F>(fn, d_w, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st, d_sums,
-                                           row0, nrows);
+                return gemv_mfma_launch<F>(fn, d_w, nullptr, act_source_q8(d_q8), d_y, M, N, K, ldy, device_id, st,
+                                           d_sums, row0, nrows);
         if constexpr (F::USE_QUAD)
             if (p.kernel == GEMV_KERNEL_QUAD)
             {

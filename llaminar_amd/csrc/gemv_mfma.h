@@ -258,7 +258,6 @@ namespace llamql
     __global__ void __launch_bounds__((DUMP ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES) * WAVE)
         gemv_mfma_q4k_kernel(const MfmaArgs a)
     {
-        static_assert(!(DUMP && PLANE), "the block-sum variant reads the prepared matrix");
         typedef typename std::conditional<PLANE, MfmaPlaneRaw, MfmaRaw>::type Raw;
         constexpr int LOADS = PLANE ? MFMA_PLANE_LOADS : MFMA_LOADS;
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];

@@ -425,7 +425,8 @@ namespace llamql
     // (eight lanes read one 128-byte line of the plane; a group's super-block is 1 KB in one
     // place), so there is no bounce buffer either.  Same block sums, same scales, same order of
     // the fp32 operations: the results are those of gemv_mfma_q6k_kernel bit for bit.
-    template <int SRC>
+    // DUMP: also store the matrix unit's exact int32 block sums (the parity hook), no fp32 output.
+    template <int SRC, bool DUMP = false>
     __global__ void __launch_bounds__((MFMA6_PLANE_COMPUTE + MFMA6_PLANE_PRODUCERS) * WAVE) gemv_mfma_q6k_plane_kernel(const Mfma6Args a)
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma6_lds[];
@@ -494,6 +495,17 @@ namespace llamql
             mfma6_keep(bufA); // the staging code must not reuse the registers of the loads in flight
             mfma6_keep(bufB);
 
+            // DUMP: byte offset from a.sums of this lane's sums of its first activation row (4 lh); the
+            // following rows lie dump_stride sums further each.  All ones outside the row window.
+            uint32_t dump_off = 0xFFFFFFFFu;
+            const size_t dump_stride = (size_t)a.nrows * ((size_t)nsb * 8);
+            if constexpr (DUMP)
+            {
+                const long own = tile_row0 + l32;
+                const long rr = own - a.row0;
+                if (l32 < a.tile_rows && own < a.N && rr >= 0 && rr < a.nrows)
+                    dump_off = (uint32_t)((((size_t)(4 * lh) * a.nrows + (size_t)rr) * ((size_t)nsb * 8)) * sizeof(int32_t));
+            }
             v16i zero;
 #pragma unroll
             for (int i = 0; i < 16; ++i)
@@ -529,6 +541,19 @@ namespace llamql
                     const float4 ad = *reinterpret_cast<const float4 *>(sb_sc + j * 16);
                     const v16i dd = idot[j & 1];
                     const float b = h2f((uint16_t)(sc[j >> 1] >> (16 * (j & 1))));
+                    if constexpr (DUMP)
+                    {
+                        if (dump_off != 0xFFFFFFFFu)
+                        {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                if (4 * lh + i < a.M)
+                                {
+                                    char *base = reinterpret_cast<char *>(a.sums) + ((size_t)(sb * 8 + j) + (size_t)i * dump_stride) * sizeof(int32_t);
+                                    *reinterpret_cast<int32_t *>(base + dump_off) = dd[i];
+                                }
+                        }
+                    }
                     acc[0] = fmaf((float)dd[0], ad.x * b, acc[0]);
                     acc[1] = fmaf((float)dd[1], ad.y * b, acc[1]);
                     acc[2] = fmaf((float)dd[2], ad.z * b, acc[2]);
@@ -586,8 +611,11 @@ namespace llamql
                     for (int s = 1; s < a.slices; ++s)
                         v += red[((wave + s) * 4 + i) * WAVE + lane];
                     const int m = 4 * (lane >> 5) + i;
-                    if (m < a.M && row < a.N)
-                        a.y[(size_t)m * a.ldy + row] = v;
+                    if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
+                    {
+                        if (m < a.M && row < a.N)
+                            a.y[(size_t)m * a.ldy + row] = v;
+                    }
                 }
             }
         }

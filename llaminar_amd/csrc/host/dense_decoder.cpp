@@ -52,6 +52,7 @@ namespace
 
         int32_t *ids = nullptr, *pos = nullptr;
         int host_max_pos = 0; // the furthest sequence's position as the host counts it
+        float *last_res = nullptr; // where the last step left the residual stream (x or x_alt)
         float *x = nullptr, *x_alt = nullptr, *delta = nullptr, *qkv = nullptr, *attn = nullptr, *gate = nullptr, *up = nullptr;
         float *logits = nullptr, *inv_freq = nullptr, *rope_table = nullptr, *att_scratch = nullptr;
         void *q8_h = nullptr, *q8_attn = nullptr, *q8_act = nullptr, *argmax_scratch = nullptr;
@@ -250,9 +251,7 @@ extern "C" void *llam_decoder_buffer(void *dec, const char *name, int layer)
     if (!strcmp(name, "logits"))
         return d->logits;
     if (!strcmp(name, "x"))
-        return d->x;
-    if (!strcmp(name, "delta"))
-        return d->delta;
+        return d->last_res ? d->last_res : d->x;
     if (layer >= 0 && layer < d->cfg.n_layers)
     {
         if (!strcmp(name, "kcache"))
@@ -315,20 +314,20 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
         return true;
     };
     // res += W q8 where the launch can, else delta = W q8 and pending
-    auto project_into_residual = [&](uint8_t fmt, const void *w, const void *q8, int K) {
+    auto project_into_residual = [&](uint8_t fmt, const void *w, const void *plane, const void *q8, int K) {
         if (llam_ql_gemv_accumulate_supported(fmt, B, H, K, dev))
             return forward(fn, llam_ql_gemv_accumulate(fmt, w, q8, res, B, H, K, H, dev, stream));
         pending = d->delta;
-        return forward(fn, llam_ql_gemv(fmt, w, q8, d->delta, B, H, K, H, dev, stream));
+        return forward(fn, llam_ql_gemv_plane(fmt, w, plane, q8, d->delta, B, H, K, H, dev, stream));
     };
     for (int l = 0; l < c.n_layers; ++l)
     {
         const llam_decoder_layer &w = d->layers[l];
         // attention half
         llam_ql_proj qkv[3];
-        qkv[0] = llam_ql_proj{w.wq, d->qkv, QD, ldqkv, w.fmt_q};
-        qkv[1] = llam_ql_proj{w.wk, d->qkv + QD, KV, ldqkv, w.fmt_k};
-        qkv[2] = llam_ql_proj{w.wv, d->qkv + QD + KV, KV, ldqkv, w.fmt_v};
+        qkv[0] = llam_ql_proj{w.wq, d->qkv, QD, ldqkv, w.fmt_q, w.plane_q};
+        qkv[1] = llam_ql_proj{w.wk, d->qkv + QD, KV, ldqkv, w.fmt_k, w.plane_k};
+        qkv[2] = llam_ql_proj{w.wv, d->qkv + QD + KV, KV, ldqkv, w.fmt_v, w.plane_v};
         if (!norm_and_project(qkv, 3, w.attn_norm))
             return false;
         // rotary embedding, the cache append and the attention in one operator; its output leaves the
@@ -337,12 +336,12 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
                                                  0, d->q8_attn, d->att_scratch, B, c.n_heads, c.n_kv, c.head_dim,
                                                  c.ctx_cap, dev, stream)))
             return false;
-        if (!project_into_residual(w.fmt_o, w.wo, d->q8_attn, QD))
+        if (!project_into_residual(w.fmt_o, w.wo, w.plane_o, d->q8_attn, QD))
             return false;
         // feed-forward half
         llam_ql_proj gu[2];
-        gu[0] = llam_ql_proj{w.wgate, d->gate, F, F, w.fmt_gate};
-        gu[1] = llam_ql_proj{w.wup, d->up, F, F, w.fmt_up};
+        gu[0] = llam_ql_proj{w.wgate, d->gate, F, F, w.fmt_gate, w.plane_gate};
+        gu[1] = llam_ql_proj{w.wup, d->up, F, F, w.fmt_up, w.plane_up};
         if (!norm_and_project(gu, 2, w.ffn_norm))
             return false;
         if (llam_ql_gemv_accumulate_supported(w.fmt_down, B, H, F, dev))
@@ -351,12 +350,12 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
             // again by every workgroup of the projection), then res += W_down act
             if (!forward(fn, llam_ql_swiglu_quantize(d->gate, d->up, nullptr, d->q8_act, B, F, dev, stream)))
                 return false;
-            if (!project_into_residual(w.fmt_down, w.wdown, d->q8_act, F))
+            if (!project_into_residual(w.fmt_down, w.wdown, w.plane_down, d->q8_act, F))
                 return false;
         }
         else
         {
-            if (!forward(fn, llam_ql_gemv_swiglu_f32(w.fmt_down, w.wdown, d->gate, d->up, F, d->delta, B, H, F, H,
+            if (!forward(fn, llam_ql_gemv_swiglu_f32(w.fmt_down, w.wdown, w.plane_down, d->gate, d->up, F, d->delta, B, H, F, H,
                                                      d->q8_act, dev, stream)))
                 return false;
             pending = d->delta;
@@ -365,8 +364,9 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
     if (!forward(fn, llam_dec_rmsnorm_q8_1(res, pending, d->globals.final_norm, c.rms_eps, nullptr, d->q8_h, B, H,
                                            dev, stream)))
         return false;
-    if (!forward(fn, llam_ql_gemv(d->globals.fmt_lm_head, d->globals.lm_head, d->q8_h, d->logits, B, c.vocab, H,
-                                  c.vocab, dev, stream)))
+    d->last_res = res; // the final norm has added what was pending
+    if (!forward(fn, llam_ql_gemv_plane(d->globals.fmt_lm_head, d->globals.lm_head, d->globals.plane_lm_head, d->q8_h,
+                                        d->logits, B, c.vocab, H, c.vocab, dev, stream)))
         return false;
     if (!forward(fn, llam_dec_argmax(d->logits, c.vocab, c.vocab, B, d->ids, d->pos, d->argmax_scratch, dev, stream)))
         return false;

@@ -305,7 +305,6 @@ namespace llaminar_amd
     {
         if (!d_plane_)
             return;
-        (void)llam_ql_attach_batch_plane(fmt_, d_weights_, nullptr, 0, 0);
         (void)hipSetDevice(device_id_);
         (void)hipFree(d_plane_); // waits for the launches that read it
         d_plane_ = nullptr;
@@ -331,10 +330,9 @@ namespace llaminar_amd
         void *p = nullptr;
         if (hipSetDevice(device_id_) != hipSuccess || hipMalloc(&p, bytes) != hipSuccess)
             return fail(fn, "hipMalloc of %zu bytes failed", bytes);
-        // built before it is attached: a launch on another stream must not find a half-written plane
+        // finished before any launch gets it: a launch on another stream must not read a half-written plane
         if (!llam_ql_build_batch_plane(fmt_, d_weights_, p, N_, K_, device_id_, stream_) ||
-            hipStreamSynchronize(static_cast<hipStream_t>(stream_)) != hipSuccess ||
-            !llam_ql_attach_batch_plane(fmt_, d_weights_, p, N_, K_))
+            hipStreamSynchronize(static_cast<hipStream_t>(stream_)) != hipSuccess)
         {
             (void)hipFree(p);
             return fail(fn, "%s", llam_ql_last_error());
@@ -414,7 +412,7 @@ namespace llaminar_amd
     {
         auto product = [&](float *dst, int ld) {
             return m <= LLAM_QL_MAX_GEMV_M
-                       ? llam_ql_gemv(fmt_, d_weights_, d_q8, dst, m, n, K_, ld, device_id_, stream)
+                       ? llam_ql_gemv_plane(fmt_, d_weights_, d_plane_, d_q8, dst, m, n, K_, ld, device_id_, stream)
                        : llam_ql_gemm(fmt_, d_weights_, d_q8, dst, m, n, K_, ld, device_id_, stream);
         };
         const float *d_bias = bias ? bias->data : nullptr;
@@ -466,8 +464,10 @@ namespace llaminar_amd
         // plain decode product: the fp32-input GEMV quantises inside its kernel where that
         // saves the quantiser launch (same bits), else through q8
         if (m <= LLAM_QL_MAX_GEMV_M && alpha == 1.0f && beta == 0.0f && !bias)
-            return forward(fn, llam_ql_gemv_f32(fmt_, d_weights_, a, k, C->data, m, n, k, C->stride(), q8, device_id_,
-                                                stream_));
+        {
+            const llam_ql_proj one{d_weights_, C->data, n, C->stride(), fmt_, d_plane_};
+            return forward(fn, llam_ql_gemv_fused_f32(&one, 1, a, k, m, k, q8, device_id_, stream_));
+        }
         return forward(fn, llam_ql_quantize_q8_1(a, q8, m, k, device_id_, stream_)) &&
                run(fn, q8, C->data, C->stride(), m, n, bias, alpha, beta, s, stream_);
     }
@@ -562,6 +562,7 @@ namespace llaminar_amd
                 projs[i].N = p.n;
                 projs[i].ldy = p.output->stride();
                 projs[i].fmt = p.kernel->fmt_;
+                projs[i].d_plane = p.kernel->d_plane_;
             }
             return forward(fn, llam_ql_gemv_fused_f32(projs, (int)projections.size(), input->data, k, m, k, q8,
                                                       device_id_, stream_));
@@ -592,7 +593,7 @@ namespace llaminar_amd
             if (!p.kernel)
                 return fail(fn, "null projection kernel");
             llam_ql_gemv_plan plan;
-            if (!forward(fn, llam_ql_gemv_describe(p.kernel->fmt_, m, p.n, k, device_id_, &plan)))
+            if (!forward(fn, llam_ql_gemv_describe(p.kernel->fmt_, m, p.n, k, p.kernel->d_plane_ != nullptr, device_id_, &plan)))
                 return false;
             if (!plan.decode_equivalent)
                 return fail(fn, "m=%d n=%d k=%d (format %d) is not served like m=1: rows would differ in the last bits",
@@ -622,7 +623,7 @@ namespace llaminar_amd
             return false;
         void *q8 = s.take(q8_bytes(m, k));
         if (m <= LLAM_QL_MAX_GEMV_M && alpha == 1.0f && beta == 0.0f)
-            return forward(fn, llam_ql_gemv_swiglu_f32(fmt_, d_weights_, gate->data, up->data, k, output->data, m, n,
+            return forward(fn, llam_ql_gemv_swiglu_f32(fmt_, d_weights_, d_plane_, gate->data, up->data, k, output->data, m, n,
                                                        k, output->stride(), q8, device_id_, stream_));
         return forward(fn, llam_ql_swiglu_quantize(gate->data, up->data, nullptr, q8, m, k, device_id_, stream_)) &&
                run(fn, q8, output->data, output->stride(), m, n, nullptr, alpha, beta, s, stream_);

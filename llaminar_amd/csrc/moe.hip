@@ -962,6 +962,29 @@ namespace llamql
         }
     }
 
+    // What decodeRouteSelect publishes beside the runtime top-k state (IMoEKernel.h:245-258;
+    // kernels/rocm/moe/ROCmMoEKernel.cpp:2956-3019): the routing as fp32 tensors for stages that
+    // still read those, and one count per selected expert in the layer's decode histogram.
+    // Integer atomics: the counts do not depend on the order of the adds.
+    __global__ void __launch_bounds__(256)
+        moe_publish_routing_kernel(const int32_t *__restrict__ ids, const float *__restrict__ weights, int n_tokens,
+                                   int top_k, int slot_stride, float *__restrict__ indices_f32,
+                                   float *__restrict__ weights_f32, unsigned long long *__restrict__ histogram,
+                                   int n_experts)
+    {
+        const int i = blockIdx.x * blockDim.x + threadIdx.x;
+        if (i >= n_tokens * top_k)
+            return;
+        const int t = i / top_k, s = i - t * top_k;
+        const int32_t e = ids[(size_t)t * slot_stride + s];
+        if (indices_f32)
+            indices_f32[i] = (float)e;
+        if (weights_f32)
+            weights_f32[i] = weights[(size_t)t * slot_stride + s];
+        if (histogram && e >= 0 && e < n_experts)
+            atomicAdd(histogram + e, 1ull);
+    }
+
     // ---- shared expert gate -----------------------------------------------------------
     // out[t,:] += sigmoid(dot(gate_inp, hidden[t,:])) * shared[t,:]
     // (CPUMoEKernel::sharedExpertGate, kernels/cpu/moe/CPUMoEKernel.cpp:162-197, followed by
@@ -1575,6 +1598,31 @@ extern "C" bool llam_ql_moe_ids_from_f32(const float *d_indices, int32_t *d_ids,
         return false;
     hipLaunchKernelGGL(moe_ids_from_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream),
                        d_indices, d_ids, n);
+    return launched(fn);
+}
+
+extern "C" bool llam_ql_moe_publish_routing(const int32_t *d_ids, const float *d_weights, int n_tokens, int top_k,
+                                            int slot_stride, float *d_indices_f32, float *d_weights_f32,
+                                            uint64_t *d_histogram, int n_experts, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_publish_routing";
+    if (n_tokens < 0 || top_k < 0 || slot_stride < top_k)
+        return fail(fn, "bad sizes: n_tokens=%d top_k=%d slot_stride=%d", n_tokens, top_k, slot_stride);
+    if (n_tokens == 0 || top_k == 0 || (!d_indices_f32 && !d_weights_f32 && !d_histogram))
+        return true;
+    if (!d_ids || (d_weights_f32 && !d_weights))
+        return fail(fn, "null pointer");
+    if (d_histogram && n_experts <= 0)
+        return fail(fn, "a histogram needs n_experts > 0");
+    if ((long)n_tokens * top_k > (1L << 30))
+        return fail(fn, "too many (token, slot) pairs");
+    if (!set_device(fn, device_id))
+        return false;
+    const int n = n_tokens * top_k;
+    hipLaunchKernelGGL(moe_publish_routing_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       d_ids, d_weights, n_tokens, top_k, slot_stride, d_indices_f32, d_weights_f32,
+                       reinterpret_cast<unsigned long long *>(d_histogram), n_experts);
     return launched(fn);
 }
 

@@ -3,7 +3,6 @@
 
 #include <cstring>
 #include <mutex>
-#include <unordered_map>
 
 #include "llaminar_amd/ql_api.h"
 
@@ -45,38 +44,8 @@ namespace llamql
         }
         return cached[device_id];
     }
-
-    namespace
-    {
-        struct BatchPlane
-        {
-            const uint8_t *plane;
-            int N, K;
-            uint8_t fmt;
-        };
-        std::mutex g_plane_mu;
-        std::unordered_map<const void *, BatchPlane> g_planes;
-    } // namespace
-
-    const uint8_t *batch_plane_of(uint8_t fmt, const void *d_w, int N, int K)
-    {
-        std::lock_guard<std::mutex> lock(g_plane_mu);
-        if (g_planes.empty())
-            return nullptr;
-        const auto it = g_planes.find(d_w);
-        return it != g_planes.end() && it->second.N == N && it->second.K == K && it->second.fmt == fmt ? it->second.plane : nullptr;
-    }
-
-    void batch_plane_attach(uint8_t fmt, const void *d_w, const void *d_plane, int N, int K)
-    {
-        std::lock_guard<std::mutex> lock(g_plane_mu);
-        if (d_plane)
-            g_planes[d_w] = BatchPlane{static_cast<const uint8_t *>(d_plane), N, K, fmt};
-        else
-            g_planes.erase(d_w);
-    }
 } // namespace llamql
 
 extern "C" const char *llam_ql_last_error(void) { return llamql::last_error_text(); }
 
-extern "C" int llam_ql_abi_version(void) { return 1; }
+extern "C" int llam_ql_abi_version(void) { return 2; }

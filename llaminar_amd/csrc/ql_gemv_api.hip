@@ -5,13 +5,16 @@
 
 namespace llamql
 {
-    bool q4k_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                         int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
-    bool q6k_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                         int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
-    bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                          int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st);
-    void gemv_describe(uint8_t fmt, int M, int N, int K, int device_id, llam_ql_gemv_plan *out);
+    bool q4k_gemv_launch(const char *fn, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                         int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id,
+                         hipStream_t st);
+    bool q6k_gemv_launch(const char *fn, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                         int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id,
+                         hipStream_t st);
+    bool iq3s_gemv_launch(const char *fn, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                          int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id,
+                          hipStream_t st);
+    void gemv_describe(uint8_t fmt, int M, int N, int K, bool has_plane, int device_id, llam_ql_gemv_plan *out);
     bool gemv_norm_fusable(uint8_t fmt, int M, int N, int K);
     bool gemv_accumulate(const char *fn, uint8_t fmt, const void *d_w, const void *d_q8, float *d_y, int M, int N,
                          int K, int ldy, int device_id, hipStream_t st, bool query);
@@ -54,17 +57,29 @@ namespace llamql
             return true;
         }
 
-        bool dispatch(const char *fn, uint8_t fmt, const void *d_w, const void *d_q8, float *d_y, int32_t *d_sums,
-                      int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
+        // A caller's batch plane must be one llam_ql_build_batch_plane can have filled for this matrix.
+        bool check_plane(const char *fn, uint8_t fmt, const void *d_plane, int N, int K)
+        {
+            if (!d_plane)
+                return true;
+            if (!aligned16(d_plane))
+                return fail(fn, "d_plane must be 16-byte aligned");
+            if (llam_ql_batch_plane_bytes(fmt, N, K) == 0)
+                return fail(fn, "format %d, N=%d, K=%d has no batch plane (llam_ql_batch_plane_bytes is 0)", (int)fmt, N, K);
+            return true;
+        }
+
+        bool dispatch(const char *fn, uint8_t fmt, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                      int32_t *d_sums, int M, int N, int K, int ldy, int row0, int nrows, int device_id, hipStream_t st)
         {
             switch (fmt)
             {
             case LLAM_FMT_Q4_K:
-                return q4k_gemv_launch(fn, d_w, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
+                return q4k_gemv_launch(fn, d_w, d_plane, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
             case LLAM_FMT_Q6_K:
-                return q6k_gemv_launch(fn, d_w, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
+                return q6k_gemv_launch(fn, d_w, d_plane, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
             default:
-                return iq3s_gemv_launch(fn, d_w, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
+                return iq3s_gemv_launch(fn, d_w, d_plane, d_q8, d_y, d_sums, M, N, K, ldy, row0, nrows, device_id, st);
             }
         }
     } // namespace
@@ -83,7 +98,23 @@ extern "C" bool llam_ql_gemv(uint8_t fmt, const void *d_w, const void *d_q8, flo
         return fail(fn, "ldy=%d smaller than N=%d", ldy, N);
     if (!set_device(fn, device_id))
         return false;
-    return dispatch(fn, fmt, d_w, d_q8, d_y, nullptr, M, N, K, ldy, 0, 0, device_id, as_stream(stream));
+    return dispatch(fn, fmt, d_w, nullptr, d_q8, d_y, nullptr, M, N, K, ldy, 0, 0, device_id, as_stream(stream));
+}
+
+extern "C" bool llam_ql_gemv_plane(uint8_t fmt, const void *d_w, const void *d_plane, const void *d_q8, float *d_y,
+                                   int M, int N, int K, int ldy, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_plane";
+    if (!check_common(fn, fmt, d_w, d_q8, M, N, K) || !check_plane(fn, fmt, d_plane, N, K))
+        return false;
+    if (!d_y)
+        return fail(fn, "null output");
+    if (ldy < N)
+        return fail(fn, "ldy=%d smaller than N=%d", ldy, N);
+    if (!set_device(fn, device_id))
+        return false;
+    return dispatch(fn, fmt, d_w, d_plane, d_q8, d_y, nullptr, M, N, K, ldy, 0, 0, device_id, as_stream(stream));
 }
 
 namespace llamql
@@ -138,8 +169,8 @@ namespace llamql
                     src = act_source_q8(d_q8_scratch);
                     continue; // groups may form again on the Q8_1 input
                 }
-                if (!dispatch(fn, projs[i].fmt, projs[i].d_w, src.q8, projs[i].d_y, nullptr, M, projs[i].N, K,
-                              projs[i].ldy, 0, 0, device_id, as_stream(stream)))
+                if (!dispatch(fn, projs[i].fmt, projs[i].d_w, projs[i].d_plane, src.q8, projs[i].d_y, nullptr, M,
+                              projs[i].N, K, projs[i].ldy, 0, 0, device_id, as_stream(stream)))
                     return false;
                 ++i;
             }
@@ -154,7 +185,8 @@ namespace llamql
                 return fail(fn, "null projection table");
             for (int i = 0; i < num; ++i)
             {
-                if (!check_matrix(fn, projs[i].fmt, projs[i].d_w, M, projs[i].N, K))
+                if (!check_matrix(fn, projs[i].fmt, projs[i].d_w, M, projs[i].N, K) ||
+                    !check_plane(fn, projs[i].fmt, projs[i].d_plane, projs[i].N, K))
                     return false;
                 if (!projs[i].d_y || projs[i].ldy < projs[i].N)
                     return fail(fn, "projection %d: bad output (ldy=%d N=%d)", i, projs[i].ldy, projs[i].N);
@@ -202,6 +234,7 @@ extern "C" bool llam_ql_gemv_f32(uint8_t fmt, const void *d_w, const float *d_x,
     p.N = N;
     p.ldy = ldy;
     p.fmt = fmt;
+    p.d_plane = nullptr;
     if (!check_projections(fn, &p, 1, M, K) || !check_f32(fn, d_x, ldx, K, d_q8_scratch))
         return false;
     if (!set_device(fn, device_id))
@@ -258,6 +291,7 @@ extern "C" bool llam_ql_gemv_f32_static(uint8_t fmt, const void *d_w, const floa
     p.N = N;
     p.ldy = ldy;
     p.fmt = fmt;
+    p.d_plane = nullptr;
     if (!check_projections(fn, &p, 1, M, K) || !check_f32(fn, d_x, ldx, K, nullptr))
         return false;
     const size_t need = (size_t)M * (size_t)(K / 32) * sizeof(llam_block_q8_1);
@@ -291,9 +325,9 @@ extern "C" bool llam_ql_gemv_fused_f32(const llam_ql_proj *projs, int num, const
                            device_id, stream);
 }
 
-extern "C" bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const float *d_gate, const float *d_up,
-                                        int ld_gu, float *d_y, int M, int N, int K, int ldy, void *d_q8_scratch,
-                                        int device_id, void *stream)
+extern "C" bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const void *d_plane, const float *d_gate,
+                                        const float *d_up, int ld_gu, float *d_y, int M, int N, int K, int ldy,
+                                        void *d_q8_scratch, int device_id, void *stream)
 {
     using namespace llamql;
     static const char *fn = "llam_ql_gemv_swiglu_f32";
@@ -303,6 +337,7 @@ extern "C" bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const floa
     p.N = N;
     p.ldy = ldy;
     p.fmt = fmt;
+    p.d_plane = d_plane;
     if (!check_projections(fn, &p, 1, M, K) || !check_f32(fn, d_gate, ld_gu, K, d_q8_scratch) ||
         !check_f32(fn, d_up, ld_gu, K, nullptr))
         return false;
@@ -363,8 +398,14 @@ extern "C" bool llam_ql_gemv_fused_rmsnorm(const llam_ql_proj *projs, int num, c
         return false;
     if (!d_gamma || !aligned16(d_gamma))
         return fail(fn, "gamma must be a 16-byte aligned device pointer");
-    if (d_delta && (!aligned16(d_delta) || !d_x_out || !aligned16(d_x_out) || d_x_out == d_x))
-        return fail(fn, "with a delta, x + delta goes to d_x_out: 16-byte aligned and not d_x itself");
+    if (d_delta)
+    {
+        // workgroup 0 writes x + delta while every other workgroup still reads x and delta
+        const size_t n = (size_t)M * (size_t)K;
+        auto overlaps = [n](const float *a, const float *b) { return a < b + n && b < a + n; };
+        if (!aligned16(d_delta) || !d_x_out || !aligned16(d_x_out) || overlaps(d_x_out, d_x) || overlaps(d_x_out, d_delta))
+            return fail(fn, "with a delta, x + delta goes to d_x_out: 16-byte aligned, overlapping neither d_x nor d_delta");
+    }
     if (!llam_ql_gemv_fused_rmsnorm_supported(projs, num, M, K))
         return fail(fn, "M=%d K=%d: not every projection's kernel can fuse the norm (ask "
                         "llam_ql_gemv_fused_rmsnorm_supported; otherwise norm and projections run as two calls)",
@@ -385,13 +426,13 @@ extern "C" bool llam_ql_gemv_fused_rmsnorm(const llam_ql_proj *projs, int num, c
     return true;
 }
 
-extern "C" bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_q8,
+extern "C" bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void *d_plane, const void *d_q8,
                                         int32_t *d_sums, int M, int N, int K, int row0,
                                         int nrows, int device_id, void *stream)
 {
     using namespace llamql;
     static const char *fn = "llam_ql_gemv_block_sums";
-    if (!check_common(fn, fmt, d_w, d_q8, M, N, K))
+    if (!check_common(fn, fmt, d_w, d_q8, M, N, K) || !check_plane(fn, fmt, d_plane, N, K))
         return false;
     if (!d_sums)
         return fail(fn, "null output");
@@ -401,10 +442,11 @@ extern "C" bool llam_ql_gemv_block_sums(uint8_t fmt, const void *d_w, const void
         return fail(fn, "M=%d x %d rows x %d blocks of sums exceed 2 GiB", M, nrows, K / 32);
     if (!set_device(fn, device_id))
         return false;
-    return dispatch(fn, fmt, d_w, d_q8, nullptr, d_sums, M, N, K, 0, row0, nrows, device_id, as_stream(stream));
+    return dispatch(fn, fmt, d_w, d_plane, d_q8, nullptr, d_sums, M, N, K, 0, row0, nrows, device_id, as_stream(stream));
 }
 
-extern "C" bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int device_id, llam_ql_gemv_plan *out)
+extern "C" bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int has_plane, int device_id,
+                                      llam_ql_gemv_plan *out)
 {
     using namespace llamql;
     static const char *fn = "llam_ql_gemv_describe";
@@ -414,6 +456,6 @@ extern "C" bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int devi
         return fail(fn, "unsupported weight format id %d", (int)fmt);
     if (M < 1 || M > LLAM_QL_MAX_GEMV_M || N < 1 || K < 1 || (K % 256) != 0)
         return fail(fn, "bad shape (M=%d N=%d K=%d)", M, N, K);
-    gemv_describe(fmt, M, N, K, device_id, out); // no device call: the unit count falls back to 256
+    gemv_describe(fmt, M, N, K, has_plane != 0, device_id, out); // no device call: the unit count falls back to 256
     return true;
 }

@@ -79,11 +79,6 @@ namespace llamql
     inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
     inline bool aligned4(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
-    // Batch planes attached to prepared matrices (llam_ql_attach_batch_plane): the plane of the
-    // matrix at d_w if one is attached for this shape, else null.
-    const uint8_t *batch_plane_of(uint8_t fmt, const void *d_w, int N, int K);
-    void batch_plane_attach(uint8_t fmt, const void *d_w, const void *d_plane, int N, int K); // null plane: detach
-
     // Number of compute units of the current device (cached per device).
     int cu_count(int device_id);
 

@@ -14,6 +14,9 @@ namespace llamql
     int gemv_rows_per_wave_override() { return g_rows_per_wave; }
     int gemv_unroll_override() { return g_unroll; }
     int gemv_mfma_tile_rows_override() { return g_mfma_tile_rows; }
+    // Rows of weight per tile of the matrix-unit kernels of batches 5..8 (16..32; anything else:
+    // the built-in choice).  Reached from the test-only probe library, not from the C ABI.
+    void set_mfma_tile_rows_override(int tile_rows) { g_mfma_tile_rows = tile_rows >= 16 && tile_rows <= 32 ? tile_rows : 0; }
 } // namespace llamql
 
 extern "C" void llam_ql_set_gemv_tuning(int rows_per_wave, int unroll)
@@ -25,8 +28,4 @@ extern "C" void llam_ql_reset_gemv_tuning(void)
 {
     llamql::g_rows_per_wave = 0;
     llamql::g_unroll = 0;
-}
-extern "C" void llam_ql_set_batch_tile_rows(int tile_rows)
-{
-    llamql::g_mfma_tile_rows = tile_rows >= 16 && tile_rows <= 32 ? tile_rows : 0;
 }

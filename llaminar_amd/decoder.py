@@ -22,11 +22,13 @@ class Config(ctypes.Structure):
 class Layer(ctypes.Structure):
     _fields_ = [(n, c_void_p) for n in ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown")] + \
                [(n, c_uint8) for n in ("fmt_q", "fmt_k", "fmt_v", "fmt_o", "fmt_gate", "fmt_up", "fmt_down")] + \
-               [("attn_norm", c_void_p), ("ffn_norm", c_void_p)]
+               [("attn_norm", c_void_p), ("ffn_norm", c_void_p)] + \
+               [(n, c_void_p) for n in ("plane_q", "plane_k", "plane_v", "plane_o", "plane_gate", "plane_up", "plane_down")]
 
 
 class Globals(ctypes.Structure):
-    _fields_ = [("embed_q4k", c_void_p), ("final_norm", c_void_p), ("lm_head", c_void_p), ("fmt_lm_head", c_uint8)]
+    _fields_ = [("embed_q4k", c_void_p), ("final_norm", c_void_p), ("lm_head", c_void_p), ("fmt_lm_head", c_uint8),
+                ("plane_lm_head", c_void_p)]
 
 
 _lib = None
@@ -109,12 +111,12 @@ class DenseDecoder:
         self.keep = []   # device tensors the handle borrows
         self.raw = {} if keep_raw else None
         self.prepared = {} if keep_prepared else None   # name -> prepared weight tensor
-        # Matrices of 4096 rows and more get a batch plane where the batch is 5..8 rows (capi.attach_batch_plane):
+        # Matrices of 4096 rows and more get a batch plane where the batch is 5..8 rows (capi.build_batch_plane):
         # Q6_K ones (down, lm_head) an int8 copy, Q4_K ones (Q, O, gate, up) their bytes in the matrix unit's
         # operand order; same results, less work per launch
         if batch_planes is None:
             batch_planes = batch >= 5
-        self.planed = []   # prepared tensors with a plane attached
+        self.planes = {}   # name -> batch plane of that matrix
         g = torch.Generator(device=device)
         g.manual_seed(seed)
 
@@ -136,30 +138,32 @@ class DenseDecoder:
             raw = synth.weights_torch(fmt, n, k, sd, device, d_lo=d_lo, d_hi=d_hi)
             w = capi.prepare_weights(fmt, raw, n, k) if prepare else raw
             self.keep.append(w)
+            plane = None
             if prepare and batch_planes and n >= 4096 and capi.batch_plane_bytes(fmt, n, k) > 0:
-                plane = capi.attach_batch_plane(fmt, w, n, k)
+                plane = capi.build_batch_plane(fmt, w, n, k)
                 if plane is not None:
-                    self.keep.append(plane)
-                    self.planed.append(w)
+                    self.planes[name] = plane
             if keep_raw:
                 self.raw[name] = raw
             if keep_prepared:
                 self.prepared[name] = w
-            return w.data_ptr()
+            return w.data_ptr(), (plane.data_ptr() if plane is not None else None)
 
         for l in range(shape.n_layers):
             lw = Layer()
             for i, (name, n, k, fmt) in enumerate(shape.projections()):
-                setattr(lw, name, weights(f"{l}.{name}", fmt, n, k, seed * 100003 + l * 16 + i))
+                w_ptr, plane_ptr = weights(f"{l}.{name}", fmt, n, k, seed * 100003 + l * 16 + i)
+                setattr(lw, name, w_ptr)
                 setattr(lw, "fmt_" + name[1:], fmt)
+                setattr(lw, "plane_" + name[1:], plane_ptr)
             lw.attn_norm = norm_weight(f"{l}.attn_norm")
             lw.ffn_norm = norm_weight(f"{l}.ffn_norm")
             if not self.L.llam_decoder_set_layer(self.h, l, ctypes.byref(lw)):
                 raise capi.QLError(self.L.llam_decoder_last_error().decode())
         gl = Globals()
-        gl.embed_q4k = weights("embed", FMT_Q4_K, shape.vocab, shape.hidden, seed * 100003 + 900001, prepare=False)
+        gl.embed_q4k, _ = weights("embed", FMT_Q4_K, shape.vocab, shape.hidden, seed * 100003 + 900001, prepare=False)
         gl.final_norm = norm_weight("final_norm")
-        gl.lm_head = weights("lm_head", FMT_Q6_K, shape.vocab, shape.hidden, seed * 100003 + 900002)
+        gl.lm_head, gl.plane_lm_head = weights("lm_head", FMT_Q6_K, shape.vocab, shape.hidden, seed * 100003 + 900002)
         gl.fmt_lm_head = FMT_Q6_K
         if not self.L.llam_decoder_set_globals(self.h, ctypes.byref(gl)):
             raise capi.QLError(self.L.llam_decoder_last_error().decode())
@@ -169,9 +173,6 @@ class DenseDecoder:
         if self.h:
             self.L.llam_decoder_destroy(self.h)
             self.h = None
-        for w in self.planed:
-            capi.detach_batch_plane(w)
-        self.planed = []
 
     def __del__(self):
         try:
@@ -188,7 +189,7 @@ class DenseDecoder:
         if not ptr:
             raise capi.QLError(self.L.llam_decoder_last_error().decode())
         shapes = {"ids": ((B,), torch.int32), "pos": ((B,), torch.int32), "logits": ((B, s.vocab), torch.float32),
-                  "x": ((B, s.hidden), torch.float32), "delta": ((B, s.hidden), torch.float32),
+                  "x": ((B, s.hidden), torch.float32),
                   "kcache": ((B, s.n_kv, self.ctx_cap, s.head_dim), torch.float16),
                   "vcache": ((B, s.n_kv, self.ctx_cap, s.head_dim), torch.float16)}   # both in tiles (capi.kcache_tiled, vcache_tiled)
         shp, dt = shapes[name]

@@ -1,10 +1,30 @@
+// MEASUREMENT AND TEST INFRASTRUCTURE ONLY: built into tests/probe/libql_probe.so, never into
+// the product library, and declared in no public header.
+//
 // Read-only probes: the load streams of the decode GEMV without its arithmetic, for measuring
 // what an order of reads is worth on its own (bench.py --workload read-order).  Every probe
 // reads the whole buffer once; nothing is written unless the xor of all bytes happens to equal a
 // fixed pattern (which keeps the loads alive).
+//   llam_probe_read(d_buf, N, K, pattern, rows_per_wave, waves_per_wg, depth, workgroups, d_sink,
+//                   device_id, stream): streams the N * (K/256) * 144 bytes of a Q4_K-sized buffer.
+//     pattern 0 / 1: the quad-lane kernel's loads (4 lanes per super-block, 3 x 16 bytes per lane
+//       and step), N rows shared by ceil(N / rows_per_wave) wavefronts, each with its rows
+//       contiguous (0) or dealt round robin (1); depth = steps in flight per wavefront (1, 2, 4).
+//     pattern 2 / 3: 1 KB per load instruction, `workgroups` workgroups, a region per wavefront
+//       (2) or grid-stride (3); depth = loads in flight per lane (3, 6, 9).
+//   llam_probe_set_batch_tile_rows(rows): sweep override for the rows of weight per tile (16..32)
+//     of the matrix-unit kernels of batches 5..8; any other value restores the built-in choice.
 #include "ql_host.h"
 
-#include "llaminar_amd/ql_api.h"
+#define LLAM_QL_PROBE_ROWS_CONTIGUOUS 0
+#define LLAM_QL_PROBE_ROWS_ROUND_ROBIN 1
+#define LLAM_QL_PROBE_STREAM_REGION 2
+#define LLAM_QL_PROBE_STREAM_GRID_STRIDE 3
+
+namespace llamql
+{
+    void set_mfma_tile_rows_override(int tile_rows); // ql_tuning.hip, not part of the C ABI
+}
 
 namespace llamql
 {
@@ -109,11 +129,11 @@ namespace llamql
 
 using namespace llamql;
 
-extern "C" bool llam_ql_read_probe(const void *d_buf, int N, int K, int pattern, int rows_per_wave,
-                                   int waves_per_wg, int depth, int workgroups, int *d_sink, int device_id,
-                                   void *stream)
+extern "C" bool llam_probe_read(const void *d_buf, int N, int K, int pattern, int rows_per_wave,
+                                int waves_per_wg, int depth, int workgroups, int *d_sink, int device_id,
+                                void *stream)
 {
-    const char *fn = "llam_ql_read_probe";
+    const char *fn = "llam_probe_read";
     clear_error();
     if (!d_buf || !d_sink)
         return fail(fn, "null buffer");
@@ -156,3 +176,5 @@ extern "C" bool llam_ql_read_probe(const void *d_buf, int N, int K, int pattern,
     }
     return fail(fn, "unknown pattern %d", pattern);
 }
+
+extern "C" void llam_probe_set_batch_tile_rows(int tile_rows) { llamql::set_mfma_tile_rows_override(tile_rows); }

@@ -62,7 +62,7 @@ def test_argument_validation_and_error_text():
     from llaminar_amd import capi
 
     lib = capi.load()
-    assert lib.llam_ql_abi_version() == 1
+    assert lib.llam_ql_abi_version() == 2
     buf = np.zeros(4096, np.uint8)
     p = buf.ctypes.data
     p16 = p + (-p % 16)

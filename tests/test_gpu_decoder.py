@@ -46,7 +46,8 @@ class NumpyDecoder:
             g = self.gemv(f"{l}.wgate", FMT_Q4_K, H, h2[0])
             u = self.gemv(f"{l}.wup", FMT_Q4_K, H, h2[0])
             delta = self.gemv(f"{l}.wdown", FMT_Q6_K, s.ffn, o.swiglu(g, u))
-        hf, _ = o.rmsnorm(x[None], self.w["final_norm"], s.rms_eps, delta=delta[None])
+        hf, xf = o.rmsnorm(x[None], self.w["final_norm"], s.rms_eps, delta=delta[None])
+        self.last_residual = xf[0]   # the residual stream with every layer's output added
         logits = self.gemv("lm_head", FMT_Q6_K, H, hf[0])
         return logits
 
@@ -82,6 +83,7 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
         sync()
         logits = dec.buffer("logits").cpu().numpy()
         new_ids = dec.buffer("ids").cpu().numpy()
+        resid = dec.buffer("x").cpu().numpy()   # wherever the step left the residual stream
         assert dec.buffer("pos").cpu().tolist() == [int(p) + step + 1 for p in pos]
         assert np.isfinite(logits).all()
         for b in range(batch):
@@ -89,6 +91,7 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
             scale = np.abs(exp).max()
             err = np.abs(logits[b] - exp).max()
             assert err <= 5e-3 * scale, (step, b, err, scale)
+            assert np.abs(resid[b] - ref.last_residual).max() <= 5e-3 * np.abs(ref.last_residual).max(), (step, b)
             assert new_ids[b] == int(np.argmax(logits[b]))           # the sampler on the device's own logits
             top2 = np.sort(exp)[-2:]
             if top2[1] - top2[0] > 2 * 5e-3 * scale:

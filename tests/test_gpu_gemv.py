@@ -319,7 +319,7 @@ def test_error_paths(capi, dev):
     y = torch.zeros(64, device=dev)
     assert not lib.llam_ql_gemv(FMT_Q4_K, w.data_ptr(), w.data_ptr(), y.data_ptr(), 0, 4, 256, 4, 0, None)
     assert not lib.llam_ql_gemv(FMT_Q4_K, w.data_ptr(), w.data_ptr(), None, 1, 4, 256, 4, 0, None)
-    assert not lib.llam_ql_gemv_block_sums(FMT_Q4_K, w.data_ptr(), w.data_ptr(), y.data_ptr(), 1, 4, 256, 2, 3, 0, None)
+    assert not lib.llam_ql_gemv_block_sums(FMT_Q4_K, w.data_ptr(), None, w.data_ptr(), y.data_ptr(), 1, 4, 256, 2, 3, 0, None)
     assert "row window" in capi.last_error()
 
 
@@ -707,53 +707,62 @@ def test_accumulating_launch_is_refused_where_the_kernel_cannot(capi, dev):
 
 
 def test_read_probe_runs_and_checks_its_arguments(capi, dev):
-    """The read-only probes behind bench.py --workload read-order: every pattern runs on a small buffer (they read
-    inside N * K/256 * 144 bytes and write nothing), bad arguments are refused."""
+    """The read-only probes behind bench.py --workload read-order (tests/probe, not part of the product library):
+    every pattern runs on a small buffer (they read inside N * K/256 * 144 bytes and write nothing), bad arguments
+    are refused."""
     import torch
 
-    lib = capi.load()
+    from tests.probe import binding as probe
+
+    lib = probe.load()
     N, K = 96, 4096
     buf = torch.randint(0, 256, (N * (K // 256) * 144 + 64,), dtype=torch.uint8, device=dev)
     guard = buf[-64:].clone()
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     for pattern, rpw, depth, wgs in ((0, 3, 2, 0), (1, 3, 1, 0), (1, 5, 4, 0), (2, 0, 3, 4), (3, 0, 6, 4), (3, 0, 9, 2)):
-        assert lib.llam_ql_read_probe(buf.data_ptr(), N, K, pattern, rpw, 4, depth, wgs, sink.data_ptr(), 0, None), capi.last_error()
+        assert lib.llam_probe_read(buf.data_ptr(), N, K, pattern, rpw, 4, depth, wgs, sink.data_ptr(), 0, None), capi.last_error()
     sync()
     assert torch.equal(buf[-64:], guard) and int(sink[0]) in (0, 1)
     for args in ((buf.data_ptr(), N, K, 7, 3, 4, 2, 0), (buf.data_ptr(), N, K, 0, 3, 4, 3, 0), (buf.data_ptr(), N, 1024, 0, 3, 4, 2, 0),
                  (buf.data_ptr(), N, K, 2, 0, 4, 3, 0), (0, N, K, 0, 3, 4, 2, 0), (buf.data_ptr(), N, K, 0, 3, 17, 2, 0)):
-        assert not lib.llam_ql_read_probe(*args, sink.data_ptr(), 0, None)
+        assert not lib.llam_probe_read(*args, sink.data_ptr(), 0, None)
 
 
 @pytest.mark.parametrize("fmt,N,K", [(FMT_Q4_K, 8192 + 40, 5120), (FMT_Q6_K, 1000, 25600)])
 def test_batch_tile_heights_agree(capi, dev, oracle, fmt, N, K):
-    """The matrix-unit kernels of batches 5..8 with tiles of 16..32 weight rows (llam_ql_set_batch_tile_rows): every
-    height against the CPU restatement on a row window, and the exact block sums of the kernel that serves the
-    shape unchanged by the height (rows that do not fill the last tile included)."""
+    """The matrix-unit kernels of batches 5..8 with tiles of 16..32 weight rows (the sweep override of tests/probe):
+    every height against the CPU restatement on a row window, and the exact block sums of the kernel that serves
+    the shape unchanged by the height (rows that do not fill the last tile included), without and with the
+    matrix's batch plane."""
     import torch
 
+    from tests.probe import binding as probe
+
     M = 8
-    lib = capi.load()
+    plib = probe.load()
     assert capi.gemv_describe(fmt, M, N, K).kernel == 3
     W = synth.weights_numpy(fmt, N, K, 31)
     w = capi.prepare_weights(fmt, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
+    plane = capi.build_batch_plane(fmt, w, N, K)
+    assert plane is not None
     x = synth.activations_numpy(M, K, 6)
     q8 = capi.quantize_q8_1(torch.from_numpy(x).to(dev))
     rows = slice(N - 70, N)
     exp, exp_sums = oracle.gemm(fmt, W[rows], K, oracle.quantize(x), want_sums=True)
     try:
         for tr in (0, 32, 27, 20, 16):
-            lib.llam_ql_set_batch_tile_rows(tr)
-            y = capi.gemv(fmt, w, q8, M, N, K)
-            s = capi.gemv_block_sums(fmt, w, q8, M, N, K, N - 70, 70)
-            sync()
-            assert rel_err(y.cpu().numpy()[:, rows], exp) <= TOL[fmt] * 1e-2, tr
-            assert np.array_equal(s.cpu().numpy(), exp_sums), tr   # bit-exact whatever the tile height
+            plib.llam_probe_set_batch_tile_rows(tr)
+            for pl in (None, plane):
+                y = capi.gemv(fmt, w, q8, M, N, K, plane=pl)
+                s = capi.gemv_block_sums(fmt, w, q8, M, N, K, N - 70, 70, plane=pl)
+                sync()
+                assert rel_err(y.cpu().numpy()[:, rows], exp) <= TOL[fmt] * 1e-2, (tr, pl is not None)
+                assert np.array_equal(s.cpu().numpy(), exp_sums), (tr, pl is not None)   # bit-exact whatever the tile height
     finally:
-        lib.llam_ql_set_batch_tile_rows(0)
+        plib.llam_probe_set_batch_tile_rows(0)
 
 
-# ---- the Q6_K batch plane (llam_ql_build_batch_plane / llam_ql_attach_batch_plane) -----------------------------
+# ---- batch planes (llam_ql_build_batch_plane; handed to the launches that may use them) ------------------------
 def _plane_rows(plane: np.ndarray, N: int, nsb: int):
     """The plane's int8 weights as [rows][nsb][256] and fp16 scale bits as [rows][nsb][8], rows = 4 ceil(N / 4):
     group g = row / 4 keeps, per super-block, eight 128-byte lines (block j: its four rows' 32 bytes in turn), and
@@ -774,25 +783,23 @@ def test_q6k_batch_plane_holds_the_requantised_weights(capi, dev, oracle, N, K):
     W = synth.weights_numpy(FMT_Q6_K, N, K, 5 + N)
     w = capi.prepare_weights(FMT_Q6_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
     assert capi.batch_plane_bytes(FMT_Q6_K, N, K) == ((N + 3) // 4) * nsb * 1088
-    plane = capi.attach_batch_plane(FMT_Q6_K, w, N, K)
-    try:
-        sync()
-        got_w, got_s = _plane_rows(plane.cpu().numpy(), N, nsb)
-        for r in range(N):
-            for t in range(nsb):
-                ew, es, _ = oracle.subblocks(FMT_Q6_K, W[r, t])
-                assert np.array_equal(got_w[r, t], ew), (r, t)
-                assert np.array_equal(got_s[r, t], es), (r, t)
-        assert not got_w[N:].any() and not got_s[N:].any()
-    finally:
-        capi.detach_batch_plane(w)
+    plane = capi.build_batch_plane(FMT_Q6_K, w, N, K)
+    sync()
+    got_w, got_s = _plane_rows(plane.cpu().numpy(), N, nsb)
+    for r in range(N):
+        for t in range(nsb):
+            ew, es, _ = oracle.subblocks(FMT_Q6_K, W[r, t])
+            assert np.array_equal(got_w[r, t], ew), (r, t)
+            assert np.array_equal(got_s[r, t], es), (r, t)
+    assert not got_w[N:].any() and not got_s[N:].any()
 
 
 def test_q6k_batch_plane_launches_match(capi, dev, oracle):
-    """Batches of 5..8 rows with a plane attached: bit-identical to the launch without one where that is the
+    """Batches of 5..8 rows launched with the matrix's plane: the exact block sums of the plane kernel equal the
+    CPU restatement's; the fp32 results are bit-identical to the launch without a plane where that is the
     matrix-unit kernel as well (K = 25600, batches the quad-lane kernel cannot hold), within the format's tolerance
     of the CPU restatement everywhere (K = 5120 and batch 5 of K = 25600 leave the quad-lane kernel for it);
-    batches of 1..4 do not look at the plane; detaching restores the old launch."""
+    batches of 1..4 do not look at the plane; the same call without the plane is the old launch."""
     import torch
 
     for N, K in ((1030, 25600), (4100, 5120), (50, 2048)):
@@ -800,29 +807,58 @@ def test_q6k_batch_plane_launches_match(capi, dev, oracle):
         w = capi.prepare_weights(FMT_Q6_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
         x = synth.activations_numpy(8, K, 9)
         q8 = capi.quantize_q8_1(torch.from_numpy(x).to(dev))
-        rows = slice(max(N - 70, 0), N)
-        exp, _ = oracle.gemm(FMT_Q6_K, W[rows], K, oracle.quantize(x), want_sums=True)
+        r0 = max(N - 70, 0)
+        rows = slice(r0, N)
+        exp, exp_sums = oracle.gemm(FMT_Q6_K, W[rows], K, oracle.quantize(x), want_sums=True)
         before = {M: capi.gemv(FMT_Q6_K, w, q8, M, N, K).clone() for M in (1, 4, 5, 7, 8)}
-        plane = capi.attach_batch_plane(FMT_Q6_K, w, N, K)
+        plane = capi.build_batch_plane(FMT_Q6_K, w, N, K)
         assert plane is not None
-        try:
-            for M in (1, 4, 5, 7, 8):
-                y = capi.gemv(FMT_Q6_K, w, q8, M, N, K)
-                sync()
-                assert rel_err(y.cpu().numpy()[:, rows], exp[:M]) <= TOL[FMT_Q6_K] * 1e-2, (N, K, M)
-                if M <= 4 or capi.gemv_describe(FMT_Q6_K, M, N, K).kernel == 3:
-                    assert torch.equal(y, before[M]), (N, K, M)
-            # fp32 input quantised inside the launch takes the plane too
-            xf = torch.from_numpy(x).to(dev)
-            scratch = torch.empty(8 * (K // 32) * 36, dtype=torch.uint8, device=dev)
-            y = capi.gemv_f32(FMT_Q6_K, w, xf, 8, N, K, q8_scratch=scratch)
+        for M in (1, 4, 5, 7, 8):
+            y = capi.gemv(FMT_Q6_K, w, q8, M, N, K, plane=plane)
+            s = capi.gemv_block_sums(FMT_Q6_K, w, q8, M, N, K, r0, N - r0, plane=plane)
             sync()
-            assert rel_err(y.cpu().numpy()[:, rows], exp) <= TOL[FMT_Q6_K] * 1e-2
-        finally:
-            capi.detach_batch_plane(w)
+            assert np.array_equal(s.cpu().numpy(), exp_sums[:M]), (N, K, M)
+            assert rel_err(y.cpu().numpy()[:, rows], exp[:M]) <= TOL[FMT_Q6_K] * 1e-2, (N, K, M)
+            with_plane = capi.gemv_describe(FMT_Q6_K, M, N, K, has_plane=True)
+            assert (with_plane.kernel == 3 and with_plane.decode_equivalent == 0) if M >= 5 else with_plane.kernel != 3
+            if M <= 4 or capi.gemv_describe(FMT_Q6_K, M, N, K).kernel == 3:
+                assert torch.equal(y, before[M]), (N, K, M)
+        # fp32 input quantised inside the launch takes the plane too
+        xf = torch.from_numpy(x).to(dev)
+        scratch = torch.empty(8 * (K // 32) * 36, dtype=torch.uint8, device=dev)
+        out = torch.empty(8, N, device=dev)
+        capi.gemv_fused_f32([(FMT_Q6_K, w, out, plane)], xf, 8, K, q8_scratch=scratch)
+        sync()
+        assert torch.equal(out, capi.gemv(FMT_Q6_K, w, q8, 8, N, K, plane=plane))
         y = capi.gemv(FMT_Q6_K, w, q8, 8, N, K)
         sync()
         assert torch.equal(y, before[8])
+
+
+def test_a_plane_is_an_argument_not_a_registration(capi, dev, oracle):
+    """Nothing is remembered between calls: two matrices that follow each other AT THE SAME ADDRESS (what a caching
+    allocator hands out after a free) each multiply against the plane passed with them, and a launch without a
+    plane never reads one."""
+    import torch
+
+    N, K, M = 4100, 5120, 8
+    x = synth.activations_numpy(M, K, 3)
+    q8 = capi.quantize_q8_1(torch.from_numpy(x).to(dev))
+    buf = torch.empty(capi.prepared_bytes(FMT_Q6_K, N, K), dtype=torch.uint8, device=dev)
+    results = []
+    for seed in (1, 2):
+        W = synth.weights_numpy(FMT_Q6_K, N, K, seed)
+        buf.copy_(capi.prepare_weights(FMT_Q6_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K))   # same address, new matrix
+        plane = capi.build_batch_plane(FMT_Q6_K, buf, N, K)
+        y = capi.gemv(FMT_Q6_K, buf, q8, M, N, K, plane=plane)
+        y0 = capi.gemv(FMT_Q6_K, buf, q8, M, N, K)
+        sync()
+        exp = oracle.gemm(FMT_Q6_K, W[-64:], K, oracle.quantize(x))
+        assert rel_err(y.cpu().numpy()[:, -64:], exp) <= TOL[FMT_Q6_K] * 1e-2, seed
+        assert rel_err(y0.cpu().numpy()[:, -64:], exp) <= TOL[FMT_Q6_K] * 1e-2, seed
+        results.append(y.clone())
+        del plane
+    assert not torch.equal(results[0], results[1])
 
 
 def test_batch_plane_refusals(capi, dev):
@@ -835,12 +871,15 @@ def test_batch_plane_refusals(capi, dev):
     assert capi.batch_plane_bytes(FMT_Q6_K, 5120, 1024) == 0        # rows of eight super-blocks and more
     assert capi.batch_plane_bytes(FMT_Q6_K, 5120, 25600) == 1280 * 100 * 1088
     buf = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    y = torch.zeros(64, device=dev)
     assert not lib.llam_ql_build_batch_plane(FMT_Q4_K, buf.data_ptr(), buf.data_ptr(), 4, 2048, 0, None)   # too few rows
     assert not lib.llam_ql_build_batch_plane(FMT_Q6_K, None, buf.data_ptr(), 4, 2048, 0, None)
-    assert not lib.llam_ql_attach_batch_plane(FMT_Q6_K, None, buf.data_ptr(), 4, 2048)
-    assert not lib.llam_ql_attach_batch_plane(FMT_Q6_K, buf.data_ptr(), buf.data_ptr(), 4, 1024)
-    assert not lib.llam_ql_attach_batch_plane(FMT_IQ3_S, buf.data_ptr(), buf.data_ptr(), 4096, 5120)
-    assert lib.llam_ql_attach_batch_plane(0, buf.data_ptr(), None, 0, 0)   # detaching what was never attached is fine
+    # a plane for a shape that has none, or a misaligned one, is refused by the launches
+    assert not lib.llam_ql_gemv_plane(FMT_Q6_K, buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), y.data_ptr(), 5, 4, 1024, 4, 0, None)
+    assert "no batch plane" in capi.last_error()
+    assert not lib.llam_ql_gemv_plane(FMT_IQ3_S, buf.data_ptr(), buf.data_ptr(), buf.data_ptr(), y.data_ptr(), 5, 4, 2048, 4, 0, None)
+    assert not lib.llam_ql_gemv_plane(FMT_Q6_K, buf.data_ptr(), buf.data_ptr() + 4, buf.data_ptr(), y.data_ptr(), 5, 4, 2048, 4, 0, None)
+    assert "16-byte aligned" in capi.last_error()
 
 
 def test_q4k_batch_plane_is_the_prepared_matrix_regrouped(capi, dev):
@@ -854,23 +893,21 @@ def test_q4k_batch_plane_is_the_prepared_matrix_regrouped(capi, dev):
     w = capi.prepare_weights(FMT_Q4_K, torch.from_numpy(W.reshape(-1)).to(dev), N, K)
     G = (N + 3) // 4
     assert capi.batch_plane_bytes(FMT_Q4_K, N, K) == G * nsb * 576
-    plane = capi.attach_batch_plane(FMT_Q4_K, w, N, K)
-    try:
-        sync()
-        p = plane.cpu().numpy()
-        pad = np.zeros((G * 4, nsb, 144), np.uint8)
-        pad[:N] = W.reshape(N, nsb, 144)
-        quants = pad[:, :, 16:].reshape(G, 4, nsb, 4, 32).transpose(0, 2, 3, 1, 4)   # [g][sb][group of quants][row][32]
-        heads = pad[:, :, :16].reshape(G, 4, nsb, 16).transpose(0, 2, 1, 3)          # [g][sb][row][16]
-        assert np.array_equal(p[:G * nsb * 512], quants.reshape(-1))
-        assert np.array_equal(p[G * nsb * 512:], heads.reshape(-1))
-    finally:
-        capi.detach_batch_plane(w)
+    plane = capi.build_batch_plane(FMT_Q4_K, w, N, K)
+    sync()
+    p = plane.cpu().numpy()
+    pad = np.zeros((G * 4, nsb, 144), np.uint8)
+    pad[:N] = W.reshape(N, nsb, 144)
+    quants = pad[:, :, 16:].reshape(G, 4, nsb, 4, 32).transpose(0, 2, 3, 1, 4)   # [g][sb][group of quants][row][32]
+    heads = pad[:, :, :16].reshape(G, 4, nsb, 16).transpose(0, 2, 1, 3)          # [g][sb][row][16]
+    assert np.array_equal(p[:G * nsb * 512], quants.reshape(-1))
+    assert np.array_equal(p[G * nsb * 512:], heads.reshape(-1))
 
 
 def test_q4k_batch_plane_launches_match(capi, dev, oracle):
-    """Q4_K batches of 5..8 with a plane attached: the matrix-unit kernel's results bit for bit, close to the CPU
-    restatement; rows that do not fill the last tile or group included; fp32 and SwiGLU input as well."""
+    """Q4_K batches of 5..8 launched with the matrix's plane: the plane kernel's exact block sums equal the CPU
+    restatement's, its results the matrix-unit kernel's bit for bit; rows that do not fill the last tile or group
+    included; fp32 and SwiGLU input as well."""
     import torch
 
     for N, K in ((4100, 5120), (4097, 8192)):
@@ -880,20 +917,23 @@ def test_q4k_batch_plane_launches_match(capi, dev, oracle):
         xd = torch.from_numpy(x).to(dev)
         q8 = capi.quantize_q8_1(xd)
         rows = slice(N - 70, N)
-        exp, _ = oracle.gemm(FMT_Q4_K, W[rows], K, oracle.quantize(x), want_sums=True)
+        exp, exp_sums = oracle.gemm(FMT_Q4_K, W[rows], K, oracle.quantize(x), want_sums=True)
         scratch = torch.empty(8 * (K // 32) * 36, dtype=torch.uint8, device=dev)
         before = {M: capi.gemv(FMT_Q4_K, w, q8, M, N, K).clone() for M in (4, 5, 6, 8)}
         before_f32 = capi.gemv_f32(FMT_Q4_K, w, xd, 8, N, K, q8_scratch=scratch).clone()
+        g, u = torch.randn(8, K, device=dev), torch.randn(8, K, device=dev)
+        before_swiglu = capi.gemv_swiglu_f32(FMT_Q4_K, w, g, u, 8, N, K, q8_scratch=scratch).clone()
         assert capi.gemv_describe(FMT_Q4_K, 5, N, K).kernel == 3
-        plane = capi.attach_batch_plane(FMT_Q4_K, w, N, K)
-        try:
-            for M in (4, 5, 6, 8):
-                y = capi.gemv(FMT_Q4_K, w, q8, M, N, K)
-                sync()
-                assert torch.equal(y, before[M]), (N, K, M)
-                assert rel_err(y.cpu().numpy()[:, rows], exp[:M]) <= TOL[FMT_Q4_K] * 1e-2
-            y = capi.gemv_f32(FMT_Q4_K, w, xd, 8, N, K, q8_scratch=scratch)
+        plane = capi.build_batch_plane(FMT_Q4_K, w, N, K)
+        for M in (4, 5, 6, 8):
+            y = capi.gemv(FMT_Q4_K, w, q8, M, N, K, plane=plane)
+            s = capi.gemv_block_sums(FMT_Q4_K, w, q8, M, N, K, N - 70, 70, plane=plane)
             sync()
-            assert torch.equal(y, before_f32)
-        finally:
-            capi.detach_batch_plane(w)
+            assert np.array_equal(s.cpu().numpy(), exp_sums[:M]), (N, K, M)
+            assert torch.equal(y, before[M]), (N, K, M)
+            assert rel_err(y.cpu().numpy()[:, rows], exp[:M]) <= TOL[FMT_Q4_K] * 1e-2
+        out = torch.empty(8, N, device=dev)
+        capi.gemv_fused_f32([(FMT_Q4_K, w, out, plane)], xd, 8, K, q8_scratch=scratch)
+        y = capi.gemv_swiglu_f32(FMT_Q4_K, w, g, u, 8, N, K, q8_scratch=scratch, plane=plane)
+        sync()
+        assert torch.equal(out, before_f32) and torch.equal(y, before_swiglu)

@@ -85,15 +85,14 @@ def test_decode_step_graph_replays_match_eager(capi, dev):
 
 
 def test_batch_plane_launches_replay(capi, dev):
-    """Batches of eight rows on matrices with batch planes attached, captured once: the plane is looked up when the
-    launch is recorded, every replay equals the eager result, and detaching afterwards does not disturb the graph
-    (it keeps the plane it was given; the buffers stay alive here)."""
+    """Batches of eight rows launched with their matrices' batch planes, captured once: every replay equals the
+    eager result, with eager launches of the same matrices (without a plane) between the replays."""
     M, H, F = 8, 2048, 4096
     mk = lambda fmt, N, K, seed: capi.prepare_weights(
         fmt, torch.from_numpy(synth.weights_numpy(fmt, N, K, seed).reshape(-1)).to(dev), N, K)
     wu, wd = mk(FMT_Q4_K, F, H, 11), mk(FMT_Q6_K, F, H, 12)
-    planes = [capi.attach_batch_plane(FMT_Q4_K, wu, F, H), capi.attach_batch_plane(FMT_Q6_K, wd, F, H)]
-    assert all(p is not None for p in planes)
+    pu, pd = capi.build_batch_plane(FMT_Q4_K, wu, F, H), capi.build_batch_plane(FMT_Q6_K, wd, F, H)
+    assert pu is not None and pd is not None
     x = torch.empty(M, H, device=dev)
     q8 = torch.empty(M * (H // 32) * 36, dtype=torch.uint8, device=dev)
     a, b = torch.empty(M, F, device=dev), torch.empty(M, F, device=dev)
@@ -101,26 +100,22 @@ def test_batch_plane_launches_replay(capi, dev):
     def step(stream):
         s = stream.cuda_stream
         capi.quantize_q8_1(x, out=q8, stream=s)
-        capi.gemv(FMT_Q4_K, wu, q8, M, F, H, out=a, stream=s)
-        capi.gemv(FMT_Q6_K, wd, q8, M, F, H, out=b, stream=s)
+        capi.gemv(FMT_Q4_K, wu, q8, M, F, H, out=a, stream=s, plane=pu)
+        capi.gemv(FMT_Q6_K, wd, q8, M, F, H, out=b, stream=s, plane=pd)
 
     inputs = [torch.from_numpy(synth.activations_numpy(M, H, 200 + i)).to(dev) for i in range(3)]
     stream = torch.cuda.Stream()
     eager = []
-    try:
-        with torch.cuda.stream(stream):
-            for inp in inputs:
-                x.copy_(inp)
-                step(stream)
-                stream.synchronize()
-                eager.append((a.clone(), b.clone()))
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                step(stream)
-        torch.cuda.synchronize()
-    finally:
-        capi.detach_batch_plane(wu)
-        capi.detach_batch_plane(wd)
+    with torch.cuda.stream(stream):
+        for inp in inputs:
+            x.copy_(inp)
+            step(stream)
+            stream.synchronize()
+            eager.append((a.clone(), b.clone()))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            step(stream)
+    torch.cuda.synchronize()
     for rep in range(2):
         for i, inp in enumerate(inputs):
             x.copy_(inp)
