@@ -372,6 +372,13 @@ def bench_read_order(args, torch, capi, synth, dev):
              ("quad-lane loads, round robin, 4 steps in flight", 1, 13, 8, 4, 0),
              ("quad-lane loads, 7 contiguous rows, 16 wavefronts, 1 step in flight", 0, 7, 16, 1, 0),
              ("quad-lane loads, 7 rows round robin, 16 wavefronts, 1 step in flight", 1, 7, 16, 1, 0),
+             ("three planes, round robin, 2 steps in flight", 5, 13, 8, 2, 0),
+             ("three planes, round robin, 3 steps in flight", 5, 13, 8, 3, 0),
+             ("three planes, round robin, 4 steps in flight", 5, 13, 8, 4, 0),
+             ("three planes, contiguous rows, 2 steps in flight", 4, 13, 8, 2, 0),
+             ("three planes, 7 rows round robin, 16 wavefronts, 1 step in flight", 5, 7, 16, 1, 0),
+             ("three planes, 7 rows round robin, 16 wavefronts, 2 steps in flight", 5, 7, 16, 2, 0),
+             ("quad-lane loads, round robin, 3 steps in flight", 1, 13, 8, 3, 0),
              ("1 KB stream, region per wavefront, 256 x 1024 threads, 3 loads in flight", 2, 0, 16, 3, 256),
              ("1 KB stream, grid-stride, 256 x 1024 threads, 3 loads in flight", 3, 0, 16, 3, 256),
              ("1 KB stream, region per wavefront, 256 x 1024 threads, 6 loads in flight", 2, 0, 16, 6, 256),

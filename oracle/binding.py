@@ -264,7 +264,27 @@ class Ref:
         self.has_swiglu = hasattr(L, "ref_swiglu")
         if self.has_swiglu:
             L.ref_swiglu.argtypes = [c_void_p, c_void_p, c_void_p, c_int]
+        self.has_route = hasattr(L, "ref_moe_route")
+        if self.has_route:
+            L.ref_softmax_row.argtypes = [c_void_p, c_int, c_int]
+            L.ref_moe_route.argtypes = [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
         self.L = L
+
+    def softmax_row(self, row, variant=0):
+        """primitives::softmax_row_fp32 on one row; variant 0 dispatch, 1 scalar, 2 AVX2, 3 AVX512."""
+        r = np.ascontiguousarray(row, dtype=np.float32).copy()
+        self.L.ref_softmax_row(_p(r), r.size, variant)
+        return r
+
+    def moe_route(self, logits, top_k, normalize=True, variant=0):
+        """CPUMoEKernel::route from the logits on: (ids, weights, probabilities)."""
+        lg = np.ascontiguousarray(logits, dtype=np.float32)
+        T, E = lg.shape
+        ids = np.zeros((T, top_k), np.int32)
+        w = np.zeros((T, top_k), np.float32)
+        probs = np.zeros((T, E), np.float32)
+        self.L.ref_moe_route(_p(lg), T, E, top_k, int(normalize), variant, _p(ids), _p(w), _p(probs))
+        return ids, w, probs
 
     def f16_to_f32(self, h):
         return float(self.L.ref_f16_to_f32(h))

@@ -15,11 +15,13 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstring>
+#include <numeric>
 #include <vector>
 
 #include "kernels/cpu/native_vnni/CPUNativeVNNIGemv.h"
 #include "kernels/cpu/primitives/RMSNormPrimitives.h"
 #include "kernels/cpu/primitives/RoPEPrimitives.h"
+#include "kernels/cpu/primitives/SoftmaxPrimitivesImpl.h"
 #include "kernels/cpu/primitives/SwiGLUPrimitives.h"
 #include "tensors/BlockStructures.h"
 #include "tensors/FP16Utils.h"
@@ -294,5 +296,44 @@ extern "C"
     void ref_swiglu(const float *gate, const float *up, float *out, int n)
     {
         primitives::compute_swiglu_serial(gate, up, out, n);
+    }
+    // The router's softmax (primitives::softmax_row_fp32, SoftmaxPrimitivesImpl.h:412-709), in place.
+    // variant: 0 = the dispatcher CPUMoEKernel::route reaches, 1 scalar, 2 AVX2, 3 AVX512
+    void ref_softmax_row(float *row, int cols, int variant)
+    {
+        if (variant == 1)
+            primitives::softmax_row_fp32_scalar(row, cols, false, 1.0f, 0);
+        else if (variant == 2)
+            primitives::softmax_row_fp32_avx2(row, cols, false, 1.0f, 0);
+        else if (variant == 3)
+            primitives::softmax_row_fp32_avx512(row, cols, false, 1.0f, 0);
+        else
+            primitives::softmax_row_fp32(row, cols, false, 1.0f, 0);
+    }
+    // CPUMoEKernel::route from the logits on (CPUMoEKernel.cpp:51-78): the reference's softmax,
+    // then the statements of its selection -- iota, std::partial_sort by probability, the sum of
+    // the top_k and the division -- which live in a translation unit that needs the whole engine.
+    // probs [n_tokens x n_experts] receives the probabilities.
+    void ref_moe_route(const float *logits, int n_tokens, int n_experts, int top_k, int normalize, int variant,
+                       int32_t *ids, float *weights, float *probs)
+    {
+        std::vector<int> indices(n_experts);
+        for (int t = 0; t < n_tokens; ++t)
+        {
+            float *p = probs + (size_t)t * n_experts;
+            std::memcpy(p, logits + (size_t)t * n_experts, (size_t)n_experts * sizeof(float));
+            ref_softmax_row(p, n_experts, variant);
+            std::iota(indices.begin(), indices.end(), 0);
+            std::partial_sort(indices.begin(), indices.begin() + top_k, indices.end(),
+                              [p](int a, int b) { return p[a] > p[b]; });
+            float topk_sum = 0.0f;
+            for (int k = 0; k < top_k; ++k)
+                topk_sum += p[indices[k]];
+            for (int k = 0; k < top_k; ++k)
+            {
+                ids[(size_t)t * top_k + k] = indices[k];
+                weights[(size_t)t * top_k + k] = normalize ? p[indices[k]] / topk_sum : p[indices[k]];
+            }
+        }
     }
 }

@@ -1,5 +1,5 @@
 """Writes tests/golden/decode_goldens.npz: inputs and the outputs of the reference's own
-RMSNorm, RoPE and SwiGLU primitives (compiled into oracle/_ref from the reference tree by
+RMSNorm, RoPE, SwiGLU and softmax primitives and of the router built on the last (compiled into oracle/_ref from the reference tree by
 oracle/Makefile).  Run in a container that holds the reference; the fixture is data only."""
 from pathlib import Path
 import sys
@@ -40,6 +40,14 @@ def main():
     g[:8] = [-100, -88, -20, -1e-3, 0, 1e-3, 20, 88]
     u = rng.standard_normal(1037).astype(np.float32)
     out["swiglu_gate"], out["swiglu_up"], out["swiglu_out"] = g, u, ref.swiglu(g, u)
+    # the router from the logits on (CPUMoEKernel::route: softmax_row_fp32 as the dispatcher runs it,
+    # partial_sort, renormalisation): 256 experts, top-8, logits of three spreads; no exact ties
+    assert ref.has_route
+    lg = np.concatenate([(rng.standard_normal((6, 256)) * s).astype(np.float32) for s in (1.0, 6.0, 40.0)])
+    ids, w, probs = ref.moe_route(lg, 8, True, 0)
+    _, w_raw, _ = ref.moe_route(lg, 8, False, 0)
+    out["route_logits"], out["route_ids"], out["route_weights"], out["route_probs"] = lg, ids, w, probs
+    out["route_weights_unnormalised"] = w_raw
     np.savez_compressed(Path(__file__).with_name("decode_goldens.npz"), **out)
     print("wrote decode_goldens.npz", {k: np.asarray(v).shape for k, v in out.items()})
 

@@ -10,6 +10,8 @@
 //     pattern 0 / 1: the quad-lane kernel's loads (4 lanes per super-block, 3 x 16 bytes per lane
 //       and step), N rows shared by ceil(N / rows_per_wave) wavefronts, each with its rows
 //       contiguous (0) or dealt round robin (1); depth = steps in flight per wavefront (1, 2, 4).
+//     pattern 4 / 5: the walk of 0 / 1 over a buffer in three planes (heads, first and second halves
+//       of the lanes' groups), so that no two load instructions touch the same cache line; depth 1..4.
 //     pattern 2 / 3: 1 KB per load instruction, `workgroups` workgroups, a region per wavefront
 //       (2) or grid-stride (3); depth = loads in flight per lane (3, 6, 9).
 //   llam_probe_set_batch_tile_rows(rows): sweep override for the rows of weight per tile (16..32)
@@ -20,6 +22,8 @@
 #define LLAM_QL_PROBE_ROWS_ROUND_ROBIN 1
 #define LLAM_QL_PROBE_STREAM_REGION 2
 #define LLAM_QL_PROBE_STREAM_GRID_STRIDE 3
+#define LLAM_QL_PROBE_PLANES_CONTIGUOUS 4
+#define LLAM_QL_PROBE_PLANES_ROUND_ROBIN 5
 
 namespace llamql
 {
@@ -34,7 +38,10 @@ namespace llamql
     // 16-byte head and its two 16-byte pieces; a wavefront step covers 16 super-blocks of the run
     // formed by the wavefront's rows.  ROUND_ROBIN: wavefront j of tw walks rows j, j + tw, ..;
     // otherwise rows j * rows_per_wave .. of its own.  DEPTH steps are in flight per wavefront.
-    template <bool ROUND_ROBIN, int DEPTH>
+    // PLANES: the same walk over a buffer laid out in three planes over all T = N * nsb super-blocks,
+    // heads [T][16] | first halves of the lanes' groups [T][64] | second halves [T][64]: every load
+    // instruction of a wavefront then reads whole runs of bytes nobody else asks for.
+    template <bool ROUND_ROBIN, int DEPTH, bool PLANES = false>
     __global__ void __launch_bounds__(1024)
         read_probe_rows_kernel(const uint8_t *p, int N, int nsb, int rows_per_wave, int *sink)
     {
@@ -64,10 +71,20 @@ namespace llamql
                     s = total - 1;
                 const int lr = s / nsb, sbr = s - lr * nsb;
                 const long row = ROUND_ROBIN ? lr * tw + j : j * rows_per_wave + lr;
-                const uint8_t *sb = p + ((size_t)row * nsb + sbr) * 144;
-                v[u][0] = *reinterpret_cast<const probe_v4i *>(sb);
-                v[u][1] = *reinterpret_cast<const probe_v4i *>(sb + 16 + 32 * l);
-                v[u][2] = *reinterpret_cast<const probe_v4i *>(sb + 32 + 32 * l);
+                if (PLANES)
+                {
+                    const size_t T = (size_t)N * nsb, t = (size_t)row * nsb + sbr;
+                    v[u][0] = *reinterpret_cast<const probe_v4i *>(p + t * 16);
+                    v[u][1] = *reinterpret_cast<const probe_v4i *>(p + T * 16 + t * 64 + 16 * l);
+                    v[u][2] = *reinterpret_cast<const probe_v4i *>(p + T * 80 + t * 64 + 16 * l);
+                }
+                else
+                {
+                    const uint8_t *sb = p + ((size_t)row * nsb + sbr) * 144;
+                    v[u][0] = *reinterpret_cast<const probe_v4i *>(sb);
+                    v[u][1] = *reinterpret_cast<const probe_v4i *>(sb + 16 + 32 * l);
+                    v[u][2] = *reinterpret_cast<const probe_v4i *>(sb + 32 + 32 * l);
+                }
             }
 #pragma unroll
             for (int u = 0; u < DEPTH; ++u)
@@ -105,16 +122,18 @@ namespace llamql
             sink[0] = 1;
     }
 
-    template <bool A>
+    template <bool A, bool PLANES = false>
     void launch_rows(int depth, dim3 grid, dim3 block, hipStream_t st, const uint8_t *p, int N, int nsb, int rpw, int *sink)
     {
         switch (depth)
         {
-        case 1: hipLaunchKernelGGL((read_probe_rows_kernel<A, 1>), grid, block, 0, st, p, N, nsb, rpw, sink); break;
-        case 2: hipLaunchKernelGGL((read_probe_rows_kernel<A, 2>), grid, block, 0, st, p, N, nsb, rpw, sink); break;
-        default: hipLaunchKernelGGL((read_probe_rows_kernel<A, 4>), grid, block, 0, st, p, N, nsb, rpw, sink); break;
+        case 1: hipLaunchKernelGGL((read_probe_rows_kernel<A, 1, PLANES>), grid, block, 0, st, p, N, nsb, rpw, sink); break;
+        case 2: hipLaunchKernelGGL((read_probe_rows_kernel<A, 2, PLANES>), grid, block, 0, st, p, N, nsb, rpw, sink); break;
+        case 3: hipLaunchKernelGGL((read_probe_rows_kernel<A, 3, PLANES>), grid, block, 0, st, p, N, nsb, rpw, sink); break;
+        default: hipLaunchKernelGGL((read_probe_rows_kernel<A, 4, PLANES>), grid, block, 0, st, p, N, nsb, rpw, sink); break;
         }
     }
+
     template <bool A>
     void launch_stream(int depth, dim3 grid, dim3 block, hipStream_t st, const uint8_t *p, size_t chunks, int *sink)
     {
@@ -147,18 +166,23 @@ extern "C" bool llam_probe_read(const void *d_buf, int N, int K, int pattern, in
     hipStream_t st = as_stream(stream);
     const uint8_t *p = static_cast<const uint8_t *>(d_buf);
     const dim3 block((unsigned)waves_per_wg * 64);
-    if (pattern == LLAM_QL_PROBE_ROWS_CONTIGUOUS || pattern == LLAM_QL_PROBE_ROWS_ROUND_ROBIN)
+    if (pattern == LLAM_QL_PROBE_ROWS_CONTIGUOUS || pattern == LLAM_QL_PROBE_ROWS_ROUND_ROBIN ||
+        pattern == LLAM_QL_PROBE_PLANES_CONTIGUOUS || pattern == LLAM_QL_PROBE_PLANES_ROUND_ROBIN)
     {
-        if (rows_per_wave < 1 || (depth != 1 && depth != 2 && depth != 4))
-            return fail(fn, "rows_per_wave=%d depth=%d (depth 1, 2 or 4)", rows_per_wave, depth);
+        if (rows_per_wave < 1 || depth < 1 || depth > 4)
+            return fail(fn, "rows_per_wave=%d depth=%d (depth 1..4)", rows_per_wave, depth);
         if ((long)rows_per_wave * nsb > 0x7FFFFFF)
             return fail(fn, "run too long");
         const long tw = ((long)N + rows_per_wave - 1) / rows_per_wave;
         const dim3 grid((unsigned)((tw + waves_per_wg - 1) / waves_per_wg));
         if (pattern == LLAM_QL_PROBE_ROWS_ROUND_ROBIN)
             launch_rows<true>(depth, grid, block, st, p, N, nsb, rows_per_wave, d_sink);
-        else
+        else if (pattern == LLAM_QL_PROBE_ROWS_CONTIGUOUS)
             launch_rows<false>(depth, grid, block, st, p, N, nsb, rows_per_wave, d_sink);
+        else if (pattern == LLAM_QL_PROBE_PLANES_ROUND_ROBIN)
+            launch_rows<true, true>(depth, grid, block, st, p, N, nsb, rows_per_wave, d_sink);
+        else
+            launch_rows<false, true>(depth, grid, block, st, p, N, nsb, rows_per_wave, d_sink);
         return launched(fn);
     }
     if (pattern == LLAM_QL_PROBE_STREAM_REGION || pattern == LLAM_QL_PROBE_STREAM_GRID_STRIDE)

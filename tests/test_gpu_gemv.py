@@ -719,11 +719,12 @@ def test_read_probe_runs_and_checks_its_arguments(capi, dev):
     buf = torch.randint(0, 256, (N * (K // 256) * 144 + 64,), dtype=torch.uint8, device=dev)
     guard = buf[-64:].clone()
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
-    for pattern, rpw, depth, wgs in ((0, 3, 2, 0), (1, 3, 1, 0), (1, 5, 4, 0), (2, 0, 3, 4), (3, 0, 6, 4), (3, 0, 9, 2)):
+    for pattern, rpw, depth, wgs in ((0, 3, 2, 0), (1, 3, 1, 0), (1, 5, 4, 0), (2, 0, 3, 4), (3, 0, 6, 4), (3, 0, 9, 2), (4, 3, 3, 0),
+                                     (5, 5, 2, 0)):
         assert lib.llam_probe_read(buf.data_ptr(), N, K, pattern, rpw, 4, depth, wgs, sink.data_ptr(), 0, None), capi.last_error()
     sync()
     assert torch.equal(buf[-64:], guard) and int(sink[0]) in (0, 1)
-    for args in ((buf.data_ptr(), N, K, 7, 3, 4, 2, 0), (buf.data_ptr(), N, K, 0, 3, 4, 3, 0), (buf.data_ptr(), N, 1024, 0, 3, 4, 2, 0),
+    for args in ((buf.data_ptr(), N, K, 7, 3, 4, 2, 0), (buf.data_ptr(), N, K, 0, 3, 4, 5, 0), (buf.data_ptr(), N, 1024, 0, 3, 4, 2, 0),
                  (buf.data_ptr(), N, K, 2, 0, 4, 3, 0), (0, N, K, 0, 3, 4, 2, 0), (buf.data_ptr(), N, K, 0, 3, 17, 2, 0)):
         assert not lib.llam_probe_read(*args, sink.data_ptr(), 0, None)
 

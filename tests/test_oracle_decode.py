@@ -247,6 +247,12 @@ def test_committed_reference_vectors(oracle):
         got = oracle.rope_head(z["rope_head"], int(pos), f)
         assert np.abs(got - z["rope_scalar"][i]).max() <= 4.8e-7 * np.abs(z["rope_head"]).max()
         assert np.abs(got - z["rope_token_q"][i][:128]).max() <= 5e-6
+    if "route_ids" in z:
+        # the router: the reference's softmax (as its dispatcher runs it), selection and renormalisation
+        ids, w, probs = oracle.route(z["route_logits"], 8, True)
+        assert np.array_equal(ids, z["route_ids"]) and np.array_equal(probs, z["route_probs"])
+        assert np.array_equal(w, z["route_weights"])
+        assert np.array_equal(oracle.route(z["route_logits"], 8, False)[1], z["route_weights_unnormalised"])
     if "swiglu_out" in z:
         mine = oracle.swiglu(z["swiglu_gate"], z["swiglu_up"])
         assert (np.abs(mine - z["swiglu_out"]) <= 8e-6 * np.abs(mine) + 1e-30).all()

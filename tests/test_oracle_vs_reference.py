@@ -41,3 +41,32 @@ def test_gemm_float_exact(oracle, ref, fmt, M, monkeypatch):
         C2 = ref.gemm(fmt, W, N, K, q8, isa=isa)
         C = oracle.gemm(fmt, W, K, q8)
         assert np.array_equal(C.view(np.uint32), C2.view(np.uint32))
+
+
+def test_router_bit_exact(oracle, ref):
+    """qlo_moe_route against CPUMoEKernel::route from the logits on (the reference's softmax_row_fp32 in every ISA
+    variant, its partial_sort and renormalisation): probabilities, ids and weights bit for bit.  With exactly equal
+    probabilities the reference's partial_sort leaves the order to the library; the restatement (and the GPU
+    kernel) take the lower expert id first, so ties are compared as sets of weights only."""
+    if not ref.has_route:
+        pytest.skip("oracle/_ref predates the router door")
+    rng = np.random.default_rng(3)
+    for spread in (0.5, 1.0, 8.0, 30.0):   # (wider spreads underflow to exact zeros: ties, below)
+        lg = (rng.standard_normal((64, 256)) * spread).astype(np.float32)
+        for variant in (0, 1, 2, 3):
+            for normalize in (True, False):
+                ids, w, probs = ref.moe_route(lg, 8, normalize, variant)
+                oi, ow, op = oracle.route(lg, 8, normalize)
+                assert np.array_equal(op, probs) and np.array_equal(oi, ids) and np.array_equal(ow, w), (spread, variant)
+    lg = rng.standard_normal((32, 256)).astype(np.float32)
+    for t in range(32):
+        top = np.argsort(-lg[t])[:10]
+        lg[t, top[3]] = lg[t, top[4]] = lg[t, top[5]]
+        lg[t, top[7]] = lg[t, top[8]]          # a tie across the cut after the eighth
+    ids, w, probs = ref.moe_route(lg, 8, True, 0)
+    oi, ow, op = oracle.route(lg, 8, True)
+    assert np.array_equal(op, probs) and np.array_equal(ow, w)
+    for t in range(32):
+        assert np.array_equal(np.sort(op[t][oi[t]]), np.sort(probs[t][ids[t]]))
+        order = np.lexsort((oi[t], -op[t][oi[t]]))          # by probability, ties by expert id
+        assert np.array_equal(order, np.arange(8)), t
