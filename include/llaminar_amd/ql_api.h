@@ -350,6 +350,21 @@ bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts,
                       int top_k, int hidden, int inter, int accumulate,
                       int device_id, void *stream);
 
+/* llam_ql_moe_gate_up followed by llam_ql_swiglu_quantize, the same Q8_1 bytes:
+ *   d_q8_out [(t*top_k+s)][inter/32] = Q8_1(silu(W_gate[e] . q8(hidden[t])) * (W_up[e] . q8(hidden[t])))
+ * For IQ3_S experts with hidden/256 in {2,4,8,16} this is ONE launch: a workgroup owns the 32
+ * gate and 32 up rows of one Q8_1 block, so the fp32 intermediate never leaves the chip and
+ * d_gate_scratch / d_up_scratch may be NULL.  Every other format and row length runs the two
+ * launches through the scratch rows (fp32 [n_tokens*top_k x inter] each; NULL is refused there).
+ * Blocks of skipped slots (id outside [0,n_experts), NULL matrix) are left untouched in the
+ * one-launch form and are quantised from whatever the scratch holds in the other; no later
+ * stage reads them.  Counterpart of the fused decode epilogue of
+ * groupedExpertGateUpDecodeFromRouting + swiGLU (IMoEKernel.h:378-643, :168-180). */
+bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                                const int32_t *d_ids, const void *d_q8, float *d_gate_scratch,
+                                float *d_up_scratch, void *d_q8_out, int n_tokens, int top_k,
+                                int hidden, int inter, int device_id, void *stream);
+
 /* ---- batches: tokens grouped by expert ---------------------------------------------------
  * With several tokens the same expert is usually picked more than once (16 tokens x 8 slots
  * of 256 experts hit about 100 distinct ones, and an always-on shared expert serves all 16).

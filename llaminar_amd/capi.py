@@ -86,6 +86,8 @@ SIGNATURES = {
                                             c_int, c_void_p, c_int, c_void_p]),
     "llam_ql_moe_gate_up": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                      c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_gate_up_swiglu": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_swiglu_quantize": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                   c_int, c_int, c_int, c_int, c_void_p]),
@@ -445,6 +447,20 @@ def moe_gate_up(fmt: int, table, n_experts: int, ids, q8, n_tokens: int, top_k: 
     _check(load().llam_ql_moe_gate_up(fmt, _ptr(table), n_experts, _ptr(ids), _ptr(q8), _ptr(gate), _ptr(up),
                                       n_tokens, top_k, hidden, inter, _dev(q8), _stream(stream)), "moe_gate_up")
     return gate, up
+
+
+def moe_gate_up_swiglu(fmt: int, table, n_experts: int, ids, q8, n_tokens: int, top_k: int, hidden: int, inter: int,
+                       q8_out=None, scratch=None, stream=None):
+    """Q8_1 of silu(gate) * up for every token slot; scratch: (gate, up) fp32 rows for the shapes that need them."""
+    import torch
+
+    if q8_out is None:
+        q8_out = torch.zeros(n_tokens * top_k * (inter // 32) * 36, dtype=torch.uint8, device=q8.device)
+    g, u = scratch if scratch is not None else (None, None)
+    _check(load().llam_ql_moe_gate_up_swiglu(fmt, _ptr(table), n_experts, _ptr(ids), _ptr(q8), _ptr(g), _ptr(u),
+                                             _ptr(q8_out), n_tokens, top_k, hidden, inter, _dev(q8), _stream(stream)),
+           "moe_gate_up_swiglu")
+    return q8_out
 
 
 def swiglu_quantize(gate, up, want_act: bool = False, stream=None):

@@ -152,19 +152,26 @@ namespace llamql
         v4i lo, hi;
         int tail;
     };
+    // thread `tid` of `nthreads` that share the `total` blocks (a workgroup, or one wavefront of it)
     template <int PASSES>
-    __device__ __forceinline__ void quad_act_issue(QuadActRaw (&r)[PASSES], const uint32_t *q8, int total)
+    __device__ __forceinline__ void quad_act_issue(QuadActRaw (&r)[PASSES], const uint32_t *q8, int total, int tid,
+                                                   int nthreads)
     {
 #pragma unroll
         for (int p = 0; p < PASSES; ++p)
         {
-            int idx = (int)threadIdx.x + p * (int)blockDim.x;
+            int idx = tid + p * nthreads;
             idx = idx < total ? idx : total - 1;
             const uint32_t *src = q8 + (size_t)idx * 9;
             asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r[p].lo) : "v"(src));
             asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=&v"(r[p].hi) : "v"(src));
             asm volatile("global_load_dword %0, %1, off offset:32" : "=&v"(r[p].tail) : "v"(src));
         }
+    }
+    template <int PASSES>
+    __device__ __forceinline__ void quad_act_issue(QuadActRaw (&r)[PASSES], const uint32_t *q8, int total)
+    {
+        quad_act_issue(r, q8, total, (int)threadIdx.x, (int)blockDim.x);
     }
     // until at most NEWER vector memory operations issued after the activation loads are pending
     template <int NEWER, int PASSES>
@@ -175,15 +182,15 @@ namespace llamql
         for (int p = 0; p < PASSES; ++p)
             asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r[p].lo), "+v"(r[p].hi), "+v"(r[p].tail) : "n"(NEWER));
     }
-    template <class Q>
-    __device__ __forceinline__ void quad_act_store(const QuadActRaw (&r)[QUAD_ACT_PASSES], int nsb, int total,
-                                                   uint8_t *aq, int aq_stride)
+    template <class Q, int PASSES>
+    __device__ __forceinline__ void quad_act_store(const QuadActRaw (&r)[PASSES], int nsb, int total,
+                                                   uint8_t *aq, int aq_stride, int tid, int nthreads)
     {
         const int nkb = nsb * 8;
 #pragma unroll
-        for (int p = 0; p < QUAD_ACT_PASSES; ++p)
+        for (int p = 0; p < PASSES; ++p)
         {
-            const int idx = (int)threadIdx.x + p * (int)blockDim.x;
+            const int idx = tid + p * nthreads;
             if (idx < total)
             {
                 const int m = idx / nkb, kb = idx - m * nkb;
@@ -198,6 +205,13 @@ namespace llamql
                 *reinterpret_cast<v4i *>(base + (odd * 2 + 1) * 64) = (v4i){r[p].hi.y, r[p].hi.z, r[p].hi.w, r[p].tail};
             }
         }
+    }
+
+    template <class Q, int PASSES>
+    __device__ __forceinline__ void quad_act_store(const QuadActRaw (&r)[PASSES], int nsb, int total,
+                                                   uint8_t *aq, int aq_stride)
+    {
+        quad_act_store<Q, PASSES>(r, nsb, total, aq, aq_stride, (int)threadIdx.x, (int)blockDim.x);
     }
 
     // One lane's share (float4 number i of the row) of a quantised 32-element block into the

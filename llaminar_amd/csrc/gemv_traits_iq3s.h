@@ -122,6 +122,35 @@ namespace llamql
             dst[i] = src[i];
     }
 
+    // The same in two halves, for a kernel that has dependent loads to wait for while the tables
+    // travel: one 16-byte piece per thread (workgroups of at least IQ3S_TABLE_BYTES / 16 threads),
+    // asked for with an assembly load so that the kernel decides where it is waited for; never
+    // predicated (threads past the end re-read the last piece).
+    struct IQ3STablesRaw
+    {
+        int v __attribute__((ext_vector_type(4)));
+    };
+    constexpr int IQ3S_TABLE_THREADS = IQ3S_TABLE_BYTES / 16;
+    __device__ __forceinline__ void iq3s_tables_issue(IQ3STablesRaw &r)
+    {
+        const int i = min((int)threadIdx.x, IQ3S_TABLE_THREADS - 1);
+        const uint4 *src = reinterpret_cast<const uint4 *>(&g_iq3s_tables) + i;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.v) : "v"(src));
+    }
+    // until at most NEWER vector memory operations issued after the tables' load are pending
+    template <int NEWER>
+    __device__ __forceinline__ void iq3s_tables_wait(IQ3STablesRaw &r)
+    {
+        static_assert(NEWER <= 63, "vmcnt is a 6-bit counter");
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r.v) : "n"(NEWER));
+    }
+    __device__ __forceinline__ void iq3s_tables_store(const IQ3STablesRaw &r)
+    {
+        typedef int v4 __attribute__((ext_vector_type(4)));
+        if (threadIdx.x < IQ3S_TABLE_THREADS)
+            reinterpret_cast<v4 *>(iq3s_tables_lds())[threadIdx.x] = r.v;
+    }
+
     // (byte N of x) << sh in one instruction (sub-dword addressing of the operand).  sh is a
     // register operand; it holds a small constant.
     template <int N>
@@ -277,6 +306,13 @@ namespace llamql
         static constexpr int RESIDENT_WAVES = 16;
         static bool addressable(long N, int SB) { return (double)N * SB * 64.0 < 4.0e9; }
         __device__ __forceinline__ static void stage() { iq3s_stage_tables(); }
+        // the tables fetched ahead (workgroups of at least TABLE_THREADS threads)
+        typedef IQ3STablesRaw TablesRaw;
+        static constexpr int TABLE_THREADS = IQ3S_TABLE_THREADS;
+        __device__ __forceinline__ static void tables_issue(TablesRaw &r) { iq3s_tables_issue(r); }
+        template <int NEWER>
+        __device__ __forceinline__ static void tables_wait(TablesRaw &r) { iq3s_tables_wait<NEWER>(r); }
+        __device__ __forceinline__ static void tables_store(const TablesRaw &r) { iq3s_tables_store(r); }
 
         struct Raw
         {

@@ -346,10 +346,11 @@ namespace llaminar_amd
                                                         stream_));
         }
         return forward(fn, llam_ql_quantize_q8_1(input->data, q8, T, d_model, device_id_, stream_)) &&
-               forward(fn, llam_ql_moe_gate_up(tg->fmt, tg->d_entries, tg->num_experts, rt->topk_expert_ids, q8, gate,
-                                               up, T, top_k, d_model, intermediate, device_id_, stream_)) &&
-               forward(fn, llam_ql_swiglu_quantize(gate, up, nullptr, qa, (int)rows, intermediate, device_id_,
-                                                   stream_)) &&
+               // gate/up, SwiGLU and its Q8_1 quantiser: one launch where the format and row length allow,
+               // else two through the fp32 rows
+               forward(fn, llam_ql_moe_gate_up_swiglu(tg->fmt, tg->d_entries, tg->num_experts, rt->topk_expert_ids, q8,
+                                                      gate, up, qa, T, top_k, d_model, intermediate, device_id_,
+                                                      stream_)) &&
                forward(fn, llam_ql_moe_down(td->fmt, td->d_entries, td->num_experts, rt->topk_expert_ids,
                                             rt->topk_weights, qa, output->data, T, top_k, d_model, intermediate, 0,
                                             device_id_, stream_));

@@ -17,27 +17,6 @@ namespace llamql
     // the top_k.  All reductions are wavefront shuffles: no LDS, no barriers.
     constexpr int ROUTE_MAX_PER_LANE = 32; // up to 2048 experts
 
-    // Maximum of a 64-bit key over the wavefront (data-parallel primitives inside a row of
-    // 16 lanes, four lane reads across rows); every lane returns it.
-    __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
-    {
-        auto step = [&](unsigned long long o) { v = o > v ? o : v; };
-        auto join = [](int hi, int lo) { return ((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo; };
-        step(join(dpp_i32<DPP_QUAD_XOR1>((int)(v >> 32)), dpp_i32<DPP_QUAD_XOR1>((int)v)));
-        step(join(dpp_i32<DPP_QUAD_XOR2>((int)(v >> 32)), dpp_i32<DPP_QUAD_XOR2>((int)v)));
-        step(join(dpp_i32<DPP_ROW_HALF_MIRROR>((int)(v >> 32)), dpp_i32<DPP_ROW_HALF_MIRROR>((int)v)));
-        step(join(dpp_i32<DPP_ROW_MIRROR>((int)(v >> 32)), dpp_i32<DPP_ROW_MIRROR>((int)v)));
-        unsigned long long r = 0ull;
-#pragma unroll
-        for (int row = 0; row < 4; ++row)
-        {
-            const unsigned long long o = join(__builtin_amdgcn_readlane((int)(v >> 32), 16 * row),
-                                              __builtin_amdgcn_readlane((int)v, 16 * row));
-            r = o > r ? o : r;
-        }
-        return r;
-    }
-
     // Workgroups past the tokens (optional) quantise `q_blocks` 32-element blocks of q_x to Q8_1
     // with the stand-alone quantiser's arithmetic: the hidden state the expert GEMVs read does
     // not depend on the routing, so its quantiser rides in the same launch.
@@ -73,9 +52,7 @@ namespace llamql
             p[i] = (e < n_experts) ? l[e] : -INFINITY;
             mx = fmaxf(mx, p[i]);
         }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1)
-            mx = fmaxf(mx, __shfl_xor(mx, off));
+        mx = wave_max(mx);
         if (!isfinite(mx))
             mx = 0.0f;
 
@@ -105,31 +82,38 @@ namespace llamql
             if (p[i] >= 0.0f)
                 p[i] = p[i] * inv;
 
-        // arg-max as a maximum over 64-bit keys: probability bits above, inverted expert id
-        // below (probabilities are >= 0, so their bit patterns order like the values; the
-        // lower id wins a tie); retired and padding entries get key 0
-        auto key_of = [&](int i) -> unsigned long long {
-            return p[i] >= 0.0f ? ((unsigned long long)__float_as_uint(p[i]) << 32) | (0xFFFFFFFFu - (uint32_t)(lane + i * WAVE))
-                                : 0ull;
-        };
-        float my_top = 0.0f; // lane k keeps the k-th winner's probability
+        // top_k rounds of arg-max: the largest live probability over the wavefront, then the lowest
+        // expert id that holds it (expert e sits in p[e / 64] of lane e % 64: the first i with a
+        // match, then the lowest matching lane); retired and padding entries are -1, below every
+        // probability.  Lane k keeps the k-th winner.
+        float my_top = 0.0f;
+        int my_id = -1;
         float topk_sum = 0.0f;
         for (int k = 0; k < top_k; ++k)
         {
-            unsigned long long best = 0ull;
+            float best = p[0];
 #pragma unroll
-            for (int i = 0; i < PER; ++i)
+            for (int i = 1; i < PER; ++i)
+                best = fmaxf(best, p[i]);
+            best = wave_max(best); // every lane now holds the winner's probability
+            int best_e = -1;
+            float bp = 0.0f;
+            if (best >= 0.0f) // uniform; false only when nothing selectable is left (NaN logits)
             {
-                const unsigned long long ki = key_of(i);
-                best = ki > best ? ki : best;
+                bp = best;
+#pragma unroll
+                for (int i = PER - 1; i >= 0; --i)
+                {
+                    const unsigned long long hit = __ballot(p[i] == best);
+                    if (hit) // uniform
+                        best_e = i * WAVE + (int)__builtin_ctzll(hit);
+                }
             }
-            best = wave_max_u64(best); // every lane now holds the winner
-            const float bp = __uint_as_float((uint32_t)(best >> 32));
-            const int best_e = (int)(0xFFFFFFFFu - (uint32_t)best);
             if (lane == k)
+            {
                 my_top = bp;
-            if (lane == 0)
-                ids[(size_t)t * slot_stride + k] = best_e;
+                my_id = best_e;
+            }
             topk_sum += bp; // same order on every lane: k = 0, 1, ...
 #pragma unroll
             for (int i = 0; i < PER; ++i)
@@ -137,7 +121,10 @@ namespace llamql
                     p[i] = -1.0f; // retire the winner
         }
         if (lane < top_k)
+        {
+            ids[(size_t)t * slot_stride + lane] = my_id;
             weights[(size_t)t * slot_stride + lane] = normalize ? __fdiv_rn(my_top, topk_sum) : my_top;
+        }
     }
 
     // ---- router logits -------------------------------------------------------------------
@@ -180,6 +167,15 @@ namespace llamql
         int n_experts, top_k, hidden, inter;
         int rows_per_wave, gshift, accumulate;
     };
+
+    // A pointer every lane holds, moved to scalar registers (the weight loads take their base there).
+    __device__ __forceinline__ const void *uniform_ptr(const void *p)
+    {
+        const uint64_t v = (uint64_t)p;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
+    }
 
     // grid: (workgroups per matrix, n_tokens*top_k, 2 = gate|up)
     template <class F>
@@ -252,6 +248,12 @@ namespace llamql
         extern __shared__ __attribute__((aligned(16))) uint8_t moe_quad_lds[];
         const int slot = blockIdx.y;
         const int t = slot / m.top_k;
+        const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
+        // what does not depend on the routing goes first: the decode tables and the token's Q8_1 row
+        typename Q::TablesRaw tab;
+        Q::tables_issue(tab);
+        QuadActRaw act[1]; // nsb * 8 <= 128 blocks: one per thread at most
+        quad_act_issue(act, m.q8 + (size_t)t * (m.hidden / 32) * 9, nsb * 8);
         const int e = m.ids[slot];
         if (e < 0 || e >= m.n_experts)
             return; // uniform for the workgroup; outputs of a bad id stay untouched
@@ -259,7 +261,7 @@ namespace llamql
         a.w = blockIdx.z == 0 ? m.experts[e].d_gate : m.experts[e].d_up;
         if (!a.w)
             return; // an expert whose matrices live elsewhere: skipped like a bad id (uniform)
-        const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
+        a.w = uniform_ptr(a.w);
         a.N = m.inter;
         a.SB = nsb;
         float *y = (blockIdx.z == 0 ? m.out0 : m.out1) + (size_t)slot * m.inter;
@@ -284,8 +286,10 @@ namespace llamql
         typename Q::Raw bufA, bufB;
         issue(bufA);
         issue(bufB);
-        quad_stage_q8<Q, 1>(m.q8 + (size_t)t * (m.hidden / 32) * 9, nsb, moe_quad_lds, moe_quad_lds, 0, 0);
-        Q::stage();
+        quad_act_wait<2 * Q::LOADS>(act);
+        Q::template tables_wait<2 * Q::LOADS>(tab); // asked for before the activations
+        quad_act_store<Q>(act, nsb, nsb * 8, moe_quad_lds, 0);
+        Q::tables_store(tab);
         __syncthreads();
         Q::keep(bufA);
         Q::keep(bufB);
@@ -349,23 +353,38 @@ namespace llamql
         const int step0 = ((int)blockIdx.x * MOE_QUAD_WAVES + wave) * m.rows_per_wave;
         const int nsteps = min(m.rows_per_wave, max(0, (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB - step0));
 
-        if (threadIdx.x == 0)
+        // what does not depend on the routing goes first: the decode tables and the token's Q8_1
+        // rows (its slots form one long activation row: slot s at super-blocks s * nsb ..)
+        typename Q::TablesRaw tab;
+        Q::tables_issue(tab);
+        QuadActRaw act[QUAD_ACT_PASSES];
+        const int total_blk = nsb * 8 * m.top_k;
+        const uint32_t *q8_token = m.q8 + (size_t)t * m.top_k * (m.inter / 32) * 9;
+        quad_act_issue(act, q8_token, total_blk);
+        if (wave == 0)
         {
-            int n = 0;
-            for (int s = 0; s < m.top_k; ++s)
+            // the live slots (good id, matrix present), in ascending order: a lane per slot
+            const bool in = lane < m.top_k;
+            const int e = in ? m.ids[t * m.top_k + lane] : -1;
+            const void *w = (e >= 0 && e < m.n_experts) ? m.experts[e].d_down : nullptr;
+            const unsigned long long mask = __ballot(w != nullptr);
+            if (w) // a bad id, or an expert whose matrices live elsewhere, is skipped
             {
-                const int e = m.ids[t * m.top_k + s];
-                const void *w = (e >= 0 && e < m.n_experts) ? m.experts[e].d_down : nullptr;
-                if (w) // a bad id, or an expert whose matrices live elsewhere, is skipped
-                {
-                    live[n].w = w;
-                    live[n].weight = m.weights[t * m.top_k + s];
-                    live[n].slot = s;
-                    ++n;
-                }
+                const int pos = __popcll(mask & ((1ull << lane) - 1ull));
+                live[pos].w = w;
+                live[pos].weight = m.weights[t * m.top_k + lane];
+                live[pos].slot = lane;
             }
-            n_live_s = n;
+            if (lane == 0)
+                n_live_s = __popcll(mask);
         }
+        quad_act_wait<0>(act);
+        Q::template tables_wait<0>(tab);
+        if (total_blk <= QUAD_ACT_PASSES * (int)blockDim.x) // uniform
+            quad_act_store<Q>(act, nsb * m.top_k, total_blk, moe_quad_lds, 0);
+        else
+            quad_stage_q8<Q, 1>(q8_token, nsb * m.top_k, moe_quad_lds, moe_quad_lds, 0, 0);
+        Q::tables_store(tab);
         __syncthreads();
         const int n_live = n_live_s;
         if (n_live == 0) // uniform
@@ -403,13 +422,6 @@ namespace llamql
         typename Q::Raw bufA, bufB;
         issue(bufA);
         issue(bufB);
-        // the token's slots form one long activation row: slot s at super-blocks s * nsb ..
-        quad_stage_q8<Q, 1>(m.q8 + (size_t)t * m.top_k * (m.inter / 32) * 9, nsb * m.top_k, moe_quad_lds, moe_quad_lds,
-                            0, 0);
-        Q::stage();
-        __syncthreads();
-        Q::keep(bufA);
-        Q::keep(bufB);
 
         const uint8_t *aq_lane = moe_quad_lds + (grp & (nsb - 1)) * QUAD_SB_LDS + (l << 4);
         const int seg_mask = (4 << nsb_log2) - 1;
@@ -422,14 +434,18 @@ namespace llamql
             float v = moe_quad_step<Q>(buf, lc, aq_lane + (size_t)slot * nsb * QUAD_SB_LDS);
             v = sb < total ? v : 0.0f;
             const float val = live[k].weight * moe_quad_row_sum(v, nsb_log2);
-            y = k == 0 ? val : y + val; // the first live slot starts the sum
+            const bool writer = sb < total && (lane & seg_mask) == 0;
+            float *const dst = m.out0 + (size_t)t * m.hidden + (writer ? (sb >> nsb_log2) : 0);
+            // the first live slot starts the sum: from what the output holds when accumulating
+            // (((out + v0) + v1) + .., the per-slot kernel's order), else from nothing
+            if (k == 0)
+                y = (m.accumulate && writer) ? *dst + val : val;
+            else
+                y = y + val;
             if (++k == n_live)
             {
-                if (sb < total && (lane & seg_mask) == 0)
-                {
-                    float *dst = m.out0 + (size_t)t * m.hidden + (sb >> nsb_log2);
-                    *dst = m.accumulate ? (*dst + y) : y;
-                }
+                if (writer)
+                    *dst = y;
                 k = 0;
                 ++step;
             }
@@ -451,6 +467,281 @@ namespace llamql
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end
         Q::keep(bufA);
         Q::keep(bufB);
+    }
+
+    // Down projection of ONE token's slots when there is little work per compute unit (a few tokens):
+    // wavefront s of the workgroup takes slot s, so the loads of every slot of a row range are in
+    // flight at once and the launch is one memory round trip deep instead of one per slot.  The
+    // launch is a chain of dependent loads (id -> expert table -> weights); what does not depend on
+    // the routing -- the decode tables and the wavefront's own Q8_1 row -- is asked for first and
+    // staged while the weights travel.  The wavefronts leave their rows' dot products in LDS; after
+    // one barrier a lane per row adds the live slots in ascending order with their routing weights
+    // -- the arithmetic and order of moe_down_quad_kernel, the same bits.
+    // grid: (workgroups per matrix, n_tokens), max(top_k, MOE_SLOTWAVE_MIN_WAVES) wavefronts;
+    // m.rows_per_wave: steps per wavefront (1..MOE_SLOTWAVE_MAX_STEPS), m.gshift: log2(nsb).
+    constexpr int MOE_SLOTWAVE_MAX_STEPS = 4;
+    template <class Q>
+    __global__ void __launch_bounds__(MOE_QUAD_MAX_SLOTS *WAVE) moe_down_slotwave_kernel(const MoEArgs m)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t moe_quad_lds[];
+        __shared__ float slot_weight[MOE_QUAD_MAX_SLOTS];
+        __shared__ int slot_live[MOE_QUAD_MAX_SLOTS];
+        constexpr int NS = MOE_SLOTWAVE_MAX_STEPS;
+        const int t = blockIdx.y;
+        const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int l = lane & 3, grp = lane >> 2;
+        const typename Q::Lane lc = Q::lane_consts(l);
+        const int total = m.hidden * nsb; // super-blocks of one down matrix
+        const int spw = m.rows_per_wave;
+        const int step0 = (int)blockIdx.x * spw;
+        const int all_steps = (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+        const int nsteps = min(spw, max(0, all_steps - step0));
+        const int rows_per_step = QUAD_STEP_SB >> nsb_log2;
+        const int rows_wg = spw * rows_per_step;
+        float *part = reinterpret_cast<float *>(moe_quad_lds + (size_t)m.top_k * nsb * QUAD_SB_LDS); // [slot][rows_wg]
+
+        typename Q::TablesRaw tab;
+        Q::tables_issue(tab);
+        const bool has_slot = wave < m.top_k; // uniform per wavefront
+        const int slot = has_slot ? wave : 0;
+        // this wavefront's slot: its Q8_1 row (nsb * 8 <= 128 blocks: two per lane at most)
+        QuadActRaw act[QUAD_ACT_PASSES];
+        const int nkb = nsb * 8;
+        quad_act_issue(act, m.q8 + ((size_t)t * m.top_k + slot) * (size_t)nkb * 9, nkb, lane, WAVE);
+        const int e = has_slot ? m.ids[t * m.top_k + slot] : -1;
+        const void *w = (e >= 0 && e < m.n_experts) ? m.experts[e].d_down : nullptr;
+        const bool mine = w != nullptr; // a bad id, or an expert whose matrices live elsewhere, is skipped
+        if (has_slot && lane == 0)
+        {
+            slot_live[slot] = mine ? 1 : 0;
+            slot_weight[slot] = mine ? m.weights[t * m.top_k + slot] : 0.0f;
+        }
+        typename Q::Raw buf[NS];
+        uint8_t *aq = moe_quad_lds + (size_t)slot * nsb * QUAD_SB_LDS;
+        if (mine) // uniform
+        {
+            GemvArgs a; // weight addressing only
+            a.N = m.hidden;
+            a.SB = nsb;
+            a.w = uniform_ptr(w);
+            // every step's loads go out at once; never predicated: past the end a lane re-reads an earlier super-block
+#pragma unroll
+            for (int i = 0; i < NS; ++i)
+            {
+                const int st = i < nsteps ? i : 0;
+                const size_t ti = (size_t)min((step0 + st) * QUAD_STEP_SB + grp, total - 1);
+                const typename Q::Cursor wc = Q::cursor(a, ti, ti, lc);
+                Q::load(buf[i], wc, lc, true);
+            }
+            quad_act_wait<NS * Q::LOADS>(act);
+            Q::template tables_wait<NS * Q::LOADS>(tab); // asked for before the activations
+            quad_act_store<Q>(act, nsb, nkb, aq, 0, lane, WAVE);
+        }
+        else
+        {
+            quad_act_wait<0>(act);
+            Q::template tables_wait<0>(tab);
+        }
+        Q::tables_store(tab);
+        __syncthreads(); // decode tables, every wavefront's activations, the slots' weights and flags
+        if (mine)
+        {
+#pragma unroll
+            for (int i = 0; i < NS; ++i)
+                Q::keep(buf[i]);
+            const uint8_t *aq_lane = aq + (grp & (nsb - 1)) * QUAD_SB_LDS + (l << 4);
+            const int seg_mask = (4 << nsb_log2) - 1;
+#pragma unroll
+            for (int i = 0; i < NS; ++i)
+            {
+                // loads issued after step i's: those of the steps behind it
+                switch (i)
+                {
+                case 0: Q::template wait<Q::LOADS *(NS - 1)>(buf[i]); break;
+                case 1: Q::template wait<Q::LOADS *(NS - 2)>(buf[i]); break;
+                case 2: Q::template wait<Q::LOADS *(NS - 3)>(buf[i]); break;
+                default: Q::template wait<0>(buf[i]); break;
+                }
+                if (i < nsteps) // uniform
+                {
+                    const int sb = (step0 + i) * QUAD_STEP_SB + grp;
+                    float v = moe_quad_step<Q>(buf[i], lc, aq_lane);
+                    v = sb < total ? v : 0.0f;
+                    const float tot = moe_quad_row_sum(v, nsb_log2);
+                    if ((lane & seg_mask) == 0)
+                        part[slot * rows_wg + i * rows_per_step + (grp >> nsb_log2)] = tot;
+                }
+            }
+        }
+        __syncthreads();
+        // one lane per row: the live slots in ascending order
+        for (int r = threadIdx.x; r < rows_wg; r += blockDim.x)
+        {
+            const long row = (long)step0 * rows_per_step + r;
+            if (row >= m.hidden)
+                break;
+            float *dst = m.out0 + (size_t)t * m.hidden + row;
+            float y = 0.0f;
+            bool first = true;
+            for (int s = 0; s < m.top_k; ++s)
+            {
+                if (!slot_live[s])
+                    continue;
+                const float val = slot_weight[s] * part[s * rows_wg + r];
+                if (first)
+                    y = m.accumulate ? *dst + val : val;
+                else
+                    y = y + val;
+                first = false;
+            }
+            if (!first || m.accumulate == 0) // no live slot: zeros unless accumulating
+                *dst = y;
+        }
+    }
+
+    // Gate and up projections of one token slot with SwiGLU and the Q8_1 quantiser of the result in the
+    // same launch: a workgroup owns 32 consecutive intermediate rows of BOTH matrices of its slot's
+    // expert, so it holds the 32 gate and 32 up values of one Q8_1 block of silu(gate) * up and
+    // quantises it itself -- the bits of llam_ql_moe_gate_up (quad-lane kernel) followed by
+    // llam_ql_swiglu_quantize, without the fp32 round trip and the second launch.  The decode
+    // tables and the token's Q8_1 row do not depend on the routing: they are asked for before the
+    // id -> expert table -> weights chain and staged while the weights travel.
+    // grid: (inter / 32, n_tokens * top_k), MOE_QUAD_WAVES wavefronts; m.gshift: log2(nsb); the
+    // 4 nsb steps of a workgroup (2 nsb per matrix) are dealt to its wavefronts in order.
+    // q8_out: Q8_1 blocks [n_tokens * top_k][inter / 32]; blocks of skipped slots are left untouched.
+    // NB: steps in flight per wavefront -- 4 when the launch is a latency chain (few slots), 2 (fewer
+    // registers, twice the resident workgroups) when there is work to overlap it with.
+    template <class Q, int NB>
+    __device__ __forceinline__ void moe_gate_up_swiglu_body(const MoEArgs &m, uint32_t *q8_out)
+    {
+        static_assert(MOE_QUAD_WAVES * WAVE >= Q::TABLE_THREADS, "one table piece per thread");
+        static_assert(NB == 2 || NB == 4, "the wait counts below are written for 2 or 4 steps");
+        extern __shared__ __attribute__((aligned(16))) uint8_t moe_quad_lds[];
+        const int slot = blockIdx.y;
+        const int t = slot / m.top_k;
+        const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
+        typename Q::TablesRaw tab;
+        Q::tables_issue(tab);
+        QuadActRaw act[1]; // nsb * 8 <= 128 blocks: one per thread at most
+        quad_act_issue(act, m.q8 + (size_t)t * (m.hidden / 32) * 9, nsb * 8);
+        const int e = m.ids[slot];
+        if (e < 0 || e >= m.n_experts)
+            return; // uniform for the workgroup
+        const void *wg = m.experts[e].d_gate, *wu = m.experts[e].d_up;
+        if (!wg || !wu)
+            return; // an expert whose matrices live elsewhere: skipped like a bad id (uniform)
+        wg = uniform_ptr(wg);
+        wu = uniform_ptr(wu);
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int l = lane & 3, grp = lane >> 2;
+        const typename Q::Lane lc = Q::lane_consts(l);
+        const int per_mat = 2 * nsb;                                         // steps of 32 rows of one matrix
+        const int spw = (2 * per_mat + MOE_QUAD_WAVES - 1) / MOE_QUAD_WAVES; // steps per wavefront (1, 2, 4, 8)
+        const int s0 = wave * spw;                                           // this wavefront's first of the 2 * per_mat steps
+        float *res = reinterpret_cast<float *>(moe_quad_lds + (size_t)nsb * QUAD_SB_LDS); // [2][32]: gate rows, up rows
+
+        GemvArgs a; // weight addressing only
+        a.N = m.inter;
+        a.SB = nsb;
+        auto issue = [&](typename Q::Raw &buf, int i) {
+            const int s = min(s0 + i, 2 * per_mat - 1); // past the end: the last step again, never predicated
+            const int mat = s >= per_mat ? 1 : 0;
+            a.w = uniform_ptr(mat ? wu : wg);
+            const size_t ti = (size_t)blockIdx.x * 32 * nsb + (size_t)(s - mat * per_mat) * QUAD_STEP_SB + grp;
+            const typename Q::Cursor wc = Q::cursor(a, ti, ti, lc);
+            Q::load(buf, wc, lc, true);
+        };
+        typename Q::Raw buf[NB];
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            issue(buf[i], i);
+        quad_act_wait<NB * Q::LOADS>(act);
+        Q::template tables_wait<NB * Q::LOADS>(tab); // asked for before the activations
+        quad_act_store<Q>(act, nsb, nsb * 8, moe_quad_lds, 0);
+        Q::tables_store(tab);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            Q::keep(buf[i]);
+
+        const uint8_t *aq_lane = moe_quad_lds + (grp & (nsb - 1)) * QUAD_SB_LDS + (l << 4);
+        const int seg_mask = (4 << nsb_log2) - 1;
+        auto compute = [&](const typename Q::Raw &r, int s) {
+            if (s < s0 + spw) // uniform (a wavefront with fewer steps than buffers)
+            {
+                const int mat = s >= per_mat ? 1 : 0;
+                const int sb = (s - mat * per_mat) * QUAD_STEP_SB + grp; // within the 32 rows
+                const float v = moe_quad_step<Q>(r, lc, aq_lane);
+                const float tot = moe_quad_row_sum(v, nsb_log2);
+                if ((lane & seg_mask) == 0)
+                    res[mat * 32 + (sb >> nsb_log2)] = tot;
+            }
+        };
+        // Rounds of NB steps.  spw and NB are powers of two, so a round is followed by a whole round
+        // or by none: while one follows, a buffer is asked for again as soon as it is used up and
+        // every wait leaves the other NB - 1 buffers' loads in flight; the last round drains.
+        int i0 = 0;
+        for (; i0 + NB < spw; i0 += NB)
+        {
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+            {
+                Q::template wait<Q::LOADS *(NB - 1)>(buf[i]);
+                compute(buf[i], s0 + i0 + i);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(buf[i], i0 + NB + i);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+        {
+            // loads issued after step i's: those of the steps behind it
+            switch (NB - 1 - i)
+            {
+            case 3: Q::template wait<Q::LOADS * 3>(buf[i]); break;
+            case 2: Q::template wait<Q::LOADS * 2>(buf[i]); break;
+            case 1: Q::template wait<Q::LOADS * 1>(buf[i]); break;
+            default: Q::template wait<0>(buf[i]); break;
+            }
+            compute(buf[i], s0 + i0 + i);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            Q::keep(buf[i]);
+        __syncthreads();
+        if (wave == 0)
+        {
+            // eight lanes quantise the block (the lane mapping of the stand-alone quantiser); the
+            // other lanes of the wavefront run along on the same values and store nothing
+            const int sub = lane & 7;
+            const float4 g = reinterpret_cast<const float4 *>(res)[sub];
+            const float4 u = reinterpret_cast<const float4 *>(res + 32)[sub];
+            const Q8Lane q = q8_1_quantize_lane(swiglu4(g, u));
+            if (lane < 8)
+            {
+                uint32_t *dst = q8_out + ((size_t)slot * (m.inter / 32) + blockIdx.x) * 9;
+                dst[1 + sub] = q.packed;
+                if (sub == 0)
+                    dst[0] = q.head;
+            }
+        }
+    }
+
+    template <class Q>
+    __global__ void __launch_bounds__(MOE_QUAD_WAVES *WAVE) moe_gate_up_swiglu_kernel(const MoEArgs m, uint32_t *q8_out)
+    {
+        moe_gate_up_swiglu_body<Q, 4>(m, q8_out);
+    }
+    // many slots: two steps in flight, fewer registers, three resident workgroups per compute unit
+    template <class Q>
+    __global__ void __launch_bounds__(MOE_QUAD_WAVES *WAVE)
+    moe_gate_up_swiglu_dense_kernel(const MoEArgs m, uint32_t *q8_out)
+    {
+        moe_gate_up_swiglu_body<Q, 2>(m, q8_out);
     }
 
     // grid: (workgroups per matrix, n_tokens).  Slots are walked in ascending
@@ -586,7 +877,11 @@ namespace llamql
             if (r + 1 < m.rows_per_wave)
                 load_rows(raw, row + (long)GEMV_WAVES * R);
 
-            float y = 0.0f;
+            // accumulate: the slots are added one by one onto what the output holds,
+            // ((out + v0) + v1) + .., as the per-slot kernel does (the reference's vec_axpy per slot)
+            const bool writer = row < m.hidden && (lane & (8 * G - 1)) == 0;
+            float *const dst = m.out0 + (size_t)t * m.hidden + (row < m.hidden ? row : 0);
+            float y = (m.accumulate && writer) ? *dst : 0.0f;
             bool first = (m.accumulate == 0);
 #pragma unroll
             for (int s = 0; s < S; ++s)
@@ -631,11 +926,8 @@ namespace llamql
                     y = y + v;
             }
             // (a token without a live slot: y is 0, which overwrites when accumulate == 0)
-            if (row < m.hidden && (lane & (8 * G - 1)) == 0)
-            {
-                float *dst = m.out0 + (size_t)t * m.hidden + row;
-                *dst = m.accumulate ? (*dst + y) : y;
-            }
+            if (writer)
+                *dst = y;
         }
     }
 
@@ -903,7 +1195,10 @@ namespace llamql
         const int h = blockIdx.x * blockDim.x + threadIdx.x;
         if (h >= hidden)
             return;
-        float y = 0.0f;
+        // accumulate: the sum starts from what the output holds and takes the slots one by one,
+        // ((out + v0) + v1) + .., as the per-slot launches do
+        float *dst = out + (size_t)t * hidden + h;
+        float y = accumulate ? *dst : 0.0f;
         bool first = accumulate == 0;
         for (int s = 0; s < slots; ++s)
         {
@@ -920,8 +1215,7 @@ namespace llamql
             else
                 y = y + v;
         }
-        float *dst = out + (size_t)t * hidden + h;
-        *dst = accumulate ? (*dst + y) : y;
+        *dst = y;
     }
 
     // ---- SwiGLU + Q8_1 ---------------------------------------------------------------
@@ -1350,6 +1644,59 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     return launched(fn);
 }
 
+extern "C" bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                                           const int32_t *d_ids, const void *d_q8, float *d_gate_scratch,
+                                           float *d_up_scratch, void *d_q8_out, int n_tokens, int top_k, int hidden,
+                                           int inter, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_gate_up_swiglu";
+    if (!check_moe(fn, fmt, n_tokens, n_experts, top_k, hidden, inter))
+        return false;
+    if (!d_experts || !d_ids || !d_q8 || !d_q8_out)
+        return fail(fn, "null pointer");
+    if (!aligned4(d_q8_out))
+        return fail(fn, "d_q8_out must be 4-byte aligned");
+    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(hidden / 256) && IQ3STraits::Quad::addressable(inter, hidden / 256) &&
+        inter % 32 == 0)
+    {
+        if (!set_device(fn, device_id))
+            return false;
+        typedef IQ3STraits::Quad Q;
+        MoEArgs m;
+        m.experts = d_experts;
+        m.ids = d_ids;
+        m.weights = nullptr;
+        m.q8 = static_cast<const uint32_t *>(d_q8);
+        m.out0 = nullptr;
+        m.out1 = nullptr;
+        m.n_experts = n_experts;
+        m.top_k = top_k;
+        m.hidden = hidden;
+        m.inter = inter;
+        m.accumulate = 0;
+        m.rows_per_wave = 0;
+        const int nsb = hidden / 256;
+        m.gshift = moe_log2(nsb);
+        const dim3 grid((unsigned)(inter / 32), (unsigned)(n_tokens * top_k));
+        const size_t lds = (size_t)nsb * QUAD_SB_LDS + 2 * 32 * sizeof(float);
+        if ((long)grid.x * grid.y >= 4L * cu_count(device_id))
+            hipLaunchKernelGGL((moe_gate_up_swiglu_dense_kernel<Q>), grid, dim3(MOE_QUAD_WAVES * WAVE), lds,
+                               as_stream(stream), m, static_cast<uint32_t *>(d_q8_out));
+        else
+            hipLaunchKernelGGL((moe_gate_up_swiglu_kernel<Q>), grid, dim3(MOE_QUAD_WAVES * WAVE), lds,
+                               as_stream(stream), m, static_cast<uint32_t *>(d_q8_out));
+        return launched(fn);
+    }
+    // other formats and row lengths: the two launches, through the caller's fp32 scratch
+    if (!d_gate_scratch || !d_up_scratch)
+        return fail(fn, "this format and shape need the fp32 scratch rows (d_gate_scratch, d_up_scratch)");
+    if (!llam_ql_moe_gate_up(fmt, d_experts, n_experts, d_ids, d_q8, d_gate_scratch, d_up_scratch, n_tokens, top_k,
+                             hidden, inter, device_id, stream))
+        return false;
+    return llam_ql_swiglu_quantize(d_gate_scratch, d_up_scratch, nullptr, d_q8_out, n_tokens * top_k, inter, device_id,
+                                   stream);
+}
 
 extern "C" size_t llam_ql_moe_group_bytes(int n_tokens, int slot_stride)
 {
@@ -1553,9 +1900,29 @@ extern "C" bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts, i
     // (with little work per compute unit the launch is a chain of memory round trips: there the kernel that
     // has the loads of all slots of a row in flight at once is faster -- 1 token 24.1 against 26.9 us per step,
     // 4 tokens 35.3 against 37.1, 8 tokens 54.9 against 47.5, 16 tokens 78.9 against 67.0)
-    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(inter / 256) && top_k <= MOE_QUAD_MAX_SLOTS &&
-        IQ3STraits::Quad::addressable(hidden, inter / 256) &&
-        (long)hidden * (inter / 256) / QUAD_STEP_SB * n_tokens * top_k >= 48L * cu_count(device_id))
+    const bool quad_down = fmt == LLAM_FMT_IQ3_S && moe_quad_rows(inter / 256) && top_k <= MOE_QUAD_MAX_SLOTS &&
+                           IQ3STraits::Quad::addressable(hidden, inter / 256) &&
+                           (size_t)top_k * (inter / 256) * QUAD_SB_LDS + IQ3STraits::Quad::STATIC_LDS + 4096 <= 64 * 1024;
+    const bool much_work = (long)hidden * (inter / 256) / QUAD_STEP_SB * n_tokens * top_k >= 48L * cu_count(device_id);
+    if (quad_down && !much_work)
+    {
+        // a few tokens: a wavefront per slot, every slot's loads of a row range in flight at once
+        typedef IQ3STraits::Quad Q;
+        const int nsb = inter / 256;
+        const long steps = ((long)hidden * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+        int spw = 1;
+        while (spw < MOE_SLOTWAVE_MAX_STEPS && steps * n_tokens / (2L * cu_count(device_id)) >= 2 * spw)
+            spw *= 2;
+        m.rows_per_wave = spw;
+        m.gshift = moe_log2(nsb);
+        const long gx = (steps + spw - 1) / spw;
+        const size_t lds = (size_t)top_k * nsb * QUAD_SB_LDS + (size_t)top_k * spw * (QUAD_STEP_SB / nsb) * sizeof(float);
+        // a wavefront per slot, and enough threads to fetch the decode tables a piece each
+        const int waves = top_k * WAVE >= Q::TABLE_THREADS ? top_k : (Q::TABLE_THREADS + WAVE - 1) / WAVE;
+        hipLaunchKernelGGL((moe_down_slotwave_kernel<Q>), dim3((unsigned)gx, (unsigned)n_tokens), dim3(waves * WAVE), lds, st, m);
+        return launched(fn);
+    }
+    if (quad_down)
     {
         // the quad-lane decoder on short rows: workgroups of a step or more per wavefront, at least
         // two of them per compute unit

@@ -228,10 +228,13 @@ def test_token_without_live_slot_gets_zeros(capi, dev):
         pair_out = torch.full((T * k, hidden), float("nan"), device=dev)
         out_g = torch.full((T, hidden), 7.0, device=dev)
         capi.moe_down_grouped(fmt, table, n_exp, grp, ids, w, q8a, pair_out, out_g, T, k, hidden, inter)
+        acc_g = torch.full((T, hidden), 7.0, device=dev)
+        capi.moe_down_grouped(fmt, table, n_exp, grp, ids, w, q8a, pair_out, acc_g, T, k, hidden, inter, accumulate=True)
         sync()
         assert float(out[1].abs().max()) == 0.0 and float(out[0].abs().max()) > 0.0
         assert float((acc[1] - 7.0).abs().max()) == 0.0
         assert torch.equal(out_g, out)
+        assert torch.equal(acc_g, acc)   # accumulate: ((out + v0) + v1) + .. on both paths
 
 
 def test_group_tokens_by_expert(capi, dev):
@@ -318,8 +321,13 @@ def test_grouped_launches_equal_ungrouped(capi, dev, fmt):
     out_g = torch.full((T, hidden), float("nan"), device=dev)
     pair_out = torch.empty((T * S, hidden), device=dev)
     capi.moe_down_grouped(fmt, tab, n_exp, grp, idd, w, q8a, pair_out, out_g, T, S, hidden, inter)
+    base = torch.from_numpy(rng.standard_normal((T, hidden)).astype(np.float32)).to(dev)
+    acc, acc_g = base.clone(), base.clone()
+    capi.moe_down(fmt, tab, n_exp, idd, w, q8a, acc, T, S, hidden, inter, accumulate=True)
+    capi.moe_down_grouped(fmt, tab, n_exp, grp, idd, w, q8a, pair_out, acc_g, T, S, hidden, inter, accumulate=True)
     sync()
     assert same(out_g, out)
+    assert same(acc_g, acc)   # the accumulate mode adds the slots onto the output in the same order
     assert bool(torch.isfinite(out).all())
 
 
@@ -450,3 +458,108 @@ def test_short_row_quad_lane_kernels_against_the_oracle(capi, dev, oracle):
     acc_h = acc.cpu().numpy()
     assert (acc_h[5] == 2.0).all()
     assert rel_err(acc_h - 2.0, want.astype(np.float32)) <= 1e-5
+
+
+@pytest.mark.parametrize("hidden", [512, 1024, 2048, 4096])
+def test_gate_up_swiglu_in_one_launch_has_the_bits_of_the_two(capi, dev, hidden):
+    """IQ3_S rows of 2, 4, 8 and 16 super-blocks: the Q8_1 blocks of the one-launch gate/up + SwiGLU + quantiser are
+    the bytes of llam_ql_moe_gate_up followed by llam_ql_swiglu_quantize; blocks of a slot with an id out of range
+    or an expert that lives elsewhere keep what the buffer held.  No scratch rows are needed (or touched)."""
+    import torch
+    from oracle.binding import FMT_IQ3_S as fmt
+
+    n_exp, inter, k, T = 5, 768, 3, 5
+    host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 33)
+    tab = table.clone()
+    tab.view(torch.int64).view(n_exp, 3)[2] = 0       # expert 2 lives elsewhere
+    rng = np.random.default_rng(hidden)
+    ids = rng.integers(0, n_exp, size=(T, k)).astype(np.int32)
+    ids[1, 2] = -3
+    ids[4, 0] = n_exp
+    idd = torch.from_numpy(ids).to(dev)
+    qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(T, hidden, 6)).to(dev))
+    gate, up = capi.moe_gate_up(fmt, tab, n_exp, idd, qd, T, k, hidden, inter)
+    want = capi.swiglu_quantize(gate, up).view(T * k, -1)
+    got = torch.full((T * k * (inter // 32) * 36,), 0x5A, dtype=torch.uint8, device=dev)
+    capi.moe_gate_up_swiglu(fmt, tab, n_exp, idd, qd, T, k, hidden, inter, q8_out=got)
+    sync()
+    got = got.view(T * k, -1)
+    live = ((ids >= 0) & (ids < n_exp) & (ids != 2)).reshape(-1)
+    assert live.sum() < T * k
+    for r in range(T * k):
+        if live[r]:
+            assert torch.equal(got[r], want[r]), r
+        else:
+            assert bool((got[r] == 0x5A).all()), r
+
+
+def test_gate_up_swiglu_other_formats_run_the_two_launches(capi, dev):
+    """Q4_K experts (and IQ3_S rows that are no power of two of super-blocks) go through the caller's fp32 scratch
+    rows; without them the call is refused."""
+    import torch
+    from oracle.binding import FMT_IQ3_S
+
+    for fmt, hidden in ((FMT_Q4_K, 512), (FMT_IQ3_S, 768)):
+        n_exp, inter, k, T = 3, 256, 2, 3
+        host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 12)
+        ids = torch.tensor([[0, 1], [2, 0], [1, 2]], dtype=torch.int32, device=dev)
+        qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(T, hidden, 2)).to(dev))
+        gate, up = capi.moe_gate_up(fmt, table, n_exp, ids, qd, T, k, hidden, inter)
+        want = capi.swiglu_quantize(gate, up)
+        scratch = (torch.empty_like(gate), torch.empty_like(up))
+        got = capi.moe_gate_up_swiglu(fmt, table, n_exp, ids, qd, T, k, hidden, inter, scratch=scratch)
+        sync()
+        assert torch.equal(got, want)
+        with pytest.raises(capi.QLError, match="scratch"):
+            capi.moe_gate_up_swiglu(fmt, table, n_exp, ids, qd, T, k, hidden, inter)
+
+
+@pytest.mark.parametrize("shape", [(2048, 512, 9, 1), (2048, 512, 9, 4), (1024, 1024, 4, 2), (512, 2048, 16, 1),
+                                   (768, 512, 3, 3)])
+def test_down_of_a_few_tokens_wavefront_per_slot(capi, dev, oracle, shape):
+    """IQ3_S down projection with little work per compute unit (a wavefront per slot): weighted sums against the CPU
+    restatement on the same Q8_1 input, overwrite and accumulate, with a dead slot, a dead token when there are
+    several, and the grouped path's bits to 1e-5 (its kernel adds a row's blocks in another order)."""
+    import torch
+    from oracle.binding import FMT_IQ3_S as fmt
+
+    hidden, inter, k, T = shape
+    n_exp = 5
+    host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 70 + k)
+    tab = table.clone()
+    tab.view(torch.int64).view(n_exp, 3)[3] = 0       # expert 3 lives elsewhere
+    rng = np.random.default_rng(31 + T)
+    ids = rng.integers(0, n_exp, size=(T, k)).astype(np.int32)
+    ids[0, k - 1] = 42
+    if T > 1:
+        ids[T - 1] = -1
+    w = rng.random((T, k)).astype(np.float32)
+    idd, wd = torch.from_numpy(ids).to(dev), torch.from_numpy(w).to(dev)
+    act = synth.activations_numpy(T * k, inter, 5)
+    q8a = capi.quantize_q8_1(torch.from_numpy(act).to(dev))
+    out = torch.full((T, hidden), float("nan"), device=dev)
+    capi.moe_down(fmt, tab, n_exp, idd, wd, q8a, out, T, k, hidden, inter, accumulate=False)
+    base = rng.standard_normal((T, hidden)).astype(np.float32)
+    acc = torch.from_numpy(base).to(dev)
+    capi.moe_down(fmt, tab, n_exp, idd, wd, q8a, acc, T, k, hidden, inter, accumulate=True)
+    grp = capi.moe_group(idd, n_exp)
+    pair_out = torch.empty((T * k, hidden), device=dev)
+    out_g = torch.full((T, hidden), float("nan"), device=dev)
+    capi.moe_down_grouped(fmt, tab, n_exp, grp, idd, wd, q8a, pair_out, out_g, T, k, hidden, inter)
+    sync()
+    q8a_h = oracle.quantize(act)
+    assert np.array_equal(q8a.cpu().numpy().reshape(q8a_h.shape), q8a_h)
+    want = np.zeros((T, hidden), np.float64)
+    for t in range(T):
+        for s in range(k):
+            e = int(ids[t, s])
+            if 0 <= e < n_exp and e != 3:
+                want[t] += float(w[t, s]) * oracle.gemm(fmt, host[e][2], inter, q8a_h[t * k + s][None])[0]
+    got = out.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert rel_err(got, want.astype(np.float32)) <= TOL[fmt] * 1e-2
+    if T > 1:
+        assert not got[T - 1].any()
+        assert np.array_equal(acc.cpu().numpy()[T - 1], base[T - 1])
+    assert rel_err(acc.cpu().numpy() - base, want.astype(np.float32)) <= 1e-5
+    assert float((out_g - out).abs().max()) <= 1e-5 * float(out.abs().max())
