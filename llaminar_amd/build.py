@@ -63,12 +63,13 @@ def check_kernel_resources(remarks: str, src_name: str) -> dict[str, dict[str, i
     usage: dict[str, dict[str, int]] = {}
     name = None
     for line in remarks.splitlines():
-        m = re.search(r"remark: Function Name: (\S+)", line)
+        # the remark's position is printed before "remark:" or, under -save-temps, after it
+        m = re.search(r"remark:(?: \S+:\d+:\d+:)? Function Name: (\S+)", line)
         if m:
             name = m.group(1)
             usage[name] = {}
             continue
-        m = re.search(r"remark:\s+(ScratchSize \[bytes/lane\]|VGPRs Spill|SGPRs Spill|VGPRs|Dynamic Stack): (\S+)", line)
+        m = re.search(r"remark:(?: \S+:\d+:\d+:)?\s+(ScratchSize \[bytes/lane\]|VGPRs Spill|SGPRs Spill|VGPRs|Dynamic Stack): (\S+)", line)
         if m and name is not None:
             v = m.group(2)
             usage[name][m.group(1)] = int(v) if v.isdigit() else int(v == "True")

@@ -1168,11 +1168,15 @@ namespace llamql
             gemv_quad_launch_mus<Q, M, U, QUAD_SRC_Q8, QUAD_MODE_DUMP>(grid, block, lds, st, a);
             return;
         }
+        // (the norm's staging holds a row's values and weights in registers across its barrier: with two
+        // steps per load chunk as well a single row's kernel would spill, so gemv_quad_launch sends the
+        // norm source to one step per chunk and the two-step instantiation does not exist)
+        constexpr bool NORM = M <= QUAD_NORM_MAX_M && !(M == 1 && U == 2);
         if constexpr (M <= QUAD_RING_MAX_M)
         {
             if (a.ring)
             {
-                if constexpr (M <= QUAD_NORM_MAX_M)
+                if constexpr (NORM)
                     if (src == QUAD_SRC_RMSNORM)
                     {
                         gemv_quad_launch_mus<Q, M, U, QUAD_SRC_RMSNORM, QUAD_MODE_RING>(grid, block, lds, st, a);
@@ -1187,7 +1191,7 @@ namespace llamql
                 return;
             }
         }
-        if constexpr (M <= QUAD_NORM_MAX_M)
+        if constexpr (NORM)
             if (src == QUAD_SRC_RMSNORM)
             {
                 gemv_quad_launch_mus<Q, M, U, QUAD_SRC_RMSNORM>(grid, block, lds, st, a);
@@ -1214,7 +1218,7 @@ namespace llamql
         switch (M)
         {
         case 1:
-            if (a.SB >= QUAD_LONG_ROW_SB)
+            if (a.SB >= QUAD_LONG_ROW_SB && src != QUAD_SRC_RMSNORM)
                 gemv_quad_launch_mu<Q, 1, 2>(src, grid, block, lds, st, a);
             else
                 gemv_quad_launch_mu<Q, 1, 1>(src, grid, block, lds, st, a);

@@ -39,6 +39,34 @@ def test_a_spilling_kernel_fails_the_build(scratch, spill):
     assert "Li4E" in str(e.value) and "Li3E" not in str(e.value)
 
 
+# with -save-temps (which the build uses, for the assembly check below) the backend runs as a step of
+# its own and prints the position AFTER "remark:", with column 0 and no source excerpt
+REMARKS_SAVE_TEMPS = """\
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0: Function Name: _ZN6llamql11gemm_kernelINS_9Q4KTraitsELb{d}EEEvNS_8GemmArgsE [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     TotalSGPRs: 68 [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     VGPRs: 128 [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     AGPRs: 0 [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     ScratchSize [bytes/lane]: {scratch} [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     Dynamic Stack: False [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     Occupancy [waves/SIMD]: 4 [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     SGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     VGPRs Spill: {spill} [-Rpass-analysis=kernel-resource-usage]
+remark: /root/repo/llaminar_amd/csrc/gemm.hip:195:0:     LDS Size [bytes/block]: 0 [-Rpass-analysis=kernel-resource-usage]
+"""
+
+
+def test_the_layout_of_the_remarks_under_save_temps_is_read_too():
+    """A build that keeps the intermediate files prints 'remark: file:line:col: field', not 'file:line:col:
+    remark: field'; a guard that only knew the second form let two spilling kernels through."""
+    clean = REMARKS_SAVE_TEMPS.format(d=1, scratch=0, spill=0)
+    usage = b.check_kernel_resources(clean, "gemm.hip")
+    assert len(usage) == 1 and next(iter(usage.values()))["VGPRs"] == 128
+    with pytest.raises(b.SpillError) as e:
+        b.check_kernel_resources(clean + REMARKS_SAVE_TEMPS.format(d=0, scratch=44, spill=10), "gemm.hip")
+    assert "Lb0E" in str(e.value) and "44 B/lane" in str(e.value) and "Lb1E" not in str(e.value)
+    assert b._drop_resource_remarks(clean.splitlines()) == []
+
+
 def test_remarks_do_not_reach_the_build_log():
     lines = (REMARKS.format(u=3, scratch=0, spill=0) + "x.hip:1:1: warning: something real\n").splitlines()
     assert b._drop_resource_remarks(lines) == ["x.hip:1:1: warning: something real"]

@@ -618,6 +618,9 @@ _NORM_CASES = [
     ((FMT_IQ3_S,), (4096,), 5120, 1),
     ((FMT_Q6_K,), (384,), 8192, 1),
     ((FMT_Q4_K,), (3000,), 12800, 1),
+    # rows of 64 super-blocks and more (plain launches take two steps per load chunk there; the norm source one)
+    ((FMT_Q6_K,), (640,), 16384, 1),
+    ((FMT_Q4_K, FMT_Q4_K), (768, 512), 20480, 1),
 ]
 
 
