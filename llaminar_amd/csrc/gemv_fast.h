@@ -22,6 +22,7 @@
 #include "gemv_quad.h"
 #include "gemv_mfma.h"
 #include "gemv_mfma_q6k.h"
+#include "gemv_mfma_q4k_long.h"
 #include <atomic>
 #include <type_traits>
 
@@ -453,7 +454,10 @@ namespace llamql
         else
             // a matrix of few 32-row tiles leaves most compute units idle here: the quad-lane kernel
             // spreads it over all of them (and shares its launch with a following Q6_K matrix)
-            return mfma_max_slices(K / 256) >= 1 && N >= MFMA_MIN_ROWS;
+            // (long rows are walked in chunks, gemv_mfma_q4k_long.h; where not even one buffer of the whole
+            // batch fits the LDS but the quad-lane kernel still holds the batch in one launch, that one is
+            // faster: 5 rows of K = 25600 28 against 32 us)
+            return N >= MFMA_MIN_ROWS && (mfma_max_slices(K / 256) >= 1 || quad_lds_bytes(M, K / 256) > QUAD_MAX_LDS);
     }
 
     template <int SRC, bool DUMP = false, bool PLANE = false>
@@ -464,6 +468,77 @@ namespace llamql
         hipLaunchKernelGGL((gemv_mfma_q4k_kernel<SRC, DUMP, PLANE>), grid, block, lds, st, a);
     }
 
+    // Rows that take the chunked kernel: those whose activations leave gemv_mfma_q4k_kernel fewer than its
+    // eight wavefronts per tile (measured at batch 8 on 5120 rows: 50 super-blocks 19.0 against 23.5 us
+    // chunked; 32 super-blocks 13.4 against 12.6 us, and 25600 rows of 20 super-blocks 32.7 against 25.1 us).
+    inline bool mfma4_long_rows(int SB) { return mfma_max_slices(SB) < MFMA_MAX_SLICES; }
+
+    template <int SRC, bool DUMP = false, bool PLANE = false>
+    void gemv_mfma_q4k_long_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const MfmaLongArgs &a)
+    {
+        static LdsGrant grant;
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_q4k_long_kernel<SRC, DUMP, PLANE>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_mfma_q4k_long_kernel<SRC, DUMP, PLANE>), grid, block, lds, st, a);
+    }
+
+    // Rows too long for gemv_mfma_q4k_kernel (the batch's activations do not fit the LDS).
+    inline bool gemv_mfma_q4k_long_launch(const char *fn, const void *d_w, const void *d_plane, const ActSource &src,
+                                          float *d_y, int M, int N, int K, int ldy, int device_id, hipStream_t st,
+                                          int32_t *d_sums, int row0, int nrows)
+    {
+        const int SB = K / 256;
+        const Mfma6Shape sh = gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA4_LONG_DUMP_COMPUTE : MFMA4_LONG_COMPUTE,
+                                               d_plane != nullptr, MFMA_BOUNCE);
+        MfmaLongArgs a;
+        a.w = static_cast<const uint8_t *>(d_w);
+        a.plane = static_cast<const uint8_t *>(d_plane);
+        a.q8 = static_cast<const uint32_t *>(src.q8);
+        a.x = src.x;
+        a.x2 = src.x2;
+        a.ldx = src.ldx;
+        a.y = d_y;
+        a.ldy = ldy;
+        a.N = N;
+        a.SB = SB;
+        a.M = M;
+        a.slices = sh.slices;
+        a.tile_rows = sh.tile_rows;
+        a.tiles = sh.tiles;
+        a.chunk = sh.chunk;
+        a.sums = d_sums;
+        a.row0 = row0;
+        a.nrows = nrows;
+        const dim3 grid((unsigned)sh.grid), block((unsigned)(sh.slices * sh.tiles + MFMA4_LONG_PRODUCERS) * WAVE);
+        const size_t lds = mfma6_act_bytes(SB, sh.chunk) + (a.plane ? 0 : (size_t)sh.slices * sh.tiles * MFMA_BOUNCE);
+        if (d_sums)
+        {
+            if (src.kind != ACT_SRC_Q8)
+                return fail(fn, "block sums are dumped on Q8_1 input");
+            if (a.plane)
+                gemv_mfma_q4k_long_launch_src<QUAD_SRC_Q8, true, true>(grid, block, lds, st, a);
+            else
+                gemv_mfma_q4k_long_launch_src<QUAD_SRC_Q8, true>(grid, block, lds, st, a);
+            return launched(fn);
+        }
+        if (a.plane)
+        {
+            switch (src.kind)
+            {
+            case ACT_SRC_F32: gemv_mfma_q4k_long_launch_src<QUAD_SRC_F32, false, true>(grid, block, lds, st, a); break;
+            case ACT_SRC_SWIGLU: gemv_mfma_q4k_long_launch_src<QUAD_SRC_SWIGLU, false, true>(grid, block, lds, st, a); break;
+            default: gemv_mfma_q4k_long_launch_src<QUAD_SRC_Q8, false, true>(grid, block, lds, st, a); break;
+            }
+            return launched(fn);
+        }
+        switch (src.kind)
+        {
+        case ACT_SRC_F32: gemv_mfma_q4k_long_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;
+        case ACT_SRC_SWIGLU: gemv_mfma_q4k_long_launch_src<QUAD_SRC_SWIGLU>(grid, block, lds, st, a); break;
+        default: gemv_mfma_q4k_long_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a); break;
+        }
+        return launched(fn);
+    }
+
     // d_plane: the matrix's batch plane (q4k_plane_bytes) or null; with one, the kernel reads it
     // instead of the prepared matrix, the block-sum variant included.
     inline bool gemv_mfma_q4k_launch(const char *fn, const void *d_w, const void *d_plane, const ActSource &src,
@@ -471,6 +546,8 @@ namespace llamql
                                      int32_t *d_sums = nullptr, int row0 = 0, int nrows = 0)
     {
         const int SB = K / 256;
+        if (mfma4_long_rows(SB))
+            return gemv_mfma_q4k_long_launch(fn, d_w, d_plane, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
         const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id), d_sums ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES);
         MfmaArgs a;
         a.w = static_cast<const uint8_t *>(d_w);

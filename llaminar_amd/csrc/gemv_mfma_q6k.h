@@ -630,7 +630,9 @@ namespace llamql
     // compute wavefronts, five at least (the scales of eight neighbouring super-blocks share a
     // cache line) and each two steps long; tiles per workgroup to fill its compute wavefronts
     // when there are tiles to spare.
-    inline Mfma6Shape gemv_mfma6_shape_of(long N, int nsb, int cus, int max_compute, int tile_rows, bool plane = false)
+    // bounce_per_wave: LDS bytes of a compute wavefront's bounce buffer (none when the weights come from a batch plane)
+    inline Mfma6Shape gemv_mfma6_shape_of(long N, int nsb, int cus, int max_compute, int tile_rows, bool plane = false,
+                                          size_t bounce_per_wave = MFMA6_BOUNCE)
     {
         const long tiles = (N + tile_rows - 1) / tile_rows;
         long want = ((long)cus * max_compute + tiles - 1) / tiles;
@@ -652,7 +654,7 @@ namespace llamql
         sh.grid = (tiles + t - 1) / t;
         // one buffer if the whole row fits beside the bounce buffers and leaves half the LDS
         // free, else two buffers of a whole number of rounds of the slices
-        const size_t bounce = plane ? 0 : (size_t)sh.slices * t * MFMA6_BOUNCE; // the plane kernel has no bounce buffers
+        const size_t bounce = plane ? 0 : (size_t)sh.slices * t * bounce_per_wave; // the plane kernels have no bounce buffers
         if (mfma_act_bytes(nsb) * 2 + bounce <= QUAD_MAX_LDS)
             sh.chunk = nsb;
         else
@@ -664,7 +666,8 @@ namespace llamql
     }
     // The tile height that leaves the busiest compute unit the fewest rows (gemv_mfma_shape):
     // 5120 rows are 160 full tiles, and 256 tiles of 20 rows.
-    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus, int max_compute = MFMA6_MAX_COMPUTE, bool plane = false)
+    inline Mfma6Shape gemv_mfma6_shape(long N, int nsb, int cus, int max_compute = MFMA6_MAX_COMPUTE, bool plane = false,
+                                       size_t bounce_per_wave = MFMA6_BOUNCE)
     {
         const int forced = gemv_mfma_tile_rows_override();
         Mfma6Shape best;
@@ -673,7 +676,7 @@ namespace llamql
         {
             if (forced > 0 && tr != forced)
                 continue;
-            const Mfma6Shape sh = gemv_mfma6_shape_of(N, nsb, cus, max_compute, tr, plane);
+            const Mfma6Shape sh = gemv_mfma6_shape_of(N, nsb, cus, max_compute, tr, plane, bounce_per_wave);
             const long cost = ((sh.grid + cus - 1) / cus) * sh.tiles * tr;
             if (best_cost < 0 || cost * 20 < best_cost * 19) // a shorter tile has to win 5 %
             {

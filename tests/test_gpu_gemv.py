@@ -503,6 +503,10 @@ def _production_cases():
         ("q6k_quad_m4_long_rows", FMT_Q6_K, 64, 25600, 4, QU),
         ("q4k_mfma_m8", FMT_Q4_K, 4100, 5120, 8, MF),
         ("q4k_mfma_m5", FMT_Q4_K, 4096, 4096, 5, MF),
+        ("q4k_mfma_m6_chunked_row", FMT_Q4_K, 4100, 25600, 6, MF),
+        ("q4k_mfma_m8_short_last_chunk", FMT_Q4_K, 4096, 17408, 8, MF),
+        ("q4k_mfma_m8_chunked_row_that_would_fit", FMT_Q4_K, 4100, 12800, 8, MF),
+        ("q4k_quad_m5_long_rows_in_one_launch", FMT_Q4_K, 4100, 25600, 5, QU),
         ("q6k_mfma_m8_chunked_row", FMT_Q6_K, 200, 25600, 8, MF),
         ("q6k_mfma_m8_short_last_chunk", FMT_Q6_K, 70, 17408, 8, MF),
         ("iq3s_quad_m1", FMT_IQ3_S, 1000, 5120, 1, QU),
@@ -941,3 +945,35 @@ def test_q4k_batch_plane_launches_match(capi, dev, oracle):
         y = capi.gemv_swiglu_f32(FMT_Q4_K, w, g, u, 8, N, K, q8_scratch=scratch, plane=plane)
         sync()
         assert torch.equal(out, before_f32) and torch.equal(y, before_swiglu)
+
+
+@pytest.mark.parametrize("M", [6, 8])
+def test_q4k_long_rows_on_the_matrix_unit(capi, dev, oracle, M):
+    """Q4_K rows of 100 super-blocks at batches of 5..8: eight activation rows do not fit the LDS, so the matrix-unit
+    kernel walks the row in chunks that producer wavefronts stage.  Repeatable; with the matrix's batch plane the same
+    bits; the fp32-input call gives the bits of quantise + GEMV; block sums (plain and from the plane) and a window
+    of rows against the CPU restatement."""
+    import torch
+
+    fmt, N, K = FMT_Q4_K, 4100, 25600
+    plan = capi.gemv_describe(fmt, M, N, K)
+    assert plan.kernel == capi.KERNEL_MFMA and not plan.decode_equivalent
+    assert capi.gemv_describe(fmt, M, N, K, has_plane=True).kernel == capi.KERNEL_MFMA
+    W = synth.weights_numpy(fmt, N, K, 4242)
+    x = synth.activations_numpy(M, K, 4243)
+    wd = upload_weights(capi, dev, fmt, W)
+    xd = torch.from_numpy(x).to(dev)
+    qd = capi.quantize_q8_1(xd)
+    y = capi.gemv(fmt, wd, qd, M, N, K)
+    again = capi.gemv(fmt, wd, qd, M, N, K)
+    plane = capi.build_batch_plane(fmt, wd, N, K)
+    yp = capi.gemv(fmt, wd, qd, M, N, K, plane=plane)
+    yf = capi.gemv_f32(fmt, wd, xd, M, N, K)
+    s0 = capi.gemv_block_sums(fmt, wd, qd, M, N, K, 4000, 100)
+    sp = capi.gemv_block_sums(fmt, wd, qd, M, N, K, 4000, 100, plane=plane)
+    sync()
+    assert torch.equal(y, again) and torch.equal(y, yp) and torch.equal(y, yf)
+    q8 = oracle.quantize(x)
+    C, sums = oracle.gemm(fmt, W, K, q8, n0=4000, n1=4100, want_sums=True)
+    assert np.array_equal(s0.cpu().numpy(), sums) and np.array_equal(sp.cpu().numpy(), sums)
+    assert rel_err(y.cpu().numpy()[:, 4000:4100], C) <= TOL[fmt] * 1e-2
