@@ -138,7 +138,7 @@ def bench_moe(args, torch, capi, synth, dev):
                      "w": torch.ones(T, TOPK + 1, device=dev)})
 
     # Batches sort the (token, slot) pairs by expert on the device and read every distinct
-    # expert's matrices once (6 launches); a single token has nothing to group (3 launches).
+    # expert's matrices once (6 launches); a single token has nothing to group (2 launches).
     # (measured: per-slot launches 67 us at 16 tokens, 107 against 135 grouped at 32, 184 against 201 at 64, 334 against 296 at 128)
     path = args.moe_path if args.moe_path != "auto" else ("grouped" if T * (TOPK + 1) >= 768 else "slots")
     S = TOPK + 1
@@ -150,11 +150,13 @@ def bench_moe(args, torch, capi, synth, dev):
         s_["qa"] = torch.empty(T * S * (I // 32) * 36, dtype=torch.uint8, device=dev)
 
     def step(s):
-        capi.moe_route_quantize(s["logits"], TOPK, s["x"], s["q8"], ids=s["ids"], weights=s["w"])
         if path == "slots":
-            # gate/up, SwiGLU and the Q8_1 quantiser of the result in one launch
-            qa = capi.moe_gate_up_swiglu(fmt, table, E + 1, s["ids"], s["q8"], T, S, H, I, q8_out=s["qa"])
+            # router, Q8_1 of the hidden state, gate/up, SwiGLU and the Q8_1 quantiser of the result in one launch
+            # (from a few tokens on the library runs the router + quantiser as a launch of its own)
+            qa = capi.moe_route_gate_up_swiglu(fmt, table, E + 1, s["logits"], TOPK, s["x"], s["ids"], s["w"], I,
+                                               q8_out=s["qa"], q8_hidden=s["q8"])
         else:
+            capi.moe_route_quantize(s["logits"], TOPK, s["x"], s["q8"], ids=s["ids"], weights=s["w"])
             capi.moe_group(s["ids"], E + 1, group=s["group"])
             gate, up = capi.moe_gate_up_grouped(fmt, table, E + 1, s["group"], s["q8"], T, S, H, I, gate=s["gate"],
                                                 up=s["up"])
@@ -185,10 +187,10 @@ def bench_moe(args, torch, capi, synth, dev):
     # algorithmic bytes: the distinct experts a step touches (a single token touches S of them)
     w_bytes = distinct_bytes
     value = w_bytes / (us * 1e-6) / 1e9
-    launches = {"slots": 3, "grouped-gate-up": 5, "grouped": 6}[path]
+    launches = {"slots": 2 if T * S * (I // 32) < 512 else 3, "grouped-gate-up": 5, "grouped": 6}[path]
     return _common(args, "MoE expert FFN decode effective GB/s", round(value, 1), "GB/s", round(us * 1e-3, 5), "int8",
                    {"workload": "MoE expert FFN decode: hidden 2048, 256 routed experts + 1 shared, top-8, expert "
-                                "intermediate 512, IQ3_S, %d token(s); route + quantise, gate/up + SwiGLU + quantise, down; shared expert in a ninth slot" % T,
+                                "intermediate 512, IQ3_S, %d token(s); route + quantise, gate/up + SwiGLU + quantise (one launch with the router inside at 1-2 tokens), down; shared expert in a ninth slot" % T,
                     "tokens": T, "weight_bytes_per_step": round(w_bytes), "slot_bytes_per_step": slot_bytes,
                     "distinct_experts_per_step": round(sum(per_set) / nsets, 1),
                     "tokens_per_s": round(T / (us * 1e-6), 1), "path": path,

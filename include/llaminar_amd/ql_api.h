@@ -365,6 +365,28 @@ bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_experts, in
                                 float *d_up_scratch, void *d_q8_out, int n_tokens, int top_k,
                                 int hidden, int inter, int device_id, void *stream);
 
+/* llam_ql_moe_route_quantize followed by llam_ql_moe_gate_up_swiglu: the same ids, weights and Q8_1
+ * bytes.  For IQ3_S experts with hidden/256 in {2,4,8,16}, at most 512 routed experts and few tokens
+ * (fewer workgroups than two per compute unit: one or two tokens of a 9-slot, 512-row expert shape)
+ * this is ONE launch: every workgroup quantises its token's hidden row into its LDS and routes the
+ * token for itself (work that precedes the first weight load in any case), so a decode step is two
+ * launches: this one and llam_ql_moe_down.  With more tokens the repeated routing costs more than the
+ * launch it saves and the call runs the two launches.  d_logits [n_tokens x n_route_experts]; d_ids / d_weights
+ * [n_tokens x slot_stride]: columns < top_k are written, columns top_k.. are READ as always-on slots
+ * (the shared expert: its table index and weight, set by the caller once); the expert table has
+ * n_experts >= n_route_experts entries.  d_hidden fp32 [n_tokens x hidden].  The two-launch form
+ * needs d_q8_hidden_scratch (Q8_1 [n_tokens x hidden/32]) and, for formats and shapes outside
+ * llam_ql_moe_gate_up_swiglu's one-launch kernel, its fp32 scratch rows; a caller that cannot tell
+ * passes all three (they are left untouched when not needed).
+ * Counterpart of decodeRouteSelect + groupedExpertGateUpDecodeFromRuntime + swiGLU
+ * (IMoEKernel.h:245-258, :378-643, :171). */
+bool llam_ql_moe_route_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                                      const float *d_logits, int n_route_experts, int top_k, int normalize,
+                                      int32_t *d_ids, float *d_weights, int slot_stride,
+                                      const float *d_hidden, void *d_q8_hidden_scratch,
+                                      float *d_gate_scratch, float *d_up_scratch, void *d_q8_out,
+                                      int n_tokens, int hidden, int inter, int device_id, void *stream);
+
 /* ---- batches: tokens grouped by expert ---------------------------------------------------
  * With several tokens the same expert is usually picked more than once (16 tokens x 8 slots
  * of 256 experts hit about 100 distinct ones, and an always-on shared expert serves all 16).

@@ -88,6 +88,9 @@ SIGNATURES = {
                                      c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_gate_up_swiglu": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_moe_route_gate_up_swiglu": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p,
+                                                  c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                  c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_swiglu_quantize": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                   c_int, c_int, c_int, c_int, c_void_p]),
@@ -460,6 +463,24 @@ def moe_gate_up_swiglu(fmt: int, table, n_experts: int, ids, q8, n_tokens: int, 
     _check(load().llam_ql_moe_gate_up_swiglu(fmt, _ptr(table), n_experts, _ptr(ids), _ptr(q8), _ptr(g), _ptr(u),
                                              _ptr(q8_out), n_tokens, top_k, hidden, inter, _dev(q8), _stream(stream)),
            "moe_gate_up_swiglu")
+    return q8_out
+
+
+def moe_route_gate_up_swiglu(fmt: int, table, n_experts: int, logits, top_k: int, x, ids, weights, inter: int,
+                             normalize: bool = True, q8_out=None, q8_hidden=None, scratch=None, stream=None):
+    """Router, Q8_1 of the hidden rows x, gate/up, SwiGLU and its quantiser; ids / weights [T, slot_stride] are
+    written in their first top_k columns and read in the others (always-on slots)."""
+    import torch
+
+    T, hidden = x.shape
+    stride = ids.shape[1]
+    if q8_out is None:
+        q8_out = torch.zeros(T * stride * (inter // 32) * 36, dtype=torch.uint8, device=x.device)
+    g, u = scratch if scratch is not None else (None, None)
+    _check(load().llam_ql_moe_route_gate_up_swiglu(fmt, _ptr(table), n_experts, _ptr(logits), logits.shape[1], top_k,
+                                                   int(normalize), _ptr(ids), _ptr(weights), stride, _ptr(x),
+                                                   _ptr(q8_hidden), _ptr(g), _ptr(u), _ptr(q8_out), T, hidden, inter,
+                                                   _dev(x), _stream(stream)), "moe_route_gate_up_swiglu")
     return q8_out
 
 

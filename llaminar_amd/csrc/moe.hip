@@ -17,32 +17,12 @@ namespace llamql
     // the top_k.  All reductions are wavefront shuffles: no LDS, no barriers.
     constexpr int ROUTE_MAX_PER_LANE = 32; // up to 2048 experts
 
-    // Workgroups past the tokens (optional) quantise `q_blocks` 32-element blocks of q_x to Q8_1
-    // with the stand-alone quantiser's arithmetic: the hidden state the expert GEMVs read does
-    // not depend on the routing, so its quantiser rides in the same launch.
+    // One wavefront routes one token: l its n_experts logits; lane k < top_k returns the k-th expert and
+    // its weight (other lanes: unspecified).
     template <int PER>
-    __global__ void __launch_bounds__(WAVE)
-        moe_route_kernel(const float *__restrict__ logits, int n_tokens, int n_experts, int top_k, int normalize,
-                         int32_t *__restrict__ ids, float *__restrict__ weights, int slot_stride,
-                         const float4 *__restrict__ q_x, uint32_t *__restrict__ q_out, long q_blocks)
+    __device__ __forceinline__ void moe_route_wave(const float *__restrict__ l, int n_experts, int top_k, int normalize,
+                                                   int lane, int &out_id, float &out_weight)
     {
-        if ((int)blockIdx.x >= n_tokens) // uniform
-        {
-            const long lane_global = (long)((int)blockIdx.x - n_tokens) * WAVE + threadIdx.x;
-            const long blk = lane_global >> 3;
-            if (blk >= q_blocks)
-                return; // whole 8-lane groups leave together
-            const Q8Lane q = q8_1_quantize_lane(q_x[lane_global]);
-            uint32_t *dst = q_out + blk * 9;
-            dst[1 + (lane_global & 7)] = q.packed;
-            if ((lane_global & 7) == 0)
-                dst[0] = q.head;
-            return;
-        }
-        const int t = blockIdx.x;
-        const int lane = threadIdx.x;
-        const float *l = logits + (size_t)t * n_experts;
-
         float p[PER];
         float mx = -INFINITY;
 #pragma unroll
@@ -120,10 +100,41 @@ namespace llamql
                 if (lane + i * WAVE == best_e)
                     p[i] = -1.0f; // retire the winner
         }
+        out_id = my_id;
+        out_weight = normalize ? __fdiv_rn(my_top, topk_sum) : my_top;
+    }
+
+    // Workgroups past the tokens (optional) quantise `q_blocks` 32-element blocks of q_x to Q8_1
+    // with the stand-alone quantiser's arithmetic: the hidden state the expert GEMVs read does
+    // not depend on the routing, so its quantiser rides in the same launch.
+    template <int PER>
+    __global__ void __launch_bounds__(WAVE)
+        moe_route_kernel(const float *__restrict__ logits, int n_tokens, int n_experts, int top_k, int normalize,
+                         int32_t *__restrict__ ids, float *__restrict__ weights, int slot_stride,
+                         const float4 *__restrict__ q_x, uint32_t *__restrict__ q_out, long q_blocks)
+    {
+        if ((int)blockIdx.x >= n_tokens) // uniform
+        {
+            const long lane_global = (long)((int)blockIdx.x - n_tokens) * WAVE + threadIdx.x;
+            const long blk = lane_global >> 3;
+            if (blk >= q_blocks)
+                return; // whole 8-lane groups leave together
+            const Q8Lane q = q8_1_quantize_lane(q_x[lane_global]);
+            uint32_t *dst = q_out + blk * 9;
+            dst[1 + (lane_global & 7)] = q.packed;
+            if ((lane_global & 7) == 0)
+                dst[0] = q.head;
+            return;
+        }
+        const int t = blockIdx.x;
+        const int lane = threadIdx.x;
+        int my_id;
+        float my_weight;
+        moe_route_wave<PER>(logits + (size_t)t * n_experts, n_experts, top_k, normalize, lane, my_id, my_weight);
         if (lane < top_k)
         {
             ids[(size_t)t * slot_stride + lane] = my_id;
-            weights[(size_t)t * slot_stride + lane] = normalize ? __fdiv_rn(my_top, topk_sum) : my_top;
+            weights[(size_t)t * slot_stride + lane] = my_weight;
         }
     }
 
@@ -613,20 +624,69 @@ namespace llamql
     // q8_out: Q8_1 blocks [n_tokens * top_k][inter / 32]; blocks of skipped slots are left untouched.
     // NB: steps in flight per wavefront -- 4 when the launch is a latency chain (few slots), 2 (fewer
     // registers, twice the resident workgroups) when there is work to overlap it with.
-    template <class Q, int NB>
-    __device__ __forceinline__ void moe_gate_up_swiglu_body(const MoEArgs &m, uint32_t *q8_out)
+    // PER > 0: the router and the Q8_1 quantiser of the hidden state run here as well.  Every workgroup
+    // quantises its token's fp32 row straight into its LDS (the arithmetic of the stand-alone quantiser) and
+    // one of its wavefronts routes the token (moe_route_wave with PER experts per lane) -- work repeated by
+    // every workgroup of the token, all of it before the first weight can be asked for anyway -- so the step
+    // needs no routing launch; the first workgroup of a token writes the ids and weights out for the down
+    // projection.  Slots past the routed ones (always-on experts) take their id from m.ids.
+    struct MoERouteArgs
+    {
+        const float *logits; // [n_tokens][n_route]
+        const float *x;      // [n_tokens][hidden] fp32
+        int32_t *ids;        // [n_tokens][m.top_k]: columns < top_k are written
+        float *weights;
+        int n_route, top_k, normalize;
+    };
+
+    template <class Q, int NB, int PER = 0>
+    __device__ __forceinline__ void moe_gate_up_swiglu_body(const MoEArgs &m, uint32_t *q8_out, const MoERouteArgs *rt = nullptr)
     {
         static_assert(MOE_QUAD_WAVES * WAVE >= Q::TABLE_THREADS, "one table piece per thread");
         static_assert(NB == 2 || NB == 4, "the wait counts below are written for 2 or 4 steps");
         extern __shared__ __attribute__((aligned(16))) uint8_t moe_quad_lds[];
+        __shared__ int routed_id[WAVE];
         const int slot = blockIdx.y;
         const int t = slot / m.top_k;
         const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
         typename Q::TablesRaw tab;
         Q::tables_issue(tab);
         QuadActRaw act[1]; // nsb * 8 <= 128 blocks: one per thread at most
-        quad_act_issue(act, m.q8 + (size_t)t * (m.hidden / 32) * 9, nsb * 8);
-        const int e = m.ids[slot];
+        int e;
+        if constexpr (PER > 0)
+        {
+            // float4 number i of the row is one lane's share of block i / 8 (whole 8-lane groups: hidden is
+            // a multiple of 256)
+            const float4 *x4 = reinterpret_cast<const float4 *>(rt->x + (size_t)t * m.hidden);
+            for (int i = threadIdx.x; i < m.hidden / 4; i += blockDim.x)
+                quad_store_q8_lane<Q>(q8_1_quantize_lane(x4[i]), i, moe_quad_lds);
+            if (threadIdx.x < WAVE) // uniform per wavefront
+            {
+                int id;
+                float w;
+                moe_route_wave<PER>(rt->logits + (size_t)t * rt->n_route, rt->n_route, rt->top_k, rt->normalize,
+                                    (int)threadIdx.x, id, w);
+                if ((int)threadIdx.x < rt->top_k)
+                {
+                    routed_id[threadIdx.x] = id;
+                    if (blockIdx.x == 0 && slot == t * m.top_k) // one workgroup per token publishes the routing
+                    {
+                        rt->ids[(size_t)t * m.top_k + threadIdx.x] = id;
+                        rt->weights[(size_t)t * m.top_k + threadIdx.x] = w;
+                    }
+                }
+            }
+            Q::template tables_wait<0>(tab);
+            Q::tables_store(tab);
+            __syncthreads();
+            const int s_in_t = slot - t * m.top_k;
+            e = s_in_t < rt->top_k ? routed_id[s_in_t] : m.ids[slot];
+        }
+        else
+        {
+            quad_act_issue(act, m.q8 + (size_t)t * (m.hidden / 32) * 9, nsb * 8);
+            e = m.ids[slot];
+        }
         if (e < 0 || e >= m.n_experts)
             return; // uniform for the workgroup
         const void *wg = m.experts[e].d_gate, *wu = m.experts[e].d_up;
@@ -658,11 +718,14 @@ namespace llamql
 #pragma unroll
         for (int i = 0; i < NB; ++i)
             issue(buf[i], i);
-        quad_act_wait<NB * Q::LOADS>(act);
-        Q::template tables_wait<NB * Q::LOADS>(tab); // asked for before the activations
-        quad_act_store<Q>(act, nsb, nsb * 8, moe_quad_lds, 0);
-        Q::tables_store(tab);
-        __syncthreads();
+        if constexpr (PER == 0)
+        {
+            quad_act_wait<NB * Q::LOADS>(act);
+            Q::template tables_wait<NB * Q::LOADS>(tab); // asked for before the activations
+            quad_act_store<Q>(act, nsb, nsb * 8, moe_quad_lds, 0);
+            Q::tables_store(tab);
+            __syncthreads();
+        }
 #pragma unroll
         for (int i = 0; i < NB; ++i)
             Q::keep(buf[i]);
@@ -742,6 +805,13 @@ namespace llamql
     moe_gate_up_swiglu_dense_kernel(const MoEArgs m, uint32_t *q8_out)
     {
         moe_gate_up_swiglu_body<Q, 2>(m, q8_out);
+    }
+    // the same with the router and the hidden state's quantiser inside (PER experts per lane of the routing wavefront)
+    template <class Q, int NB, int PER>
+    __global__ void __launch_bounds__(MOE_QUAD_WAVES *WAVE)
+    moe_route_gate_up_swiglu_kernel(const MoEArgs m, uint32_t *q8_out, const MoERouteArgs r)
+    {
+        moe_gate_up_swiglu_body<Q, NB, PER>(m, q8_out, &r);
     }
 
     // grid: (workgroups per matrix, n_tokens).  Slots are walked in ascending
@@ -1696,6 +1766,80 @@ extern "C" bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_
         return false;
     return llam_ql_swiglu_quantize(d_gate_scratch, d_up_scratch, nullptr, d_q8_out, n_tokens * top_k, inter, device_id,
                                    stream);
+}
+
+extern "C" bool llam_ql_moe_route_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_experts, int n_experts,
+                                                 const float *d_logits, int n_route_experts, int top_k, int normalize,
+                                                 int32_t *d_ids, float *d_weights, int slot_stride,
+                                                 const float *d_hidden, void *d_q8_hidden_scratch,
+                                                 float *d_gate_scratch, float *d_up_scratch, void *d_q8_out,
+                                                 int n_tokens, int hidden, int inter, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_moe_route_gate_up_swiglu";
+    if (!check_moe(fn, fmt, n_tokens, n_experts, slot_stride, hidden, inter))
+        return false;
+    if (!d_experts || !d_logits || !d_ids || !d_weights || !d_hidden || !d_q8_out)
+        return fail(fn, "null pointer");
+    if (n_route_experts < 1 || n_route_experts > n_experts)
+        return fail(fn, "n_route_experts=%d outside 1..n_experts=%d", n_route_experts, n_experts);
+    if (top_k < 1 || top_k > n_route_experts || top_k > 64 || top_k > slot_stride)
+        return fail(fn, "top_k=%d outside 1..min(n_route_experts, 64, slot_stride=%d)", top_k, slot_stride);
+    if (!aligned16(d_hidden) || !aligned4(d_q8_out))
+        return fail(fn, "d_hidden must be 16-byte aligned, d_q8_out 4-byte aligned");
+    const int per = (n_route_experts + WAVE - 1) / WAVE;
+    // One launch while the step is a chain of latencies (fewer workgroups than two per compute unit: one or
+    // two tokens of the 256-expert shape: 16.2 against 17.5 us per step at 1 token); with more work the
+    // routing repeated by every workgroup costs more than the launch it saves (4 tokens 30.4 against 29.7 us,
+    // 16 tokens 64.3 against 59.4-61.8 us).
+    const bool few = (long)(inter / 32) * n_tokens * slot_stride < 2L * cu_count(device_id);
+    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(hidden / 256) && IQ3STraits::Quad::addressable(inter, hidden / 256) &&
+        inter % 32 == 0 && per <= 8 && few)
+    {
+        if (!set_device(fn, device_id))
+            return false;
+        typedef IQ3STraits::Quad Q;
+        MoEArgs m;
+        m.experts = d_experts;
+        m.ids = d_ids;
+        m.weights = nullptr;
+        m.q8 = nullptr;
+        m.out0 = nullptr;
+        m.out1 = nullptr;
+        m.n_experts = n_experts;
+        m.top_k = slot_stride;
+        m.hidden = hidden;
+        m.inter = inter;
+        m.accumulate = 0;
+        m.rows_per_wave = 0;
+        const int nsb = hidden / 256;
+        m.gshift = moe_log2(nsb);
+        MoERouteArgs r;
+        r.logits = d_logits;
+        r.x = d_hidden;
+        r.ids = d_ids;
+        r.weights = d_weights;
+        r.n_route = n_route_experts;
+        r.top_k = top_k;
+        r.normalize = normalize;
+        const dim3 grid((unsigned)(inter / 32), (unsigned)(n_tokens * slot_stride)), block(MOE_QUAD_WAVES * WAVE);
+        const size_t lds = (size_t)nsb * QUAD_SB_LDS + 2 * 32 * sizeof(float);
+        hipStream_t st = as_stream(stream);
+        uint32_t *out = static_cast<uint32_t *>(d_q8_out);
+        if (per <= 4)
+            hipLaunchKernelGGL((moe_route_gate_up_swiglu_kernel<Q, 4, 4>), grid, block, lds, st, m, out, r);
+        else
+            hipLaunchKernelGGL((moe_route_gate_up_swiglu_kernel<Q, 4, 8>), grid, block, lds, st, m, out, r);
+        return launched(fn);
+    }
+    // more tokens, other formats and row lengths, more than 512 routed experts: the launches one by one
+    if (!d_q8_hidden_scratch)
+        return fail(fn, "this format, shape or token count needs the Q8_1 scratch of the hidden state (d_q8_hidden_scratch)");
+    if (!llam_ql_moe_route_quantize(d_logits, n_tokens, n_route_experts, top_k, normalize, d_ids, d_weights, slot_stride,
+                                    d_hidden, hidden, d_q8_hidden_scratch, device_id, stream))
+        return false;
+    return llam_ql_moe_gate_up_swiglu(fmt, d_experts, n_experts, d_ids, d_q8_hidden_scratch, d_gate_scratch, d_up_scratch,
+                                      d_q8_out, n_tokens, slot_stride, hidden, inter, device_id, stream);
 }
 
 extern "C" size_t llam_ql_moe_group_bytes(int n_tokens, int slot_stride)

@@ -563,3 +563,60 @@ def test_down_of_a_few_tokens_wavefront_per_slot(capi, dev, oracle, shape):
         assert np.array_equal(acc.cpu().numpy()[T - 1], base[T - 1])
     assert rel_err(acc.cpu().numpy() - base, want.astype(np.float32)) <= 1e-5
     assert float((out_g - out).abs().max()) <= 1e-5 * float(out.abs().max())
+
+
+@pytest.mark.parametrize("T,n_route,hidden", [(1, 256, 2048), (16, 256, 2048), (3, 60, 512), (5, 300, 1024)])
+def test_router_inside_the_gate_up_launch(capi, dev, T, n_route, hidden):
+    """llam_ql_moe_route_gate_up_swiglu against llam_ql_moe_route_quantize + llam_ql_moe_gate_up_swiglu: the same
+    ids and weights in the routed columns, the always-on column left as the caller set it, the same Q8_1 bytes for
+    every slot (up to 512 routed experts: four or eight per lane of the routing wavefront)."""
+    import torch
+    from oracle.binding import FMT_IQ3_S as fmt
+
+    inter, k = 256, 4
+    n_tab = n_route + 1                                  # the last table entry is the always-on expert
+    rng = np.random.default_rng(T + n_route)
+    # few distinct expert matrices, many table entries: the table repeats them
+    host, devs, _ = _experts(capi, dev, fmt, 7, hidden, inter, 50)
+    table = capi.expert_table([devs[e % 7] for e in range(n_tab)], dev)
+    x = torch.from_numpy(rng.standard_normal((T, hidden)).astype(np.float32)).to(dev)
+    logits = torch.from_numpy(rng.standard_normal((T, n_route)).astype(np.float32)).to(dev)
+
+    def fresh():
+        ids = torch.full((T, k + 1), n_route, dtype=torch.int32, device=dev)
+        w = torch.ones((T, k + 1), device=dev)
+        return ids, w
+
+    ids0, w0 = fresh()
+    q8h = torch.empty(T * (hidden // 32) * 36, dtype=torch.uint8, device=dev)
+    capi.moe_route_quantize(logits, k, x, q8h, ids=ids0, weights=w0)
+    want = capi.moe_gate_up_swiglu(fmt, table, n_tab, ids0, q8h, T, k + 1, hidden, inter)
+    ids1, w1 = fresh()
+    got = capi.moe_route_gate_up_swiglu(fmt, table, n_tab, logits, k, x, ids1, w1, inter, q8_hidden=torch.empty_like(q8h))
+    sync()
+    assert torch.equal(ids1, ids0) and torch.equal(w1, w0)
+    assert bool((ids1[:, k] == n_route).all()) and bool((w1[:, k] == 1.0).all())
+    assert torch.equal(got, want)
+
+
+def test_router_inside_other_formats_run_the_launches_one_by_one(capi, dev):
+    import torch
+
+    fmt, T, n_route, hidden, inter, k = FMT_Q4_K, 2, 5, 512, 256, 2
+    host, devs, table = _experts(capi, dev, fmt, n_route, hidden, inter, 77)
+    rng = np.random.default_rng(5)
+    x = torch.from_numpy(rng.standard_normal((T, hidden)).astype(np.float32)).to(dev)
+    logits = torch.from_numpy(rng.standard_normal((T, n_route)).astype(np.float32)).to(dev)
+    ids0 = torch.zeros((T, k), dtype=torch.int32, device=dev)
+    w0 = torch.zeros((T, k), device=dev)
+    q8h = torch.empty(T * (hidden // 32) * 36, dtype=torch.uint8, device=dev)
+    capi.moe_route_quantize(logits, k, x, q8h, ids=ids0, weights=w0)
+    gate, up = capi.moe_gate_up(fmt, table, n_route, ids0, q8h, T, k, hidden, inter)
+    want = capi.swiglu_quantize(gate, up)
+    ids1, w1 = torch.zeros_like(ids0), torch.zeros_like(w0)
+    got = capi.moe_route_gate_up_swiglu(fmt, table, n_route, logits, k, x, ids1, w1, inter, q8_hidden=torch.empty_like(q8h),
+                                        scratch=(torch.empty_like(gate), torch.empty_like(up)))
+    sync()
+    assert torch.equal(ids1, ids0) and torch.equal(w1, w0) and torch.equal(got, want)
+    with pytest.raises(capi.QLError, match="scratch"):
+        capi.moe_route_gate_up_swiglu(fmt, table, n_route, logits, k, x, ids1, w1, inter)
