@@ -430,6 +430,15 @@ namespace llamql
         // seven wavefronts per compute unit against 8.2 us with four)
         static constexpr int RESIDENT_WAVES = 16;
         __device__ __forceinline__ static void stage() {}
+        // decode tables fetched ahead of dependent loads (formats that have tables): none here
+        struct TablesRaw
+        {
+        };
+        static constexpr int TABLE_THREADS = 0;
+        __device__ __forceinline__ static void tables_issue(TablesRaw &) {}
+        template <int NEWER>
+        __device__ __forceinline__ static void tables_wait(TablesRaw &) {}
+        __device__ __forceinline__ static void tables_store(const TablesRaw &) {}
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         // workgroup size bound: one activation row leaves room for 16 wavefronts of 128 registers
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
@@ -634,6 +643,15 @@ namespace llamql
         // wavefronts per compute unit, 25.7 with seven)
         static constexpr int RESIDENT_WAVES = 8;
         __device__ __forceinline__ static void stage() {}
+        // decode tables fetched ahead of dependent loads (formats that have tables): none here
+        struct TablesRaw
+        {
+        };
+        static constexpr int TABLE_THREADS = 0;
+        __device__ __forceinline__ static void tables_issue(TablesRaw &) {}
+        template <int NEWER>
+        __device__ __forceinline__ static void tables_wait(TablesRaw &) {}
+        __device__ __forceinline__ static void tables_store(const TablesRaw &) {}
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
         static bool addressable(long N, int SB) { return (double)N * SB * 128.0 < 4.0e9; }
 

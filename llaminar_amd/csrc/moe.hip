@@ -1599,6 +1599,97 @@ namespace llamql
                                    normalize, d_ids, d_weights, slot_stride, qx, qo, q_blocks);
             return launched(fn);
         }
+        // ---- the quad-lane kernels on expert rows of 2, 4, 8 or 16 super-blocks, any format with such a decoder ----
+        template <class F>
+        bool moe_quad_ok(int rows, int nsb)
+        {
+            return moe_quad_rows(nsb) && F::Quad::addressable(rows, nsb);
+        }
+
+        // gate/up as fp32 rows: steps per wavefront so that a compute unit sees a few workgroups, each long
+        // enough to be worth its staging
+        template <class F>
+        bool moe_gate_up_quad_launch(const char *fn, MoEArgs m, int n_tokens, int device_id, hipStream_t st)
+        {
+            typedef typename F::Quad Q;
+            const int nsb = m.hidden / 256;
+            const long steps = ((long)m.inter * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+            const long all_steps = steps * n_tokens * m.top_k * 2;
+            int spw = 2;
+            while (spw < 8 && all_steps / ((long)cu_count(device_id) * MOE_QUAD_WAVES * 2) >= 2 * spw)
+                spw *= 2;
+            m.rows_per_wave = spw;
+            m.gshift = moe_log2(nsb);
+            const long gx = (steps + (long)MOE_QUAD_WAVES * spw - 1) / ((long)MOE_QUAD_WAVES * spw);
+            const dim3 grid((unsigned)gx, (unsigned)(n_tokens * m.top_k), 2);
+            hipLaunchKernelGGL((moe_gate_up_quad_kernel<Q>), grid, dim3(MOE_QUAD_WAVES * WAVE),
+                               (size_t)nsb * QUAD_SB_LDS, st, m);
+            return launched(fn);
+        }
+
+        // gate/up + SwiGLU + Q8_1 in one launch; rt: with the router and the hidden state's quantiser inside
+        template <class F>
+        bool moe_gate_up_swiglu_launch(const char *fn, MoEArgs m, uint32_t *q8_out, int n_tokens, int device_id,
+                                       hipStream_t st, const MoERouteArgs *rt = nullptr)
+        {
+            typedef typename F::Quad Q;
+            const int nsb = m.hidden / 256;
+            m.gshift = moe_log2(nsb);
+            m.rows_per_wave = 0;
+            const dim3 grid((unsigned)(m.inter / 32), (unsigned)(n_tokens * m.top_k)), block(MOE_QUAD_WAVES * WAVE);
+            const size_t lds = (size_t)nsb * QUAD_SB_LDS + 2 * 32 * sizeof(float);
+            if (rt)
+            {
+                if ((rt->n_route + WAVE - 1) / WAVE <= 4)
+                    hipLaunchKernelGGL((moe_route_gate_up_swiglu_kernel<Q, 4, 4>), grid, block, lds, st, m, q8_out, *rt);
+                else
+                    hipLaunchKernelGGL((moe_route_gate_up_swiglu_kernel<Q, 4, 8>), grid, block, lds, st, m, q8_out, *rt);
+            }
+            else if ((long)grid.x * grid.y >= 4L * cu_count(device_id))
+                hipLaunchKernelGGL((moe_gate_up_swiglu_dense_kernel<Q>), grid, block, lds, st, m, q8_out);
+            else
+                hipLaunchKernelGGL((moe_gate_up_swiglu_kernel<Q>), grid, block, lds, st, m, q8_out);
+            return launched(fn);
+        }
+
+        // down projection: 1 launched, 0 failed, -1 this format and shape have no quad-lane launch
+        template <class F>
+        int moe_down_quad_launch(const char *fn, MoEArgs m, int n_tokens, int device_id, hipStream_t st)
+        {
+            typedef typename F::Quad Q;
+            const int nsb = m.inter / 256, top_k = m.top_k;
+            if (!(moe_quad_ok<F>(m.hidden, nsb) && top_k <= MOE_QUAD_MAX_SLOTS &&
+                  (size_t)top_k * nsb * QUAD_SB_LDS + Q::STATIC_LDS + 4096 <= 64 * 1024))
+                return -1;
+            const long steps = ((long)m.hidden * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+            m.gshift = moe_log2(nsb);
+            // (with little work per compute unit the launch is a chain of memory round trips: there a wavefront
+            // per slot has every slot's loads of a row range in flight at once; it loses from 8 tokens of the
+            // 9-slot, 2-super-block shape on: 41.5 against 39.9 us per step)
+            if ((long)m.hidden * nsb / QUAD_STEP_SB * n_tokens * top_k < 48L * cu_count(device_id))
+            {
+                int spw = 1;
+                while (spw < MOE_SLOTWAVE_MAX_STEPS && steps * n_tokens / (2L * cu_count(device_id)) >= 2 * spw)
+                    spw *= 2;
+                m.rows_per_wave = spw;
+                const long gx = (steps + spw - 1) / spw;
+                const size_t lds = (size_t)top_k * nsb * QUAD_SB_LDS + (size_t)top_k * spw * (QUAD_STEP_SB / nsb) * sizeof(float);
+                // a wavefront per slot, and enough threads to fetch the decode tables a piece each
+                const int waves = top_k * WAVE >= Q::TABLE_THREADS ? top_k : (Q::TABLE_THREADS + WAVE - 1) / WAVE;
+                hipLaunchKernelGGL((moe_down_slotwave_kernel<Q>), dim3((unsigned)gx, (unsigned)n_tokens), dim3(waves * WAVE),
+                                   lds, st, m);
+                return launched(fn) ? 1 : 0;
+            }
+            // workgroups of a step or more per wavefront, at least two of them per compute unit
+            int spw = 1;
+            while (spw < 8 && steps * n_tokens / ((long)cu_count(device_id) * MOE_QUAD_WAVES * 2) >= 2 * spw)
+                spw *= 2;
+            m.rows_per_wave = spw;
+            const long gx = (steps + (long)MOE_QUAD_WAVES * spw - 1) / ((long)MOE_QUAD_WAVES * spw);
+            hipLaunchKernelGGL((moe_down_quad_kernel<Q>), dim3((unsigned)gx, (unsigned)n_tokens), dim3(MOE_QUAD_WAVES * WAVE),
+                               (size_t)top_k * nsb * QUAD_SB_LDS, st, m);
+            return launched(fn) ? 1 : 0;
+        }
     } // namespace
 } // namespace llamql
 
@@ -1662,23 +1753,20 @@ extern "C" bool llam_ql_moe_gate_up(uint8_t fmt, const llam_ql_expert *d_experts
     m.inter = inter;
     m.accumulate = 0;
     hipStream_t st = as_stream(stream);
-    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(hidden / 256) && IQ3STraits::Quad::addressable(inter, hidden / 256))
+    switch (fmt) // the quad-lane decoder on short rows
     {
-        // the quad-lane decoder on short rows: steps per wavefront so that a compute unit sees a few
-        // workgroups, each long enough to be worth its staging
-        typedef IQ3STraits::Quad Q;
-        const int nsb = hidden / 256;
-        const long steps = ((long)inter * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
-        const long all_steps = steps * n_tokens * top_k * 2;
-        int spw = 2;
-        while (spw < 8 && all_steps / ((long)cu_count(device_id) * MOE_QUAD_WAVES * 2) >= 2 * spw)
-            spw *= 2;
-        m.rows_per_wave = spw;
-        m.gshift = moe_log2(nsb);
-        const long gx = (steps + (long)MOE_QUAD_WAVES * spw - 1) / ((long)MOE_QUAD_WAVES * spw);
-        const dim3 grid((unsigned)gx, (unsigned)(n_tokens * top_k), 2);
-        hipLaunchKernelGGL((moe_gate_up_quad_kernel<Q>), grid, dim3(MOE_QUAD_WAVES * WAVE), (size_t)nsb * QUAD_SB_LDS, st, m);
-        return launched(fn);
+    case LLAM_FMT_Q4_K:
+        if (moe_quad_ok<Q4KTraits>(inter, hidden / 256))
+            return moe_gate_up_quad_launch<Q4KTraits>(fn, m, n_tokens, device_id, st);
+        break;
+    case LLAM_FMT_Q6_K:
+        if (moe_quad_ok<Q6KTraits>(inter, hidden / 256))
+            return moe_gate_up_quad_launch<Q6KTraits>(fn, m, n_tokens, device_id, st);
+        break;
+    default:
+        if (moe_quad_ok<IQ3STraits>(inter, hidden / 256))
+            return moe_gate_up_quad_launch<IQ3STraits>(fn, m, n_tokens, device_id, st);
+        break;
     }
     long gx;
     moe_shape(inter, hidden / 256, (long)n_tokens * top_k * 2, device_id, m.gshift, m.rows_per_wave, gx);
@@ -1727,12 +1815,13 @@ extern "C" bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_
         return fail(fn, "null pointer");
     if (!aligned4(d_q8_out))
         return fail(fn, "d_q8_out must be 4-byte aligned");
-    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(hidden / 256) && IQ3STraits::Quad::addressable(inter, hidden / 256) &&
-        inter % 32 == 0)
+    const bool one_launch = fmt == LLAM_FMT_Q4_K   ? moe_quad_ok<Q4KTraits>(inter, hidden / 256)
+                            : fmt == LLAM_FMT_Q6_K ? moe_quad_ok<Q6KTraits>(inter, hidden / 256)
+                                                   : moe_quad_ok<IQ3STraits>(inter, hidden / 256);
+    if (one_launch) // (inter is a multiple of 256: whole Q8_1 blocks per workgroup)
     {
         if (!set_device(fn, device_id))
             return false;
-        typedef IQ3STraits::Quad Q;
         MoEArgs m;
         m.experts = d_experts;
         m.ids = d_ids;
@@ -1745,22 +1834,18 @@ extern "C" bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_
         m.hidden = hidden;
         m.inter = inter;
         m.accumulate = 0;
-        m.rows_per_wave = 0;
-        const int nsb = hidden / 256;
-        m.gshift = moe_log2(nsb);
-        const dim3 grid((unsigned)(inter / 32), (unsigned)(n_tokens * top_k));
-        const size_t lds = (size_t)nsb * QUAD_SB_LDS + 2 * 32 * sizeof(float);
-        if ((long)grid.x * grid.y >= 4L * cu_count(device_id))
-            hipLaunchKernelGGL((moe_gate_up_swiglu_dense_kernel<Q>), grid, dim3(MOE_QUAD_WAVES * WAVE), lds,
-                               as_stream(stream), m, static_cast<uint32_t *>(d_q8_out));
-        else
-            hipLaunchKernelGGL((moe_gate_up_swiglu_kernel<Q>), grid, dim3(MOE_QUAD_WAVES * WAVE), lds,
-                               as_stream(stream), m, static_cast<uint32_t *>(d_q8_out));
-        return launched(fn);
+        uint32_t *out = static_cast<uint32_t *>(d_q8_out);
+        hipStream_t st = as_stream(stream);
+        switch (fmt)
+        {
+        case LLAM_FMT_Q4_K: return moe_gate_up_swiglu_launch<Q4KTraits>(fn, m, out, n_tokens, device_id, st);
+        case LLAM_FMT_Q6_K: return moe_gate_up_swiglu_launch<Q6KTraits>(fn, m, out, n_tokens, device_id, st);
+        default: return moe_gate_up_swiglu_launch<IQ3STraits>(fn, m, out, n_tokens, device_id, st);
+        }
     }
-    // other formats and row lengths: the two launches, through the caller's fp32 scratch
+    // other row lengths: the two launches, through the caller's fp32 scratch
     if (!d_gate_scratch || !d_up_scratch)
-        return fail(fn, "this format and shape need the fp32 scratch rows (d_gate_scratch, d_up_scratch)");
+        return fail(fn, "this shape needs the fp32 scratch rows (d_gate_scratch, d_up_scratch)");
     if (!llam_ql_moe_gate_up(fmt, d_experts, n_experts, d_ids, d_q8, d_gate_scratch, d_up_scratch, n_tokens, top_k,
                              hidden, inter, device_id, stream))
         return false;
@@ -1793,12 +1878,13 @@ extern "C" bool llam_ql_moe_route_gate_up_swiglu(uint8_t fmt, const llam_ql_expe
     // routing repeated by every workgroup costs more than the launch it saves (4 tokens 30.4 against 29.7 us,
     // 16 tokens 64.3 against 59.4-61.8 us).
     const bool few = (long)(inter / 32) * n_tokens * slot_stride < 2L * cu_count(device_id);
-    if (fmt == LLAM_FMT_IQ3_S && moe_quad_rows(hidden / 256) && IQ3STraits::Quad::addressable(inter, hidden / 256) &&
-        inter % 32 == 0 && per <= 8 && few)
+    const bool quad = fmt == LLAM_FMT_Q4_K   ? moe_quad_ok<Q4KTraits>(inter, hidden / 256)
+                      : fmt == LLAM_FMT_Q6_K ? moe_quad_ok<Q6KTraits>(inter, hidden / 256)
+                                             : moe_quad_ok<IQ3STraits>(inter, hidden / 256);
+    if (quad && per <= 8 && few)
     {
         if (!set_device(fn, device_id))
             return false;
-        typedef IQ3STraits::Quad Q;
         MoEArgs m;
         m.experts = d_experts;
         m.ids = d_ids;
@@ -1811,9 +1897,6 @@ extern "C" bool llam_ql_moe_route_gate_up_swiglu(uint8_t fmt, const llam_ql_expe
         m.hidden = hidden;
         m.inter = inter;
         m.accumulate = 0;
-        m.rows_per_wave = 0;
-        const int nsb = hidden / 256;
-        m.gshift = moe_log2(nsb);
         MoERouteArgs r;
         r.logits = d_logits;
         r.x = d_hidden;
@@ -1822,19 +1905,18 @@ extern "C" bool llam_ql_moe_route_gate_up_swiglu(uint8_t fmt, const llam_ql_expe
         r.n_route = n_route_experts;
         r.top_k = top_k;
         r.normalize = normalize;
-        const dim3 grid((unsigned)(inter / 32), (unsigned)(n_tokens * slot_stride)), block(MOE_QUAD_WAVES * WAVE);
-        const size_t lds = (size_t)nsb * QUAD_SB_LDS + 2 * 32 * sizeof(float);
         hipStream_t st = as_stream(stream);
         uint32_t *out = static_cast<uint32_t *>(d_q8_out);
-        if (per <= 4)
-            hipLaunchKernelGGL((moe_route_gate_up_swiglu_kernel<Q, 4, 4>), grid, block, lds, st, m, out, r);
-        else
-            hipLaunchKernelGGL((moe_route_gate_up_swiglu_kernel<Q, 4, 8>), grid, block, lds, st, m, out, r);
-        return launched(fn);
+        switch (fmt)
+        {
+        case LLAM_FMT_Q4_K: return moe_gate_up_swiglu_launch<Q4KTraits>(fn, m, out, n_tokens, device_id, st, &r);
+        case LLAM_FMT_Q6_K: return moe_gate_up_swiglu_launch<Q6KTraits>(fn, m, out, n_tokens, device_id, st, &r);
+        default: return moe_gate_up_swiglu_launch<IQ3STraits>(fn, m, out, n_tokens, device_id, st, &r);
+        }
     }
-    // more tokens, other formats and row lengths, more than 512 routed experts: the launches one by one
+    // more tokens, other row lengths, more than 512 routed experts: the launches one by one
     if (!d_q8_hidden_scratch)
-        return fail(fn, "this format, shape or token count needs the Q8_1 scratch of the hidden state (d_q8_hidden_scratch)");
+        return fail(fn, "this shape or token count needs the Q8_1 scratch of the hidden state (d_q8_hidden_scratch)");
     if (!llam_ql_moe_route_quantize(d_logits, n_tokens, n_route_experts, top_k, normalize, d_ids, d_weights, slot_stride,
                                     d_hidden, hidden, d_q8_hidden_scratch, device_id, stream))
         return false;
@@ -2041,47 +2123,12 @@ extern "C" bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts, i
     m.inter = inter;
     m.accumulate = accumulate;
     hipStream_t st = as_stream(stream);
-    // (with little work per compute unit the launch is a chain of memory round trips: there the kernel that
-    // has the loads of all slots of a row in flight at once is faster -- 1 token 24.1 against 26.9 us per step,
-    // 4 tokens 35.3 against 37.1, 8 tokens 54.9 against 47.5, 16 tokens 78.9 against 67.0)
-    const bool quad_down = fmt == LLAM_FMT_IQ3_S && moe_quad_rows(inter / 256) && top_k <= MOE_QUAD_MAX_SLOTS &&
-                           IQ3STraits::Quad::addressable(hidden, inter / 256) &&
-                           (size_t)top_k * (inter / 256) * QUAD_SB_LDS + IQ3STraits::Quad::STATIC_LDS + 4096 <= 64 * 1024;
-    const bool much_work = (long)hidden * (inter / 256) / QUAD_STEP_SB * n_tokens * top_k >= 48L * cu_count(device_id);
-    if (quad_down && !much_work)
     {
-        // a few tokens: a wavefront per slot, every slot's loads of a row range in flight at once
-        typedef IQ3STraits::Quad Q;
-        const int nsb = inter / 256;
-        const long steps = ((long)hidden * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
-        int spw = 1;
-        while (spw < MOE_SLOTWAVE_MAX_STEPS && steps * n_tokens / (2L * cu_count(device_id)) >= 2 * spw)
-            spw *= 2;
-        m.rows_per_wave = spw;
-        m.gshift = moe_log2(nsb);
-        const long gx = (steps + spw - 1) / spw;
-        const size_t lds = (size_t)top_k * nsb * QUAD_SB_LDS + (size_t)top_k * spw * (QUAD_STEP_SB / nsb) * sizeof(float);
-        // a wavefront per slot, and enough threads to fetch the decode tables a piece each
-        const int waves = top_k * WAVE >= Q::TABLE_THREADS ? top_k : (Q::TABLE_THREADS + WAVE - 1) / WAVE;
-        hipLaunchKernelGGL((moe_down_slotwave_kernel<Q>), dim3((unsigned)gx, (unsigned)n_tokens), dim3(waves * WAVE), lds, st, m);
-        return launched(fn);
-    }
-    if (quad_down)
-    {
-        // the quad-lane decoder on short rows: workgroups of a step or more per wavefront, at least
-        // two of them per compute unit
-        typedef IQ3STraits::Quad Q;
-        const int nsb = inter / 256;
-        const long steps = ((long)hidden * nsb + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
-        int spw = 1;
-        while (spw < 8 && steps * n_tokens / ((long)cu_count(device_id) * MOE_QUAD_WAVES * 2) >= 2 * spw)
-            spw *= 2;
-        m.rows_per_wave = spw;
-        m.gshift = moe_log2(nsb);
-        const long gx = (steps + (long)MOE_QUAD_WAVES * spw - 1) / ((long)MOE_QUAD_WAVES * spw);
-        hipLaunchKernelGGL((moe_down_quad_kernel<Q>), dim3((unsigned)gx, (unsigned)n_tokens), dim3(MOE_QUAD_WAVES * WAVE),
-                           (size_t)top_k * nsb * QUAD_SB_LDS, st, m);
-        return launched(fn);
+        const int r = fmt == LLAM_FMT_Q4_K   ? moe_down_quad_launch<Q4KTraits>(fn, m, n_tokens, device_id, st)
+                      : fmt == LLAM_FMT_Q6_K ? moe_down_quad_launch<Q6KTraits>(fn, m, n_tokens, device_id, st)
+                                             : moe_down_quad_launch<IQ3STraits>(fn, m, n_tokens, device_id, st);
+        if (r >= 0)
+            return r == 1;
     }
     long gx;
     moe_shape(hidden, inter / 256, (long)n_tokens, device_id, m.gshift, m.rows_per_wave, gx);

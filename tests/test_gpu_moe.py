@@ -279,15 +279,12 @@ def test_group_tokens_by_expert(capi, dev):
 def test_grouped_launches_equal_ungrouped(capi, dev, fmt):
     """Tokens grouped by expert: every gate/up row and every token output carries the bits of
     the ungrouped launches (12 tokens on 5 experts + an always-on slot: segments of 1..12 tokens,
-    an expert missing from the table, an id out of range).  IQ3_S: the per-slot launches run the
-    quad-lane decoder, which adds a row's blocks in another order than the grouped launches' kernel:
-    equal to 1e-5 of the largest value there, and exactly equal where nothing is written."""
+    an expert missing from the table, an id out of range).  On rows of 2, 4, 8 or 16 super-blocks (as here) the
+    per-slot launches run the quad-lane decoders, which add a row's blocks in another order than the grouped
+    launches' kernel: equal to 1e-5 of the largest value there, and exactly equal where nothing is written."""
     import torch
-    from oracle.binding import FMT_IQ3_S
 
     def same(a, b):
-        if fmt != FMT_IQ3_S:
-            return torch.equal(a, b)
         untouched = (b == 3.0) | torch.isnan(b)
         return bool((a[untouched] == b[untouched]).all() | torch.isnan(a[untouched]).all()) and \
             float((a[~untouched] - b[~untouched]).abs().max()) <= 1e-5 * float(b[~untouched].abs().max())
@@ -460,13 +457,13 @@ def test_short_row_quad_lane_kernels_against_the_oracle(capi, dev, oracle):
     assert rel_err(acc_h - 2.0, want.astype(np.float32)) <= 1e-5
 
 
-@pytest.mark.parametrize("hidden", [512, 1024, 2048, 4096])
-def test_gate_up_swiglu_in_one_launch_has_the_bits_of_the_two(capi, dev, hidden):
-    """IQ3_S rows of 2, 4, 8 and 16 super-blocks: the Q8_1 blocks of the one-launch gate/up + SwiGLU + quantiser are
+@pytest.mark.parametrize("fmt,hidden", [(FMT_IQ3_S, 512), (FMT_IQ3_S, 1024), (FMT_IQ3_S, 2048), (FMT_IQ3_S, 4096),
+                                        (FMT_Q4_K, 512), (FMT_Q4_K, 2048), (FMT_Q6_K, 1024), (FMT_Q6_K, 4096)])
+def test_gate_up_swiglu_in_one_launch_has_the_bits_of_the_two(capi, dev, fmt, hidden):
+    """Rows of 2, 4, 8 and 16 super-blocks: the Q8_1 blocks of the one-launch gate/up + SwiGLU + quantiser are
     the bytes of llam_ql_moe_gate_up followed by llam_ql_swiglu_quantize; blocks of a slot with an id out of range
     or an expert that lives elsewhere keep what the buffer held.  No scratch rows are needed (or touched)."""
     import torch
-    from oracle.binding import FMT_IQ3_S as fmt
 
     n_exp, inter, k, T = 5, 768, 3, 5
     host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 33)
@@ -493,13 +490,12 @@ def test_gate_up_swiglu_in_one_launch_has_the_bits_of_the_two(capi, dev, hidden)
             assert bool((got[r] == 0x5A).all()), r
 
 
-def test_gate_up_swiglu_other_formats_run_the_two_launches(capi, dev):
-    """Q4_K experts (and IQ3_S rows that are no power of two of super-blocks) go through the caller's fp32 scratch
-    rows; without them the call is refused."""
+def test_gate_up_swiglu_other_row_lengths_run_the_two_launches(capi, dev):
+    """Rows that are no power of two of super-blocks go through the caller's fp32 scratch rows; without them the
+    call is refused."""
     import torch
-    from oracle.binding import FMT_IQ3_S
 
-    for fmt, hidden in ((FMT_Q4_K, 512), (FMT_IQ3_S, 768)):
+    for fmt, hidden in ((FMT_Q4_K, 768), (FMT_IQ3_S, 768)):
         n_exp, inter, k, T = 3, 256, 2, 3
         host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 12)
         ids = torch.tensor([[0, 1], [2, 0], [1, 2]], dtype=torch.int32, device=dev)
@@ -514,16 +510,16 @@ def test_gate_up_swiglu_other_formats_run_the_two_launches(capi, dev):
             capi.moe_gate_up_swiglu(fmt, table, n_exp, ids, qd, T, k, hidden, inter)
 
 
-@pytest.mark.parametrize("shape", [(2048, 512, 9, 1), (2048, 512, 9, 4), (1024, 1024, 4, 2), (512, 2048, 16, 1),
-                                   (768, 512, 3, 3)])
+@pytest.mark.parametrize("shape", [(FMT_IQ3_S, 2048, 512, 9, 1), (FMT_IQ3_S, 2048, 512, 9, 4), (FMT_IQ3_S, 1024, 1024, 4, 2),
+                                   (FMT_IQ3_S, 512, 2048, 16, 1), (FMT_IQ3_S, 768, 512, 3, 3), (FMT_Q4_K, 1024, 512, 5, 2),
+                                   (FMT_Q6_K, 512, 1024, 3, 1), (FMT_Q4_K, 768, 4096, 2, 3)])
 def test_down_of_a_few_tokens_wavefront_per_slot(capi, dev, oracle, shape):
-    """IQ3_S down projection with little work per compute unit (a wavefront per slot): weighted sums against the CPU
+    """Down projection with little work per compute unit (a wavefront per slot): weighted sums against the CPU
     restatement on the same Q8_1 input, overwrite and accumulate, with a dead slot, a dead token when there are
     several, and the grouped path's bits to 1e-5 (its kernel adds a row's blocks in another order)."""
     import torch
-    from oracle.binding import FMT_IQ3_S as fmt
 
-    hidden, inter, k, T = shape
+    fmt, hidden, inter, k, T = shape
     n_exp = 5
     host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 70 + k)
     tab = table.clone()
@@ -565,13 +561,13 @@ def test_down_of_a_few_tokens_wavefront_per_slot(capi, dev, oracle, shape):
     assert float((out_g - out).abs().max()) <= 1e-5 * float(out.abs().max())
 
 
-@pytest.mark.parametrize("T,n_route,hidden", [(1, 256, 2048), (16, 256, 2048), (3, 60, 512), (5, 300, 1024)])
-def test_router_inside_the_gate_up_launch(capi, dev, T, n_route, hidden):
+@pytest.mark.parametrize("fmt,T,n_route,hidden", [(FMT_IQ3_S, 1, 256, 2048), (FMT_IQ3_S, 16, 256, 2048), (FMT_IQ3_S, 3, 60, 512),
+                                                  (FMT_IQ3_S, 5, 300, 1024), (FMT_Q4_K, 2, 128, 1024), (FMT_Q6_K, 1, 64, 2048)])
+def test_router_inside_the_gate_up_launch(capi, dev, fmt, T, n_route, hidden):
     """llam_ql_moe_route_gate_up_swiglu against llam_ql_moe_route_quantize + llam_ql_moe_gate_up_swiglu: the same
     ids and weights in the routed columns, the always-on column left as the caller set it, the same Q8_1 bytes for
     every slot (up to 512 routed experts: four or eight per lane of the routing wavefront)."""
     import torch
-    from oracle.binding import FMT_IQ3_S as fmt
 
     inter, k = 256, 4
     n_tab = n_route + 1                                  # the last table entry is the always-on expert
@@ -599,10 +595,10 @@ def test_router_inside_the_gate_up_launch(capi, dev, T, n_route, hidden):
     assert torch.equal(got, want)
 
 
-def test_router_inside_other_formats_run_the_launches_one_by_one(capi, dev):
+def test_router_inside_other_row_lengths_run_the_launches_one_by_one(capi, dev):
     import torch
 
-    fmt, T, n_route, hidden, inter, k = FMT_Q4_K, 2, 5, 512, 256, 2
+    fmt, T, n_route, hidden, inter, k = FMT_Q4_K, 2, 5, 768, 256, 2   # rows of three super-blocks: no quad-lane launch
     host, devs, table = _experts(capi, dev, fmt, n_route, hidden, inter, 77)
     rng = np.random.default_rng(5)
     x = torch.from_numpy(rng.standard_normal((T, hidden)).astype(np.float32)).to(dev)
