@@ -352,9 +352,9 @@ bool llam_ql_moe_down(uint8_t fmt, const llam_ql_expert *d_experts,
 
 /* llam_ql_moe_gate_up followed by llam_ql_swiglu_quantize, the same Q8_1 bytes:
  *   d_q8_out [(t*top_k+s)][inter/32] = Q8_1(silu(W_gate[e] . q8(hidden[t])) * (W_up[e] . q8(hidden[t])))
- * For IQ3_S experts with hidden/256 in {2,4,8,16} this is ONE launch: a workgroup owns the 32
+ * For expert rows of 2, 4, 8 or 16 super-blocks (hidden/256) this is ONE launch: a workgroup owns the 32
  * gate and 32 up rows of one Q8_1 block, so the fp32 intermediate never leaves the chip and
- * d_gate_scratch / d_up_scratch may be NULL.  Every other format and row length runs the two
+ * d_gate_scratch / d_up_scratch may be NULL.  Every other row length runs the two
  * launches through the scratch rows (fp32 [n_tokens*top_k x inter] each; NULL is refused there).
  * Blocks of skipped slots (id outside [0,n_experts), NULL matrix) are left untouched in the
  * one-launch form and are quantised from whatever the scratch holds in the other; no later
@@ -366,7 +366,7 @@ bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_experts, in
                                 int hidden, int inter, int device_id, void *stream);
 
 /* llam_ql_moe_route_quantize followed by llam_ql_moe_gate_up_swiglu: the same ids, weights and Q8_1
- * bytes.  For IQ3_S experts with hidden/256 in {2,4,8,16}, at most 512 routed experts and few tokens
+ * bytes.  For expert rows of 2, 4, 8 or 16 super-blocks (hidden/256), at most 512 routed experts and few tokens
  * (fewer workgroups than two per compute unit: one or two tokens of a 9-slot, 512-row expert shape)
  * this is ONE launch: every workgroup quantises its token's hidden row into its LDS and routes the
  * token for itself (work that precedes the first weight load in any case), so a decode step is two
@@ -375,7 +375,7 @@ bool llam_ql_moe_gate_up_swiglu(uint8_t fmt, const llam_ql_expert *d_experts, in
  * [n_tokens x slot_stride]: columns < top_k are written, columns top_k.. are READ as always-on slots
  * (the shared expert: its table index and weight, set by the caller once); the expert table has
  * n_experts >= n_route_experts entries.  d_hidden fp32 [n_tokens x hidden].  The two-launch form
- * needs d_q8_hidden_scratch (Q8_1 [n_tokens x hidden/32]) and, for formats and shapes outside
+ * needs d_q8_hidden_scratch (Q8_1 [n_tokens x hidden/32]) and, for row lengths outside
  * llam_ql_moe_gate_up_swiglu's one-launch kernel, its fp32 scratch rows; a caller that cannot tell
  * passes all three (they are left untouched when not needed).
  * Counterpart of decodeRouteSelect + groupedExpertGateUpDecodeFromRuntime + swiGLU
