@@ -139,8 +139,8 @@ def bench_moe(args, torch, capi, synth, dev):
 
     # Batches sort the (token, slot) pairs by expert on the device and read every distinct
     # expert's matrices once (6 launches); a single token has nothing to group (2 launches).
-    # (measured: per-slot launches 67 us at 16 tokens, 107 against 135 grouped at 32, 184 against 201 at 64, 334 against 296 at 128)
-    path = args.moe_path if args.moe_path != "auto" else ("grouped" if T * (TOPK + 1) >= 768 else "slots")
+    # (measured, grouped against per slot: 32 tokens 115 / 107 us, 48 tokens 142 / 144, 64 tokens 155 / 188, 128 tokens 228 / 340)
+    path = args.moe_path if args.moe_path != "auto" else ("grouped" if T * (TOPK + 1) >= 432 else "slots")
     S = TOPK + 1
     for s_ in sets:
         s_["group"] = torch.empty(int(capi.load().llam_ql_moe_group_bytes(T, S)), dtype=torch.uint8, device=dev)

@@ -280,8 +280,8 @@ namespace llamql
                     {
                         const size_t orow = a.pairs ? (size_t)a.pairs[m] : (size_t)m;
                         float *dst = a.y + orow * a.ldy + row;
-                        const float v = a.out_scale * total;
-                        *dst = a.accumulate ? (*dst + v) : v;
+                        const float v = weighted(a.out_scale, total);
+                        *dst = a.accumulate ? add_rounded(*dst, v) : v;
                     }
                 }
             }

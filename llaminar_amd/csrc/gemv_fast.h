@@ -218,8 +218,8 @@ namespace llamql
                     if (lane == 0)
                     {
                         float *dst = a.y + (size_t)m * a.ldy + row;
-                        const float v = a.out_scale * total;
-                        *dst = a.accumulate ? (*dst + v) : v;
+                        const float v = weighted(a.out_scale, total);
+                        *dst = a.accumulate ? add_rounded(*dst, v) : v;
                     }
                 }
             }

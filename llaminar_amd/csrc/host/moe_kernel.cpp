@@ -31,7 +31,7 @@ namespace llaminar_amd
             return ok;
         }
         constexpr size_t ALIGN = 256;
-        constexpr size_t GROUP_MIN_PAIRS = 768; // (token, slot) pairs from which batches are grouped by expert
+        constexpr size_t GROUP_MIN_PAIRS = 432; // (token, slot) pairs from which batches are grouped by expert
         size_t round_up(size_t b) { return (b + ALIGN - 1) / ALIGN * ALIGN; }
         size_t q8_bytes(size_t rows, int k) { return rows * (size_t)(k / 32) * sizeof(llam_block_q8_1); }
     } // namespace
@@ -313,9 +313,9 @@ namespace llaminar_amd
         const int T = input->rows;
         const size_t rows = (size_t)T * top_k;
         // Batches of GROUP_MIN_PAIRS (token, slot) pairs and more are sorted by expert on the
-        // device, so that every distinct expert's matrices are read once per chunk of its
-        // tokens (measured on the 256-expert IQ3_S shape with 9 slots per token: 64 tokens 201 us grouped
-        // against 184 us per slot, 128 tokens 296 against 334 us).
+        // device, so that every distinct expert's matrices are decoded once per chunk of its
+        // tokens (measured on the 256-expert IQ3_S shape with 9 slots per token, grouped against per slot:
+        // 40 tokens 126 / 127 us, 48 tokens 142 / 144, 64 tokens 155 / 188, 128 tokens 228 / 340 us).
         const bool grouped = rows >= GROUP_MIN_PAIRS && rows <= 4096 && tg->num_experts <= 2048 &&
                              tg->num_experts == td->num_experts;
         Scratch s;

@@ -444,15 +444,15 @@ namespace llamql
             const int slot = live[k].slot;
             float v = moe_quad_step<Q>(buf, lc, aq_lane + (size_t)slot * nsb * QUAD_SB_LDS);
             v = sb < total ? v : 0.0f;
-            const float val = live[k].weight * moe_quad_row_sum(v, nsb_log2);
+            const float val = weighted(live[k].weight, moe_quad_row_sum(v, nsb_log2));
             const bool writer = sb < total && (lane & seg_mask) == 0;
             float *const dst = m.out0 + (size_t)t * m.hidden + (writer ? (sb >> nsb_log2) : 0);
             // the first live slot starts the sum: from what the output holds when accumulating
             // (((out + v0) + v1) + .., the per-slot kernel's order), else from nothing
             if (k == 0)
-                y = (m.accumulate && writer) ? *dst + val : val;
+                y = (m.accumulate && writer) ? add_rounded(*dst, val) : val;
             else
-                y = y + val;
+                y = add_rounded(y, val);
             if (++k == n_live)
             {
                 if (writer)
@@ -600,11 +600,11 @@ namespace llamql
             {
                 if (!slot_live[s])
                     continue;
-                const float val = slot_weight[s] * part[s * rows_wg + r];
+                const float val = weighted(slot_weight[s], part[s * rows_wg + r]);
                 if (first)
-                    y = m.accumulate ? *dst + val : val;
+                    y = m.accumulate ? add_rounded(*dst, val) : val;
                 else
-                    y = y + val;
+                    y = add_rounded(y, val);
                 first = false;
             }
             if (!first || m.accumulate == 0) // no live slot: zeros unless accumulating
@@ -986,14 +986,14 @@ namespace llamql
                         acc = fmaf(asd[kb], bmin, acc);
                 }
                 const float total = segment_sum(acc, m.gshift);
-                const float v = wt[s] * total;
+                const float v = weighted(wt[s], total);
                 if (first)
                 {
                     y = v; // accumulate == 0: the first live slot overwrites
                     first = false;
                 }
                 else
-                    y = y + v;
+                    y = add_rounded(y, v);
             }
             // (a token without a live slot: y is 0, which overwrites when accumulate == 0)
             if (writer)
@@ -1253,6 +1253,129 @@ namespace llamql
         moe_chunk_body<F, MAXM>(a, g, chunk, lds);
     }
 
+    // The grouped launches on the quad-lane decoder (expert rows of 2, 4, 8 or 16 super-blocks): a workgroup
+    // row takes one chunk -- an expert and 1..MAXM of its (token, slot) pairs -- decodes every step of the
+    // expert's matrix ONCE and multiplies it with each pair's activation row: per pair the decode, the dots
+    // and the row sum of moe_gate_up_quad_kernel / moe_down_quad_kernel, the same bits.
+    // DOWN = false: grid (workgroups per matrix, chunks (upper bound), 2 = gate|up), activations = the
+    // pair's token's hidden row, outputs out0/out1[pair][inter].  DOWN = true: grid (workgroups, chunks),
+    // activations = the pair's own row of inter values, outputs out1[pair][hidden] (unweighted).
+    // m.rows_per_wave: steps per wavefront, m.gshift: log2(nsb).
+    template <class Q, int MAXM, bool DOWN>
+    __global__ void __launch_bounds__(MOE_QUAD_WAVES *WAVE) moe_grouped_quad_kernel(const MoEArgs m, void *ws, int P)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t moe_quad_lds[];
+        const MoEGroupView g = moe_group_view(ws, P);
+        const int chunk = blockIdx.y;
+        if (chunk >= g.head[2])
+            return; // uniform
+        const int e = g.chunk_expert[chunk];
+        const void *w = DOWN ? m.experts[e].d_down : (blockIdx.z == 0 ? m.experts[e].d_gate : m.experts[e].d_up);
+        if (!w)
+            return; // an expert whose matrices live elsewhere (uniform)
+        const int n = g.chunk_count[chunk]; // uniform, 1..MAXM
+        const int32_t *pairs = g.pair_sorted + g.chunk_begin[chunk];
+        const int K = DOWN ? m.inter : m.hidden, N = DOWN ? m.hidden : m.inter;
+        const int nsb_log2 = m.gshift, nsb = 1 << nsb_log2;
+        GemvArgs a; // weight addressing only
+        a.w = uniform_ptr(w);
+        a.N = N;
+        a.SB = nsb;
+
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int l = lane & 3, grp = lane >> 2;
+        const typename Q::Lane lc = Q::lane_consts(l);
+        const int total = N * nsb; // super-blocks of the matrix
+        const int step0 = ((int)blockIdx.x * MOE_QUAD_WAVES + wave) * m.rows_per_wave;
+        const int nsteps = min(m.rows_per_wave, max(0, (total + QUAD_STEP_SB - 1) / QUAD_STEP_SB - step0));
+        // loads are never predicated: past the end a lane re-reads its first super-block
+        const size_t t0 = (size_t)min(step0 * QUAD_STEP_SB + grp, total - 1);
+        typename Q::Cursor wc = Q::cursor(a, t0, t0, lc);
+        const typename Q::Stride stride = Q::stride(0);
+        int ld_step = 0;
+        auto issue = [&](typename Q::Raw &buf) {
+            Q::load(buf, wc, lc, ld_step < nsteps && (step0 + ld_step) * QUAD_STEP_SB + grp < total);
+            Q::next(wc, false, stride);
+            ++ld_step;
+        };
+        typename Q::Raw bufA, bufB;
+        issue(bufA);
+        issue(bufB);
+        // the chunk's activation rows, one thread per Q8_1 block (row mm of the chunk at mm * nsb super-blocks)
+        const int nkb = nsb * 8;
+        for (int idx = threadIdx.x; idx < n * nkb; idx += blockDim.x)
+        {
+            const int mm = idx / nkb, kb = idx - mm * nkb;
+            const int pair = pairs[mm];
+            const uint32_t *src = m.q8 + ((size_t)(DOWN ? pair : pair / m.top_k) * nkb + kb) * 9;
+            uint32_t v[9];
+#pragma unroll
+            for (int i = 0; i < 9; ++i)
+                v[i] = src[i];
+            const float d = h2f((uint16_t)(v[0] & 0xFFFFu));
+            const int sb = kb >> 3, j = kb & 7;
+            int ll, odd;
+            Q::owner(j, ll, odd);
+            uint8_t *base = moe_quad_lds + ((size_t)mm * nsb + sb) * QUAD_SB_LDS + ll * 16;
+            *reinterpret_cast<float2 *>(base + 256 + odd * 8) = make_float2(d, (float)(int16_t)(v[0] >> 16) * d);
+            *reinterpret_cast<uint4 *>(base + (odd * 2) * 64) = make_uint4(v[1], v[2], v[3], v[4]);
+            *reinterpret_cast<uint4 *>(base + (odd * 2 + 1) * 64) = make_uint4(v[5], v[6], v[7], v[8]);
+        }
+        Q::stage();
+        __syncthreads();
+        Q::keep(bufA);
+        Q::keep(bufB);
+
+        const uint8_t *aq_lane = moe_quad_lds + (grp & (nsb - 1)) * QUAD_SB_LDS + (l << 4);
+        const int seg_mask = (4 << nsb_log2) - 1;
+        float *out = DOWN ? m.out1 : (blockIdx.z == 0 ? m.out0 : m.out1);
+        int step = 0;
+        auto compute = [&](const typename Q::Raw &buf) {
+            const int sb = (step0 + step) * QUAD_STEP_SB + grp;
+            v4i wq[4];
+            typename Q::Scale S;
+            Q::decode(buf, lc, wq, S);
+#pragma unroll
+            for (int mm = 0; mm < MAXM; ++mm)
+            {
+                if (mm < n) // uniform
+                {
+                    const uint8_t *ar = aq_lane + (size_t)mm * nsb * QUAD_SB_LDS;
+                    const v4i a0 = *reinterpret_cast<const v4i *>(ar);
+                    const v4i a1 = *reinterpret_cast<const v4i *>(ar + 64);
+                    const v4i a2 = *reinterpret_cast<const v4i *>(ar + 128);
+                    const v4i a3 = *reinterpret_cast<const v4i *>(ar + 192);
+                    const float4 sd = *reinterpret_cast<const float4 *>(ar + 256);
+                    const int i0 = dot16(a1, wq[1], dot16z(a0, wq[0]));
+                    const int i1 = dot16(a3, wq[3], dot16z(a2, wq[2]));
+                    float v = Q::apply(S, i0, i1, sd, 0.0f);
+                    v = sb < total ? v : 0.0f;
+                    const float tot = moe_quad_row_sum(v, nsb_log2);
+                    if (sb < total && (lane & seg_mask) == 0)
+                        out[(size_t)pairs[mm] * N + (sb >> nsb_log2)] = tot;
+                }
+            }
+            ++step;
+        };
+        for (int c0 = 0; c0 < nsteps; c0 += 2)
+        {
+            Q::template wait<Q::LOADS>(bufA);
+            if (step < nsteps) // uniform
+                compute(bufA);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufA);
+            Q::template wait<Q::LOADS>(bufB);
+            if (step < nsteps)
+                compute(bufB);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(bufB);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // loads issued past the end
+        Q::keep(bufA);
+        Q::keep(bufB);
+    }
+
     // out[t][h] (+)= sum over the token's live slots, ascending, of weight * pair_out[pair][h]:
     // the arithmetic and order of moe_down_kernel, so the same bits.  A token without a live
     // slot gets zeros when accumulate == 0.
@@ -1276,14 +1399,14 @@ namespace llamql
             const int e = ids[pair];
             if (e < 0 || e >= n_experts || !experts[e].d_down)
                 continue;
-            const float v = weights[pair] * pair_out[(size_t)pair * hidden + h];
+            const float v = weighted(weights[pair], pair_out[(size_t)pair * hidden + h]);
             if (first)
             {
                 y = v;
                 first = false;
             }
             else
-                y = y + v;
+                y = add_rounded(y, v);
         }
         *dst = y;
     }
@@ -1958,9 +2081,47 @@ namespace llamql
 {
     namespace
     {
-        template <class F>
-        bool moe_grouped_launch(const char *fn, bool down, const MoEArgs &m, void *ws, int P, dim3 grid, hipStream_t st)
+        template <class Q, bool DOWN>
+        void moe_grouped_quad_launch_m(bool four, dim3 grid, size_t lds, hipStream_t st, const MoEArgs &m, void *ws, int P)
         {
+            if (four)
+                hipLaunchKernelGGL((moe_grouped_quad_kernel<Q, 4, DOWN>), grid, dim3(MOE_QUAD_WAVES * WAVE), lds, st, m, ws, P);
+            else
+                hipLaunchKernelGGL((moe_grouped_quad_kernel<Q, 2, DOWN>), grid, dim3(MOE_QUAD_WAVES * WAVE), lds, st, m, ws, P);
+        }
+
+        template <class F>
+        bool moe_grouped_launch(const char *fn, bool down, const MoEArgs &m_in, void *ws, int P, dim3 grid, int device_id,
+                                hipStream_t st)
+        {
+            const MoEArgs &m = m_in;
+            {
+                // expert rows of 2, 4, 8 or 16 super-blocks: the quad-lane decoder, every step decoded once per chunk
+                const int rows = down ? m.hidden : m.inter, nsbq = (down ? m.inter : m.hidden) / 256;
+                if (moe_quad_ok<F>(rows, nsbq))
+                {
+                    typedef typename F::Quad Q;
+                    MoEArgs q = m;
+                    const long steps = ((long)rows * nsbq + QUAD_STEP_SB - 1) / QUAD_STEP_SB;
+                    // about the chunks there are: two pairs a chunk below 512 pairs, four from there on
+                    const long chunks = (P + moe_chunk_size(P) - 1) / moe_chunk_size(P) + (P >= 64 ? P / 8 : P / 2);
+                    const long all_steps = steps * chunks * (down ? 1 : 2);
+                    int spw = 1;
+                    while (spw < 8 && all_steps / ((long)cu_count(device_id) * MOE_QUAD_WAVES * 2) >= 2 * spw)
+                        spw *= 2;
+                    q.rows_per_wave = spw;
+                    q.gshift = moe_log2(nsbq);
+                    const long gx = (steps + (long)MOE_QUAD_WAVES * spw - 1) / ((long)MOE_QUAD_WAVES * spw);
+                    const bool four = moe_chunk_size(P) > 2;
+                    const size_t lds = (size_t)(four ? 4 : 2) * nsbq * QUAD_SB_LDS;
+                    const dim3 qgrid((unsigned)gx, grid.y, down ? 1 : 2);
+                    if (down)
+                        moe_grouped_quad_launch_m<Q, true>(four, qgrid, lds, st, q, ws, P);
+                    else
+                        moe_grouped_quad_launch_m<Q, false>(four, qgrid, lds, st, q, ws, P);
+                    return launched(fn);
+                }
+            }
             const int nsb = (down ? m.inter : m.hidden) / 256;
             const size_t lds = gemv_lds_bytes<F>(4, nsb);
             if (lds + F::TABLE_BYTES > 64 * 1024)
@@ -2016,9 +2177,9 @@ extern "C" bool llam_ql_moe_gate_up_grouped(uint8_t fmt, const llam_ql_expert *d
     hipStream_t st = as_stream(stream);
     switch (fmt)
     {
-    case LLAM_FMT_Q4_K: return moe_grouped_launch<Q4KTraits>(fn, false, m, ws, (int)P, grid, st);
-    case LLAM_FMT_Q6_K: return moe_grouped_launch<Q6KTraits>(fn, false, m, ws, (int)P, grid, st);
-    default: return moe_grouped_launch<IQ3STraits>(fn, false, m, ws, (int)P, grid, st);
+    case LLAM_FMT_Q4_K: return moe_grouped_launch<Q4KTraits>(fn, false, m, ws, (int)P, grid, device_id, st);
+    case LLAM_FMT_Q6_K: return moe_grouped_launch<Q6KTraits>(fn, false, m, ws, (int)P, grid, device_id, st);
+    default: return moe_grouped_launch<IQ3STraits>(fn, false, m, ws, (int)P, grid, device_id, st);
     }
 }
 
@@ -2059,9 +2220,9 @@ extern "C" bool llam_ql_moe_down_grouped(uint8_t fmt, const llam_ql_expert *d_ex
     bool ok;
     switch (fmt)
     {
-    case LLAM_FMT_Q4_K: ok = moe_grouped_launch<Q4KTraits>(fn, true, m, ws, (int)P, grid, st); break;
-    case LLAM_FMT_Q6_K: ok = moe_grouped_launch<Q6KTraits>(fn, true, m, ws, (int)P, grid, st); break;
-    default: ok = moe_grouped_launch<IQ3STraits>(fn, true, m, ws, (int)P, grid, st); break;
+    case LLAM_FMT_Q4_K: ok = moe_grouped_launch<Q4KTraits>(fn, true, m, ws, (int)P, grid, device_id, st); break;
+    case LLAM_FMT_Q6_K: ok = moe_grouped_launch<Q6KTraits>(fn, true, m, ws, (int)P, grid, device_id, st); break;
+    default: ok = moe_grouped_launch<IQ3STraits>(fn, true, m, ws, (int)P, grid, device_id, st); break;
     }
     if (!ok)
         return false;

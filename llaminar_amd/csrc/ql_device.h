@@ -247,6 +247,22 @@ namespace llamql
         return v;
     }
 
+    // weight * v, and that added to y, each rounded on its own: never contracted into a fused multiply-add, so
+    // that every kernel that weighs and adds partial results (expert slots, accumulating launches) forms
+    // the same bits whatever the compiler makes of the code around it.
+    // (contraction is switched off for these two operations themselves: __fmul_rn / __fadd_rn are plain
+    // operators to this compiler and fuse like any others)
+    __device__ __forceinline__ float weighted(float weight, float v)
+    {
+#pragma clang fp contract(off)
+        return weight * v;
+    }
+    __device__ __forceinline__ float add_rounded(float y, float v)
+    {
+#pragma clang fp contract(off)
+        return y + v;
+    }
+
     // ---- integer dot ------------------------------------------------------------
 
     // acc + sum of four signed-byte products (v_dot4_i32_i8).

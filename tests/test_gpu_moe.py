@@ -279,15 +279,12 @@ def test_group_tokens_by_expert(capi, dev):
 def test_grouped_launches_equal_ungrouped(capi, dev, fmt):
     """Tokens grouped by expert: every gate/up row and every token output carries the bits of
     the ungrouped launches (12 tokens on 5 experts + an always-on slot: segments of 1..12 tokens,
-    an expert missing from the table, an id out of range).  On rows of 2, 4, 8 or 16 super-blocks (as here) the
-    per-slot launches run the quad-lane decoders, which add a row's blocks in another order than the grouped
-    launches' kernel: equal to 1e-5 of the largest value there, and exactly equal where nothing is written."""
+    an expert missing from the table, an id out of range).  Rows of 4 and 2 super-blocks: both paths run the
+    quad-lane decoders, the grouped one decoding each step once per chunk of an expert's tokens."""
     import torch
 
     def same(a, b):
-        untouched = (b == 3.0) | torch.isnan(b)
-        return bool((a[untouched] == b[untouched]).all() | torch.isnan(a[untouched]).all()) and \
-            float((a[~untouched] - b[~untouched]).abs().max()) <= 1e-5 * float(b[~untouched].abs().max())
+        return torch.equal(a, b)
 
     n_exp, hidden, inter, k, T = 6, 1024, 512, 3, 12
     host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 60)
