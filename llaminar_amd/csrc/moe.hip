@@ -488,7 +488,7 @@ namespace llamql
     // staged while the weights travel.  The wavefronts leave their rows' dot products in LDS; after
     // one barrier a lane per row adds the live slots in ascending order with their routing weights
     // -- the arithmetic and order of moe_down_quad_kernel, the same bits.
-    // grid: (workgroups per matrix, n_tokens), max(top_k, MOE_SLOTWAVE_MIN_WAVES) wavefronts;
+    // grid: (workgroups per matrix, n_tokens), top_k wavefronts (more where the decode tables need a thread a piece);
     // m.rows_per_wave: steps per wavefront (1..MOE_SLOTWAVE_MAX_STEPS), m.gshift: log2(nsb).
     constexpr int MOE_SLOTWAVE_MAX_STEPS = 4;
     template <class Q>
