@@ -245,7 +245,10 @@ bool llam_ql_gemv_describe(uint8_t fmt, int M, int N, int K, int has_plane, int 
  * int32 accumulation per 32-column block and fp32 rescale.  Replaces
  * gemm_native_vnni_preq (CPUNativeVNNIGemv.h:2046-2287); device-side
  * counterpart of launch_native_vnni_gemm
- * (src/v2/kernels/rocm/gemm/ROCmQuantisedGemmKernel_native_VNNI.hip:2580-2632). */
+ * (src/v2/kernels/rocm/gemm/ROCmQuantisedGemmKernel_native_VNNI.hip:2580-2632).
+ * Token tiles of 32 (M <= 32), 64 (M <= 64) or 128 tokens: the fp32 sum of a row's blocks
+ * is formed in an order that depends on the tile, so a row's last bits may differ between
+ * calls of different M (the per-block int32 sums never do). */
 bool llam_ql_gemm(uint8_t fmt, const void *d_w, const void *d_q8, float *d_y,
                   int M, int N, int K, int ldy, int device_id, void *stream);
 

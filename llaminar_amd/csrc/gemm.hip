@@ -36,12 +36,12 @@ namespace llamql
     typedef float v32f __attribute__((ext_vector_type(32)));
 
     constexpr int GEMM_BM = 128;        // tokens per workgroup
+    // (launches of up to 32 and up to 64 tokens run tiles of 32 and 64 tokens: gemm_kernel's BM)
     constexpr int GEMM_BN = 64;         // weight rows per workgroup
     constexpr int GEMM_THREADS = 512;
     constexpr int GEMM_STRIDE = 256 + 16; // bytes per LDS row (one super-block + pad)
     // per-block scale tables [8][rows + 8]: the pad spreads the four threads that write one
     // row's scales of different blocks over different banks
-    constexpr int GEMM_SM = GEMM_BM + 8;
     constexpr int GEMM_SN = GEMM_BN + 8;
 
     struct GemmArgs
@@ -57,10 +57,10 @@ namespace llamql
         int tile0; // first 64-row tile of the launch (0 unless DUMP)
     };
 
-    template <class F>
+    template <class F, int BM>
     constexpr size_t gemm_lds_bytes()
     {
-        return (size_t)(GEMM_BM + GEMM_BN) * GEMM_STRIDE + (size_t)2 * 8 * (GEMM_SM + GEMM_SN) * sizeof(float);
+        return (size_t)(BM + GEMM_BN) * GEMM_STRIDE + (size_t)2 * 8 * (BM + 8 + GEMM_SN) * sizeof(float);
     }
 
     // Two adjacent Q8_1 blocks (72 bytes, 4-byte aligned) of one token, fetched with loads
@@ -181,13 +181,26 @@ namespace llamql
 
     // DUMP: also store the matrix unit's results, the exact int32 block sums (the parity hook of
     // the C-ABI), for a window of weight rows; otherwise the same code.
-    template <class F, bool DUMP = false>
-    __global__ void __launch_bounds__(GEMM_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
+    // BM = 128: wavefront w owns one 32x32 tile (tokens 32 (w / 2).., weight rows 32 (w % 2)..) and all eight
+    // blocks of a K step.  BM = 64 and 32 (few tokens): the workgroup has four or two tiles only, so two or
+    // four wavefronts share a tile and take four or two of a step's eight blocks each -- the rescale work per
+    // wavefront falls with the tokens -- and their partial accumulators are added in wavefront order at the
+    // end.
+    template <class F, bool DUMP = false, int BM = GEMM_BM>
+    // (the block-sum variant of the small tile also carries the addresses of the sums: it may take the
+    // registers of three wavefronts per SIMD unit; it is the parity hook, not a timed path)
+    __global__ void __launch_bounds__(GEMM_THREADS)
+        __attribute__((amdgpu_waves_per_eu(DUMP && BM != GEMM_BM ? 3 : 4, 4)))
         gemm_kernel(const GemmArgs g)
     {
+        static_assert(BM == 128 || BM == 64 || BM == 32, "tiles of 128, 64 or 32 tokens");
+        constexpr int GEMM_SM = BM + 8; // per-block scale table [8][tokens + 8]
+        constexpr int MTILES = BM / 32;             // 32-token tiles of the workgroup
+        constexpr int KPARTS = 4 / MTILES;          // wavefronts that share a tile's K step
+        constexpr int KB_PER = 8 / KPARTS;          // blocks of a K step per wavefront
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         uint8_t *Al = smem;                             // [BM][STRIDE] activations int8
-        uint8_t *Wl = Al + GEMM_BM * GEMM_STRIDE;       // [BN][STRIDE] weights int8
+        uint8_t *Wl = Al + BM * GEMM_STRIDE;            // [BN][STRIDE] weights int8
         float *ad = reinterpret_cast<float *>(Wl + GEMM_BN * GEMM_STRIDE); // [8][SM] a_d
         float *asd = ad + 8 * GEMM_SM;                  // [8][SM]
         float *bs = asd + 8 * GEMM_SM;                  // [8][SN]
@@ -199,18 +212,22 @@ namespace llamql
 
         const int tid = threadIdx.x;
         const int lane = tid & 63;
-        const int wave = tid >> 6;
+        // (small tiles: in a scalar register, like all it leads to -- they have no vector register to spare)
+        const int wave = BM == GEMM_BM ? tid >> 6 : __builtin_amdgcn_readfirstlane(tid >> 6);
         const int ntile = wave & 1;
-        const int mtile = wave >> 1;
+        const int mtile = KPARTS == 1 ? wave >> 1 : (wave >> 1) % MTILES;
+        const int kpart = KPARTS == 1 ? 0 : (wave >> 1) / MTILES; // this wavefront's blocks of a step: kpart * KB_PER ..
         const int l32 = lane & 31;
         const int lh = lane >> 5;
 
         const long n0 = ((long)blockIdx.x + g.tile0) * GEMM_BN;
-        const long m0 = (long)blockIdx.y * GEMM_BM;
+        const long m0 = (long)blockIdx.y * BM;
         const int KB = g.w.SB * 8;
 
-        // activations: thread = (token, pair of adjacent Q8_1 blocks) -> 72 contiguous bytes
-        const int am = tid >> 2;
+        // activations: thread = (token, pair of adjacent Q8_1 blocks) -> 72 contiguous bytes; the first
+        // 4 BM threads (whole wavefronts) have a token, the others load and store nothing
+        const bool a_thread = BM * 4 >= GEMM_THREADS || __builtin_amdgcn_readfirstlane(tid) < BM * 4; // per wavefront
+        const int am = (tid >> 2) & (BM - 1);
         const int ap = tid & 3;
         long am_src = m0 + am;
         if (am_src >= g.M)
@@ -223,7 +240,8 @@ namespace llamql
 
         auto issue = [&](int sb) {
             pf.issue(g, sb);
-            areg.load(asrc + (size_t)sb * 72);
+            if (a_thread)
+                areg.load(asrc + (size_t)sb * 72);
         };
 
         // One K step's staging: registers -> LDS (weights as int8 [row][k] + scales, activations
@@ -234,6 +252,7 @@ namespace llamql
             __syncthreads(); // previous step's LDS reads (and the table staging) are done
             pf.store(Wl, bs, bm, tab);
             areg.wait();
+            if (a_thread)
             {
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
@@ -305,13 +324,15 @@ namespace llamql
             };
             v32f cs;
             v16f cs1;
+            const int kb0 = kpart * KB_PER; // (KB_PER is even: the pairs of the scale and min-term products stay whole)
             if constexpr (F::GEMM_PAIR_SCALES)
-                cs = scales(0);
+                cs = scales(kb0);
             else
-                cs1 = scales1(0);
+                cs1 = scales1(kb0);
 #pragma unroll
-            for (int kb = 0; kb < 8; ++kb)
+            for (int kk8 = 0; kk8 < KB_PER; ++kk8)
             {
+                const int kb = kb0 + kk8;
                 // (one set of result registers: with the scale products held as well, a second
                 // set would not fit the 128 registers that four wavefronts per SIMD unit leave;
                 // the other wavefronts cover the product's latency)
@@ -333,20 +354,20 @@ namespace llamql
                 }
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    acc[r] = fmaf((float)d[r], F::GEMM_PAIR_SCALES ? cs[16 * (kb & 1) + r] : cs1[r], acc[r]);
+                    acc[r] = fmaf((float)d[r], F::GEMM_PAIR_SCALES ? cs[16 * (kk8 & 1) + r] : cs1[r], acc[r]);
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (F::GEMM_PAIR_SCALES)
                 {
-                    if ((kb & 1) && kb + 1 < 8)
+                    if ((kk8 & 1) && kk8 + 1 < KB_PER)
                         cs = scales(kb + 1); // the other wavefronts of the unit cover its latency
                 }
                 else
                 {
-                    if (kb + 1 < 8)
+                    if (kk8 + 1 < KB_PER)
                         cs1 = scales1(kb + 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (F::HAS_MIN && (kb & 1))
+                if (F::HAS_MIN && (kk8 & 1))
                 {
                     // rank-2 update over blocks kb-1, kb, straight into the accumulator: lane
                     // half lh supplies block kb-1+lh
@@ -359,6 +380,24 @@ namespace llamql
         }
         pf.finish();
         areg.wait();
+
+        if constexpr (KPARTS > 1 && !DUMP)
+        {
+            // the tile's wavefronts add their partial accumulators in wavefront order (kpart 0 + 1 + ..)
+            __syncthreads(); // every wavefront is done with the step's LDS
+            float *red = reinterpret_cast<float *>(smem); // [wavefront][16][64]
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                red[(wave * 16 + r) * 64 + lane] = acc[r];
+            __syncthreads();
+            if (kpart != 0)
+                return;
+#pragma unroll
+            for (int p = 1; p < KPARTS; ++p)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[r] += red[((wave + 2 * MTILES * p) * 16 + r) * 64 + lane];
+        }
 
         // ---- store: lane holds weight row n, 16 tokens -------------------------------------
         const long n = n0 + ntile * 32 + l32;
@@ -391,6 +430,20 @@ namespace llamql
         *dst = v;
     }
 
+    template <class F, bool DUMP, int BM>
+    bool gemm_launch_bm(const char *fn, const GemmArgs &g, int tiles_n, int M, hipStream_t st)
+    {
+        constexpr size_t lds = gemm_lds_bytes<F, BM>();
+        static_assert(lds >= (size_t)8 * 16 * 64 * sizeof(float), "room for the partial accumulators");
+        static LdsGrant grant;
+        const hipError_t e = allow_lds(grant, reinterpret_cast<const void *>(&gemm_kernel<F, DUMP, BM>), lds);
+        if (e != hipSuccess)
+            return fail(fn, "cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        const dim3 grid((unsigned)tiles_n, (unsigned)((M + BM - 1) / BM));
+        hipLaunchKernelGGL((gemm_kernel<F, DUMP, BM>), grid, dim3(GEMM_THREADS), lds, st, g);
+        return launched(fn);
+    }
+
     // d_sums: the block-sum variant over weight rows [row0, row0+nrows); only the workgroups
     // whose 64-row tile meets the window are launched.
     template <class F, bool DUMP = false>
@@ -411,14 +464,12 @@ namespace llamql
         g.nrows = nrows;
         g.tile0 = DUMP ? row0 / GEMM_BN : 0;
         const int tile_end = DUMP ? (row0 + nrows + GEMM_BN - 1) / GEMM_BN : (N + GEMM_BN - 1) / GEMM_BN;
-        constexpr size_t lds = gemm_lds_bytes<F>();
-        static LdsGrant grant;
-        const hipError_t e = allow_lds(grant, reinterpret_cast<const void *>(&gemm_kernel<F, DUMP>), lds);
-        if (e != hipSuccess)
-            return fail(fn, "cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-        const dim3 grid((unsigned)(tile_end - g.tile0), (unsigned)((M + GEMM_BM - 1) / GEMM_BM));
-        hipLaunchKernelGGL((gemm_kernel<F, DUMP>), grid, dim3(GEMM_THREADS), lds, st, g);
-        return launched(fn);
+        // few tokens: one smaller tile of tokens (a 128-token tile would rescale 128 rows for them)
+        if (M <= 32)
+            return gemm_launch_bm<F, DUMP, 32>(fn, g, tile_end - g.tile0, M, st);
+        if (M <= 64)
+            return gemm_launch_bm<F, DUMP, 64>(fn, g, tile_end - g.tile0, M, st);
+        return gemm_launch_bm<F, DUMP, GEMM_BM>(fn, g, tile_end - g.tile0, M, st);
     }
 } // namespace llamql
 

@@ -27,7 +27,10 @@ def test_golden_fixture(capi, dev, golden, fmt):
 
 
 @pytest.mark.parametrize("fmt", list(FMTS.values()), ids=list(FMTS))
-@pytest.mark.parametrize("M,N,K", [(1, 128, 256), (17, 100, 512), (128, 128, 1024), (130, 257, 768), (300, 64, 2048)])
+@pytest.mark.parametrize("M,N,K", [(1, 128, 256), (17, 100, 512), (128, 128, 1024), (130, 257, 768), (300, 64, 2048),
+                                   # launches of few tokens run tiles of 32 tokens: one, two (the second
+                                   # holds one token) and three rows of tiles, then the first 128-token launch
+                                   (32, 200, 1024), (33, 130, 5120), (96, 64, 2048), (97, 64, 2048)])
 def test_random_shapes(capi, dev, oracle, fmt, M, N, K):
     W = synth.weights_numpy(fmt, N, K, 7 + M + N)
     q8 = oracle.quantize(synth.activations_numpy(M, K, 9 + K))
@@ -56,11 +59,12 @@ def test_gemm_rows_equal_gemv(capi, dev, oracle, fmt):
 
 @pytest.mark.parametrize("fmt", list(FMTS.values()), ids=list(FMTS))
 @pytest.mark.parametrize("M,N,K,r0,nr", [(1, 128, 256, 0, 128), (17, 100, 512, 37, 63), (130, 257, 768, 190, 67),
-                                         (300, 200, 2048, 60, 70)])
+                                         (300, 200, 2048, 60, 70), (40, 130, 1280, 60, 70), (96, 70, 512, 0, 70)])
 def test_block_sums_of_the_gemm_kernel(capi, dev, oracle, fmt, M, N, K, r0, nr):
     """The matrix unit's per-block results of llam_ql_gemm's own kernel (block-sum variant) are
     the reference's int32 sums bit for bit: ragged tiles, windows that start and end inside a
-    64-row tile, token tails."""
+    64-row tile, token tails, and the 32-token tiles that launches of up to 96 tokens run (there four
+    wavefronts share a tile's blocks of a step)."""
     W = synth.weights_numpy(fmt, N, K, 70 + M + N)
     q8 = oracle.quantize(synth.activations_numpy(M, K, 90 + K))
     wd = upload_weights(capi, dev, fmt, W)
