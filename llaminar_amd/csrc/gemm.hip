@@ -106,9 +106,11 @@ namespace llamql
         int row, l;
         bool active; // wavefront-uniform: BN rows x 4 quad lanes = the first 4*BN threads
 
-        __device__ __forceinline__ void init(const GemmArgs &g, long n0, int tid)
+        // first: the first of the 4 BN decoding threads (a multiple of 4 BN)
+        __device__ __forceinline__ void init(const GemmArgs &g, long n0, int tid, int first)
         {
-            active = __builtin_amdgcn_readfirstlane(tid) < GEMM_BN * 4;
+            const int t0 = __builtin_amdgcn_readfirstlane(tid);
+            active = t0 >= first && t0 < first + GEMM_BN * 4;
             row = (tid >> 2) & (GEMM_BN - 1);
             l = tid & 3;
             lc = Q::lane_consts(l);
@@ -121,6 +123,7 @@ namespace llamql
         {
             // the other wavefronts load the same bytes again (cache hits) and drop them: a
             // load under a condition would need a register copy that waits for it at once
+            // (asking for the rows of a later step instead, to warm the L2 cache, changed nothing)
             Q::load_at(raw, wc, lc, sb);
         }
         __device__ __forceinline__ void store(uint8_t *Wl, float *bs, float *bm, const void *)
@@ -154,7 +157,7 @@ namespace llamql
         long n;
         int row, c;
 
-        __device__ __forceinline__ void init(const GemmArgs &g, long n0, int tid)
+        __device__ __forceinline__ void init(const GemmArgs &g, long n0, int tid, int)
         {
             row = tid >> 3;
             c = tid & 7;
@@ -236,7 +239,9 @@ namespace llamql
         GemmActRaw areg;
 
         GemmPrefetch<F> pf;
-        pf.init(g, n0, tid);
+        // small tiles: the wavefronts that stage no activations decode the weights (the second half of
+        // the workgroup), so that the two kinds of staging run side by side
+        pf.init(g, n0, tid, BM == GEMM_BM ? 0 : GEMM_THREADS - GEMM_BN * 4);
 
         auto issue = [&](int sb) {
             pf.issue(g, sb);
