@@ -181,6 +181,26 @@ bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const void *d_plane, 
                              const float *d_up, int ld_gu, float *d_y, int M, int N, int K,
                              int ldy, void *d_q8_scratch, int device_id, void *stream);
 
+/* The feed-forward block's first half in one launch, batches of 5..8 rows:
+ *   d_q8_out = Q8_1( silu(W_gate a) * (W_up a) )   [M x N/32 blocks], the down projection's input.
+ * Both projections run on the matrix unit with their 32-row tiles paired inside a workgroup, which then
+ * holds both operands of 32 consecutive columns and quantises the block itself: no launch for the
+ * second projection, none for llam_ql_swiglu_quantize, no fp32 round trip.  d_y_gate / d_y_up (row
+ * stride ldy) receive the fp32 projections when not NULL; d_q8_out is bit for bit
+ * llam_ql_swiglu_quantize of those.  The projections are those of the matrix-unit kernel (the
+ * reference's ascending block order within a wavefront's share of the row, llam_ql_gemv's contract for
+ * batches of 5..8); their last bits may differ from two llam_ql_gemv calls, which split a row into
+ * other shares.  Served (llam_ql_gemv_gate_up_swiglu_supported) for Q4_K, M = 5..8, N a multiple of 32
+ * and at least 4096, rows of 8..64 super-blocks; d_plane_gate / d_plane_up: both matrices' batch planes
+ * or both NULL.  Replaces multiply_fused_tensor over {gate, up} + compute_swiglu + the quantiser of
+ * the down projection (CPUNativeVNNIGemmKernel.h:572, :325-431; the decode flow of
+ * MoEExpertComputeStage.cpp:1450-1708 for a dense block). */
+bool llam_ql_gemv_gate_up_swiglu_supported(uint8_t fmt, int M, int N, int K);
+bool llam_ql_gemv_gate_up_swiglu(uint8_t fmt, const void *d_w_gate, const void *d_plane_gate,
+                                 const void *d_w_up, const void *d_plane_up, const void *d_q8,
+                                 float *d_y_gate, float *d_y_up, int ldy, void *d_q8_out, int M, int N,
+                                 int K, int device_id, void *stream);
+
 /* Parity hook: the exact per-block int32 sums the GEMV forms, for rows
  * [row0, row0+nrows): d_sums[(m*nrows + r)*(K/32) + kb].  The call makes the choices
  * llam_ql_gemv makes for (fmt, M, N, K) -- quad-lane, matrix-unit, chunked or generic

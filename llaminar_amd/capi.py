@@ -91,6 +91,9 @@ SIGNATURES = {
     "llam_ql_moe_route_gate_up_swiglu": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p,
                                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                   c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv_gate_up_swiglu_supported": (c_bool, [c_uint8, c_int, c_int, c_int]),
+    "llam_ql_gemv_gate_up_swiglu": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                             c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_ql_swiglu_quantize": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "llam_ql_moe_down": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                   c_int, c_int, c_int, c_int, c_void_p]),
@@ -482,6 +485,26 @@ def moe_route_gate_up_swiglu(fmt: int, table, n_experts: int, logits, top_k: int
                                                    _ptr(q8_hidden), _ptr(g), _ptr(u), _ptr(q8_out), T, hidden, inter,
                                                    _dev(x), _stream(stream)), "moe_route_gate_up_swiglu")
     return q8_out
+
+
+def gemv_gate_up_swiglu_supported(fmt: int, M: int, N: int, K: int) -> bool:
+    return bool(load().llam_ql_gemv_gate_up_swiglu_supported(fmt, M, N, K))
+
+
+def gemv_gate_up_swiglu(fmt: int, w_gate, w_up, q8, M: int, N: int, K: int, plane_gate=None, plane_up=None,
+                        want_projections: bool = False, q8_out=None, stream=None):
+    """Q8_1 blocks [M x N/32] of silu(W_gate a) * (W_up a) in one launch (batches of 5..8); with
+    want_projections also the fp32 projections the blocks were formed from."""
+    import torch
+
+    if q8_out is None:
+        q8_out = torch.empty(M * (N // 32) * 36, dtype=torch.uint8, device=w_gate.device)
+    yg = torch.empty(M, N, dtype=torch.float32, device=w_gate.device) if want_projections else None
+    yu = torch.empty(M, N, dtype=torch.float32, device=w_gate.device) if want_projections else None
+    _check(load().llam_ql_gemv_gate_up_swiglu(fmt, _ptr(w_gate), _ptr(plane_gate), _ptr(w_up), _ptr(plane_up), _ptr(q8),
+                                              _ptr(yg), _ptr(yu), N, _ptr(q8_out), M, N, K, _dev(w_gate),
+                                              _stream(stream)), "gemv_gate_up_swiglu")
+    return (q8_out, yg, yu) if want_projections else q8_out
 
 
 def swiglu_quantize(gate, up, want_act: bool = False, stream=None):

@@ -278,6 +278,38 @@ namespace llamql
     }
 } // namespace llamql
 
+extern "C" bool llam_ql_gemv_gate_up_swiglu_supported(uint8_t fmt, int M, int N, int K)
+{
+    return fmt == LLAM_FMT_Q4_K && M >= 1 && M <= LLAM_QL_MAX_GEMV_M && N >= 1 && K >= 1 &&
+           llamql::gemv_mfma_q4k_swiglu_ok(M, N, K);
+}
+
+extern "C" bool llam_ql_gemv_gate_up_swiglu(uint8_t fmt, const void *d_w_gate, const void *d_plane_gate,
+                                            const void *d_w_up, const void *d_plane_up, const void *d_q8,
+                                            float *d_y_gate, float *d_y_up, int ldy, void *d_q8_out, int M, int N,
+                                            int K, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_gate_up_swiglu";
+    if (!llam_ql_gemv_gate_up_swiglu_supported(fmt, M, N, K))
+        return fail(fn, "not served for format %d, M=%d, N=%d, K=%d (llam_ql_gemv_gate_up_swiglu_supported)", (int)fmt, M,
+                    N, K);
+    if (!d_w_gate || !d_w_up || !d_q8 || !d_q8_out)
+        return fail(fn, "null pointer");
+    if (!aligned16(d_w_gate) || !aligned16(d_w_up) || !aligned4(d_q8) || !aligned4(d_q8_out))
+        return fail(fn, "the matrices must be 16-byte, the Q8_1 buffers 4-byte aligned");
+    if ((d_plane_gate == nullptr) != (d_plane_up == nullptr))
+        return fail(fn, "batch planes for both matrices or for neither");
+    if (d_plane_gate && (!aligned16(d_plane_gate) || !aligned16(d_plane_up) || llam_ql_batch_plane_bytes(fmt, N, K) == 0))
+        return fail(fn, "the planes must be 16-byte aligned and of a shape that has one (llam_ql_batch_plane_bytes)");
+    if ((d_y_gate || d_y_up) && ldy < N)
+        return fail(fn, "ldy=%d smaller than N=%d", ldy, N);
+    if (!set_device(fn, device_id))
+        return false;
+    return gemv_mfma_q4k_swiglu_launch(fn, d_w_gate, d_plane_gate, d_w_up, d_plane_up, d_q8, d_y_gate, d_y_up, ldy,
+                                       d_q8_out, M, N, K, device_id, as_stream(stream));
+}
+
 extern "C" size_t llam_ql_batch_plane_bytes(uint8_t fmt, int N, int K)
 {
     return llamql::batch_plane_shape(fmt, N, K) ? llamql::batch_plane_size(fmt, N, K) : 0;

@@ -489,7 +489,7 @@ namespace llamql
         const int SB = K / 256;
         const Mfma6Shape sh = gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA4_LONG_DUMP_COMPUTE : MFMA4_LONG_COMPUTE,
                                                d_plane != nullptr, MFMA_BOUNCE);
-        MfmaLongArgs a;
+        MfmaLongArgs a{};
         a.w = static_cast<const uint8_t *>(d_w);
         a.plane = static_cast<const uint8_t *>(d_plane);
         a.q8 = static_cast<const uint32_t *>(src.q8);
@@ -549,7 +549,7 @@ namespace llamql
         if (mfma4_long_rows(SB))
             return gemv_mfma_q4k_long_launch(fn, d_w, d_plane, src, d_y, M, N, K, ldy, device_id, st, d_sums, row0, nrows);
         const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id), d_sums ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES);
-        MfmaArgs a;
+        MfmaArgs a{};
         a.w = static_cast<const uint8_t *>(d_w);
         a.plane = static_cast<const uint8_t *>(d_plane);
         a.q8 = static_cast<const uint32_t *>(src.q8);
@@ -593,6 +593,56 @@ namespace llamql
         case ACT_SRC_F32: gemv_mfma_q4k_launch_src<QUAD_SRC_F32>(grid, block, lds, st, a); break;
         case ACT_SRC_SWIGLU: gemv_mfma_q4k_launch_src<QUAD_SRC_SWIGLU>(grid, block, lds, st, a); break;
         default: gemv_mfma_q4k_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a); break;
+        }
+        return launched(fn);
+    }
+
+    // Gate and up projection with SwiGLU and the Q8_1 quantiser of the result in one launch
+    // (gemv_mfma_q4k_kernel<.., SWIGLU>): Q4_K, batches of 5..8, rows the unchunked matrix-unit kernel
+    // walks, N a multiple of 32; both matrices with a batch plane or neither.
+    inline bool gemv_mfma_q4k_swiglu_ok(int M, int N, int K)
+    {
+        return K % 256 == 0 && mfma_eligible<Q4KTraits>(M, N, K) && !mfma4_long_rows(K / 256) && N % MFMA_TILE_ROWS == 0;
+    }
+    inline bool gemv_mfma_q4k_swiglu_launch(const char *fn, const void *d_w_gate, const void *d_plane_gate,
+                                            const void *d_w_up, const void *d_plane_up, const void *d_q8,
+                                            float *d_y_gate, float *d_y_up, int ldy, void *d_q8_out, int M, int N,
+                                            int K, int device_id, hipStream_t st)
+    {
+        const int SB = K / 256;
+        const MfmaShape sh = gemv_mfma_swiglu_shape(N, SB, cu_count(device_id));
+        MfmaArgs a{};
+        a.w = static_cast<const uint8_t *>(d_w_gate);
+        a.plane = static_cast<const uint8_t *>(d_plane_gate);
+        a.w2 = static_cast<const uint8_t *>(d_w_up);
+        a.plane2 = static_cast<const uint8_t *>(d_plane_up);
+        a.q8 = static_cast<const uint32_t *>(d_q8);
+        a.y = d_y_gate;
+        a.y2 = d_y_up;
+        a.ldy = ldy;
+        a.q8_out = static_cast<uint32_t *>(d_q8_out);
+        a.N = N;
+        a.SB = SB;
+        a.M = M;
+        a.slices = sh.slices;
+        a.tile_rows = MFMA_TILE_ROWS;
+        const int waves = sh.slices * sh.tiles_per_wg;
+        if (waves > MFMA_MAX_WAVES)
+            return fail(fn, "launch shape of %d wavefronts (N=%d K=%d)", waves, N, K);
+        const dim3 grid((unsigned)sh.grid), block((unsigned)waves * WAVE);
+        const size_t lds = mfma_swiglu_lds_bytes(SB, waves, sh.tiles_per_wg, a.plane != nullptr);
+        if (lds > QUAD_MAX_LDS)
+            return fail(fn, "%zu bytes of LDS (N=%d K=%d)", lds, N, K);
+        static LdsGrant grant_plane, grant_plain;
+        if (a.plane)
+        {
+            (void)allow_lds(grant_plane, reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<QUAD_SRC_Q8, false, true, true>), QUAD_MAX_LDS);
+            hipLaunchKernelGGL((gemv_mfma_q4k_kernel<QUAD_SRC_Q8, false, true, true>), grid, block, lds, st, a);
+        }
+        else
+        {
+            (void)allow_lds(grant_plain, reinterpret_cast<const void *>(&gemv_mfma_q4k_kernel<QUAD_SRC_Q8, false, false, true>), QUAD_MAX_LDS);
+            hipLaunchKernelGGL((gemv_mfma_q4k_kernel<QUAD_SRC_Q8, false, false, true>), grid, block, lds, st, a);
         }
         return launched(fn);
     }

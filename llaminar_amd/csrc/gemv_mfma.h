@@ -58,6 +58,13 @@ namespace llamql
         // sums[(m * nrows + row - row0) * (SB * 8) + block]
         int32_t *sums;
         int row0, nrows;
+        // SWIGLU kernels only (gate and up projection in one launch): the second matrix (w, plane are the
+        // gate matrix) and its optional fp32 output (y: the gate's, may be null too), and the Q8_1 blocks of
+        // silu(gate) * up, [M][N/32] blocks of 9 dwords
+        const uint8_t *w2;
+        const uint8_t *plane2;
+        float *y2;
+        uint32_t *q8_out;
     };
 
     // LDS: per 32-column block 8 activation rows x 32 int8 (16 bytes of padding: neighbouring
@@ -254,10 +261,18 @@ namespace llamql
     // regrouped so that lane (row, h) finds its operands at one address, 128-byte lines shared by
     // four rows): no bounce buffer, a step is computed straight from the registers its loads
     // filled.  Same decode, same products, same order: bit-identical results.
-    template <int SRC, bool DUMP = false, bool PLANE = false>
+    // SWIGLU: the gate and the up projection of a feed-forward block in one launch.  The tiles of a
+    // workgroup come in pairs (rows 32 t .. 32 t + 31 of the gate matrix, the same rows of the up matrix),
+    // so the workgroup holds both operands of silu(gate) * up for 32 consecutive columns of every
+    // activation row: one Q8_1 block of the down projection's input each, quantised here with the
+    // stand-alone quantiser's arithmetic (the bits of the two projections followed by
+    // llam_ql_swiglu_quantize for the same partition of the rows into slices); the fp32 results go to
+    // memory only if asked for.  Tiles are 32 rows, N a multiple of 32.
+    template <int SRC, bool DUMP = false, bool PLANE = false, bool SWIGLU = false>
     __global__ void __launch_bounds__((DUMP ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES) * WAVE)
         gemv_mfma_q4k_kernel(const MfmaArgs a)
     {
+        static_assert(!(SWIGLU && DUMP), "the block-sum variant walks one matrix");
         typedef typename std::conditional<PLANE, MfmaPlaneRaw, MfmaRaw>::type Raw;
         constexpr int LOADS = PLANE ? MFMA_PLANE_LOADS : MFMA_LOADS;
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];
@@ -278,7 +293,13 @@ namespace llamql
         // super-blocks (144 bytes each) is asked for by two wavefronts of the workgroup at the
         // same time and crosses the fabric once
         const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
-        const long tile_row0 = ((long)blockIdx.x * tiles_per_wg + tile_local) * a.tile_rows;
+        // SWIGLU: tile 2 p of the workgroup is the gate half, tile 2 p + 1 the up half of pair p
+        const int mat = SWIGLU ? tile_local & 1 : 0;
+        const long tile_idx = SWIGLU ? (long)blockIdx.x * (tiles_per_wg >> 1) + (tile_local >> 1)
+                                     : (long)blockIdx.x * tiles_per_wg + tile_local;
+        const long tile_row0 = tile_idx * a.tile_rows;
+        const uint8_t *const w_mat = SWIGLU && mat ? a.w2 : a.w;
+        const uint8_t *const plane_mat = SWIGLU && mat ? a.plane2 : a.plane;
         const long row = tile_row0 + l32;
         const bool row_ok = l32 < a.tile_rows && row < a.N;
         const int last_step = nsteps > 0 ? nsteps - 1 : 0;
@@ -300,7 +321,7 @@ namespace llamql
                 r = max_local;
             off[i] = (uint32_t)r * (uint32_t)(nsb * 144) + (uint32_t)(piece * 16);
         }
-        const uint8_t *tile_base = a.w + (size_t)base_row * nsb * 144;
+        const uint8_t *tile_base = w_mat + (size_t)base_row * nsb * 144;
         uint8_t *bounce = mfma_lds + nkb * (MFMA_AQ_STRIDE + 64) + wave * MFMA_BOUNCE;
         uint8_t *bounce_wr = bounce + lane * 16;                     // piece lane + 64 i at + 1024 i
         const uint8_t *bounce_rd = bounce + l32 * 144;               // this lane's weight row
@@ -322,8 +343,8 @@ namespace llamql
         auto issue = [&](Raw &r, int step) {
             const int sb = nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0;
             if constexpr (PLANE)
-                mfma_plane_load(r, uniform(a.plane + (size_t)sb * 512),
-                                uniform(a.plane + q4k_plane_heads_offset(a.N, nsb) + (size_t)sb * 64), poff_w, poff_h);
+                mfma_plane_load(r, uniform(plane_mat + (size_t)sb * 512),
+                                uniform(plane_mat + q4k_plane_heads_offset(a.N, nsb) + (size_t)sb * 64), poff_w, poff_h);
             else
                 mfma_load(r, uniform(tile_base + (size_t)sb * 144), off);
         };
@@ -508,6 +529,8 @@ namespace llamql
         for (int i = 0; i < 4; ++i)
             red[(wave * 4 + i) * WAVE + lane] = acc[i];
         __syncthreads();
+        // SWIGLU: the tiles' sums meet in LDS behind the partial sums, [tile][8 activation rows][32 weight rows]
+        float *res = red + (size_t)(blockDim.x >> 6) * 4 * WAVE;
         if (slice == 0)
         {
 #pragma unroll
@@ -517,10 +540,37 @@ namespace llamql
                 for (int s = 1; s < a.slices; ++s)
                     v += red[((wave + s) * 4 + i) * WAVE + lane];
                 const int m = 4 * lh + i;
-                if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
+                if constexpr (SWIGLU)
+                {
+                    res[(tile_local * 8 + m) * 32 + l32] = v; // (rows past the batch: never read as results)
+                    float *const y_mat = mat ? a.y2 : a.y;
+                    if (y_mat && m < a.M && row_ok)
+                        y_mat[(size_t)m * a.ldy + row] = v;
+                }
+                else if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
                 {
                     if (m < a.M && row_ok)
                         a.y[(size_t)m * a.ldy + row] = v;
+                }
+            }
+        }
+        if constexpr (SWIGLU)
+        {
+            __syncthreads();
+            // the first wavefront of a pair: eight lanes per activation row quantise its block (the lane
+            // mapping of the stand-alone quantiser)
+            if (slice == 0 && mat == 0)
+            {
+                const int m = lane >> 3, sub = lane & 7;
+                const float4 g = reinterpret_cast<const float4 *>(res + (tile_local * 8 + m) * 32)[sub];
+                const float4 u = reinterpret_cast<const float4 *>(res + ((tile_local + 1) * 8 + m) * 32)[sub];
+                const Q8Lane q = q8_1_quantize_lane(swiglu4(g, u));
+                if (m < a.M && tile_row0 < a.N)
+                {
+                    uint32_t *dst = a.q8_out + ((size_t)m * (size_t)(a.N / 32) + (size_t)tile_idx) * 9;
+                    dst[1 + sub] = q.packed;
+                    if (sub == 0)
+                        dst[0] = q.head;
                 }
             }
         }
@@ -580,6 +630,25 @@ namespace llamql
     // the others walk 128 rows each.  A compute unit's time goes with the rows it streams, so the
     // tile height that leaves the busiest compute unit the fewest rows wins; ties go to the
     // taller tile.
+    // Gate and up in one launch: 2 N / 32 full tiles, an even number per workgroup.
+    inline MfmaShape gemv_mfma_swiglu_shape(long N, int nsb, int cus)
+    {
+        MfmaShape sh = gemv_mfma_shape_of(2 * N, nsb, cus, MFMA_MAX_WAVES, MFMA_TILE_ROWS);
+        if (sh.tiles_per_wg < 2)
+            sh.tiles_per_wg = 2; // (slices <= 8: two tiles fit the 16 wavefronts)
+        const long pairs = N / MFMA_TILE_ROWS, per_wg = sh.tiles_per_wg / 2;
+        sh.grid = (pairs + per_wg - 1) / per_wg;
+        return sh;
+    }
+    // LDS bytes of the launch: the activations (and bounce buffers), and at the end the partial sums of
+    // every wavefront with the tiles' sums behind them
+    inline size_t mfma_swiglu_lds_bytes(int nsb, int waves, int tiles, bool plane)
+    {
+        const size_t run = plane ? mfma_act_bytes(nsb) : mfma_lds_bytes(nsb, waves);
+        const size_t end = (size_t)waves * 4 * WAVE * sizeof(float) + (size_t)tiles * 8 * 32 * sizeof(float);
+        return run > end ? run : end;
+    }
+
     inline MfmaShape gemv_mfma_shape(long N, int nsb, int cus, int max_waves = MFMA_MAX_WAVES)
     {
         const int forced = gemv_mfma_tile_rows_override();

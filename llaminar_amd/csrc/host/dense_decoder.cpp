@@ -342,6 +342,20 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
         llam_ql_proj gu[2];
         gu[0] = llam_ql_proj{w.wgate, d->gate, F, F, w.fmt_gate, w.plane_gate};
         gu[1] = llam_ql_proj{w.wup, d->up, F, F, w.fmt_up, w.plane_up};
+        // batches the matrix unit serves: gate, up, SwiGLU and the Q8_1 quantiser of the result in one launch
+        if (w.fmt_gate == w.fmt_up && (w.plane_gate != nullptr) == (w.plane_up != nullptr) &&
+            llam_ql_gemv_gate_up_swiglu_supported(w.fmt_gate, B, F, H))
+        {
+            if (!forward(fn, llam_dec_rmsnorm_q8_1(res, pending, w.ffn_norm, c.rms_eps, nullptr, d->q8_h, B, H, dev, stream)))
+                return false;
+            pending = nullptr;
+            if (!forward(fn, llam_ql_gemv_gate_up_swiglu(w.fmt_gate, w.wgate, w.plane_gate, w.wup, w.plane_up, d->q8_h,
+                                                         nullptr, nullptr, 0, d->q8_act, B, F, H, dev, stream)))
+                return false;
+            if (!project_into_residual(w.fmt_down, w.wdown, w.plane_down, d->q8_act, F))
+                return false;
+            continue;
+        }
         if (!norm_and_project(gu, 2, w.ffn_norm))
             return false;
         if (llam_ql_gemv_accumulate_supported(w.fmt_down, B, H, F, dev))
