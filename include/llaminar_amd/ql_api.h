@@ -191,7 +191,7 @@ bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const void *d_plane, 
  * reference's ascending block order within a wavefront's share of the row, llam_ql_gemv's contract for
  * batches of 5..8); their last bits may differ from two llam_ql_gemv calls, which split a row into
  * other shares.  Served (llam_ql_gemv_gate_up_swiglu_supported) for Q4_K, M = 5..8, N a multiple of 32
- * and at least 4096, rows of 8..64 super-blocks; d_plane_gate / d_plane_up: both matrices' batch planes
+ * and at least 4096, rows of 8..45 super-blocks (K = 2048..11520); d_plane_gate / d_plane_up: both matrices' batch planes
  * or both NULL.  Replaces multiply_fused_tensor over {gate, up} + compute_swiglu + the quantiser of
  * the down projection (CPUNativeVNNIGemmKernel.h:572, :325-431; the decode flow of
  * MoEExpertComputeStage.cpp:1450-1708 for a dense block). */

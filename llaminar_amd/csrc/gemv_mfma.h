@@ -635,7 +635,13 @@ namespace llamql
     {
         MfmaShape sh = gemv_mfma_shape_of(2 * N, nsb, cus, MFMA_MAX_WAVES, MFMA_TILE_ROWS);
         if (sh.tiles_per_wg < 2)
-            sh.tiles_per_wg = 2; // (slices <= 8: two tiles fit the 16 wavefronts)
+        {
+            // a pair needs both tiles in the workgroup: fewer wavefronts per tile where two tiles of the
+            // chosen slices do not fit the LDS (slices <= 8, so 16 wavefronts always suffice)
+            sh.tiles_per_wg = 2;
+            while (sh.slices > 1 && mfma_lds_bytes(nsb, 2 * sh.slices) > QUAD_MAX_LDS)
+                --sh.slices;
+        }
         const long pairs = N / MFMA_TILE_ROWS, per_wg = sh.tiles_per_wg / 2;
         sh.grid = (pairs + per_wg - 1) / per_wg;
         return sh;

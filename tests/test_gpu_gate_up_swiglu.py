@@ -12,8 +12,9 @@ from tests.helpers import TOL, rel_err, sync, upload_q8, upload_weights
 pytestmark = pytest.mark.gpu
 
 # (M, N, K): one pair of tiles per workgroup and several; a count of pairs that leaves the last workgroup
-# partly empty (129 pairs); the shortest rows served (8 super-blocks); rows of 32 super-blocks
-_CASES = [(8, 4096, 2048), (5, 4128, 5120), (7, 8192, 8192), (6, 12800, 5120)]
+# partly empty (129 pairs); the shortest rows served (8 super-blocks); rows of 32 super-blocks;
+# the longest rows served with few tiles (two tiles of eight wavefronts would not fit the LDS: fewer per tile)
+_CASES = [(8, 4096, 2048), (5, 4128, 5120), (7, 8192, 8192), (6, 12800, 5120), (8, 4096, 10240), (5, 4096, 11520)]
 
 
 @pytest.mark.parametrize("with_planes", [False, True], ids=["prepared", "planes"])
@@ -99,6 +100,7 @@ def test_shapes_that_are_not_served(capi, dev):
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 8, 8200, 5120)      # N not a multiple of 32
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 8, 2048, 5120)      # too few rows for the matrix unit
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 8, 5120, 25600)     # rows walked in chunks
+    assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 8, 8192, 11776)     # (from 46 super-blocks on)
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q6_K, 8, 8192, 5120)
     assert not capi.gemv_gate_up_swiglu_supported(FMT_IQ3_S, 8, 8192, 5120)
     w = torch.zeros(8192 * 20 * 144, dtype=torch.uint8, device=dev)
