@@ -302,6 +302,9 @@ def bench_decode(args, torch, capi, synth, dev):
         W = dec.prepared
         P = lambda name: dec.planes.get(name)   # the matrix's batch plane, if the decoder built one
 
+        fused_ffn = (capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, B, F, H) and
+                     (P("0.wgate") is None) == (P("0.wup") is None))
+
         def linear_only():
             for l in range(shape.n_layers):
                 capi.quantize_q8_1(x, out=q8)
@@ -310,6 +313,11 @@ def bench_decode(args, torch, capi, synth, dev):
                                  (FMT_Q6_K, W[f"{l}.wv"], qkv[:, QD + KV:], P(f"{l}.wv"))], q8, B, H)
                 capi.gemv_fused_f32([(FMT_Q4_K, W[f"{l}.wo"], o, P(f"{l}.wo"))], attn, B, QD, q8_scratch=q8)
                 capi.quantize_q8_1(x, out=q8)
+                if fused_ffn:   # as the decoder does at these batches: gate, up, SwiGLU and its quantiser in one launch
+                    capi.gemv_gate_up_swiglu(FMT_Q4_K, W[f"{l}.wgate"], W[f"{l}.wup"], q8, B, F, H,
+                                             plane_gate=P(f"{l}.wgate"), plane_up=P(f"{l}.wup"), q8_out=q8a)
+                    capi.gemv(FMT_Q6_K, W[f"{l}.wdown"], q8a, B, H, F, out=o, plane=P(f"{l}.wdown"))
+                    continue
                 capi.gemv_fused([(FMT_Q4_K, W[f"{l}.wgate"], gate, P(f"{l}.wgate")),
                                  (FMT_Q4_K, W[f"{l}.wup"], up, P(f"{l}.wup"))], q8, B, H)
                 capi.gemv_swiglu_f32(FMT_Q6_K, W[f"{l}.wdown"], gate, up, B, H, F, out=o, q8_scratch=q8a,
@@ -498,6 +506,15 @@ def main():
     down = torch.empty(M, HIDDEN, device=dev)
     lib = capi.load()
 
+    # batches the matrix unit serves: gate, up, SwiGLU and the Q8_1 quantiser of the result as one launch
+    fused_ffn = capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, M, FFN, HIDDEN)
+
+    def ffn_fused(w):
+        capi.quantize_q8_1(x2, out=q8_x2)
+        capi.gemv_gate_up_swiglu(FMT_Q4_K, w["gate"], w["up"], q8_x2, M, FFN, HIDDEN, plane_gate=w["plane_gate"],
+                                 plane_up=w["plane_up"], q8_out=q8_act)
+        capi.gemv(FMT_Q6_K, w["down"], q8_act, M, HIDDEN, FFN, out=down, plane=w["plane_down"])
+
     def step_separate(w):
         # quantiser kernels of their own, Q8_1 blocks through memory
         capi.quantize_q8_1(x, out=q8_x)
@@ -506,6 +523,8 @@ def main():
                          (FMT_Q6_K, w["v"], qkv[:, QDIM + KVDIM:], w["plane_v"])], q8_x, M, HIDDEN)
         capi.quantize_q8_1(attn, out=q8_attn)
         capi.gemv(FMT_Q4_K, w["o"], q8_attn, M, HIDDEN, QDIM, out=o_out, plane=w["plane_o"])
+        if fused_ffn:
+            return ffn_fused(w)
         capi.quantize_q8_1(x2, out=q8_x2)
         capi.gemv_fused([(FMT_Q4_K, w["gate"], gate, w["plane_gate"]), (FMT_Q4_K, w["up"], up, w["plane_up"])],
                         q8_x2, M, HIDDEN)
@@ -520,6 +539,8 @@ def main():
                              (FMT_Q4_K, w["k"], qkv[:, QDIM:QDIM + KVDIM], w["plane_k"]),
                              (FMT_Q6_K, w["v"], qkv[:, QDIM + KVDIM:], w["plane_v"])], x, M, HIDDEN, q8_scratch=q8_x)
         capi.gemv_fused_f32([(FMT_Q4_K, w["o"], o_out, w["plane_o"])], attn, M, QDIM, q8_scratch=q8_attn)
+        if fused_ffn:
+            return ffn_fused(w)
         capi.gemv_fused_f32([(FMT_Q4_K, w["gate"], gate, w["plane_gate"]), (FMT_Q4_K, w["up"], up, w["plane_up"])],
                             x2, M, HIDDEN, q8_scratch=q8_x2)
         capi.gemv_swiglu_f32(FMT_Q6_K, w["down"], gate, up, M, HIDDEN, FFN, out=down, q8_scratch=q8_act,
@@ -685,6 +706,7 @@ def main():
                 "pct_of_hbm_peak": round(100.0 * layer_gbs / HBM_PEAK_GBS, 2),
                 "distinct_weight_sets": args.layers,
                 "batch_planes": n_planes // max(args.layers, 1),   # projections per layer read from batch planes (batches of 5..8)
+                "fused_ffn": bool(fused_ffn),   # gate + up + SwiGLU + Q8_1 in one launch (batches of 5..8)
                 "steps": args.steps,
                 "launch": "eager" if graphs is None else "hip-graph replay",
             },
