@@ -468,6 +468,12 @@ namespace llamql
         g.row0 = row0;
         g.nrows = nrows;
         g.tile0 = DUMP ? row0 / GEMM_BN : 0;
+        // (the quad-lane decoders address a matrix through 32-bit offsets)
+        if constexpr (F::USE_QUAD)
+        {
+            if (!F::Quad::addressable(N, K / 256))
+                return fail(fn, "matrix too large for the kernel's 32-bit offsets (N=%d K=%d)", N, K);
+        }
         const int tile_end = DUMP ? (row0 + nrows + GEMM_BN - 1) / GEMM_BN : (N + GEMM_BN - 1) / GEMM_BN;
         // few tokens: one smaller tile of tokens (a 128-token tile would rescale 128 rows for them)
         if (M <= 32)

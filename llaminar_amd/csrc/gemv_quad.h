@@ -442,8 +442,9 @@ namespace llamql
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
         // workgroup size bound: one activation row leaves room for 16 wavefronts of 128 registers
         static constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
-        // whether this matrix can be addressed by the kernel at all
-        static bool addressable(long, int) { return true; }
+        // whether this matrix can be addressed by the kernel at all: super-block indices are 24-bit
+        // multiplicands, byte offsets from the matrix's base 32-bit
+        static bool addressable(long N, int SB) { return (double)N * SB < 16777216.0; }
         // lane l decodes blocks 2l (first) and 2l+1 (second)
         __device__ __forceinline__ static void owner(int j, int &l, int &which)
         {
@@ -484,53 +485,57 @@ namespace llamql
         // Where a lane reads: its current super-block, and the one it reads instead once it
         // is past the end of its run (its last valid one, still in the caches): loads are
         // never predicated, a load under a lane mask would be waited for at once.
+        // The cursor is a super-block index; addresses are the matrix's base (uniform, in scalar
+        // registers) plus a 32-bit byte offset per lane: one multiply-add per load address where
+        // 64-bit pointers per lane took six vector instructions a step to move and select.
         struct Cursor
         {
-            const uint8_t *p, *first;
+            const uint8_t *base; // uniform
+            uint32_t t, first;
         };
         __device__ __forceinline__ static Cursor cursor(const GemvArgs &a, size_t t, size_t t_safe, const Lane &)
         {
             Cursor c;
-            c.p = static_cast<const uint8_t *>(a.w) + t * SB_BYTES;
-            c.first = static_cast<const uint8_t *>(a.w) + t_safe * SB_BYTES;
+            c.base = static_cast<const uint8_t *>(a.w);
+            c.t = (uint32_t)t;
+            c.first = (uint32_t)t_safe;
             return c;
         }
-        // What a lane's position moves by from one step to the next (uniform): the step's
-        // super-blocks, and `jump` more when the lane's next super-block lies in the next row.
+        // What a lane's position moves by from one step to the next (uniform), in super-blocks: the
+        // step's, and `jump` more when the lane's next super-block lies in the next row.
         struct Stride
         {
-            size_t plain, cross;
+            uint32_t plain, cross;
         };
         __device__ __forceinline__ static Stride stride(uint32_t jump)
         {
             Stride st;
-            st.plain = (size_t)QUAD_STEP_SB * SB_BYTES;
-            st.cross = ((size_t)QUAD_STEP_SB + jump) * SB_BYTES;
+            st.plain = (uint32_t)QUAD_STEP_SB;
+            st.cross = (uint32_t)QUAD_STEP_SB + jump;
             return st;
         }
         __device__ __forceinline__ static void next(Cursor &c, bool cross, const Stride &st)
         {
-            c.p += cross ? st.cross : st.plain;
+            c.t += cross ? st.cross : st.plain;
         }
         __device__ __forceinline__ static void load(Raw &r, const Cursor &c, const Lane &lc, bool valid)
         {
-            const uint8_t *p = valid ? c.p : c.first;
-            load(r, p, p + lc.byte_off);
+            load_index(r, c, lc, valid ? c.t : c.first);
         }
         // super-block sb_off after the cursor's
         __device__ __forceinline__ static void load_at(Raw &r, const Cursor &c, const Lane &lc, int sb_off)
         {
-            const uint8_t *p = c.p + (size_t)sb_off * SB_BYTES;
-            load(r, p, p + lc.byte_off);
+            load_index(r, c, lc, c.t + (uint32_t)sb_off);
         }
-        // sb: this lane's super-block, grp: the same plus the lane's group offset.  The
-        // loads are issued as assembly so that the kernel, not the compiler, decides where
+        // The loads are issued as assembly so that the kernel, not the compiler, decides where
         // they are waited for (wait() below); the compiler would wait right after issue.
-        __device__ __forceinline__ static void load(Raw &r, const uint8_t *sb, const uint8_t *grp)
+        __device__ __forceinline__ static void load_index(Raw &r, const Cursor &c, const Lane &lc, uint32_t t)
         {
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.head) : "v"(sb));
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(r.qa) : "v"(grp));
-            asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=&v"(r.qb) : "v"(grp));
+            const uint32_t osb = __umul24(t, (uint32_t)SB_BYTES);
+            const uint32_t ogrp = __umul24(t, (uint32_t)SB_BYTES) + (uint32_t)lc.byte_off;
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.head) : "v"(osb), "s"(c.base));
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(r.qa) : "v"(ogrp), "s"(c.base));
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(r.qb) : "v"(ogrp), "s"(c.base));
         }
         // Marks r's registers as in use up to this point (emits nothing).
         __device__ __forceinline__ static void keep(Raw &r)
