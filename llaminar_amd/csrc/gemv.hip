@@ -92,10 +92,45 @@ namespace llamql
             // batches that go to the matrix-unit kernel launch one matrix at a time
             if constexpr (F::USE_MFMA_BATCH)
                 if (mfma_eligible<F>(M, projs[0].N, K) || batch_plane_for<F>(projs[0].d_plane, M, projs[0].N, K))
+                {
+                    // .. unless a run of small matrices for the quad-lane kernel follows a Q4_K one (Q, then K
+                    // and V): those share its launch
+                    if constexpr (std::is_same<F, Q4KTraits>::value)
+                        if (src.kind == ACT_SRC_Q8 && gemv_mfma_quad_ok(M, projs[0].N, K, device_id))
+                        {
+                            QuadProj pr[QUAD_MAX_PROJ];
+                            int na = 0, nb = 0;
+                            auto quad_only = [&](auto tag, const llam_ql_proj &q) {
+                                typedef decltype(tag) G;
+                                return quad_eligible<G>(M, q.N, K) && !mfma_eligible<G>(M, q.N, K) &&
+                                       !batch_plane_for<G>(q.d_plane, M, q.N, K);
+                            };
+                            while (1 + na < num && na < QUAD_MAX_PROJ && projs[1 + na].fmt == LLAM_FMT_Q4_K &&
+                                   quad_only(Q4KTraits{}, projs[1 + na]))
+                            {
+                                pr[na] = QuadProj{projs[1 + na].d_w, projs[1 + na].d_y, projs[1 + na].N, projs[1 + na].ldy};
+                                ++na;
+                            }
+                            while (1 + na + nb < num && na + nb < QUAD_MAX_PROJ && projs[1 + na + nb].fmt == LLAM_FMT_Q6_K &&
+                                   quad_only(Q6KTraits{}, projs[1 + na + nb]))
+                            {
+                                pr[na + nb] = QuadProj{projs[1 + na + nb].d_w, projs[1 + na + nb].d_y, projs[1 + na + nb].N,
+                                                       projs[1 + na + nb].ldy};
+                                ++nb;
+                            }
+                            if (na + nb > 0 && quad_lds_bytes(M, K / 256) <= QUAD_MAX_LDS)
+                                return gemv_mfma_quad_launch(fn, projs[0].d_w,
+                                                             batch_plane_for<F>(projs[0].d_plane, M, projs[0].N, K),
+                                                             projs[0].d_y, projs[0].N, projs[0].ldy, pr, na, nb, src.q8, M, K,
+                                                             device_id, st)
+                                           ? 1 + na + nb
+                                           : -1;
+                        }
                     return gemv_mfma_launch<F>(fn, projs[0].d_w, batch_plane_for<F>(projs[0].d_plane, M, projs[0].N, K), src,
                                                 projs[0].d_y, M, projs[0].N, K, projs[0].ldy, device_id, st)
                                ? 1
                                : -1;
+                }
             QuadProj pr[QUAD_MAX_PROJ];
             int n = 0;
             while (n < num && n < QUAD_MAX_PROJ && projs[n].fmt == projs[0].fmt &&

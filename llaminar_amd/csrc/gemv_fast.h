@@ -562,6 +562,7 @@ namespace llamql
         a.SB = SB;
         a.M = M;
         a.slices = sh.slices;
+        a.tiles_per_wg = sh.tiles_per_wg;
         a.tile_rows = sh.tile_rows;
         a.sums = d_sums;
         a.row0 = row0;
@@ -625,6 +626,7 @@ namespace llamql
         a.SB = SB;
         a.M = M;
         a.slices = sh.slices;
+        a.tiles_per_wg = sh.tiles_per_wg;
         a.tile_rows = MFMA_TILE_ROWS;
         const int waves = sh.slices * sh.tiles_per_wg;
         if (waves > MFMA_MAX_WAVES)
@@ -863,20 +865,27 @@ namespace llamql
     // The same over two runs of matrices in two formats (na of FA, then nb of FB; na + nb <=
     // QUAD_MAX_PROJ), Q8_1 or plain fp32 activations.  The second format starts at a
     // workgroup boundary.
+    // What a two-format launch is made of.  force_nw: wavefronts per workgroup the caller needs (0: chosen here).
+    struct QuadDualLaunch
+    {
+        QuadArgs a;
+        long grid, nw;
+        size_t lds;
+    };
     template <class FA, class FB>
-    bool gemv_quad_dual(const char *fn, const QuadProj *pr, int na, int nb, const ActSource &src, int M, int K,
-                        int device_id, hipStream_t st)
+    bool gemv_quad_dual_setup(const char *fn, const QuadProj *pr, int na, int nb, const ActSource &src, int M, int K,
+                              int device_id, int force_nw, QuadDualLaunch &out)
     {
         if constexpr (FA::USE_QUAD && FB::USE_QUAD)
         {
             typedef typename FA::Quad QA;
             typedef typename FB::Quad QB;
+            QuadArgs &a = out.a;
             const int SB = K / 256;
             const int cus = cu_count(device_id);
             const int mta = QA::max_threads(M), mtb = QB::max_threads(M);
             const int max_waves = (mta < mtb ? mta : mtb) / WAVE;
             const int n = na + nb;
-            QuadArgs a;
             a.q8 = static_cast<const uint32_t *>(src.q8);
             a.x = src.x;
             a.x2 = src.x2;
@@ -915,6 +924,12 @@ namespace llamql
                 nw = waves;
             if (nw < 1)
                 nw = 1;
+            if (force_nw > 0)
+            {
+                if (force_nw > max_waves)
+                    return fail(fn, "workgroups of %d wavefronts at M=%d", force_nw, M);
+                nw = force_nw;
+            }
             long at = 0;
             for (int i = 0; i < QUAD_MAX_PROJ; ++i)
             {
@@ -938,7 +953,29 @@ namespace llamql
             lds += norm;
             if (lds > QUAD_MAX_LDS)
                 return fail(fn, "K=%d: %d activation row(s) and the norm's scratch do not fit the LDS", K, M);
-            gemv_quad_dual_launch<QA, QB>(M, src.kind, dim3((unsigned)grid), dim3((unsigned)nw * WAVE), lds, st, a);
+            out.grid = grid;
+            out.nw = nw;
+            out.lds = lds;
+            return true;
+        }
+        else
+        {
+            (void)pr; (void)na; (void)nb; (void)src; (void)M; (void)K; (void)device_id; (void)force_nw; (void)out;
+            return fail(fn, "formats have no quad-lane kernel");
+        }
+    }
+
+    template <class FA, class FB>
+    bool gemv_quad_dual(const char *fn, const QuadProj *pr, int na, int nb, const ActSource &src, int M, int K,
+                        int device_id, hipStream_t st)
+    {
+        if constexpr (FA::USE_QUAD && FB::USE_QUAD)
+        {
+            QuadDualLaunch L;
+            if (!gemv_quad_dual_setup<FA, FB>(fn, pr, na, nb, src, M, K, device_id, 0, L))
+                return false;
+            gemv_quad_dual_launch<typename FA::Quad, typename FB::Quad>(M, src.kind, dim3((unsigned)L.grid),
+                                                                         dim3((unsigned)L.nw * WAVE), L.lds, st, L.a);
             return launched(fn);
         }
         else
@@ -946,6 +983,101 @@ namespace llamql
             (void)pr; (void)na; (void)nb; (void)src; (void)M; (void)K; (void)device_id; (void)st;
             return fail(fn, "formats have no quad-lane kernel");
         }
+    }
+
+    // ---- a matrix-unit matrix and a quad-lane group in ONE launch (batches of 5..8) -------------------------------
+    // Q (thousands of rows: the matrix unit) and K, V (a thousand rows each: the quad-lane kernel) read the
+    // same activations and used to be two launches of about 10 us each, most of it the latency chain of a
+    // launch.  Here the first workgroups of the launch run the matrix-unit body on Q, the others the
+    // quad-lane bodies on the group: every matrix keeps the tiling, slices and rows per wavefront of its
+    // own launch, so the results are those of the separate launches bit for bit.
+    constexpr int MIXED_WAVES = 8; // wavefronts per workgroup: what the quad-lane kernels run at these batches
+    template <bool PLANE, int M>
+    __global__ void __launch_bounds__(MIXED_WAVES *WAVE)
+        gemv_mfma_quad_kernel(const MfmaArgs a, const QuadArgs qa, const int mfma_blocks)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t mixed_lds[];
+        if ((int)blockIdx.x < mfma_blocks) // uniform per workgroup
+        {
+            gemv_mfma_q4k_body<QUAD_SRC_Q8, false, PLANE, false>(a, mixed_lds, (int)blockIdx.x);
+            return;
+        }
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int wid_all = ((int)blockIdx.x - mfma_blocks) * MIXED_WAVES + wave;
+        int p, w_first;
+        quad_which(qa, wid_all, p, w_first);
+        if (p < qa.first_b)
+            quad_body<Q4KQuad, M, quad_unroll<Q4KQuad>(M), QUAD_SRC_Q8>(qa, mixed_lds, p, w_first, wid_all);
+        else
+            quad_body<Q6KQuad, M, quad_unroll<Q6KQuad>(M), QUAD_SRC_Q8>(qa, mixed_lds, p, w_first, wid_all);
+    }
+
+    template <bool PLANE, int M>
+    void gemv_mfma_quad_launch_pm(dim3 grid, size_t lds, hipStream_t st, const MfmaArgs &a, const QuadArgs &qa,
+                                  int mfma_blocks)
+    {
+        static LdsGrant grant;
+        (void)allow_lds(grant, reinterpret_cast<const void *>(&gemv_mfma_quad_kernel<PLANE, M>), QUAD_MAX_LDS);
+        hipLaunchKernelGGL((gemv_mfma_quad_kernel<PLANE, M>), grid, dim3(MIXED_WAVES * WAVE), lds, st, a, qa, mfma_blocks);
+    }
+
+    // Whether the Q4_K matrix's own matrix-unit launch fits workgroups of MIXED_WAVES wavefronts (then the
+    // mixed launch can run it unchanged).
+    inline bool gemv_mfma_quad_ok(int M, int N, int K, int device_id)
+    {
+        if (M < 5 || M > 8 || !mfma_eligible<Q4KTraits>(M, N, K) || mfma4_long_rows(K / 256))
+            return false;
+        const MfmaShape sh = gemv_mfma_shape(N, K / 256, cu_count(device_id), MFMA_MAX_WAVES);
+        return sh.slices * sh.tiles_per_wg <= MIXED_WAVES;
+    }
+
+    // d_w / d_plane / d_y / N / ldy: the matrix-unit matrix (Q4_K); pr: na Q4_K then nb Q6_K matrices for the
+    // quad-lane kernel (na + nb >= 1); Q8_1 activations.
+    inline bool gemv_mfma_quad_launch(const char *fn, const void *d_w, const void *d_plane, float *d_y, int N, int ldy,
+                                      const QuadProj *pr, int na, int nb, const void *d_q8, int M, int K,
+                                      int device_id, hipStream_t st)
+    {
+        const int SB = K / 256;
+        const MfmaShape sh = gemv_mfma_shape(N, SB, cu_count(device_id), MFMA_MAX_WAVES);
+        MfmaArgs a{};
+        a.w = static_cast<const uint8_t *>(d_w);
+        a.plane = static_cast<const uint8_t *>(d_plane);
+        a.q8 = static_cast<const uint32_t *>(d_q8);
+        a.y = d_y;
+        a.ldy = ldy;
+        a.N = N;
+        a.SB = SB;
+        a.M = M;
+        a.slices = sh.slices;
+        a.tiles_per_wg = sh.tiles_per_wg;
+        a.tile_rows = sh.tile_rows;
+        QuadDualLaunch L;
+        if (!gemv_quad_dual_setup<Q4KTraits, Q6KTraits>(fn, pr, na, nb, act_source_q8(d_q8), M, K, device_id, MIXED_WAVES, L))
+            return false;
+        const size_t lds_mfma = a.plane ? mfma_act_bytes(SB) : mfma_lds_bytes(SB, sh.slices * sh.tiles_per_wg);
+        // (the partial sums of all eight wavefronts lie over the activations at the end)
+        const size_t lds = lds_mfma > L.lds ? lds_mfma : L.lds;
+        if (lds > QUAD_MAX_LDS || lds < (size_t)MIXED_WAVES * 4 * WAVE * sizeof(float))
+            return fail(fn, "%zu bytes of LDS (N=%d K=%d)", lds, N, K);
+        const dim3 grid((unsigned)(sh.grid + L.grid));
+        const int mb = (int)sh.grid;
+#define LLAM_MIXED_CASE(m)                                                                                             \
+    case m:                                                                                                            \
+        if (a.plane)                                                                                                   \
+            gemv_mfma_quad_launch_pm<true, m>(grid, lds, st, a, L.a, mb);                                              \
+        else                                                                                                           \
+            gemv_mfma_quad_launch_pm<false, m>(grid, lds, st, a, L.a, mb);                                             \
+        break;
+        switch (M)
+        {
+            LLAM_MIXED_CASE(5)
+            LLAM_MIXED_CASE(6)
+            LLAM_MIXED_CASE(7)
+        default:
+            LLAM_MIXED_CASE(8)
+        }
+#undef LLAM_MIXED_CASE
+        return launched(fn);
     }
 
     // What the launcher does with a shape: the one place where the kernel, the batch split and

@@ -50,8 +50,9 @@ namespace llamql
         int N;
         int SB;           // super-blocks per weight row
         int M;            // activation rows, 1..8
-        int slices;       // wavefronts per tile (wavefront j walks super-blocks j, j + slices, ..);
-                          // a workgroup holds blockDim/64/slices tiles
+        int slices;       // wavefronts per tile (wavefront j walks super-blocks j, j + slices, ..)
+        int tiles_per_wg; // tiles of a workgroup; wavefronts beyond slices * tiles_per_wg help to stage the
+                          // activations and idle otherwise
         int tile_rows;    // weight rows of a tile, 1..32: fewer than 32 leave columns of the matrix
                           // instruction unused, and let the tiles of a launch fill every compute unit
         // DUMP kernels only: the exact per-block int32 sums of rows [row0, row0+nrows) go to
@@ -268,14 +269,13 @@ namespace llamql
     // stand-alone quantiser's arithmetic (the bits of the two projections followed by
     // llam_ql_swiglu_quantize for the same partition of the rows into slices); the fp32 results go to
     // memory only if asked for.  Tiles are 32 rows, N a multiple of 32.
+    // block: the workgroup's index among those of this kernel body (a launch may hold other workgroups).
     template <int SRC, bool DUMP = false, bool PLANE = false, bool SWIGLU = false>
-    __global__ void __launch_bounds__((DUMP ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES) * WAVE)
-        gemv_mfma_q4k_kernel(const MfmaArgs a)
+    __device__ __forceinline__ void gemv_mfma_q4k_body(const MfmaArgs &a, uint8_t *mfma_lds, const int block)
     {
         static_assert(!(SWIGLU && DUMP), "the block-sum variant walks one matrix");
         typedef typename std::conditional<PLANE, MfmaPlaneRaw, MfmaRaw>::type Raw;
         constexpr int LOADS = PLANE ? MFMA_PLANE_LOADS : MFMA_LOADS;
-        extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];
         const int nsb = a.SB;
         const int nkb = nsb * 8;
         uint8_t *aq = mfma_lds;                                                 // [kb][8 rows][32 B] (+16)
@@ -287,21 +287,22 @@ namespace llamql
 
         // this wavefront's tile and slice of the row, and this lane's weight row
         const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
-        const int tiles_per_wg = (int)(blockDim.x >> 6) / a.slices;
+        const int tiles_per_wg = a.tiles_per_wg;
+        const bool idle = tile_local >= tiles_per_wg; // (uniform) a wavefront without a tile
         // slice j walks super-blocks j, j + slices, ..: at any moment the wavefronts of a tile
         // read NEIGHBOURING super-blocks of every row, so a 128-byte line that straddles two
         // super-blocks (144 bytes each) is asked for by two wavefronts of the workgroup at the
         // same time and crosses the fabric once
-        const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
+        const int nsteps = !idle && slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
         // SWIGLU: tile 2 p of the workgroup is the gate half, tile 2 p + 1 the up half of pair p
         const int mat = SWIGLU ? tile_local & 1 : 0;
-        const long tile_idx = SWIGLU ? (long)blockIdx.x * (tiles_per_wg >> 1) + (tile_local >> 1)
-                                     : (long)blockIdx.x * tiles_per_wg + tile_local;
+        const long tile_idx = SWIGLU ? (long)block * (tiles_per_wg >> 1) + (tile_local >> 1)
+                                     : (long)block * tiles_per_wg + tile_local;
         const long tile_row0 = tile_idx * a.tile_rows;
         const uint8_t *const w_mat = SWIGLU && mat ? a.w2 : a.w;
         const uint8_t *const plane_mat = SWIGLU && mat ? a.plane2 : a.plane;
         const long row = tile_row0 + l32;
-        const bool row_ok = l32 < a.tile_rows && row < a.N;
+        const bool row_ok = !idle && l32 < a.tile_rows && row < a.N;
         const int last_step = nsteps > 0 ? nsteps - 1 : 0;
 
         // piece p = lane + 64 i of the step: 16 bytes at offset 16 (p % 9) of row p / 9.  Rows
@@ -531,7 +532,7 @@ namespace llamql
         __syncthreads();
         // SWIGLU: the tiles' sums meet in LDS behind the partial sums, [tile][8 activation rows][32 weight rows]
         float *res = red + (size_t)(blockDim.x >> 6) * 4 * WAVE;
-        if (slice == 0)
+        if (slice == 0 && !idle)
         {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -559,7 +560,7 @@ namespace llamql
             __syncthreads();
             // the first wavefront of a pair: eight lanes per activation row quantise its block (the lane
             // mapping of the stand-alone quantiser)
-            if (slice == 0 && mat == 0)
+            if (slice == 0 && mat == 0 && !idle)
             {
                 const int m = lane >> 3, sub = lane & 7;
                 const float4 g = reinterpret_cast<const float4 *>(res + (tile_local * 8 + m) * 32)[sub];
@@ -574,6 +575,14 @@ namespace llamql
                 }
             }
         }
+    }
+
+    template <int SRC, bool DUMP = false, bool PLANE = false, bool SWIGLU = false>
+    __global__ void __launch_bounds__((DUMP ? MFMA_DUMP_WAVES : MFMA_MAX_WAVES) * WAVE)
+        gemv_mfma_q4k_kernel(const MfmaArgs a)
+    {
+        extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[];
+        gemv_mfma_q4k_body<SRC, DUMP, PLANE, SWIGLU>(a, mfma_lds, (int)blockIdx.x);
     }
 
     struct MfmaShape

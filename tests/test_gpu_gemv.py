@@ -174,6 +174,37 @@ def test_fused_groups_equal_separate_calls(capi, dev, M):
     assert torch.isnan(out[:, total:]).all()
 
 
+@pytest.mark.parametrize("with_plane", [False, True], ids=["prepared", "plane"])
+@pytest.mark.parametrize("M", [5, 6, 7, 8])
+def test_matrix_unit_matrix_and_quad_lane_group_in_one_launch(capi, dev, M, with_plane):
+    """Batches of 5..8: a Q4_K matrix of thousands of rows (the matrix unit) followed by small matrices for the
+    quad-lane kernel (Q, then K and V) go out as ONE launch whose first workgroups run the matrix-unit body;
+    every output carries the bits of its own llam_ql_gemv call.  Followers: Q4_K and Q6_K, Q6_K only, Q4_K
+    only; ragged row counts; a batch plane for the large matrix."""
+    import torch
+
+    K = 5120
+    qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(8, K, 123)).to(dev))
+    for g, specs in enumerate([[(FMT_Q4_K, 8192), (FMT_Q4_K, 1024), (FMT_Q6_K, 1024)],
+                               [(FMT_Q4_K, 4100), (FMT_Q6_K, 333), (FMT_Q6_K, 64)],
+                               [(FMT_Q4_K, 5120), (FMT_Q4_K, 77), (FMT_Q4_K, 512), (FMT_Q4_K, 640)]]):
+        total = sum(n for _, n in specs)
+        out = torch.full((M, total + 3), float("nan"), device=dev)
+        projs, singles, col = [], [], 0
+        for i, (fmt, N) in enumerate(specs):
+            wd = capi.prepare_weights(fmt, synth.weights_torch(fmt, N, K, 1900 + 10 * g + i, dev), N, K)
+            plane = capi.build_batch_plane(fmt, wd, N, K) if (with_plane and i == 0) else None
+            assert (plane is not None) == (with_plane and i == 0)
+            projs.append((fmt, wd, out[:, col:col + N], plane))
+            singles.append((col, N, capi.gemv(fmt, wd, qd, M, N, K, plane=plane)))
+            col += N
+        capi.gemv_fused(projs, qd, M, K)
+        sync()
+        for c0, N, y in singles:
+            assert torch.equal(out[:, c0:c0 + N], y), f"group {g}: projection at column {c0} differs"
+        assert torch.isnan(out[:, total:]).all()
+
+
 @pytest.mark.parametrize("M", [1, 3, 8])
 def test_fp32_input_equals_quantise_then_gemv(capi, dev, M):
     """llam_ql_gemv_f32 / _fused_f32 / _swiglu_f32 quantise inside the kernel: bits of the
