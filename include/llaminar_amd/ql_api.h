@@ -139,7 +139,11 @@ typedef struct
 /* Several projections of ONE quantised input in one launch (QKV, gate+up,
  * 2*top_k MoE gate/up).  Replaces gemv_native_vnni_fused_preq
  * (CPUNativeVNNIGemv.h:3807-3881).  num <= LLAM_QL_MAX_FUSED; `projs` is a host
- * array read during the call. */
+ * array read during the call.  Neighbours in the array share a launch where their kernels
+ * allow it (up to four quad-lane matrices of one format, a second run in the other quad-lane
+ * format behind them, and at batches of 5..8 a Q4_K matrix on the matrix unit with the small
+ * quad-lane matrices that follow it: Q, then K and V); every output carries the bits of its own
+ * llam_ql_gemv / llam_ql_gemv_plane call. */
 bool llam_ql_gemv_fused(const llam_ql_proj *projs, int num, const void *d_q8,
                         int M, int K, int device_id, void *stream);
 
