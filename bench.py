@@ -304,6 +304,8 @@ def bench_decode(args, torch, capi, synth, dev):
 
         fused_ffn = (capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, B, F, H) and
                      (P("0.wgate") is None) == (P("0.wup") is None))
+        split_down = capi.gemv_plane_split_supported(FMT_Q6_K, B, H, F)
+        o_hi = torch.empty(B, H, device=dev)
 
         def linear_only():
             for l in range(shape.n_layers):
@@ -316,7 +318,10 @@ def bench_decode(args, torch, capi, synth, dev):
                 if fused_ffn:   # as the decoder does at these batches: gate, up, SwiGLU and its quantiser in one launch
                     capi.gemv_gate_up_swiglu(FMT_Q4_K, W[f"{l}.wgate"], W[f"{l}.wup"], q8, B, F, H,
                                              plane_gate=P(f"{l}.wgate"), plane_up=P(f"{l}.wup"), q8_out=q8a)
-                    capi.gemv(FMT_Q6_K, W[f"{l}.wdown"], q8a, B, H, F, out=o, plane=P(f"{l}.wdown"))
+                    if split_down and P(f"{l}.wdown") is not None:
+                        capi.gemv_plane_split(FMT_Q6_K, P(f"{l}.wdown"), q8a, B, H, F, out_lo=o, out_hi=o_hi)
+                    else:
+                        capi.gemv(FMT_Q6_K, W[f"{l}.wdown"], q8a, B, H, F, out=o, plane=P(f"{l}.wdown"))
                     continue
                 capi.gemv_fused([(FMT_Q4_K, W[f"{l}.wgate"], gate, P(f"{l}.wgate")),
                                  (FMT_Q4_K, W[f"{l}.wup"], up, P(f"{l}.wup"))], q8, B, H)
@@ -508,12 +513,17 @@ def main():
 
     # batches the matrix unit serves: gate, up, SwiGLU and the Q8_1 quantiser of the result as one launch
     fused_ffn = capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, M, FFN, HIDDEN)
+    split_down = capi.gemv_plane_split_supported(FMT_Q6_K, M, HIDDEN, FFN)
+    down_hi = torch.empty(M, HIDDEN, device=dev)
 
     def ffn_fused(w):
         capi.quantize_q8_1(x2, out=q8_x2)
         capi.gemv_gate_up_swiglu(FMT_Q4_K, w["gate"], w["up"], q8_x2, M, FFN, HIDDEN, plane_gate=w["plane_gate"],
                                  plane_up=w["plane_up"], q8_out=q8_act)
-        capi.gemv(FMT_Q6_K, w["down"], q8_act, M, HIDDEN, FFN, out=down, plane=w["plane_down"])
+        if split_down and w["plane_down"] is not None:   # the rows' halves as two partial sums (the next norm adds them)
+            capi.gemv_plane_split(FMT_Q6_K, w["plane_down"], q8_act, M, HIDDEN, FFN, out_lo=down, out_hi=down_hi)
+        else:
+            capi.gemv(FMT_Q6_K, w["down"], q8_act, M, HIDDEN, FFN, out=down, plane=w["plane_down"])
 
     def step_separate(w):
         # quantiser kernels of their own, Q8_1 blocks through memory
@@ -707,6 +717,7 @@ def main():
                 "distinct_weight_sets": args.layers,
                 "batch_planes": n_planes // max(args.layers, 1),   # projections per layer read from batch planes (batches of 5..8)
                 "fused_ffn": bool(fused_ffn),   # gate + up + SwiGLU + Q8_1 in one launch (batches of 5..8)
+                "split_down": bool(split_down and n_planes > 0),   # down projection summed in two halves (batches of 5..8)
                 "steps": args.steps,
                 "launch": "eager" if graphs is None else "hip-graph replay",
             },

@@ -45,6 +45,10 @@ bool llam_dec_embed_q4k(const void *d_table, int vocab, const int32_t *d_ids, fl
  * activation quantiser of the next projection.  H % 32 == 0, rows 16-byte aligned. */
 bool llam_dec_rmsnorm_q8_1(float *d_x, const float *d_delta, const float *d_gamma, float eps,
                            float *d_y, void *d_q8, int M, int H, int device_id, void *stream);
+/* The same with the delta in two partial sums (a projection whose rows were summed in two halves,
+ * llam_ql_gemv_plane_split): d_x[m] += (d_delta[m] + d_delta2[m]).  d_delta2 == NULL is the call above. */
+bool llam_dec_rmsnorm2_q8_1(float *d_x, const float *d_delta, const float *d_delta2, const float *d_gamma,
+                            float eps, float *d_y, void *d_q8, int M, int H, int device_id, void *stream);
 
 /* inv_freq[i] = exp(-log(theta) * (2 i / head_dim)), i < head_dim/2, in fp32 with the
  * host's libm: get_inv_freq_cached (src/v2/kernels/cpu/primitives/RoPEPrimitives.cpp:50-77).

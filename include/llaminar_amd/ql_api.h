@@ -200,6 +200,21 @@ bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const void *d_plane, 
  * the down projection (CPUNativeVNNIGemmKernel.h:572, :325-431; the decode flow of
  * MoEExpertComputeStage.cpp:1450-1708 for a dense block). */
 bool llam_ql_gemv_gate_up_swiglu_supported(uint8_t fmt, int M, int N, int K);
+
+/* A projection with long rows at batches of 5..8, its rows summed in two halves:
+ *     d_y_lo[m][n] = sum over the first K/2 columns,  d_y_hi[m][n] = sum over the last K/2
+ * from the matrix's batch plane (d_plane, llam_ql_build_batch_plane), per 32-column block the arithmetic of
+ * llam_ql_gemv_plane.  The caller adds the two (llam_dec_rmsnorm2_q8_1 does, in front of the next norm).
+ * Why: every workgroup of a matrix-unit launch stages the batch's activations for the columns it
+ * walks; for K = 25600 that is 230 KB per workgroup, as much traffic as its weights.  Here a workgroup
+ * walks half of the columns of twice the rows: 5120 x 25600 at batch 8 31 against 36 us.  The split is
+ * the reference's row-parallel tensor split of this projection run on one device (each K slice yields a
+ * partial sum, TPAllreduceStage adds them), without the exchange.  Served
+ * (llam_ql_gemv_plane_split_supported) for Q6_K, M = 5..8, K a multiple of 512 with K >= 16384; both
+ * outputs have row stride ldy and must be different buffers. */
+bool llam_ql_gemv_plane_split_supported(uint8_t fmt, int M, int N, int K);
+bool llam_ql_gemv_plane_split(uint8_t fmt, const void *d_plane, const void *d_q8, float *d_y_lo, float *d_y_hi, int M,
+                              int N, int K, int ldy, int device_id, void *stream);
 bool llam_ql_gemv_gate_up_swiglu(uint8_t fmt, const void *d_w_gate, const void *d_plane_gate,
                                  const void *d_w_up, const void *d_plane_up, const void *d_q8,
                                  float *d_y_gate, float *d_y_up, int ldy, void *d_q8_out, int M, int N,

@@ -91,6 +91,9 @@ SIGNATURES = {
     "llam_ql_moe_route_gate_up_swiglu": (c_bool, [c_uint8, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p,
                                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                   c_int, c_int, c_int, c_int, c_void_p]),
+    "llam_ql_gemv_plane_split_supported": (c_bool, [c_uint8, c_int, c_int, c_int]),
+    "llam_ql_gemv_plane_split": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                          c_void_p]),
     "llam_ql_gemv_gate_up_swiglu_supported": (c_bool, [c_uint8, c_int, c_int, c_int]),
     "llam_ql_gemv_gate_up_swiglu": (c_bool, [c_uint8, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                              c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
@@ -116,6 +119,8 @@ SIGNATURES = {
     "llam_dec_embed_q4k": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "llam_dec_rmsnorm_q8_1": (c_bool, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
                                        c_void_p]),
+    "llam_dec_rmsnorm2_q8_1": (c_bool, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int,
+                                        c_int, c_void_p]),
     "llam_dec_rope_inv_freq": (None, [c_int, c_float, c_void_p]),
     "llam_dec_rope_kv_append": (c_bool, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                          c_int, c_int, c_int, c_void_p]),
@@ -487,6 +492,24 @@ def moe_route_gate_up_swiglu(fmt: int, table, n_experts: int, logits, top_k: int
     return q8_out
 
 
+def gemv_plane_split_supported(fmt: int, M: int, N: int, K: int) -> bool:
+    return bool(load().llam_ql_gemv_plane_split_supported(fmt, M, N, K))
+
+
+def gemv_plane_split(fmt: int, plane, q8, M: int, N: int, K: int, out_lo=None, out_hi=None, stream=None):
+    """The sums over the first and the second half of every row's super-blocks as two outputs [M,N] (batches of
+    5..8 on long Q6_K rows, from the matrix's batch plane); their sum is the projection."""
+    import torch
+
+    if out_lo is None:
+        out_lo = torch.empty(M, N, dtype=torch.float32, device=plane.device)
+    if out_hi is None:
+        out_hi = torch.empty(M, N, dtype=torch.float32, device=plane.device)
+    _check(load().llam_ql_gemv_plane_split(fmt, _ptr(plane), _ptr(q8), _ptr(out_lo), _ptr(out_hi), M, N, K, _ld(out_lo),
+                                           _dev(plane), _stream(stream)), "gemv_plane_split")
+    return out_lo, out_hi
+
+
 def gemv_gate_up_swiglu_supported(fmt: int, M: int, N: int, K: int) -> bool:
     return bool(load().llam_ql_gemv_gate_up_swiglu_supported(fmt, M, N, K))
 
@@ -578,8 +601,9 @@ def embed_q4k(table, vocab: int, ids, H: int, out=None, stream=None):
 
 
 def rmsnorm_q8_1(x, gamma, eps: float, delta=None, want_y: bool = True, want_q8: bool = True, y=None, q8=None,
-                 stream=None):
-    """x [M,H] contiguous; with delta, x += delta in place first.  Returns (y, q8)."""
+                 stream=None, delta2=None):
+    """x [M,H] contiguous; with delta, x += delta in place first (x += delta + delta2 when the delta comes as two
+    partial sums).  Returns (y, q8)."""
     import torch
 
     M, H = x.shape
@@ -588,8 +612,12 @@ def rmsnorm_q8_1(x, gamma, eps: float, delta=None, want_y: bool = True, want_q8:
         y = torch.empty_like(x)
     if want_q8 and q8 is None:
         q8 = torch.empty(M * (H // 32) * 36, dtype=torch.uint8, device=x.device)
-    _check(load().llam_dec_rmsnorm_q8_1(_ptr(x), _ptr(delta), _ptr(gamma), eps, _ptr(y), _ptr(q8), M, H, _dev(x),
-                                        _stream(stream)), "rmsnorm_q8_1")
+    if delta2 is not None:
+        _check(load().llam_dec_rmsnorm2_q8_1(_ptr(x), _ptr(delta), _ptr(delta2), _ptr(gamma), eps, _ptr(y), _ptr(q8), M, H,
+                                             _dev(x), _stream(stream)), "rmsnorm2_q8_1")
+    else:
+        _check(load().llam_dec_rmsnorm_q8_1(_ptr(x), _ptr(delta), _ptr(gamma), eps, _ptr(y), _ptr(q8), M, H, _dev(x),
+                                            _stream(stream)), "rmsnorm_q8_1")
     return y, q8
 
 

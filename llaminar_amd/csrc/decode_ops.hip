@@ -55,14 +55,17 @@ namespace llamql
     constexpr int NORM_KEEP = 4;
 
     __global__ void __launch_bounds__(NORM_THREADS)
-        rmsnorm_q8_1_kernel(float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ gamma,
-                            float eps, float *__restrict__ y, uint32_t *__restrict__ q8, int H)
+        rmsnorm_q8_1_kernel(float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ delta2,
+                            const float *__restrict__ gamma, float eps, float *__restrict__ y,
+                            uint32_t *__restrict__ q8, int H)
     {
+        // delta2 (only with delta): the delta arrives as two partial sums, x += (delta + delta2)
         __shared__ double s_part[NORM_THREADS / WAVE];
         const int m = blockIdx.x;
         const int nvec = H >> 2;
         float4 *row = reinterpret_cast<float4 *>(x + (size_t)m * H);
         const float4 *drow = delta ? reinterpret_cast<const float4 *>(delta + (size_t)m * H) : nullptr;
+        const float4 *d2row = delta && delta2 ? reinterpret_cast<const float4 *>(delta2 + (size_t)m * H) : nullptr;
         const float4 *g4 = reinterpret_cast<const float4 *>(gamma);
 
         float4 keep[NORM_KEEP], dk[NORM_KEEP], gk[NORM_KEEP];
@@ -77,6 +80,24 @@ namespace llamql
                 if (drow)
                     dk[t] = drow[i];
                 gk[t] = g4[i];
+            }
+        }
+        if (d2row) // (uniform; its loads go out with the others, before anything is waited for)
+        {
+            float4 d2[NORM_KEEP];
+#pragma unroll
+            for (int t = 0; t < NORM_KEEP; ++t)
+            {
+                const int i = threadIdx.x + t * NORM_THREADS;
+                d2[t] = i < nvec ? d2row[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
+#pragma unroll
+            for (int t = 0; t < NORM_KEEP; ++t)
+            {
+                dk[t].x += d2[t].x;
+                dk[t].y += d2[t].y;
+                dk[t].z += d2[t].z;
+                dk[t].w += d2[t].w;
             }
         }
 
@@ -109,7 +130,15 @@ namespace llamql
             float4 v = row[i];
             if (drow)
             {
-                const float4 d = drow[i];
+                float4 d = drow[i];
+                if (d2row)
+                {
+                    const float4 e = d2row[i];
+                    d.x += e.x;
+                    d.y += e.y;
+                    d.z += e.z;
+                    d.w += e.w;
+                }
                 v.x += d.x;
                 v.y += d.y;
                 v.z += d.z;
@@ -800,7 +829,15 @@ extern "C" bool llam_dec_embed_q4k(const void *d_table, int vocab, const int32_t
 extern "C" bool llam_dec_rmsnorm_q8_1(float *d_x, const float *d_delta, const float *d_gamma, float eps,
                                       float *d_y, void *d_q8, int M, int H, int device_id, void *stream)
 {
+    return llam_dec_rmsnorm2_q8_1(d_x, d_delta, nullptr, d_gamma, eps, d_y, d_q8, M, H, device_id, stream);
+}
+
+extern "C" bool llam_dec_rmsnorm2_q8_1(float *d_x, const float *d_delta, const float *d_delta2, const float *d_gamma,
+                                       float eps, float *d_y, void *d_q8, int M, int H, int device_id, void *stream)
+{
     static const char *fn = "llam_dec_rmsnorm_q8_1";
+    if (d_delta2 && (!d_delta || !aligned16(d_delta2)))
+        return fail(fn, "a second delta needs the first, and 16-byte alignment");
     if (M < 0 || H < 1)
         return fail(fn, "bad size (M=%d H=%d)", M, H);
     if (M == 0)
@@ -814,7 +851,7 @@ extern "C" bool llam_dec_rmsnorm_q8_1(float *d_x, const float *d_delta, const fl
         return fail(fn, "fp32 rows must be 16-byte aligned, d_q8 4-byte aligned");
     if (!set_device(fn, device_id))
         return false;
-    hipLaunchKernelGGL(rmsnorm_q8_1_kernel, dim3(M), dim3(NORM_THREADS), 0, as_stream(stream), d_x, d_delta,
+    hipLaunchKernelGGL(rmsnorm_q8_1_kernel, dim3(M), dim3(NORM_THREADS), 0, as_stream(stream), d_x, d_delta, d_delta2,
                        d_gamma, eps, d_y, static_cast<uint32_t *>(d_q8), H);
     return launched(fn);
 }

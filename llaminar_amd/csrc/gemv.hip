@@ -313,6 +313,29 @@ namespace llamql
     }
 } // namespace llamql
 
+extern "C" bool llam_ql_gemv_plane_split_supported(uint8_t fmt, int M, int N, int K)
+{
+    return fmt == LLAM_FMT_Q6_K && K >= 1 && llamql::gemv_mfma_q6k_split_ok(M, N, K);
+}
+
+extern "C" bool llam_ql_gemv_plane_split(uint8_t fmt, const void *d_plane, const void *d_q8, float *d_y_lo,
+                                         float *d_y_hi, int M, int N, int K, int ldy, int device_id, void *stream)
+{
+    using namespace llamql;
+    static const char *fn = "llam_ql_gemv_plane_split";
+    if (!llam_ql_gemv_plane_split_supported(fmt, M, N, K))
+        return fail(fn, "not served for format %d, M=%d, N=%d, K=%d (llam_ql_gemv_plane_split_supported)", (int)fmt, M, N, K);
+    if (!d_plane || !d_q8 || !d_y_lo || !d_y_hi || d_y_lo == d_y_hi)
+        return fail(fn, "null pointer, or one buffer for both halves");
+    if (!aligned16(d_plane) || !aligned4(d_q8))
+        return fail(fn, "d_plane must be 16-byte and d_q8 4-byte aligned");
+    if (ldy < N)
+        return fail(fn, "ldy=%d smaller than N=%d", ldy, N);
+    if (!set_device(fn, device_id))
+        return false;
+    return gemv_mfma_q6k_split_launch(fn, d_plane, d_q8, d_y_lo, d_y_hi, M, N, K, ldy, device_id, as_stream(stream));
+}
+
 extern "C" bool llam_ql_gemv_gate_up_swiglu_supported(uint8_t fmt, int M, int N, int K)
 {
     return fmt == LLAM_FMT_Q4_K && M >= 1 && M <= LLAM_QL_MAX_GEMV_M && N >= 1 && K >= 1 &&

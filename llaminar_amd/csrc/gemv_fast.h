@@ -657,6 +657,12 @@ namespace llamql
         hipLaunchKernelGGL((gemv_mfma_q6k_kernel<SRC, DUMP>), grid, block, lds, st, a);
     }
 
+    inline bool batch_plane_usable_q6k(int M, int N, int K)
+    {
+        return M >= 5 && M <= 8 && gemv_unroll_override() == 0 && gemv_rows_per_wave_override() == 0 && K / 256 >= 8 &&
+               q6k_plane_bytes(N, K / 256) < ((size_t)1 << 32);
+    }
+
     template <int SRC, bool DUMP = false>
     void gemv_mfma_q6k_plane_launch_src(dim3 grid, dim3 block, size_t lds, hipStream_t st, const Mfma6Args &a)
     {
@@ -676,7 +682,8 @@ namespace llamql
         const Mfma6Shape sh =
             gemv_mfma6_shape(N, SB, cu_count(device_id), plane ? MFMA6_PLANE_COMPUTE : d_sums ? MFMA6_DUMP_COMPUTE : MFMA6_MAX_COMPUTE,
                              plane != nullptr);
-        Mfma6Args a;
+        Mfma6Args a{};
+        a.ksplit = 1;
         a.w = static_cast<const uint8_t *>(d_w);
         a.plane = plane;
         a.q8 = static_cast<const uint32_t *>(src.q8);
@@ -723,6 +730,50 @@ namespace llamql
         case ACT_SRC_SWIGLU: gemv_mfma_q6k_launch_src<QUAD_SRC_SWIGLU>(grid, block, lds, st, a); break;
         default: gemv_mfma_q6k_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a); break;
         }
+        return launched(fn);
+    }
+
+    // The plane kernel with the rows' super-blocks in two halves, one workgroup per (two tiles, half): a
+    // workgroup stages half of the batch's activations (what every workgroup stages of a long row costs as much
+    // as its weights: 8 rows of K = 25600 are 230 KB), the halves' sums go to two outputs and the caller adds them.
+    // Served for long rows only: each half must keep the wavefronts of a tile busy for several steps.
+    inline bool gemv_mfma_q6k_split_ok(int M, int N, int K)
+    {
+        return M >= 5 && M <= 8 && K % 512 == 0 && K / 256 >= 64 && N >= 1 && batch_plane_usable_q6k(M, N, K);
+    }
+    inline bool gemv_mfma_q6k_split_launch(const char *fn, const void *d_plane, const void *d_q8, float *d_y_lo,
+                                           float *d_y_hi, int M, int N, int K, int ldy, int device_id, hipStream_t st)
+    {
+        const int SB = K / 256;
+        // the shape of a matrix with rows of half the length, two tiles per workgroup (half the wavefronts per tile)
+        Mfma6Shape sh = gemv_mfma6_shape(N, SB / 2, cu_count(device_id), MFMA6_PLANE_COMPUTE, true);
+        if (sh.tiles == 1 && sh.slices >= 2)
+        {
+            sh.tiles = 2;
+            sh.slices /= 2;
+            sh.grid = (sh.grid + 1) / 2;
+            if (sh.chunk < SB / 2)
+                sh.chunk = sh.chunk / sh.slices * sh.slices;
+        }
+        Mfma6Args a{};
+        a.ksplit = 2;
+        a.plane = static_cast<const uint8_t *>(d_plane);
+        a.q8 = static_cast<const uint32_t *>(d_q8);
+        a.y = d_y_lo;
+        a.y2 = d_y_hi;
+        a.ldy = ldy;
+        a.N = N;
+        a.SB = SB;
+        a.M = M;
+        a.slices = sh.slices;
+        a.tiles = sh.tiles;
+        a.tile_rows = sh.tile_rows;
+        a.chunk = sh.chunk;
+        const dim3 grid((unsigned)(sh.grid * 2)), block((unsigned)(sh.slices * sh.tiles + MFMA6_PLANE_PRODUCERS) * WAVE);
+        const size_t lds = mfma6_act_bytes(SB / 2, sh.chunk);
+        if (lds > QUAD_MAX_LDS || sh.chunk < sh.slices)
+            return fail(fn, "launch shape (N=%d K=%d)", N, K);
+        gemv_mfma_q6k_plane_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a);
         return launched(fn);
     }
 

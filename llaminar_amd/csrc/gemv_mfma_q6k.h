@@ -60,6 +60,10 @@ namespace llamql
         // sums[(m * nrows + row - row0) * (SB * 8) + block]
         int32_t *sums;
         int row0, nrows;
+        // gemv_mfma_q6k_plane_kernel only: the row's super-blocks in ksplit (1 or 2) equal parts, one workgroup
+        // per (tiles, part); part 1's sums go to y2 (the caller adds the two)
+        int ksplit;
+        float *y2;
     };
 
     struct Mfma6Raw
@@ -431,7 +435,13 @@ namespace llamql
     {
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma6_lds[];
         const int nsb = a.SB;
-        const int nph = (nsb + a.chunk - 1) / a.chunk; // activation chunks
+        // this workgroup's part of the rows: super-blocks sb0 .. sb0 + nsbp (the whole row unless ksplit = 2)
+        const int part = a.ksplit > 1 ? (int)(blockIdx.x % (unsigned)a.ksplit) : 0;
+        const int wg = a.ksplit > 1 ? (int)(blockIdx.x / (unsigned)a.ksplit) : (int)blockIdx.x;
+        const int sb_per = (nsb + a.ksplit - 1) / a.ksplit;
+        const int sb0 = part * sb_per;
+        const int nsbp = sb0 + sb_per <= nsb ? sb_per : (nsb > sb0 ? nsb - sb0 : 0);
+        const int nph = (nsbp + a.chunk - 1) / a.chunk; // activation chunks
         const size_t buf_bytes = mfma_act_bytes(a.chunk);
         const int ncomp = a.slices * a.tiles; // compute wavefronts
         const int lane = threadIdx.x & (WAVE - 1);
@@ -443,8 +453,8 @@ namespace llamql
             return reinterpret_cast<float *>(mfma6_lds + (size_t)(ph & 1) * buf_bytes + (size_t)a.chunk * 8 * MFMA_AQ_STRIDE);
         };
         auto stage = [&](int ph, int tid, int nthreads, auto un) {
-            const int c0 = ph * a.chunk;
-            const int c1 = c0 + a.chunk < nsb ? c0 + a.chunk : nsb;
+            const int c0 = sb0 + ph * a.chunk;
+            const int c1 = ph * a.chunk + a.chunk < nsbp ? c0 + a.chunk : sb0 + nsbp;
             mfma_stage_acts<SRC, decltype(un)::value>(a.q8, a.x, a.x2, a.ldx, a.M, nsb * 8, c0 * 8, (c1 - c0) * 8,
                                                       buf_aq(ph), buf_asc(ph), tid, nthreads);
         };
@@ -465,9 +475,9 @@ namespace llamql
         {
             const int l32 = lane & 31, lh = lane >> 5;
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
-            const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
+            const int nsteps = slice < nsbp ? (nsbp - slice + a.slices - 1) / a.slices : 0;
             const int last_step = nsteps > 0 ? nsteps - 1 : 0;
-            const long tile_row0 = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows;
+            const long tile_row0 = ((long)wg * a.tiles + tile_local) * a.tile_rows;
             // rows past the end of the tile or of the matrix re-read the last one
             const long r_tile = tile_row0 + (l32 < a.tile_rows ? l32 : a.tile_rows - 1);
             const long row = r_tile < a.N ? r_tile : a.N - 1;
@@ -478,7 +488,7 @@ namespace llamql
 
             // loads are never predicated: past its last step a lane re-reads that step
             auto issue = [&](Mfma6PlaneRaw &r, int step) {
-                const uint32_t sb = nsteps > 0 ? (uint32_t)(slice + (step < last_step ? step : last_step) * a.slices) : 0u;
+                const uint32_t sb = (uint32_t)sb0 + (nsteps > 0 ? (uint32_t)(slice + (step < last_step ? step : last_step) * a.slices) : 0u);
                 auto uniform = [](const uint8_t *p) {
                     const uint64_t b = (uint64_t)p;
                     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
@@ -514,14 +524,15 @@ namespace llamql
             int step = 0, cur_ph = 0;
 
             auto compute = [&](const Mfma6PlaneRaw &r) {
-                const int sb = slice + step * a.slices;
-                const int ph = sb / a.chunk;
+                const int sbl = slice + step * a.slices; // within the part
+                const int sb = sb0 + sbl;
+                const int ph = sbl / a.chunk;
                 while (cur_ph < ph) // uniform: wait until the chunk this step needs has been staged
                 {
                     mfma6_barrier();
                     ++cur_ph;
                 }
-                const int kb0 = (sb - ph * a.chunk) * 8;
+                const int kb0 = (sbl - ph * a.chunk) * 8;
                 const uint8_t *ab = buf_aq(ph) + (size_t)kb0 * MFMA_AQ_STRIDE + a_lane;
                 const float *sb_sc = buf_asc(ph) + (size_t)kb0 * 16 + lh * 8;
                 const v4i wv[8] = {r.w0, r.w1, r.w2, r.w3, r.w4, r.w5, r.w6, r.w7};
@@ -601,7 +612,8 @@ namespace llamql
         if (wave < ncomp)
         {
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
-            const long row = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows + (lane & 31);
+            const long row = ((long)wg * a.tiles + tile_local) * a.tile_rows + (lane & 31);
+            float *const y_part = part ? a.y2 : a.y;
             if (slice == 0 && (lane & 31) < a.tile_rows)
             {
 #pragma unroll
@@ -614,7 +626,7 @@ namespace llamql
                     if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
                     {
                         if (m < a.M && row < a.N)
-                            a.y[(size_t)m * a.ldy + row] = v;
+                            y_part[(size_t)m * a.ldy + row] = v;
                     }
                 }
             }

@@ -53,7 +53,7 @@ namespace
         int32_t *ids = nullptr, *pos = nullptr;
         int host_max_pos = 0; // the furthest sequence's position as the host counts it
         float *last_res = nullptr; // where the last step left the residual stream (x or x_alt)
-        float *x = nullptr, *x_alt = nullptr, *delta = nullptr, *qkv = nullptr, *attn = nullptr, *gate = nullptr, *up = nullptr;
+        float *x = nullptr, *x_alt = nullptr, *delta = nullptr, *delta2 = nullptr, *qkv = nullptr, *attn = nullptr, *gate = nullptr, *up = nullptr;
         float *logits = nullptr, *inv_freq = nullptr, *rope_table = nullptr, *att_scratch = nullptr;
         void *q8_h = nullptr, *q8_attn = nullptr, *q8_act = nullptr, *argmax_scratch = nullptr;
         std::vector<void *> kcache, vcache;
@@ -134,7 +134,7 @@ extern "C" void *llam_decoder_create(const llam_decoder_config *c)
     const int wide = H > d->qdim() ? H : d->qdim();
     bool ok = d->alloc(d->ids, (size_t)B * 4) && d->alloc(d->pos, (size_t)B * 4) &&
               d->alloc(d->x, (size_t)B * H * 4) && d->alloc(d->x_alt, (size_t)B * H * 4) &&
-              d->alloc(d->delta, (size_t)B * H * 4) &&
+              d->alloc(d->delta, (size_t)B * H * 4) && d->alloc(d->delta2, (size_t)B * H * 4) &&
               d->alloc(d->qkv, (size_t)B * (d->qdim() + 2 * d->kvdim()) * 4) &&
               d->alloc(d->attn, (size_t)B * d->qdim() * 4) && d->alloc(d->gate, (size_t)B * F * 4) &&
               d->alloc(d->up, (size_t)B * F * 4) && d->alloc(d->logits, (size_t)B * c->vocab * 4) &&
@@ -292,10 +292,11 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
     // Where the projections' kernels can run the norm themselves (llam_ql_gemv_fused_rmsnorm: no
     // launch for the norm) a pending delta is added into the other of the two buffers, elsewhere the
     // norm updates `res` in place.
+    // (a projection whose rows were summed in two halves leaves two deltas: pending and pending2)
     float *res = d->x, *spare = d->x_alt;
-    const float *pending = nullptr;
+    const float *pending = nullptr, *pending2 = nullptr;
     auto norm_and_project = [&](const llam_ql_proj *projs, int num, const float *gamma) {
-        if (llam_ql_gemv_fused_rmsnorm_supported(projs, num, B, H))
+        if (!pending2 && llam_ql_gemv_fused_rmsnorm_supported(projs, num, B, H))
         {
             if (!forward(fn, llam_ql_gemv_fused_rmsnorm(projs, num, res, pending, gamma, c.rms_eps, spare, B, H, dev,
                                                         stream)))
@@ -305,12 +306,12 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
         }
         else
         {
-            if (!forward(fn, llam_dec_rmsnorm_q8_1(res, pending, gamma, c.rms_eps, nullptr, d->q8_h, B, H, dev, stream)))
+            if (!forward(fn, llam_dec_rmsnorm2_q8_1(res, pending, pending2, gamma, c.rms_eps, nullptr, d->q8_h, B, H, dev, stream)))
                 return false;
             if (!forward(fn, llam_ql_gemv_fused(projs, num, d->q8_h, B, H, dev, stream)))
                 return false;
         }
-        pending = nullptr;
+        pending = pending2 = nullptr;
         return true;
     };
     // res += W q8 where the launch can, else delta = W q8 and pending
@@ -318,6 +319,13 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
         if (llam_ql_gemv_accumulate_supported(fmt, B, H, K, dev))
             return forward(fn, llam_ql_gemv_accumulate(fmt, w, q8, res, B, H, K, H, dev, stream));
         pending = d->delta;
+        // long rows at batches the matrix unit serves: the row's halves as two launches' worth of workgroups, each
+        // staging half of the activations; the next norm adds both partial sums
+        if (plane && llam_ql_gemv_plane_split_supported(fmt, B, H, K))
+        {
+            pending2 = d->delta2;
+            return forward(fn, llam_ql_gemv_plane_split(fmt, plane, q8, d->delta, d->delta2, B, H, K, H, dev, stream));
+        }
         return forward(fn, llam_ql_gemv_plane(fmt, w, plane, q8, d->delta, B, H, K, H, dev, stream));
     };
     for (int l = 0; l < c.n_layers; ++l)
@@ -346,9 +354,10 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
         if (w.fmt_gate == w.fmt_up && (w.plane_gate != nullptr) == (w.plane_up != nullptr) &&
             llam_ql_gemv_gate_up_swiglu_supported(w.fmt_gate, B, F, H))
         {
-            if (!forward(fn, llam_dec_rmsnorm_q8_1(res, pending, w.ffn_norm, c.rms_eps, nullptr, d->q8_h, B, H, dev, stream)))
+            if (!forward(fn, llam_dec_rmsnorm2_q8_1(res, pending, pending2, w.ffn_norm, c.rms_eps, nullptr, d->q8_h, B, H, dev,
+                                                    stream)))
                 return false;
-            pending = nullptr;
+            pending = pending2 = nullptr;
             if (!forward(fn, llam_ql_gemv_gate_up_swiglu(w.fmt_gate, w.wgate, w.plane_gate, w.wup, w.plane_up, d->q8_h,
                                                          nullptr, nullptr, 0, d->q8_act, B, F, H, dev, stream)))
                 return false;
@@ -375,8 +384,8 @@ extern "C" bool llam_decoder_step(void *dec, void *stream)
             pending = d->delta;
         }
     }
-    if (!forward(fn, llam_dec_rmsnorm_q8_1(res, pending, d->globals.final_norm, c.rms_eps, nullptr, d->q8_h, B, H,
-                                           dev, stream)))
+    if (!forward(fn, llam_dec_rmsnorm2_q8_1(res, pending, pending2, d->globals.final_norm, c.rms_eps, nullptr, d->q8_h, B,
+                                            H, dev, stream)))
         return false;
     d->last_res = res; // the final norm has added what was pending
     if (!forward(fn, llam_ql_gemv_plane(d->globals.fmt_lm_head, d->globals.lm_head, d->globals.plane_lm_head, d->q8_h,

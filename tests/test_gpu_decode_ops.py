@@ -67,6 +67,27 @@ def test_rmsnorm_q8_1(capi, dev, oracle, M, H):
     sync()
 
 
+@pytest.mark.parametrize("M,H", [(8, 5120), (5, 9216)])
+def test_rmsnorm_with_the_delta_in_two_partial_sums(capi, dev, M, H):
+    """llam_dec_rmsnorm2_q8_1: x += (delta + delta2), then the norm: the bits of the one-delta call on the sum of
+    the two (rows longer than the registers hold included)."""
+    import torch
+
+    rng = np.random.default_rng(7 * M + H)
+    x = torch.from_numpy(rng.standard_normal((M, H)).astype(np.float32)).to(dev)
+    g = torch.from_numpy(rng.uniform(0.2, 2.0, H).astype(np.float32)).to(dev)
+    d1 = torch.from_numpy(rng.standard_normal((M, H)).astype(np.float32)).to(dev)
+    d2 = torch.from_numpy((rng.standard_normal((M, H)) * 1e-3).astype(np.float32)).to(dev)
+    xa, xb = x.clone(), x.clone()
+    ya, qa = capi.rmsnorm_q8_1(xa, g, 1e-6, delta=d1, delta2=d2)
+    yb, qb = capi.rmsnorm_q8_1(xb, g, 1e-6, delta=d1 + d2)
+    sync()
+    assert torch.equal(xa, xb) and torch.equal(xa, x + (d1 + d2))
+    assert torch.equal(ya, yb) and torch.equal(qa, qb)
+    with pytest.raises(capi.QLError, match="second delta"):
+        capi.rmsnorm_q8_1(x.clone(), g, 1e-6, delta=None, delta2=d2)
+
+
 @pytest.mark.parametrize("B,n_heads,n_kv", [(1, 64, 8), (8, 64, 8), (3, 4, 1), (2, 6, 6)])
 def test_rope_kv_append(capi, dev, oracle, B, n_heads, n_kv):
     import torch

@@ -205,6 +205,38 @@ def test_matrix_unit_matrix_and_quad_lane_group_in_one_launch(capi, dev, M, with
         assert torch.isnan(out[:, total:]).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(8, 5120, 25600), (5, 1000, 16384), (6, 130, 17408)])
+def test_long_q6k_rows_summed_in_two_halves(capi, dev, oracle, M, N, K):
+    """llam_ql_gemv_plane_split (batches of 5..8, Q6_K rows of 64 super-blocks and more, from the batch plane): the
+    first output is the projection over the first half of every row's super-blocks, the second over the second half
+    -- each checked against the oracle on that half of the matrix and of the activations -- and their sum is the
+    projection (the one-launch plane kernel to re-association accuracy)."""
+    fmt = FMT_Q6_K
+    assert capi.gemv_plane_split_supported(fmt, M, N, K)
+    W = synth.weights_numpy(fmt, N, K, 4000 + N)
+    q8 = oracle.quantize(synth.activations_numpy(M, K, 4100 + K))
+    wd, qd = upload_weights(capi, dev, fmt, W), upload_q8(dev, q8)
+    plane = capi.build_batch_plane(fmt, wd, N, K)
+    lo, hi = capi.gemv_plane_split(fmt, plane, qd, M, N, K)
+    y = capi.gemv(fmt, wd, qd, M, N, K, plane=plane)
+    sync()
+    lo, hi, y = lo.cpu().numpy(), hi.cpu().numpy(), y.cpu().numpy()
+    assert rel_err(lo + hi, y) <= 2e-6
+    half = K // 2
+    rows = slice(0, min(N, 96))
+    q8r = q8.reshape(M, K // 32, -1)
+    for part, got in ((0, lo), (1, hi)):
+        Wp = np.ascontiguousarray(W[rows, part * (half // 256):(part + 1) * (half // 256)])
+        qp = np.ascontiguousarray(q8r[:, part * (half // 32):(part + 1) * (half // 32)])
+        C = oracle.gemm(fmt, Wp, half, qp)
+        assert rel_err(got[:, rows], C) <= TOL[fmt] * 1e-2
+    # not served: short rows, batches of 1..4, other formats, an odd number of super-blocks
+    assert not capi.gemv_plane_split_supported(fmt, M, N, 8192)
+    assert not capi.gemv_plane_split_supported(fmt, 4, N, K)
+    assert not capi.gemv_plane_split_supported(FMT_Q4_K, M, N, K)
+    assert not capi.gemv_plane_split_supported(fmt, M, N, 16640)
+
+
 @pytest.mark.parametrize("M", [1, 3, 8])
 def test_fp32_input_equals_quantise_then_gemv(capi, dev, M):
     """llam_ql_gemv_f32 / _fused_f32 / _swiglu_f32 quantise inside the kernel: bits of the
