@@ -210,8 +210,9 @@ bool llam_ql_gemv_gate_up_swiglu_supported(uint8_t fmt, int M, int N, int K);
  * walks half of the columns of twice the rows: 5120 x 25600 at batch 8 31 against 36 us.  The split is
  * the reference's row-parallel tensor split of this projection run on one device (each K slice yields a
  * partial sum, TPAllreduceStage adds them), without the exchange.  Served
- * (llam_ql_gemv_plane_split_supported) for Q6_K, M = 5..8, K a multiple of 512 with K >= 16384; both
- * outputs have row stride ldy and must be different buffers. */
+ * (llam_ql_gemv_plane_split_supported) for M = 5..8 and K a multiple of 512 with K >= 16384: Q6_K, and
+ * Q4_K matrices whose batch goes to the chunked matrix-unit kernel (4096 rows and more, rows too long for the
+ * whole batch in LDS); both outputs have row stride ldy and must be different buffers. */
 bool llam_ql_gemv_plane_split_supported(uint8_t fmt, int M, int N, int K);
 bool llam_ql_gemv_plane_split(uint8_t fmt, const void *d_plane, const void *d_q8, float *d_y_lo, float *d_y_hi, int M,
                               int N, int K, int ldy, int device_id, void *stream);

@@ -315,7 +315,10 @@ namespace llamql
 
 extern "C" bool llam_ql_gemv_plane_split_supported(uint8_t fmt, int M, int N, int K)
 {
-    return fmt == LLAM_FMT_Q6_K && K >= 1 && llamql::gemv_mfma_q6k_split_ok(M, N, K);
+    if (K < 1)
+        return false;
+    return fmt == LLAM_FMT_Q6_K ? llamql::gemv_mfma_q6k_split_ok(M, N, K)
+                                : fmt == LLAM_FMT_Q4_K && llamql::gemv_mfma_q4k_split_ok(M, N, K);
 }
 
 extern "C" bool llam_ql_gemv_plane_split(uint8_t fmt, const void *d_plane, const void *d_q8, float *d_y_lo,
@@ -333,6 +336,8 @@ extern "C" bool llam_ql_gemv_plane_split(uint8_t fmt, const void *d_plane, const
         return fail(fn, "ldy=%d smaller than N=%d", ldy, N);
     if (!set_device(fn, device_id))
         return false;
+    if (fmt == LLAM_FMT_Q4_K)
+        return gemv_mfma_q4k_split_launch(fn, d_plane, d_q8, d_y_lo, d_y_hi, M, N, K, ldy, device_id, as_stream(stream));
     return gemv_mfma_q6k_split_launch(fn, d_plane, d_q8, d_y_lo, d_y_hi, M, N, K, ldy, device_id, as_stream(stream));
 }
 

@@ -490,6 +490,7 @@ namespace llamql
         const Mfma6Shape sh = gemv_mfma6_shape(N, SB, cu_count(device_id), d_sums ? MFMA4_LONG_DUMP_COMPUTE : MFMA4_LONG_COMPUTE,
                                                d_plane != nullptr, MFMA_BOUNCE);
         MfmaLongArgs a{};
+        a.ksplit = 1;
         a.w = static_cast<const uint8_t *>(d_w);
         a.plane = static_cast<const uint8_t *>(d_plane);
         a.q8 = static_cast<const uint32_t *>(src.q8);
@@ -774,6 +775,47 @@ namespace llamql
         if (lds > QUAD_MAX_LDS || sh.chunk < sh.slices)
             return fail(fn, "launch shape (N=%d K=%d)", N, K);
         gemv_mfma_q6k_plane_launch_src<QUAD_SRC_Q8>(grid, block, lds, st, a);
+        return launched(fn);
+    }
+
+    // The same for Q4_K rows the chunked kernel walks (gemv_mfma_q4k_long_kernel), from the matrix's batch plane.
+    inline bool gemv_mfma_q4k_split_ok(int M, int N, int K)
+    {
+        return M >= 5 && M <= 8 && K % 512 == 0 && K / 256 >= 64 && N >= 1 && mfma_eligible<Q4KTraits>(M, N, K) &&
+               mfma4_long_rows(K / 256) && q4k_plane_bytes(N, K / 256) < ((size_t)1 << 32);
+    }
+    inline bool gemv_mfma_q4k_split_launch(const char *fn, const void *d_plane, const void *d_q8, float *d_y_lo,
+                                           float *d_y_hi, int M, int N, int K, int ldy, int device_id, hipStream_t st)
+    {
+        const int SB = K / 256;
+        Mfma6Shape sh = gemv_mfma6_shape(N, SB / 2, cu_count(device_id), MFMA4_LONG_COMPUTE, true, MFMA_BOUNCE);
+        if (sh.tiles == 1 && sh.slices >= 2)
+        {
+            sh.tiles = 2;
+            sh.slices /= 2;
+            sh.grid = (sh.grid + 1) / 2;
+            if (sh.chunk < SB / 2)
+                sh.chunk = sh.chunk / sh.slices * sh.slices;
+        }
+        MfmaLongArgs a{};
+        a.ksplit = 2;
+        a.plane = static_cast<const uint8_t *>(d_plane);
+        a.q8 = static_cast<const uint32_t *>(d_q8);
+        a.y = d_y_lo;
+        a.y2 = d_y_hi;
+        a.ldy = ldy;
+        a.N = N;
+        a.SB = SB;
+        a.M = M;
+        a.slices = sh.slices;
+        a.tile_rows = sh.tile_rows;
+        a.tiles = sh.tiles;
+        a.chunk = sh.chunk;
+        const dim3 grid((unsigned)(sh.grid * 2)), block((unsigned)(sh.slices * sh.tiles + MFMA4_LONG_PRODUCERS) * WAVE);
+        const size_t lds = mfma6_act_bytes(SB / 2, sh.chunk);
+        if (lds > QUAD_MAX_LDS || sh.chunk < sh.slices)
+            return fail(fn, "launch shape (N=%d K=%d)", N, K);
+        gemv_mfma_q4k_long_launch_src<QUAD_SRC_Q8, false, true>(grid, block, lds, st, a);
         return launched(fn);
     }
 

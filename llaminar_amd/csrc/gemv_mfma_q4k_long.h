@@ -18,6 +18,10 @@ namespace llamql
     {
         int tiles; // tiles per workgroup
         int chunk; // super-blocks per activation buffer; a multiple of slices when SB > chunk
+        // the row's super-blocks in ksplit (1 or 2) equal parts, one workgroup per (tiles, part); part 1's sums go
+        // to y2 (the caller adds the two: gemv_mfma_q6k_plane_kernel has the same)
+        int ksplit;
+        float *y2;
     };
 
     constexpr int MFMA4_LONG_COMPUTE = MFMA6_MAX_COMPUTE; // compute wavefronts per workgroup
@@ -35,7 +39,13 @@ namespace llamql
         extern __shared__ __attribute__((aligned(16))) uint8_t mfma4_lds[];
         const int nsb = a.SB;
         const int nkb = nsb * 8;
-        const int nph = (nsb + a.chunk - 1) / a.chunk; // activation chunks
+        // this workgroup's part of the rows: super-blocks sb0 .. sb0 + nsbp (the whole row unless ksplit = 2)
+        const int part = a.ksplit > 1 ? (int)(blockIdx.x % (unsigned)a.ksplit) : 0;
+        const int wg = a.ksplit > 1 ? (int)(blockIdx.x / (unsigned)a.ksplit) : (int)blockIdx.x;
+        const int sb_per = (nsb + a.ksplit - 1) / a.ksplit;
+        const int sb0 = part * sb_per;
+        const int nsbp = sb0 + sb_per <= nsb ? sb_per : (nsb > sb0 ? nsb - sb0 : 0);
+        const int nph = (nsbp + a.chunk - 1) / a.chunk; // activation chunks
         const size_t buf_bytes = mfma_act_bytes(a.chunk);
         const int ncomp = a.slices * a.tiles; // compute wavefronts
         const int lane = threadIdx.x & (WAVE - 1);
@@ -48,8 +58,8 @@ namespace llamql
         };
         // chunk ph into its buffer, by `nthreads` threads that keep UN loads in flight each
         auto stage_acts = [&](int ph, int tid, int nthreads, auto un) {
-            const int c0 = ph * a.chunk;
-            const int c1 = c0 + a.chunk < nsb ? c0 + a.chunk : nsb;
+            const int c0 = sb0 + ph * a.chunk;
+            const int c1 = ph * a.chunk + a.chunk < nsbp ? c0 + a.chunk : sb0 + nsbp;
             mfma_stage_acts<SRC, decltype(un)::value>(a.q8, a.x, a.x2, a.ldx, a.M, nkb, c0 * 8, (c1 - c0) * 8, buf_aq(ph),
                                                       buf_asc(ph), tid, nthreads);
         };
@@ -73,9 +83,9 @@ namespace llamql
             // ---- compute wavefronts --------------------------------------------------------------
             const int l32 = lane & 31, lh = lane >> 5;
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
-            const int nsteps = slice < nsb ? (nsb - slice + a.slices - 1) / a.slices : 0;
+            const int nsteps = slice < nsbp ? (nsbp - slice + a.slices - 1) / a.slices : 0;
             const int last_step = nsteps > 0 ? nsteps - 1 : 0;
-            const long tile_row0 = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows;
+            const long tile_row0 = ((long)wg * a.tiles + tile_local) * a.tile_rows;
             const long row = tile_row0 + l32;
             const bool row_ok = l32 < a.tile_rows && row < a.N;
 
@@ -115,7 +125,7 @@ namespace llamql
             };
             // loads are never predicated: past its last step a lane re-reads that step
             auto issue = [&](Raw &r, int step) {
-                const int sb = nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0;
+                const int sb = sb0 + (nsteps > 0 ? slice + (step < last_step ? step : last_step) * a.slices : 0);
                 if constexpr (PLANE)
                     mfma_plane_load(r, uniform(a.plane + (size_t)sb * 512),
                                     uniform(a.plane + q4k_plane_heads_offset(a.N, nsb) + (size_t)sb * 64), poff_w, poff_h);
@@ -161,14 +171,15 @@ namespace llamql
 
             // this lane's operands: the head of its row's super-block and its half of the four groups
             auto compute = [&](const v4i head, const v4i q0, const v4i q1, const v4i q2, const v4i q3) {
-                const int sb = slice + step * a.slices;
-                const int ph = sb / a.chunk;
+                const int sbl = slice + step * a.slices; // within the part
+                const int sb = sb0 + sbl;
+                const int ph = sbl / a.chunk;
                 while (cur_ph < ph) // uniform: wait until the chunk this step needs has been staged
                 {
                     mfma6_barrier();
                     ++cur_ph;
                 }
-                const int kb0 = (sb - ph * a.chunk) * 8;
+                const int kb0 = (sbl - ph * a.chunk) * 8;
                 const uint8_t *ab = buf_aq(ph) + (size_t)kb0 * MFMA_AQ_STRIDE + a_lane;
                 const float *sb_sc = buf_asc(ph) + (size_t)kb0 * 16 + lh * 8;
                 const v4i q[4] = {q0, q1, q2, q3};
@@ -295,7 +306,8 @@ namespace llamql
         if (wave < ncomp)
         {
             const int tile_local = wave / a.slices, slice = wave - tile_local * a.slices;
-            const long row = ((long)blockIdx.x * a.tiles + tile_local) * a.tile_rows + (lane & 31);
+            const long row = ((long)wg * a.tiles + tile_local) * a.tile_rows + (lane & 31);
+            float *const y_part = part ? a.y2 : a.y;
             if (slice == 0 && (lane & 31) < a.tile_rows)
             {
 #pragma unroll
@@ -308,7 +320,7 @@ namespace llamql
                     if constexpr (!DUMP) // the block-sum variant has no fp32 output (y is null)
                     {
                         if (m < a.M && row < a.N)
-                            a.y[(size_t)m * a.ldy + row] = v;
+                            y_part[(size_t)m * a.ldy + row] = v;
                     }
                 }
             }

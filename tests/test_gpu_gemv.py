@@ -205,13 +205,14 @@ def test_matrix_unit_matrix_and_quad_lane_group_in_one_launch(capi, dev, M, with
         assert torch.isnan(out[:, total:]).all()
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 5120, 25600), (5, 1000, 16384), (6, 130, 17408)])
-def test_long_q6k_rows_summed_in_two_halves(capi, dev, oracle, M, N, K):
-    """llam_ql_gemv_plane_split (batches of 5..8, Q6_K rows of 64 super-blocks and more, from the batch plane): the
-    first output is the projection over the first half of every row's super-blocks, the second over the second half
-    -- each checked against the oracle on that half of the matrix and of the activations -- and their sum is the
-    projection (the one-launch plane kernel to re-association accuracy)."""
-    fmt = FMT_Q6_K
+@pytest.mark.parametrize("fmt,M,N,K", [(FMT_Q6_K, 8, 5120, 25600), (FMT_Q6_K, 5, 1000, 16384), (FMT_Q6_K, 6, 130, 17408),
+                                       (FMT_Q4_K, 8, 5120, 25600), (FMT_Q4_K, 8, 4100, 17408)],
+                         ids=["q6k-m8", "q6k-m5", "q6k-m6-few-rows", "q4k-m8", "q4k-m8-ragged"])
+def test_long_rows_summed_in_two_halves(capi, dev, oracle, fmt, M, N, K):
+    """llam_ql_gemv_plane_split (batches of 5..8, rows of 64 super-blocks and more, from the batch plane; Q6_K, and
+    Q4_K matrices of 4096 rows and more): the first output is the projection over the first half of every row's
+    super-blocks, the second over the second half -- each checked against the oracle on that half of the matrix and
+    of the activations -- and their sum is the projection (the one-launch plane kernel to re-association accuracy)."""
     assert capi.gemv_plane_split_supported(fmt, M, N, K)
     W = synth.weights_numpy(fmt, N, K, 4000 + N)
     q8 = oracle.quantize(synth.activations_numpy(M, K, 4100 + K))
@@ -233,7 +234,8 @@ def test_long_q6k_rows_summed_in_two_halves(capi, dev, oracle, M, N, K):
     # not served: short rows, batches of 1..4, other formats, an odd number of super-blocks
     assert not capi.gemv_plane_split_supported(fmt, M, N, 8192)
     assert not capi.gemv_plane_split_supported(fmt, 4, N, K)
-    assert not capi.gemv_plane_split_supported(FMT_Q4_K, M, N, K)
+    assert not capi.gemv_plane_split_supported(FMT_IQ3_S, M, N, K)
+    assert not capi.gemv_plane_split_supported(FMT_Q4_K, M, 1024, K)    # too few rows for the matrix unit
     assert not capi.gemv_plane_split_supported(fmt, M, N, 16640)
 
 
