@@ -487,6 +487,40 @@ def test_gate_up_swiglu_in_one_launch_has_the_bits_of_the_two(capi, dev, fmt, hi
             assert bool((got[r] == 0x5A).all()), r
 
 
+@pytest.mark.parametrize("fmt,hidden,T", [(FMT_IQ3_S, 2048, 24), (FMT_IQ3_S, 512, 40), (FMT_Q4_K, 1024, 24), (FMT_Q6_K, 2048, 30),
+                                          (FMT_IQ3_S, 2048, 64), (FMT_IQ3_S, 2048, 70), (FMT_IQ3_S, 4096, 24)])
+def test_gate_up_swiglu_many_slots_of_few_experts(capi, dev, fmt, hidden, T):
+    """Many slots (72..210) of five experts, one of them used by every token: the launch shape for much work (two
+    steps in flight per wavefront).  Every slot's blocks are the bytes of the two-launch path; dead slots keep what
+    the buffer held."""
+    import torch
+
+    n_exp, inter, k = 5, 768, 3
+    host, devs, table = _experts(capi, dev, fmt, n_exp, hidden, inter, 71)
+    tab = table.clone()
+    tab.view(torch.int64).view(n_exp, 3)[3] = 0       # expert 3 lives elsewhere
+    rng = np.random.default_rng(hidden + T)
+    ids = rng.integers(0, n_exp, size=(T, k)).astype(np.int32)
+    ids[1, 2] = -3
+    ids[T - 1, 0] = n_exp
+    ids[:, 1] = 4                                     # an expert every token uses (the always-on expert of a model)
+    idd = torch.from_numpy(ids).to(dev)
+    qd = capi.quantize_q8_1(torch.from_numpy(synth.activations_numpy(T, hidden, 8)).to(dev))
+    gate, up = capi.moe_gate_up(fmt, tab, n_exp, idd, qd, T, k, hidden, inter)
+    want = capi.swiglu_quantize(gate, up).view(T * k, -1)
+    got = torch.full((T * k * (inter // 32) * 36,), 0x5A, dtype=torch.uint8, device=dev)
+    capi.moe_gate_up_swiglu(fmt, tab, n_exp, idd, qd, T, k, hidden, inter, q8_out=got)
+    sync()
+    got = got.view(T * k, -1)
+    live = ((ids >= 0) & (ids < n_exp) & (ids != 3)).reshape(-1)
+    assert 0 < live.sum() < T * k
+    for r in range(T * k):
+        if live[r]:
+            assert torch.equal(got[r], want[r]), r
+        else:
+            assert bool((got[r] == 0x5A).all()), r
+
+
 def test_gate_up_swiglu_other_row_lengths_run_the_two_launches(capi, dev):
     """Rows that are no power of two of super-blocks go through the caller's fp32 scratch rows; without them the
     call is refused."""
