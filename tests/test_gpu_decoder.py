@@ -108,15 +108,19 @@ def test_three_tokens_against_numpy_walk(capi, dev, oracle, batch):
     dec.close()
 
 
-def test_batch_eight_against_numpy_walk(capi, dev, oracle):
-    """One step at batch 8 (the matrix-unit GEMV kernels, the batched attention and sampler)
-    against the numpy walk, sequence by sequence: logits, greedy token and the appended K row."""
+@pytest.mark.parametrize("ffn,n_layers", [(4096, 2), (16384, 1)], ids=["ffn4096", "ffn16384-split-down"])
+def test_batch_eight_against_numpy_walk(capi, dev, oracle, ffn, n_layers):
+    """One step at batch 8 (the matrix-unit GEMV kernels: Q with K and V in one launch, gate + up + SwiGLU in one
+    launch; the batched attention and sampler) against the numpy walk, sequence by sequence: logits, greedy token
+    and the appended K row.  With a feed-forward width of 16384 the down projection's rows are long enough to be
+    summed in two halves, which the following norm adds."""
     import torch
 
     from llaminar_amd.decoder import DenseDecoder, Shape
 
     batch = 8
-    shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
+    shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=ffn, vocab=2048, n_layers=n_layers)
+    assert capi.gemv_plane_split_supported(FMT_Q6_K, batch, shape.hidden, ffn) == (ffn >= 16384)
     cap, start = 64, 20
     dec = DenseDecoder(shape, batch, cap, dev, seed=9, keep_raw=True, d_lo=0.002, d_hi=0.004, norm_scale=1.0)
     ref = NumpyDecoder(oracle, shape, dec.raw, cap)
