@@ -192,14 +192,15 @@ def test_a_full_context_is_reported(capi, dev):
     dec.close()
 
 
-@pytest.mark.parametrize("batch", [2, 6])
-def test_step_replays_as_a_graph(capi, dev, batch):
-    """A captured step replayed gives the tokens of eager steps (batch 6: the matrix-unit kernels)."""
+@pytest.mark.parametrize("batch,ffn", [(2, 4096), (6, 4096), (6, 16384)])
+def test_step_replays_as_a_graph(capi, dev, batch, ffn):
+    """A captured step replayed gives the tokens of eager steps (batch 6: the matrix-unit kernels and their merged
+    launches; feed-forward width 16384: the down projection summed in two halves)."""
     import torch
 
     from llaminar_amd.decoder import DenseDecoder, Shape
 
-    shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=4096, vocab=2048, n_layers=2)
+    shape = Shape(hidden=4096, n_heads=8, n_kv=2, head_dim=128, ffn=ffn, vocab=2048, n_layers=2)
     dec = DenseDecoder(shape, batch, 160, dev, seed=6)
     ids0 = np.array([7, 1999, 3, 1024, 77, 500][:batch], np.int32)
     pos0 = np.array([0, 0, 5, 17, 1, 130][:batch], np.int32)
