@@ -487,9 +487,11 @@ def main():
             raw = synth.weights_torch(fmt, N, K, 1000 * l + i, dev)
             w[name] = capi.prepare_weights(fmt, raw, N, K)
             del raw
-            # batches of 5..8 rows: the projections of 4096 rows and more read their weights from batch planes
+            # batches of 5..8 rows: the projections of 4096 rows and more read their weights from batch planes; batches
+            # of 2..4: the feed-forward matrices only (the launches that name the matrix unit serve them)
             w["plane_" + name] = None
-            if M >= 5 and N >= 4096 and not args.no_batch_planes and capi.batch_plane_bytes(fmt, N, K) > 0:
+            if ((M >= 5 or (M >= 2 and name in ("gate", "up", "down"))) and N >= 4096 and not args.no_batch_planes and
+                    capi.batch_plane_bytes(fmt, N, K) > 0):
                 w["plane_" + name] = capi.build_batch_plane(fmt, w[name], N, K)
                 n_planes += 1
         layers.append(w)

@@ -185,7 +185,7 @@ bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const void *d_plane, 
                              const float *d_up, int ld_gu, float *d_y, int M, int N, int K,
                              int ldy, void *d_q8_scratch, int device_id, void *stream);
 
-/* The feed-forward block's first half in one launch, batches of 5..8 rows:
+/* The feed-forward block's first half in one launch, batches of 2..8 rows:
  *   d_q8_out = Q8_1( silu(W_gate a) * (W_up a) )   [M x N/32 blocks], the down projection's input.
  * Both projections run on the matrix unit with their 32-row tiles paired inside a workgroup, which then
  * holds both operands of 32 consecutive columns and quantises the block itself: no launch for the
@@ -194,14 +194,16 @@ bool llam_ql_gemv_swiglu_f32(uint8_t fmt, const void *d_w, const void *d_plane, 
  * llam_ql_swiglu_quantize of those.  The projections are those of the matrix-unit kernel (the
  * reference's ascending block order within a wavefront's share of the row, llam_ql_gemv's contract for
  * batches of 5..8); their last bits may differ from two llam_ql_gemv calls, which split a row into
- * other shares.  Served (llam_ql_gemv_gate_up_swiglu_supported) for Q4_K, M = 5..8, N a multiple of 32
+ * other shares -- and at M = 2..4 a row does not carry the bits of its single-row call, which llam_ql_gemv
+ * guarantees there: the entry point is for callers whose rows are independent sequences.
+ * Served (llam_ql_gemv_gate_up_swiglu_supported) for Q4_K, M = 2..8, N a multiple of 32
  * and at least 4096, rows of 8..45 super-blocks (K = 2048..11520); d_plane_gate / d_plane_up: both matrices' batch planes
  * or both NULL.  Replaces multiply_fused_tensor over {gate, up} + compute_swiglu + the quantiser of
  * the down projection (CPUNativeVNNIGemmKernel.h:572, :325-431; the decode flow of
  * MoEExpertComputeStage.cpp:1450-1708 for a dense block). */
 bool llam_ql_gemv_gate_up_swiglu_supported(uint8_t fmt, int M, int N, int K);
 
-/* A projection with long rows at batches of 5..8, its rows summed in two halves:
+/* A projection with long rows at batches of 2..8 (Q4_K: 5..8), its rows summed in two halves:
  *     d_y_lo[m][n] = sum over the first K/2 columns,  d_y_hi[m][n] = sum over the last K/2
  * from the matrix's batch plane (d_plane, llam_ql_build_batch_plane), per 32-column block the arithmetic of
  * llam_ql_gemv_plane.  The caller adds the two (llam_dec_rmsnorm2_q8_1 does, in front of the next norm).
@@ -210,9 +212,11 @@ bool llam_ql_gemv_gate_up_swiglu_supported(uint8_t fmt, int M, int N, int K);
  * walks half of the columns of twice the rows: 5120 x 25600 at batch 8 31 against 36 us.  The split is
  * the reference's row-parallel tensor split of this projection run on one device (each K slice yields a
  * partial sum, TPAllreduceStage adds them), without the exchange.  Served
- * (llam_ql_gemv_plane_split_supported) for M = 5..8 and K a multiple of 512 with K >= 16384: Q6_K, and
- * Q4_K matrices whose batch goes to the chunked matrix-unit kernel (4096 rows and more, rows too long for the
- * whole batch in LDS); both outputs have row stride ldy and must be different buffers. */
+ * (llam_ql_gemv_plane_split_supported) for K a multiple of 512 with K >= 16384: Q6_K at M = 2..8 (like the
+ * entry point above it names the matrix-unit kernel: rows of batches of 2..4 do not carry the bits of their
+ * single-row calls), and Q4_K matrices whose batch goes to the chunked matrix-unit kernel (4096 rows and more,
+ * a batch too large for the LDS whole: M = 5..8 at most); both outputs have row stride ldy and must be
+ * different buffers. */
 bool llam_ql_gemv_plane_split_supported(uint8_t fmt, int M, int N, int K);
 bool llam_ql_gemv_plane_split(uint8_t fmt, const void *d_plane, const void *d_q8, float *d_y_lo, float *d_y_hi, int M,
                               int N, int K, int ldy, int device_id, void *stream);

@@ -599,12 +599,21 @@ namespace llamql
         return launched(fn);
     }
 
+    // Smallest batch the entry points that NAME the matrix-unit kernels serve (the fused feed-forward launch, the
+    // projection summed in two halves).  llam_ql_gemv keeps batches of up to 4 on the quad-lane kernel, whose rows
+    // carry the bits of their single-row calls; a caller that does not need that (independent sequences of a
+    // decode batch) is faster on the matrix unit from two rows on: the 64-layer decode step at batches of 2, 3 and 4
+    // 279 -> 292, 359 -> 395 and 430 -> 500 tokens/s.
+    constexpr int MFMA_NAMED_MIN_M = 2;
     // Gate and up projection with SwiGLU and the Q8_1 quantiser of the result in one launch
     // (gemv_mfma_q4k_kernel<.., SWIGLU>): Q4_K, batches of 5..8, rows the unchunked matrix-unit kernel
     // walks, N a multiple of 32; both matrices with a batch plane or neither.
     inline bool gemv_mfma_q4k_swiglu_ok(int M, int N, int K)
     {
-        return K % 256 == 0 && mfma_eligible<Q4KTraits>(M, N, K) && !mfma4_long_rows(K / 256) && N % MFMA_TILE_ROWS == 0;
+        // (the shape rules of a batch of 5..8; the entry point itself serves smaller batches too: its caller asks
+        // for the matrix unit by name and does not need a row to carry the bits of its single-row call)
+        return M >= MFMA_NAMED_MIN_M && M <= 8 && K % 256 == 0 && mfma_eligible<Q4KTraits>(M < 5 ? 5 : M, N, K) &&
+               !mfma4_long_rows(K / 256) && N % MFMA_TILE_ROWS == 0;
     }
     inline bool gemv_mfma_q4k_swiglu_launch(const char *fn, const void *d_w_gate, const void *d_plane_gate,
                                             const void *d_w_up, const void *d_plane_up, const void *d_q8,
@@ -740,7 +749,8 @@ namespace llamql
     // Served for long rows only: each half must keep the wavefronts of a tile busy for several steps.
     inline bool gemv_mfma_q6k_split_ok(int M, int N, int K)
     {
-        return M >= 5 && M <= 8 && K % 512 == 0 && K / 256 >= 64 && N >= 1 && batch_plane_usable_q6k(M, N, K);
+        return M >= MFMA_NAMED_MIN_M && M <= 8 && K % 512 == 0 && K / 256 >= 64 && N >= 1 &&
+               batch_plane_usable_q6k(M < 5 ? 5 : M, N, K);
     }
     inline bool gemv_mfma_q6k_split_launch(const char *fn, const void *d_plane, const void *d_q8, float *d_y_lo,
                                            float *d_y_hi, int M, int N, int K, int ldy, int device_id, hipStream_t st)

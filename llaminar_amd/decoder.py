@@ -113,9 +113,12 @@ class DenseDecoder:
         self.prepared = {} if keep_prepared else None   # name -> prepared weight tensor
         # Matrices of 4096 rows and more get a batch plane where the batch is 5..8 rows (capi.build_batch_plane):
         # Q6_K ones (down, lm_head) an int8 copy, Q4_K ones (Q, O, gate, up) their bytes in the matrix unit's
-        # operand order; same results, less work per launch
+        # operand order; same results, less work per launch.  At batches of 2..4 only the feed-forward matrices get
+        # one: the step runs them on the launches that name the matrix unit (gate + up + SwiGLU in one, the down
+        # projection in two halves), the other projections stay on the quad-lane kernel, which reads no plane.
         if batch_planes is None:
-            batch_planes = batch >= 5
+            batch_planes = batch >= 2
+        ffn_only = batch < 5
         self.planes = {}   # name -> batch plane of that matrix
         g = torch.Generator(device=device)
         g.manual_seed(seed)
@@ -139,7 +142,8 @@ class DenseDecoder:
             w = capi.prepare_weights(fmt, raw, n, k) if prepare else raw
             self.keep.append(w)
             plane = None
-            if prepare and batch_planes and n >= 4096 and capi.batch_plane_bytes(fmt, n, k) > 0:
+            wanted = not ffn_only or name.endswith((".wgate", ".wup", ".wdown"))
+            if prepare and batch_planes and wanted and n >= 4096 and capi.batch_plane_bytes(fmt, n, k) > 0:
                 plane = capi.build_batch_plane(fmt, w, n, k)
                 if plane is not None:
                     self.planes[name] = plane

@@ -1,4 +1,4 @@
-"""The feed-forward block's first half in one launch at batches of 5..8 (llam_ql_gemv_gate_up_swiglu): gate and
+"""The feed-forward block's first half in one launch at batches of 2..8 (llam_ql_gemv_gate_up_swiglu): gate and
 up projection on the matrix unit, SwiGLU and the Q8_1 quantiser of the down projection's input in the workgroup
 that holds both operands.  The projections are checked against the oracle and the unfused launches, the Q8_1
 blocks bit for bit against the stand-alone SwiGLU quantiser on the launch's own projections."""
@@ -14,7 +14,9 @@ pytestmark = pytest.mark.gpu
 # (M, N, K): one pair of tiles per workgroup and several; a count of pairs that leaves the last workgroup
 # partly empty (129 pairs); the shortest rows served (8 super-blocks); rows of 32 super-blocks;
 # the longest rows served with few tiles (two tiles of eight wavefronts would not fit the LDS: fewer per tile)
-_CASES = [(8, 4096, 2048), (5, 4128, 5120), (7, 8192, 8192), (6, 12800, 5120), (8, 4096, 10240), (5, 4096, 11520)]
+# batches of 2..4 (served for callers that do not need the bits of single-row calls)
+_CASES = [(8, 4096, 2048), (5, 4128, 5120), (7, 8192, 8192), (6, 12800, 5120), (8, 4096, 10240), (5, 4096, 11520),
+          (2, 4096, 5120), (3, 8192, 4096), (4, 25600, 5120)]
 
 
 @pytest.mark.parametrize("with_planes", [False, True], ids=["prepared", "planes"])
@@ -96,7 +98,7 @@ def test_full_size_block_against_the_oracles_swiglu(capi, dev, oracle):
 def test_shapes_that_are_not_served(capi, dev):
     import torch
 
-    assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 4, 8192, 5120)      # batches of 1..4: the quad-lane kernel
+    assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 1, 8192, 5120)      # a single row: the quad-lane kernel
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 8, 8200, 5120)      # N not a multiple of 32
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 8, 2048, 5120)      # too few rows for the matrix unit
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q4_K, 8, 5120, 25600)     # rows walked in chunks
@@ -104,9 +106,9 @@ def test_shapes_that_are_not_served(capi, dev):
     assert not capi.gemv_gate_up_swiglu_supported(FMT_Q6_K, 8, 8192, 5120)
     assert not capi.gemv_gate_up_swiglu_supported(FMT_IQ3_S, 8, 8192, 5120)
     w = torch.zeros(8192 * 20 * 144, dtype=torch.uint8, device=dev)
-    q = torch.zeros(4 * 160 * 36, dtype=torch.uint8, device=dev)
+    q = torch.zeros(160 * 36, dtype=torch.uint8, device=dev)
     with pytest.raises(capi.QLError, match="not served"):
-        capi.gemv_gate_up_swiglu(FMT_Q4_K, w, w, q, 4, 8192, 5120)
+        capi.gemv_gate_up_swiglu(FMT_Q4_K, w, w, q, 1, 8192, 5120)
     # a plane for one matrix only
     q = torch.zeros(8 * 160 * 36, dtype=torch.uint8, device=dev)
     plane = torch.zeros(capi.batch_plane_bytes(FMT_Q4_K, 8192, 5120), dtype=torch.uint8, device=dev)

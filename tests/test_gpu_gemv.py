@@ -206,11 +206,12 @@ def test_matrix_unit_matrix_and_quad_lane_group_in_one_launch(capi, dev, M, with
 
 
 @pytest.mark.parametrize("fmt,M,N,K", [(FMT_Q6_K, 8, 5120, 25600), (FMT_Q6_K, 5, 1000, 16384), (FMT_Q6_K, 6, 130, 17408),
+                                       (FMT_Q6_K, 2, 5120, 25600), (FMT_Q6_K, 3, 700, 16384),
                                        (FMT_Q4_K, 8, 5120, 25600), (FMT_Q4_K, 8, 4100, 17408)],
-                         ids=["q6k-m8", "q6k-m5", "q6k-m6-few-rows", "q4k-m8", "q4k-m8-ragged"])
+                         ids=["q6k-m8", "q6k-m5", "q6k-m6-few-rows", "q6k-m2", "q6k-m3", "q4k-m8", "q4k-m8-ragged"])
 def test_long_rows_summed_in_two_halves(capi, dev, oracle, fmt, M, N, K):
-    """llam_ql_gemv_plane_split (batches of 5..8, rows of 64 super-blocks and more, from the batch plane; Q6_K, and
-    Q4_K matrices of 4096 rows and more): the first output is the projection over the first half of every row's
+    """llam_ql_gemv_plane_split (rows of 64 super-blocks and more, from the batch plane; Q6_K at batches of 2..8, and
+    Q4_K matrices of 4096 rows and more at batches of 5..8): the first output is the projection over the first half of every row's
     super-blocks, the second over the second half -- each checked against the oracle on that half of the matrix and
     of the activations -- and their sum is the projection (the one-launch plane kernel to re-association accuracy)."""
     assert capi.gemv_plane_split_supported(fmt, M, N, K)
@@ -219,7 +220,7 @@ def test_long_rows_summed_in_two_halves(capi, dev, oracle, fmt, M, N, K):
     wd, qd = upload_weights(capi, dev, fmt, W), upload_q8(dev, q8)
     plane = capi.build_batch_plane(fmt, wd, N, K)
     lo, hi = capi.gemv_plane_split(fmt, plane, qd, M, N, K)
-    y = capi.gemv(fmt, wd, qd, M, N, K, plane=plane)
+    y = capi.gemv(fmt, wd, qd, M, N, K, plane=plane)   # (batches of up to 4: the quad-lane kernel)
     sync()
     lo, hi, y = lo.cpu().numpy(), hi.cpu().numpy(), y.cpu().numpy()
     assert rel_err(lo + hi, y) <= 2e-6
@@ -233,7 +234,7 @@ def test_long_rows_summed_in_two_halves(capi, dev, oracle, fmt, M, N, K):
         assert rel_err(got[:, rows], C) <= TOL[fmt] * 1e-2
     # not served: short rows, batches of 1..4, other formats, an odd number of super-blocks
     assert not capi.gemv_plane_split_supported(fmt, M, N, 8192)
-    assert not capi.gemv_plane_split_supported(fmt, 4, N, K)
+    assert not capi.gemv_plane_split_supported(fmt, 1, N, K)
     assert not capi.gemv_plane_split_supported(FMT_IQ3_S, M, N, K)
     assert not capi.gemv_plane_split_supported(FMT_Q4_K, M, 1024, K)    # too few rows for the matrix unit
     assert not capi.gemv_plane_split_supported(fmt, M, N, 16640)
