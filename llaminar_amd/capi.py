@@ -516,7 +516,7 @@ def gemv_gate_up_swiglu_supported(fmt: int, M: int, N: int, K: int) -> bool:
 
 def gemv_gate_up_swiglu(fmt: int, w_gate, w_up, q8, M: int, N: int, K: int, plane_gate=None, plane_up=None,
                         want_projections: bool = False, q8_out=None, stream=None):
-    """Q8_1 blocks [M x N/32] of silu(W_gate a) * (W_up a) in one launch (batches of 5..8); with
+    """Q8_1 blocks [M x N/32] of silu(W_gate a) * (W_up a) in one launch (batches of 2..8); with
     want_projections also the fp32 projections the blocks were formed from."""
     import torch
 
