@@ -498,7 +498,7 @@ def gemv_plane_split_supported(fmt: int, M: int, N: int, K: int) -> bool:
 
 def gemv_plane_split(fmt: int, plane, q8, M: int, N: int, K: int, out_lo=None, out_hi=None, stream=None):
     """The sums over the first and the second half of every row's super-blocks as two outputs [M,N] (batches of
-    5..8 on long Q6_K rows, from the matrix's batch plane); their sum is the projection."""
+    2..8 on long Q6_K rows, 5..8 on Q4_K, from the matrix's batch plane); their sum is the projection."""
     import torch
 
     if out_lo is None:
